@@ -1,0 +1,195 @@
+/*
+ * st_hip.h — C ABI of libsthip.so, the gfx950 (MI355X) dense-compute backend for SpiralTorch's
+ * `st-backend-hip` crate.
+ *
+ * Every entry point returns an `int` status: 0 on success, otherwise one of ST_HIP_ERR_*; the text of
+ * the last failure on the calling thread is read with st_hip_last_error_message().  All matrices are
+ * contiguous row-major.  "Host-slice" entry points take host pointers plus the slice lengths the Rust
+ * caller holds, validate them BEFORE touching `out`, and are synchronous.  "_dev" entry points take
+ * device pointers and an explicit stream (NULL = the default stream), enqueue work and return.
+ *
+ * Reference interfaces these replace (paths below the SpiralTorch checkout):
+ *   crates/st-backend-hip/src/lib.rs:607-799   gemm_f32 / gemm_scaled_f32 /
+ *                                              gemm_lhs_transpose_scaled_f32 /
+ *                                              gemm_bias_activation_f32 / gemm_f32_raw
+ *   crates/st-backend-hip/src/real.rs:45-157   the extern "C" block the Rust crate binds
+ *   crates/st-backend-hip/src/hip_kernels/hip_gemm_epilogue.cu:46-54   st_gemm_epilogue_f32
+ */
+#ifndef ST_HIP_H
+#define ST_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- status codes ------------------------------------------------------------------------- */
+enum {
+    ST_HIP_OK = 0,
+    ST_HIP_ERR_NOT_ENABLED = 1, /* HipErr::NotEnabled — no usable HIP device (lib.rs:14-20)        */
+    ST_HIP_ERR_INVALID = 2,     /* HipErr::Other from a validator; `out` was not touched            */
+    ST_HIP_ERR_RUNTIME = 3,     /* HIP call failed: "{ctx}: {name} ({rc}) - {text}" (real.rs:166)   */
+    ST_HIP_ERR_NONFINITE = 4,   /* TensorError::NonFiniteValue{label} (pure.rs:5521-5533)           */
+    ST_HIP_ERR_UNSUPPORTED = 5  /* shape outside what the kernels implement                         */
+};
+
+/* GemmActivation wire codes — crates/st-backend-hip/src/lib.rs:29-34 (Relu = 1, Gelu = 2);
+ * 0 (bias only) extends them for the convolution, whose reference applies ReLU as a separate layer. */
+enum { ST_HIP_ACT_NONE = 0, ST_HIP_ACT_RELU = 1, ST_HIP_ACT_GELU = 2 };
+
+/* ---- runtime ------------------------------------------------------------------------------ */
+
+/* st_backend_hip::init() — lib.rs:168-186.  Idempotent, thread-safe. */
+int st_hip_init(void);
+/* st_backend_hip::real_backend_compiled() — lib.rs:47-49.  Always 1 for this library. */
+int st_hip_real_backend_compiled(void);
+/* HipRuntime::device_count() — lib.rs:188-207 (probe) / real.rs enumerate_devices. */
+int st_hip_device_count(void);
+int st_hip_device_name(int index, char *buf, size_t len);
+
+typedef struct {
+    int compute_units;
+    int clock_khz;
+    int memory_clock_khz;
+    int memory_bus_bits;
+    int wavefront_size;
+    int lds_bytes_per_block;
+    int l2_bytes;
+    uint64_t total_memory_bytes;
+    char arch[64];
+} st_hip_device_props;
+int st_hip_device_properties(int index, st_hip_device_props *out);
+
+/* Copies the calling thread's last error text (NUL-terminated, truncated to len) and returns its full
+ * length.  Precedent: spiraltorch_last_error_* in bindings/spiraltorch-sys/src/lib.rs:149-185. */
+size_t st_hip_last_error_message(char *buf, size_t len);
+
+/* DeviceBuffer / HipStream RAII pairs of real.rs:649-667 and :190-220, flattened to C. */
+int st_hip_malloc(void **device_ptr, size_t bytes);
+int st_hip_free(void *device_ptr);
+int st_hip_memcpy_h2d(void *device_dst, const void *host_src, size_t bytes, void *stream);
+int st_hip_memcpy_d2h(void *host_dst, const void *device_src, size_t bytes, void *stream);
+int st_hip_memset_zero(void *device_dst, size_t bytes, void *stream);
+int st_hip_stream_create(void **stream);
+int st_hip_stream_synchronize(void *stream);
+int st_hip_stream_destroy(void *stream);
+int st_hip_device_synchronize(void);
+/* Timing events recorded on the stream the kernels run on. */
+int st_hip_event_create(void **event);
+int st_hip_event_record(void *event, void *stream);
+int st_hip_event_synchronize(void *event);
+int st_hip_event_elapsed_ms(void *start, void *stop, float *milliseconds);
+int st_hip_event_destroy(void *event);
+
+/* ---- host-slice (drop-in) forms ----------------------------------------------------------- */
+
+/* gemm_f32 / gemm_scaled_f32 / gemm_lhs_transpose_scaled_f32 — lib.rs:607-700.
+ * out(m×n) = (lhs·rhs)·scale; lhs is m×k, or k×m when lhs_transposed != 0; rhs is k×n.
+ * Errors (out untouched): "lhs buffer length {} does not match m*k={}", "rhs buffer length ...",
+ * "output buffer length ...", "gemm scale must be finite, received {}", null pointers. */
+int st_hip_gemm_f32(size_t m, size_t n, size_t k, float scale, int lhs_transposed,
+                    const float *lhs, size_t lhs_len, const float *rhs, size_t rhs_len,
+                    float *out, size_t out_len);
+
+/* gemm_bias_activation_f32 — lib.rs:700-720; epilogue semantics of lib.rs:572-605:
+ * out = act((lhs·rhs + bias[col]) + residual).  residual may be NULL (residual_len ignored).
+ * k == 0 still runs the epilogue on zeros (real.rs:869-871). */
+int st_hip_gemm_bias_act_f32(size_t m, size_t n, size_t k, int activation, const float *lhs,
+                             size_t lhs_len, const float *rhs, size_t rhs_len, const float *bias,
+                             size_t bias_len, const float *residual, size_t residual_len,
+                             float *out, size_t out_len);
+
+/* bf16 operands (raw bit patterns), f32 accumulate and output.  No reference counterpart (the
+ * reference lists bf16 as roadmap in docs/backend_matrix.md); same slice contract as gemm_f32. */
+int st_hip_gemm_bf16_f32acc(size_t m, size_t n, size_t k, const uint16_t *lhs, size_t lhs_len,
+                            const uint16_t *rhs, size_t rhs_len, float *out, size_t out_len);
+
+/* Conv2d::forward (+ bias, + optional activation) — crates/st-nn/src/layers/conv.rs:952-969,
+ * 2559-2599: NCHW input (batch, c_in·h·w), OIHW weight (c_out, c_in·kh·kw), bias (c_out) or NULL,
+ * NCHW output (batch, c_out·oh·ow) with oh/ow from conv.rs:685-700. */
+int st_hip_conv2d_output_hw(size_t h, size_t w, size_t kh, size_t kw, size_t stride_h,
+                            size_t stride_w, size_t pad_h, size_t pad_w, size_t dil_h, size_t dil_w,
+                            size_t *oh, size_t *ow);
+int st_hip_conv2d_bias_act_f32(size_t batch, size_t c_in, size_t h, size_t w, size_t c_out,
+                               size_t kh, size_t kw, size_t stride_h, size_t stride_w, size_t pad_h,
+                               size_t pad_w, size_t dil_h, size_t dil_w, int activation,
+                               const float *input, size_t input_len, const float *weight,
+                               size_t weight_len, const float *bias, size_t bias_len, float *out,
+                               size_t out_len);
+
+/* Tensor::scaled_dot_attention_with_backend — crates/st-tensor/src/pure.rs:4083-4354 with the CPU
+ * kernel of :11845-11919.  q,k,v,out are (contexts·sequence, head_dim); z_bias (contexts, sequence)
+ * or NULL; attn_bias (contexts·sequence, sequence) or NULL.  `causal` != 0 limits query i to keys
+ * 0..=i (crates/st-core/src/backend/cuda_attention.cu:160-164).  Inputs and scale are checked finite
+ * first (pure.rs:4148-4157), the output afterwards (:4206-4210); failures give
+ * ST_HIP_ERR_NONFINITE with the reference's label in the message.  Empty volume returns zeros. */
+int st_hip_attention_f32(size_t contexts, size_t sequence, size_t head_dim, float scale, int causal,
+                         const float *q, size_t q_len, const float *k, size_t k_len, const float *v,
+                         size_t v_len, const float *z_bias, size_t z_bias_len,
+                         const float *attn_bias, size_t attn_bias_len, float *out, size_t out_len);
+
+/* ---- device-resident forms (caller owns device buffers; asynchronous on `stream`) ---------- */
+
+int st_hip_gemm_f32_dev(size_t m, size_t n, size_t k, float scale, int lhs_transposed,
+                        const float *lhs, const float *rhs, float *out, void *stream);
+/* Replaces sgemm + st_gemm_epilogue_f32 (hip_gemm_epilogue.cu:46-71) with one fused launch. */
+int st_hip_gemm_bias_act_f32_dev(size_t m, size_t n, size_t k, int activation, const float *lhs,
+                                 const float *rhs, const float *bias, const float *residual,
+                                 float *out, void *stream);
+int st_hip_gemm_bf16_f32acc_dev(size_t m, size_t n, size_t k, const uint16_t *lhs,
+                                const uint16_t *rhs, float *out, void *stream);
+/* bf16 GEMM with the fused epilogue act((lhs·rhs + bias) + residual); bias/residual may be NULL;
+ * the result is written as f32 to out_f32 and/or rounded (nearest-even) to bf16 into out_bf16. */
+int st_hip_gemm_bf16_bias_act_dev(size_t m, size_t n, size_t k, int activation,
+                                  const uint16_t *lhs, const uint16_t *rhs, const float *bias,
+                                  const float *residual, float *out_f32, uint16_t *out_bf16,
+                                  void *stream);
+int st_hip_conv2d_bias_act_f32_dev(size_t batch, size_t c_in, size_t h, size_t w, size_t c_out,
+                                   size_t kh, size_t kw, size_t stride_h, size_t stride_w,
+                                   size_t pad_h, size_t pad_w, size_t dil_h, size_t dil_w,
+                                   int activation, const float *input, const float *weight,
+                                   const float *bias, float *out, void *stream);
+int st_hip_attention_f32_dev(size_t contexts, size_t sequence, size_t head_dim, float scale,
+                             int causal, const float *q, const float *k, const float *v,
+                             const float *z_bias, const float *attn_bias, float *out, void *stream);
+
+/* Row-wise building blocks of the decoder stack.
+ * layer_norm: crates/st-tensor/src/pure.rs:4008-4058; writes f32 and/or bf16 (either may be NULL).
+ * embedding:  crates/st-nn/src/layers/embedding.rs:42-100,325-330 (round, clamp, gather).
+ * split_heads / merge_heads: (B·S, width) column slices <-> (B·H·S, D) contexts, the re-layout
+ * crates/st-vision/src/models/vit.rs:151-180 performs by indexing. */
+int st_hip_layer_norm_f32_dev(size_t rows, size_t cols, const float *x, const float *residual,
+                              const float *gamma, const float *beta, float epsilon, float *out_f32,
+                              uint16_t *out_bf16, void *stream);
+int st_hip_embedding_f32_dev(size_t tokens, size_t vocab, size_t dim, const float *token_ids,
+                             const float *table, float *out, void *stream);
+int st_hip_f32_to_bf16_dev(size_t count, const float *in, uint16_t *out, void *stream);
+int st_hip_split_heads_f32_dev(size_t batch, size_t seq, size_t heads, size_t head_dim,
+                               const float *qkv, float *q, float *k, float *v, void *stream);
+int st_hip_merge_heads_f32_dev(size_t batch, size_t seq, size_t heads, size_t head_dim,
+                               const float *contexts_in, float *out_f32, uint16_t *out_bf16,
+                               void *stream);
+
+/* ---- byte-level decoder stack (built from the ops above) ------------------------------------ */
+typedef struct {
+    size_t vocab, d_model, heads, layers, d_ff, batch, seq;
+    float ln_eps;
+} st_hip_decoder_config;
+/* Number of f32 values in the flat weight blob: embed (vocab,d); per layer ln1_g, ln1_b,
+ * w_qkv (d,3d), b_qkv, w_o (d,d), b_o, ln2_g, ln2_b, w_fc1 (d,ff), b_fc1, w_fc2 (ff,d), b_fc2;
+ * then lnf_g, lnf_b, w_head (d,vocab), b_head.  Linear weights are (in, out) as in
+ * crates/st-nn/src/layers/linear.rs:49-64. */
+size_t st_hip_decoder_weight_count(const st_hip_decoder_config *config);
+/* Uploads the weights (GEMM operands rounded once to bf16) and allocates all activations. */
+int st_hip_decoder_create(const st_hip_decoder_config *config, const float *host_weights,
+                          size_t weight_len, void **decoder);
+/* tokens: device (batch·seq) f32 ids; logits: device (batch·seq, vocab) f32.  Asynchronous. */
+int st_hip_decoder_forward_dev(void *decoder, const float *tokens, float *logits, void *stream);
+int st_hip_decoder_destroy(void *decoder);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ST_HIP_H */

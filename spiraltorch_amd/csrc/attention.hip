@@ -1,0 +1,310 @@
+// Scaled-dot-product attention with online softmax on the f32 matrix cores of gfx950
+// (flash-style: the S×S score matrix lives only in registers).
+//
+// Semantics: Tensor::scaled_dot_attention_with_backend / fused_attention_cpu,
+// crates/st-tensor/src/pure.rs:4083-4354,11845-11919:
+//   logit[i][j] = (q_i·k_j)*scale (+ z_bias[c][j]) (+ attn_bias[c*S+i][j]);  out_i = softmax_j(logit) · V
+// `causal` keeps keys 0..=i (crates/st-core/src/backend/cuda_attention.cu:160-164).  The CPU path keeps
+// a normalised accumulator per key; this kernel keeps the un-normalised sum and divides once at the end,
+// which is the same value up to rounding.
+//
+// Work split: a 256-thread workgroup owns 128 consecutive queries of one context, 32 per wavefront, and
+// streams K/V tiles of BKV keys through two LDS stages.  Everything is computed TRANSPOSED so that one
+// lane owns one query:
+//   Sᵀ(32 keys × 32 queries) = K_tile · Qᵀ   — A operand = K rows from LDS (one 128-bit read per 4 MFMAs,
+//                                              k issued as the pairs {s, s+4}), B operand = Q from registers
+//   Oᵀ(D × 32 queries)      += Vᵀ · Pᵀ       — B operand = the probabilities exactly where the Sᵀ
+//                                              accumulator left them (register r of lane half h holds key
+//                                              (r/4)*8 + 4h + r%4), A operand = V[that key][d] from LDS
+// so the running max / sum / rescale factors are per-lane scalars, and the only cross-lane traffic of
+// the softmax is one exchange between lane l and lane l^32 for the row maximum.
+#include "device_math.h"
+#include "kernels.h"
+
+namespace sthip {
+
+namespace {
+
+struct AttnArgs {
+    const float *q;
+    const float *k;
+    const float *v;
+    const float *z_bias;
+    const float *attn_bias;
+    float *out;
+    int contexts, S, D;
+    int q_tiles;
+    int swizzle;
+    float scale;
+};
+
+constexpr int kBQ = 128;
+constexpr float kLog2e = 1.4426950408889634f;
+
+template <bool VEC>
+__device__ __forceinline__ float4 load_d4(const float *row, int d, int D, bool row_valid)
+{
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (!row_valid) return v;
+    if (VEC) {
+        if (d < D) v = *reinterpret_cast<const float4 *>(row + d);
+    } else {
+        if (d + 0 < D) v.x = row[d + 0];
+        if (d + 1 < D) v.y = row[d + 1];
+        if (d + 2 < D) v.z = row[d + 2];
+        if (d + 3 < D) v.w = row[d + 3];
+    }
+    return v;
+}
+
+template <int DPAD, int BKV, bool CAUSAL, bool BIAS, bool VEC>
+__global__ __launch_bounds__(256) void attention_f32_kernel(AttnArgs p)
+{
+    constexpr int KS = DPAD + 4;  // K row stride (floats): 128-bit row reads, rows 16 B skewed
+    constexpr int VS = DPAD + 8;  // V row stride: lane halves read rows 4 apart -> different banks
+    constexpr int K_ELEMS = BKV * KS, V_ELEMS = BKV * VS;
+    constexpr int CHUNKS = DPAD / 8;    // groups of 8 head-dim values = 4 MFMAs each
+    constexpr int DT = DPAD / 32;       // 32-row tiles of Oᵀ
+    constexpr int KT = BKV / 32;        // 32-key tiles per stage
+    constexpr int LOADS = BKV * DPAD / 4 / 256;  // float4 per thread per matrix per stage
+    static_assert(LOADS >= 1, "stage too small");
+
+    extern __shared__ __attribute__((aligned(16))) float attn_lds[];
+    float *Ks = attn_lds;                 // [2][K_ELEMS]
+    float *Vs = attn_lds + 2 * K_ELEMS;   // [2][V_ELEMS]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int li = lane & 31, lh = lane >> 5;
+    const int S = p.S, D = p.D;
+
+    int logical = blockIdx.x;
+    if (p.swizzle) logical = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+    const int ctx = logical / p.q_tiles;
+    // Later query tiles see more keys under the causal mask; run them first.
+    const int q_tile = CAUSAL ? (p.q_tiles - 1 - logical % p.q_tiles) : (logical % p.q_tiles);
+    const int q0 = q_tile * kBQ;
+    const int wq0 = q0 + wave * 32;  // first query of this wavefront
+    const int my_q = wq0 + li;
+    const size_t ctx_row0 = static_cast<size_t>(ctx) * S;
+
+    // Q fragments: qf[c][s] = Q[my_q][8c + 4h + s]
+    float qf[CHUNKS][4];
+    {
+        const float *qrow = p.q + (ctx_row0 + my_q) * D;
+        const bool valid = my_q < S;
+#pragma unroll
+        for (int c = 0; c < CHUNKS; ++c) {
+            const float4 v = load_d4<VEC>(qrow, c * 8 + lh * 4, D, valid);
+            qf[c][0] = v.x; qf[c][1] = v.y; qf[c][2] = v.z; qf[c][3] = v.w;
+        }
+    }
+
+    f32x16 oacc[DT];
+#pragma unroll
+    for (int t = 0; t < DT; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[t][r] = 0.0f;
+    float run_max = -INFINITY;  // in log2 units
+    float run_sum = 0.0f;       // this lane half's share of the row sum
+
+    const int key_end = CAUSAL ? min(S, q0 + kBQ) : S;
+    const int stages = (key_end + BKV - 1) / BKV;
+
+    float4 rk[LOADS], rv[LOADS];
+    auto load_global = [&](int key0) {
+#pragma unroll
+        for (int r = 0; r < LOADS; ++r) {
+            const int f = tid + 256 * r;
+            const int row = f / (DPAD / 4), c4 = (f % (DPAD / 4)) * 4;
+            const bool valid = key0 + row < S;
+            const size_t off = (ctx_row0 + key0 + row) * D;
+            rk[r] = load_d4<VEC>(p.k + off, c4, D, valid);
+            rv[r] = load_d4<VEC>(p.v + off, c4, D, valid);
+        }
+    };
+    auto store_lds = [&](int stage) {
+        float *ks = Ks + stage * K_ELEMS;
+        float *vs = Vs + stage * V_ELEMS;
+#pragma unroll
+        for (int r = 0; r < LOADS; ++r) {
+            const int f = tid + 256 * r;
+            const int row = f / (DPAD / 4), c4 = (f % (DPAD / 4)) * 4;
+            *reinterpret_cast<float4 *>(&ks[row * KS + c4]) = rk[r];
+            *reinterpret_cast<float4 *>(&vs[row * VS + c4]) = rv[r];
+        }
+    };
+
+    const float scale = p.scale;
+    const float scale_log2e = p.scale * kLog2e;
+    auto compute = [&](int stage, int key0) {
+        const float *ks = Ks + stage * K_ELEMS;
+        const float *vs = Vs + stage * V_ELEMS;
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) {
+            const int tile_key0 = key0 + kt * 32;
+            if (tile_key0 >= S) continue;                      // workgroup-uniform
+            if (CAUSAL && tile_key0 > wq0 + 31) continue;      // wavefront-uniform: tile entirely masked
+            f32x16 sacc;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sacc[r] = 0.0f;
+#pragma unroll
+            for (int c = 0; c < CHUNKS; ++c) {
+                const float4 kv = *reinterpret_cast<const float4 *>(&ks[(kt * 32 + li) * KS + c * 8 + lh * 4]);
+                sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.x, qf[c][0], sacc, 0, 0, 0);
+                sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.y, qf[c][1], sacc, 0, 0, 0);
+                sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.z, qf[c][2], sacc, 0, 0, 0);
+                sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.w, qf[c][3], sacc, 0, 0, 0);
+            }
+            // logits in log2 units; masked entries become -inf
+            const bool need_mask = (tile_key0 + 32 > S) || (CAUSAL && tile_key0 + 31 > wq0);
+            float tile_max = -INFINITY;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int key = tile_key0 + (r >> 2) * 8 + lh * 4 + (r & 3);
+                float t;
+                if (BIAS) {
+                    // reference order: dot*scale, + z_bias, + attn_bias (pure.rs:11878-11887)
+                    float logit = sacc[r] * scale;
+                    if (key < S && my_q < S) {
+                        if (p.z_bias) logit += p.z_bias[ctx_row0 + key];
+                        if (p.attn_bias) logit += p.attn_bias[(ctx_row0 + my_q) * S + key];
+                    }
+                    t = logit * kLog2e;
+                } else {
+                    t = sacc[r] * scale_log2e;
+                }
+                if (need_mask) {
+                    if (key >= S || (CAUSAL && key > my_q)) t = -INFINITY;
+                }
+                sacc[r] = t;
+                tile_max = fmaxf(tile_max, t);
+            }
+            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32));
+            const float new_max = fmaxf(run_max, tile_max);
+            const float safe_max = new_max == -INFINITY ? 0.0f : new_max;
+            const float alpha = exp2f(run_max - safe_max);  // run_max = -inf -> 0
+            float tile_sum = 0.0f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float pr = exp2f(sacc[r] - safe_max);
+                sacc[r] = pr;
+                tile_sum += pr;
+            }
+            run_sum = run_sum * alpha + tile_sum;
+            run_max = new_max;
+#pragma unroll
+            for (int t = 0; t < DT; ++t)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) oacc[t][r] *= alpha;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int krow = kt * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
+#pragma unroll
+                for (int t = 0; t < DT; ++t) {
+                    const float vv = vs[krow * VS + t * 32 + li];
+                    oacc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv, sacc[r], oacc[t], 0, 0, 0);
+                }
+            }
+        }
+    };
+
+    if (stages > 0) {
+        load_global(0);
+        store_lds(0);
+    }
+    __syncthreads();
+    for (int t = 0; t < stages; ++t) {
+        const bool more = t + 1 < stages;
+        if (more) load_global((t + 1) * BKV);
+        compute(t & 1, t * BKV);
+        if (more) store_lds((t + 1) & 1);
+        __syncthreads();
+    }
+
+    const float total = run_sum + __shfl_xor(run_sum, 32);
+    const float inv = total > 0.0f ? 1.0f / total : 0.0f;
+    if (my_q < S) {
+        float *orow = p.out + (ctx_row0 + my_q) * D;
+#pragma unroll
+        for (int t = 0; t < DT; ++t) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int d = t * 32 + g * 8 + lh * 4;
+                if (VEC) {
+                    if (d < D)
+                        *reinterpret_cast<float4 *>(orow + d) =
+                            make_float4(oacc[t][g * 4 + 0] * inv, oacc[t][g * 4 + 1] * inv, oacc[t][g * 4 + 2] * inv,
+                                        oacc[t][g * 4 + 3] * inv);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (d + e < D) orow[d + e] = oacc[t][g * 4 + e] * inv;
+                }
+            }
+        }
+    }
+}
+
+template <int DPAD, int BKV, bool CAUSAL, bool BIAS, bool VEC>
+hipError_t launch_variant(const AttnArgs &args, hipStream_t stream)
+{
+    constexpr size_t lds_bytes = 2 * static_cast<size_t>(BKV) * ((DPAD + 4) + (DPAD + 8)) * sizeof(float);
+    auto kernel = attention_f32_kernel<DPAD, BKV, CAUSAL, BIAS, VEC>;
+    hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
+    if (rc != hipSuccess) return rc;
+    const size_t blocks = static_cast<size_t>(args.contexts) * args.q_tiles;
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), lds_bytes, stream, args);
+    return hipGetLastError();
+}
+
+template <int DPAD, int BKV>
+hipError_t launch_dpad(const AttnArgs &args, bool causal, bool bias, bool vec, hipStream_t stream)
+{
+    if (causal) {
+        if (bias) return vec ? launch_variant<DPAD, BKV, true, true, true>(args, stream)
+                             : launch_variant<DPAD, BKV, true, true, false>(args, stream);
+        return vec ? launch_variant<DPAD, BKV, true, false, true>(args, stream)
+                   : launch_variant<DPAD, BKV, true, false, false>(args, stream);
+    }
+    if (bias) return vec ? launch_variant<DPAD, BKV, false, true, true>(args, stream)
+                         : launch_variant<DPAD, BKV, false, true, false>(args, stream);
+    return vec ? launch_variant<DPAD, BKV, false, false, true>(args, stream)
+               : launch_variant<DPAD, BKV, false, false, false>(args, stream);
+}
+
+}  // namespace
+
+hipError_t launch_attention_f32(size_t contexts, size_t sequence, size_t head_dim, float scale, bool causal,
+                                const float *q, const float *k, const float *v, const float *z_bias,
+                                const float *attn_bias, float *out, hipStream_t stream)
+{
+    if (contexts == 0 || sequence == 0 || head_dim == 0) return hipSuccess;
+    if (head_dim > static_cast<size_t>(kAttentionMaxHeadDim)) return hipErrorInvalidValue;
+    AttnArgs args;
+    args.q = q;
+    args.k = k;
+    args.v = v;
+    args.z_bias = z_bias;
+    args.attn_bias = attn_bias;
+    args.out = out;
+    args.contexts = static_cast<int>(contexts);
+    args.S = static_cast<int>(sequence);
+    args.D = static_cast<int>(head_dim);
+    args.q_tiles = static_cast<int>((sequence + kBQ - 1) / kBQ);
+    const size_t blocks = contexts * static_cast<size_t>(args.q_tiles);
+    if (blocks > 0x7fffffffu) return hipErrorInvalidConfiguration;
+    args.swizzle = (blocks % 8 == 0) ? 1 : 0;
+    args.scale = scale;
+    const bool bias = z_bias != nullptr || attn_bias != nullptr;
+    auto aligned = [](const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; };
+    const bool vec = (head_dim % 4 == 0) && aligned(q) && aligned(k) && aligned(v) && aligned(out);
+    if (head_dim <= 32) return launch_dpad<32, 64>(args, causal, bias, vec, stream);
+    if (head_dim <= 64) return launch_dpad<64, 64>(args, causal, bias, vec, stream);
+    if (head_dim <= 128) return launch_dpad<128, 64>(args, causal, bias, vec, stream);
+    return launch_dpad<256, 32>(args, causal, bias, vec, stream);
+}
+
+}  // namespace sthip

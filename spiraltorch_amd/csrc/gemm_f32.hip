@@ -1,0 +1,245 @@
+// f32 GEMM on the native f32 matrix cores of gfx950 (v_mfma_f32_32x32x2_f32) with the fused
+// scale / bias / residual / activation epilogue.
+//
+// Replaces rocBLAS sgemm + st_gemm_epilogue_f32 in crates/st-backend-hip/src/real.rs:598-646,817-957
+// and crates/st-backend-hip/src/hip_kernels/hip_gemm_epilogue.cu:19-71.
+//
+// Tiling: one 256-thread workgroup (4 wavefronts, 2×2) owns a BM×BN tile of C and walks K in steps of
+// 16 through two LDS stages; global loads for step t+1 are issued into registers before the MFMAs of
+// step t and written to the other stage afterwards, so a step costs one barrier.
+//
+// MFMA operand layout (32x32x2): lane l supplies A[l%32][l/32] and B[l/32][l%32]; accumulator register
+// r of lane l is C[(r/4)*8 + (l/32)*4 + r%4][l%32].  Because the sum over k is order-free, each group
+// of 8 k-values is issued as the pairs {s, s+4}: lane half h = l/32 then needs k = 4h..4h+3 of the
+// group, which is ONE 128-bit LDS read per operand row when the tile is stored k-contiguous.
+#include "device_math.h"
+#include "kernels.h"
+
+namespace sthip {
+
+namespace {
+
+struct GemmF32Args {
+    const float *A;
+    const float *B;
+    float *C;
+    const float *bias;
+    const float *residual;
+    int M, N, K;
+    int tiles_n;  // tiles along N; the grid is one-dimensional over (tile_m, tile_n)
+    float scale;
+    int activation;
+};
+
+constexpr int kBK = 16;
+
+template <bool VEC>
+__device__ __forceinline__ float4 load_row4(const float *base, size_t row_offset, int col, int col_limit,
+                                            bool row_valid)
+{
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (!row_valid) return v;
+    const float *src = base + row_offset + col;
+    if (VEC) {
+        if (col < col_limit) v = *reinterpret_cast<const float4 *>(src);
+    } else {
+        if (col + 0 < col_limit) v.x = src[0];
+        if (col + 1 < col_limit) v.y = src[1];
+        if (col + 2 < col_limit) v.z = src[2];
+        if (col + 3 < col_limit) v.w = src[3];
+    }
+    return v;
+}
+
+template <int BM, int BN, bool AT, bool VEC>
+__global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32Args p)
+{
+    constexpr int TM = BM / 64;  // 32×32 MFMA tiles per wavefront along M (wave tile = BM/2 × BN/2)
+    constexpr int TN = BN / 64;
+    constexpr int A_STRIDE = AT ? (BM + 8) : (kBK + 4);
+    constexpr int A_ELEMS = AT ? kBK * A_STRIDE : BM * A_STRIDE;
+    constexpr int B_STRIDE = BN + 8;
+    constexpr int B_ELEMS = kBK * B_STRIDE;
+    __shared__ __attribute__((aligned(16))) float As[2][A_ELEMS];
+    __shared__ __attribute__((aligned(16))) float Bs[2][B_ELEMS];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int li = lane & 31, lh = lane >> 5;
+    const int tile_m = blockIdx.x / p.tiles_n, tile_n = blockIdx.x % p.tiles_n;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int M = p.M, N = p.N, K = p.K;
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int a = 0; a < TM; ++a)
+#pragma unroll
+        for (int b = 0; b < TN; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.0f;
+
+    float4 ra[TM], rb[TN];
+
+    auto load_global = [&](int k0) {
+#pragma unroll
+        for (int r = 0; r < TM; ++r) {
+            const int f = tid + 256 * r;
+            if (!AT) {
+                const int row = f >> 2, c4 = (f & 3) * 4;
+                ra[r] = load_row4<VEC>(p.A, static_cast<size_t>(m0 + row) * K, k0 + c4, K, m0 + row < M);
+            } else {
+                const int krow = f / (BM / 4), c4 = (f % (BM / 4)) * 4;
+                ra[r] = load_row4<VEC>(p.A, static_cast<size_t>(k0 + krow) * M, m0 + c4, M, k0 + krow < K);
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < TN; ++r) {
+            const int f = tid + 256 * r;
+            const int krow = f / (BN / 4), c4 = (f % (BN / 4)) * 4;
+            rb[r] = load_row4<VEC>(p.B, static_cast<size_t>(k0 + krow) * N, n0 + c4, N, k0 + krow < K);
+        }
+    };
+    auto store_lds = [&](int stage) {
+#pragma unroll
+        for (int r = 0; r < TM; ++r) {
+            const int f = tid + 256 * r;
+            if (!AT) {
+                const int row = f >> 2, c4 = (f & 3) * 4;
+                *reinterpret_cast<float4 *>(&As[stage][row * A_STRIDE + c4]) = ra[r];
+            } else {
+                const int krow = f / (BM / 4), c4 = (f % (BM / 4)) * 4;
+                *reinterpret_cast<float4 *>(&As[stage][krow * A_STRIDE + c4]) = ra[r];
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < TN; ++r) {
+            const int f = tid + 256 * r;
+            const int krow = f / (BN / 4), c4 = (f % (BN / 4)) * 4;
+            *reinterpret_cast<float4 *>(&Bs[stage][krow * B_STRIDE + c4]) = rb[r];
+        }
+    };
+    auto compute = [&](int stage) {
+        const float *as = As[stage];
+        const float *bs = Bs[stage];
+#pragma unroll
+        for (int kk = 0; kk < kBK / 8; ++kk) {
+            float a[TM][4], b[TN][4];
+#pragma unroll
+            for (int tm = 0; tm < TM; ++tm) {
+                const int row = wm * (BM / 2) + tm * 32 + li;
+                if (!AT) {
+                    const float4 v = *reinterpret_cast<const float4 *>(&as[row * A_STRIDE + kk * 8 + lh * 4]);
+                    a[tm][0] = v.x; a[tm][1] = v.y; a[tm][2] = v.z; a[tm][3] = v.w;
+                } else {
+#pragma unroll
+                    for (int s = 0; s < 4; ++s) a[tm][s] = as[(kk * 8 + lh * 4 + s) * A_STRIDE + row];
+                }
+            }
+#pragma unroll
+            for (int tn = 0; tn < TN; ++tn) {
+                const int col = wn * (BN / 2) + tn * 32 + li;
+#pragma unroll
+                for (int s = 0; s < 4; ++s) b[tn][s] = bs[(kk * 8 + lh * 4 + s) * B_STRIDE + col];
+            }
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+#pragma unroll
+                for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+                    for (int tn = 0; tn < TN; ++tn)
+                        acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[tm][s], b[tn][s], acc[tm][tn], 0, 0, 0);
+        }
+    };
+
+    const int steps = (K + kBK - 1) / kBK;
+    if (steps > 0) {
+        load_global(0);
+        store_lds(0);
+    }
+    __syncthreads();
+    for (int t = 0; t < steps; ++t) {
+        const bool more = t + 1 < steps;
+        if (more) load_global((t + 1) * kBK);
+        compute(t & 1);
+        if (more) store_lds((t + 1) & 1);
+        __syncthreads();
+    }
+
+    // Epilogue: value = acc*scale; (value + bias[col]) + residual; activation.
+    const bool scaled = p.scale != 1.0f;
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) {
+        const int col = n0 + wn * (BN / 2) + tn * 32 + li;
+        if (col >= N) continue;
+        const float bias = p.bias ? p.bias[col] : 0.0f;
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = m0 + wm * (BM / 2) + tm * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
+                if (row >= M) continue;
+                const size_t idx = static_cast<size_t>(row) * N + col;
+                float value = acc[tm][tn][r];
+                if (scaled) value *= p.scale;
+                if (p.bias) value += bias;
+                if (p.residual) value += p.residual[idx];
+                p.C[idx] = apply_activation(value, p.activation);
+            }
+        }
+    }
+}
+
+template <int BM, int BN>
+hipError_t launch_tile(GemmF32Args args, bool lhs_transposed, bool vec, hipStream_t stream)
+{
+    args.tiles_n = (args.N + BN - 1) / BN;
+    const size_t tiles = static_cast<size_t>(args.tiles_n) * static_cast<size_t>((args.M + BM - 1) / BM);
+    if (tiles > 0x7fffffffu) return hipErrorInvalidConfiguration;
+    const dim3 grid(static_cast<unsigned>(tiles));
+    const dim3 block(256);
+    if (lhs_transposed) {
+        if (vec)
+            hipLaunchKernelGGL((gemm_f32_kernel<BM, BN, true, true>), grid, block, 0, stream, args);
+        else
+            hipLaunchKernelGGL((gemm_f32_kernel<BM, BN, true, false>), grid, block, 0, stream, args);
+    } else {
+        if (vec)
+            hipLaunchKernelGGL((gemm_f32_kernel<BM, BN, false, true>), grid, block, 0, stream, args);
+        else
+            hipLaunchKernelGGL((gemm_f32_kernel<BM, BN, false, false>), grid, block, 0, stream, args);
+    }
+    return hipGetLastError();
+}
+
+bool aligned16(const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
+
+}  // namespace
+
+hipError_t launch_gemm_f32(size_t m, size_t n, size_t k, bool lhs_transposed, const float *lhs,
+                           const float *rhs, float *out, const GemmEpilogue &epilogue, hipStream_t stream)
+{
+    if (m == 0 || n == 0) return hipSuccess;
+    GemmF32Args args;
+    args.A = lhs;
+    args.B = rhs;
+    args.C = out;
+    args.bias = epilogue.bias;
+    args.residual = epilogue.residual;
+    args.M = static_cast<int>(m);
+    args.N = static_cast<int>(n);
+    args.K = static_cast<int>(k);
+    args.scale = epilogue.scale;
+    args.activation = epilogue.activation;
+    // 128-bit global loads need every row start 16-byte aligned.
+    const size_t lhs_ld = lhs_transposed ? m : k;
+    const bool vec = (lhs_ld % 4 == 0) && (n % 4 == 0) && aligned16(lhs) && aligned16(rhs);
+    // Large tiles once they give every compute unit at least one workgroup, otherwise small tiles so
+    // that small problems still spread over the chip.
+    const size_t big_tiles = ((m + 127) / 128) * ((n + 127) / 128);
+    if (big_tiles >= 256) return launch_tile<128, 128>(args, lhs_transposed, vec, stream);
+    return launch_tile<64, 64>(args, lhs_transposed, vec, stream);
+}
+
+}  // namespace sthip

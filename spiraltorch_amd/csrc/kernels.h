@@ -1,0 +1,54 @@
+// Internal launcher interface between the C-ABI entry points and the gfx950 kernels.
+// Every launcher validates nothing: callers have already checked shapes, pointers and alignment
+// assumptions that the kernels rely on are re-derived inside the launcher from the arguments.
+#pragma once
+
+#include "common.h"
+
+namespace sthip {
+
+struct GemmEpilogue {
+    float scale = 1.0f;              // applied to the full sum, before bias (pure.rs:2256-2262)
+    const float *bias = nullptr;     // per column (per row for the convolution)
+    const float *residual = nullptr; // same shape as the output
+    int activation = ST_HIP_ACT_NONE;
+};
+
+// C(m×n) = epilogue(A·B); A is m×k (k×m when lhs_transposed), B is k×n, all f32 row-major.
+hipError_t launch_gemm_f32(size_t m, size_t n, size_t k, bool lhs_transposed, const float *lhs,
+                           const float *rhs, float *out, const GemmEpilogue &epilogue,
+                           hipStream_t stream);
+
+// bf16 operands, f32 accumulation; writes out_f32 and/or out_bf16 (either may be null).
+hipError_t launch_gemm_bf16(size_t m, size_t n, size_t k, const uint16_t *lhs, const uint16_t *rhs,
+                            float *out_f32, uint16_t *out_bf16, const GemmEpilogue &epilogue,
+                            hipStream_t stream);
+
+struct ConvShape {
+    int batch, c_in, h, w, c_out, kh, kw, stride_h, stride_w, pad_h, pad_w, dil_h, dil_w, oh, ow;
+};
+// Largest c_in*kh*kw the implicit-GEMM kernel's LDS offset table holds.
+constexpr int kConvMaxReduction = 8192;
+hipError_t launch_conv2d_f32(const ConvShape &shape, int activation, const float *input,
+                             const float *weight, const float *bias, float *out, hipStream_t stream);
+
+// Largest head_dim the attention kernel is instantiated for.
+constexpr int kAttentionMaxHeadDim = 256;
+hipError_t launch_attention_f32(size_t contexts, size_t sequence, size_t head_dim, float scale,
+                                bool causal, const float *q, const float *k, const float *v,
+                                const float *z_bias, const float *attn_bias, float *out,
+                                hipStream_t stream);
+
+hipError_t launch_layer_norm_f32(size_t rows, size_t cols, const float *x, const float *residual,
+                                 const float *gamma, const float *beta, float epsilon, float *out_f32,
+                                 uint16_t *out_bf16, hipStream_t stream);
+hipError_t launch_embedding_f32(size_t tokens, size_t vocab, size_t dim, const float *token_ids,
+                                const float *table, float *out, hipStream_t stream);
+hipError_t launch_f32_to_bf16(size_t count, const float *in, uint16_t *out, hipStream_t stream);
+hipError_t launch_split_heads_f32(size_t batch, size_t seq, size_t heads, size_t head_dim,
+                                  const float *qkv, float *q, float *k, float *v, hipStream_t stream);
+hipError_t launch_merge_heads_f32(size_t batch, size_t seq, size_t heads, size_t head_dim,
+                                  const float *contexts_in, float *out_f32, uint16_t *out_bf16,
+                                  hipStream_t stream);
+
+}  // namespace sthip

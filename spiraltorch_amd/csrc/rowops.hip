@@ -1,0 +1,171 @@
+// Row-wise, HBM-bound helpers of the decoder stack: layer-norm, embedding gather, f32->bf16 rounding
+// and the (tokens, heads*dim) <-> (contexts*seq, dim) re-layouts around attention.
+#include "device_math.h"
+#include "kernels.h"
+
+namespace sthip {
+
+namespace {
+
+__device__ __forceinline__ float wave_sum(float v)
+{
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) v += __shfl_xor(v, offset);
+    return v;
+}
+
+// One wavefront per row.  layer_norm_cpu, crates/st-tensor/src/pure.rs:4008-4058:
+// mean = Σv/cols; var = max(Σv²/cols − mean², 0); out = ((v − mean)/sqrt(var + eps))·γ + β.
+__global__ __launch_bounds__(256) void layer_norm_kernel(int rows, int cols, const float *x, const float *residual,
+                                                         const float *gamma, const float *beta, float epsilon,
+                                                         float *out_f32, uint16_t *out_bf16)
+{
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const size_t offset = static_cast<size_t>(row) * cols;
+    float sum = 0.0f, sumsq = 0.0f;
+    for (int c = lane; c < cols; c += 64) {
+        float v = x[offset + c];
+        if (residual) v += residual[offset + c];
+        sum += v;
+        sumsq += v * v;
+    }
+    sum = wave_sum(sum);
+    sumsq = wave_sum(sumsq);
+    const float cols_f = static_cast<float>(cols);
+    const float mean = sum / cols_f;
+    const float var = fmaxf(sumsq / cols_f - mean * mean, 0.0f);
+    const float denom = sqrtf(var + epsilon);
+    for (int c = lane; c < cols; c += 64) {
+        float v = x[offset + c];
+        if (residual) v += residual[offset + c];
+        const float value = ((v - mean) / denom) * gamma[c] + beta[c];
+        if (out_f32) out_f32[offset + c] = value;
+        if (out_bf16) out_bf16[offset + c] = f32_to_bf16_rne(value);
+    }
+}
+
+// token_to_index + row gather, crates/st-nn/src/layers/embedding.rs:42-100,325-330.
+__global__ __launch_bounds__(256) void embedding_kernel(int tokens, int vocab, int dim, const float *token_ids,
+                                                        const float *table, float *out)
+{
+    const int token = blockIdx.x;
+    if (token >= tokens) return;
+    const float value = token_ids[token];
+    int index = 0;
+    if (isfinite(value)) {
+        const float rounded = roundf(value);
+        if (rounded > 0.0f) index = rounded >= static_cast<float>(vocab) ? vocab - 1 : static_cast<int>(rounded);
+        if (index > vocab - 1) index = vocab - 1;
+    }
+    const float *src = table + static_cast<size_t>(index) * dim;
+    float *dst = out + static_cast<size_t>(token) * dim;
+    for (int c = threadIdx.x; c < dim; c += 256) dst[c] = src[c];
+}
+
+__global__ __launch_bounds__(256) void f32_to_bf16_kernel(size_t count, const float *in, uint16_t *out)
+{
+    const size_t stride = static_cast<size_t>(gridDim.x) * 256;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < count; i += stride)
+        out[i] = f32_to_bf16_rne(in[i]);
+}
+
+// qkv (B·S, 3·H·D) with column blocks [Q | K | V] -> q, k, v each (B·H·S, D).
+__global__ __launch_bounds__(256) void split_heads_kernel(int batch, int seq, int heads, int dim, const float *qkv,
+                                                          float *q, float *k, float *v)
+{
+    const size_t total = static_cast<size_t>(batch) * seq * heads * dim;
+    const size_t stride = static_cast<size_t>(gridDim.x) * 256;
+    const int width = heads * dim;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < total; i += stride) {
+        const int d = static_cast<int>(i % dim);
+        size_t rest = i / dim;
+        const int s = static_cast<int>(rest % seq);
+        rest /= seq;
+        const int h = static_cast<int>(rest % heads);
+        const int b = static_cast<int>(rest / heads);
+        const size_t src = (static_cast<size_t>(b) * seq + s) * 3 * width + static_cast<size_t>(h) * dim + d;
+        q[i] = qkv[src];
+        k[i] = qkv[src + width];
+        v[i] = qkv[src + 2 * width];
+    }
+}
+
+// (B·H·S, D) -> (B·S, H·D)
+__global__ __launch_bounds__(256) void merge_heads_kernel(int batch, int seq, int heads, int dim, const float *in,
+                                                          float *out_f32, uint16_t *out_bf16)
+{
+    const size_t total = static_cast<size_t>(batch) * seq * heads * dim;
+    const size_t stride = static_cast<size_t>(gridDim.x) * 256;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < total; i += stride) {
+        // i indexes the OUTPUT (b, s, h, d) so stores are contiguous
+        const int d = static_cast<int>(i % dim);
+        size_t rest = i / dim;
+        const int h = static_cast<int>(rest % heads);
+        rest /= heads;
+        const int s = static_cast<int>(rest % seq);
+        const int b = static_cast<int>(rest / seq);
+        const float value = in[((static_cast<size_t>(b) * heads + h) * seq + s) * dim + d];
+        if (out_f32) out_f32[i] = value;
+        if (out_bf16) out_bf16[i] = f32_to_bf16_rne(value);
+    }
+}
+
+unsigned grid_for(size_t count)
+{
+    const size_t blocks = (count + 255) / 256;
+    return static_cast<unsigned>(blocks < 65536 ? (blocks ? blocks : 1) : 65536);
+}
+
+}  // namespace
+
+hipError_t launch_layer_norm_f32(size_t rows, size_t cols, const float *x, const float *residual, const float *gamma,
+                                 const float *beta, float epsilon, float *out_f32, uint16_t *out_bf16,
+                                 hipStream_t stream)
+{
+    if (rows == 0 || cols == 0) return hipSuccess;
+    hipLaunchKernelGGL(layer_norm_kernel, dim3(static_cast<unsigned>((rows + 3) / 4)), dim3(256), 0, stream,
+                       static_cast<int>(rows), static_cast<int>(cols), x, residual, gamma, beta, epsilon, out_f32,
+                       out_bf16);
+    return hipGetLastError();
+}
+
+hipError_t launch_embedding_f32(size_t tokens, size_t vocab, size_t dim, const float *token_ids, const float *table,
+                                float *out, hipStream_t stream)
+{
+    if (tokens == 0 || dim == 0) return hipSuccess;
+    hipLaunchKernelGGL(embedding_kernel, dim3(static_cast<unsigned>(tokens)), dim3(256), 0, stream,
+                       static_cast<int>(tokens), static_cast<int>(vocab), static_cast<int>(dim), token_ids, table, out);
+    return hipGetLastError();
+}
+
+hipError_t launch_f32_to_bf16(size_t count, const float *in, uint16_t *out, hipStream_t stream)
+{
+    if (count == 0) return hipSuccess;
+    hipLaunchKernelGGL(f32_to_bf16_kernel, dim3(grid_for(count)), dim3(256), 0, stream, count, in, out);
+    return hipGetLastError();
+}
+
+hipError_t launch_split_heads_f32(size_t batch, size_t seq, size_t heads, size_t head_dim, const float *qkv, float *q,
+                                  float *k, float *v, hipStream_t stream)
+{
+    const size_t total = batch * seq * heads * head_dim;
+    if (total == 0) return hipSuccess;
+    hipLaunchKernelGGL(split_heads_kernel, dim3(grid_for(total)), dim3(256), 0, stream, static_cast<int>(batch),
+                       static_cast<int>(seq), static_cast<int>(heads), static_cast<int>(head_dim), qkv, q, k, v);
+    return hipGetLastError();
+}
+
+hipError_t launch_merge_heads_f32(size_t batch, size_t seq, size_t heads, size_t head_dim, const float *contexts_in,
+                                  float *out_f32, uint16_t *out_bf16, hipStream_t stream)
+{
+    const size_t total = batch * seq * heads * head_dim;
+    if (total == 0) return hipSuccess;
+    hipLaunchKernelGGL(merge_heads_kernel, dim3(grid_for(total)), dim3(256), 0, stream, static_cast<int>(batch),
+                       static_cast<int>(seq), static_cast<int>(heads), static_cast<int>(head_dim), contexts_in, out_f32,
+                       out_bf16);
+    return hipGetLastError();
+}
+
+}  // namespace sthip

@@ -1,0 +1,240 @@
+// Runtime half of the C ABI: init/probe, error text, device buffers, streams and events.
+// Mirrors crates/st-backend-hip/src/lib.rs:148-207 (init once, shared by all threads) and the RAII
+// wrappers of crates/st-backend-hip/src/real.rs:190-220,649-697, flattened to C handles.
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "common.h"
+
+namespace sthip {
+
+namespace {
+thread_local std::string g_last_error;
+
+struct Runtime {
+    std::mutex mutex;
+    bool ready = false;
+    int status = ST_HIP_ERR_NOT_ENABLED;
+    std::string error;
+    std::vector<hipDeviceProp_t> devices;
+};
+
+Runtime &runtime()
+{
+    static Runtime instance;
+    return instance;
+}
+}  // namespace
+
+int fail(int code, const char *fmt, ...)
+{
+    char buffer[512];
+    va_list args;
+    va_start(args, fmt);
+    vsnprintf(buffer, sizeof buffer, fmt, args);
+    va_end(args);
+    g_last_error = buffer;
+    return code;
+}
+
+int hip_fail(hipError_t rc, const char *ctx)
+{
+    (void)hipGetLastError();  // clear the sticky flag so the next call starts clean
+    return fail(ST_HIP_ERR_RUNTIME, "%s: %s (%d) - %s", ctx, hipGetErrorName(rc), static_cast<int>(rc),
+                hipGetErrorString(rc));
+}
+
+void clear_error() { g_last_error.clear(); }
+
+int ensure_init()
+{
+    Runtime &rt = runtime();
+    std::lock_guard<std::mutex> lock(rt.mutex);
+    if (rt.ready) return ST_HIP_OK;
+    int count = 0;
+    hipError_t rc = hipGetDeviceCount(&count);
+    if (rc != hipSuccess || count <= 0) {
+        (void)hipGetLastError();
+        return fail(ST_HIP_ERR_NOT_ENABLED, "HIP not enabled (no usable HIP device: %s)",
+                    rc == hipSuccess ? "device count is 0" : hipGetErrorString(rc));
+    }
+    std::vector<hipDeviceProp_t> devices(static_cast<size_t>(count));
+    for (int i = 0; i < count; ++i) {
+        rc = hipGetDeviceProperties(&devices[static_cast<size_t>(i)], i);
+        if (rc != hipSuccess) return hip_fail(rc, "hipGetDeviceProperties");
+    }
+    if (std::strncmp(devices[0].gcnArchName, "gfx950", 6) != 0) {
+        return fail(ST_HIP_ERR_NOT_ENABLED,
+                    "HIP not enabled (device 0 is %s; this library carries gfx950 code only)",
+                    devices[0].gcnArchName);
+    }
+    rt.devices.swap(devices);
+    rt.ready = true;
+    return ST_HIP_OK;
+}
+
+}  // namespace sthip
+
+using namespace sthip;
+
+extern "C" {
+
+int st_hip_init(void) { return ensure_init(); }
+
+int st_hip_real_backend_compiled(void) { return 1; }
+
+int st_hip_device_count(void)
+{
+    if (ensure_init() != ST_HIP_OK) return 0;
+    return static_cast<int>(runtime().devices.size());
+}
+
+int st_hip_device_name(int index, char *buf, size_t len)
+{
+    ST_HIP_CHECK(ensure_init());
+    if (index < 0 || static_cast<size_t>(index) >= runtime().devices.size() || !buf || len == 0)
+        return fail(ST_HIP_ERR_INVALID, "device index %d out of range", index);
+    const hipDeviceProp_t &p = runtime().devices[static_cast<size_t>(index)];
+    snprintf(buf, len, "%s", p.name[0] ? p.name : p.gcnArchName);
+    return ST_HIP_OK;
+}
+
+int st_hip_device_properties(int index, st_hip_device_props *out)
+{
+    ST_HIP_CHECK(ensure_init());
+    if (index < 0 || static_cast<size_t>(index) >= runtime().devices.size() || !out)
+        return fail(ST_HIP_ERR_INVALID, "device index %d out of range", index);
+    const hipDeviceProp_t &p = runtime().devices[static_cast<size_t>(index)];
+    std::memset(out, 0, sizeof *out);
+    out->compute_units = p.multiProcessorCount;
+    out->clock_khz = p.clockRate;
+    out->memory_clock_khz = p.memoryClockRate;
+    out->memory_bus_bits = p.memoryBusWidth;
+    out->wavefront_size = p.warpSize;
+    out->lds_bytes_per_block = static_cast<int>(p.sharedMemPerBlock);
+    out->l2_bytes = p.l2CacheSize;
+    out->total_memory_bytes = p.totalGlobalMem;
+    snprintf(out->arch, sizeof out->arch, "%s", p.gcnArchName);
+    return ST_HIP_OK;
+}
+
+size_t st_hip_last_error_message(char *buf, size_t len)
+{
+    if (buf && len > 0) snprintf(buf, len, "%s", g_last_error.c_str());
+    return g_last_error.size();
+}
+
+int st_hip_malloc(void **device_ptr, size_t bytes)
+{
+    ST_HIP_CHECK(ensure_init());
+    if (!device_ptr) return fail(ST_HIP_ERR_INVALID, "st_hip_malloc received a null out-pointer");
+    *device_ptr = nullptr;
+    ST_HIP_TRY(hipMalloc(device_ptr, bytes ? bytes : 1), "hipMalloc");  // real.rs:652 max(1)
+    return ST_HIP_OK;
+}
+
+int st_hip_free(void *device_ptr)
+{
+    if (!device_ptr) return ST_HIP_OK;
+    ST_HIP_TRY(hipFree(device_ptr), "hipFree");
+    return ST_HIP_OK;
+}
+
+int st_hip_memcpy_h2d(void *device_dst, const void *host_src, size_t bytes, void *stream)
+{
+    if (bytes == 0) return ST_HIP_OK;
+    ST_HIP_TRY(hipMemcpyAsync(device_dst, host_src, bytes, hipMemcpyHostToDevice, as_stream(stream)),
+               "hipMemcpyAsync(H2D)");
+    ST_HIP_TRY(hipStreamSynchronize(as_stream(stream)), "hipStreamSynchronize");
+    return ST_HIP_OK;
+}
+
+int st_hip_memcpy_d2h(void *host_dst, const void *device_src, size_t bytes, void *stream)
+{
+    if (bytes == 0) return ST_HIP_OK;
+    ST_HIP_TRY(hipMemcpyAsync(host_dst, device_src, bytes, hipMemcpyDeviceToHost, as_stream(stream)),
+               "hipMemcpyAsync(D2H)");
+    ST_HIP_TRY(hipStreamSynchronize(as_stream(stream)), "hipStreamSynchronize");
+    return ST_HIP_OK;
+}
+
+int st_hip_memset_zero(void *device_dst, size_t bytes, void *stream)
+{
+    if (bytes == 0) return ST_HIP_OK;
+    ST_HIP_TRY(hipMemsetAsync(device_dst, 0, bytes, as_stream(stream)), "hipMemsetAsync");
+    return ST_HIP_OK;
+}
+
+int st_hip_stream_create(void **stream)
+{
+    ST_HIP_CHECK(ensure_init());
+    if (!stream) return fail(ST_HIP_ERR_INVALID, "st_hip_stream_create received a null out-pointer");
+    hipStream_t raw = nullptr;
+    ST_HIP_TRY(hipStreamCreate(&raw), "hipStreamCreate");
+    *stream = raw;
+    return ST_HIP_OK;
+}
+
+int st_hip_stream_synchronize(void *stream)
+{
+    ST_HIP_TRY(hipStreamSynchronize(as_stream(stream)), "hipStreamSynchronize");
+    return ST_HIP_OK;
+}
+
+int st_hip_stream_destroy(void *stream)
+{
+    if (!stream) return ST_HIP_OK;
+    // Same order as HipStream::drop (real.rs:207-214): drain, then release.
+    (void)hipStreamSynchronize(as_stream(stream));
+    ST_HIP_TRY(hipStreamDestroy(as_stream(stream)), "hipStreamDestroy");
+    return ST_HIP_OK;
+}
+
+int st_hip_device_synchronize(void)
+{
+    ST_HIP_TRY(hipDeviceSynchronize(), "hipDeviceSynchronize");
+    return ST_HIP_OK;
+}
+
+int st_hip_event_create(void **event)
+{
+    ST_HIP_CHECK(ensure_init());
+    if (!event) return fail(ST_HIP_ERR_INVALID, "st_hip_event_create received a null out-pointer");
+    hipEvent_t raw = nullptr;
+    ST_HIP_TRY(hipEventCreate(&raw), "hipEventCreate");
+    *event = raw;
+    return ST_HIP_OK;
+}
+
+int st_hip_event_record(void *event, void *stream)
+{
+    ST_HIP_TRY(hipEventRecord(static_cast<hipEvent_t>(event), as_stream(stream)), "hipEventRecord");
+    return ST_HIP_OK;
+}
+
+int st_hip_event_synchronize(void *event)
+{
+    ST_HIP_TRY(hipEventSynchronize(static_cast<hipEvent_t>(event)), "hipEventSynchronize");
+    return ST_HIP_OK;
+}
+
+int st_hip_event_elapsed_ms(void *start, void *stop, float *milliseconds)
+{
+    if (!milliseconds) return fail(ST_HIP_ERR_INVALID, "st_hip_event_elapsed_ms received a null out-pointer");
+    ST_HIP_TRY(hipEventElapsedTime(milliseconds, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)),
+               "hipEventElapsedTime");
+    return ST_HIP_OK;
+}
+
+int st_hip_event_destroy(void *event)
+{
+    if (!event) return ST_HIP_OK;
+    ST_HIP_TRY(hipEventDestroy(static_cast<hipEvent_t>(event)), "hipEventDestroy");
+    return ST_HIP_OK;
+}
+
+}  // extern "C"

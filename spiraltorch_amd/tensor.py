@@ -1,0 +1,244 @@
+"""Mirror of the `st-tensor` operator surface that reaches the HIP backend.
+
+`Tensor` is the reference's 2-D row-major f32 matrix (crates/st-tensor/src/pure.rs:1406-1411); the
+methods below are the ones whose `MatmulBackend::GpuHip` arm exists in the reference
+(pure.rs:2008-2556, 4411-4634) plus `scaled_dot_attention` (pure.rs:4061-4354) and the Conv2d layer
+(crates/st-nn/src/layers/conv.rs:607-969), which this build adds to the HIP backend.  Method names and
+keyword arguments follow the Python binding (bindings/st-py/src/tensor.rs:970-1299).
+
+Only `backend="hip"` (or "auto", which selects hip) is served.  There is no CPU path in this package:
+every method runs on the GPU or raises.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import numpy as np
+
+from . import hip
+from . import _lib
+
+
+class TensorError(Exception):
+    """`TensorError` variants of the reference that this surface can raise; `kind` is the variant name."""
+
+    def __init__(self, kind: str, message: str, **fields):
+        super().__init__(f"{kind}: {message}")
+        self.kind = kind
+        self.message = message
+        self.fields = fields
+
+
+def _resolve_backend(backend: Optional[str]) -> str:
+    label = "auto" if backend is None else backend
+    if label in ("auto", "hip", "rocm"):
+        return "hip"
+    raise TensorError("BackendFailure", f"backend '{label}' is not provided by this package; only 'hip' is",
+                      backend=label)
+
+
+def _backend_failure(err: hip.HipErr) -> TensorError:
+    # pure.rs:2158-2163 wraps HIP errors as BackendFailure{backend:"hip", message}; the finite checks the
+    # Tensor layer performs itself surface as NonFiniteValue (pure.rs:5521-5533).
+    if err.status == _lib.ERR_NONFINITE:
+        label = err.message.split(" in ", 1)[-1].split(":", 1)[0]
+        return TensorError("NonFiniteValue", err.message, label=label)
+    return TensorError("BackendFailure", err.message, backend="hip")
+
+
+def _validate_finite(label: str, data: np.ndarray) -> None:
+    if not np.isfinite(data).all():
+        bad = data[~np.isfinite(data)].ravel()[0]
+        raise TensorError("NonFiniteValue", f"non-finite value encountered in {label}: {bad}", label=label)
+
+
+class Tensor:
+    """2-D row-major float32 matrix held on the host (pure.rs:1406-1411)."""
+
+    def __init__(self, rows: int, cols: int, data=None):
+        if data is None:
+            buf = np.zeros(rows * cols, dtype=np.float32)
+        else:
+            buf = np.ascontiguousarray(np.asarray(data, dtype=np.float32)).reshape(-1)
+            if buf.size != rows * cols:
+                raise TensorError("DataLength", f"expected {rows * cols} values, got {buf.size}",
+                                  expected=rows * cols, got=buf.size)
+        self.rows, self.cols = int(rows), int(cols)
+        self._data = buf
+
+    @classmethod
+    def zeros(cls, rows: int, cols: int) -> "Tensor":
+        return cls(rows, cols)
+
+    @classmethod
+    def from_numpy(cls, array) -> "Tensor":
+        a = np.asarray(array, dtype=np.float32)
+        if a.ndim != 2:
+            raise TensorError("InvalidDimensions", "expected a 2-D array", rows=a.ndim, cols=2)
+        return cls(a.shape[0], a.shape[1], a)
+
+    def shape(self) -> Tuple[int, int]:
+        return (self.rows, self.cols)
+
+    def data(self) -> np.ndarray:
+        return self._data
+
+    def numpy(self) -> np.ndarray:
+        return self._data.reshape(self.rows, self.cols)
+
+    # ---- dense matmul family ---------------------------------------------------------------------
+    def _check_inner(self, other: "Tensor") -> None:
+        if self.cols != other.rows:
+            raise TensorError("ShapeMismatch", f"left {self.shape()} right {other.shape()}",
+                              left=self.shape(), right=other.shape())
+
+    def matmul(self, other: "Tensor", *, backend: Optional[str] = None) -> "Tensor":
+        """C = A·B — Tensor::matmul_with_backend, pure.rs:2013-2197."""
+        return self.matmul_scaled(other, 1.0, backend=backend, _op="matmul")
+
+    def matmul_scaled(self, other: "Tensor", scale: float, *, backend: Optional[str] = None,
+                      _op: str = "matmul_scaled") -> "Tensor":
+        """C = (A·B)·scale — pure.rs:2200-2369."""
+        _resolve_backend(backend)
+        self._check_inner(other)
+        out = Tensor.zeros(self.rows, other.cols)
+        try:
+            hip.gemm_scaled_f32(self.rows, other.cols, self.cols, scale, self._data, other._data, out._data)
+        except hip.HipErr as err:
+            raise _backend_failure(err) from err
+        _validate_finite(f"{_op}_output", out._data)  # pure.rs:2169
+        return out
+
+    def matmul_lhs_transpose_scaled(self, other: "Tensor", scale: float, *,
+                                    backend: Optional[str] = None) -> "Tensor":
+        """C = (Aᵀ·B)·scale with A stored (k, m) — pure.rs:2372-2556."""
+        _resolve_backend(backend)
+        if self.rows != other.rows:
+            raise TensorError("ShapeMismatch", f"left {self.shape()} right {other.shape()}",
+                              left=self.shape(), right=other.shape())
+        out = Tensor.zeros(self.cols, other.cols)
+        try:
+            hip.gemm_lhs_transpose_scaled_f32(self.cols, other.cols, self.rows, scale, self._data, other._data,
+                                              out._data)
+        except hip.HipErr as err:
+            raise _backend_failure(err) from err
+        _validate_finite("matmul_lhs_transpose_scaled_output", out._data)
+        return out
+
+    def _fused(self, other: "Tensor", bias, residual: Optional["Tensor"], activation, label: str) -> "Tensor":
+        self._check_inner(other)
+        bias = np.ascontiguousarray(np.asarray(bias, dtype=np.float32)).reshape(-1)
+        if bias.size != other.cols:
+            raise TensorError("DataLength", f"expected {other.cols} values, got {bias.size}",
+                              expected=other.cols, got=bias.size)
+        if residual is not None and residual.shape() != (self.rows, other.cols):
+            raise TensorError("ShapeMismatch", f"left {residual.shape()} right {(self.rows, other.cols)}",
+                              left=residual.shape(), right=(self.rows, other.cols))
+        out = Tensor.zeros(self.rows, other.cols)
+        try:
+            hip.gemm_bias_activation_f32(self.rows, other.cols, self.cols, activation, self._data, other._data, bias,
+                                         None if residual is None else residual._data, out._data)
+        except hip.HipErr as err:
+            raise _backend_failure(err) from err
+        _validate_finite(label, out._data)  # pure.rs:4537
+        return out
+
+    def matmul_bias_relu(self, other: "Tensor", bias, *, backend: Optional[str] = None) -> "Tensor":
+        """relu(A·B + bias) — pure.rs:4411-4550."""
+        _resolve_backend(backend)
+        return self._fused(other, bias, None, hip.GemmActivation.Relu, "matmul_bias_relu_output")
+
+    def matmul_bias_gelu(self, other: "Tensor", bias, *, backend: Optional[str] = None) -> "Tensor":
+        _resolve_backend(backend)
+        return self._fused(other, bias, None, hip.GemmActivation.Gelu, "matmul_bias_gelu_output")
+
+    def matmul_bias_add_relu(self, other: "Tensor", bias, residual: "Tensor", *,
+                             backend: Optional[str] = None) -> "Tensor":
+        _resolve_backend(backend)
+        return self._fused(other, bias, residual, hip.GemmActivation.Relu, "matmul_bias_add_relu_output")
+
+    def matmul_bias_add_gelu(self, other: "Tensor", bias, residual: "Tensor", *,
+                             backend: Optional[str] = None) -> "Tensor":
+        _resolve_backend(backend)
+        return self._fused(other, bias, residual, hip.GemmActivation.Gelu, "matmul_bias_add_gelu_output")
+
+    # ---- attention -------------------------------------------------------------------------------
+    def scaled_dot_attention(self, keys: "Tensor", values: "Tensor", *, contexts: int, sequence: int,
+                             scale: float, z_bias: Optional["Tensor"] = None,
+                             attn_bias: Optional["Tensor"] = None, causal: bool = False,
+                             backend: Optional[str] = None) -> "Tensor":
+        """softmax(QKᵀ·scale + biases)·V per context — pure.rs:4083-4354.  `causal` is this build's
+        addition (keys 0..=query, crates/st-core/src/backend/cuda_attention.cu:160-164)."""
+        _resolve_backend(backend)
+        expected_rows = contexts * sequence
+        for t in (self, keys, values):
+            if t.rows != expected_rows or t.cols != self.cols:
+                raise TensorError("ShapeMismatch", f"left {t.shape()} right {(expected_rows, self.cols)}",
+                                  left=t.shape(), right=(expected_rows, self.cols))
+        if z_bias is not None and z_bias.shape() != (contexts, sequence):
+            raise TensorError("ShapeMismatch", f"left {z_bias.shape()} right {(contexts, sequence)}",
+                              left=z_bias.shape(), right=(contexts, sequence))
+        if attn_bias is not None and attn_bias.shape() != (expected_rows, sequence):
+            raise TensorError("ShapeMismatch", f"left {attn_bias.shape()} right {(expected_rows, sequence)}",
+                              left=attn_bias.shape(), right=(expected_rows, sequence))
+        out = Tensor.zeros(expected_rows, self.cols)
+        try:
+            hip.attention_f32(contexts, sequence, self.cols, scale, causal, self._data, keys._data, values._data,
+                              None if z_bias is None else z_bias._data,
+                              None if attn_bias is None else attn_bias._data, out._data)
+        except hip.HipErr as err:
+            raise _backend_failure(err) from err
+        return out
+
+
+class Conv2d:
+    """Conv2d layer of crates/st-nn/src/layers/conv.rs:607-969 (forward only), with the optional fused
+    activation the reference composes as a separate Relu layer."""
+
+    def __init__(self, name: str, in_channels: int, out_channels: int, kernel, stride, padding, dilation,
+                 input_hw, activation: int = hip.ACT_NONE):
+        self.name = name
+        self.in_channels, self.out_channels = int(in_channels), int(out_channels)
+        self.kernel, self.stride = tuple(kernel), tuple(stride)
+        self.padding, self.dilation = tuple(padding), tuple(dilation)
+        self.input_hw = tuple(input_hw)
+        self.activation = activation
+        for value, label in ((in_channels, "in_channels"), (out_channels, "out_channels"),
+                             (self.kernel[0], "kernel_h"), (self.kernel[1], "kernel_w"),
+                             (self.stride[0], "stride_h"), (self.stride[1], "stride_w"),
+                             (self.dilation[0], "dilation_h"), (self.dilation[1], "dilation_w"),
+                             (self.input_hw[0], "input_height"), (self.input_hw[1], "input_width")):
+            if value <= 0:
+                raise TensorError("InvalidDimensions", f"{label} must be positive", rows=value, cols=0)
+        span = self.in_channels * self.kernel[0] * self.kernel[1]
+        # Deterministic default weight ramp and zero bias of Conv2d::new (conv.rs:641-649).
+        seed = np.float32(0.02)
+        ramp = np.empty(self.out_channels * span, dtype=np.float32)
+        for i in range(ramp.size):
+            ramp[i] = seed
+            seed = np.float32(max(np.fmod(np.float32(seed * np.float32(1.57)), np.float32(0.15)), np.float32(5e-3)))
+        self.weight = Tensor(self.out_channels, span, ramp)
+        self.bias = Tensor.zeros(1, self.out_channels)
+        self.output_hw()  # validates the configuration once (conv.rs:662)
+
+    def output_hw(self) -> Tuple[int, int]:
+        try:
+            return hip.conv2d_output_hw(self.input_hw[0], self.input_hw[1], self.kernel, self.stride, self.padding,
+                                        self.dilation)
+        except hip.HipErr as err:
+            raise TensorError("InvalidDimensions", err.message) from err
+
+    def forward(self, input: Tensor) -> Tensor:
+        h, w = self.input_hw
+        if input.cols != self.in_channels * h * w:
+            raise TensorError("ShapeMismatch", f"left {input.shape()} right {(input.rows, self.in_channels * h * w)}",
+                              left=input.shape(), right=(input.rows, self.in_channels * h * w))
+        oh, ow = self.output_hw()
+        out = Tensor.zeros(input.rows, self.out_channels * oh * ow)
+        try:
+            hip.conv2d_bias_activation_f32(input.rows, self.in_channels, h, w, self.out_channels, self.kernel,
+                                           self.stride, self.padding, self.dilation, self.activation, input.data(),
+                                           self.weight.data(), self.bias.data(), out.data())
+        except hip.HipErr as err:
+            raise _backend_failure(err) from err
+        return out

@@ -1,0 +1,150 @@
+"""Parity of the flash-style attention kernel against the CPU oracle (1e-4 rel / 1e-5 abs, row sums)."""
+import numpy as np
+import pytest
+
+from conftest import F32_ABS, F32_REL, assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+def run(hip, contexts, seq, dim, scale, q, k, v, zb=None, ab=None, causal=False):
+    out = np.zeros(contexts * seq * dim, np.float32)
+    hip.attention_f32(contexts, seq, dim, scale, causal, q, k, v, zb, ab, out)
+    return out
+
+
+def test_reference_vectors(hip, oracle, golden):
+    for c in golden["attention"]:
+        f = lambda name: None if c[name] is None else np.array(c[name], np.float32)
+        got = run(hip, c["contexts"], c["sequence"], c["head_dim"], c["scale"], f("q"), f("k"), f("v"), f("z_bias"),
+                  f("attn_bias"))
+        want = oracle.attention_f64(c["contexts"], c["sequence"], c["head_dim"], c["scale"], c["q"], c["k"], c["v"],
+                                    c["z_bias"], c["attn_bias"])
+        assert_close(got, want, 0, c["tolerance"], c["source"])
+
+
+CASES = [
+    # contexts, seq, dim, causal, biased
+    (1, 1, 1, False, False), (2, 7, 3, False, False), (3, 33, 8, True, False), (2, 19, 5, False, True),
+    (1, 40, 16, True, True), (4, 64, 64, False, False), (2, 129, 64, True, False), (3, 200, 32, False, False),
+    (2, 257, 64, False, True), (1, 300, 128, True, False), (1, 130, 80, False, False), (2, 96, 256, True, False),
+    (1, 70, 200, False, True), (5, 128, 64, True, True), (8, 384, 64, True, False),
+]
+
+
+@pytest.mark.parametrize("contexts,seq,dim,causal,biased", CASES)
+def test_random_cases(hip, oracle, contexts, seq, dim, causal, biased):
+    rng = np.random.default_rng(contexts * 1000 + seq * 7 + dim)
+    q, k, v = (rng.normal(size=contexts * seq * dim).astype(np.float32) for _ in range(3))
+    zb = rng.normal(size=contexts * seq).astype(np.float32) if biased else None
+    ab = rng.normal(size=contexts * seq * seq).astype(np.float32) if biased else None
+    scale = float(1.0 / np.sqrt(dim))
+    got = run(hip, contexts, seq, dim, scale, q, k, v, zb, ab, causal)
+    want = oracle.attention_f32(contexts, seq, dim, scale, q, k, v, zb, ab, causal, threads=8)
+    assert_close(got, want, F32_REL, F32_ABS, f"attention {contexts}x{seq}x{dim} causal={causal} bias={biased}")
+    # softmax row sums: V = 1 must give exactly-normalised rows
+    ones = run(hip, contexts, seq, dim, scale, q, k, np.ones_like(v), zb, ab, causal)
+    assert_close(ones, np.ones_like(ones), F32_REL, F32_ABS, "row sums")
+
+
+def test_invariants(hip, oracle):
+    rng = np.random.default_rng(5)
+    contexts, seq, dim = 3, 150, 64
+    q, k, v = (rng.normal(size=contexts * seq * dim).astype(np.float32) for _ in range(3))
+    vv = v.reshape(contexts, seq, dim).astype(np.float64)
+    mean = run(hip, contexts, seq, dim, 0.125, np.zeros_like(q), k, v)
+    assert_close(mean, np.repeat(vv.mean(axis=1, keepdims=True), seq, axis=1), F32_REL, F32_ABS, "column means")
+    prefix = run(hip, contexts, seq, dim, 0.125, np.zeros_like(q), k, v, causal=True)
+    assert_close(prefix, np.cumsum(vv, axis=1) / np.arange(1, seq + 1).reshape(1, seq, 1), F32_REL, F32_ABS,
+                 "prefix means")
+    causal = run(hip, contexts, seq, dim, 0.125, q, k, v, causal=True).reshape(contexts, seq, dim)
+    assert_close(causal[:, 0, :], v.reshape(contexts, seq, dim)[:, 0, :], 1e-6, 1e-6, "causal row 0 is V[0]")
+    # the causal flag equals the reference's way of masking: a large negative additive bias
+    bias = np.where(np.triu(np.ones((seq, seq), bool), 1), np.float32(-1e30), np.float32(0))
+    bias = np.ascontiguousarray(np.tile(bias.reshape(1, seq, seq), (contexts, 1, 1)), np.float32).ravel()
+    masked = run(hip, contexts, seq, dim, 0.125, q, k, v, ab=bias)
+    assert_close(masked, causal, F32_REL, F32_ABS, "causal == -1e30 bias")
+
+
+def test_empty_and_validation(hip):
+    out = np.zeros(0, np.float32)
+    e = np.zeros(0, np.float32)
+    hip.attention_f32(0, 5, 4, 1.0, False, e, e, e, None, None, out)
+    hip.attention_f32(3, 5, 0, 1.0, False, e, e, e, None, None, out)
+    q = np.ones(8, np.float32)
+    keep = np.full(8, 13.0, np.float32)
+    with pytest.raises(hip.HipErr, match="key buffer length"):
+        hip.attention_f32(1, 4, 2, 1.0, False, q, q[:-1], q, None, None, keep)
+    with pytest.raises(hip.HipErr, match="z_bias buffer length"):
+        hip.attention_f32(1, 4, 2, 1.0, False, q, q, q, np.zeros(3, np.float32), None, keep)
+    with pytest.raises(hip.HipErr, match="attn_bias buffer length"):
+        hip.attention_f32(1, 4, 2, 1.0, False, q, q, q, None, np.zeros(15, np.float32), keep)
+    with pytest.raises(hip.HipErr, match="scaled_dot_attention_scale"):
+        hip.attention_f32(1, 4, 2, float("nan"), False, q, q, q, None, None, keep)
+    bad = q.copy()
+    bad[3] = np.inf
+    with pytest.raises(hip.HipErr, match="scaled_dot_attention_key"):
+        hip.attention_f32(1, 4, 2, 1.0, False, q, bad, q, None, None, keep)
+    with pytest.raises(hip.HipErr, match="head_dim 300 exceeds"):
+        hip.attention_f32(1, 1, 300, 1.0, False, np.ones(300, np.float32), np.ones(300, np.float32),
+                          np.ones(300, np.float32), None, None, np.zeros(300, np.float32))
+    assert (keep == 13.0).all()
+
+
+def test_overflow_is_reported_as_nonfinite(hip, golden):
+    """crates/st-tensor/src/pure.rs:15365-15389: q = f32::MAX, k = 2 overflows.  The CPU path names the
+    first overflowing intermediate (…_dot); the GPU path reports the non-finite output (…_output)."""
+    from spiraltorch_amd import Tensor, TensorError
+    q = Tensor(1, 1, [np.finfo(np.float32).max])
+    with pytest.raises(TensorError) as err:
+        q.scaled_dot_attention(Tensor(1, 1, [2.0]), Tensor(1, 1, [1.0]), contexts=1, sequence=1, scale=1.0)
+    assert err.value.kind == "NonFiniteValue"
+    assert err.value.fields["label"] == "scaled_dot_attention_output"
+
+
+def test_tensor_mirror(hip, oracle, golden):
+    from spiraltorch_amd import Tensor, TensorError
+    c = golden["attention"][1]
+    q, k, v = (Tensor(2, 2, c[name]) for name in ("q", "k", "v"))
+    out = q.scaled_dot_attention(k, v, contexts=1, sequence=2, scale=1.0, z_bias=Tensor(1, 2, c["z_bias"]),
+                                 attn_bias=Tensor(2, 2, c["attn_bias"]), backend="hip")
+    want = oracle.attention_f64(1, 2, 2, 1.0, c["q"], c["k"], c["v"], c["z_bias"], c["attn_bias"])
+    assert out.shape() == (2, 2)
+    assert_close(out.data(), want, 0, 1e-5, "Tensor.scaled_dot_attention")
+    with pytest.raises(TensorError) as err:
+        q.scaled_dot_attention(k, Tensor(3, 2), contexts=1, sequence=2, scale=1.0)
+    assert err.value.kind == "ShapeMismatch"
+
+
+def test_config3_full_size(hip, oracle):
+    """BASELINE config 3: B8 H16 S2048 D64 (128 contexts), scale 1/8, non-causal and causal.
+    The oracle checks three whole contexts per mode; every context is covered by the row-sum check
+    (V = 1) and by context-permutation equivariance."""
+    from spiraltorch_amd import inputs
+    contexts, seq, dim = 128, 2048, 64
+    count = contexts * seq * dim
+    q = inputs.normal(inputs.seed_for(3, 0), count)
+    k = inputs.normal(inputs.seed_for(3, 1), count)
+    v = inputs.normal(inputs.seed_for(3, 2), count)
+    d_q, d_k, d_v = (hip.DeviceBuffer.from_array(a) for a in (q, k, v))
+    d_ones = hip.DeviceBuffer.from_array(np.ones(count, np.float32))
+    d_out = hip.DeviceBuffer(count * 4)
+    per = seq * dim
+    for causal in (False, True):
+        hip.attention_f32_dev(contexts, seq, dim, 0.125, causal, d_q, d_k, d_v, None, None, d_out)
+        hip.device_synchronize()
+        got = d_out.to_array(np.float32, (contexts, per))
+        for ctx in (0, 77, 127):
+            sl = slice(ctx * per, (ctx + 1) * per)
+            want = oracle.attention_f32(1, seq, dim, 0.125, q[sl], k[sl], v[sl], causal=causal)
+            assert_close(got[ctx], want, F32_REL, F32_ABS, f"config 3 causal={causal} context {ctx}")
+        hip.attention_f32_dev(contexts, seq, dim, 0.125, causal, d_q, d_k, d_ones, None, None, d_out)
+        hip.device_synchronize()
+        sums = d_out.to_array(np.float32, count)
+        assert_close(sums, np.ones(count), F32_REL, F32_ABS, f"config 3 causal={causal} row sums")
+        # contexts are independent: reversing their order reverses the output blocks bit for bit
+        rev = lambda a: np.ascontiguousarray(a.reshape(contexts, per)[::-1])
+        d_qr, d_kr, d_vr = (hip.DeviceBuffer.from_array(rev(a)) for a in (q, k, v))
+        hip.attention_f32_dev(contexts, seq, dim, 0.125, causal, d_qr, d_kr, d_vr, None, None, d_out)
+        hip.device_synchronize()
+        assert (d_out.to_array(np.float32, (contexts, per)) == got[::-1]).all()

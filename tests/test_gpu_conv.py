@@ -1,0 +1,126 @@
+"""Parity of the fused implicit-GEMM conv2d (+bias, +activation) against the CPU oracle."""
+import numpy as np
+import pytest
+
+from conftest import F32_ABS, F32_REL, assert_close
+from test_oracle_conv import generated_case
+
+pytestmark = pytest.mark.gpu
+
+
+def run(hip, batch, c_in, h, w, c_out, kernel, stride, padding, dilation, act, x, wt, b):
+    oh, ow = hip.conv2d_output_hw(h, w, kernel, stride, padding, dilation)
+    out = np.zeros(batch * c_out * oh * ow, np.float32)
+    hip.conv2d_bias_activation_f32(batch, c_in, h, w, c_out, kernel, stride, padding, dilation, act,
+                                   np.ascontiguousarray(x, np.float32).ravel(),
+                                   np.ascontiguousarray(wt, np.float32).ravel(), b, out)
+    return out
+
+
+def test_layout_known_answer(hip, golden):
+    c = golden["conv_layout"]
+    out = run(hip, c["batch"], c["c_in"], *c["input_hw"], c["c_out"], c["kernel"], c["stride"], c["padding"],
+              c["dilation"], 0, np.array(c["input"], np.float32), np.array(c["weight"], np.float32),
+              np.array(c["bias"], np.float32))
+    assert out.tolist() == c["expected"]
+
+
+def test_output_hw(hip, golden):
+    for c in golden["conv_output_hw"]:
+        assert list(hip.conv2d_output_hw(*c["input_hw"], c["kernel"], c["stride"], c["padding"],
+                                         c["dilation"])) == c["expected"]
+    with pytest.raises(hip.HipErr):
+        hip.conv2d_output_hw(2, 2, (5, 5), (1, 1), (0, 0), (1, 1))
+
+
+def test_reference_generated_cases(hip, oracle, golden):
+    for case in golden["conv_generated"]:
+        x, weight, bias = generated_case(case)
+        h, w = case["input_hw"]
+        args = (case["batch"], case["c_in"], h, w, case["c_out"], case["kernel"], case["stride"], case["padding"],
+                case["dilation"])
+        got = run(hip, *args, 0, x, weight, bias)
+        want = oracle.conv2d_bias_act_f32(*args, oracle.ACT_NONE, x, weight, bias)
+        assert_close(got, want, 0, case["tolerance"], case["source"])
+
+
+@pytest.mark.parametrize("shape", [
+    (2, 3, 9, 7, 4, (3, 3), (1, 1), (1, 1), (1, 1)),
+    (1, 2, 9, 9, 3, (3, 3), (1, 1), (0, 0), (2, 2)),
+    (3, 5, 6, 11, 7, (2, 4), (2, 3), (1, 2), (1, 1)),
+    (2, 4, 5, 5, 6, (1, 1), (1, 1), (0, 0), (1, 1)),
+    (1, 1, 4, 4, 1, (4, 4), (1, 1), (0, 0), (1, 1)),
+    (2, 16, 20, 20, 70, (3, 3), (1, 1), (1, 1), (1, 1)),
+    (1, 8, 33, 17, 130, (5, 3), (2, 1), (2, 1), (1, 2)),
+    (5, 7, 12, 12, 64, (3, 3), (2, 2), (0, 0), (1, 1)),
+])
+def test_random_shapes(hip, oracle, shape):
+    batch, c_in, h, w, c_out, kernel, stride, padding, dilation = shape
+    rng = np.random.default_rng(abs(hash(shape)) % 2 ** 32)
+    x = rng.normal(size=batch * c_in * h * w).astype(np.float32)
+    wt = rng.normal(0, np.sqrt(2.0 / (c_in * kernel[0] * kernel[1])), c_out * c_in * kernel[0] * kernel[1]).astype(np.float32)
+    b = rng.uniform(-0.1, 0.1, c_out).astype(np.float32)
+    for act, code in ((0, oracle.ACT_NONE), (1, oracle.ACT_RELU), (2, oracle.ACT_GELU)):
+        got = run(hip, *shape, act, x, wt, b)
+        want = oracle.conv2d_bias_act_f32(*shape, code, x, wt, b)
+        assert_close(got, want, F32_REL, F32_ABS, f"conv {shape} act={act}")
+    got = run(hip, *shape, 1, x, wt, None)
+    assert_close(got, oracle.conv2d_bias_act_f32(*shape, oracle.ACT_RELU, x, wt, None), F32_REL, F32_ABS, "no bias")
+
+
+def test_conv2d_layer_mirror(hip, oracle):
+    from spiraltorch_amd import Conv2d, Tensor, TensorError
+    conv = Conv2d("conv_gpu", 3, 8, (3, 3), (1, 1), (1, 1), (1, 1), (8, 8))
+    assert conv.output_hw() == (8, 8)
+    assert conv.bias.data().tolist() == [0.0] * 8
+    x = Tensor(4, 3 * 8 * 8, np.random.default_rng(0).normal(size=4 * 192))
+    got = conv.forward(x)
+    want = oracle.conv2d_bias_act_f32(4, 3, 8, 8, 8, (3, 3), (1, 1), (1, 1), (1, 1), oracle.ACT_NONE, x.data(),
+                                      conv.weight.data(), conv.bias.data())
+    assert got.shape() == (4, 8 * 8 * 8)
+    assert_close(got.data(), want, F32_REL, F32_ABS, "Conv2d.forward")
+    with pytest.raises(TensorError):
+        conv.forward(Tensor(4, 10))
+    with pytest.raises(TensorError):
+        Conv2d("bad", 1, 1, (5, 5), (1, 1), (0, 0), (1, 1), (2, 2))
+    empty = conv.forward(Tensor(0, 192))
+    assert empty.shape() == (0, 512)  # conv.rs:4132-4137
+
+
+def test_validation_before_mutation(hip):
+    out = np.full(2 * 4 * 4 * 4, 13.0, np.float32)
+    x = np.zeros(2 * 3 * 4 * 4, np.float32)
+    w = np.zeros(4 * 3 * 3 * 3, np.float32)
+    args = (2, 3, 4, 4, 4, (3, 3), (1, 1), (1, 1), (1, 1), 1)
+    with pytest.raises(hip.HipErr, match="input buffer length"):
+        hip.conv2d_bias_activation_f32(*args, x[:-1], w, None, out)
+    with pytest.raises(hip.HipErr, match="weight buffer length"):
+        hip.conv2d_bias_activation_f32(*args, x, w[:-1], None, out)
+    with pytest.raises(hip.HipErr, match="bias buffer length 3 does not match c_out=4"):
+        hip.conv2d_bias_activation_f32(*args, x, w, np.zeros(3, np.float32), out)
+    with pytest.raises(hip.HipErr, match="output buffer length"):
+        hip.conv2d_bias_activation_f32(*args, x, w, None, out[:-1])
+    with pytest.raises(hip.HipErr, match="unknown activation"):
+        hip.conv2d_bias_activation_f32(*args[:-1], 7, x, w, None, out)
+    assert (out == 13.0).all()
+
+
+def test_config2_full_size(hip, oracle):
+    """BASELINE config 2: N32 C64->128 56x56 3x3 s1 p1, bias + ReLU.  The oracle checks two whole images
+    (first and last); all 32 are covered by batch-permutation equivariance and by exact 2x linearity."""
+    from spiraltorch_amd import inputs
+    batch, c_in, h, w, c_out = 32, 64, 56, 56, 128
+    x = inputs.normal(inputs.seed_for(2, 0), batch * c_in * h * w)
+    wt = inputs.normal(inputs.seed_for(2, 1), c_out * c_in * 9, 0.0, float(np.sqrt(2.0 / (c_in * 9))))
+    b = inputs.uniform(inputs.seed_for(2, 2), c_out, -0.1, 0.1)
+    geom = ((3, 3), (1, 1), (1, 1), (1, 1))
+    got = run(hip, batch, c_in, h, w, c_out, *geom, 1, x, wt, b).reshape(batch, -1)
+    xi = x.reshape(batch, -1)
+    for image in (0, 31):
+        want = oracle.conv2d_bias_act_f32(1, c_in, h, w, c_out, *geom, oracle.ACT_RELU, xi[image], wt, b, threads=8)
+        assert_close(got[image], want, F32_REL, F32_ABS, f"config 2 image {image}")
+    perm = np.random.default_rng(2).permutation(batch)
+    got_perm = run(hip, batch, c_in, h, w, c_out, *geom, 1, xi[perm], wt, b).reshape(batch, -1)
+    assert (got_perm == got[perm]).all()
+    doubled = run(hip, batch, c_in, h, w, c_out, *geom, 1, 2 * x, wt, 2 * b).reshape(batch, -1)
+    assert (doubled == 2 * got).all()

@@ -1,0 +1,103 @@
+"""Row-wise operators and the decoder stack against the CPU oracle."""
+import numpy as np
+import pytest
+
+from conftest import BF16_REL, F32_ABS, F32_REL, assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+def test_layer_norm(hip, oracle):
+    from spiraltorch_amd import inputs
+    rng = np.random.default_rng(4)
+    for rows, cols in ((1, 1), (5, 48), (130, 512), (7, 1000)):
+        x = rng.normal(1.0, 2.0, rows * cols).astype(np.float32)
+        res = rng.normal(size=rows * cols).astype(np.float32)
+        g, b = rng.normal(size=cols).astype(np.float32), rng.normal(size=cols).astype(np.float32)
+        d = {n: hip.DeviceBuffer.from_array(a) for n, a in (("x", x), ("r", res), ("g", g), ("b", b))}
+        o32, o16 = hip.DeviceBuffer(rows * cols * 4), hip.DeviceBuffer(rows * cols * 2)
+        for residual, dr in ((None, None), (res, d["r"])):
+            hip.layer_norm_f32_dev(rows, cols, d["x"], dr, d["g"], d["b"], 1e-5, o32, o16)
+            hip.device_synchronize()
+            got = o32.to_array(np.float32, rows * cols)
+            assert_close(got, oracle.layer_norm_f32(rows, cols, x, g, b, 1e-5, residual), F32_REL, 2e-5, "layer norm")
+            assert (o16.to_array(np.uint16, rows * cols) == inputs.to_bf16(got)).all()
+
+
+def test_embedding_split_merge_and_rounding(hip, oracle):
+    from spiraltorch_amd import inputs
+    table = np.arange(12, dtype=np.float32).reshape(4, 3)
+    ids = np.array([0, 1.4, 1.5, 2.6, 9.0, -3.0, np.nan, np.inf], np.float32)
+    d_out = hip.DeviceBuffer(ids.size * 3 * 4)
+    hip.embedding_f32_dev(ids.size, 4, 3, hip.DeviceBuffer.from_array(ids), hip.DeviceBuffer.from_array(table), d_out)
+    hip.device_synchronize()
+    assert (d_out.to_array(np.float32, ids.size * 3) == oracle.embedding_f32(ids.size, 4, 3, ids, table)).all()
+
+    vals = np.random.default_rng(0).normal(size=1000).astype(np.float32)
+    d16 = hip.DeviceBuffer(2000)
+    hip.f32_to_bf16_dev(1000, hip.DeviceBuffer.from_array(vals), d16)
+    hip.device_synchronize()
+    assert (d16.to_array(np.uint16, 1000) == oracle.f32_to_bf16(vals)).all()
+
+    batch, seq, heads, dim = 2, 5, 3, 4
+    qkv = np.random.default_rng(1).normal(size=(batch, seq, 3, heads, dim)).astype(np.float32)
+    dq, dk, dv = (hip.DeviceBuffer(batch * seq * heads * dim * 4) for _ in range(3))
+    hip.split_heads_f32_dev(batch, seq, heads, dim, hip.DeviceBuffer.from_array(qkv), dq, dk, dv)
+    hip.device_synchronize()
+    for i, buf in enumerate((dq, dk, dv)):
+        want = qkv[:, :, i].transpose(0, 2, 1, 3)
+        assert (buf.to_array(np.float32, want.shape) == want).all()
+    merged = hip.DeviceBuffer(batch * seq * heads * dim * 4)
+    hip.merge_heads_f32_dev(batch, seq, heads, dim, dq, merged, None)
+    hip.device_synchronize()
+    assert (merged.to_array(np.float32, (batch, seq, heads, dim)) == qkv[:, :, 0]).all()
+
+
+def decoder_case(vocab, d, heads, layers, ff, batch, seq, seed):
+    from spiraltorch_amd import hip as hipmod, inputs
+    count = hipmod.Decoder.weight_count(vocab, d, heads, layers, ff)
+    weights = inputs.normal(seed, count, 0.0, 0.02)
+    # layer-norm gains are 1 (+ a small perturbation so a dropped gamma is visible), as in the reference's init
+    return weights, inputs.tokens(seed + 1, batch * seq, vocab)
+
+
+def set_gains(weights, vocab, d, layers, ff):
+    w = weights.copy()
+    pos = vocab * d
+    per_layer = 2 * d + d * 3 * d + 3 * d + d * d + d + 2 * d + d * ff + ff + ff * d + d
+    for _ in range(layers):
+        w[pos:pos + d] += 1.0
+        ln2 = pos + 2 * d + d * 3 * d + 3 * d + d * d + d
+        w[ln2:ln2 + d] += 1.0
+        pos += per_layer
+    w[pos:pos + d] += 1.0
+    return w
+
+
+@pytest.mark.parametrize("cfg", [(32, 16, 2, 2, 24, 2, 9), (256, 128, 2, 2, 256, 2, 160)])
+def test_decoder_matches_the_oracle(hip, oracle, cfg):
+    vocab, d, heads, layers, ff, batch, seq = cfg
+    weights, tokens = decoder_case(*cfg, seed=500)
+    weights = set_gains(weights, vocab, d, layers, ff)
+    assert hip.Decoder.weight_count(vocab, d, heads, layers, ff) == oracle.decoder_weight_count(vocab, d, heads, layers, ff)
+    dec = hip.Decoder(vocab, d, heads, layers, ff, batch, seq, 1e-5, weights)
+    d_tok = hip.DeviceBuffer.from_array(tokens)
+    d_logits = hip.DeviceBuffer(batch * seq * vocab * 4)
+    dec.forward_dev(d_tok, d_logits)
+    hip.device_synchronize()
+    got = d_logits.to_array(np.float32, batch * seq * vocab)
+    want = oracle.decoder_forward(vocab, d, heads, layers, ff, batch, seq, 1e-5, weights, tokens, threads=8)
+    # 2e-2 relative on logits, with the floor at 2e-2 of the logits' RMS for values near zero
+    rms = float(np.sqrt(np.mean(np.square(want))))
+    assert_close(got, want, BF16_REL, BF16_REL * rms, f"decoder {cfg}")
+    # replay is deterministic
+    dec.forward_dev(d_tok, d_logits)
+    hip.device_synchronize()
+    assert (d_logits.to_array(np.float32, batch * seq * vocab) == got).all()
+
+
+def test_decoder_validation(hip):
+    with pytest.raises(hip.HipErr, match="not divisible"):
+        hip.Decoder(32, 10, 3, 1, 8, 1, 4, 1e-5, np.zeros(hip.Decoder.weight_count(32, 10, 3, 1, 8), np.float32))
+    with pytest.raises(hip.HipErr, match="weight buffer length"):
+        hip.Decoder(32, 16, 2, 1, 8, 1, 4, 1e-5, np.zeros(10, np.float32))

@@ -1,0 +1,177 @@
+"""Parity of the HIP f32 GEMM family against the CPU oracle, through the C ABI."""
+import numpy as np
+import pytest
+
+from conftest import F32_ABS, F32_REL, assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+def test_reference_known_answers(hip, golden):
+    for case in golden["gemm"]:
+        out = np.zeros(case["m"] * case["n"], np.float32)
+        lhs, rhs = np.array(case["lhs"], np.float32), np.array(case["rhs"], np.float32)
+        if case["lhs_transposed"]:
+            hip.gemm_lhs_transpose_scaled_f32(case["m"], case["n"], case["k"], case["scale"], lhs, rhs, out)
+        else:
+            hip.gemm_scaled_f32(case["m"], case["n"], case["k"], case["scale"], lhs, rhs, out)
+        assert out.tolist() == case["expected"], case["source"]
+
+
+def test_ones_and_epilogue_known_answers(hip, golden):
+    c = golden["gemm_ones"]
+    lhs = np.full(c["m"] * c["k"], c["lhs_value"], np.float32)
+    rhs = np.full(c["k"] * c["n"], c["rhs_value"], np.float32)
+    out = np.zeros(c["m"] * c["n"], np.float32)
+    hip.gemm_f32(c["m"], c["n"], c["k"], lhs, rhs, out)
+    assert (out == c["expected_value"]).all()
+    hip.gemm_bias_activation_f32(c["m"], c["n"], c["k"], hip.GemmActivation.Relu, lhs, rhs,
+                                 np.full(c["n"], c["bias_value"], np.float32), None, out)
+    assert (out == c["expected_bias_relu_value"]).all()
+
+    e = golden["gemm_epilogue"]
+    lhs, rhs = np.array(e["lhs"], np.float32), np.array(e["rhs"], np.float32)
+    bias, residual = np.array(e["bias"], np.float32), np.array(e["residual"], np.float32)
+    out = np.zeros(4, np.float32)
+    hip.gemm_bias_activation_f32(2, 2, 3, hip.GemmActivation.Relu, lhs, rhs, bias, None, out)
+    assert out.tolist() == e["relu"]
+    hip.gemm_bias_activation_f32(2, 2, 3, hip.GemmActivation.Relu, lhs, rhs, bias, residual, out)
+    assert out.tolist() == e["residual_relu"]
+    gelu64 = lambda x: 0.5 * x * (1.0 + np.tanh(np.sqrt(2.0 / np.pi) * (x + 0.044715 * x ** 3)))
+    for res, pre in ((None, e["gelu_pre_activation"]), (residual, e["residual_gelu_pre_activation"])):
+        hip.gemm_bias_activation_f32(2, 2, 3, hip.GemmActivation.Gelu, lhs, rhs, bias, res, out)
+        np.testing.assert_allclose(out, gelu64(np.array(pre, np.float64)), atol=2e-5, rtol=1e-6)
+
+
+def test_zero_inner_runs_the_epilogue(hip, golden):
+    c = golden["gemm_zero_inner"]
+    out = np.full(4, 99.0, np.float32)
+    hip.gemm_bias_activation_f32(2, 2, 0, hip.GemmActivation.Relu, np.zeros(0, np.float32), np.zeros(0, np.float32),
+                                 np.array(c["bias"], np.float32), np.array(c["residual"], np.float32), out)
+    assert out.tolist() == c["expected_relu"]
+    plain = np.full(4, 99.0, np.float32)
+    hip.gemm_f32(2, 2, 0, np.zeros(0, np.float32), np.zeros(0, np.float32), plain)
+    assert (plain == 0).all()
+
+
+def test_validation_happens_before_mutation(hip):
+    # crates/st-backend-hip/src/lib.rs:1236-1277,1310-1326
+    lhs, rhs = np.array([1, 2, 3, 4], np.float32), np.array([5, 6, 7, 8], np.float32)
+    out = np.full(4, 13.0, np.float32)
+    with pytest.raises(hip.HipErr, match="bias buffer length 1 does not match n=2"):
+        hip.gemm_bias_activation_f32(2, 2, 2, hip.GemmActivation.Relu, lhs, rhs, np.ones(1, np.float32), None, out)
+    with pytest.raises(hip.HipErr, match="residual buffer length 1 does not match m\\*n=4"):
+        hip.gemm_bias_activation_f32(2, 2, 2, hip.GemmActivation.Gelu, lhs, rhs, np.ones(2, np.float32),
+                                     np.ones(1, np.float32), out)
+    with pytest.raises(hip.HipErr, match="scale must be finite, received inf"):
+        hip.gemm_scaled_f32(2, 2, 2, float("inf"), lhs, rhs, out)
+    with pytest.raises(hip.HipErr, match="lhs buffer length 4 does not match m\\*k=6"):
+        hip.gemm_f32(2, 2, 3, lhs, rhs, out)
+    with pytest.raises(hip.HipErr, match="rhs buffer length 4 does not match k\\*n=6"):
+        hip.gemm_f32(2, 3, 2, lhs, rhs, np.zeros(6, np.float32))
+    with pytest.raises(hip.HipErr, match="output buffer length 4 does not match m\\*n=2"):
+        hip.gemm_f32(1, 2, 2, lhs[:2], rhs, out)
+    with pytest.raises(hip.HipErr, match="overflow"):
+        hip.gemm_f32(2 ** 40, 2 ** 40, 2, lhs, rhs, out)
+    assert (out == 13.0).all()
+
+
+def test_empty_output_is_a_no_op(hip):
+    hip.gemm_f32(0, 5, 3, np.zeros(0, np.float32), np.zeros(15, np.float32), np.zeros(0, np.float32))
+    hip.gemm_f32(4, 0, 3, np.zeros(12, np.float32), np.zeros(0, np.float32), np.zeros(0, np.float32))
+
+
+SHAPES = [(1, 1, 1), (2, 3, 4), (8, 12, 7), (10, 13, 9), (8, 16, 6), (4, 16, 5), (33, 65, 17), (64, 64, 64),
+          (100, 130, 70), (129, 127, 31), (256, 64, 200), (5, 300, 19), (300, 5, 23)]
+
+
+@pytest.mark.parametrize("m,n,k", SHAPES)
+def test_random_shapes_match_the_oracle(hip, oracle, m, n, k):
+    rng = np.random.default_rng(m * 7919 + n * 31 + k)
+    a = rng.uniform(-1, 1, m * k).astype(np.float32)
+    b = rng.uniform(-1, 1, k * n).astype(np.float32)
+    out = np.zeros(m * n, np.float32)
+    hip.gemm_f32(m, n, k, a, b, out)
+    assert_close(out, oracle.gemm_f32(m, n, k, a, b), F32_REL, F32_ABS, f"gemm {m}x{n}x{k}")
+    hip.gemm_scaled_f32(m, n, k, -0.37, a, b, out)
+    assert_close(out, oracle.gemm_f32(m, n, k, a, b, scale=-0.37), F32_REL, F32_ABS, "scaled")
+    at = np.ascontiguousarray(a.reshape(m, k).T).ravel()
+    hip.gemm_lhs_transpose_scaled_f32(m, n, k, 0.5, at, b, out)
+    assert_close(out, oracle.gemm_f32(m, n, k, at, b, scale=0.5, lhs_transposed=True), F32_REL, F32_ABS, "lhs^T")
+    bias = rng.uniform(-1, 1, n).astype(np.float32)
+    res = rng.uniform(-1, 1, m * n).astype(np.float32)
+    for act, code in ((hip.GemmActivation.Relu, oracle.ACT_RELU), (hip.GemmActivation.Gelu, oracle.ACT_GELU)):
+        hip.gemm_bias_activation_f32(m, n, k, act, a, b, bias, None, out)
+        assert_close(out, oracle.gemm_bias_act_f32(m, n, k, code, a, b, bias), F32_REL, F32_ABS, f"bias+{act.name}")
+        hip.gemm_bias_activation_f32(m, n, k, act, a, b, bias, res, out)
+        assert_close(out, oracle.gemm_bias_act_f32(m, n, k, code, a, b, bias, res), F32_REL, F32_ABS,
+                     f"bias+residual+{act.name}")
+
+
+def test_config1_512_cubed(hip, oracle):
+    """BASELINE config 1: f32 C = A.B, M=N=K=512, U[-1,1) from the fixed seeds."""
+    from spiraltorch_amd import inputs
+    a = inputs.uniform(inputs.seed_for(1, 0), 512 * 512, -1.0, 1.0)
+    b = inputs.uniform(inputs.seed_for(1, 1), 512 * 512, -1.0, 1.0)
+    out = np.zeros(512 * 512, np.float32)
+    hip.gemm_f32(512, 512, 512, a, b, out)
+    assert_close(out, oracle.gemm_f32(512, 512, 512, a, b, threads=8), F32_REL, F32_ABS, "config 1")
+
+
+def test_large_tile_path_and_linearity(hip, oracle):
+    """Shapes that select the 128x128 tile (>= 256 tiles), checked on sampled rows and by linearity."""
+    rng = np.random.default_rng(99)
+    m, n, k = 2048, 2048, 160
+    a = rng.uniform(-1, 1, m * k).astype(np.float32)
+    b = rng.uniform(-1, 1, k * n).astype(np.float32)
+    out = np.zeros(m * n, np.float32)
+    hip.gemm_f32(m, n, k, a, b, out)
+    rows = [0, 1, 127, 128, 1000, 2047]
+    want = oracle.gemm_f32(len(rows), n, k, a.reshape(m, k)[rows].ravel(), b)
+    assert_close(out.reshape(m, n)[rows], want, F32_REL, F32_ABS, "sampled rows")
+    # size-independent property: (2A).B == 2(A.B) exactly (power-of-two scaling commutes with rounding)
+    out2 = np.zeros(m * n, np.float32)
+    hip.gemm_f32(m, n, k, 2 * a, b, out2)
+    assert (out2 == 2 * out).all()
+
+
+def test_tensor_mirror_matches_the_reference_api(hip, oracle):
+    from spiraltorch_amd import Tensor, TensorError
+    a = Tensor(2, 3, [1, 2, 3, 4, 5, 6])
+    b = Tensor(3, 2, [7, 8, 9, 10, 11, 12])
+    assert a.matmul(b, backend="hip").data().tolist() == [58, 64, 139, 154]
+    assert a.matmul(b).shape() == (2, 2)
+    assert a.matmul_scaled(b, 0.5, backend="hip").data().tolist() == [29, 32, 69.5, 77]
+    at = Tensor(3, 2, [1, 4, 2, 5, 3, 6])
+    assert at.matmul_lhs_transpose_scaled(b, 1.0, backend="hip").data().tolist() == [58, 64, 139, 154]
+    assert a.matmul_bias_relu(b, [-60, 1], backend="hip").data().tolist() == [0, 65, 79, 155]
+    res = Tensor(2, 2, [3, -70, -140, 2])
+    assert a.matmul_bias_add_relu(b, [-60, 1], res, backend="hip").data().tolist() == [1, 0, 0, 157]
+    with pytest.raises(TensorError) as err:
+        a.matmul(a, backend="hip")
+    assert err.value.kind == "ShapeMismatch"
+    big = Tensor(1, 1, [3e38])
+    with pytest.raises(TensorError) as err:
+        big.matmul(Tensor(1, 1, [10.0]), backend="hip")
+    assert err.value.kind == "NonFiniteValue"
+
+
+def test_concurrent_callers(hip, oracle):
+    """Python releases the GIL in ctypes calls; the reference expects concurrent callers
+    (bindings/st-py/src/tensor.rs:988-1006)."""
+    import threading
+    rng = np.random.default_rng(1)
+    problems = []
+    for i in range(8):
+        m, n, k = 40 + 8 * i, 24 + 4 * i, 64 + i
+        a = rng.uniform(-1, 1, m * k).astype(np.float32)
+        b = rng.uniform(-1, 1, k * n).astype(np.float32)
+        problems.append((m, n, k, a, b, np.zeros(m * n, np.float32)))
+    def work(p):
+        for _ in range(5):
+            hip.gemm_f32(p[0], p[1], p[2], p[3], p[4], p[5])
+    threads = [threading.Thread(target=work, args=(p,)) for p in problems]
+    for t in threads: t.start()
+    for t in threads: t.join()
+    for m, n, k, a, b, out in problems:
+        assert_close(out, oracle.gemm_f32(m, n, k, a, b), F32_REL, F32_ABS, f"thread {m}x{n}x{k}")

@@ -1,0 +1,125 @@
+"""Parity of the bf16 GEMM (f32 accumulate) against the CPU oracle: 2e-2 relative."""
+import numpy as np
+import pytest
+
+from conftest import BF16_REL, assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+def bf16_pair(rng, m, n, k, std=0.02):
+    from spiraltorch_amd import inputs
+    a = inputs.to_bf16(rng.normal(0, std, m * k).astype(np.float32))
+    b = inputs.to_bf16(rng.normal(0, std, k * n).astype(np.float32))
+    return a, b
+
+
+def check(out, want, what):
+    # 2e-2 relative per element, with an absolute floor of 2e-2 x the typical magnitude for sums that
+    # cancel to (almost) zero.  In practice the only difference is f32 summation order (~1e-6 relative).
+    floor = BF16_REL * float(np.sqrt(np.mean(np.square(want)))) * 1e-2
+    assert_close(out, want, BF16_REL, floor, what)
+    # and the tighter bound the arithmetic actually supports
+    scale = float(np.abs(want).max()) or 1.0
+    assert float(np.abs(out - want).max()) <= 1e-4 * scale, what
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 8, 8), (16, 64, 32), (33, 40, 72), (128, 128, 128), (130, 136, 264),
+                                   (16, 256, 512), (7, 24, 1000), (200, 8, 16)])
+def test_random_shapes(hip, oracle, m, n, k):
+    rng = np.random.default_rng(m * 131 + n * 17 + k)
+    a, b = bf16_pair(rng, m, n, k, std=1.0)
+    out = np.zeros(m * n, np.float32)
+    hip.gemm_bf16_f32acc(m, n, k, a, b, out)
+    check(out, oracle.gemm_bf16_f32acc(m, n, k, a, b), f"bf16 gemm {m}x{n}x{k}")
+
+
+@pytest.mark.parametrize("m,n,k", [(5, 7, 9), (17, 33, 20), (64, 100, 36)])
+def test_unaligned_shapes(hip, oracle, m, n, k):
+    rng = np.random.default_rng(m + n + k)
+    a, b = bf16_pair(rng, m, n, k, std=1.0)
+    out = np.zeros(m * n, np.float32)
+    hip.gemm_bf16_f32acc(m, n, k, a, b, out)
+    check(out, oracle.gemm_bf16_f32acc(m, n, k, a, b), f"unaligned {m}x{n}x{k}")
+
+
+def test_exact_small_integers(hip):
+    from spiraltorch_amd import inputs
+    a = inputs.to_bf16(np.arange(1, 7, dtype=np.float32))
+    b = inputs.to_bf16(np.arange(7, 13, dtype=np.float32))
+    out = np.zeros(4, np.float32)
+    hip.gemm_bf16_f32acc(2, 2, 3, a, b, out)
+    assert out.tolist() == [58, 64, 139, 154]
+
+
+def test_config4_skinny(hip, oracle):
+    """BASELINE config 4 (decode-like): M=16, N=K=4096, N(0, 0.02^2) rounded to bf16."""
+    from spiraltorch_amd import inputs
+    m, n, k = 16, 4096, 4096
+    a = inputs.to_bf16(inputs.normal(inputs.seed_for(4, 2), m * k, 0.0, 0.02))
+    b = inputs.to_bf16(inputs.normal(inputs.seed_for(4, 1), k * n, 0.0, 0.02))
+    out = np.zeros(m * n, np.float32)
+    hip.gemm_bf16_f32acc(m, n, k, a, b, out)
+    check(out, oracle.gemm_bf16_f32acc(m, n, k, a, b, threads=8), "config 4 skinny")
+
+
+def test_config4_4096_cubed_sampled_rows_and_properties(hip, oracle):
+    """BASELINE config 4: M=N=K=4096.  The oracle checks 24 sampled rows; the rest of the matrix is
+    covered by size-independent properties (row permutation equivariance, exact power-of-two linearity)."""
+    from spiraltorch_amd import inputs
+    n = 4096
+    a = inputs.to_bf16(inputs.normal(inputs.seed_for(4, 0), n * n, 0.0, 0.02))
+    b = inputs.to_bf16(inputs.normal(inputs.seed_for(4, 1), n * n, 0.0, 0.02))
+    d_a, d_b = hip.DeviceBuffer.from_array(a), hip.DeviceBuffer.from_array(b)
+    d_out = hip.DeviceBuffer(n * n * 4)
+    hip.gemm_bf16_f32acc_dev(n, n, n, d_a, d_b, d_out)
+    hip.device_synchronize()
+    out = d_out.to_array(np.float32, (n, n))
+    rows = [0, 1, 31, 32, 255, 256, 257, 1023, 2048, 3000, 4094, 4095] + list(range(1500, 1512))
+    want = oracle.gemm_bf16_f32acc(len(rows), n, n, a.reshape(n, n)[rows].ravel(), b, threads=8)
+    check(out[rows].ravel(), want, "4096^3 sampled rows")
+    # permuting the rows of A permutes the rows of C (every row goes through a different tile position)
+    perm = np.random.default_rng(0).permutation(n)
+    d_ap = hip.DeviceBuffer.from_array(a.reshape(n, n)[perm])
+    hip.gemm_bf16_f32acc_dev(n, n, n, d_ap, d_b, d_out)
+    hip.device_synchronize()
+    assert (d_out.to_array(np.float32, (n, n)) == out[perm]).all()
+    # doubling A (exact in bf16) doubles C exactly
+    a2 = inputs.to_bf16(2 * inputs.from_bf16(a))
+    d_a2 = hip.DeviceBuffer.from_array(a2)
+    hip.gemm_bf16_f32acc_dev(n, n, n, d_a2, d_b, d_out)
+    hip.device_synchronize()
+    assert (d_out.to_array(np.float32, (n, n)) == 2 * out).all()
+
+
+def test_fused_epilogue_and_bf16_output(hip, oracle):
+    from spiraltorch_amd import inputs
+    rng = np.random.default_rng(21)
+    m, n, k = 96, 160, 64
+    a, b = bf16_pair(rng, m, n, k, std=0.5)
+    bias = rng.normal(size=n).astype(np.float32)
+    res = rng.normal(size=m * n).astype(np.float32)
+    d = {name: hip.DeviceBuffer.from_array(v) for name, v in (("a", a), ("b", b), ("bias", bias), ("res", res))}
+    d32, d16 = hip.DeviceBuffer(m * n * 4), hip.DeviceBuffer(m * n * 2)
+    base = oracle.gemm_bf16_f32acc(m, n, k, a, b).astype(np.float64)
+    for act in (0, 1, 2):
+        hip.gemm_bf16_bias_act_dev(m, n, k, act, d["a"], d["b"], d["bias"], d["res"], d32, d16)
+        hip.device_synchronize()
+        pre = (base.reshape(m, n) + bias).ravel() + res
+        if act == 1:
+            want = np.maximum(pre, 0)
+        elif act == 2:
+            want = np.array([oracle.gelu(float(np.float32(x))) for x in pre])
+        else:
+            want = pre
+        got32 = d32.to_array(np.float32, m * n)
+        assert_close(got32, want, 1e-4, 1e-5, f"epilogue act={act}")
+        got16 = d16.to_array(np.uint16, m * n)
+        assert (got16 == inputs.to_bf16(got32)).all(), "bf16 output must be the RNE rounding of the f32 output"
+
+
+def test_validation(hip):
+    out = np.full(4, 13.0, np.float32)
+    with pytest.raises(hip.HipErr, match="lhs buffer length 4 does not match m\\*k=6"):
+        hip.gemm_bf16_f32acc(2, 2, 3, np.zeros(4, np.uint16), np.zeros(6, np.uint16), out)
+    assert (out == 13.0).all()
