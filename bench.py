@@ -1,0 +1,260 @@
+#!/usr/bin/env python3
+"""Benchmark of the HIP hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--only NAME]
+
+A "step" is one pass of the headline workload over one batch of synthetic input that is already
+resident in HBM: BASELINE config 2, the fused conv2d + bias + ReLU (f32, N32 C64->128 56x56 3x3 s1 p1).
+The single JSON line printed at the end carries that workload as `value` and lists every other
+BASELINE configuration (f32 GEMM 512^3, bf16 GEMM 4096^3 and 16x4096x4096, attention S2048 causal and
+non-causal, the decoder stack) under `workloads`, each with its own roofline figures.
+
+Timing: W untimed warm-up steps, then exactly K steps bracketed by a device synchronisation on both
+sides (wall clock) and by HIP events recorded on the stream the kernels are launched on (kernel time).
+The CPU baseline times the C restatement of the reference's CPU path (oracle/) on the host cores of the
+same box; it is a reported baseline, never part of `value`.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+# Published MI355X peaks the roofline fractions are priced against.
+PEAK_TFLOPS = {"f32": 157.3, "bf16": 2500.0}
+PEAK_HBM_GBS = 8000.0
+
+
+def log(*items):
+    print(*items, file=sys.stderr, flush=True)
+
+
+class Timer:
+    def __init__(self, hip):
+        self.hip = hip
+        self.stream = hip.Stream()
+        self.start, self.stop = hip.Event(), hip.Event()
+
+    def run(self, step, warmup, steps):
+        """Returns (wall ms per step, event ms per step)."""
+        for _ in range(warmup):
+            step(self.stream)
+        self.stream.synchronize()
+        self.hip.device_synchronize()
+        self.start.record(self.stream)
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step(self.stream)
+        self.stop.record(self.stream)
+        self.stream.synchronize()
+        self.hip.device_synchronize()
+        wall = (time.perf_counter() - t0) * 1e3 / steps
+        return wall, self.start.elapsed_ms(self.stop) / steps
+
+
+def roofline(bound, dtype, flops, bytes_, ms):
+    if bound == "mfma":
+        achieved = flops / (ms * 1e-3) / 1e12
+        peak = PEAK_TFLOPS[dtype]
+        return {"bound": "mfma", "achieved": round(achieved, 3), "peak": peak, "unit": "TFLOP/s",
+                "frac": round(achieved / peak, 4), "traffic": None}
+    achieved = bytes_ / (ms * 1e-3) / 1e9
+    return {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+            "frac": round(achieved / PEAK_HBM_GBS, 4), "traffic": None}
+
+
+def entry(name, dtype, flops, bytes_, bound, wall_ms, event_ms, extra=None):
+    out = {"workload": name, "dtype": dtype, "flops_per_step": flops, "min_bytes_per_step": bytes_,
+           "ms_per_step": round(wall_ms, 5), "kernel_ms_per_step": round(event_ms, 5),
+           "gflops": round(flops / (wall_ms * 1e-3) / 1e9, 1),
+           "roofline": roofline(bound, "bf16" if dtype == "bf16" else "f32", flops, bytes_, event_ms)}
+    if extra:
+        out.update(extra)
+    return out
+
+
+# ---- workloads (BASELINE.json configs) ---------------------------------------------------------------
+
+def wl_conv2d(hip, inputs, timer, warmup, steps):
+    batch, c_in, h, w, c_out = 32, 64, 56, 56, 128
+    x = inputs.normal(inputs.seed_for(2, 0), batch * c_in * h * w)
+    wt = inputs.normal(inputs.seed_for(2, 1), c_out * c_in * 9, 0.0, math.sqrt(2.0 / (c_in * 9)))
+    b = inputs.uniform(inputs.seed_for(2, 2), c_out, -0.1, 0.1)
+    d_x, d_w, d_b = (hip.DeviceBuffer.from_array(a) for a in (x, wt, b))
+    d_out = hip.DeviceBuffer(batch * c_out * h * w * 4)
+    geom = ((3, 3), (1, 1), (1, 1), (1, 1))
+
+    def step(stream):
+        hip.conv2d_bias_act_f32_dev(batch, c_in, h, w, c_out, *geom, 1, d_x, d_w, d_b, d_out, stream)
+
+    wall, ev = timer.run(step, warmup, steps)
+    flops = 2 * batch * c_out * h * w * c_in * 9
+    bytes_ = 4 * (x.size + wt.size + b.size + batch * c_out * h * w)
+    return entry("conv2d_bias_relu_f32_n32_c64to128_56x56_k3s1p1", "f32", flops, bytes_, "mfma", wall, ev), \
+        (x, wt, b, geom, (batch, c_in, h, w, c_out))
+
+
+def wl_gemm_f32(hip, inputs, timer, warmup, steps, m, n, k, name):
+    a = inputs.uniform(inputs.seed_for(1, 0), m * k, -1.0, 1.0)
+    b = inputs.uniform(inputs.seed_for(1, 1), k * n, -1.0, 1.0)
+    d_a, d_b = hip.DeviceBuffer.from_array(a), hip.DeviceBuffer.from_array(b)
+    d_c = hip.DeviceBuffer(m * n * 4)
+
+    def step(stream):
+        hip.gemm_f32_dev(m, n, k, 1.0, False, d_a, d_b, d_c, stream)
+
+    wall, ev = timer.run(step, warmup, steps)
+    return entry(name, "f32", 2 * m * n * k, 4 * (m * k + k * n + m * n), "mfma", wall, ev)
+
+
+def wl_gemm_bf16(hip, inputs, timer, warmup, steps, m, n, k, name, bound):
+    a = inputs.to_bf16(inputs.normal(inputs.seed_for(4, 0 if m == n else 2), m * k, 0.0, 0.02))
+    b = inputs.to_bf16(inputs.normal(inputs.seed_for(4, 1), k * n, 0.0, 0.02))
+    d_a, d_b = hip.DeviceBuffer.from_array(a), hip.DeviceBuffer.from_array(b)
+    d_c = hip.DeviceBuffer(m * n * 4)
+
+    def step(stream):
+        hip.gemm_bf16_f32acc_dev(m, n, k, d_a, d_b, d_c, stream)
+
+    wall, ev = timer.run(step, warmup, steps)
+    return entry(name, "bf16", 2 * m * n * k, 2 * (m * k + k * n) + 4 * m * n, bound, wall, ev)
+
+
+def wl_attention(hip, inputs, timer, warmup, steps, causal):
+    contexts, seq, dim = 128, 2048, 64
+    count = contexts * seq * dim
+    q, k, v = (inputs.normal(inputs.seed_for(3, i), count) for i in range(3))
+    d_q, d_k, d_v = (hip.DeviceBuffer.from_array(a) for a in (q, k, v))
+    d_o = hip.DeviceBuffer(count * 4)
+
+    def step(stream):
+        hip.attention_f32_dev(contexts, seq, dim, 0.125, causal, d_q, d_k, d_v, None, None, d_o, stream)
+
+    wall, ev = timer.run(step, warmup, steps)
+    flops = 4 * dim * contexts * (seq * (seq + 1) // 2 if causal else seq * seq)
+    name = "attention_f32_b8_h16_s2048_d64_" + ("causal" if causal else "noncausal")
+    return entry(name, "f32", flops, 4 * 4 * count, "mfma", wall, ev)
+
+
+def wl_decoder(hip, inputs, timer, warmup, steps):
+    vocab, d, heads, layers, ff, batch, seq = 256, 512, 8, 6, 2048, 16, 1024
+    count = hip.Decoder.weight_count(vocab, d, heads, layers, ff)
+    weights = inputs.normal(inputs.seed_for(5, 0), count, 0.0, 0.02)
+    tokens = inputs.tokens(inputs.seed_for(5, 1), batch * seq, vocab)
+    dec = hip.Decoder(vocab, d, heads, layers, ff, batch, seq, 1e-5, weights)
+    d_tok = hip.DeviceBuffer.from_array(tokens)
+    d_logits = hip.DeviceBuffer(batch * seq * vocab * 4)
+
+    def step(stream):
+        dec.forward_dev(d_tok, d_logits, stream)
+
+    wall, ev = timer.run(step, warmup, steps)
+    T = batch * seq
+    hd = d // heads
+    per_layer = 3 * 2 * T * d * d + 2 * T * d * d + 4 * hd * batch * heads * (seq * (seq + 1) // 2) + 2 * 2 * T * d * ff
+    flops = layers * per_layer + 2 * T * d * vocab
+    out = entry("decoder_bf16_v256_d512_h8_l6_ff2048_b16_s1024", "bf16", flops, 0, "mfma", wall, ev,
+                {"tokens_per_s": round(T / (wall * 1e-3), 1)})
+    dec.destroy()
+    return out
+
+
+# ---- CPU baseline ---------------------------------------------------------------------------------------
+
+def cpu_baseline_conv(conv_inputs):
+    """Times the C restatement of Conv2d::forward_cpu (single-threaded, as the reference's contraction is)
+    on one full pass of config 2."""
+    from oracle import oracle
+    x, wt, b, geom, (batch, c_in, h, w, c_out) = conv_inputs
+    oracle.load()
+    t0 = time.perf_counter()
+    oracle.conv2d_bias_act_f32(batch, c_in, h, w, c_out, *geom, oracle.ACT_RELU, x, wt, b, threads=1)
+    seconds = time.perf_counter() - t0
+    flops = 2 * batch * c_out * h * w * c_in * 9
+    return {"value": round(flops / seconds / 1e9, 3), "unit": "GFLOP/s", "cores": 1, "kind": "port",
+            "sample": f"one full pass of config 2 ({batch} images) through oracle/st_oracle.c, single thread, "
+                      f"{seconds:.2f} s; host has {os.cpu_count()} logical CPUs"}
+
+
+def main():
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=50)
+    parser.add_argument("--warmup", type=int, default=10)
+    parser.add_argument("--no-cpu-baseline", action="store_true")
+    parser.add_argument("--only", default=None, help="run only the headline plus workloads whose name contains this")
+    args = parser.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (every op shards into independent "
+              "units; see DESIGN.md). Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    from spiraltorch_amd import hip, inputs
+    hip.init()  # raises when libsthip.so or the device is missing: there is no fallback to measure
+    props = hip.device_properties(0)
+    log("device:", props)
+    timer = Timer(hip)
+
+    headline, conv_inputs = wl_conv2d(hip, inputs, timer, args.warmup, args.steps)
+    log(json.dumps(headline))
+    others = []
+    side_steps = max(5, min(args.steps, 20))
+    side_warm = max(2, min(args.warmup, 5))
+    plan = [
+        ("gemm_f32_512", lambda: wl_gemm_f32(hip, inputs, timer, side_warm, side_steps, 512, 512, 512,
+                                              "gemm_f32_512x512x512")),
+        ("gemm_f32_conv_equivalent", lambda: wl_gemm_f32(hip, inputs, timer, side_warm, side_steps, 100352, 128, 576,
+                                                         "gemm_f32_100352x128x576_conv_equivalent")),
+        ("gemm_bf16_4096", lambda: wl_gemm_bf16(hip, inputs, timer, side_warm, side_steps, 4096, 4096, 4096,
+                                                "gemm_bf16_f32acc_4096x4096x4096", "mfma")),
+        ("gemm_bf16_skinny", lambda: wl_gemm_bf16(hip, inputs, timer, side_warm, side_steps, 16, 4096, 4096,
+                                                  "gemm_bf16_f32acc_16x4096x4096", "hbm")),
+        ("attention_noncausal", lambda: wl_attention(hip, inputs, timer, 2, 5, False)),
+        ("attention_causal", lambda: wl_attention(hip, inputs, timer, 2, 5, True)),
+        ("decoder", lambda: wl_decoder(hip, inputs, timer, 2, 5)),
+    ]
+    for name, fn in plan:
+        if args.only and args.only not in name:
+            continue
+        result = fn()
+        log(json.dumps(result))
+        others.append(result)
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        cpu = cpu_baseline_conv(conv_inputs)
+        log(json.dumps(cpu))
+
+    line = {
+        "metric": "GFLOP/s and % of MFMA roofline (GEMM, conv, attention) on 1 MI355X; value = fused conv2d+bias+ReLU",
+        "value": headline["gflops"],
+        "unit": "GFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": headline["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": headline["workload"], "batch": 32, "c_in": 64, "c_out": 128, "hw": 56, "kernel": 3,
+                   "resident": "HBM"},
+        "roofline": headline["roofline"],
+        "cpu_baseline": cpu,
+        "device": {"arch": props["arch"], "compute_units": props["compute_units"], "clock_khz": props["clock_khz"]},
+        "workloads": others,
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()
