@@ -12,6 +12,8 @@
 //
 // MFMA operand layout (32x32x16): lane l supplies A[l%32][8*(l/32) .. +7] and B[8*(l/32) .. +7][l%32];
 // accumulator register r of lane l is C[(r/4)*8 + (l/32)*4 + r%4][l%32].
+#include <type_traits>
+
 #include "device_math.h"
 #include "kernels.h"
 
@@ -98,8 +100,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmBf16Args p)
     for (int a = 0; a < TM; ++a)
 #pragma unroll
         for (int b = 0; b < TN; ++b)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.0f;
+            acc[a][b] = f32x16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
     uint4 ra[A_CHUNKS], rb[B_CHUNKS];
 
@@ -153,13 +154,11 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmBf16Args p)
 #pragma unroll
             for (int tn = 0; tn < TN; ++tn) {
                 const uint16_t *src = &bs[(kk * 16 + b_row) * B_STRIDE + b_col + tn * 32];
-                union {
-                    s16x4 half[2];
-                    bf16x8 full;
-                } frag;
-                frag.half[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(src));
-                frag.half[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(src + 4 * B_STRIDE));
-                b[tn] = frag.full;
+                const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(src));
+                const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(src + 4 * B_STRIDE));
+                typedef short s16x8 __attribute__((ext_vector_type(8)));
+                const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                b[tn] = __builtin_bit_cast(bf16x8, both);
             }
 #pragma unroll
             for (int tm = 0; tm < TM; ++tm)
@@ -183,29 +182,257 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmBf16Args p)
         __syncthreads();
     }
 
+    // Epilogue.  The loops carry no early exits so that they unroll completely and the accumulators
+    // stay in registers.
     const bool scaled = p.scale != 1.0f;
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn) {
         const int col = n0 + wn * WTN + tn * 32 + li;
-        if (col >= N) continue;
-        const float bias = p.bias ? p.bias[col] : 0.0f;
+        const bool col_ok = col < N;
+        const float bias = (p.bias && col_ok) ? p.bias[col] : 0.0f;
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm) {
+            const f32x16 tile = acc[tm][tn];
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int row = m0 + wm * WTM + tm * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
-                if (row >= M) continue;
-                const size_t idx = static_cast<size_t>(row) * N + col;
-                float value = acc[tm][tn][r];
-                if (scaled) value *= p.scale;
-                if (p.bias) value += bias;
-                if (p.residual) value += p.residual[idx];
-                value = apply_activation(value, p.activation);
-                if (p.C32) p.C32[idx] = value;
-                if (p.C16) p.C16[idx] = f32_to_bf16_rne(value);
+                if (col_ok && row < M) {
+                    const size_t idx = static_cast<size_t>(row) * N + col;
+                    float value = tile[r];
+                    if (scaled) value *= p.scale;
+                    value += bias;
+                    if (p.residual) value += p.residual[idx];
+                    value = apply_activation(value, p.activation);
+                    if (p.C32) p.C32[idx] = value;
+                    if (p.C16) p.C16[idx] = f32_to_bf16_rne(value);
+                }
             }
         }
     }
+}
+
+
+// -------------------------------------------------------------------------------------------------
+// Large-problem kernel: 256×256×64 tiles, K a multiple of 64, N a multiple of 256 (M may be ragged:
+// rows past the end read as zero through the buffer descriptor's range check and are never stored).
+//
+// One iteration consumes LDS stage s = t&1 while tile t+1 (already sitting in registers) is written to
+// stage s^1 and tile t+2 is requested from memory.  The fragment reads run one 16-wide k sub-step
+// ahead of the MFMAs and cross the stage boundary: the single barrier of the iteration sits before
+// the last sub-step's MFMAs, so the first fragments of the next stage arrive while those MFMAs run.
+// The epilogue goes through LDS (each wavefront owns a 32×128 f32 strip) so that bias/residual loads and
+// the stores are 128-bit and row-contiguous.
+// -------------------------------------------------------------------------------------------------
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+
+__global__ __launch_bounds__(256) void gemm_bf16_256_kernel(GemmBf16Args p)
+{
+    constexpr int BM = 256, BN = 256, BK = 64;
+    constexpr int A_STRIDE = BK + 8, B_STRIDE = BN + 32;
+    constexpr int A_STAGE = BM * A_STRIDE, B_STAGE = BK * B_STRIDE;  // elements
+    constexpr int C_STRIDE = 128 + 4;                                 // floats, epilogue strip
+    extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+    uint16_t *As = lds;
+    uint16_t *Bs = lds + 2 * A_STAGE;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int li = lane & 31, lh = lane >> 5;
+    const int M = p.M, N = p.N, K = p.K;
+
+    int logical = blockIdx.x;
+    if (p.swizzle) logical = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+    constexpr int GROUP_M = 4;
+    const int width = GROUP_M * p.tiles_n;
+    const int group = logical / width;
+    const int first_m = group * GROUP_M;
+    const int group_size = min(p.tiles_m - first_m, GROUP_M);
+    const int tile_m = first_m + (logical % width) % group_size;
+    const int tile_n = (logical % width) / group_size;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t *>(p.A), 0, static_cast<int>(static_cast<unsigned>(M) * static_cast<unsigned>(K) * 2u), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t *>(p.B), 0, static_cast<int>(static_cast<unsigned>(K) * static_cast<unsigned>(N) * 2u), 0x00020000);
+    // byte offsets of this thread's first 16-byte chunk of the current k-tile
+    unsigned a_off = (static_cast<unsigned>(m0 + (tid >> 3)) * K + (tid & 7) * 8) * 2u;
+    unsigned b_off = (static_cast<unsigned>(tid >> 5) * N + n0 + (tid & 31) * 8) * 2u;
+    const unsigned a_row_step = 32u * K * 2u;  // 32 rows per chunk index
+    const unsigned b_row_step = 8u * N * 2u;   // 8 k-rows per chunk index
+    const unsigned b_tile_step = static_cast<unsigned>(BK) * N * 2u;
+
+    f32x16 acc[4][4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+            acc[a][b] = f32x16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+
+    u32x4 ra[8], rb[8];
+    auto load_global = [&]() {
+#pragma unroll
+        for (int r = 0; r < 8; ++r) ra[r] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, a_off + r * a_row_step, 0, 0);
+#pragma unroll
+        for (int r = 0; r < 8; ++r) rb[r] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, b_off + r * b_row_step, 0, 0);
+        a_off += BK * 2u;
+        b_off += b_tile_step;
+    };
+    const int a_store = (tid >> 3) * A_STRIDE + (tid & 7) * 8;
+    const int b_store = (tid >> 5) * B_STRIDE + (tid & 31) * 8;
+    auto store_lds = [&](int stage) {
+        uint16_t *as = As + stage * A_STAGE + a_store;
+        uint16_t *bs = Bs + stage * B_STAGE + b_store;
+#pragma unroll
+        for (int r = 0; r < 8; ++r) *reinterpret_cast<u32x4 *>(as + r * 32 * A_STRIDE) = ra[r];
+#pragma unroll
+        for (int r = 0; r < 8; ++r) *reinterpret_cast<u32x4 *>(bs + r * 8 * B_STRIDE) = rb[r];
+    };
+    const int i16 = lane & 15;
+    const int c16 = (lane >> 4) & 1;
+    const int a_frag = (wm * 128 + li) * A_STRIDE + lh * 8;
+    const int b_frag = (lh * 8 + (i16 >> 2)) * B_STRIDE + wn * 128 + c16 * 16 + (i16 & 3) * 4;
+    bf16x8 fa[2][4], fb[2][4];
+    auto read_frags = [&](int buf, int stage, int kk) {
+        const uint16_t *as = As + stage * A_STAGE + a_frag + kk * 16;
+        const uint16_t *bs = Bs + stage * B_STAGE + b_frag + kk * 16 * B_STRIDE;
+#pragma unroll
+        for (int tm = 0; tm < 4; ++tm) fa[buf][tm] = *reinterpret_cast<const bf16x8 *>(as + tm * 32 * A_STRIDE);
+#pragma unroll
+        for (int tn = 0; tn < 4; ++tn) {
+            const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(bs + tn * 32));
+            const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(bs + tn * 32 + 4 * B_STRIDE));
+            fb[buf][tn] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        }
+    };
+    auto mfma_step = [&](int buf) {
+#pragma unroll
+        for (int tm = 0; tm < 4; ++tm)
+#pragma unroll
+            for (int tn = 0; tn < 4; ++tn)
+                acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[buf][tm], fb[buf][tn], acc[tm][tn], 0, 0, 0);
+    };
+
+    // One k-tile.  STORE: tile t+1 goes from registers to the other stage; LOAD: tile t+2 is requested;
+    // NEXT: the first fragments of tile t+1 are fetched after the barrier.  The sched_group_barrier
+    // sequences pin the issue order to "one MFMA, then at most two memory instructions", so the matrix
+    // pipe is never left waiting behind a burst of LDS or buffer instructions.
+    auto iteration = [&](auto store_tag, auto load_tag, auto next_tag, int s) {
+        constexpr bool STORE = decltype(store_tag)::value;
+        constexpr bool LOAD = decltype(load_tag)::value;
+        constexpr bool NEXT = decltype(next_tag)::value;
+        read_frags(1, s, 1);
+        mfma_step(0);
+        if constexpr (STORE) store_lds(s ^ 1);
+        if constexpr (LOAD) load_global();
+        read_frags(0, s, 2);
+        mfma_step(1);
+        read_frags(1, s, 3);
+        mfma_step(0);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {  // kk = 0 MFMAs: fragment reads of kk = 1, LDS writes of tile t+1
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (i < 12) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            if (STORE) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {  // kk = 1 MFMAs: fragment reads of kk = 2, buffer loads of tile t+2
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (i < 12) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            if (LOAD) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {  // kk = 2 MFMAs: fragment reads of kk = 3
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (i < 12) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __syncthreads();  // stage s^1 complete; every wavefront is done reading stage s
+        if constexpr (NEXT) read_frags(0, s ^ 1, 0);
+        mfma_step(1);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {  // kk = 3 MFMAs: first fragment reads of the next tile
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (NEXT && i < 12) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+    };
+
+    const int steps = K / BK;
+    load_global();
+    store_lds(0);
+    if (steps > 1) load_global();
+    __syncthreads();
+    read_frags(0, 0, 0);
+    int t = 0;
+    for (; t + 2 < steps; ++t) iteration(std::true_type{}, std::true_type{}, std::true_type{}, t & 1);
+    if (t + 1 < steps) {
+        iteration(std::true_type{}, std::false_type{}, std::true_type{}, t & 1);
+        ++t;
+    }
+    iteration(std::false_type{}, std::false_type{}, std::false_type{}, t & 1);
+
+    // ---- epilogue through LDS ---------------------------------------------------------------------
+    __syncthreads();
+    float *strip = reinterpret_cast<float *>(lds) + wave * (32 * C_STRIDE);
+    const bool scaled = p.scale != 1.0f;
+    const int col0 = n0 + wn * 128 + (lane & 31) * 4;  // this lane's 4 columns in the read-back phase
+    float4 bias4 = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (p.bias) bias4 = *reinterpret_cast<const float4 *>(p.bias + col0);
+#pragma unroll
+    for (int tm = 0; tm < 4; ++tm) {
+#pragma unroll
+        for (int tn = 0; tn < 4; ++tn) {
+            const f32x16 tile = acc[tm][tn];
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                strip[((r >> 2) * 8 + lh * 4 + (r & 3)) * C_STRIDE + tn * 32 + li] = tile[r];
+        }
+        const int row_base = m0 + wm * 128 + tm * 32;
+#pragma unroll 2
+        for (int j = 0; j < 16; ++j) {
+            const int local_row = j * 2 + (lane >> 5);
+            const int row = row_base + local_row;
+            float4 v = *reinterpret_cast<const float4 *>(&strip[local_row * C_STRIDE + (lane & 31) * 4]);
+            if (row < M) {
+                const size_t idx = static_cast<size_t>(row) * N + col0;
+                if (scaled) { v.x *= p.scale; v.y *= p.scale; v.z *= p.scale; v.w *= p.scale; }
+                v.x += bias4.x; v.y += bias4.y; v.z += bias4.z; v.w += bias4.w;
+                if (p.residual) {
+                    const float4 rr = *reinterpret_cast<const float4 *>(p.residual + idx);
+                    v.x += rr.x; v.y += rr.y; v.z += rr.z; v.w += rr.w;
+                }
+                v.x = apply_activation(v.x, p.activation);
+                v.y = apply_activation(v.y, p.activation);
+                v.z = apply_activation(v.z, p.activation);
+                v.w = apply_activation(v.w, p.activation);
+                if (p.C32) *reinterpret_cast<float4 *>(p.C32 + idx) = v;
+                if (p.C16) {
+                    uint2 packed;
+                    packed.x = f32_to_bf16_rne(v.x) | (static_cast<uint32_t>(f32_to_bf16_rne(v.y)) << 16);
+                    packed.y = f32_to_bf16_rne(v.z) | (static_cast<uint32_t>(f32_to_bf16_rne(v.w)) << 16);
+                    *reinterpret_cast<uint2 *>(p.C16 + idx) = packed;
+                }
+            }
+        }
+    }
+}
+
+hipError_t launch_256(GemmBf16Args args, hipStream_t stream)
+{
+    args.tiles_m = (args.M + 255) / 256;
+    args.tiles_n = args.N / 256;
+    const size_t tiles = static_cast<size_t>(args.tiles_m) * static_cast<size_t>(args.tiles_n);
+    if (tiles > 0x7fffffffu) return hipErrorInvalidConfiguration;
+    args.swizzle = (tiles % 8 == 0) ? 1 : 0;
+    constexpr size_t lds_bytes = 2 * (256 * (64 + 8) + 64 * (256 + 32)) * 2;
+    static_assert(lds_bytes >= 4 * 32 * (128 + 4) * sizeof(float), "epilogue strips must fit in the stage buffers");
+    hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_bf16_256_kernel),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
+    if (rc != hipSuccess) return rc;
+    hipLaunchKernelGGL(gemm_bf16_256_kernel, dim3(static_cast<unsigned>(tiles)), dim3(256), lds_bytes, stream, args);
+    return hipGetLastError();
 }
 
 template <int BM, int BN, int BK>
@@ -261,7 +488,13 @@ hipError_t launch_gemm_bf16(size_t m, size_t n, size_t k, const uint16_t *lhs, c
     args.activation = epilogue.activation;
     const bool vec = (k % 8 == 0) && (n % 8 == 0) && aligned16(lhs) && aligned16(rhs);
     const size_t big_tiles = ((m + 255) / 256) * ((n + 255) / 256);
-    if (big_tiles >= 192) return launch_tile<256, 256, 64>(args, vec, stream);
+    // The 256-tile kernel addresses its operands through 32-bit buffer offsets and reads bias/residual/output
+    // in 16-byte pieces.
+    const bool fits_buffer = m * k * 2 < (1ull << 31) && k * n * 2 < (1ull << 31);
+    const bool epilogue_aligned = aligned16(out_f32) && aligned16(epilogue.bias) && aligned16(epilogue.residual) &&
+                                  (reinterpret_cast<uintptr_t>(out_bf16) & 7u) == 0;
+    if (big_tiles >= 128 && vec && k >= 64 && k % 64 == 0 && n % 256 == 0 && fits_buffer && epilogue_aligned)
+        return launch_256(args, stream);
     return launch_tile<128, 128, 32>(args, vec, stream);
 }
 
