@@ -12,8 +12,11 @@
 //
 // MFMA operand layout (32x32x16): lane l supplies A[l%32][8*(l/32) .. +7] and B[8*(l/32) .. +7][l%32];
 // accumulator register r of lane l is C[(r/4)*8 + (l/32)*4 + r%4][l%32].
+#include <algorithm>
 #include <cstdlib>
+#include <mutex>
 #include <type_traits>
+#include <vector>
 
 #include "device_math.h"
 #include "kernels.h"
@@ -723,6 +726,259 @@ __global__ __launch_bounds__(512) void gemm_bf16_256w8_kernel(GemmBf16Args p)
     }
 }
 
+// -------------------------------------------------------------------------------------------------
+// Skinny kernel (M <= 64, decode-like): HBM-bound on B, so the job is to keep many bytes of B in flight
+// on every compute unit.  The grid is (N/128 column strips) × (k-splits); a workgroup streams its
+// 64-row k-tiles of B straight into a four-deep LDS ring with buffer_load ... lds (three tiles are always
+// in flight), reads them back with the LDS transpose load and feeds 32x32x16 MFMAs whose A operand comes
+// from global memory (A is tiny and cache-resident).  Split-k partial sums go to a workspace and are
+// added in a fixed order by a second kernel that also applies the epilogue, so results are reproducible.
+//
+// Ring layout: row k of a tile holds 128 columns = 16 chunks of 16 B; chunk c of row k is stored at chunk
+// position c ^ (2 * (k & 3)), which spreads the four rows a transpose read touches over all banks.
+// -------------------------------------------------------------------------------------------------
+struct SkinnyArgs {
+    const uint16_t *A;
+    const uint16_t *B;
+    float *partial;         // [k_splits][M][N]
+    float *C32;
+    uint16_t *C16;
+    const float *bias;
+    const float *residual;
+    int M, N, K;
+    int tiles_n, k_splits, tiles_per_split;
+    float scale;
+    int activation;
+};
+
+template <int MT, int RING>  // MT row blocks of 32; RING stages
+__device__ __forceinline__ void gemm_bf16_skinny_body(const SkinnyArgs &p)
+{
+    constexpr int BK = 64, BN = 128;
+    constexpr int B_BYTES = BK * BN * 2;       // 16 KB
+    constexpr int A_BYTES = MT * 32 * BK * 2;  // 4 KB per row block
+    constexpr int STAGE = B_BYTES + A_BYTES;
+    // Each wavefront issues 4 + MT direct loads per k-tile (the vmcnt immediates below count them).
+    extern __shared__ __attribute__((aligned(16))) unsigned char ring[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int li = lane & 31, lh = lane >> 5;
+    const int strip = blockIdx.x % p.tiles_n;
+    const int split = blockIdx.x / p.tiles_n;
+    const int n0 = strip * BN;
+    const int tile0 = split * p.tiles_per_split;
+    const int tiles = min(p.tiles_per_split, p.K / BK - tile0);
+    const int N = p.N, K = p.K;
+
+    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t *>(p.A), 0, static_cast<int>(static_cast<unsigned>(p.M) * static_cast<unsigned>(K) * 2u), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t *>(p.B), 0, static_cast<int>(static_cast<unsigned>(K) * static_cast<unsigned>(N) * 2u), 0x00020000);
+
+    // B: instruction r of wavefront w fills rows (r*4 + w)*4 .. +3 of the stage (16 lanes per row).
+    unsigned b_off[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int row = (r * 4 + wave) * 4 + (lane >> 4);
+        const int chunk = (lane & 15) ^ (2 * (row & 3));
+        b_off[r] = (static_cast<unsigned>(tile0 * BK + row) * N + n0 + chunk * 8) * 2u;
+    }
+    // A: instruction mt of wavefront w fills rows mt*32 + w*8 .. +7 (8 lanes per row, 128 B = this tile's 64
+    // k-values); chunk q of row r is stored at q ^ ((r >> 1) & 7).  Rows >= M read as zero.
+    unsigned a_off[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int row = mt * 32 + wave * 8 + (lane >> 3);
+        const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+        a_off[mt] = (static_cast<unsigned>(row) * K + tile0 * BK + chunk * 8) * 2u;
+    }
+    const unsigned b_tile_step = static_cast<unsigned>(BK) * N * 2u;
+    auto load_tile = [&](int tile, int stage) {
+        unsigned char *base = ring + stage * STAGE;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_void_ptr)(base + (r * 4 + wave) * 1024), 16,
+                                                     b_off[r] + tile * b_tile_step, 0, 0, 0);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_ptr)(base + B_BYTES + (mt * 4 + wave) * 1024), 16,
+                                                     a_off[mt] + tile * (BK * 2u), 0, 0, 0);
+    };
+
+    // Transpose-read addresses: this wavefront owns columns wave*32 .. +31.  Lane roles as in the tiled
+    // kernel: i16 supplies row i16/4 and the 8-byte piece i16%4 of a 4×16 block.
+    const int i16 = lane & 15, c16 = (lane >> 4) & 1;
+    const int piece = wave * 8 + c16 * 4 + (i16 & 3);  // 8-byte piece index within the 128-column row
+    unsigned b_read[2];
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+        const int row = lh * 8 + half * 4 + (i16 >> 2);
+        b_read[half] = row * 256 + (((piece >> 1) ^ (2 * (row & 3))) * 16) + (piece & 1) * 8;
+    }
+    unsigned a_read[4];
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) a_read[kk] = B_BYTES + li * 128 + (((2 * kk + lh) ^ ((li >> 1) & 7)) & 7) * 16;
+
+    f32x16 acc[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+        acc[mt] = f32x16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+
+    // Prologue: RING-1 tiles in flight.
+#pragma unroll
+    for (int i = 0; i < RING - 1; ++i)
+        if (i < tiles) load_tile(i, i);
+    for (int t = 0; t < tiles; ++t) {
+        // Tile t must have landed; the (up to RING-2) tiles requested after it may stay in flight.
+        const int newer = min(tiles - 1 - t, RING - 2);
+        if (newer >= 2) {
+            if constexpr (MT == 1) ST_WAIT_VMCNT(10); else ST_WAIT_VMCNT(12);
+        } else if (newer == 1) {
+            if constexpr (MT == 1) ST_WAIT_VMCNT(5); else ST_WAIT_VMCNT(6);
+        } else {
+            ST_WAIT_VMCNT(0);
+        }
+        __syncthreads();  // tile t visible to all; everyone is done with tile t-1, whose stage is refilled next
+        if (t + RING - 1 < tiles) load_tile(t + RING - 1, (t + RING - 1) % RING);
+        const unsigned char *stage = ring + (t % RING) * STAGE;
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+            const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(stage + b_read[0] + kk * 16 * 256));
+            const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(stage + b_read[1] + kk * 16 * 256));
+            const bf16x8 fb = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const bf16x8 fa = *reinterpret_cast<const bf16x8 *>(stage + a_read[kk] + mt * 4096);
+                acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb, acc[mt], 0, 0, 0);
+            }
+        }
+    }
+
+    float *dst = p.partial + static_cast<size_t>(split) * p.M * N;
+    const int col = n0 + wave * 32 + li;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int row = mt * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
+            if (row < p.M) dst[static_cast<size_t>(row) * N + col] = acc[mt][r];
+        }
+
+}
+
+// Plain (non-template) kernel entry points: the host-side stub of a kernel template whose body calls the
+// LDS-load builtins is not emitted by this compiler, so the template stays a device function.
+__global__ __launch_bounds__(256) void gemm_bf16_skinny32_kernel(SkinnyArgs p) { gemm_bf16_skinny_body<1, 4>(p); }
+__global__ __launch_bounds__(256) void gemm_bf16_skinny64_kernel(SkinnyArgs p) { gemm_bf16_skinny_body<2, 3>(p); }
+
+// Adds the k-split partial sums in split order (so the result does not depend on scheduling) and applies
+// the epilogue.  One thread per output element; the partials of eight splits are requested together so
+// the loads overlap, then added one by one.
+__global__ __launch_bounds__(256) void gemm_bf16_skinny_reduce_kernel(SkinnyArgs p)
+{
+    const size_t plane = static_cast<size_t>(p.M) * p.N;
+    const size_t idx = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (idx >= plane) return;
+    float value = 0.0f;
+    for (int s0 = 0; s0 < p.k_splits; s0 += 8) {
+        float part[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) part[j] = (s0 + j < p.k_splits) ? p.partial[(s0 + j) * plane + idx] : 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) value += part[j];
+    }
+    if (p.scale != 1.0f) value *= p.scale;
+    if (p.bias) value += p.bias[idx % p.N];
+    if (p.residual) value += p.residual[idx];
+    value = apply_activation(value, p.activation);
+    if (p.C32) p.C32[idx] = value;
+    if (p.C16) p.C16[idx] = f32_to_bf16_rne(value);
+}
+
+// Split-k partial sums live in one grow-only device buffer per stream: work on a stream is ordered, so two
+// launches on the same stream never use the buffer at the same time, and different streams get different
+// buffers.  (hipMallocAsync/hipFreeAsync per call cost several times the kernel itself.)
+hipError_t split_k_workspace(hipStream_t stream, size_t bytes, float **out)
+{
+    struct Entry {
+        hipStream_t stream;
+        void *ptr;
+        size_t capacity;
+    };
+    static std::mutex mutex;
+    static std::vector<Entry> entries;
+    std::lock_guard<std::mutex> lock(mutex);
+    for (Entry &e : entries) {
+        if (e.stream != stream) continue;
+        if (e.capacity < bytes) {
+            hipError_t rc = hipStreamSynchronize(stream);
+            if (rc != hipSuccess) return rc;
+            rc = hipFree(e.ptr);
+            if (rc != hipSuccess) return rc;
+            e.ptr = nullptr;
+            e.capacity = 0;
+            rc = hipMalloc(&e.ptr, bytes);
+            if (rc != hipSuccess) return rc;
+            e.capacity = bytes;
+        }
+        *out = static_cast<float *>(e.ptr);
+        return hipSuccess;
+    }
+    Entry fresh{stream, nullptr, bytes};
+    hipError_t rc = hipMalloc(&fresh.ptr, bytes);
+    if (rc != hipSuccess) return rc;
+    entries.push_back(fresh);
+    *out = static_cast<float *>(fresh.ptr);
+    return hipSuccess;
+}
+
+hipError_t launch_skinny(const GemmBf16Args &args, hipStream_t stream)
+{
+    SkinnyArgs sk;
+    sk.A = args.A;
+    sk.B = args.B;
+    sk.M = args.M;
+    sk.N = args.N;
+    sk.K = args.K;
+    sk.tiles_n = args.N / 128;
+    const int k_tiles = args.K / 64;
+    // Aim for about two workgroups per compute unit, but keep at least four k-tiles per split so the
+    // partial-sum traffic stays a small fraction of B.
+    int splits = (512 + sk.tiles_n - 1) / sk.tiles_n;
+    splits = std::max(1, std::min(splits, k_tiles / 4 > 0 ? k_tiles / 4 : 1));
+    sk.tiles_per_split = (k_tiles + splits - 1) / splits;
+    sk.k_splits = (k_tiles + sk.tiles_per_split - 1) / sk.tiles_per_split;
+    const size_t bytes = static_cast<size_t>(sk.k_splits) * args.M * args.N * sizeof(float);
+    hipError_t rc = split_k_workspace(stream, bytes, &sk.partial);
+    if (rc != hipSuccess) return rc;
+    sk.C32 = args.C32;
+    sk.C16 = args.C16;
+    sk.bias = args.bias;
+    sk.residual = args.residual;
+    sk.scale = args.scale;
+    sk.activation = args.activation;
+    const dim3 grid(static_cast<unsigned>(sk.tiles_n * sk.k_splits));
+    if (args.M <= 32) {
+        constexpr int lds = 4 * (16384 + 4096);
+        auto kernel = gemm_bf16_skinny32_kernel;
+        rc = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        if (rc == hipSuccess) hipLaunchKernelGGL(kernel, grid, dim3(256), lds, stream, sk);
+    } else {
+        constexpr int lds = 3 * (16384 + 8192);
+        auto kernel = gemm_bf16_skinny64_kernel;
+        rc = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        if (rc == hipSuccess) hipLaunchKernelGGL(kernel, grid, dim3(256), lds, stream, sk);
+    }
+    if (rc == hipSuccess) rc = hipGetLastError();
+    if (rc != hipSuccess) return rc;
+    const size_t plane = static_cast<size_t>(args.M) * args.N;
+    hipLaunchKernelGGL(gemm_bf16_skinny_reduce_kernel, dim3(static_cast<unsigned>((plane + 255) / 256)), dim3(256), 0, stream,
+                       sk);
+    return hipGetLastError();
+}
+
 template <bool EIGHT_WAVES>
 hipError_t launch_256(GemmBf16Args args, hipStream_t stream)
 {
@@ -800,6 +1056,8 @@ hipError_t launch_gemm_bf16(size_t m, size_t n, size_t k, const uint16_t *lhs, c
     const bool fits_buffer = m * k * 2 < (1ull << 31) && k * n * 2 < (1ull << 31);
     const bool epilogue_aligned = aligned16(out_f32) && aligned16(epilogue.bias) && aligned16(epilogue.residual) &&
                                   (reinterpret_cast<uintptr_t>(out_bf16) & 7u) == 0;
+    if (m <= 64 && vec && k >= 256 && k % 64 == 0 && n % 128 == 0 && fits_buffer)
+        return launch_skinny(args, stream);
     if (big_tiles >= 128 && vec && k >= 64 && k % 64 == 0 && n % 256 == 0 && fits_buffer && epilogue_aligned)
         return getenv("STHIP_GEMM_W4") ? launch_256<false>(args, stream) : launch_256<true>(args, stream);
     return launch_tile<128, 128, 32>(args, vec, stream);

@@ -92,10 +92,23 @@ def test_config4_4096_cubed_sampled_rows_and_properties(hip, oracle):
     assert (d_out.to_array(np.float32, (n, n)) == 2 * out).all()
 
 
-def test_fused_epilogue_and_bf16_output(hip, oracle):
+@pytest.mark.parametrize("m,n,k", [(1, 128, 256), (16, 384, 320), (33, 256, 512), (64, 128, 1024), (7, 1024, 2048)])
+def test_skinny_split_k_path(hip, oracle, m, n, k):
+    """Decode-like shapes (M <= 64) take the split-k kernel; partial sums are reduced in a fixed order."""
+    rng = np.random.default_rng(m * 7 + n + k)
+    a, b = bf16_pair(rng, m, n, k, std=1.0)
+    out = np.zeros(m * n, np.float32)
+    hip.gemm_bf16_f32acc(m, n, k, a, b, out)
+    check(out, oracle.gemm_bf16_f32acc(m, n, k, a, b), f"skinny {m}x{n}x{k}")
+    again = np.zeros(m * n, np.float32)
+    hip.gemm_bf16_f32acc(m, n, k, a, b, again)
+    assert (again == out).all(), "split-k reduction must be reproducible"
+
+
+@pytest.mark.parametrize("m,n,k", [(96, 160, 64), (24, 256, 512), (256, 512, 128)])
+def test_fused_epilogue_and_bf16_output(hip, oracle, m, n, k):
     from spiraltorch_amd import inputs
     rng = np.random.default_rng(21)
-    m, n, k = 96, 160, 64
     a, b = bf16_pair(rng, m, n, k, std=0.5)
     bias = rng.normal(size=n).astype(np.float32)
     res = rng.normal(size=m * n).astype(np.float32)
