@@ -18,6 +18,8 @@
 //                                              (r/4)*8 + 4h + r%4), A operand = V[that key][d] from LDS
 // so the running max / sum / rescale factors are per-lane scalars, and the only cross-lane traffic of
 // the softmax is one exchange between lane l and lane l^32 for the row maximum.
+#include <type_traits>
+
 #include "device_math.h"
 #include "kernels.h"
 
@@ -247,6 +249,265 @@ __global__ __launch_bounds__(256) void attention_f32_kernel(AttnArgs p)
     }
 }
 
+// -------------------------------------------------------------------------------------------------
+// Fast path: no additive biases, head_dim a multiple of 4, 16-byte aligned operands.
+//
+// Same transposed formulation as the general kernel above, tuned for the matrix pipe:
+//   * 64 keys (two 32-key tiles) per softmax step: the two QKᵀ accumulations are independent MFMA
+//     chains, and the max / exchange / rescale bookkeeping is paid once per 64 keys;
+//   * V is staged TRANSPOSED (Vt[d][key]) so that the four keys a lane needs for four consecutive
+//     PV steps are one 128-bit LDS read (8 reads per 64 keys and 32 output rows, instead of 64);
+//   * the output accumulator is rescaled only when some lane's running maximum actually moved
+//     (wavefront-uniform test) — after the first few key tiles it almost never does;
+//   * exp2 is the bare v_exp_f32 (arguments are <= 0; results below 2^-126 may flush to zero);
+//   * K/V rows are fetched through a buffer descriptor that covers exactly this context, so rows past
+//     the sequence end read as zero without branches; masking code runs only on the tiles that
+//     touch the sequence end or the causal diagonal.
+// -------------------------------------------------------------------------------------------------
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+
+template <int DPAD, bool CAUSAL>
+__global__ __launch_bounds__(256) void attention_f32_fast_kernel(AttnArgs p)
+{
+    constexpr int BKV = 64;
+    constexpr int KS = DPAD + 4;   // K row stride (floats)
+    constexpr int VTS = BKV + 4;   // Vt row stride (floats): rows are head-dim indices, columns keys
+    constexpr int K_ELEMS = BKV * KS, V_ELEMS = DPAD * VTS;
+    constexpr int CHUNKS = DPAD / 8;
+    constexpr int DT = DPAD / 32;
+    constexpr int LOADS = BKV * DPAD / 4 / 256;
+    extern __shared__ __attribute__((aligned(16))) float attn_lds[];
+    float *Ks = attn_lds;                // [2][K_ELEMS]
+    float *Vt = attn_lds + 2 * K_ELEMS;  // [2][V_ELEMS]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int li = lane & 31, lh = lane >> 5;
+    const int S = p.S, D = p.D;
+
+    // Workgroup -> (context, query tile).  Workgroup ids are dealt round-robin to the 8 XCDs, so id & 7 picks
+    // the XCD; each XCD keeps its own slice of the contexts (their K/V stay in that XCD's L2).  Under the
+    // causal mask a query tile's cost grows with its index, so every XCD runs its tiles longest-first
+    // across ALL of its contexts (tile q_tiles-1 of every context, then q_tiles-2, ...): the short tiles at
+    // the end fill the gaps the long ones leave.
+    int ctx, q_tile;
+    if (p.swizzle) {
+        const int per_xcd = p.contexts >> 3;
+        const int xcd = blockIdx.x & 7, i = blockIdx.x >> 3;
+        if (CAUSAL) {
+            q_tile = p.q_tiles - 1 - i / per_xcd;
+            ctx = xcd * per_xcd + i % per_xcd;
+        } else {
+            ctx = xcd * per_xcd + i / p.q_tiles;
+            q_tile = i % p.q_tiles;
+        }
+    } else {
+        if (CAUSAL) {
+            q_tile = p.q_tiles - 1 - blockIdx.x / p.contexts;
+            ctx = blockIdx.x % p.contexts;
+        } else {
+            ctx = blockIdx.x / p.q_tiles;
+            q_tile = blockIdx.x % p.q_tiles;
+        }
+    }
+    const int q0 = q_tile * kBQ;
+    const int wq0 = q0 + wave * 32;
+    const int my_q = wq0 + li;
+    const size_t ctx_elem0 = static_cast<size_t>(ctx) * S * D;
+    const unsigned ctx_bytes = static_cast<unsigned>(S) * static_cast<unsigned>(D) * 4u;
+    const __amdgpu_buffer_rsrc_t rsrc_q =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.q + ctx_elem0), 0, static_cast<int>(ctx_bytes), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_k =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.k + ctx_elem0), 0, static_cast<int>(ctx_bytes), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_v =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.v + ctx_elem0), 0, static_cast<int>(ctx_bytes), 0x00020000);
+    const bool ragged_d = D != DPAD;  // chunks past head_dim must read as zero
+
+    auto fetch4 = [&](const __amdgpu_buffer_rsrc_t &rsrc, int row, int d) -> float4 {
+        const u32x4_t raw = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (static_cast<unsigned>(row) * D + d) * 4u, 0, 0);
+        float4 v = make_float4(__uint_as_float(raw.x), __uint_as_float(raw.y), __uint_as_float(raw.z), __uint_as_float(raw.w));
+        if (ragged_d && d >= D) v = make_float4(0.f, 0.f, 0.f, 0.f);
+        return v;
+    };
+
+    // Q fragments: qf[c][s] = Q[my_q][8c + 4h + s]; rows past the end read as zero.
+    float qf[CHUNKS][4];
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+        const float4 v = fetch4(rsrc_q, my_q, c * 8 + lh * 4);
+        qf[c][0] = v.x; qf[c][1] = v.y; qf[c][2] = v.z; qf[c][3] = v.w;
+    }
+
+    f32x16 oacc[DT];
+#pragma unroll
+    for (int t = 0; t < DT; ++t)
+        oacc[t] = f32x16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    float run_max = -INFINITY;
+    float run_sum = 0.0f;
+
+    const int key_end = CAUSAL ? min(S, q0 + kBQ) : S;
+    const int stages = (key_end + BKV - 1) / BKV;
+
+    float4 rk[LOADS], rv[LOADS];
+    auto load_global = [&](int key0) {
+#pragma unroll
+        for (int r = 0; r < LOADS; ++r) {
+            const int f = tid + 256 * r;
+            const int row = f / (DPAD / 4), c4 = (f % (DPAD / 4)) * 4;
+            rk[r] = fetch4(rsrc_k, key0 + row, c4);
+            rv[r] = fetch4(rsrc_v, key0 + row, c4);
+        }
+    };
+    auto store_lds = [&](int stage) {
+        float *ks = Ks + stage * K_ELEMS;
+        float *vt = Vt + stage * V_ELEMS;
+#pragma unroll
+        for (int r = 0; r < LOADS; ++r) {
+            const int f = tid + 256 * r;
+            const int row = f / (DPAD / 4), c4 = (f % (DPAD / 4)) * 4;
+            *reinterpret_cast<float4 *>(&ks[row * KS + c4]) = rk[r];
+            vt[(c4 + 0) * VTS + row] = rv[r].x;
+            vt[(c4 + 1) * VTS + row] = rv[r].y;
+            vt[(c4 + 2) * VTS + row] = rv[r].z;
+            vt[(c4 + 3) * VTS + row] = rv[r].w;
+        }
+    };
+
+    const float scale_log2e = p.scale * kLog2e;
+    // NT = number of 32-key tiles of this stage this wavefront works on (1 or 2).
+    auto compute = [&](auto nt_tag, int stage, int key0) {
+        constexpr int NT = decltype(nt_tag)::value;
+        const float *ks = Ks + stage * K_ELEMS;
+        const float *vt = Vt + stage * V_ELEMS;
+        f32x16 sacc[NT];
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+            sacc[t] = f32x16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < CHUNKS; ++c) {
+            float4 kv[NT];
+#pragma unroll
+            for (int t = 0; t < NT; ++t) kv[t] = *reinterpret_cast<const float4 *>(&ks[(t * 32 + li) * KS + c * 8 + lh * 4]);
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                sacc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(kv[t].x, qf[c][0], sacc[t], 0, 0, 0);
+                sacc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(kv[t].y, qf[c][1], sacc[t], 0, 0, 0);
+                sacc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(kv[t].z, qf[c][2], sacc[t], 0, 0, 0);
+                sacc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(kv[t].w, qf[c][3], sacc[t], 0, 0, 0);
+            }
+        }
+        // logits in log2 units; the masking code only runs where a tile crosses the sequence end or the diagonal
+        const bool need_mask = (key0 + NT * 32 > S) || (CAUSAL && key0 + NT * 32 - 1 > wq0);
+        float tile_max = -INFINITY;
+        if (need_mask) {
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int key = key0 + t * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
+                    float v = sacc[t][r] * scale_log2e;
+                    if (key >= S || (CAUSAL && key > my_q)) v = -INFINITY;
+                    sacc[t][r] = v;
+                    tile_max = fmaxf(tile_max, v);
+                }
+        } else {
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float v = sacc[t][r] * scale_log2e;
+                    sacc[t][r] = v;
+                    tile_max = fmaxf(tile_max, v);
+                }
+        }
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32));
+        const float new_max = fmaxf(run_max, tile_max);
+        const float safe_max = new_max == -INFINITY ? 0.0f : new_max;
+        if (__any(new_max != run_max)) {  // wavefront-uniform: some row's maximum moved
+            const float alpha = __builtin_amdgcn_exp2f(run_max - safe_max);  // run_max = -inf -> 0
+            run_sum *= alpha;
+#pragma unroll
+            for (int t = 0; t < DT; ++t)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) oacc[t][r] *= alpha;
+            run_max = new_max;
+        }
+        float tile_sum = 0.0f;
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float pr = __builtin_amdgcn_exp2f(sacc[t][r] - safe_max);
+                sacc[t][r] = pr;
+                tile_sum += pr;
+            }
+        run_sum += tile_sum;
+        // Oᵀ += Vᵀ·Pᵀ: for register group g the lane needs keys 8g + 4h .. +3 of its head-dim row: one 128-bit read.
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                float4 vv[DT];
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+                    vv[dt] = *reinterpret_cast<const float4 *>(&vt[(dt * 32 + li) * VTS + t * 32 + g * 8 + lh * 4]);
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+                    oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv[dt].x, sacc[t][g * 4 + 0], oacc[dt], 0, 0, 0);
+                    oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv[dt].y, sacc[t][g * 4 + 1], oacc[dt], 0, 0, 0);
+                    oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv[dt].z, sacc[t][g * 4 + 2], oacc[dt], 0, 0, 0);
+                    oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv[dt].w, sacc[t][g * 4 + 3], oacc[dt], 0, 0, 0);
+                }
+            }
+    };
+
+    if (stages > 0) {
+        load_global(0);
+        store_lds(0);
+    }
+    __syncthreads();
+    for (int t = 0; t < stages; ++t) {
+        const bool more = t + 1 < stages;
+        if (more) load_global((t + 1) * BKV);
+        const int key0 = t * BKV;
+        // Tiles entirely past the sequence end or (causal) entirely above this wavefront's rows are skipped.
+        const int limit = CAUSAL ? min(S, wq0 + 32) : S;
+        if (key0 + 32 < limit) compute(std::integral_constant<int, 2>{}, t & 1, key0);
+        else if (key0 < limit) compute(std::integral_constant<int, 1>{}, t & 1, key0);
+        if (more) store_lds((t + 1) & 1);
+        __syncthreads();
+    }
+
+    const float total = run_sum + __shfl_xor(run_sum, 32);
+    const float inv = total > 0.0f ? 1.0f / total : 0.0f;
+    if (my_q < S) {
+        float *orow = p.out + ctx_elem0 + static_cast<size_t>(my_q) * D;
+#pragma unroll
+        for (int t = 0; t < DT; ++t)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int d = t * 32 + g * 8 + lh * 4;
+                if (d < D)
+                    *reinterpret_cast<float4 *>(orow + d) = make_float4(oacc[t][g * 4 + 0] * inv, oacc[t][g * 4 + 1] * inv,
+                                                                        oacc[t][g * 4 + 2] * inv, oacc[t][g * 4 + 3] * inv);
+            }
+    }
+}
+
+template <int DPAD, bool CAUSAL>
+hipError_t launch_fast(const AttnArgs &args, hipStream_t stream)
+{
+    constexpr size_t lds_bytes = 2 * (static_cast<size_t>(64) * (DPAD + 4) + static_cast<size_t>(DPAD) * (64 + 4)) * sizeof(float);
+    auto kernel = attention_f32_fast_kernel<DPAD, CAUSAL>;
+    hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
+    if (rc != hipSuccess) return rc;
+    const size_t blocks = static_cast<size_t>(args.contexts) * args.q_tiles;
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), lds_bytes, stream, args);
+    return hipGetLastError();
+}
+
 template <int DPAD, int BKV, bool CAUSAL, bool BIAS, bool VEC>
 hipError_t launch_variant(const AttnArgs &args, hipStream_t stream)
 {
@@ -296,11 +557,18 @@ hipError_t launch_attention_f32(size_t contexts, size_t sequence, size_t head_di
     args.q_tiles = static_cast<int>((sequence + kBQ - 1) / kBQ);
     const size_t blocks = contexts * static_cast<size_t>(args.q_tiles);
     if (blocks > 0x7fffffffu) return hipErrorInvalidConfiguration;
-    args.swizzle = (blocks % 8 == 0) ? 1 : 0;
+    args.swizzle = (contexts % 8 == 0) ? 1 : 0;  // each XCD gets whole contexts
     args.scale = scale;
     const bool bias = z_bias != nullptr || attn_bias != nullptr;
     auto aligned = [](const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; };
     const bool vec = (head_dim % 4 == 0) && aligned(q) && aligned(k) && aligned(v) && aligned(out);
+    // The fast kernel addresses one context through a 32-bit buffer range.
+    const bool fits_buffer = sequence * head_dim * sizeof(float) < (1ull << 31);
+    if (!bias && vec && fits_buffer && head_dim <= 128) {
+        if (head_dim <= 32) return causal ? launch_fast<32, true>(args, stream) : launch_fast<32, false>(args, stream);
+        if (head_dim <= 64) return causal ? launch_fast<64, true>(args, stream) : launch_fast<64, false>(args, stream);
+        return causal ? launch_fast<128, true>(args, stream) : launch_fast<128, false>(args, stream);
+    }
     if (head_dim <= 32) return launch_dpad<32, 64>(args, causal, bias, vec, stream);
     if (head_dim <= 64) return launch_dpad<64, 64>(args, causal, bias, vec, stream);
     if (head_dim <= 128) return launch_dpad<128, 64>(args, causal, bias, vec, stream);
