@@ -35,18 +35,26 @@ struct ConvArgs {
 
 constexpr int kConvBK = 16;
 
-template <int BM, int BN, bool VEC>
-__global__ __launch_bounds__(256) void conv2d_f32_kernel(ConvArgs p)
+// FULLK: c_in*kh*kw is a multiple of the 16-wide k-tile and weight rows are 16-byte aligned, so the loop
+// carries no k bounds checks; weight rows past c_out are clamped to the last row (what they contribute
+// only reaches output channels that are never stored).
+template <int BM, int BN, int WM, int WN, bool VEC, bool FULLK>
+__global__ __launch_bounds__(64 * WM * WN) void conv2d_f32_kernel(ConvArgs p)
 {
-    constexpr int TM = BM / 64;  // wave tile = BM/2 output channels × BN/2 pixels
-    constexpr int TN = BN / 64;
-    static_assert(TN >= 1, "pixel tile must be at least 64 wide");
+    // WM×WN wavefronts, each owning (BM/WM) output channels × (BN/WN) pixels.  As in the f32 GEMM, many
+    // wavefronts with 32×32 tiles keep the (slow) f32 matrix pipe busier than few wavefronts with big tiles.
+    constexpr int T = 64 * WM * WN;
+    constexpr int WTM = BM / WM, WTN = BN / WN;
+    constexpr int TM = WTM / 32, TN = WTN / 32;
+    static_assert(TM >= 1 && TN >= 1, "wavefront tile must be at least 32×32");
+    static_assert(T % BN == 0 && (kConvBK * BN) % T == 0 && (BM * kConvBK / 4) % T == 0, "loader mapping");
     constexpr int A_STRIDE = kConvBK + 4;
     constexpr int B_STRIDE = BN + 8;
     constexpr int A_ELEMS = BM * A_STRIDE;
     constexpr int B_ELEMS = kConvBK * B_STRIDE;
-    constexpr int B_PER_THREAD = kConvBK * BN / 256;
-    constexpr int B_ROW_STEP = 256 / BN;
+    constexpr int B_PER_THREAD = kConvBK * BN / T;
+    constexpr int B_ROW_STEP = T / BN;
+    constexpr int A_LOADS = BM * kConvBK / 4 / T;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char conv_lds[];
     const int K = p.K;
@@ -58,7 +66,7 @@ __global__ __launch_bounds__(256) void conv2d_f32_kernel(ConvArgs p)
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / WN, wn = wave % WN;
     const int li = lane & 31, lh = lane >> 5;
 
     int bid = blockIdx.x;
@@ -71,7 +79,7 @@ __global__ __launch_bounds__(256) void conv2d_f32_kernel(ConvArgs p)
     const ConvShape &s = p.s;
     const int H = s.h, W = s.w;
     const int khw = s.kh * s.kw;
-    for (int k = tid; k < K; k += 256) {
+    for (int k = tid; k < K; k += T) {
         const int ic = k / khw, rem = k - ic * khw;
         const int ky = rem / s.kw, kx = rem - ky * s.kw;
         const int dy = ky * s.dil_h, dx = kx * s.dil_w;
@@ -97,13 +105,23 @@ __global__ __launch_bounds__(256) void conv2d_f32_kernel(ConvArgs p)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.0f;
 
-    float4 ra[TM];
+    float4 ra[A_LOADS];
     float rb[B_PER_THREAD];
 
+    const float *w_src[A_LOADS];
+#pragma unroll
+    for (int r = 0; r < A_LOADS; ++r) {
+        const int f = tid + T * r;
+        w_src[r] = p.weight + static_cast<size_t>(min(oc0 + (f >> 2), s.c_out - 1)) * K + (f & 3) * 4;
+    }
     auto load_global = [&](int k0) {
 #pragma unroll
-        for (int r = 0; r < TM; ++r) {
-            const int f = tid + 256 * r;
+        for (int r = 0; r < A_LOADS; ++r) {
+            if (FULLK) {
+                ra[r] = *reinterpret_cast<const float4 *>(w_src[r] + k0);
+                continue;
+            }
+            const int f = tid + T * r;
             const int row = f >> 2, c4 = (f & 3) * 4;
             float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
             if (oc0 + row < s.c_out) {
@@ -123,7 +141,7 @@ __global__ __launch_bounds__(256) void conv2d_f32_kernel(ConvArgs p)
         for (int r = 0; r < B_PER_THREAD; ++r) {
             const int k = k0 + krow0 + B_ROW_STEP * r;
             float v = 0.0f;
-            if (px_valid && k < K) {
+            if (px_valid && (FULLK || k < K)) {
                 const int2 e = lut[k];
                 const int iy = iy0 + (e.y & 0xffff);
                 const int ix = ix0 + (e.y >> 16);
@@ -138,8 +156,8 @@ __global__ __launch_bounds__(256) void conv2d_f32_kernel(ConvArgs p)
         float *as = As + stage * A_ELEMS;
         float *bs = Bs + stage * B_ELEMS;
 #pragma unroll
-        for (int r = 0; r < TM; ++r) {
-            const int f = tid + 256 * r;
+        for (int r = 0; r < A_LOADS; ++r) {
+            const int f = tid + T * r;
             const int row = f >> 2, c4 = (f & 3) * 4;
             *reinterpret_cast<float4 *>(&as[row * A_STRIDE + c4]) = ra[r];
         }
@@ -154,13 +172,13 @@ __global__ __launch_bounds__(256) void conv2d_f32_kernel(ConvArgs p)
             float a[TM][4], b[TN][4];
 #pragma unroll
             for (int tm = 0; tm < TM; ++tm) {
-                const int row = wm * (BM / 2) + tm * 32 + li;
+                const int row = wm * WTM + tm * 32 + li;
                 const float4 v = *reinterpret_cast<const float4 *>(&as[row * A_STRIDE + kk * 8 + lh * 4]);
                 a[tm][0] = v.x; a[tm][1] = v.y; a[tm][2] = v.z; a[tm][3] = v.w;
             }
 #pragma unroll
             for (int tn = 0; tn < TN; ++tn) {
-                const int col = wn * (BN / 2) + tn * 32 + li;
+                const int col = wn * WTN + tn * 32 + li;
 #pragma unroll
                 for (int t = 0; t < 4; ++t) b[tn][t] = bs[(kk * 8 + lh * 4 + t) * B_STRIDE + col];
             }
@@ -190,13 +208,13 @@ __global__ __launch_bounds__(256) void conv2d_f32_kernel(ConvArgs p)
     float *out_image = p.out + static_cast<size_t>(image) * s.c_out * p.spatial;
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn) {
-        const int col = px0 + wn * (BN / 2) + tn * 32 + li;
+        const int col = px0 + wn * WTN + tn * 32 + li;
         if (col >= p.spatial) continue;
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int oc = oc0 + wm * (BM / 2) + tm * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
+                const int oc = oc0 + wm * WTM + tm * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
                 if (oc >= s.c_out) continue;
                 float value = acc[tm][tn][r];
                 if (p.bias) value += p.bias[oc];
@@ -206,7 +224,7 @@ __global__ __launch_bounds__(256) void conv2d_f32_kernel(ConvArgs p)
     }
 }
 
-template <int BM, int BN>
+template <int BM, int BN, int WM, int WN>
 hipError_t launch_tile(ConvArgs args, bool vec, hipStream_t stream)
 {
     args.tiles_oc = (args.s.c_out + BM - 1) / BM;
@@ -217,21 +235,22 @@ hipError_t launch_tile(ConvArgs args, bool vec, hipStream_t stream)
     const size_t lds_bytes = k_padded * sizeof(int2) +
                              2 * (static_cast<size_t>(BM) * (kConvBK + 4) + static_cast<size_t>(kConvBK) * (BN + 8)) * sizeof(float);
     const dim3 grid(static_cast<unsigned>(tiles));
-    const dim3 block(256);
+    const dim3 block(64 * WM * WN);
     hipError_t rc;
-    if (vec) {
-        auto kernel = conv2d_f32_kernel<BM, BN, true>;
-        rc = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                 static_cast<int>(lds_bytes));
-        if (rc != hipSuccess) return rc;
+    auto launch = [&](auto kernel) -> hipError_t {
+        hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
+        if (status != hipSuccess) return status;
         hipLaunchKernelGGL(kernel, grid, block, lds_bytes, stream, args);
-    } else {
-        auto kernel = conv2d_f32_kernel<BM, BN, false>;
-        rc = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                 static_cast<int>(lds_bytes));
-        if (rc != hipSuccess) return rc;
-        hipLaunchKernelGGL(kernel, grid, block, lds_bytes, stream, args);
-    }
+        return hipSuccess;
+    };
+    if (vec && args.K % kConvBK == 0)
+        rc = launch(conv2d_f32_kernel<BM, BN, WM, WN, true, true>);
+    else if (vec)
+        rc = launch(conv2d_f32_kernel<BM, BN, WM, WN, true, false>);
+    else
+        rc = launch(conv2d_f32_kernel<BM, BN, WM, WN, false, false>);
+    if (rc != hipSuccess) return rc;
     return hipGetLastError();
 }
 
@@ -256,8 +275,8 @@ hipError_t launch_conv2d_f32(const ConvShape &shape, int activation, const float
         (shape.kw - 1) * static_cast<long long>(shape.dil_w) > 0x7fff || args.K > kConvMaxReduction)
         return hipErrorInvalidValue;
     const bool vec = (args.K % 4 == 0) && ((reinterpret_cast<uintptr_t>(weight) & 15u) == 0);
-    if (shape.c_out > 64) return launch_tile<128, 64>(args, vec, stream);
-    return launch_tile<64, 64>(args, vec, stream);
+    if (shape.c_out > 64) return launch_tile<128, 64, 4, 2>(args, vec, stream);
+    return launch_tile<64, 64, 2, 2>(args, vec, stream);
 }
 
 }  // namespace sthip

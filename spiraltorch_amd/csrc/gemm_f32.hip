@@ -4,9 +4,12 @@
 // Replaces rocBLAS sgemm + st_gemm_epilogue_f32 in crates/st-backend-hip/src/real.rs:598-646,817-957
 // and crates/st-backend-hip/src/hip_kernels/hip_gemm_epilogue.cu:19-71.
 //
-// Tiling: one 256-thread workgroup (4 wavefronts, 2×2) owns a BM×BN tile of C and walks K in steps of
-// 16 through two LDS stages; global loads for step t+1 are issued into registers before the MFMAs of
-// step t and written to the other stage afterwards, so a step costs one barrier.
+// Tiling: a workgroup of WM×WN wavefronts owns a BM×BN tile of C and walks K in steps of 16 through two
+// LDS stages; global loads for step t+1 are issued into registers before the MFMAs of step t and written
+// to the other stage afterwards, so a step costs one barrier.  The f32 MFMA is slow (64 cycles for
+// 32x32x2) and needs two LDS values per lane, so register blocking buys nothing here; what keeps the
+// matrix pipe busy is MANY wavefronts with small tiles (measured: 32×32 or 64×64 per wavefront, 4 to 16
+// wavefronts per workgroup, beat 2×2 wavefronts with 64×64 tiles by 1.5×).
 //
 // MFMA operand layout (32x32x2): lane l supplies A[l%32][l/32] and B[l/32][l%32]; accumulator register
 // r of lane l is C[(r/4)*8 + (l/32)*4 + r%4][l%32].  Because the sum over k is order-free, each group
@@ -51,22 +54,26 @@ __device__ __forceinline__ float4 load_row4(const float *base, size_t row_offset
     return v;
 }
 
-template <int BM, int BN, bool AT, bool VEC>
-__global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32Args p)
+template <int BM, int BN, int WM, int WN, bool AT, bool VEC>
+__global__ __launch_bounds__(64 * WM * WN) void gemm_f32_kernel(GemmF32Args p)
 {
-    constexpr int TM = BM / 64;  // 32×32 MFMA tiles per wavefront along M (wave tile = BM/2 × BN/2)
-    constexpr int TN = BN / 64;
+    constexpr int T = 64 * WM * WN;
+    constexpr int WTM = BM / WM, WTN = BN / WN;  // wavefront tile
+    constexpr int TM = WTM / 32, TN = WTN / 32;  // 32×32 MFMA tiles per wavefront
+    static_assert(TM >= 1 && TN >= 1, "wavefront tile must be at least 32×32");
     constexpr int A_STRIDE = AT ? (BM + 8) : (kBK + 4);
     constexpr int A_ELEMS = AT ? kBK * A_STRIDE : BM * A_STRIDE;
     constexpr int B_STRIDE = BN + 8;
     constexpr int B_ELEMS = kBK * B_STRIDE;
+    constexpr int A_VECS = BM * kBK / 4, B_VECS = kBK * BN / 4;  // float4 per stage
+    constexpr int A_LOADS = (A_VECS + T - 1) / T, B_LOADS = (B_VECS + T - 1) / T;
     __shared__ __attribute__((aligned(16))) float As[2][A_ELEMS];
     __shared__ __attribute__((aligned(16))) float Bs[2][B_ELEMS];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / WN, wn = wave % WN;
     const int li = lane & 31, lh = lane >> 5;
     const int tile_m = blockIdx.x / p.tiles_n, tile_n = blockIdx.x % p.tiles_n;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
@@ -77,15 +84,53 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32Args p)
     for (int a = 0; a < TM; ++a)
 #pragma unroll
         for (int b = 0; b < TN; ++b)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.0f;
+            acc[a][b] = f32x16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
-    float4 ra[TM], rb[TN];
+    float4 ra[A_LOADS], rb[B_LOADS];
 
-    auto load_global = [&](int k0) {
+    // Fast-path source pointers (k-tile 0): rows/columns outside the matrix are clamped to the last valid
+    // one instead of being masked — what they load only reaches output elements that are never stored.
+    // Only a ragged last k-tile needs real zero-fill, and it takes the checked path below.
+    const float *a_src[A_LOADS];
+    const float *b_src[B_LOADS];
+    if (VEC) {
 #pragma unroll
-        for (int r = 0; r < TM; ++r) {
-            const int f = tid + 256 * r;
+        for (int r = 0; r < A_LOADS; ++r) {
+            const int f = tid + T * r;
+            if (!AT) {
+                const int row = min(m0 + (f >> 2), M - 1), c4 = (f & 3) * 4;
+                a_src[r] = p.A + static_cast<size_t>(row) * K + c4;
+            } else {
+                const int krow = f / (BM / 4), col = min(m0 + (f % (BM / 4)) * 4, M - 4);
+                a_src[r] = p.A + static_cast<size_t>(krow) * M + col;
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < B_LOADS; ++r) {
+            const int f = tid + T * r;
+            const int krow = f / (BN / 4), col = min(n0 + (f % (BN / 4)) * 4, N - 4);
+            b_src[r] = p.B + static_cast<size_t>(krow) * N + col;
+        }
+    }
+    const int full_steps = K / kBK;  // k-tiles that lie completely inside K
+
+    auto load_fast = [&](int k0) {
+#pragma unroll
+        for (int r = 0; r < A_LOADS; ++r) {
+            if (A_VECS % T != 0 && tid + T * r >= A_VECS) continue;
+            ra[r] = *reinterpret_cast<const float4 *>(a_src[r] + (AT ? static_cast<size_t>(k0) * M : static_cast<size_t>(k0)));
+        }
+#pragma unroll
+        for (int r = 0; r < B_LOADS; ++r) {
+            if (B_VECS % T != 0 && tid + T * r >= B_VECS) continue;
+            rb[r] = *reinterpret_cast<const float4 *>(b_src[r] + static_cast<size_t>(k0) * N);
+        }
+    };
+    auto load_checked = [&](int k0) {
+#pragma unroll
+        for (int r = 0; r < A_LOADS; ++r) {
+            const int f = tid + T * r;
+            if (A_VECS % T != 0 && f >= A_VECS) continue;
             if (!AT) {
                 const int row = f >> 2, c4 = (f & 3) * 4;
                 ra[r] = load_row4<VEC>(p.A, static_cast<size_t>(m0 + row) * K, k0 + c4, K, m0 + row < M);
@@ -95,16 +140,18 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32Args p)
             }
         }
 #pragma unroll
-        for (int r = 0; r < TN; ++r) {
-            const int f = tid + 256 * r;
+        for (int r = 0; r < B_LOADS; ++r) {
+            const int f = tid + T * r;
+            if (B_VECS % T != 0 && f >= B_VECS) continue;
             const int krow = f / (BN / 4), c4 = (f % (BN / 4)) * 4;
             rb[r] = load_row4<VEC>(p.B, static_cast<size_t>(k0 + krow) * N, n0 + c4, N, k0 + krow < K);
         }
     };
     auto store_lds = [&](int stage) {
 #pragma unroll
-        for (int r = 0; r < TM; ++r) {
-            const int f = tid + 256 * r;
+        for (int r = 0; r < A_LOADS; ++r) {
+            const int f = tid + T * r;
+            if (A_VECS % T != 0 && f >= A_VECS) continue;
             if (!AT) {
                 const int row = f >> 2, c4 = (f & 3) * 4;
                 *reinterpret_cast<float4 *>(&As[stage][row * A_STRIDE + c4]) = ra[r];
@@ -114,8 +161,9 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32Args p)
             }
         }
 #pragma unroll
-        for (int r = 0; r < TN; ++r) {
-            const int f = tid + 256 * r;
+        for (int r = 0; r < B_LOADS; ++r) {
+            const int f = tid + T * r;
+            if (B_VECS % T != 0 && f >= B_VECS) continue;
             const int krow = f / (BN / 4), c4 = (f % (BN / 4)) * 4;
             *reinterpret_cast<float4 *>(&Bs[stage][krow * B_STRIDE + c4]) = rb[r];
         }
@@ -128,7 +176,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32Args p)
             float a[TM][4], b[TN][4];
 #pragma unroll
             for (int tm = 0; tm < TM; ++tm) {
-                const int row = wm * (BM / 2) + tm * 32 + li;
+                const int row = wm * WTM + tm * 32 + li;
                 if (!AT) {
                     const float4 v = *reinterpret_cast<const float4 *>(&as[row * A_STRIDE + kk * 8 + lh * 4]);
                     a[tm][0] = v.x; a[tm][1] = v.y; a[tm][2] = v.z; a[tm][3] = v.w;
@@ -139,7 +187,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32Args p)
             }
 #pragma unroll
             for (int tn = 0; tn < TN; ++tn) {
-                const int col = wn * (BN / 2) + tn * 32 + li;
+                const int col = wn * WTN + tn * 32 + li;
 #pragma unroll
                 for (int s = 0; s < 4; ++s) b[tn][s] = bs[(kk * 8 + lh * 4 + s) * B_STRIDE + col];
             }
@@ -155,13 +203,23 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32Args p)
 
     const int steps = (K + kBK - 1) / kBK;
     if (steps > 0) {
-        load_global(0);
+        if (VEC && full_steps > 0) load_fast(0); else load_checked(0);
         store_lds(0);
     }
     __syncthreads();
-    for (int t = 0; t < steps; ++t) {
+    int t = 0;
+    if (VEC) {
+        // Steady state: the next k-tile lies completely inside K, so its loads need no checks.
+        for (; t + 1 < full_steps; ++t) {
+            load_fast((t + 1) * kBK);
+            compute(t & 1);
+            store_lds((t + 1) & 1);
+            __syncthreads();
+        }
+    }
+    for (; t < steps; ++t) {
         const bool more = t + 1 < steps;
-        if (more) load_global((t + 1) * kBK);
+        if (more) load_checked((t + 1) * kBK);
         compute(t & 1);
         if (more) store_lds((t + 1) & 1);
         __syncthreads();
@@ -171,44 +229,46 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32Args p)
     const bool scaled = p.scale != 1.0f;
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn) {
-        const int col = n0 + wn * (BN / 2) + tn * 32 + li;
-        if (col >= N) continue;
-        const float bias = p.bias ? p.bias[col] : 0.0f;
+        const int col = n0 + wn * WTN + tn * 32 + li;
+        const bool col_ok = col < N;
+        const float bias = (p.bias && col_ok) ? p.bias[col] : 0.0f;
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm) {
+            const f32x16 tile = acc[tm][tn];
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int row = m0 + wm * (BM / 2) + tm * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
-                if (row >= M) continue;
-                const size_t idx = static_cast<size_t>(row) * N + col;
-                float value = acc[tm][tn][r];
-                if (scaled) value *= p.scale;
-                if (p.bias) value += bias;
-                if (p.residual) value += p.residual[idx];
-                p.C[idx] = apply_activation(value, p.activation);
+                const int row = m0 + wm * WTM + tm * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
+                if (col_ok && row < M) {
+                    const size_t idx = static_cast<size_t>(row) * N + col;
+                    float value = tile[r];
+                    if (scaled) value *= p.scale;
+                    value += bias;
+                    if (p.residual) value += p.residual[idx];
+                    p.C[idx] = apply_activation(value, p.activation);
+                }
             }
         }
     }
 }
 
-template <int BM, int BN>
+template <int BM, int BN, int WM, int WN>
 hipError_t launch_tile(GemmF32Args args, bool lhs_transposed, bool vec, hipStream_t stream)
 {
     args.tiles_n = (args.N + BN - 1) / BN;
     const size_t tiles = static_cast<size_t>(args.tiles_n) * static_cast<size_t>((args.M + BM - 1) / BM);
     if (tiles > 0x7fffffffu) return hipErrorInvalidConfiguration;
     const dim3 grid(static_cast<unsigned>(tiles));
-    const dim3 block(256);
+    const dim3 block(64 * WM * WN);
     if (lhs_transposed) {
         if (vec)
-            hipLaunchKernelGGL((gemm_f32_kernel<BM, BN, true, true>), grid, block, 0, stream, args);
+            hipLaunchKernelGGL((gemm_f32_kernel<BM, BN, WM, WN, true, true>), grid, block, 0, stream, args);
         else
-            hipLaunchKernelGGL((gemm_f32_kernel<BM, BN, true, false>), grid, block, 0, stream, args);
+            hipLaunchKernelGGL((gemm_f32_kernel<BM, BN, WM, WN, true, false>), grid, block, 0, stream, args);
     } else {
         if (vec)
-            hipLaunchKernelGGL((gemm_f32_kernel<BM, BN, false, true>), grid, block, 0, stream, args);
+            hipLaunchKernelGGL((gemm_f32_kernel<BM, BN, WM, WN, false, true>), grid, block, 0, stream, args);
         else
-            hipLaunchKernelGGL((gemm_f32_kernel<BM, BN, false, false>), grid, block, 0, stream, args);
+            hipLaunchKernelGGL((gemm_f32_kernel<BM, BN, WM, WN, false, false>), grid, block, 0, stream, args);
     }
     return hipGetLastError();
 }
@@ -235,11 +295,12 @@ hipError_t launch_gemm_f32(size_t m, size_t n, size_t k, bool lhs_transposed, co
     // 128-bit global loads need every row start 16-byte aligned.
     const size_t lhs_ld = lhs_transposed ? m : k;
     const bool vec = (lhs_ld % 4 == 0) && (n % 4 == 0) && aligned16(lhs) && aligned16(rhs);
-    // Large tiles once they give every compute unit at least one workgroup, otherwise small tiles so
-    // that small problems still spread over the chip.
-    const size_t big_tiles = ((m + 127) / 128) * ((n + 127) / 128);
-    if (big_tiles >= 256) return launch_tile<128, 128>(args, lhs_transposed, vec, stream);
-    return launch_tile<64, 64>(args, lhs_transposed, vec, stream);
+    // 256×256 tiles (16 wavefronts of 64×64) once they give every compute unit a full tile without padding
+    // waste; otherwise 64×64 tiles (4 wavefronts of 32×32), which spread small and narrow problems over the chip.
+    const size_t big_tiles = ((m + 255) / 256) * ((n + 255) / 256);
+    const bool little_padding = (m % 256 == 0 || m >= 2048) && (n % 256 == 0 || n >= 2048);
+    if (big_tiles >= 256 && little_padding) return launch_tile<256, 256, 4, 4>(args, lhs_transposed, vec, stream);
+    return launch_tile<64, 64, 2, 2>(args, lhs_transposed, vec, stream);
 }
 
 }  // namespace sthip
