@@ -167,6 +167,21 @@ def wl_decoder(hip, inputs, timer, warmup, steps):
     return out
 
 
+def wl_calibration(hip, inputs, timer, warmup, steps):
+    """Plain streaming kernel of known traffic (f32 -> bf16 rounding of 64 Mi values: 256 MiB read, 128 MiB
+    written).  It anchors the FETCH_SIZE / WRITE_SIZE counters and shows the HBM rate a trivial kernel reaches."""
+    count = 64 * 1024 * 1024
+    d_src = hip.DeviceBuffer(count * 4)
+    d_src.zero()
+    d_dst = hip.DeviceBuffer(count * 2)
+
+    def step(stream):
+        hip.f32_to_bf16_dev(count, d_src, d_dst, stream)
+
+    wall, ev = timer.run(step, warmup, steps)
+    return entry("calibration_f32_to_bf16_64mi", "f32", 0, count * 6, "hbm", wall, ev)
+
+
 # ---- CPU baseline ---------------------------------------------------------------------------------------
 
 def cpu_baseline_conv(conv_inputs):
@@ -220,6 +235,7 @@ def main():
         ("attention_noncausal", lambda: wl_attention(hip, inputs, timer, 2, 5, False)),
         ("attention_causal", lambda: wl_attention(hip, inputs, timer, 2, 5, True)),
         ("decoder", lambda: wl_decoder(hip, inputs, timer, 2, 5)),
+        ("calibration", lambda: wl_calibration(hip, inputs, timer, 2, 5)),
     ]
     for name, fn in plan:
         if args.only and args.only not in name:

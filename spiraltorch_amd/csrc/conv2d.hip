@@ -30,15 +30,15 @@ struct ConvArgs {
     int K;        // c_in * kh * kw
     int spatial;  // oh * ow
     int tiles_px, tiles_oc;
+    int xcd_swizzle;
     int activation;
 };
 
-constexpr int kConvBK = 16;
 
 // FULLK: c_in*kh*kw is a multiple of the 16-wide k-tile and weight rows are 16-byte aligned, so the loop
 // carries no k bounds checks; weight rows past c_out are clamped to the last row (what they contribute
 // only reaches output channels that are never stored).
-template <int BM, int BN, int WM, int WN, bool VEC, bool FULLK>
+template <int BM, int BN, int BK, int WM, int WN, bool VEC, bool FULLK>
 __global__ __launch_bounds__(64 * WM * WN) void conv2d_f32_kernel(ConvArgs p)
 {
     // WM×WN wavefronts, each owning (BM/WM) output channels × (BN/WN) pixels.  As in the f32 GEMM, many
@@ -47,14 +47,14 @@ __global__ __launch_bounds__(64 * WM * WN) void conv2d_f32_kernel(ConvArgs p)
     constexpr int WTM = BM / WM, WTN = BN / WN;
     constexpr int TM = WTM / 32, TN = WTN / 32;
     static_assert(TM >= 1 && TN >= 1, "wavefront tile must be at least 32×32");
-    static_assert(T % BN == 0 && (kConvBK * BN) % T == 0 && (BM * kConvBK / 4) % T == 0, "loader mapping");
-    constexpr int A_STRIDE = kConvBK + 4;
+    static_assert(T % BN == 0 && (BK * BN) % T == 0 && (BM * BK / 4) % T == 0, "loader mapping");
+    constexpr int A_STRIDE = BK + 4;
     constexpr int B_STRIDE = BN + 8;
     constexpr int A_ELEMS = BM * A_STRIDE;
-    constexpr int B_ELEMS = kConvBK * B_STRIDE;
-    constexpr int B_PER_THREAD = kConvBK * BN / T;
+    constexpr int B_ELEMS = BK * B_STRIDE;
+    constexpr int B_PER_THREAD = BK * BN / T;
     constexpr int B_ROW_STEP = T / BN;
-    constexpr int A_LOADS = BM * kConvBK / 4 / T;
+    constexpr int A_LOADS = BM * BK / 4 / T;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char conv_lds[];
     const int K = p.K;
@@ -69,7 +69,10 @@ __global__ __launch_bounds__(64 * WM * WN) void conv2d_f32_kernel(ConvArgs p)
     const int wm = wave / WN, wn = wave % WN;
     const int li = lane & 31, lh = lane >> 5;
 
+    // Workgroup ids are dealt round-robin to the 8 XCDs (id & 7).  When the batch divides by 8 every XCD
+    // keeps whole images, so an image (and its halo re-reads) is fetched into one L2 only.
     int bid = blockIdx.x;
+    if (p.xcd_swizzle) bid = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
     const int tile_oc = bid % p.tiles_oc;
     bid /= p.tiles_oc;
     const int tile_px = bid % p.tiles_px;
@@ -168,7 +171,7 @@ __global__ __launch_bounds__(64 * WM * WN) void conv2d_f32_kernel(ConvArgs p)
         const float *as = As + stage * A_ELEMS;
         const float *bs = Bs + stage * B_ELEMS;
 #pragma unroll
-        for (int kk = 0; kk < kConvBK / 8; ++kk) {
+        for (int kk = 0; kk < BK / 8; ++kk) {
             float a[TM][4], b[TN][4];
 #pragma unroll
             for (int tm = 0; tm < TM; ++tm) {
@@ -193,13 +196,13 @@ __global__ __launch_bounds__(64 * WM * WN) void conv2d_f32_kernel(ConvArgs p)
     };
 
     __syncthreads();  // offset table complete
-    const int steps = (K + kConvBK - 1) / kConvBK;
+    const int steps = (K + BK - 1) / BK;
     load_global(0);
     store_lds(0);
     __syncthreads();
     for (int t = 0; t < steps; ++t) {
         const bool more = t + 1 < steps;
-        if (more) load_global((t + 1) * kConvBK);
+        if (more) load_global((t + 1) * BK);
         compute(t & 1);
         if (more) store_lds((t + 1) & 1);
         __syncthreads();
@@ -224,16 +227,17 @@ __global__ __launch_bounds__(64 * WM * WN) void conv2d_f32_kernel(ConvArgs p)
     }
 }
 
-template <int BM, int BN, int WM, int WN>
+template <int BM, int BN, int BK, int WM, int WN>
 hipError_t launch_tile(ConvArgs args, bool vec, hipStream_t stream)
 {
     args.tiles_oc = (args.s.c_out + BM - 1) / BM;
     args.tiles_px = (args.spatial + BN - 1) / BN;
     const size_t tiles = static_cast<size_t>(args.tiles_oc) * args.tiles_px * static_cast<size_t>(args.s.batch);
     if (tiles > 0x7fffffffu) return hipErrorInvalidConfiguration;
+    args.xcd_swizzle = (args.s.batch % 8 == 0) ? 1 : 0;
     const size_t k_padded = (static_cast<size_t>(args.K) + 15) & ~static_cast<size_t>(15);
     const size_t lds_bytes = k_padded * sizeof(int2) +
-                             2 * (static_cast<size_t>(BM) * (kConvBK + 4) + static_cast<size_t>(kConvBK) * (BN + 8)) * sizeof(float);
+                             2 * (static_cast<size_t>(BM) * (BK + 4) + static_cast<size_t>(BK) * (BN + 8)) * sizeof(float);
     const dim3 grid(static_cast<unsigned>(tiles));
     const dim3 block(64 * WM * WN);
     hipError_t rc;
@@ -244,12 +248,12 @@ hipError_t launch_tile(ConvArgs args, bool vec, hipStream_t stream)
         hipLaunchKernelGGL(kernel, grid, block, lds_bytes, stream, args);
         return hipSuccess;
     };
-    if (vec && args.K % kConvBK == 0)
-        rc = launch(conv2d_f32_kernel<BM, BN, WM, WN, true, true>);
+    if (vec && args.K % BK == 0)
+        rc = launch(conv2d_f32_kernel<BM, BN, BK, WM, WN, true, true>);
     else if (vec)
-        rc = launch(conv2d_f32_kernel<BM, BN, WM, WN, true, false>);
+        rc = launch(conv2d_f32_kernel<BM, BN, BK, WM, WN, true, false>);
     else
-        rc = launch(conv2d_f32_kernel<BM, BN, WM, WN, false, false>);
+        rc = launch(conv2d_f32_kernel<BM, BN, BK, WM, WN, false, false>);
     if (rc != hipSuccess) return rc;
     return hipGetLastError();
 }
@@ -269,14 +273,17 @@ hipError_t launch_conv2d_f32(const ConvShape &shape, int activation, const float
     args.K = shape.c_in * shape.kh * shape.kw;
     args.spatial = shape.oh * shape.ow;
     args.tiles_px = args.tiles_oc = 0;
+    args.xcd_swizzle = 0;
     args.activation = activation;
     // The offset table packs ky*dh and kx*dw into 16 bits each.
     if ((shape.kh - 1) * static_cast<long long>(shape.dil_h) > 0x7fff ||
         (shape.kw - 1) * static_cast<long long>(shape.dil_w) > 0x7fff || args.K > kConvMaxReduction)
         return hipErrorInvalidValue;
     const bool vec = (args.K % 4 == 0) && ((reinterpret_cast<uintptr_t>(weight) & 15u) == 0);
-    if (shape.c_out > 64) return launch_tile<128, 64, 4, 2>(args, vec, stream);
-    return launch_tile<64, 64, 2, 2>(args, vec, stream);
+    // 8 wavefronts of 32×32 per 128×64 tile measured best for wide layers (128×128 tiles, 32-deep k-tiles and
+    // 4-wavefront layouts were all 10-20 % slower on the 64->128 channel 56×56 case).
+    if (shape.c_out > 64) return launch_tile<128, 64, 16, 4, 2>(args, vec, stream);
+    return launch_tile<64, 64, 16, 2, 2>(args, vec, stream);
 }
 
 }  // namespace sthip
