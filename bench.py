@@ -32,6 +32,16 @@ sys.path.insert(0, ROOT)
 PEAK_TFLOPS = {"f32": 157.3, "bf16": 2500.0}
 PEAK_HBM_GBS = 8000.0
 
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch; FETCH_SIZE
+# scaled x2.0 and WRITE_SIZE x1.0, the factors a streaming kernel of known size gives on this chip).  The
+# summaries live in profiles/dominant_kernels_counters.md; workloads not listed there report null.
+MEASURED_TRAFFIC_BYTES = {
+    "conv2d_bias_relu_f32_n32_c64to128_56x56_k3s1p1": (13958 * 2 + 50176) * 1024,
+    "gemm_bf16_f32acc_4096x4096x4096": (98422 * 2 + 65536) * 1024,
+    "gemm_bf16_f32acc_16x4096x4096": (16924 * 2 + 4096) * 1024,
+    "attention_f32_b8_h16_s2048_d64_noncausal": (98387 * 2 + 65536) * 1024,
+}
+
 
 def log(*items):
     print(*items, file=sys.stderr, flush=True)
@@ -76,6 +86,7 @@ def entry(name, dtype, flops, bytes_, bound, wall_ms, event_ms, extra=None):
            "ms_per_step": round(wall_ms, 5), "kernel_ms_per_step": round(event_ms, 5),
            "gflops": round(flops / (wall_ms * 1e-3) / 1e9, 1),
            "roofline": roofline(bound, "bf16" if dtype == "bf16" else "f32", flops, bytes_, event_ms)}
+    out["roofline"]["traffic"] = MEASURED_TRAFFIC_BYTES.get(name)
     if extra:
         out.update(extra)
     return out
@@ -142,6 +153,24 @@ def wl_attention(hip, inputs, timer, warmup, steps, causal):
     flops = 4 * dim * contexts * (seq * (seq + 1) // 2 if causal else seq * seq)
     name = "attention_f32_b8_h16_s2048_d64_" + ("causal" if causal else "noncausal")
     return entry(name, "f32", flops, 4 * 4 * count, "mfma", wall, ev)
+
+
+def wl_attention_bf16(hip, inputs, timer, warmup, steps):
+    """The decoder's attention on its own: batch 16, 8 heads, seq 1024, head_dim 64, causal, bf16 operands read
+    in place from a fused (tokens, 3*512) projection."""
+    batch, heads, seq, dim = 16, 8, 1024, 64
+    width = heads * dim
+    qkv = inputs.to_bf16(inputs.normal(inputs.seed_for(5, 2), batch * seq * 3 * width))
+    d_qkv = hip.DeviceBuffer.from_array(qkv)
+    d_out = hip.DeviceBuffer(batch * seq * width * 2)
+
+    def step(stream):
+        hip.attention_bf16_dev(batch, heads, seq, dim, 0.125, True, d_qkv, d_qkv.at(width * 2), d_qkv.at(width * 4),
+                               3 * width, d_out, width, stream)
+
+    wall, ev = timer.run(step, warmup, steps)
+    flops = 4 * dim * batch * heads * (seq * (seq + 1) // 2)
+    return entry("attention_bf16_b16_h8_s1024_d64_causal", "bf16", flops, 2 * 4 * batch * seq * width, "mfma", wall, ev)
 
 
 def wl_decoder(hip, inputs, timer, warmup, steps):
@@ -234,6 +263,7 @@ def main():
                                                   "gemm_bf16_f32acc_16x4096x4096", "hbm")),
         ("attention_noncausal", lambda: wl_attention(hip, inputs, timer, 2, 5, False)),
         ("attention_causal", lambda: wl_attention(hip, inputs, timer, 2, 5, True)),
+        ("attention_bf16", lambda: wl_attention_bf16(hip, inputs, timer, side_warm, side_steps)),
         ("decoder", lambda: wl_decoder(hip, inputs, timer, 2, 5)),
         ("calibration", lambda: wl_calibration(hip, inputs, timer, 2, 5)),
     ]

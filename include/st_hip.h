@@ -154,6 +154,19 @@ int st_hip_conv2d_bias_act_f32_dev(size_t batch, size_t c_in, size_t h, size_t w
 int st_hip_attention_f32_dev(size_t contexts, size_t sequence, size_t head_dim, float scale,
                              int causal, const float *q, const float *k, const float *v,
                              const float *z_bias, const float *attn_bias, float *out, void *stream);
+/* Attention on bf16 operands (both matrix products take bf16 inputs and accumulate in f32; the softmax
+ * stays in f32; the result is rounded nearest-even to bf16), same recurrence as
+ * crates/st-tensor/src/pure.rs:11845-11919 with `causal` limiting keys to 0..=query.  Heads are read in place
+ * from row-major (batch*sequence, ld_in) matrices: context (b, h) owns columns h*head_dim .. +head_dim-1 of rows
+ * b*sequence .. b*sequence+sequence-1 of q, k and v (the head slicing of
+ * crates/st-vision/src/models/vit.rs:151-180), and writes the same columns of `out` (row stride ld_out).
+ * A fused [Q | K | V] projection is passed as q = qkv, k = qkv + heads*head_dim, v = qkv + 2*heads*head_dim,
+ * ld_in = 3*heads*head_dim; a (contexts*sequence, head_dim) layout as batch = contexts, heads = 1.
+ * head_dim must be 64 or 128, ld_in a multiple of 8, ld_out a multiple of 4, q/k/v 16-byte aligned, out
+ * 8-byte aligned; anything else returns ST_HIP_ERR_UNSUPPORTED. */
+int st_hip_attention_bf16_dev(size_t batch, size_t heads, size_t sequence, size_t head_dim, float scale,
+                              int causal, const uint16_t *q, const uint16_t *k, const uint16_t *v,
+                              size_t ld_in, uint16_t *out, size_t ld_out, void *stream);
 
 /* Row-wise building blocks of the decoder stack.
  * layer_norm: crates/st-tensor/src/pure.rs:4008-4058; writes f32 and/or bf16 (either may be NULL).

@@ -439,7 +439,10 @@ int st_oracle_embedding_f32(size_t tokens, size_t vocab, size_t dim, const float
  * crates/st-vision/src/models/vit.rs:256-265: h = x + Attn(LN1(x)); y = h + FC2(GELU(FC1(LN2(h))))).
  * Linear layers follow crates/st-nn/src/layers/linear.rs:49-64,96-104: W is (in, out), y = x·W + b.
  * Rounding points of the bf16 build: every GEMM rounds BOTH operands to bf16 (RNE) and accumulates
- * in f32; bias, residual, GELU, layer-norm and attention run in f32.
+ * in f32; bias, residual, GELU and layer-norm run in f32.  The attention's q, k and v are GEMM operands
+ * as well and are rounded to bf16 after the projection's bias add; its softmax recurrence runs in f32
+ * (a device kernel that also rounds the softmax weights to bf16 before the value product differs from
+ * this by rounding noise only).
  * ---------------------------------------------------------------------------------------------- */
 size_t st_oracle_decoder_weight_count(const st_oracle_decoder_config *c)
 {
@@ -520,6 +523,9 @@ int st_oracle_decoder_forward(const st_oracle_decoder_config *cfg, const float *
         if (rc) goto done;
         rc = linear_bf16(T, d, 3 * d, h, w_qkv, b_qkv, NULL, ST_ORACLE_ACT_NONE, qkv, threads);
         if (rc) goto done;
+        /* The attention's two matrix products are GEMMs too: their q, k, v inputs are rounded to bf16
+         * like every other GEMM operand (the softmax and the weighted sum stay in f32 here). */
+        for (size_t i = 0; i < T * 3 * d; ++i) qkv[i] = bf16_bits_to_f32(f32_to_bf16_bits(qkv[i]));
         /* (B·S, 3·H·D) -> three (B·H·S, D) tensors; column blocks are [Q | K | V], heads are
          * contiguous head_dim-wide slices (vit.rs:151-180). */
         for (size_t b = 0; b < batch; ++b)

@@ -90,6 +90,8 @@ SIGNATURES = {
                                                                  c_void_p]),
     "st_hip_attention_f32_dev": (c_int, [c_size_t, c_size_t, c_size_t, c_float, c_int, c_void_p, c_void_p, c_void_p,
                                          c_void_p, c_void_p, c_void_p, c_void_p]),
+    "st_hip_attention_bf16_dev": (c_int, [c_size_t, c_size_t, c_size_t, c_size_t, c_float, c_int, c_void_p, c_void_p,
+                                          c_void_p, c_size_t, c_void_p, c_size_t, c_void_p]),
     "st_hip_layer_norm_f32_dev": (c_int, [c_size_t, c_size_t, c_void_p, c_void_p, c_void_p, c_void_p, c_float,
                                           c_void_p, c_void_p, c_void_p]),
     "st_hip_embedding_f32_dev": (c_int, [c_size_t, c_size_t, c_size_t, c_void_p, c_void_p, c_void_p, c_void_p]),

@@ -1,0 +1,324 @@
+// Scaled-dot-product attention with online softmax on bf16 operands (gfx950), used by the decoder stack.
+//
+// Same mathematics as crates/st-tensor/src/pure.rs:11845-11919 (per query: softmax over keys of
+// q·k·scale, weighted sum of value rows, optional causal key range 0..=query), with the two matrix
+// products taking bf16 inputs and accumulating in f32 on v_mfma_f32_32x32x16_bf16; the softmax itself
+// (maximum, exponentials, sums, final division) stays in f32.  Heads are read in place from row-major
+// (batch·sequence, width) matrices — context (b, h) owns columns h·D .. h·D+D-1 of rows b·S .. b·S+S-1,
+// the layout crates/st-vision/src/models/vit.rs:151-180 indexes — so a fused [Q | K | V] projection output is
+// consumed without a split pass and the result lands directly in the (tokens, heads·D) matrix the
+// output projection reads.
+//
+// The kernel computes the transposed problem, Sᵀ = K·Qᵀ and Oᵀ += Vᵀ·Pᵀ: every lane then owns one query
+// column, so the running maximum and sum are per-lane scalars and the probabilities leave the first
+// product's accumulators already in the register layout the second product's B operand needs (no
+// shuffle, no LDS round trip).  The accumulator of a 32x32 tile hands lane half h the keys
+// {8a + 4h + c}; the second product wants eight consecutive k-indices per lane, so V is staged
+// transposed with key bits 2 and 3 swapped, which makes those eight keys one 128-bit LDS read.
+#include "device_math.h"
+#include "kernels.h"
+
+#include <type_traits>
+
+namespace sthip {
+
+namespace {
+
+struct AttnBf16Args {
+    const uint16_t *q;
+    const uint16_t *k;
+    const uint16_t *v;
+    uint16_t *out;
+    int batch, heads, S;
+    int ld_in, ld_out;  // row strides in elements
+    int q_tiles;
+    int swizzle;
+    float scale;
+};
+
+constexpr int kBQ16 = 128;
+constexpr float kLog2e16 = 1.4426950408889634f;
+
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ unsigned pack_bf16x2(float lo, float hi)
+{
+    const bf16x2_t v = {static_cast<__bf16>(lo), static_cast<__bf16>(hi)};  // round-to-nearest-even
+    return __builtin_bit_cast(unsigned, v);
+}
+
+template <int D, bool CAUSAL>
+__global__ __launch_bounds__(256) void attention_bf16_kernel(AttnBf16Args p)
+{
+    constexpr int BKV = 64;
+    constexpr int KS = D + 8;      // K row stride (elements): 16 bytes of padding keep 128-bit reads conflict-free
+    constexpr int VTS = BKV + 8;   // Vt row stride: rows are head-dim indices, columns (permuted) keys
+    constexpr int K_ELEMS = BKV * KS, V_ELEMS = D * VTS;
+    constexpr int KC = D / 16;     // k-blocks of K·Qᵀ
+    constexpr int DT = D / 32;     // 32-row tiles of Oᵀ
+    constexpr int LOADS = BKV * D / 8 / 256;
+    extern __shared__ __attribute__((aligned(16))) uint16_t attn16_lds[];
+    uint16_t *Ks = attn16_lds;                // [2][K_ELEMS]
+    uint16_t *Vt = attn16_lds + 2 * K_ELEMS;  // [2][V_ELEMS]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int li = lane & 31, lh = lane >> 5;
+    const int S = p.S;
+    const int contexts = p.batch * p.heads;
+
+    // Workgroup -> (context, query tile): each XCD (workgroup id mod 8) keeps whole contexts so their K/V
+    // stay in its L2; causal tiles run longest-first across all contexts of the XCD.
+    int ctx, q_tile;
+    if (p.swizzle) {
+        const int per_xcd = contexts >> 3;
+        const int xcd = blockIdx.x & 7, i = blockIdx.x >> 3;
+        if (CAUSAL) {
+            q_tile = p.q_tiles - 1 - i / per_xcd;
+            ctx = xcd * per_xcd + i % per_xcd;
+        } else {
+            ctx = xcd * per_xcd + i / p.q_tiles;
+            q_tile = i % p.q_tiles;
+        }
+    } else {
+        if (CAUSAL) {
+            q_tile = p.q_tiles - 1 - blockIdx.x / contexts;
+            ctx = blockIdx.x % contexts;
+        } else {
+            ctx = blockIdx.x / p.q_tiles;
+            q_tile = blockIdx.x % p.q_tiles;
+        }
+    }
+    const int q0 = q_tile * kBQ16;
+    const int wq0 = q0 + wave * 32;
+    const int my_q = wq0 + li;
+    const int b = ctx / p.heads, h = ctx % p.heads;
+    const size_t in_base = static_cast<size_t>(b) * S * p.ld_in + static_cast<size_t>(h) * D;
+    // One descriptor per operand covering exactly this context's rows: rows past the end read as zero.
+    const unsigned in_bytes = (static_cast<unsigned>(S - 1) * static_cast<unsigned>(p.ld_in) + D) * 2u;
+    const __amdgpu_buffer_rsrc_t rsrc_q =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(p.q + in_base), 0, static_cast<int>(in_bytes), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_k =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(p.k + in_base), 0, static_cast<int>(in_bytes), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_v =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(p.v + in_base), 0, static_cast<int>(in_bytes), 0x00020000);
+
+    auto fetch8 = [&](const __amdgpu_buffer_rsrc_t &rsrc, int row, int d) -> u32x4_t {
+        return __builtin_amdgcn_raw_buffer_load_b128(
+            rsrc, (static_cast<unsigned>(row) * static_cast<unsigned>(p.ld_in) + d) * 2u, 0, 0);
+    };
+
+    // Qᵀ fragments (B operand): lane (li, lh) holds Q[my_q][16c + 8·lh .. +7].
+    bf16x8 qf[KC];
+#pragma unroll
+    for (int c = 0; c < KC; ++c) qf[c] = __builtin_bit_cast(bf16x8, fetch8(rsrc_q, my_q, c * 16 + lh * 8));
+
+    f32x16 oacc[DT];
+#pragma unroll
+    for (int t = 0; t < DT; ++t)
+        oacc[t] = f32x16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    float run_max = -INFINITY;
+    float run_sum = 0.0f;
+
+    const int key_end = CAUSAL ? min(S, q0 + kBQ16) : S;
+    const int stages = (key_end + BKV - 1) / BKV;
+
+    u32x4_t rk[LOADS], rv[LOADS];
+    auto load_global = [&](int key0) {
+#pragma unroll
+        for (int r = 0; r < LOADS; ++r) {
+            const int f = tid + 256 * r;
+            const int row = f / (D / 8), c8 = (f % (D / 8)) * 8;
+            rk[r] = fetch8(rsrc_k, key0 + row, c8);
+            rv[r] = fetch8(rsrc_v, key0 + row, c8);
+        }
+    };
+    auto store_lds = [&](int stage) {
+        uint16_t *ks = Ks + stage * K_ELEMS;
+        uint16_t *vt = Vt + stage * V_ELEMS;
+#pragma unroll
+        for (int r = 0; r < LOADS; ++r) {
+            const int f = tid + 256 * r;
+            const int row = f / (D / 8), c8 = (f % (D / 8)) * 8;
+            *reinterpret_cast<u32x4_t *>(&ks[row * KS + c8]) = rk[r];
+            const int pos = (row & ~12) | ((row & 4) << 1) | ((row & 8) >> 1);  // key bits 2 and 3 swapped
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                vt[(c8 + 2 * e + 0) * VTS + pos] = static_cast<uint16_t>(rv[r][e] & 0xffffu);
+                vt[(c8 + 2 * e + 1) * VTS + pos] = static_cast<uint16_t>(rv[r][e] >> 16);
+            }
+        }
+    };
+
+    const float scale_log2e = p.scale * kLog2e16;
+    // NT = number of 32-key tiles of this stage this wavefront works on (1 or 2).
+    auto compute = [&](auto nt_tag, int stage, int key0) {
+        constexpr int NT = decltype(nt_tag)::value;
+        const uint16_t *ks = Ks + stage * K_ELEMS;
+        const uint16_t *vt = Vt + stage * V_ELEMS;
+        f32x16 sacc[NT];
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+            sacc[t] = f32x16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < KC; ++c) {
+            bf16x8 kf[NT];
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+                kf[t] = *reinterpret_cast<const bf16x8 *>(&ks[(t * 32 + li) * KS + c * 16 + lh * 8]);
+#pragma unroll
+            for (int t = 0; t < NT; ++t) sacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[t], qf[c], sacc[t], 0, 0, 0);
+        }
+        // logits in log2 units; masking only where a tile crosses the sequence end or the diagonal
+        const bool need_mask = (key0 + NT * 32 > S) || (CAUSAL && key0 + NT * 32 - 1 > wq0);
+        float tile_max = -INFINITY;
+        if (need_mask) {
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int key = key0 + t * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
+                    float v = sacc[t][r] * scale_log2e;
+                    if (key >= S || (CAUSAL && key > my_q)) v = -INFINITY;
+                    sacc[t][r] = v;
+                    tile_max = fmaxf(tile_max, v);
+                }
+        } else {
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float v = sacc[t][r] * scale_log2e;
+                    sacc[t][r] = v;
+                    tile_max = fmaxf(tile_max, v);
+                }
+        }
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32));
+        const float new_max = fmaxf(run_max, tile_max);
+        const float safe_max = new_max == -INFINITY ? 0.0f : new_max;
+        if (__any(new_max != run_max)) {  // wavefront-uniform: some query's maximum moved
+            const float alpha = __builtin_amdgcn_exp2f(run_max - safe_max);  // run_max = -inf -> 0
+            run_sum *= alpha;
+#pragma unroll
+            for (int t = 0; t < DT; ++t)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) oacc[t][r] *= alpha;
+            run_max = new_max;
+        }
+        float tile_sum = 0.0f;
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float pr = __builtin_amdgcn_exp2f(sacc[t][r] - safe_max);
+                sacc[t][r] = pr;
+                tile_sum += pr;
+            }
+        run_sum += tile_sum;
+        // Oᵀ += Vᵀ·Pᵀ, 16 keys per MFMA: accumulator registers 8j .. 8j+7 are this lane's k-indices 8·lh .. 8·lh+7.
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                u32x4_t packed;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) packed[e] = pack_bf16x2(sacc[t][8 * j + 2 * e], sacc[t][8 * j + 2 * e + 1]);
+                const bf16x8 pf = __builtin_bit_cast(bf16x8, packed);
+                bf16x8 vf[DT];
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+                    vf[dt] = *reinterpret_cast<const bf16x8 *>(&vt[(dt * 32 + li) * VTS + t * 32 + j * 16 + lh * 8]);
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[dt], pf, oacc[dt], 0, 0, 0);
+            }
+    };
+
+    if (stages > 0) {
+        load_global(0);
+        store_lds(0);
+    }
+    __syncthreads();
+    for (int t = 0; t < stages; ++t) {
+        const bool more = t + 1 < stages;
+        if (more) load_global((t + 1) * BKV);
+        const int key0 = t * BKV;
+        // Tiles entirely past the sequence end or (causal) entirely above this wavefront's rows are skipped.
+        const int limit = CAUSAL ? min(S, wq0 + 32) : S;
+        if (key0 + 32 < limit) compute(std::integral_constant<int, 2>{}, t & 1, key0);
+        else if (key0 < limit) compute(std::integral_constant<int, 1>{}, t & 1, key0);
+        if (more) store_lds((t + 1) & 1);
+        __syncthreads();
+    }
+
+    const float total = run_sum + __shfl_xor(run_sum, 32);
+    const float inv = total > 0.0f ? 1.0f / total : 0.0f;
+    if (my_q < S) {
+        uint16_t *orow = p.out + (static_cast<size_t>(b) * S + my_q) * p.ld_out + static_cast<size_t>(h) * D;
+#pragma unroll
+        for (int t = 0; t < DT; ++t)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int d = t * 32 + g * 8 + lh * 4;
+                u32x2_t packed;
+                packed[0] = pack_bf16x2(oacc[t][g * 4 + 0] * inv, oacc[t][g * 4 + 1] * inv);
+                packed[1] = pack_bf16x2(oacc[t][g * 4 + 2] * inv, oacc[t][g * 4 + 3] * inv);
+                *reinterpret_cast<u32x2_t *>(orow + d) = packed;
+            }
+    }
+}
+
+template <int D, bool CAUSAL>
+hipError_t launch_variant(const AttnBf16Args &args, hipStream_t stream)
+{
+    constexpr size_t lds_bytes = 2 * (static_cast<size_t>(64) * (D + 8) + static_cast<size_t>(D) * (64 + 8)) * sizeof(uint16_t);
+    auto kernel = attention_bf16_kernel<D, CAUSAL>;
+    hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
+    if (rc != hipSuccess) return rc;
+    const size_t blocks = static_cast<size_t>(args.batch) * args.heads * args.q_tiles;
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), lds_bytes, stream, args);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+bool attention_bf16_supported(size_t sequence, size_t head_dim, size_t ld_in, size_t ld_out, const void *q,
+                              const void *k, const void *v, const void *out)
+{
+    auto aligned = [](const void *ptr, uintptr_t a) { return (reinterpret_cast<uintptr_t>(ptr) & (a - 1)) == 0; };
+    if (head_dim != 64 && head_dim != 128) return false;
+    if (ld_in % 8 != 0 || ld_out % 4 != 0) return false;
+    if (!aligned(q, 16) || !aligned(k, 16) || !aligned(v, 16) || !aligned(out, 8)) return false;
+    // one context is addressed through a 32-bit byte offset
+    return sequence == 0 || ((sequence - 1) * ld_in + head_dim) * 2 < (1ull << 31);
+}
+
+hipError_t launch_attention_bf16(size_t batch, size_t heads, size_t sequence, size_t head_dim, float scale, bool causal,
+                                 const uint16_t *q, const uint16_t *k, const uint16_t *v, size_t ld_in, uint16_t *out,
+                                 size_t ld_out, hipStream_t stream)
+{
+    if (batch == 0 || heads == 0 || sequence == 0) return hipSuccess;
+    if (!attention_bf16_supported(sequence, head_dim, ld_in, ld_out, q, k, v, out)) return hipErrorInvalidValue;
+    AttnBf16Args args;
+    args.q = q;
+    args.k = k;
+    args.v = v;
+    args.out = out;
+    args.batch = static_cast<int>(batch);
+    args.heads = static_cast<int>(heads);
+    args.S = static_cast<int>(sequence);
+    args.ld_in = static_cast<int>(ld_in);
+    args.ld_out = static_cast<int>(ld_out);
+    args.q_tiles = static_cast<int>((sequence + kBQ16 - 1) / kBQ16);
+    const size_t contexts = batch * heads;
+    if (contexts * static_cast<size_t>(args.q_tiles) > 0x7fffffffu) return hipErrorInvalidConfiguration;
+    args.swizzle = (contexts % 8 == 0) ? 1 : 0;
+    args.scale = scale;
+    if (head_dim == 64) return causal ? launch_variant<64, true>(args, stream) : launch_variant<64, false>(args, stream);
+    return causal ? launch_variant<128, true>(args, stream) : launch_variant<128, false>(args, stream);
+}
+
+}  // namespace sthip

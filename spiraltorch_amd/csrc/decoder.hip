@@ -3,7 +3,9 @@
 // (h = x + Attn(LN1(x)); y = h + FC2(GELU(FC1(LN2(h))))), linear layers follow
 // crates/st-nn/src/layers/linear.rs:49-64,96-104 (W is (in, out), y = x·W + b).
 // Every GEMM takes bf16 operands (weights rounded once at creation, activations rounded by the
-// producing kernel) and accumulates in f32; layer-norm, attention, bias, residual and GELU run in f32.
+// producing kernel) and accumulates in f32 — including the two matrix products inside the attention,
+// whose q, k, v are the bf16 output of the fused projection; layer-norm, softmax, bias, residual and
+// GELU run in f32.
 #include <new>
 #include <vector>
 
@@ -27,7 +29,8 @@ struct Decoder {
     uint16_t *w_head = nullptr;
     // activations
     float *x = nullptr, *x2 = nullptr, *qkv = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *ctx = nullptr;
-    uint16_t *h16 = nullptr, *attn16 = nullptr, *u16 = nullptr;
+    uint16_t *h16 = nullptr, *attn16 = nullptr, *u16 = nullptr, *qkv16 = nullptr;
+    bool fused_attention = false;  // bf16 attention straight from the fused [Q | K | V] projection
 
     ~Decoder()
     {
@@ -141,11 +144,17 @@ int st_hip_decoder_create(const st_hip_decoder_config *config, const float *host
 
     if (status == ST_HIP_OK) status = dec->alloc(&dec->x, tokens * d);
     if (status == ST_HIP_OK) status = dec->alloc(&dec->x2, tokens * d);
-    if (status == ST_HIP_OK) status = dec->alloc(&dec->qkv, tokens * 3 * d);
-    if (status == ST_HIP_OK) status = dec->alloc(&dec->q, tokens * d);
-    if (status == ST_HIP_OK) status = dec->alloc(&dec->k, tokens * d);
-    if (status == ST_HIP_OK) status = dec->alloc(&dec->v, tokens * d);
-    if (status == ST_HIP_OK) status = dec->alloc(&dec->ctx, tokens * d);
+    const size_t head_dim = d / config->heads;
+    dec->fused_attention = (head_dim == 64 || head_dim == 128) && ((config->seq - 1) * 3 * d + head_dim) * 2 < (1ull << 31);
+    if (dec->fused_attention) {
+        if (status == ST_HIP_OK) status = dec->alloc(&dec->qkv16, tokens * 3 * d);
+    } else {
+        if (status == ST_HIP_OK) status = dec->alloc(&dec->qkv, tokens * 3 * d);
+        if (status == ST_HIP_OK) status = dec->alloc(&dec->q, tokens * d);
+        if (status == ST_HIP_OK) status = dec->alloc(&dec->k, tokens * d);
+        if (status == ST_HIP_OK) status = dec->alloc(&dec->v, tokens * d);
+        if (status == ST_HIP_OK) status = dec->alloc(&dec->ctx, tokens * d);
+    }
     if (status == ST_HIP_OK) status = dec->alloc(&dec->h16, tokens * d);
     if (status == ST_HIP_OK) status = dec->alloc(&dec->attn16, tokens * d);
     if (status == ST_HIP_OK) status = dec->alloc(&dec->u16, tokens * ff);
@@ -184,14 +193,24 @@ int st_hip_decoder_forward_dev(void *decoder, const float *tokens, float *logits
                   "layer_norm launch");
         ep = GemmEpilogue();
         ep.bias = w.b_qkv;
-        ST_LAUNCH(launch_gemm_bf16(T, 3 * d, d, dec.h16, w.w_qkv, dec.qkv, nullptr, ep, stream), "qkv gemm launch");
-        ST_LAUNCH(launch_split_heads_f32(c.batch, c.seq, heads, hd, dec.qkv, dec.q, dec.k, dec.v, stream),
-                  "split_heads launch");
-        ST_LAUNCH(launch_attention_f32(c.batch * heads, c.seq, hd, scale, true, dec.q, dec.k, dec.v, nullptr, nullptr,
-                                       dec.ctx, stream),
-                  "attention launch");
-        ST_LAUNCH(launch_merge_heads_f32(c.batch, c.seq, heads, hd, dec.ctx, nullptr, dec.attn16, stream),
-                  "merge_heads launch");
+        if (dec.fused_attention) {
+            // q, k, v leave the projection as bf16 and are consumed in place, head by head.
+            ST_LAUNCH(launch_gemm_bf16(T, 3 * d, d, dec.h16, w.w_qkv, nullptr, dec.qkv16, ep, stream), "qkv gemm launch");
+            ST_LAUNCH(launch_attention_bf16(c.batch, heads, c.seq, hd, scale, true, dec.qkv16, dec.qkv16 + d,
+                                            dec.qkv16 + 2 * d, 3 * d, dec.attn16, d, stream),
+                      "attention launch");
+        } else {
+            // Head sizes the bf16 kernel does not cover: same rounding points (q, k, v rounded to bf16,
+            // attention output rounded to bf16), carried out by the f32 attention kernel.
+            ST_LAUNCH(launch_gemm_bf16(T, 3 * d, d, dec.h16, w.w_qkv, dec.qkv, nullptr, ep, stream), "qkv gemm launch");
+            ST_LAUNCH(launch_split_heads_f32(c.batch, c.seq, heads, hd, dec.qkv, dec.q, dec.k, dec.v, true, stream),
+                      "split_heads launch");
+            ST_LAUNCH(launch_attention_f32(c.batch * heads, c.seq, hd, scale, true, dec.q, dec.k, dec.v, nullptr,
+                                           nullptr, dec.ctx, stream),
+                      "attention launch");
+            ST_LAUNCH(launch_merge_heads_f32(c.batch, c.seq, heads, hd, dec.ctx, nullptr, dec.attn16, stream),
+                      "merge_heads launch");
+        }
         ep = GemmEpilogue();
         ep.bias = w.b_o;
         ep.residual = dec.x;

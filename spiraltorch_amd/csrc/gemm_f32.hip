@@ -29,7 +29,7 @@ struct GemmF32Args {
     const float *bias;
     const float *residual;
     int M, N, K;
-    int tiles_n;  // tiles along N; the grid is one-dimensional over (tile_m, tile_n)
+    int tiles_m, tiles_n;  // the grid is one-dimensional over (tile_m, tile_n)
     float scale;
     int activation;
 };
@@ -75,7 +75,16 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_f32_kernel(GemmF32Args p)
     const int wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
     const int li = lane & 31, lh = lane >> 5;
-    const int tile_m = blockIdx.x / p.tiles_n, tile_n = blockIdx.x % p.tiles_n;
+    // Workgroup ids go round-robin over the 8 XCDs, each with its own L2.  Give every XCD one contiguous run of
+    // tile ids, and walk the tiles in groups of GROUP_M tile-rows (column by column inside a group), so the
+    // tiles resident on one XCD at a time share their A row panels and B column panels through that L2.
+    constexpr int GROUP_M = BM >= 256 ? 4 : 8;
+    const int grid = static_cast<int>(gridDim.x), xcd = static_cast<int>(blockIdx.x) & 7;
+    const int tile_id = xcd * (grid >> 3) + min(xcd, grid & 7) + (static_cast<int>(blockIdx.x) >> 3);
+    const int group_size = GROUP_M * p.tiles_n;
+    const int first_m = (tile_id / group_size) * GROUP_M, in_group = tile_id % group_size;
+    const int group_rows = min(p.tiles_m - first_m, GROUP_M);
+    const int tile_m = first_m + in_group % group_rows, tile_n = in_group / group_rows;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int M = p.M, N = p.N, K = p.K;
 
@@ -255,7 +264,8 @@ template <int BM, int BN, int WM, int WN>
 hipError_t launch_tile(GemmF32Args args, bool lhs_transposed, bool vec, hipStream_t stream)
 {
     args.tiles_n = (args.N + BN - 1) / BN;
-    const size_t tiles = static_cast<size_t>(args.tiles_n) * static_cast<size_t>((args.M + BM - 1) / BM);
+    args.tiles_m = (args.M + BM - 1) / BM;
+    const size_t tiles = static_cast<size_t>(args.tiles_n) * static_cast<size_t>(args.tiles_m);
     if (tiles > 0x7fffffffu) return hipErrorInvalidConfiguration;
     const dim3 grid(static_cast<unsigned>(tiles));
     const dim3 block(64 * WM * WN);

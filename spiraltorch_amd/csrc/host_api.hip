@@ -588,6 +588,37 @@ int st_hip_attention_f32_dev(size_t contexts, size_t sequence, size_t head_dim, 
                          "attention launch");
 }
 
+int st_hip_attention_bf16_dev(size_t batch, size_t heads, size_t sequence, size_t head_dim, float scale, int causal,
+                              const uint16_t *q, const uint16_t *k, const uint16_t *v, size_t ld_in, uint16_t *out,
+                              size_t ld_out, void *stream)
+{
+    ST_HIP_CHECK(ensure_init());
+    size_t contexts = 0, width = 0;
+    if (!checked_mul(batch, heads, &contexts) || !checked_mul(heads, head_dim, &width))
+        return fail(ST_HIP_ERR_INVALID, "attention dimensions overflow");
+    AttentionPlan plan;
+    ST_HIP_CHECK(plan_attention(contexts, sequence, head_dim, &plan));
+    if (!std::isfinite(scale))
+        return fail(ST_HIP_ERR_NONFINITE, "non-finite value encountered in scaled_dot_attention_scale: %g",
+                    static_cast<double>(scale));
+    if (plan.rows == 0 || head_dim == 0) return ST_HIP_OK;
+    ST_HIP_CHECK(check_attention_kernel_limits(contexts, sequence, head_dim));
+    if (!q || !k || !v || !out)
+        return fail(ST_HIP_ERR_INVALID, "attention received a null pointer; provide contiguous buffers");
+    if (ld_in < width || ld_out < width)
+        return fail(ST_HIP_ERR_INVALID, "attention row stride %zu/%zu is smaller than heads*head_dim=%zu", ld_in, ld_out,
+                    width);
+    if (ld_in > kMaxDim || ld_out > kMaxDim) return fail(ST_HIP_ERR_UNSUPPORTED, "attention row stride exceeds i32");
+    if (!attention_bf16_supported(sequence, head_dim, ld_in, ld_out, q, k, v, out))
+        return fail(ST_HIP_ERR_UNSUPPORTED,
+                    "bf16 attention needs head_dim 64 or 128 (got %zu), ld_in %% 8 == 0, ld_out %% 4 == 0 and aligned "
+                    "buffers",
+                    head_dim);
+    return launch_status(launch_attention_bf16(batch, heads, sequence, head_dim, scale, causal != 0, q, k, v, ld_in, out,
+                                               ld_out, as_stream(stream)),
+                         "attention launch");
+}
+
 int st_hip_layer_norm_f32_dev(size_t rows, size_t cols, const float *x, const float *residual, const float *gamma,
                               const float *beta, float epsilon, float *out_f32, uint16_t *out_bf16, void *stream)
 {
@@ -632,7 +663,7 @@ int st_hip_split_heads_f32_dev(size_t batch, size_t seq, size_t heads, size_t he
         return fail(ST_HIP_ERR_UNSUPPORTED, "split_heads volume exceeds i32");
     if (total == 0) return ST_HIP_OK;
     if (!qkv || !q || !k || !v) return fail(ST_HIP_ERR_INVALID, "split_heads received a null pointer");
-    return launch_status(launch_split_heads_f32(batch, seq, heads, head_dim, qkv, q, k, v, as_stream(stream)),
+    return launch_status(launch_split_heads_f32(batch, seq, heads, head_dim, qkv, q, k, v, false, as_stream(stream)),
                          "split_heads launch");
 }
 

@@ -39,6 +39,13 @@ hipError_t launch_attention_f32(size_t contexts, size_t sequence, size_t head_di
                                 const float *z_bias, const float *attn_bias, float *out,
                                 hipStream_t stream);
 
+// bf16 attention over heads stored as column slices of (batch·sequence, ld) matrices; head_dim 64 or 128.
+bool attention_bf16_supported(size_t sequence, size_t head_dim, size_t ld_in, size_t ld_out, const void *q,
+                              const void *k, const void *v, const void *out);
+hipError_t launch_attention_bf16(size_t batch, size_t heads, size_t sequence, size_t head_dim, float scale,
+                                 bool causal, const uint16_t *q, const uint16_t *k, const uint16_t *v,
+                                 size_t ld_in, uint16_t *out, size_t ld_out, hipStream_t stream);
+
 hipError_t launch_layer_norm_f32(size_t rows, size_t cols, const float *x, const float *residual,
                                  const float *gamma, const float *beta, float epsilon, float *out_f32,
                                  uint16_t *out_bf16, hipStream_t stream);
@@ -46,7 +53,8 @@ hipError_t launch_embedding_f32(size_t tokens, size_t vocab, size_t dim, const f
                                 const float *table, float *out, hipStream_t stream);
 hipError_t launch_f32_to_bf16(size_t count, const float *in, uint16_t *out, hipStream_t stream);
 hipError_t launch_split_heads_f32(size_t batch, size_t seq, size_t heads, size_t head_dim,
-                                  const float *qkv, float *q, float *k, float *v, hipStream_t stream);
+                                  const float *qkv, float *q, float *k, float *v, bool round_to_bf16,
+                                  hipStream_t stream);
 hipError_t launch_merge_heads_f32(size_t batch, size_t seq, size_t heads, size_t head_dim,
                                   const float *contexts_in, float *out_f32, uint16_t *out_bf16,
                                   hipStream_t stream);

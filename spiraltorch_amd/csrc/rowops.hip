@@ -72,9 +72,13 @@ __global__ __launch_bounds__(256) void f32_to_bf16_kernel(size_t count, const fl
 }
 
 // qkv (B·S, 3·H·D) with column blocks [Q | K | V] -> q, k, v each (B·H·S, D).
+template <bool ROUND_BF16>
 __global__ __launch_bounds__(256) void split_heads_kernel(int batch, int seq, int heads, int dim, const float *qkv,
                                                           float *q, float *k, float *v)
 {
+    auto keep = [](float x) {
+        return ROUND_BF16 ? __uint_as_float(static_cast<uint32_t>(f32_to_bf16_rne(x)) << 16) : x;
+    };
     const size_t total = static_cast<size_t>(batch) * seq * heads * dim;
     const size_t stride = static_cast<size_t>(gridDim.x) * 256;
     const int width = heads * dim;
@@ -86,9 +90,9 @@ __global__ __launch_bounds__(256) void split_heads_kernel(int batch, int seq, in
         const int h = static_cast<int>(rest % heads);
         const int b = static_cast<int>(rest / heads);
         const size_t src = (static_cast<size_t>(b) * seq + s) * 3 * width + static_cast<size_t>(h) * dim + d;
-        q[i] = qkv[src];
-        k[i] = qkv[src + width];
-        v[i] = qkv[src + 2 * width];
+        q[i] = keep(qkv[src]);
+        k[i] = keep(qkv[src + width]);
+        v[i] = keep(qkv[src + 2 * width]);
     }
 }
 
@@ -148,12 +152,16 @@ hipError_t launch_f32_to_bf16(size_t count, const float *in, uint16_t *out, hipS
 }
 
 hipError_t launch_split_heads_f32(size_t batch, size_t seq, size_t heads, size_t head_dim, const float *qkv, float *q,
-                                  float *k, float *v, hipStream_t stream)
+                                  float *k, float *v, bool round_to_bf16, hipStream_t stream)
 {
     const size_t total = batch * seq * heads * head_dim;
     if (total == 0) return hipSuccess;
-    hipLaunchKernelGGL(split_heads_kernel, dim3(grid_for(total)), dim3(256), 0, stream, static_cast<int>(batch),
-                       static_cast<int>(seq), static_cast<int>(heads), static_cast<int>(head_dim), qkv, q, k, v);
+    if (round_to_bf16)
+        hipLaunchKernelGGL(split_heads_kernel<true>, dim3(grid_for(total)), dim3(256), 0, stream, static_cast<int>(batch),
+                           static_cast<int>(seq), static_cast<int>(heads), static_cast<int>(head_dim), qkv, q, k, v);
+    else
+        hipLaunchKernelGGL(split_heads_kernel<false>, dim3(grid_for(total)), dim3(256), 0, stream, static_cast<int>(batch),
+                           static_cast<int>(seq), static_cast<int>(heads), static_cast<int>(head_dim), qkv, q, k, v);
     return hipGetLastError();
 }
 

@@ -196,6 +196,12 @@ class DeviceBuffer:
                                              _stream_ptr(stream)))
         return out
 
+    def at(self, byte_offset: int) -> int:
+        """Device address `byte_offset` bytes into the allocation (for entry points that take sub-ranges)."""
+        if not 0 <= byte_offset <= self.nbytes:
+            raise ValueError("offset outside the device buffer")
+        return int(self.ptr.value) + int(byte_offset)
+
     def zero(self, stream=None) -> None:
         _check(_lib.load().st_hip_memset_zero(self.ptr, self.nbytes, _stream_ptr(stream)))
 
@@ -308,6 +314,14 @@ def attention_f32_dev(contexts, sequence, head_dim, scale, causal, q, k, v, z_bi
     _check(_lib.load().st_hip_attention_f32_dev(contexts, sequence, head_dim, scale, int(bool(causal)), _dev(q),
                                                 _dev(k), _dev(v), _dev(z_bias), _dev(attn_bias), _dev(out),
                                                 _stream_ptr(stream)))
+
+
+def attention_bf16_dev(batch, heads, sequence, head_dim, scale, causal, q, k, v, ld_in, out, ld_out,
+                       stream=None) -> None:
+    """bf16 attention over heads stored as column slices of (batch*sequence, ld) matrices; q/k/v/out are
+    DeviceBuffers or raw device addresses (DeviceBuffer.at) of bf16 bit patterns."""
+    _check(_lib.load().st_hip_attention_bf16_dev(batch, heads, sequence, head_dim, scale, int(bool(causal)), _dev(q),
+                                                 _dev(k), _dev(v), ld_in, _dev(out), ld_out, _stream_ptr(stream)))
 
 
 def layer_norm_f32_dev(rows, cols, x, residual, gamma, beta, epsilon, out_f32, out_bf16, stream=None) -> None:
