@@ -13,7 +13,6 @@
 // MFMA operand layout (32x32x16): lane l supplies A[l%32][8*(l/32) .. +7] and B[8*(l/32) .. +7][l%32];
 // accumulator register r of lane l is C[(r/4)*8 + (l/32)*4 + r%4][l%32].
 #include <algorithm>
-#include <cstdlib>
 #include <mutex>
 #include <type_traits>
 #include <vector>
@@ -233,7 +232,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmBf16Args p)
 //     registers with 32 v_perm_b32 and stored as rows of Bᵀ, so its fragments are 128-bit reads too
 //     (the LDS transpose read, ds_read_b64_tr_b16, moves a third of the bytes per cycle).
 // Fragment reads run one 16-wide k sub-step ahead of the MFMAs and cross the tile boundary; there is one
-// barrier per k-tile.  The epilogue goes through LDS (each wavefront owns a 32×128 f32 strip) so that
+// barrier per k-tile.  The epilogue goes through LDS (each wavefront owns a 32-row f32 strip) so that
 // bias/residual loads and the stores are 128-bit and row-contiguous.
 // -------------------------------------------------------------------------------------------------
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
@@ -242,270 +241,30 @@ typedef __attribute__((address_space(3))) void *lds_void_ptr;
 // s_waitcnt vmcnt(n) only (expcnt and lgkmcnt left at their maxima), gfx9 encoding.
 #define ST_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (7 << 4) | (15 << 8) | ((((n) >> 4) & 3) << 14))
 
-__global__ __launch_bounds__(256) void gemm_bf16_256_kernel(GemmBf16Args p)
+// Eight wavefronts, two per SIMD (each owns a 64 × BN/2 tile of C), so that one can issue MFMAs while the
+// other waits on LDS, memory or the barrier.  Wavefronts 0 .. BN/64-1 stage
+// B (fetch, transpose, store), wavefronts 4-7 issue the direct-to-LDS loads of A.  BN = 256 is the main
+// shape; BN = 128 halves the tile for problems whose 256-wide tiling would leave compute units idle.
+template <int BN>
+__device__ __forceinline__ void gemm_bf16_w8_body(const GemmBf16Args &p)
 {
+    static_assert(BN == 256 || BN == 128, "tile width");
     constexpr int BM = 256, BK = 64;
+    constexpr int WTN = BN / 2;              // wavefront tile width
+    constexpr int TN = WTN / 32;             // 32-column MFMA tiles per wavefront
+    constexpr int B_THREADS = BN;            // threads that stage B: 8 k-groups × BN/8 column groups
     constexpr int STAGE = 32768;             // bytes: 256 rows × 128 B, for A and for Bᵀ alike
     constexpr int B_REGION = 3 * STAGE;      // [A0][A1][A2][B0][B1]
-    constexpr int C_STRIDE = 128 + 4;        // floats, epilogue strip
+    constexpr int C_STRIDE = WTN + 4;        // floats, epilogue strip
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_bytes[];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave >> 1, wn = wave & 1;  // 4 × 2 wavefronts, 64 × WTN each
     const int li = lane & 31, lh = lane >> 5;
-    const int M = p.M, N = p.N, K = p.K;
-
-    int logical = blockIdx.x;
-    if (p.swizzle) logical = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
-    constexpr int GROUP_M = 4;
-    const int width = GROUP_M * p.tiles_n;
-    const int group = logical / width;
-    const int first_m = group * GROUP_M;
-    const int group_size = min(p.tiles_m - first_m, GROUP_M);
-    const int tile_m = first_m + (logical % width) % group_size;
-    const int tile_n = (logical % width) / group_size;
-    const int m0 = tile_m * BM, n0 = tile_n * 256;
-
-    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint16_t *>(p.A), 0, static_cast<int>(static_cast<unsigned>(M) * static_cast<unsigned>(K) * 2u), 0x00020000);
-    const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint16_t *>(p.B), 0, static_cast<int>(static_cast<unsigned>(K) * static_cast<unsigned>(N) * 2u), 0x00020000);
-
-    // ---- A: direct global->LDS.  Instruction r of wavefront w fills rows r*32 + w*8 .. +7; lane l lands at
-    // chunk position l&7 of row (l>>3), so it must fetch logical chunk (l&7) ^ swz(row).
-    unsigned a_off[8];
-    {
-        const int row_in = wave * 8 + (lane >> 3);
-        const int sw_base = ((wave * 4 + (lane >> 4)) ^ (wave >> 1)) & 7;
-#pragma unroll
-        for (int r = 0; r < 8; ++r) {
-            const int chunk = ((lane & 7) ^ sw_base ^ ((2 * r) & 7)) & 7;
-            a_off[r] = (static_cast<unsigned>(m0 + r * 32 + row_in) * K + chunk * 8) * 2u;
-        }
-    }
-    // ---- B: thread (kg, nc) owns k-rows kg*8 .. +7 and columns nc*8 .. +7 of the tile.
-    const int kg = tid >> 5, nc = tid & 31;
-    unsigned b_off = (static_cast<unsigned>(kg * 8) * N + n0 + nc * 8) * 2u;
-    const unsigned b_row_step = static_cast<unsigned>(N) * 2u;
-    const unsigned b_tile_step = static_cast<unsigned>(BK) * N * 2u;
-    // Store instruction s writes column s ^ (nc & 1): odd and even lanes then hit rows of different parity
-    // and, with the swizzle, a 16-lane group covers all 64 banks.
-    const unsigned sel_even = (nc & 1) ? 0x07060302u : 0x05040100u;  // column parity 0 for even lanes
-    const unsigned sel_odd = (nc & 1) ? 0x05040100u : 0x07060302u;
-    unsigned b_store[8];
-#pragma unroll
-    for (int sidx = 0; sidx < 8; ++sidx) {
-        const int col = nc * 8 + (sidx ^ (nc & 1));
-        const int pc = (kg ^ ((col >> 1) ^ (col >> 4))) & 7;
-        b_store[sidx] = B_REGION + col * 128 + pc * 16;
-    }
-
-    f32x16 acc[4][4];
-#pragma unroll
-    for (int a = 0; a < 4; ++a)
-#pragma unroll
-        for (int b = 0; b < 4; ++b)
-            acc[a][b] = f32x16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-
-    u32x4 rb[8];
-    unsigned k_bytes = 0;  // byte offset of the next k-tile to request, within a row of A
-    auto load_a = [&](int stage) {
-#pragma unroll
-        for (int r = 0; r < 8; ++r)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_ptr)(lds_bytes + stage * STAGE + (r * 4 + wave) * 1024),
-                                                     16, a_off[r] + k_bytes, 0, 0, 0);
-    };
-    auto load_b = [&]() {
-#pragma unroll
-        for (int r = 0; r < 8; ++r) rb[r] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, b_off + r * b_row_step, 0, 0);
-        b_off += b_tile_step;
-    };
-    auto store_b = [&](int stage) {
-        // out[c].dword[j] = {rb[2j] element c, rb[2j+1] element c}; element c sits in dword c>>1, half c&1.
-#pragma unroll
-        for (int sidx = 0; sidx < 8; ++sidx) {
-            const int d = sidx >> 1;  // (sidx ^ 1) >> 1 == sidx >> 1: both lane parities read the same dword
-            const unsigned sel = (sidx & 1) ? sel_odd : sel_even;
-            u32x4 out;
-            out.x = __builtin_amdgcn_perm(rb[1][d], rb[0][d], sel);
-            out.y = __builtin_amdgcn_perm(rb[3][d], rb[2][d], sel);
-            out.z = __builtin_amdgcn_perm(rb[5][d], rb[4][d], sel);
-            out.w = __builtin_amdgcn_perm(rb[7][d], rb[6][d], sel);
-            *reinterpret_cast<u32x4 *>(lds_bytes + b_store[sidx] + stage * STAGE) = out;
-        }
-    };
-
-    // Fragment addresses: row*128 + ((q ^ swz(row)) << 4) with q = 2*kk + lh; for row = base + t*32 + li the
-    // swizzle is sw0 ^ 2t, so the four values of (2kk) ^ (2t) select one of four precomputed addresses.
-    unsigned a_frag[4], b_frag[4];
-    {
-        const int sw0 = ((li >> 1) ^ (li >> 4)) & 7;
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            const int pc = (lh ^ sw0 ^ (2 * c)) & 7;
-            a_frag[c] = (wm * 128 + li) * 128 + pc * 16;
-            b_frag[c] = B_REGION + (wn * 128 + li) * 128 + pc * 16;
-        }
-    }
-    bf16x8 fa[2][4], fb[2][4];
-    auto read_frags = [&](int buf, int a_stage, int b_stage, int kk) {
-#pragma unroll
-        for (int t4 = 0; t4 < 4; ++t4) {
-            fa[buf][t4] = *reinterpret_cast<const bf16x8 *>(lds_bytes + a_frag[kk ^ t4] + a_stage * STAGE + t4 * 4096);
-            fb[buf][t4] = *reinterpret_cast<const bf16x8 *>(lds_bytes + b_frag[kk ^ t4] + b_stage * STAGE + t4 * 4096);
-        }
-    };
-    auto mfma_step = [&](int buf) {
-#pragma unroll
-        for (int tm = 0; tm < 4; ++tm)
-#pragma unroll
-            for (int tn = 0; tn < 4; ++tn)
-                acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[buf][tm], fb[buf][tn], acc[tm][tn], 0, 0, 0);
-    };
-
-    // One k-tile t.  On entry: fragment buffer 0 holds sub-step 0 of tile t; rb holds B(t+1); the direct loads
-    // of A(t+1) are in flight.  STORE: B(t+1) is transposed into the other B stage; LOAD: B(t+2) and A(t+2)
-    // are requested; NEXT: sub-step 0 of tile t+1 is fetched after the barrier.
-    int a_stage = 0;  // t % 3
-    auto iteration = [&](auto store_tag, auto load_tag, auto next_tag, int t) {
-        constexpr bool STORE = decltype(store_tag)::value;
-        constexpr bool LOAD = decltype(load_tag)::value;
-        constexpr bool NEXT = decltype(next_tag)::value;
-        const int b_stage = t & 1;
-        const int a_next = a_stage == 2 ? 0 : a_stage + 1;
-        read_frags(1, a_stage, b_stage, 1);
-        mfma_step(0);
-        if constexpr (STORE) store_b(b_stage ^ 1);
-        if constexpr (LOAD) {
-            load_b();
-            load_a(a_next == 2 ? 0 : a_next + 1);
-            k_bytes += BK * 2u;
-        }
-        read_frags(0, a_stage, b_stage, 2);
-        mfma_step(1);
-        read_frags(1, a_stage, b_stage, 3);
-        mfma_step(0);
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            if (i < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            if (STORE && (i & 1)) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-        }
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            if (i < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            if (LOAD) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-        }
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            if (i < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        }
-        // A(t+1) must have landed before the barrier publishes it; the requests issued in this iteration
-        // (8 for B, then 8 for A) may stay in flight.
-        if constexpr (NEXT) {
-            if constexpr (LOAD) ST_WAIT_VMCNT(16); else ST_WAIT_VMCNT(0);
-        }
-        __syncthreads();
-        if constexpr (NEXT) read_frags(0, a_next, b_stage ^ 1, 0);
-        mfma_step(1);
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            if (NEXT && i < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        }
-        a_stage = a_next;
-    };
-
-    const int steps = K / BK;
-    load_a(0);
-    load_b();
-    k_bytes += BK * 2u;
-    store_b(0);  // waits for B(0), and with it (requests complete in order) for A(0)
-    if (steps > 1) {
-        load_b();
-        load_a(1);
-        k_bytes += BK * 2u;
-        ST_WAIT_VMCNT(16);
-    } else {
-        ST_WAIT_VMCNT(0);
-    }
-    __syncthreads();
-    read_frags(0, 0, 0, 0);
-    int t = 0;
-    for (; t + 2 < steps; ++t) iteration(std::true_type{}, std::true_type{}, std::true_type{}, t);
-    if (t + 1 < steps) {
-        iteration(std::true_type{}, std::false_type{}, std::true_type{}, t);
-        ++t;
-    }
-    iteration(std::false_type{}, std::false_type{}, std::false_type{}, t);
-
-    // ---- epilogue through LDS ---------------------------------------------------------------------
-    __syncthreads();
-    float *strip = reinterpret_cast<float *>(lds_bytes) + wave * (32 * C_STRIDE);
-    const bool scaled = p.scale != 1.0f;
-    const int col0 = n0 + wn * 128 + (lane & 31) * 4;  // this lane's 4 columns in the read-back phase
-    float4 bias4 = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (p.bias) bias4 = *reinterpret_cast<const float4 *>(p.bias + col0);
-#pragma unroll
-    for (int tm = 0; tm < 4; ++tm) {
-#pragma unroll
-        for (int tn = 0; tn < 4; ++tn) {
-            const f32x16 tile = acc[tm][tn];
-#pragma unroll
-            for (int r = 0; r < 16; ++r)
-                strip[((r >> 2) * 8 + lh * 4 + (r & 3)) * C_STRIDE + tn * 32 + li] = tile[r];
-        }
-        const int row_base = m0 + wm * 128 + tm * 32;
-#pragma unroll 2
-        for (int j = 0; j < 16; ++j) {
-            const int local_row = j * 2 + (lane >> 5);
-            const int row = row_base + local_row;
-            float4 v = *reinterpret_cast<const float4 *>(&strip[local_row * C_STRIDE + (lane & 31) * 4]);
-            if (row < M) {
-                const size_t idx = static_cast<size_t>(row) * N + col0;
-                if (scaled) { v.x *= p.scale; v.y *= p.scale; v.z *= p.scale; v.w *= p.scale; }
-                v.x += bias4.x; v.y += bias4.y; v.z += bias4.z; v.w += bias4.w;
-                if (p.residual) {
-                    const float4 rr = *reinterpret_cast<const float4 *>(p.residual + idx);
-                    v.x += rr.x; v.y += rr.y; v.z += rr.z; v.w += rr.w;
-                }
-                v.x = apply_activation(v.x, p.activation);
-                v.y = apply_activation(v.y, p.activation);
-                v.z = apply_activation(v.z, p.activation);
-                v.w = apply_activation(v.w, p.activation);
-                if (p.C32) *reinterpret_cast<float4 *>(p.C32 + idx) = v;
-                if (p.C16) {
-                    uint2 packed;
-                    packed.x = f32_to_bf16_rne(v.x) | (static_cast<uint32_t>(f32_to_bf16_rne(v.y)) << 16);
-                    packed.y = f32_to_bf16_rne(v.z) | (static_cast<uint32_t>(f32_to_bf16_rne(v.w)) << 16);
-                    *reinterpret_cast<uint2 *>(p.C16 + idx) = packed;
-                }
-            }
-        }
-    }
-}
-
-// Eight-wavefront variant of the kernel above: two wavefronts per SIMD (each owns a 64×128 tile of C) so
-// that one can issue MFMAs while the other waits on LDS, memory or the barrier.  Wavefronts 0-3 stage B
-// (fetch, transpose, store), wavefronts 4-7 issue the direct-to-LDS loads of A.
-__global__ __launch_bounds__(512) void gemm_bf16_256w8_kernel(GemmBf16Args p)
-{
-    constexpr int BM = 256, BK = 64;
-    constexpr int STAGE = 32768;             // bytes: 256 rows × 128 B, for A and for Bᵀ alike
-    constexpr int B_REGION = 3 * STAGE;      // [A0][A1][A2][B0][B1]
-    constexpr int C_STRIDE = 128 + 4;        // floats, epilogue strip
-    extern __shared__ __attribute__((aligned(16))) unsigned char lds_bytes[];
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;  // 4 × 2 wavefronts, 64 × 128 each
-    const int li = lane & 31, lh = lane >> 5;
-    const bool stages_b = wave < 4;  // wavefront-uniform role
+    const bool stages_b = wave < B_THREADS / 64;  // wavefront-uniform roles
+    const bool loads_a = wave >= 4;
     const int lw = wave & 3;         // index within the role
     const int M = p.M, N = p.N, K = p.K;
 
@@ -518,7 +277,7 @@ __global__ __launch_bounds__(512) void gemm_bf16_256w8_kernel(GemmBf16Args p)
     const int group_size = min(p.tiles_m - first_m, GROUP_M);
     const int tile_m = first_m + (logical % width) % group_size;
     const int tile_n = (logical % width) / group_size;
-    const int m0 = tile_m * BM, n0 = tile_n * 256;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
 
     const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint16_t *>(p.A), 0, static_cast<int>(static_cast<unsigned>(M) * static_cast<unsigned>(K) * 2u), 0x00020000);
@@ -538,7 +297,7 @@ __global__ __launch_bounds__(512) void gemm_bf16_256w8_kernel(GemmBf16Args p)
         }
     }
     // ---- B: thread (kg, nc) owns k-rows kg*8 .. +7 and columns nc*8 .. +7 of the tile.
-    const int kg = (tid & 255) >> 5, nc = tid & 31;
+    const int kg = (tid & (B_THREADS - 1)) / (BN / 8), nc = tid & (BN / 8 - 1);
     unsigned b_off = (static_cast<unsigned>(kg * 8) * N + n0 + nc * 8) * 2u;
     const unsigned b_row_step = static_cast<unsigned>(N) * 2u;
     const unsigned b_tile_step = static_cast<unsigned>(BK) * N * 2u;
@@ -554,11 +313,11 @@ __global__ __launch_bounds__(512) void gemm_bf16_256w8_kernel(GemmBf16Args p)
         b_store[sidx] = B_REGION + col * 128 + pc * 16;
     }
 
-    f32x16 acc[2][4];
+    f32x16 acc[2][TN];
 #pragma unroll
     for (int a = 0; a < 2; ++a)
 #pragma unroll
-        for (int b = 0; b < 4; ++b)
+        for (int b = 0; b < TN; ++b)
             acc[a][b] = f32x16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
     u32x4 rb[8];
@@ -597,23 +356,23 @@ __global__ __launch_bounds__(512) void gemm_bf16_256w8_kernel(GemmBf16Args p)
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             a_frag[c] = (wm * 64 + li) * 128 + ((lh ^ sw0 ^ ((wm & 1) * 4) ^ (2 * c)) & 7) * 16;
-            b_frag[c] = B_REGION + (wn * 128 + li) * 128 + ((lh ^ sw0 ^ (2 * c)) & 7) * 16;
+            b_frag[c] = B_REGION + (wn * WTN + li) * 128 + ((lh ^ sw0 ^ ((wn * WTN / 16) & 7) ^ (2 * c)) & 7) * 16;
         }
     }
-    bf16x8 fa[2][2], fb[2][4];
+    bf16x8 fa[2][2], fb[2][TN];
     auto read_frags = [&](int buf, int a_stage, int b_stage, int kk) {
 #pragma unroll
         for (int t2 = 0; t2 < 2; ++t2)
             fa[buf][t2] = *reinterpret_cast<const bf16x8 *>(lds_bytes + a_frag[kk ^ t2] + a_stage * STAGE + t2 * 4096);
 #pragma unroll
-        for (int t4 = 0; t4 < 4; ++t4)
+        for (int t4 = 0; t4 < TN; ++t4)
             fb[buf][t4] = *reinterpret_cast<const bf16x8 *>(lds_bytes + b_frag[kk ^ t4] + b_stage * STAGE + t4 * 4096);
     };
     auto mfma_step = [&](int buf) {
 #pragma unroll
         for (int tm = 0; tm < 2; ++tm)
 #pragma unroll
-            for (int tn = 0; tn < 4; ++tn)
+            for (int tn = 0; tn < TN; ++tn)
                 acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[buf][tm], fb[buf][tn], acc[tm][tn], 0, 0, 0);
     };
 
@@ -632,7 +391,7 @@ __global__ __launch_bounds__(512) void gemm_bf16_256w8_kernel(GemmBf16Args p)
         if (stages_b) {
             if constexpr (STORE) store_b(b_stage ^ 1);
             if constexpr (LOAD) load_b();
-        } else {
+        } else if (loads_a) {
             if constexpr (LOAD) load_a(a_next == 2 ? 0 : a_next + 1);
         }
         if constexpr (LOAD) k_bytes += BK * 2u;
@@ -643,7 +402,7 @@ __global__ __launch_bounds__(512) void gemm_bf16_256w8_kernel(GemmBf16Args p)
         // A(t+1) must have landed before the barrier publishes it; this iteration's 8 requests may stay
         // in flight.  (The B wavefronts' loads are register loads; the compiler waits where they are used.)
         if constexpr (NEXT) {
-            if (!stages_b) {
+            if (loads_a) {
                 if constexpr (LOAD) ST_WAIT_VMCNT(8); else ST_WAIT_VMCNT(0);
             }
         }
@@ -658,7 +417,7 @@ __global__ __launch_bounds__(512) void gemm_bf16_256w8_kernel(GemmBf16Args p)
         load_b();
         store_b(0);
         if (steps > 1) load_b();
-    } else {
+    } else if (loads_a) {
         load_a(0);
         if (steps > 1) {
             k_bytes += BK * 2u;
@@ -684,13 +443,15 @@ __global__ __launch_bounds__(512) void gemm_bf16_256w8_kernel(GemmBf16Args p)
     __syncthreads();
     float *strip = reinterpret_cast<float *>(lds_bytes) + wave * (32 * C_STRIDE);
     const bool scaled = p.scale != 1.0f;
-    const int col0 = n0 + wn * 128 + (lane & 31) * 4;  // this lane's 4 columns in the read-back phase
+    constexpr int LPR = WTN / 4;        // lanes per strip row in the read-back phase (4 columns each)
+    constexpr int ROWS_PER_PASS = 64 / LPR;
+    const int col0 = n0 + wn * WTN + (lane & (LPR - 1)) * 4;  // this lane's 4 columns in the read-back phase
     float4 bias4 = make_float4(0.f, 0.f, 0.f, 0.f);
     if (p.bias) bias4 = *reinterpret_cast<const float4 *>(p.bias + col0);
 #pragma unroll
     for (int tm = 0; tm < 2; ++tm) {
 #pragma unroll
-        for (int tn = 0; tn < 4; ++tn) {
+        for (int tn = 0; tn < TN; ++tn) {
             const f32x16 tile = acc[tm][tn];
 #pragma unroll
             for (int r = 0; r < 16; ++r)
@@ -698,10 +459,10 @@ __global__ __launch_bounds__(512) void gemm_bf16_256w8_kernel(GemmBf16Args p)
         }
         const int row_base = m0 + wm * 64 + tm * 32;
 #pragma unroll 2
-        for (int j = 0; j < 16; ++j) {
-            const int local_row = j * 2 + (lane >> 5);
+        for (int j = 0; j < 32 / ROWS_PER_PASS; ++j) {
+            const int local_row = j * ROWS_PER_PASS + lane / LPR;
             const int row = row_base + local_row;
-            float4 v = *reinterpret_cast<const float4 *>(&strip[local_row * C_STRIDE + (lane & 31) * 4]);
+            float4 v = *reinterpret_cast<const float4 *>(&strip[local_row * C_STRIDE + (lane & (LPR - 1)) * 4]);
             if (row < M) {
                 const size_t idx = static_cast<size_t>(row) * N + col0;
                 if (scaled) { v.x *= p.scale; v.y *= p.scale; v.z *= p.scale; v.w *= p.scale; }
@@ -725,6 +486,9 @@ __global__ __launch_bounds__(512) void gemm_bf16_256w8_kernel(GemmBf16Args p)
         }
     }
 }
+
+__global__ __launch_bounds__(512) void gemm_bf16_256w8_kernel(GemmBf16Args p) { gemm_bf16_w8_body<256>(p); }
+__global__ __launch_bounds__(512) void gemm_bf16_256x128w8_kernel(GemmBf16Args p) { gemm_bf16_w8_body<128>(p); }
 
 // -------------------------------------------------------------------------------------------------
 // Skinny kernel (M <= 64, decode-like): HBM-bound on B, so the job is to keep many bytes of B in flight
@@ -979,22 +743,21 @@ hipError_t launch_skinny(const GemmBf16Args &args, hipStream_t stream)
     return hipGetLastError();
 }
 
-template <bool EIGHT_WAVES>
+template <int BN>
 hipError_t launch_256(GemmBf16Args args, hipStream_t stream)
 {
     args.tiles_m = (args.M + 255) / 256;
-    args.tiles_n = args.N / 256;
+    args.tiles_n = args.N / BN;
     const size_t tiles = static_cast<size_t>(args.tiles_m) * static_cast<size_t>(args.tiles_n);
     if (tiles > 0x7fffffffu) return hipErrorInvalidConfiguration;
     args.swizzle = (tiles % 8 == 0) ? 1 : 0;
     constexpr size_t lds_bytes = 5 * 32768;  // three A stages + two B stages
-    static_assert(lds_bytes >= 4 * 32 * (128 + 4) * sizeof(float), "epilogue strips must fit in the stage buffers");
-    static_assert(lds_bytes >= 8 * 32 * (128 + 4) * sizeof(float), "eight epilogue strips must fit as well");
-    auto kernel = EIGHT_WAVES ? gemm_bf16_256w8_kernel : gemm_bf16_256_kernel;
+    static_assert(lds_bytes >= 8 * 32 * (128 + 4) * sizeof(float), "eight epilogue strips must fit in the stage buffers");
+    auto kernel = BN == 256 ? gemm_bf16_256w8_kernel : gemm_bf16_256x128w8_kernel;
     hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
     if (rc != hipSuccess) return rc;
-    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(tiles)), dim3(EIGHT_WAVES ? 512 : 256), lds_bytes, stream, args);
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(tiles)), dim3(512), lds_bytes, stream, args);
     return hipGetLastError();
 }
 
@@ -1058,8 +821,14 @@ hipError_t launch_gemm_bf16(size_t m, size_t n, size_t k, const uint16_t *lhs, c
                                   (reinterpret_cast<uintptr_t>(out_bf16) & 7u) == 0;
     if (m <= 64 && vec && k >= 256 && k % 64 == 0 && n % 128 == 0 && fits_buffer)
         return launch_skinny(args, stream);
-    if (big_tiles >= 128 && vec && k >= 64 && k % 64 == 0 && n % 256 == 0 && fits_buffer && epilogue_aligned)
-        return getenv("STHIP_GEMM_W4") ? launch_256<false>(args, stream) : launch_256<true>(args, stream);
+    if (big_tiles >= 128 && vec && k >= 64 && k % 64 == 0 && n % 256 == 0 && fits_buffer && epilogue_aligned) {
+        // One workgroup per compute unit at a time: the launch runs in rounds of 256 tiles.  Halving the tile
+        // width costs about 15 % in the main loop (more LDS traffic per flop), so do it only when it fills
+        // rounds that the 256-wide tiling would leave partly empty.
+        auto fill = [](size_t tiles) { return static_cast<double>(tiles) / static_cast<double>((tiles + 255) / 256 * 256); };
+        if (fill(2 * big_tiles) > 1.15 * fill(big_tiles)) return launch_256<128>(args, stream);
+        return launch_256<256>(args, stream);
+    }
     return launch_tile<128, 128, 32>(args, vec, stream);
 }
 

@@ -131,6 +131,30 @@ def test_fused_epilogue_and_bf16_output(hip, oracle, m, n, k):
         assert (got16 == inputs.to_bf16(got32)).all(), "bf16 output must be the RNE rounding of the f32 output"
 
 
+@pytest.mark.parametrize("m,n,k,ragged", [(8192, 1024, 128, 0), (8192, 2048, 64, 0), (16384, 512, 192, 0),
+                                          (8192 - 37, 2048, 128, 1), (16384 - 5, 768, 64, 1)])
+def test_large_tile_kernels_with_epilogue(hip, oracle, m, n, k, ragged):
+    """Shapes that take the 256x256 and 256x128 tile kernels (>= 128 tiles), with bias + residual + GELU and
+    both output types; m may be ragged."""
+    from spiraltorch_amd import inputs
+    rng = np.random.default_rng(m + n + k)
+    a, b = bf16_pair(rng, m, n, k, std=0.5)
+    bias = rng.normal(size=n).astype(np.float32)
+    res = rng.normal(size=m * n).astype(np.float32)
+    d = {name: hip.DeviceBuffer.from_array(v) for name, v in (("a", a), ("b", b), ("bias", bias), ("res", res))}
+    d32, d16 = hip.DeviceBuffer(m * n * 4), hip.DeviceBuffer(m * n * 2)
+    base = oracle.gemm_bf16_f32acc(m, n, k, a, b, threads=8).astype(np.float64)
+    pre = (base.reshape(m, n) + bias).ravel() + res
+    for act in (0, 2):
+        hip.gemm_bf16_bias_act_dev(m, n, k, act, d["a"], d["b"], d["bias"], d["res"], d32, d16)
+        hip.device_synchronize()
+        want = pre if act == 0 else 0.5 * pre * (1.0 + np.tanh(0.7978846 * (pre + 0.044715 * pre ** 3)))
+        got32 = d32.to_array(np.float32, m * n)
+        assert_close(got32, want, 1e-4, 1e-5, f"{m}x{n}x{k} act={act}")
+        got16 = d16.to_array(np.uint16, m * n)
+        assert (got16 == inputs.to_bf16(got32)).all(), "bf16 output must be the RNE rounding of the f32 output"
+
+
 def test_validation(hip):
     out = np.full(4, 13.0, np.float32)
     with pytest.raises(hip.HipErr, match="lhs buffer length 4 does not match m\\*k=6"):
