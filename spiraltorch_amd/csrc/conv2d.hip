@@ -227,6 +227,228 @@ __global__ __launch_bounds__(64 * WM * WN) void conv2d_f32_kernel(ConvArgs p)
     }
 }
 
+// -------------------------------------------------------------------------------------------------
+// Ring kernel: the same implicit GEMM, but both operands travel global memory -> LDS without passing
+// through registers (buffer_load ... lds) into a three-deep ring of 16-wide k-tiles, so two k-tiles of
+// loads are in flight while the matrix cores work on the third.  Per k-tile a wavefront issues one
+// 16-byte-per-lane load of weights and 16/WAVES one-pixel-per-lane gathers; a tap that falls into the padding
+// is given an out-of-range offset, for which the buffer load writes zero into LDS.  Whether tap (ky, kx) of
+// this lane's pixel is inside the image is a bit of a per-lane mask computed once, and which (channel, tap) a
+// gathered row belongs to is wavefront-uniform and tracked in scalar registers, so the loop's vector address
+// arithmetic is a shift, a compare, an add and a select per gathered row.
+//
+// Needs: c_in*kh*kw a multiple of 16 with 16-byte aligned weight rows, kh*kw <= 32, one image and the weights
+// each smaller than 2 GiB (32-bit buffer offsets).  Everything else takes the register-staged kernel above.
+//
+// LDS per stage: weights BM rows × 64 B, 16-byte chunk c of row r stored at position c ^ ((r >> 2) & 3)
+// (the swizzle is applied by choosing which chunk each lane fetches), then 16 patch rows of 64 pixels with a
+// 288-byte row pitch; both make the fragment reads conflict-free.  Three stages of the 128-row tile are
+// 38 KB, so four workgroups share a compute unit.
+// -------------------------------------------------------------------------------------------------
+typedef __attribute__((address_space(3))) void *lds_void_ptr;
+
+#define ST_CONV_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (7 << 4) | (15 << 8) | ((((n) >> 4) & 3) << 14))
+
+constexpr int kRingStages = 3;
+
+template <int BM, int WM, int WN>
+__device__ __forceinline__ void conv2d_f32_ring_body(const ConvArgs &p)
+{
+    constexpr int BN = 64, BK = 16, RING = kRingStages;
+    constexpr int WAVES = WM * WN;
+    constexpr int WTM = BM / WM, WTN = BN / WN;
+    constexpr int TM = WTM / 32, TN = WTN / 32;
+    static_assert(TM >= 1 && TN >= 1, "wavefront tile must be at least 32×32");
+    static_assert(BM == 16 * WAVES, "one 16-row weight load per wavefront and k-tile");
+    static_assert(BK % WAVES == 0, "patch rows divide over the wavefronts");
+    constexpr int B_ROWS = BK / WAVES;           // gathered rows per wavefront and k-tile
+    constexpr int LOADS = 1 + B_ROWS;            // load instructions per wavefront and k-tile
+    constexpr int B_PITCH = (BN + 8) * 4;        // bytes
+    constexpr int A_BYTES = BM * BK * 4;
+    constexpr int STAGE = A_BYTES + BK * B_PITCH;
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char conv_lds[];
+    const int K = p.K;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: the per-row tap bookkeeping stays on the SALU
+    const int wm = wave / WN, wn = wave % WN;
+    const int li = lane & 31, lh = lane >> 5;
+
+    int bid = blockIdx.x;
+    if (p.xcd_swizzle) bid = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+    const int tile_oc = bid % p.tiles_oc;
+    bid /= p.tiles_oc;
+    const int tile_px = bid % p.tiles_px;
+    const int image = bid / p.tiles_px;
+    const int oc0 = tile_oc * BM, px0 = tile_px * BN;
+
+    const ConvShape &s = p.s;
+    const int H = s.h, W = s.w;
+    const int khw = s.kh * s.kw;
+    // Lane j < kh*kw keeps the byte offset of tap j = ky*kw + kx relative to a pixel's top-left tap; the loop
+    // fetches the entry of the (wavefront-uniform) tap it needs with v_readlane.
+    unsigned tap_offset = 0;
+    if (lane < khw) {
+        const int ky = lane / s.kw, kx = lane - ky * s.kw;
+        tap_offset = static_cast<unsigned>(ky * s.dil_h * W + kx * s.dil_w) * 4u;
+    }
+    const unsigned channel_bytes = static_cast<unsigned>(H) * W * 4u;
+
+    // This lane's pixel (the same in every wavefront) and the validity of each of its kh*kw taps.
+    const int px = px0 + lane;
+    const bool px_valid = px < p.spatial;
+    const int oy = px / s.ow, ox = px - oy * s.ow;
+    const int iy0 = oy * s.stride_h - s.pad_h;
+    const int ix0 = ox * s.stride_w - s.pad_w;
+    const unsigned base_bytes = static_cast<unsigned>(iy0 * W + ix0) * 4u;  // may wrap; valid taps unwrap it
+    unsigned tap_mask = 0;
+    for (int j = 0; j < khw; ++j) {
+        const int ky = j / s.kw, kx = j - ky * s.kw;
+        const bool ok = px_valid && static_cast<unsigned>(iy0 + ky * s.dil_h) < static_cast<unsigned>(H) &&
+                        static_cast<unsigned>(ix0 + kx * s.dil_w) < static_cast<unsigned>(W);
+        tap_mask |= (ok ? 1u : 0u) << j;
+    }
+
+    const size_t image_elems = static_cast<size_t>(s.c_in) * H * W;
+    const __amdgpu_buffer_rsrc_t rsrc_x = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float *>(p.input + static_cast<size_t>(image) * image_elems), 0, static_cast<int>(image_elems * 4), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_w = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float *>(p.weight), 0, static_cast<int>(static_cast<size_t>(s.c_out) * K * 4), 0x00020000);
+
+    // Weights: wavefront w fills rows 16w .. 16w+15 of the stage; lane L lands at row L/4, chunk position L%4.
+    const int a_row = wave * 16 + (lane >> 2);
+    const int a_chunk = (lane & 3) ^ ((a_row >> 2) & 3);
+    const unsigned a_off = (static_cast<unsigned>(min(oc0 + a_row, s.c_out - 1)) * K + a_chunk * 4) * 4u;
+
+    // Patch row `wave*B_ROWS + r` of k-tile t is reduction index k = 16t + row = ic*kh*kw + tap.  issue() is called
+    // for t = 0, 1, 2, ... in order, so (ic, tap) of each of this wavefront's rows is advanced by 16 per call.
+    int row_ic[B_ROWS], row_tap[B_ROWS];
+#pragma unroll
+    for (int r = 0; r < B_ROWS; ++r) {
+        const int row = wave * B_ROWS + r;
+        row_ic[r] = row / khw;
+        row_tap[r] = row - row_ic[r] * khw;
+    }
+    const int step_ic = BK / khw, step_tap = BK - step_ic * khw;
+
+    auto issue = [&](int t) {  // requests k-tile t into ring slot t % RING
+        unsigned char *stage = conv_lds + (t % RING) * STAGE;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_w, (lds_void_ptr)(stage + wave * 1024), 16, a_off, t * (BK * 4), 0, 0);
+#pragma unroll
+        for (int r = 0; r < B_ROWS; ++r) {
+            const int row = wave * B_ROWS + r;
+            const unsigned tap_bytes = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(tap_offset), row_tap[r])) +
+                                       static_cast<unsigned>(row_ic[r]) * channel_bytes;
+            const unsigned off = ((tap_mask >> row_tap[r]) & 1u) ? base_bytes + tap_bytes : 0x80000000u;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (lds_void_ptr)(stage + A_BYTES + row * B_PITCH), 4, off, 0, 0, 0);
+            row_tap[r] += step_tap;
+            row_ic[r] += step_ic;
+            if (row_tap[r] >= khw) {
+                row_tap[r] -= khw;
+                ++row_ic[r];
+            }
+        }
+    };
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int a = 0; a < TM; ++a)
+#pragma unroll
+        for (int b = 0; b < TN; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.0f;
+
+    auto compute = [&](int slot) {
+        const unsigned char *stage = conv_lds + slot * STAGE;
+#pragma unroll
+        for (int kk = 0; kk < BK / 8; ++kk) {
+            float a[TM][4], b[TN][4];
+#pragma unroll
+            for (int tm = 0; tm < TM; ++tm) {
+                const int row = wm * WTM + tm * 32 + li;
+                const int chunk = (kk * 2 + lh) ^ ((row >> 2) & 3);
+                const float4 v = *reinterpret_cast<const float4 *>(stage + row * 64 + chunk * 16);
+                a[tm][0] = v.x; a[tm][1] = v.y; a[tm][2] = v.z; a[tm][3] = v.w;
+            }
+#pragma unroll
+            for (int tn = 0; tn < TN; ++tn) {
+                const int col = wn * WTN + tn * 32 + li;
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    b[tn][t] = *reinterpret_cast<const float *>(stage + A_BYTES + (kk * 8 + lh * 4 + t) * B_PITCH + col * 4);
+            }
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+                    for (int tn = 0; tn < TN; ++tn)
+                        acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[tm][t], b[tn][t], acc[tm][tn], 0, 0, 0);
+        }
+    };
+
+    const int steps = K / BK;
+#pragma unroll
+    for (int t = 0; t < RING - 1; ++t)
+        if (t < steps) issue(t);
+    // Drain the prologue once.  (With prologue loads still counted as outstanding at the loop header the
+    // compiler's wait-count insertion falls back to a full vmcnt(0) inside the loop.)
+    ST_CONV_WAIT_VMCNT(0);
+    for (int t = 0; t < steps; ++t) {
+        // This wavefront's loads of k-tile t have landed once at most the loads of the (up to RING-2) later
+        // k-tiles it has already requested are outstanding; the barrier then extends that to every wavefront
+        // and also says that everyone is done reading the slot k-tile t+RING-1 is about to overwrite.
+        if (RING >= 4 && t + 2 < steps) ST_CONV_WAIT_VMCNT(2 * LOADS);
+        else if (t + 1 < steps) ST_CONV_WAIT_VMCNT(LOADS);
+        else ST_CONV_WAIT_VMCNT(0);
+        __syncthreads();
+        if (t + RING - 1 < steps) issue(t + RING - 1);
+        compute(t % RING);
+    }
+
+    float *out_image = p.out + static_cast<size_t>(image) * s.c_out * p.spatial;
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) {
+        const int col = px0 + wn * WTN + tn * 32 + li;
+        if (col >= p.spatial) continue;
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int oc = oc0 + wm * WTM + tm * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
+                if (oc >= s.c_out) continue;
+                float value = acc[tm][tn][r];
+                if (p.bias) value += p.bias[oc];
+                out_image[static_cast<size_t>(oc) * p.spatial + col] = apply_activation(value, p.activation);
+            }
+        }
+    }
+}
+
+// (A kernel template whose body uses the LDS-load builtins loses its host-side launch stub with this
+// compiler, hence plain kernels around the templated body.)
+__global__ __launch_bounds__(512) void conv2d_f32_ring128_kernel(ConvArgs p) { conv2d_f32_ring_body<128, 4, 2>(p); }
+__global__ __launch_bounds__(256) void conv2d_f32_ring64_kernel(ConvArgs p) { conv2d_f32_ring_body<64, 2, 2>(p); }
+
+template <int BM>
+hipError_t launch_ring(ConvArgs args, hipStream_t stream)
+{
+    args.tiles_oc = (args.s.c_out + BM - 1) / BM;
+    args.tiles_px = (args.spatial + 63) / 64;
+    const size_t tiles = static_cast<size_t>(args.tiles_oc) * args.tiles_px * static_cast<size_t>(args.s.batch);
+    if (tiles > 0x7fffffffu) return hipErrorInvalidConfiguration;
+    args.xcd_swizzle = (args.s.batch % 8 == 0) ? 1 : 0;
+    const size_t lds_bytes = kRingStages * (static_cast<size_t>(BM) * 64 + 16 * 288);
+    auto kernel = BM == 128 ? conv2d_f32_ring128_kernel : conv2d_f32_ring64_kernel;
+    hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        static_cast<int>(lds_bytes));
+    if (rc != hipSuccess) return rc;
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(tiles)), dim3(BM == 128 ? 512 : 256), lds_bytes, stream, args);
+    return hipGetLastError();
+}
+
 template <int BM, int BN, int BK, int WM, int WN>
 hipError_t launch_tile(ConvArgs args, bool vec, hipStream_t stream)
 {
@@ -282,6 +504,10 @@ hipError_t launch_conv2d_f32(const ConvShape &shape, int activation, const float
     const bool vec = (args.K % 4 == 0) && ((reinterpret_cast<uintptr_t>(weight) & 15u) == 0);
     // 8 wavefronts of 32×32 per 128×64 tile measured best for wide layers (128×128 tiles, 32-deep k-tiles and
     // 4-wavefront layouts were all 10-20 % slower on the 64->128 channel 56×56 case).
+    const bool ring_ok = vec && args.K % 16 == 0 && shape.kh * shape.kw <= 32 &&
+                         static_cast<size_t>(shape.c_in) * shape.h * shape.w * 4 < (1ull << 31) &&
+                         static_cast<size_t>(shape.c_out) * args.K * 4 < (1ull << 31);
+    if (ring_ok) return shape.c_out > 64 ? launch_ring<128>(args, stream) : launch_ring<64>(args, stream);
     if (shape.c_out > 64) return launch_tile<128, 64, 16, 4, 2>(args, vec, stream);
     return launch_tile<64, 64, 16, 2, 2>(args, vec, stream);
 }
