@@ -360,33 +360,41 @@ __device__ __forceinline__ void conv2d_f32_ring_body(const ConvArgs &p)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.0f;
 
+    // All fragments of the k-tile are read first and the MFMAs then run back to back at raised priority: the
+    // wavefront holds the matrix pipe for one uninterrupted run instead of stalling on LDS between pairs.
     auto compute = [&](int slot) {
         const unsigned char *stage = conv_lds + slot * STAGE;
+        float a[BK / 8][TM][4], b[BK / 8][TN][4];
 #pragma unroll
         for (int kk = 0; kk < BK / 8; ++kk) {
-            float a[TM][4], b[TN][4];
 #pragma unroll
             for (int tm = 0; tm < TM; ++tm) {
                 const int row = wm * WTM + tm * 32 + li;
                 const int chunk = (kk * 2 + lh) ^ ((row >> 2) & 3);
                 const float4 v = *reinterpret_cast<const float4 *>(stage + row * 64 + chunk * 16);
-                a[tm][0] = v.x; a[tm][1] = v.y; a[tm][2] = v.z; a[tm][3] = v.w;
+                a[kk][tm][0] = v.x; a[kk][tm][1] = v.y; a[kk][tm][2] = v.z; a[kk][tm][3] = v.w;
             }
 #pragma unroll
             for (int tn = 0; tn < TN; ++tn) {
                 const int col = wn * WTN + tn * 32 + li;
 #pragma unroll
                 for (int t = 0; t < 4; ++t)
-                    b[tn][t] = *reinterpret_cast<const float *>(stage + A_BYTES + (kk * 8 + lh * 4 + t) * B_PITCH + col * 4);
+                    b[kk][tn][t] = *reinterpret_cast<const float *>(stage + A_BYTES + (kk * 8 + lh * 4 + t) * B_PITCH + col * 4);
             }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_setprio(2);
+#pragma unroll
+        for (int kk = 0; kk < BK / 8; ++kk)
 #pragma unroll
             for (int t = 0; t < 4; ++t)
 #pragma unroll
                 for (int tm = 0; tm < TM; ++tm)
 #pragma unroll
                     for (int tn = 0; tn < TN; ++tn)
-                        acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[tm][t], b[tn][t], acc[tm][tn], 0, 0, 0);
-        }
+                        acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kk][tm][t], b[kk][tn][t], acc[tm][tn], 0, 0, 0);
+        __builtin_amdgcn_s_setprio(0);
+        __builtin_amdgcn_sched_barrier(0);
     };
 
     const int steps = K / BK;
