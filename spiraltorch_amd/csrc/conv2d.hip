@@ -17,6 +17,8 @@
 #include "device_math.h"
 #include "kernels.h"
 
+#include <type_traits>
+
 namespace sthip {
 
 namespace {
@@ -32,6 +34,7 @@ struct ConvArgs {
     int tiles_px, tiles_oc;
     int xcd_swizzle;
     int activation;
+    unsigned tap_bytes[32];  // ring kernel: byte offset of tap ky*kw + kx relative to a pixel's top-left tap
 };
 
 
@@ -235,10 +238,10 @@ __global__ __launch_bounds__(64 * WM * WN) void conv2d_f32_kernel(ConvArgs p)
 // is given an out-of-range offset, for which the buffer load writes zero into LDS.  Whether tap (ky, kx) of
 // this lane's pixel is inside the image is a bit of a per-lane mask computed once, and which (channel, tap) a
 // gathered row belongs to is wavefront-uniform and tracked in scalar registers, so the loop's vector address
-// arithmetic is a shift, a compare, an add and a select per gathered row.
+// arithmetic is a shift, an add and a shift-add per gathered row.
 //
-// Needs: c_in*kh*kw a multiple of 16 with 16-byte aligned weight rows, kh*kw <= 32, one image and the weights
-// each smaller than 2 GiB (32-bit buffer offsets).  Everything else takes the register-staged kernel above.
+// Needs: c_in*kh*kw a multiple of 16 with 16-byte aligned weight rows, kh*kw <= 32, one image smaller than
+// 1 GiB and the weights smaller than 2 GiB (32-bit buffer offsets).  Everything else takes the register-staged kernel above.
 //
 // LDS per stage: weights BM rows × 64 B, 16-byte chunk c of row r stored at position c ^ ((r >> 2) & 3)
 // (the swizzle is applied by choosing which chunk each lane fetches), then 16 patch rows of 64 pixels with a
@@ -287,13 +290,6 @@ __device__ __forceinline__ void conv2d_f32_ring_body(const ConvArgs &p)
     const ConvShape &s = p.s;
     const int H = s.h, W = s.w;
     const int khw = s.kh * s.kw;
-    // Lane j < kh*kw keeps the byte offset of tap j = ky*kw + kx relative to a pixel's top-left tap; the loop
-    // fetches the entry of the (wavefront-uniform) tap it needs with v_readlane.
-    unsigned tap_offset = 0;
-    if (lane < khw) {
-        const int ky = lane / s.kw, kx = lane - ky * s.kw;
-        tap_offset = static_cast<unsigned>(ky * s.dil_h * W + kx * s.dil_w) * 4u;
-    }
     const unsigned channel_bytes = static_cast<unsigned>(H) * W * 4u;
 
     // This lane's pixel (the same in every wavefront) and the validity of each of its kh*kw taps.
@@ -310,6 +306,7 @@ __device__ __forceinline__ void conv2d_f32_ring_body(const ConvArgs &p)
                         static_cast<unsigned>(ix0 + kx * s.dil_w) < static_cast<unsigned>(W);
         tap_mask |= (ok ? 1u : 0u) << j;
     }
+    const unsigned tap_outside = ~tap_mask;  // bit j set: tap j of this pixel reads padding (or the pixel is past the end)
 
     const size_t image_elems = static_cast<size_t>(s.c_in) * H * W;
     const __amdgpu_buffer_rsrc_t rsrc_x = __builtin_amdgcn_make_buffer_rsrc(
@@ -333,15 +330,19 @@ __device__ __forceinline__ void conv2d_f32_ring_body(const ConvArgs &p)
     }
     const int step_ic = BK / khw, step_tap = BK - step_ic * khw;
 
-    auto issue = [&](int t) {  // requests k-tile t into ring slot t % RING
-        unsigned char *stage = conv_lds + (t % RING) * STAGE;
+    // Every vector instruction of the loop costs matrix-pipe time (the f32 MFMAs and the ordinary VALU do not
+    // overlap on a SIMD), so the gather address is three of them: the tap's outside-bit is shifted to bit 31 and
+    // added to the in-image offset, which pushes the offset of a padding tap past the buffer's range.  (Needs the
+    // image and its top/left padding to stay below 2^30 bytes so that no wrapped offset lands back in range.)
+    auto issue = [&](auto slot_tag, int t) {  // requests k-tile t into ring slot SLOT
+        constexpr int SLOT = decltype(slot_tag)::value;
+        unsigned char *stage = conv_lds + SLOT * STAGE;
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_w, (lds_void_ptr)(stage + wave * 1024), 16, a_off, t * (BK * 4), 0, 0);
 #pragma unroll
         for (int r = 0; r < B_ROWS; ++r) {
             const int row = wave * B_ROWS + r;
-            const unsigned tap_bytes = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(tap_offset), row_tap[r])) +
-                                       static_cast<unsigned>(row_ic[r]) * channel_bytes;
-            const unsigned off = ((tap_mask >> row_tap[r]) & 1u) ? base_bytes + tap_bytes : 0x80000000u;
+            const unsigned tap_bytes = p.tap_bytes[row_tap[r]] + static_cast<unsigned>(row_ic[r]) * channel_bytes;
+            const unsigned off = ((tap_outside >> row_tap[r]) << 31) + (base_bytes + tap_bytes);
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (lds_void_ptr)(stage + A_BYTES + row * B_PITCH), 4, off, 0, 0, 0);
             row_tap[r] += step_tap;
             row_ic[r] += step_ic;
@@ -351,6 +352,19 @@ __device__ __forceinline__ void conv2d_f32_ring_body(const ConvArgs &p)
             }
         }
     };
+
+    // Per-lane fragment addresses within a stage; the stage offset is a compile-time constant in the unrolled loop,
+    // so the reads need no address arithmetic.
+    unsigned a_lane[BK / 8][TM], b_lane[TN];
+#pragma unroll
+    for (int kk = 0; kk < BK / 8; ++kk)
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm) {
+            const int row = wm * WTM + tm * 32 + li;
+            a_lane[kk][tm] = row * 64 + (((kk * 2 + lh) ^ ((row >> 2) & 3)) * 16);
+        }
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) b_lane[tn] = A_BYTES + lh * 4 * B_PITCH + (wn * WTN + tn * 32 + li) * 4;
 
     f32x16 acc[TM][TN];
 #pragma unroll
@@ -362,25 +376,22 @@ __device__ __forceinline__ void conv2d_f32_ring_body(const ConvArgs &p)
 
     // All fragments of the k-tile are read first and the MFMAs then run back to back at raised priority: the
     // wavefront holds the matrix pipe for one uninterrupted run instead of stalling on LDS between pairs.
-    auto compute = [&](int slot) {
-        const unsigned char *stage = conv_lds + slot * STAGE;
+    auto compute = [&](auto slot_tag) {
+        constexpr int SLOT = decltype(slot_tag)::value;
+        const unsigned char *stage = conv_lds + SLOT * STAGE;
         float a[BK / 8][TM][4], b[BK / 8][TN][4];
 #pragma unroll
         for (int kk = 0; kk < BK / 8; ++kk) {
 #pragma unroll
             for (int tm = 0; tm < TM; ++tm) {
-                const int row = wm * WTM + tm * 32 + li;
-                const int chunk = (kk * 2 + lh) ^ ((row >> 2) & 3);
-                const float4 v = *reinterpret_cast<const float4 *>(stage + row * 64 + chunk * 16);
-                a[kk][tm][0] = v.x; a[kk][tm][1] = v.y; a[kk][tm][2] = v.z; a[kk][tm][3] = v.w;
+                const f32x4 v = *reinterpret_cast<const f32x4 *>(stage + a_lane[kk][tm]);
+                a[kk][tm][0] = v[0]; a[kk][tm][1] = v[1]; a[kk][tm][2] = v[2]; a[kk][tm][3] = v[3];
             }
 #pragma unroll
-            for (int tn = 0; tn < TN; ++tn) {
-                const int col = wn * WTN + tn * 32 + li;
+            for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
                 for (int t = 0; t < 4; ++t)
-                    b[kk][tn][t] = *reinterpret_cast<const float *>(stage + A_BYTES + (kk * 8 + lh * 4 + t) * B_PITCH + col * 4);
-            }
+                    b[kk][tn][t] = *reinterpret_cast<const float *>(stage + b_lane[tn] + (kk * 8 + t) * B_PITCH);
         }
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_setprio(2);
@@ -397,24 +408,39 @@ __device__ __forceinline__ void conv2d_f32_ring_body(const ConvArgs &p)
         __builtin_amdgcn_sched_barrier(0);
     };
 
+    static_assert(RING == 3, "the loop below is unrolled for three ring slots");
     const int steps = K / BK;
-#pragma unroll
-    for (int t = 0; t < RING - 1; ++t)
-        if (t < steps) issue(t);
+    if (steps > 0) issue(std::integral_constant<int, 0>{}, 0);
+    if (steps > 1) issue(std::integral_constant<int, 1>{}, 1);
     // Drain the prologue once.  (With prologue loads still counted as outstanding at the loop header the
     // compiler's wait-count insertion falls back to a full vmcnt(0) inside the loop.)
     ST_CONV_WAIT_VMCNT(0);
-    for (int t = 0; t < steps; ++t) {
-        // This wavefront's loads of k-tile t have landed once at most the loads of the (up to RING-2) later
-        // k-tiles it has already requested are outstanding; the barrier then extends that to every wavefront
-        // and also says that everyone is done reading the slot k-tile t+RING-1 is about to overwrite.
-        if (RING >= 4 && t + 2 < steps) ST_CONV_WAIT_VMCNT(2 * LOADS);
-        else if (t + 1 < steps) ST_CONV_WAIT_VMCNT(LOADS);
+    auto step = [&](auto slot_tag, int t) {
+        constexpr int SLOT = decltype(slot_tag)::value;
+        // This wavefront's loads of k-tile t have landed once only the loads of k-tile t+1 are outstanding; the
+        // barrier then extends that to every wavefront and also says that everyone is done reading the slot
+        // k-tile t+2 is about to overwrite.
+        //
+        // A bare s_barrier, not __syncthreads(): the latter's workgroup release fence makes the compiler wait for
+        // every outstanding load, including the k-tile that was just requested.  Nothing in the loop writes LDS
+        // with ordinary stores, the loads into LDS are ordered by the vmcnt wait above, and a wavefront's LDS
+        // reads of a slot have returned (its MFMAs consumed them) before it arrives at the next barrier.
+        if (t + 1 < steps) ST_CONV_WAIT_VMCNT(LOADS);
         else ST_CONV_WAIT_VMCNT(0);
-        __syncthreads();
-        if (t + RING - 1 < steps) issue(t + RING - 1);
-        compute(t % RING);
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if (t + 2 < steps) issue(std::integral_constant<int, (SLOT + 2) % RING>{}, t + 2);
+        compute(slot_tag);
+    };
+    int t = 0;
+    for (; t + 3 <= steps; t += 3) {
+        step(std::integral_constant<int, 0>{}, t);
+        step(std::integral_constant<int, 1>{}, t + 1);
+        step(std::integral_constant<int, 2>{}, t + 2);
     }
+    if (t < steps) step(std::integral_constant<int, 0>{}, t);
+    if (t + 1 < steps) step(std::integral_constant<int, 1>{}, t + 1);
 
     float *out_image = p.out + static_cast<size_t>(image) * s.c_out * p.spatial;
 #pragma unroll
@@ -448,6 +474,11 @@ hipError_t launch_ring(ConvArgs args, hipStream_t stream)
     const size_t tiles = static_cast<size_t>(args.tiles_oc) * args.tiles_px * static_cast<size_t>(args.s.batch);
     if (tiles > 0x7fffffffu) return hipErrorInvalidConfiguration;
     args.xcd_swizzle = (args.s.batch % 8 == 0) ? 1 : 0;
+    for (int j = 0; j < 32; ++j) {
+        const int ky = j / args.s.kw, kx = j % args.s.kw;
+        args.tap_bytes[j] = j < args.s.kh * args.s.kw
+                                ? static_cast<unsigned>(ky * args.s.dil_h * args.s.w + kx * args.s.dil_w) * 4u : 0u;
+    }
     const size_t lds_bytes = kRingStages * (static_cast<size_t>(BM) * 64 + 16 * 288);
     auto kernel = BM == 128 ? conv2d_f32_ring128_kernel : conv2d_f32_ring64_kernel;
     hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -513,7 +544,9 @@ hipError_t launch_conv2d_f32(const ConvShape &shape, int activation, const float
     // 8 wavefronts of 32×32 per 128×64 tile measured best for wide layers (128×128 tiles, 32-deep k-tiles and
     // 4-wavefront layouts were all 10-20 % slower on the 64->128 channel 56×56 case).
     const bool ring_ok = vec && args.K % 16 == 0 && shape.kh * shape.kw <= 32 &&
-                         static_cast<size_t>(shape.c_in) * shape.h * shape.w * 4 < (1ull << 31) &&
+                         static_cast<size_t>(shape.c_in) * shape.h * shape.w * 4 < (1ull << 30) &&
+                         (static_cast<size_t>(shape.pad_h) * shape.w + shape.pad_w) * 4 < (1ull << 30) &&
+                         (static_cast<size_t>(shape.oh + 64) * shape.stride_h * shape.w + static_cast<size_t>(shape.ow) * shape.stride_w) * 4 < (1ull << 30) &&
                          static_cast<size_t>(shape.c_out) * args.K * 4 < (1ull << 31);
     if (ring_ok) return shape.c_out > 64 ? launch_ring<128>(args, stream) : launch_ring<64>(args, stream);
     if (shape.c_out > 64) return launch_tile<128, 64, 16, 4, 2>(args, vec, stream);
