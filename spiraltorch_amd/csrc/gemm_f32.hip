@@ -18,6 +18,8 @@
 #include "device_math.h"
 #include "kernels.h"
 
+#include <type_traits>
+
 namespace sthip {
 
 namespace {
@@ -283,7 +285,245 @@ hipError_t launch_tile(GemmF32Args args, bool lhs_transposed, bool vec, hipStrea
     return hipGetLastError();
 }
 
+
 bool aligned16(const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
+
+// -------------------------------------------------------------------------------------------------
+// Ring kernel for K % 16 == 0 and 16-byte aligned rows.  On a SIMD the f32 MFMAs and ordinary vector
+// instructions do not overlap — measured, every VALU, LDS or memory instruction a wavefront issues takes
+// roughly 8 to 15 cycles away from the matrix pipe — so this loop issues as few of them as possible:
+// both operands go global memory -> LDS with buffer_load ... lds (16 bytes per lane, no registers, no
+// ds_write) into a three-deep ring of 16-wide k-tiles; the per-lane memory offsets are loop constants and
+// the k-tile advance rides in the instruction's scalar offset; the ring slot is a compile-time constant of
+// the 3x unrolled loop, so the fragment reads use immediate offsets.  What is left per k-tile and wavefront
+// is the fragment reads, LOADS load instructions and the MFMAs.
+//
+// Everything that could read outside a matrix is flagged through the vector offset alone (rows past M or
+// columns past N get an offset beyond the buffer's range and read as zero); K needs no guard.
+//
+// A (row-major m×k): stage rows hold 16 k-values (64 B); 16-byte chunk c of row r sits at c ^ ((r >> 2) & 3).
+// A stored k×m (lhs_transposed) and B (k×n): stage rows are k, BM or BN floats long, unpadded.
+// -------------------------------------------------------------------------------------------------
+typedef __attribute__((address_space(3))) void *lds_void_ptr;
+
+#define ST_F32_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (7 << 4) | (15 << 8) | ((((n) >> 4) & 3) << 14))
+
+template <int BM, int BN, int WM, int WN, bool AT>
+__device__ __forceinline__ void gemm_f32_ring_body(const GemmF32Args &p)
+{
+    constexpr int BK = 16, RING = 3;
+    constexpr int WAVES = WM * WN;
+    constexpr int WTM = BM / WM, WTN = BN / WN;
+    constexpr int TM = WTM / 32, TN = WTN / 32;
+    static_assert(TM >= 1 && TN >= 1, "wavefront tile must be at least 32×32");
+    constexpr int NA = BM / 16, NB = BN / 16;  // 1 KB load instructions per stage and operand
+    static_assert(NA % WAVES == 0 && NB % WAVES == 0, "load instructions divide evenly over the wavefronts");
+    constexpr int LOADS_A = NA / WAVES, LOADS = (NA + NB) / WAVES;  // per wavefront: first the A loads, then B
+    constexpr int A_BYTES = BM * BK * 4, B_BYTES = BK * BN * 4;
+    constexpr int STAGE = A_BYTES + B_BYTES;
+    static_assert(RING * STAGE <= 65536, "fragment reads address the ring with 16-bit immediates");
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char ring_lds[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WN, wn = wave % WN;
+    const int li = lane & 31, lh = lane >> 5;
+    const int M = p.M, N = p.N, K = p.K;
+
+    constexpr int GROUP_M = 8;
+    const int grid = static_cast<int>(gridDim.x), xcd = static_cast<int>(blockIdx.x) & 7;
+    const int tile_id = xcd * (grid >> 3) + min(xcd, grid & 7) + (static_cast<int>(blockIdx.x) >> 3);
+    const int group_size = GROUP_M * p.tiles_n;
+    const int first_m = (tile_id / group_size) * GROUP_M, in_group = tile_id % group_size;
+    const int group_rows = min(p.tiles_m - first_m, GROUP_M);
+    const int tile_m = first_m + in_group % group_rows, tile_n = in_group / group_rows;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float *>(p.A), 0, static_cast<int>(static_cast<size_t>(M) * K * 4), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float *>(p.B), 0, static_cast<int>(static_cast<size_t>(K) * N * 4), 0x00020000);
+    constexpr unsigned kOutside = 0x80000000u;
+
+    // This wavefront's load instructions: A instructions wave, wave + WAVES, ..., then B instructions likewise.
+    unsigned load_off[LOADS];     // per-lane byte offset at k-tile 0
+    int load_lds[LOADS];          // LDS byte offset of the instruction's 1 KB within a stage (wavefront-uniform)
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+        if (i < LOADS_A) {
+            const int idx = wave + i * WAVES;
+            load_lds[i] = idx * 1024;
+            if (AT) {  // tile [16 k][BM]: lane covers floats idx*256 + lane*4 .. +3
+                const int f = idx * 256 + lane * 4;
+                const int k = f / BM, col = f % BM;
+                load_off[i] = (m0 + col < M) ? (static_cast<unsigned>(k) * M + m0 + col) * 4u : kOutside;
+            } else {   // tile [BM][16 k]: lane lands at row idx*16 + lane/4, chunk position lane%4
+                const int row = idx * 16 + (lane >> 2);
+                const int chunk = (lane & 3) ^ ((row >> 2) & 3);
+                load_off[i] = (m0 + row < M) ? (static_cast<unsigned>(m0 + row) * K + chunk * 4) * 4u : kOutside;
+            }
+        } else {
+            const int j = wave + (i - LOADS_A) * WAVES;
+            load_lds[i] = A_BYTES + j * 1024;
+            const int f = j * 256 + lane * 4;
+            const int k = f / BN, col = f % BN;
+            load_off[i] = (n0 + col < N) ? (static_cast<unsigned>(k) * N + n0 + col) * 4u : kOutside;
+        }
+    }
+    const unsigned a_step = AT ? static_cast<unsigned>(BK) * M * 4u : BK * 4u;  // bytes per k-tile
+    const unsigned b_step = static_cast<unsigned>(BK) * N * 4u;
+
+    auto issue = [&](auto slot_tag, int t) {
+        constexpr int SLOT = decltype(slot_tag)::value;
+#pragma unroll
+        for (int i = 0; i < LOADS; ++i) {
+            lds_void_ptr dst = (lds_void_ptr)(ring_lds + SLOT * STAGE + load_lds[i]);
+            if (i < LOADS_A)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, dst, 16, load_off[i], t * a_step, 0, 0);
+            else
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, dst, 16, load_off[i], t * b_step, 0, 0);
+        }
+    };
+
+    // Per-lane fragment offsets within a stage.
+    unsigned a_lane[BK / 8][TM], b_lane[TN];
+#pragma unroll
+    for (int kk = 0; kk < BK / 8; ++kk)
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm) {
+            const int row = wm * WTM + tm * 32 + li;
+            a_lane[kk][tm] = AT ? ((kk * 8 + lh * 4) * BM + row) * 4
+                                : row * 64 + (((kk * 2 + lh) ^ ((row >> 2) & 3)) * 16);
+        }
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) b_lane[tn] = A_BYTES + (lh * 4 * BN + wn * WTN + tn * 32 + li) * 4;
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int a = 0; a < TM; ++a)
+#pragma unroll
+        for (int b = 0; b < TN; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.0f;
+
+    auto compute = [&](auto slot_tag) {
+        constexpr int SLOT = decltype(slot_tag)::value;
+        const unsigned char *stage = ring_lds + SLOT * STAGE;
+        float a[BK / 8][TM][4], b[BK / 8][TN][4];
+#pragma unroll
+        for (int kk = 0; kk < BK / 8; ++kk) {
+#pragma unroll
+            for (int tm = 0; tm < TM; ++tm) {
+                if (AT) {
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+                        a[kk][tm][t] = *reinterpret_cast<const float *>(stage + a_lane[kk][tm] + t * BM * 4);
+                } else {
+                    const f32x4 v = *reinterpret_cast<const f32x4 *>(stage + a_lane[kk][tm]);
+                    a[kk][tm][0] = v[0]; a[kk][tm][1] = v[1]; a[kk][tm][2] = v[2]; a[kk][tm][3] = v[3];
+                }
+            }
+#pragma unroll
+            for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    b[kk][tn][t] = *reinterpret_cast<const float *>(stage + b_lane[tn] + (kk * 8 + t) * BN * 4);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_setprio(2);
+#pragma unroll
+        for (int kk = 0; kk < BK / 8; ++kk)
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+                    for (int tn = 0; tn < TN; ++tn)
+                        acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kk][tm][t], b[kk][tn][t], acc[tm][tn], 0, 0, 0);
+        __builtin_amdgcn_s_setprio(0);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    const int steps = K / BK;
+    if (steps > 0) issue(std::integral_constant<int, 0>{}, 0);
+    if (steps > 1) issue(std::integral_constant<int, 1>{}, 1);
+    // Drain the prologue once: loads still counted as outstanding at the loop header make the compiler's
+    // wait-count insertion fall back to a full vmcnt(0) inside the loop.
+    ST_F32_WAIT_VMCNT(0);
+    auto step = [&](auto slot_tag, int t) {
+        constexpr int SLOT = decltype(slot_tag)::value;
+        // This wavefront's loads of k-tile t have landed once only those of k-tile t+1 are outstanding; the
+        // barrier extends that to every wavefront and says that all are done reading the slot k-tile t+2
+        // overwrites.  It is a bare s_barrier: __syncthreads() carries a release fence that makes the
+        // compiler wait for every outstanding load, including the k-tile just requested.  No ordinary store
+        // writes LDS in the loop, and a wavefront's reads of a slot have returned before its next barrier.
+        if (t + 1 < steps) ST_F32_WAIT_VMCNT(LOADS);
+        else ST_F32_WAIT_VMCNT(0);
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if (t + 2 < steps) issue(std::integral_constant<int, (SLOT + 2) % RING>{}, t + 2);
+        compute(slot_tag);
+    };
+    int t = 0;
+    for (; t + 3 <= steps; t += 3) {
+        step(std::integral_constant<int, 0>{}, t);
+        step(std::integral_constant<int, 1>{}, t + 1);
+        step(std::integral_constant<int, 2>{}, t + 2);
+    }
+    if (t < steps) step(std::integral_constant<int, 0>{}, t);
+    if (t + 1 < steps) step(std::integral_constant<int, 1>{}, t + 1);
+
+    const bool scaled = p.scale != 1.0f;
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) {
+        const int col = n0 + wn * WTN + tn * 32 + li;
+        const bool col_ok = col < N;
+        const float bias = (p.bias && col_ok) ? p.bias[col] : 0.0f;
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm) {
+            const f32x16 tile = acc[tm][tn];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = m0 + wm * WTM + tm * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
+                if (col_ok && row < M) {
+                    const size_t idx = static_cast<size_t>(row) * N + col;
+                    float value = tile[r];
+                    if (scaled) value *= p.scale;
+                    value += bias;
+                    if (p.residual) value += p.residual[idx];
+                    p.C[idx] = apply_activation(value, p.activation);
+                }
+            }
+        }
+    }
+}
+
+// (Plain kernels around the templated body: a kernel template whose body uses the LDS-load builtins loses
+// its host-side launch stub with this compiler.)
+__global__ __launch_bounds__(512) void gemm_f32_ring_128x128_kernel(GemmF32Args p) { gemm_f32_ring_body<128, 128, 4, 2, false>(p); }
+__global__ __launch_bounds__(512) void gemm_f32_ring_128x128_at_kernel(GemmF32Args p) { gemm_f32_ring_body<128, 128, 4, 2, true>(p); }
+__global__ __launch_bounds__(256) void gemm_f32_ring_64x64_kernel(GemmF32Args p) { gemm_f32_ring_body<64, 64, 2, 2, false>(p); }
+__global__ __launch_bounds__(256) void gemm_f32_ring_64x64_at_kernel(GemmF32Args p) { gemm_f32_ring_body<64, 64, 2, 2, true>(p); }
+
+hipError_t launch_ring(GemmF32Args args, bool lhs_transposed, bool big, hipStream_t stream)
+{
+    const int bm = big ? 128 : 64, bn = big ? 128 : 64;
+    args.tiles_n = (args.N + bn - 1) / bn;
+    args.tiles_m = (args.M + bm - 1) / bm;
+    const size_t tiles = static_cast<size_t>(args.tiles_n) * static_cast<size_t>(args.tiles_m);
+    if (tiles > 0x7fffffffu) return hipErrorInvalidConfiguration;
+    const size_t lds_bytes = 3 * static_cast<size_t>(bm + bn) * 16 * 4;
+    auto kernel = big ? (lhs_transposed ? gemm_f32_ring_128x128_at_kernel : gemm_f32_ring_128x128_kernel)
+                      : (lhs_transposed ? gemm_f32_ring_64x64_at_kernel : gemm_f32_ring_64x64_kernel);
+    hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        static_cast<int>(lds_bytes));
+    if (rc != hipSuccess) return rc;
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(tiles)), dim3(big ? 512 : 256), lds_bytes, stream, args);
+    return hipGetLastError();
+}
 
 }  // namespace
 
@@ -307,9 +547,19 @@ hipError_t launch_gemm_f32(size_t m, size_t n, size_t k, bool lhs_transposed, co
     const bool vec = (lhs_ld % 4 == 0) && (n % 4 == 0) && aligned16(lhs) && aligned16(rhs);
     // 256×256 tiles (16 wavefronts of 64×64) once they give every compute unit a full tile without padding
     // waste; otherwise 64×64 tiles (4 wavefronts of 32×32), which spread small and narrow problems over the chip.
+    // The ring kernel wants whole 16-wide k-tiles, 16-byte aligned rows and 32-bit byte offsets.
+    const bool ring_ok = vec && k >= 16 && k % 16 == 0 && m * k * 4 < (1ull << 31) && k * n * 4 < (1ull << 31) &&
+                         (!lhs_transposed || m % 4 == 0);
     const size_t big_tiles = ((m + 255) / 256) * ((n + 255) / 256);
     const bool little_padding = (m % 256 == 0 || m >= 2048) && (n % 256 == 0 || n >= 2048);
     if (big_tiles >= 256 && little_padding) return launch_tile<256, 256, 4, 4>(args, lhs_transposed, vec, stream);
+    if (ring_ok) {
+        // 128×128 tiles (three workgroups per compute unit, 768 at a time) when they come in full rounds or many
+        // rounds; 64×64 tiles otherwise, which spread small problems and leave a shorter tail.
+        const size_t tiles128 = ((m + 127) / 128) * ((n + 127) / 128);
+        const bool big = tiles128 >= 512 && (tiles128 >= 3072 || tiles128 % 768 == 0 || tiles128 % 768 >= 384);
+        return launch_ring(args, lhs_transposed, big, stream);
+    }
     return launch_tile<64, 64, 2, 2>(args, lhs_transposed, vec, stream);
 }
 

@@ -82,7 +82,9 @@ def test_empty_output_is_a_no_op(hip):
 
 
 SHAPES = [(1, 1, 1), (2, 3, 4), (8, 12, 7), (10, 13, 9), (8, 16, 6), (4, 16, 5), (33, 65, 17), (64, 64, 64),
-          (100, 130, 70), (129, 127, 31), (256, 64, 200), (5, 300, 19), (300, 5, 23)]
+          (100, 130, 70), (129, 127, 31), (256, 64, 200), (5, 300, 19), (300, 5, 23),
+          # whole 16-wide k-tiles and 16-byte aligned rows: the direct-to-LDS ring kernel, ragged in m and n
+          (132, 136, 48), (260, 68, 160), (96, 260, 16), (1000, 128, 32)]
 
 
 @pytest.mark.parametrize("m,n,k", SHAPES)
@@ -133,6 +135,27 @@ def test_large_tile_path_and_linearity(hip, oracle):
     out2 = np.zeros(m * n, np.float32)
     hip.gemm_f32(m, n, k, 2 * a, b, out2)
     assert (out2 == 2 * out).all()
+
+
+def test_ring_kernel_128_tiles_ragged_edges(hip, oracle):
+    """24 x 23 tiles of 128x128 with ragged last tiles in both directions, plain and lhs-transposed, with the
+    fused epilogue; every element is checked."""
+    rng = np.random.default_rng(4)
+    m, n, k = 3000, 2820, 64
+    a = rng.uniform(-1, 1, m * k).astype(np.float32)
+    b = rng.uniform(-1, 1, k * n).astype(np.float32)
+    bias = rng.uniform(-1, 1, n).astype(np.float32)
+    res = rng.uniform(-1, 1, m * n).astype(np.float32)
+    out = np.zeros(m * n, np.float32)
+    want = oracle.gemm_f32(m, n, k, a, b, threads=8)
+    hip.gemm_f32(m, n, k, a, b, out)
+    assert_close(out, want, F32_REL, F32_ABS, "plain")
+    at = np.ascontiguousarray(a.reshape(m, k).T).ravel()
+    hip.gemm_lhs_transpose_scaled_f32(m, n, k, 0.5, at, b, out)
+    assert_close(out, 0.5 * want.astype(np.float64), F32_REL, F32_ABS, "lhs^T scaled")
+    hip.gemm_bias_activation_f32(m, n, k, hip.GemmActivation.Relu, a, b, bias, res, out)
+    pre = (want.astype(np.float64).reshape(m, n) + bias).ravel() + res
+    assert_close(out, np.maximum(pre, 0), F32_REL, F32_ABS, "bias+residual+relu")
 
 
 def test_tensor_mirror_matches_the_reference_api(hip, oracle):
