@@ -168,6 +168,23 @@ int st_hip_attention_bf16_dev(size_t batch, size_t heads, size_t sequence, size_
                               int causal, const uint16_t *q, const uint16_t *k, const uint16_t *v,
                               size_t ld_in, uint16_t *out, size_t ld_out, void *stream);
 
+/* Tensor utilities the reference's HIP policy still leaves on the CPU (device pointers, async on `stream`).
+ * row_softmax:   Tensor::row_softmax CPU path, crates/st-tensor/src/pure.rs:3277-3335 with
+ *                cpu_row_softmax_hardmax :11930-11980 (NaN entries skipped, one-hot fallback when the
+ *                denominator is not above f32 epsilon).
+ * gelu_backward: out = gelu_prime(z) * grad, pure.rs:6454-6552, gelu_prime :12033-12040.
+ * scale:         out = in * scale (out may alias in), pure.rs:5625-5700, scale_inplace :11993-11997;
+ *                a non-finite scale is rejected like validate_scale_factor :5535-5543.
+ * add_row:       data[r][c] += bias[c] in place, pure.rs:6196-6290.
+ * sum_axis0:     out[c] = (sum over rows of in[r][c]) * scale, pure.rs:6999-7210 (scale 1 is sum_axis0). */
+int st_hip_row_softmax_f32_dev(size_t rows, size_t cols, const float *in, float *out, void *stream);
+int st_hip_gelu_backward_f32_dev(size_t count, const float *z, const float *grad, float *out,
+                                 void *stream);
+int st_hip_scale_f32_dev(size_t count, const float *in, float scale, float *out, void *stream);
+int st_hip_add_row_f32_dev(size_t rows, size_t cols, float *data, const float *bias, void *stream);
+int st_hip_sum_axis0_f32_dev(size_t rows, size_t cols, const float *in, float scale, float *out,
+                             void *stream);
+
 /* Row-wise building blocks of the decoder stack.
  * layer_norm: crates/st-tensor/src/pure.rs:4008-4058; writes f32 and/or bf16 (either may be NULL).
  * embedding:  crates/st-nn/src/layers/embedding.rs:42-100,325-330 (round, clamp, gather).

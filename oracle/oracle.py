@@ -62,6 +62,11 @@ def load() -> ctypes.CDLL:
     lib.st_oracle_attention_f64.argtypes = [S, S, S, c_double, I, P, P, P, P, P, P]
     lib.st_oracle_layer_norm_f32.argtypes = [S, S, P, P, P, P, F, P]
     lib.st_oracle_embedding_f32.argtypes = [S, S, S, P, P, P]
+    lib.st_oracle_row_softmax_f32.argtypes = [S, S, P, P]
+    lib.st_oracle_gelu_backward_f32.argtypes = [S, P, P, P]
+    lib.st_oracle_scale_f32.argtypes = [S, P, F, P]
+    lib.st_oracle_add_row_f32.argtypes = [S, S, P, P]
+    lib.st_oracle_sum_axis0_f32.argtypes = [S, S, P, F, P]
     lib.st_oracle_gelu.argtypes = [F]
     lib.st_oracle_gelu.restype = F
     lib.st_oracle_f32_to_bf16.argtypes = [S, P, P]
@@ -164,6 +169,40 @@ def layer_norm_f32(rows, cols, x, gamma, beta, epsilon, residual=None) -> np.nda
     residual = None if residual is None else _f32(residual)
     out = np.zeros(rows * cols, dtype=np.float32)
     _check(load().st_oracle_layer_norm_f32(rows, cols, _p(x), _p(residual), _p(gamma), _p(beta), epsilon, _p(out)))
+    return out
+
+
+def row_softmax_f32(rows, cols, x) -> np.ndarray:
+    x = _f32(x)
+    out = np.zeros(rows * cols, dtype=np.float32)
+    _check(load().st_oracle_row_softmax_f32(rows, cols, _p(x), _p(out)))
+    return out
+
+
+def gelu_backward_f32(z, grad) -> np.ndarray:
+    z, grad = _f32(z), _f32(grad)
+    out = np.zeros(z.size, dtype=np.float32)
+    _check(load().st_oracle_gelu_backward_f32(z.size, _p(z), _p(grad), _p(out)))
+    return out
+
+
+def scale_f32(x, scale) -> np.ndarray:
+    x = _f32(x)
+    out = np.zeros(x.size, dtype=np.float32)
+    _check(load().st_oracle_scale_f32(x.size, _p(x), scale, _p(out)))
+    return out
+
+
+def add_row_f32(rows, cols, data, bias) -> np.ndarray:
+    out, bias = _f32(data).copy(), _f32(bias)
+    _check(load().st_oracle_add_row_f32(rows, cols, _p(out), _p(bias)))
+    return out
+
+
+def sum_axis0_f32(rows, cols, x, scale=1.0) -> np.ndarray:
+    x = _f32(x)
+    out = np.zeros(cols, dtype=np.float32)
+    _check(load().st_oracle_sum_axis0_f32(rows, cols, _p(x), scale, _p(out)))
     return out
 
 

@@ -18,6 +18,7 @@
  */
 #include "st_oracle.h"
 
+#include <float.h>
 #include <math.h>
 #include <stdlib.h>
 #include <string.h>
@@ -375,6 +376,85 @@ int st_oracle_attention_f64(size_t contexts, size_t sequence, size_t head_dim, d
         }
     }
     free(logits);
+    return ST_ORACLE_OK;
+}
+
+/* crates/st-tensor/src/pure.rs:11930-11986 (cpu_row_softmax_hardmax, softmax half). */
+int st_oracle_row_softmax_f32(size_t rows, size_t cols, const float *in, float *out)
+{
+    for (size_t row = 0; row < rows; ++row) {
+        const float *x = in + row * cols;
+        float *y = out + row * cols;
+        float max_value = -INFINITY;
+        size_t max_index = 0;
+        int found = 0;
+        for (size_t i = 0; i < cols; ++i) {
+            const float value = x[i];
+            if (isnan(value)) continue;
+            if (!found || value > max_value) {
+                max_value = value;
+                max_index = i;
+                found = 1;
+            }
+        }
+        const float base = (found && isfinite(max_value)) ? max_value : 0.0f;
+        float denom = 0.0f;
+        for (size_t i = 0; i < cols; ++i) {
+            const float weight = (!found || isnan(x[i])) ? 0.0f : expf(x[i] - base);
+            y[i] = weight;
+            denom = denom + weight;
+        }
+        if (found) {
+            if (isfinite(denom) && denom > FLT_EPSILON) {
+                const float inv = 1.0f / denom;
+                for (size_t i = 0; i < cols; ++i) y[i] = y[i] * inv;
+            } else {
+                for (size_t i = 0; i < cols; ++i) y[i] = 0.0f;
+                y[max_index] = 1.0f;
+            }
+        }
+    }
+    return ST_ORACLE_OK;
+}
+
+/* crates/st-tensor/src/pure.rs:12033-12040 (gelu_prime) times the incoming gradient (:6549-6552). */
+int st_oracle_gelu_backward_f32(size_t count, const float *z, const float *grad, float *out)
+{
+    const float sqrt_2_over_pi = 0.7978846f, kappa = 0.044715f;
+    for (size_t i = 0; i < count; ++i) {
+        const float x = z[i];
+        const float x2 = x * x;
+        const float inner = sqrt_2_over_pi * (x + (kappa * x) * x2);
+        const float t = tanhf(inner);
+        const float left = 0.5f * (1.0f + t);
+        const float right = (((0.5f * x) * (1.0f - t * t)) * sqrt_2_over_pi) * (1.0f + (3.0f * kappa) * x2);
+        out[i] = (left + right) * grad[i];
+    }
+    return ST_ORACLE_OK;
+}
+
+/* crates/st-tensor/src/pure.rs:11993-11997 (scale_inplace). */
+int st_oracle_scale_f32(size_t count, const float *in, float scale, float *out)
+{
+    for (size_t i = 0; i < count; ++i) out[i] = in[i] * scale;
+    return ST_ORACLE_OK;
+}
+
+/* crates/st-tensor/src/pure.rs:6284-6288 (add_row_inplace: value += bias per column). */
+int st_oracle_add_row_f32(size_t rows, size_t cols, float *data, const float *bias)
+{
+    for (size_t r = 0; r < rows; ++r)
+        for (size_t c = 0; c < cols; ++c) data[r * cols + c] = data[r * cols + c] + bias[c];
+    return ST_ORACLE_OK;
+}
+
+/* crates/st-tensor/src/pure.rs:7201-7210 (sum_axis0_scaled: rows added in order, then one multiply). */
+int st_oracle_sum_axis0_f32(size_t rows, size_t cols, const float *in, float scale, float *out)
+{
+    for (size_t c = 0; c < cols; ++c) out[c] = 0.0f;
+    for (size_t r = 0; r < rows; ++r)
+        for (size_t c = 0; c < cols; ++c) out[c] = out[c] + in[r * cols + c];
+    for (size_t c = 0; c < cols; ++c) out[c] = out[c] * scale;
     return ST_ORACLE_OK;
 }
 

@@ -80,6 +80,14 @@ int st_oracle_attention_f64(size_t contexts, size_t sequence, size_t head_dim, d
 int st_oracle_layer_norm_f32(size_t rows, size_t cols, const float *x, const float *residual,
                              const float *gamma, const float *beta, float epsilon, float *out);
 
+/* Tensor utilities: row_softmax (pure.rs:11930-11986), gelu_backward (:12033-12040, :6549-6552),
+ * scale (:11993-11997), add_row (:6284-6288), sum_axis0[_scaled] (:7201-7210). */
+int st_oracle_row_softmax_f32(size_t rows, size_t cols, const float *in, float *out);
+int st_oracle_gelu_backward_f32(size_t count, const float *z, const float *grad, float *out);
+int st_oracle_scale_f32(size_t count, const float *in, float scale, float *out);
+int st_oracle_add_row_f32(size_t rows, size_t cols, float *data, const float *bias);
+int st_oracle_sum_axis0_f32(size_t rows, size_t cols, const float *in, float scale, float *out);
+
 /* Token ids as f32 -> rows of table(vocab, dim); round, clamp to [0, vocab-1], non-finite -> 0. */
 int st_oracle_embedding_f32(size_t tokens, size_t vocab, size_t dim, const float *token_ids,
                             const float *table, float *out);

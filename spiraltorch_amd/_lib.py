@@ -92,6 +92,11 @@ SIGNATURES = {
                                          c_void_p, c_void_p, c_void_p, c_void_p]),
     "st_hip_attention_bf16_dev": (c_int, [c_size_t, c_size_t, c_size_t, c_size_t, c_float, c_int, c_void_p, c_void_p,
                                           c_void_p, c_size_t, c_void_p, c_size_t, c_void_p]),
+    "st_hip_row_softmax_f32_dev": (c_int, [c_size_t, c_size_t, c_void_p, c_void_p, c_void_p]),
+    "st_hip_gelu_backward_f32_dev": (c_int, [c_size_t, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "st_hip_scale_f32_dev": (c_int, [c_size_t, c_void_p, c_float, c_void_p, c_void_p]),
+    "st_hip_add_row_f32_dev": (c_int, [c_size_t, c_size_t, c_void_p, c_void_p, c_void_p]),
+    "st_hip_sum_axis0_f32_dev": (c_int, [c_size_t, c_size_t, c_void_p, c_float, c_void_p, c_void_p]),
     "st_hip_layer_norm_f32_dev": (c_int, [c_size_t, c_size_t, c_void_p, c_void_p, c_void_p, c_void_p, c_float,
                                           c_void_p, c_void_p, c_void_p]),
     "st_hip_embedding_f32_dev": (c_int, [c_size_t, c_size_t, c_size_t, c_void_p, c_void_p, c_void_p, c_void_p]),

@@ -661,43 +661,6 @@ __global__ __launch_bounds__(256) void gemm_bf16_skinny_reduce_kernel(SkinnyArgs
     if (p.C16) p.C16[idx] = f32_to_bf16_rne(value);
 }
 
-// Split-k partial sums live in one grow-only device buffer per stream: work on a stream is ordered, so two
-// launches on the same stream never use the buffer at the same time, and different streams get different
-// buffers.  (hipMallocAsync/hipFreeAsync per call cost several times the kernel itself.)
-hipError_t split_k_workspace(hipStream_t stream, size_t bytes, float **out)
-{
-    struct Entry {
-        hipStream_t stream;
-        void *ptr;
-        size_t capacity;
-    };
-    static std::mutex mutex;
-    static std::vector<Entry> entries;
-    std::lock_guard<std::mutex> lock(mutex);
-    for (Entry &e : entries) {
-        if (e.stream != stream) continue;
-        if (e.capacity < bytes) {
-            hipError_t rc = hipStreamSynchronize(stream);
-            if (rc != hipSuccess) return rc;
-            rc = hipFree(e.ptr);
-            if (rc != hipSuccess) return rc;
-            e.ptr = nullptr;
-            e.capacity = 0;
-            rc = hipMalloc(&e.ptr, bytes);
-            if (rc != hipSuccess) return rc;
-            e.capacity = bytes;
-        }
-        *out = static_cast<float *>(e.ptr);
-        return hipSuccess;
-    }
-    Entry fresh{stream, nullptr, bytes};
-    hipError_t rc = hipMalloc(&fresh.ptr, bytes);
-    if (rc != hipSuccess) return rc;
-    entries.push_back(fresh);
-    *out = static_cast<float *>(fresh.ptr);
-    return hipSuccess;
-}
-
 hipError_t launch_skinny(const GemmBf16Args &args, hipStream_t stream)
 {
     SkinnyArgs sk;
@@ -715,7 +678,9 @@ hipError_t launch_skinny(const GemmBf16Args &args, hipStream_t stream)
     sk.tiles_per_split = (k_tiles + splits - 1) / splits;
     sk.k_splits = (k_tiles + sk.tiles_per_split - 1) / sk.tiles_per_split;
     const size_t bytes = static_cast<size_t>(sk.k_splits) * args.M * args.N * sizeof(float);
-    hipError_t rc = split_k_workspace(stream, bytes, &sk.partial);
+    void *workspace = nullptr;
+    hipError_t rc = stream_workspace(stream, bytes, &workspace);  // hipMallocAsync/hipFreeAsync per call cost more than the kernel
+    sk.partial = static_cast<float *>(workspace);
     if (rc != hipSuccess) return rc;
     sk.C32 = args.C32;
     sk.C16 = args.C16;

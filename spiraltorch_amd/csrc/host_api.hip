@@ -619,6 +619,56 @@ int st_hip_attention_bf16_dev(size_t batch, size_t heads, size_t sequence, size_
                          "attention launch");
 }
 
+int st_hip_row_softmax_f32_dev(size_t rows, size_t cols, const float *in, float *out, void *stream)
+{
+    ST_HIP_CHECK(ensure_init());
+    if (rows > kMaxDim || cols > kMaxDim) return fail(ST_HIP_ERR_UNSUPPORTED, "row_softmax dimension exceeds i32");
+    if (rows == 0 || cols == 0) return ST_HIP_OK;
+    if (!in || !out) return fail(ST_HIP_ERR_INVALID, "row_softmax received a null pointer");
+    return launch_status(launch_row_softmax_f32(rows, cols, in, out, as_stream(stream)), "row_softmax launch");
+}
+
+int st_hip_gelu_backward_f32_dev(size_t count, const float *z, const float *grad, float *out, void *stream)
+{
+    ST_HIP_CHECK(ensure_init());
+    if (count == 0) return ST_HIP_OK;
+    if (!z || !grad || !out) return fail(ST_HIP_ERR_INVALID, "gelu_backward received a null pointer");
+    return launch_status(launch_gelu_backward_f32(count, z, grad, out, as_stream(stream)), "gelu_backward launch");
+}
+
+int st_hip_scale_f32_dev(size_t count, const float *in, float scale, float *out, void *stream)
+{
+    ST_HIP_CHECK(ensure_init());
+    if (!std::isfinite(scale))
+        return fail(ST_HIP_ERR_NONFINITE, "non-finite value encountered in scale_factor: %g", static_cast<double>(scale));
+    if (count == 0) return ST_HIP_OK;
+    if (!in || !out) return fail(ST_HIP_ERR_INVALID, "scale received a null pointer");
+    return launch_status(launch_scale_f32(count, in, scale, out, as_stream(stream)), "scale launch");
+}
+
+int st_hip_add_row_f32_dev(size_t rows, size_t cols, float *data, const float *bias, void *stream)
+{
+    ST_HIP_CHECK(ensure_init());
+    size_t count = 0;
+    if (!checked_mul(rows, cols, &count)) return fail(ST_HIP_ERR_INVALID, "add_row dimensions overflow");
+    if (cols > kMaxDim) return fail(ST_HIP_ERR_UNSUPPORTED, "add_row dimension exceeds i32");
+    if (count == 0) return ST_HIP_OK;
+    if (!data || !bias) return fail(ST_HIP_ERR_INVALID, "add_row received a null pointer");
+    return launch_status(launch_add_row_f32(rows, cols, data, bias, as_stream(stream)), "add_row launch");
+}
+
+int st_hip_sum_axis0_f32_dev(size_t rows, size_t cols, const float *in, float scale, float *out, void *stream)
+{
+    ST_HIP_CHECK(ensure_init());
+    if (!std::isfinite(scale))
+        return fail(ST_HIP_ERR_NONFINITE, "non-finite value encountered in sum_axis0_scaled_factor: %g",
+                    static_cast<double>(scale));
+    if (rows > kMaxDim || cols > kMaxDim) return fail(ST_HIP_ERR_UNSUPPORTED, "sum_axis0 dimension exceeds i32");
+    if (cols == 0) return ST_HIP_OK;
+    if (!out || (rows != 0 && !in)) return fail(ST_HIP_ERR_INVALID, "sum_axis0 received a null pointer");
+    return launch_status(launch_sum_axis0_f32(rows, cols, in, scale, out, as_stream(stream)), "sum_axis0 launch");
+}
+
 int st_hip_layer_norm_f32_dev(size_t rows, size_t cols, const float *x, const float *residual, const float *gamma,
                               const float *beta, float epsilon, float *out_f32, uint16_t *out_bf16, void *stream)
 {

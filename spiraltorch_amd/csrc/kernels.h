@@ -59,4 +59,16 @@ hipError_t launch_merge_heads_f32(size_t batch, size_t seq, size_t heads, size_t
                                   const float *contexts_in, float *out_f32, uint16_t *out_bf16,
                                   hipStream_t stream);
 
+// Element-wise and row-wise tensor utilities (all f32, row-major).
+hipError_t launch_row_softmax_f32(size_t rows, size_t cols, const float *in, float *out, hipStream_t stream);
+hipError_t launch_gelu_backward_f32(size_t count, const float *z, const float *grad, float *out, hipStream_t stream);
+hipError_t launch_scale_f32(size_t count, const float *in, float scale, float *out, hipStream_t stream);
+hipError_t launch_add_row_f32(size_t rows, size_t cols, float *data, const float *bias, hipStream_t stream);
+hipError_t launch_sum_axis0_f32(size_t rows, size_t cols, const float *in, float scale, float *out, hipStream_t stream);
+
+// One grow-only device buffer per stream for kernels that need scratch memory (split-k partial sums, column-sum
+// partials).  Work on a stream is ordered, so two launches on the same stream never use it at the same time.
+hipError_t stream_workspace(hipStream_t stream, size_t bytes, void **out);
+void release_stream_workspace(hipStream_t stream);
+
 }  // namespace sthip

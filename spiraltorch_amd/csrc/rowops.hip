@@ -116,6 +116,111 @@ __global__ __launch_bounds__(256) void merge_heads_kernel(int batch, int seq, in
     }
 }
 
+__device__ __forceinline__ float wave_max(float v)
+{
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) v = fmaxf(v, __shfl_xor(v, offset));
+    return v;
+}
+
+// One wavefront per row.  cpu_row_softmax_hardmax, crates/st-tensor/src/pure.rs:11930-11980: the maximum is
+// taken over the non-NaN entries (first occurrence wins), base = max if finite else 0, weights exp(v - base)
+// (0 for NaN), divided by their sum when that is finite and above f32 epsilon; otherwise the row becomes the
+// one-hot of the maximum.  A row of only NaNs gives zeros.
+__global__ __launch_bounds__(256) void row_softmax_kernel(int rows, int cols, const float *in, float *out)
+{
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const float *x = in + static_cast<size_t>(row) * cols;
+    float *y = out + static_cast<size_t>(row) * cols;
+    float best = -INFINITY;
+    int best_index = 0x7fffffff;
+    for (int c = lane; c < cols; c += 64) {
+        const float v = x[c];
+        if (v != v) continue;
+        if (best_index == 0x7fffffff || v > best) {
+            best = v;
+            best_index = c;
+        }
+    }
+    // first occurrence of the largest value across the wavefront
+    const float row_max = wave_max(best_index == 0x7fffffff ? -INFINITY : best);
+    int candidate = (best_index != 0x7fffffff && best == row_max) ? best_index : 0x7fffffff;
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) candidate = min(candidate, __shfl_xor(candidate, offset));
+    const bool found = candidate != 0x7fffffff;
+    const float base = (found && isfinite(row_max)) ? row_max : 0.0f;
+    float denom = 0.0f;
+    for (int c = lane; c < cols; c += 64) {
+        const float v = x[c];
+        denom += (!found || v != v) ? 0.0f : expf(v - base);
+    }
+    denom = wave_sum(denom);
+    const bool normal = isfinite(denom) && denom > 1.1920929e-7f;
+    const float inv = normal ? 1.0f / denom : 0.0f;
+    for (int c = lane; c < cols; c += 64) {
+        const float v = x[c];
+        const float weight = (!found || v != v) ? 0.0f : expf(v - base);
+        float value = weight * inv;
+        if (found && !normal) value = c == candidate ? 1.0f : 0.0f;
+        y[c] = value;
+    }
+}
+
+// gelu_prime(z)·g, crates/st-tensor/src/pure.rs:12033-12040 and :6549-6552.
+__global__ __launch_bounds__(256) void gelu_backward_kernel(size_t count, const float *z, const float *grad, float *out)
+{
+    const size_t stride = static_cast<size_t>(gridDim.x) * 256;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < count; i += stride) {
+        const float x = z[i];
+        const float x2 = x * x;
+        const float inner = 0.7978846f * (x + (0.044715f * x) * x2);
+        const float t = tanhf(inner);
+        const float prime = 0.5f * (1.0f + t) + (((0.5f * x) * (1.0f - t * t)) * 0.7978846f) * (1.0f + (3.0f * 0.044715f) * x2);
+        out[i] = prime * grad[i];
+    }
+}
+
+// scale_inplace, crates/st-tensor/src/pure.rs:11993-11997 (out may alias in).
+__global__ __launch_bounds__(256) void scale_kernel(size_t count, const float *in, float scale, float *out)
+{
+    const size_t stride = static_cast<size_t>(gridDim.x) * 256;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < count; i += stride) out[i] = in[i] * scale;
+}
+
+// add_row_inplace, crates/st-tensor/src/pure.rs:6196-6290: data[r][c] += bias[c].
+__global__ __launch_bounds__(256) void add_row_kernel(size_t count, int cols, float *data, const float *bias)
+{
+    const size_t stride = static_cast<size_t>(gridDim.x) * 256;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < count; i += stride)
+        data[i] += bias[i % static_cast<size_t>(cols)];
+}
+
+// Column sums, crates/st-tensor/src/pure.rs:7201-7210: stage one adds the rows of one chunk per workgroup row
+// (threads along columns, so loads are coalesced); stage two adds the chunks in order and applies the scale.
+__global__ __launch_bounds__(256) void sum_axis0_partial_kernel(int rows, int cols, int rows_per_chunk, const float *in,
+                                                                float *partial)
+{
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= cols) return;
+    const int r0 = blockIdx.y * rows_per_chunk;
+    const int r1 = min(rows, r0 + rows_per_chunk);
+    float sum = 0.0f;
+    for (int r = r0; r < r1; ++r) sum += in[static_cast<size_t>(r) * cols + c];
+    partial[static_cast<size_t>(blockIdx.y) * cols + c] = sum;
+}
+
+__global__ __launch_bounds__(256) void sum_axis0_final_kernel(int chunks, int cols, const float *partial, float scale,
+                                                              float *out)
+{
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= cols) return;
+    float sum = 0.0f;
+    for (int k = 0; k < chunks; ++k) sum += partial[static_cast<size_t>(k) * cols + c];
+    out[c] = sum * scale;
+}
+
 unsigned grid_for(size_t count)
 {
     const size_t blocks = (count + 255) / 256;
@@ -173,6 +278,62 @@ hipError_t launch_merge_heads_f32(size_t batch, size_t seq, size_t heads, size_t
     hipLaunchKernelGGL(merge_heads_kernel, dim3(grid_for(total)), dim3(256), 0, stream, static_cast<int>(batch),
                        static_cast<int>(seq), static_cast<int>(heads), static_cast<int>(head_dim), contexts_in, out_f32,
                        out_bf16);
+    return hipGetLastError();
+}
+
+hipError_t launch_row_softmax_f32(size_t rows, size_t cols, const float *in, float *out, hipStream_t stream)
+{
+    if (rows == 0 || cols == 0) return hipSuccess;
+    hipLaunchKernelGGL(row_softmax_kernel, dim3(static_cast<unsigned>((rows + 3) / 4)), dim3(256), 0, stream,
+                       static_cast<int>(rows), static_cast<int>(cols), in, out);
+    return hipGetLastError();
+}
+
+hipError_t launch_gelu_backward_f32(size_t count, const float *z, const float *grad, float *out, hipStream_t stream)
+{
+    if (count == 0) return hipSuccess;
+    hipLaunchKernelGGL(gelu_backward_kernel, dim3(grid_for(count)), dim3(256), 0, stream, count, z, grad, out);
+    return hipGetLastError();
+}
+
+hipError_t launch_scale_f32(size_t count, const float *in, float scale, float *out, hipStream_t stream)
+{
+    if (count == 0) return hipSuccess;
+    hipLaunchKernelGGL(scale_kernel, dim3(grid_for(count)), dim3(256), 0, stream, count, in, scale, out);
+    return hipGetLastError();
+}
+
+hipError_t launch_add_row_f32(size_t rows, size_t cols, float *data, const float *bias, hipStream_t stream)
+{
+    if (rows == 0 || cols == 0) return hipSuccess;
+    hipLaunchKernelGGL(add_row_kernel, dim3(grid_for(rows * cols)), dim3(256), 0, stream, rows * cols,
+                       static_cast<int>(cols), data, bias);
+    return hipGetLastError();
+}
+
+hipError_t launch_sum_axis0_f32(size_t rows, size_t cols, const float *in, float scale, float *out, hipStream_t stream)
+{
+    if (cols == 0) return hipSuccess;
+    // Enough row chunks to occupy the chip, at least 64 rows each; the partial sums live in the stream's workspace.
+    const size_t col_blocks = (cols + 255) / 256;
+    size_t chunks = (2048 + col_blocks - 1) / col_blocks;
+    const size_t max_chunks = (rows + 63) / 64;
+    if (chunks > max_chunks) chunks = max_chunks;
+    if (chunks == 0) chunks = 1;
+    const size_t rows_per_chunk = (rows + chunks - 1) / chunks;
+    if (rows_per_chunk > 0) chunks = (rows + rows_per_chunk - 1) / rows_per_chunk;
+    if (chunks == 0) chunks = 1;
+    void *workspace = nullptr;
+    hipError_t rc = stream_workspace(stream, chunks * cols * sizeof(float), &workspace);
+    if (rc != hipSuccess) return rc;
+    float *partial = static_cast<float *>(workspace);
+    hipLaunchKernelGGL(sum_axis0_partial_kernel, dim3(static_cast<unsigned>(col_blocks), static_cast<unsigned>(chunks)),
+                       dim3(256), 0, stream, static_cast<int>(rows), static_cast<int>(cols),
+                       static_cast<int>(rows_per_chunk), in, partial);
+    rc = hipGetLastError();
+    if (rc != hipSuccess) return rc;
+    hipLaunchKernelGGL(sum_axis0_final_kernel, dim3(static_cast<unsigned>(col_blocks)), dim3(256), 0, stream,
+                       static_cast<int>(chunks), static_cast<int>(cols), partial, scale, out);
     return hipGetLastError();
 }
 

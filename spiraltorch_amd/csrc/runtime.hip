@@ -9,6 +9,7 @@
 #include <vector>
 
 #include "common.h"
+#include "kernels.h"
 
 namespace sthip {
 
@@ -75,6 +76,56 @@ int ensure_init()
     rt.devices.swap(devices);
     rt.ready = true;
     return ST_HIP_OK;
+}
+
+namespace {
+struct WorkspaceEntry {
+    hipStream_t stream;
+    void *ptr;
+    size_t capacity;
+};
+std::mutex workspace_mutex;
+std::vector<WorkspaceEntry> workspace_entries;
+}  // namespace
+
+hipError_t stream_workspace(hipStream_t stream, size_t bytes, void **out)
+{
+    std::lock_guard<std::mutex> lock(workspace_mutex);
+    for (WorkspaceEntry &e : workspace_entries) {
+        if (e.stream != stream) continue;
+        if (e.capacity < bytes) {
+            // Grow: earlier launches on this stream may still be using the old buffer.
+            hipError_t rc = hipStreamSynchronize(stream);
+            if (rc != hipSuccess) return rc;
+            rc = hipFree(e.ptr);
+            if (rc != hipSuccess) return rc;
+            e.ptr = nullptr;
+            e.capacity = 0;
+            rc = hipMalloc(&e.ptr, bytes);
+            if (rc != hipSuccess) return rc;
+            e.capacity = bytes;
+        }
+        *out = e.ptr;
+        return hipSuccess;
+    }
+    WorkspaceEntry fresh{stream, nullptr, bytes ? bytes : 256};
+    hipError_t rc = hipMalloc(&fresh.ptr, fresh.capacity);
+    if (rc != hipSuccess) return rc;
+    workspace_entries.push_back(fresh);
+    *out = fresh.ptr;
+    return hipSuccess;
+}
+
+// Called after the stream has been drained, before it is destroyed.
+void release_stream_workspace(hipStream_t stream)
+{
+    std::lock_guard<std::mutex> lock(workspace_mutex);
+    for (size_t i = 0; i < workspace_entries.size(); ++i) {
+        if (workspace_entries[i].stream != stream) continue;
+        (void)hipFree(workspace_entries[i].ptr);
+        workspace_entries.erase(workspace_entries.begin() + static_cast<long>(i));
+        return;
+    }
 }
 
 }  // namespace sthip
@@ -190,6 +241,7 @@ int st_hip_stream_destroy(void *stream)
     if (!stream) return ST_HIP_OK;
     // Same order as HipStream::drop (real.rs:207-214): drain, then release.
     (void)hipStreamSynchronize(as_stream(stream));
+    release_stream_workspace(as_stream(stream));
     ST_HIP_TRY(hipStreamDestroy(as_stream(stream)), "hipStreamDestroy");
     return ST_HIP_OK;
 }

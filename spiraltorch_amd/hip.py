@@ -324,6 +324,26 @@ def attention_bf16_dev(batch, heads, sequence, head_dim, scale, causal, q, k, v,
                                                  _dev(k), _dev(v), ld_in, _dev(out), ld_out, _stream_ptr(stream)))
 
 
+def row_softmax_f32_dev(rows, cols, src, dst, stream=None) -> None:
+    _check(_lib.load().st_hip_row_softmax_f32_dev(rows, cols, _dev(src), _dev(dst), _stream_ptr(stream)))
+
+
+def gelu_backward_f32_dev(count, z, grad, out, stream=None) -> None:
+    _check(_lib.load().st_hip_gelu_backward_f32_dev(count, _dev(z), _dev(grad), _dev(out), _stream_ptr(stream)))
+
+
+def scale_f32_dev(count, src, scale, dst, stream=None) -> None:
+    _check(_lib.load().st_hip_scale_f32_dev(count, _dev(src), scale, _dev(dst), _stream_ptr(stream)))
+
+
+def add_row_f32_dev(rows, cols, data, bias, stream=None) -> None:
+    _check(_lib.load().st_hip_add_row_f32_dev(rows, cols, _dev(data), _dev(bias), _stream_ptr(stream)))
+
+
+def sum_axis0_f32_dev(rows, cols, src, scale, dst, stream=None) -> None:
+    _check(_lib.load().st_hip_sum_axis0_f32_dev(rows, cols, _dev(src), scale, _dev(dst), _stream_ptr(stream)))
+
+
 def layer_norm_f32_dev(rows, cols, x, residual, gamma, beta, epsilon, out_f32, out_bf16, stream=None) -> None:
     _check(_lib.load().st_hip_layer_norm_f32_dev(rows, cols, _dev(x), _dev(residual), _dev(gamma), _dev(beta),
                                                  epsilon, _dev(out_f32), _dev(out_bf16), _stream_ptr(stream)))

@@ -1,0 +1,88 @@
+"""Parity of the tensor-utility kernels against the CPU oracle (1e-4 rel / 1e-5 abs), through the C ABI."""
+import numpy as np
+import pytest
+
+from conftest import F32_ABS, F32_REL, assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+def on_device(hip, *arrays):
+    return [hip.DeviceBuffer.from_array(np.ascontiguousarray(a, dtype=np.float32)) for a in arrays]
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 1), (2, 4), (5, 63), (7, 64), (3, 65), (33, 1000), (1024, 256), (4, 5000)])
+def test_row_softmax(hip, oracle, rows, cols):
+    rng = np.random.default_rng(rows * 31 + cols)
+    x = (rng.normal(size=rows * cols) * 3).astype(np.float32)
+    (d_in,) = on_device(hip, x)
+    d_out = hip.DeviceBuffer(x.nbytes)
+    hip.row_softmax_f32_dev(rows, cols, d_in, d_out)
+    hip.device_synchronize()
+    got = d_out.to_array(np.float32, rows * cols)
+    assert_close(got, oracle.row_softmax_f32(rows, cols, x), F32_REL, F32_ABS, f"row_softmax {rows}x{cols}")
+    assert_close(got.reshape(rows, cols).sum(axis=1), np.ones(rows), F32_REL, F32_ABS, "row sums")
+
+
+def test_row_softmax_reference_input_and_edge_rows(hip, oracle, golden):
+    c = golden["row_softmax"]
+    nan, inf = float("nan"), float("inf")
+    edge = [[1.0, nan, 3.0, 2.0], [nan, nan, nan, nan], [0.0, inf, 1.0, inf], [-1000.0] * 4]
+    x = np.array(list(c["input"]) + [v for row in edge for v in row], np.float32)
+    (d_in,) = on_device(hip, x)
+    d_out = hip.DeviceBuffer(x.nbytes)
+    hip.row_softmax_f32_dev(6, 4, d_in, d_out)
+    hip.device_synchronize()
+    got = d_out.to_array(np.float32, 24)
+    assert_close(got, oracle.row_softmax_f32(6, 4, x), F32_REL, F32_ABS, "reference input + edge rows")
+    assert got[12:16].tolist() == [0.0] * 4 and got[16:20].tolist() == [0.0, 1.0, 0.0, 0.0]
+
+
+def test_gelu_backward(hip, oracle, golden):
+    c = golden["gelu_backward"]
+    rng = np.random.default_rng(8)
+    z = np.concatenate([np.array(c["z"], np.float32), (rng.normal(size=100003) * 2).astype(np.float32)])
+    g = np.concatenate([np.array(c["grad"], np.float32), rng.normal(size=100003).astype(np.float32)])
+    d_z, d_g = on_device(hip, z, g)
+    d_out = hip.DeviceBuffer(z.nbytes)
+    hip.gelu_backward_f32_dev(z.size, d_z, d_g, d_out)
+    hip.device_synchronize()
+    assert_close(d_out.to_array(np.float32, z.size), oracle.gelu_backward_f32(z, g), F32_REL, F32_ABS, "gelu_backward")
+
+
+def test_scale_and_add_row(hip, oracle):
+    rng = np.random.default_rng(12)
+    rows, cols = 301, 77
+    x = rng.normal(size=rows * cols).astype(np.float32)
+    bias = rng.normal(size=cols).astype(np.float32)
+    d_x, d_b = on_device(hip, x, bias)
+    d_out = hip.DeviceBuffer(x.nbytes)
+    hip.scale_f32_dev(x.size, d_x, -0.37, d_out)
+    hip.device_synchronize()
+    assert (d_out.to_array(np.float32, x.size) == oracle.scale_f32(x, -0.37)).all()
+    hip.add_row_f32_dev(rows, cols, d_x, d_b)
+    hip.device_synchronize()
+    assert (d_x.to_array(np.float32, x.size) == oracle.add_row_f32(rows, cols, x, bias)).all()
+    with pytest.raises(hip.HipErr, match="scale_factor"):
+        hip.scale_f32_dev(x.size, d_x, float("nan"), d_out)
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 1), (3, 2), (64, 256), (65, 257), (1000, 19), (16384, 512), (100000, 8)])
+def test_sum_axis0(hip, oracle, rows, cols):
+    rng = np.random.default_rng(rows + cols)
+    x = rng.normal(size=rows * cols).astype(np.float32)
+    (d_x,) = on_device(hip, x)
+    d_out = hip.DeviceBuffer(cols * 4)
+    for scale in (1.0, -0.25):
+        hip.sum_axis0_f32_dev(rows, cols, d_x, scale, d_out)
+        hip.device_synchronize()
+        got = d_out.to_array(np.float32, cols)
+        # summation order differs from the oracle's row-by-row order: tolerance relative to sum of magnitudes
+        want = x.astype(np.float64).reshape(rows, cols).sum(axis=0) * scale
+        floor = 1e-6 * float(np.abs(x).reshape(rows, cols).sum(axis=0).max())
+        assert_close(got, want, F32_REL, F32_ABS + floor, f"sum_axis0 {rows}x{cols} scale={scale}")
+        assert_close(oracle.sum_axis0_f32(rows, cols, x, scale), want, F32_REL, F32_ABS + floor, "oracle agrees")
+    again = hip.DeviceBuffer(cols * 4)
+    hip.sum_axis0_f32_dev(rows, cols, d_x, -0.25, again)
+    hip.device_synchronize()
+    assert (again.to_array(np.float32, cols) == got).all(), "column sums must be reproducible"
