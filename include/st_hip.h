@@ -101,6 +101,17 @@ int st_hip_gemm_bias_act_f32(size_t m, size_t n, size_t k, int activation, const
                              size_t bias_len, const float *residual, size_t residual_len,
                              float *out, size_t out_len);
 
+/* out = act((lhs · B + bias) + residual) with B prepacked column-major, i.e. `packed_rhs` is the
+ * n×k row-major transpose that PackedB::from_row_major builds (crates/st-tensor/src/pure.rs:1285-1323).
+ * Replaces Tensor::matmul_prepacked[_bias]_with_backend (pure.rs:2559-2757), the path
+ * crates/st-nn/src/layers/linear.rs:96-104 takes.  bias (length n) and residual (m*n) may be NULL with
+ * length 0; activation may be ST_HIP_ACT_NONE. */
+int st_hip_gemm_prepacked_bias_act_f32(size_t m, size_t n, size_t k, int activation,
+                                       const float *lhs, size_t lhs_len, const float *packed_rhs,
+                                       size_t packed_len, const float *bias, size_t bias_len,
+                                       const float *residual, size_t residual_len, float *out,
+                                       size_t out_len);
+
 /* bf16 operands (raw bit patterns), f32 accumulate and output.  No reference counterpart (the
  * reference lists bf16 as roadmap in docs/backend_matrix.md); same slice contract as gemm_f32. */
 int st_hip_gemm_bf16_f32acc(size_t m, size_t n, size_t k, const uint16_t *lhs, size_t lhs_len,
@@ -138,6 +149,13 @@ int st_hip_gemm_f32_dev(size_t m, size_t n, size_t k, float scale, int lhs_trans
 int st_hip_gemm_bias_act_f32_dev(size_t m, size_t n, size_t k, int activation, const float *lhs,
                                  const float *rhs, const float *bias, const float *residual,
                                  float *out, void *stream);
+/* Device-resident form of st_hip_gemm_prepacked_bias_act_f32, and the packing itself done on the device:
+ * packed(n×k) = rhs(k×n) transposed (PackedB::from_row_major, pure.rs:1299-1316). */
+int st_hip_gemm_prepacked_bias_act_f32_dev(size_t m, size_t n, size_t k, int activation,
+                                           const float *lhs, const float *packed_rhs,
+                                           const float *bias, const float *residual, float *out,
+                                           void *stream);
+int st_hip_pack_rhs_f32_dev(size_t k, size_t n, const float *rhs, float *packed, void *stream);
 int st_hip_gemm_bf16_f32acc_dev(size_t m, size_t n, size_t k, const uint16_t *lhs,
                                 const uint16_t *rhs, float *out, void *stream);
 /* bf16 GEMM with the fused epilogue act((lhs·rhs + bias) + residual); bias/residual may be NULL;

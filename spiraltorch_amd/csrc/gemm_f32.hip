@@ -303,12 +303,14 @@ bool aligned16(const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u
 //
 // A (row-major m×k): stage rows hold 16 k-values (64 B); 16-byte chunk c of row r sits at c ^ ((r >> 2) & 3).
 // A stored k×m (lhs_transposed) and B (k×n): stage rows are k, BM or BN floats long, unpadded.
+// BT: B is given prepacked as n×k (the column-major packing of PackedB, crates/st-tensor/src/pure.rs:1285-1323)
+// and is staged exactly like a row-major A, so its fragments are 128-bit reads too.
 // -------------------------------------------------------------------------------------------------
 typedef __attribute__((address_space(3))) void *lds_void_ptr;
 
 #define ST_F32_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (7 << 4) | (15 << 8) | ((((n) >> 4) & 3) << 14))
 
-template <int BM, int BN, int WM, int WN, bool AT>
+template <int BM, int BN, int WM, int WN, bool AT, bool BT>
 __device__ __forceinline__ void gemm_f32_ring_body(const GemmF32Args &p)
 {
     constexpr int BK = 16, RING = 3;
@@ -367,13 +369,19 @@ __device__ __forceinline__ void gemm_f32_ring_body(const GemmF32Args &p)
         } else {
             const int j = wave + (i - LOADS_A) * WAVES;
             load_lds[i] = A_BYTES + j * 1024;
-            const int f = j * 256 + lane * 4;
-            const int k = f / BN, col = f % BN;
-            load_off[i] = (n0 + col < N) ? (static_cast<unsigned>(k) * N + n0 + col) * 4u : kOutside;
+            if (BT) {  // tile [BN][16 k]: lane lands at row j*16 + lane/4, chunk position lane%4
+                const int row = j * 16 + (lane >> 2);
+                const int chunk = (lane & 3) ^ ((row >> 2) & 3);
+                load_off[i] = (n0 + row < N) ? (static_cast<unsigned>(n0 + row) * K + chunk * 4) * 4u : kOutside;
+            } else {
+                const int f = j * 256 + lane * 4;
+                const int k = f / BN, col = f % BN;
+                load_off[i] = (n0 + col < N) ? (static_cast<unsigned>(k) * N + n0 + col) * 4u : kOutside;
+            }
         }
     }
     const unsigned a_step = AT ? static_cast<unsigned>(BK) * M * 4u : BK * 4u;  // bytes per k-tile
-    const unsigned b_step = static_cast<unsigned>(BK) * N * 4u;
+    const unsigned b_step = BT ? BK * 4u : static_cast<unsigned>(BK) * N * 4u;
 
     auto issue = [&](auto slot_tag, int t) {
         constexpr int SLOT = decltype(slot_tag)::value;
@@ -388,9 +396,9 @@ __device__ __forceinline__ void gemm_f32_ring_body(const GemmF32Args &p)
     };
 
     // Per-lane fragment offsets within a stage.
-    unsigned a_lane[BK / 8][TM], b_lane[TN];
+    unsigned a_lane[BK / 8][TM], b_lane[BK / 8][TN];
 #pragma unroll
-    for (int kk = 0; kk < BK / 8; ++kk)
+    for (int kk = 0; kk < BK / 8; ++kk) {
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm) {
             const int row = wm * WTM + tm * 32 + li;
@@ -398,7 +406,12 @@ __device__ __forceinline__ void gemm_f32_ring_body(const GemmF32Args &p)
                                 : row * 64 + (((kk * 2 + lh) ^ ((row >> 2) & 3)) * 16);
         }
 #pragma unroll
-    for (int tn = 0; tn < TN; ++tn) b_lane[tn] = A_BYTES + (lh * 4 * BN + wn * WTN + tn * 32 + li) * 4;
+        for (int tn = 0; tn < TN; ++tn) {
+            const int col = wn * WTN + tn * 32 + li;
+            b_lane[kk][tn] = A_BYTES + (BT ? col * 64 + (((kk * 2 + lh) ^ ((col >> 2) & 3)) * 16)
+                                           : ((kk * 8 + lh * 4) * BN + col) * 4);
+        }
+    }
 
     f32x16 acc[TM][TN];
 #pragma unroll
@@ -426,10 +439,16 @@ __device__ __forceinline__ void gemm_f32_ring_body(const GemmF32Args &p)
                 }
             }
 #pragma unroll
-            for (int tn = 0; tn < TN; ++tn)
+            for (int tn = 0; tn < TN; ++tn) {
+                if (BT) {
+                    const f32x4 v = *reinterpret_cast<const f32x4 *>(stage + b_lane[kk][tn]);
+                    b[kk][tn][0] = v[0]; b[kk][tn][1] = v[1]; b[kk][tn][2] = v[2]; b[kk][tn][3] = v[3];
+                } else {
 #pragma unroll
-                for (int t = 0; t < 4; ++t)
-                    b[kk][tn][t] = *reinterpret_cast<const float *>(stage + b_lane[tn] + (kk * 8 + t) * BN * 4);
+                    for (int t = 0; t < 4; ++t)
+                        b[kk][tn][t] = *reinterpret_cast<const float *>(stage + b_lane[kk][tn] + t * BN * 4);
+                }
+            }
         }
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_setprio(2);
@@ -503,12 +522,14 @@ __device__ __forceinline__ void gemm_f32_ring_body(const GemmF32Args &p)
 
 // (Plain kernels around the templated body: a kernel template whose body uses the LDS-load builtins loses
 // its host-side launch stub with this compiler.)
-__global__ __launch_bounds__(512) void gemm_f32_ring_128x128_kernel(GemmF32Args p) { gemm_f32_ring_body<128, 128, 4, 2, false>(p); }
-__global__ __launch_bounds__(512) void gemm_f32_ring_128x128_at_kernel(GemmF32Args p) { gemm_f32_ring_body<128, 128, 4, 2, true>(p); }
-__global__ __launch_bounds__(256) void gemm_f32_ring_64x64_kernel(GemmF32Args p) { gemm_f32_ring_body<64, 64, 2, 2, false>(p); }
-__global__ __launch_bounds__(256) void gemm_f32_ring_64x64_at_kernel(GemmF32Args p) { gemm_f32_ring_body<64, 64, 2, 2, true>(p); }
+__global__ __launch_bounds__(512) void gemm_f32_ring_128x128_kernel(GemmF32Args p) { gemm_f32_ring_body<128, 128, 4, 2, false, false>(p); }
+__global__ __launch_bounds__(512) void gemm_f32_ring_128x128_at_kernel(GemmF32Args p) { gemm_f32_ring_body<128, 128, 4, 2, true, false>(p); }
+__global__ __launch_bounds__(512) void gemm_f32_ring_128x128_bt_kernel(GemmF32Args p) { gemm_f32_ring_body<128, 128, 4, 2, false, true>(p); }
+__global__ __launch_bounds__(256) void gemm_f32_ring_64x64_kernel(GemmF32Args p) { gemm_f32_ring_body<64, 64, 2, 2, false, false>(p); }
+__global__ __launch_bounds__(256) void gemm_f32_ring_64x64_at_kernel(GemmF32Args p) { gemm_f32_ring_body<64, 64, 2, 2, true, false>(p); }
+__global__ __launch_bounds__(256) void gemm_f32_ring_64x64_bt_kernel(GemmF32Args p) { gemm_f32_ring_body<64, 64, 2, 2, false, true>(p); }
 
-hipError_t launch_ring(GemmF32Args args, bool lhs_transposed, bool big, hipStream_t stream)
+hipError_t launch_ring(GemmF32Args args, bool lhs_transposed, bool rhs_packed, bool big, hipStream_t stream)
 {
     const int bm = big ? 128 : 64, bn = big ? 128 : 64;
     args.tiles_n = (args.N + bn - 1) / bn;
@@ -516,13 +537,35 @@ hipError_t launch_ring(GemmF32Args args, bool lhs_transposed, bool big, hipStrea
     const size_t tiles = static_cast<size_t>(args.tiles_n) * static_cast<size_t>(args.tiles_m);
     if (tiles > 0x7fffffffu) return hipErrorInvalidConfiguration;
     const size_t lds_bytes = 3 * static_cast<size_t>(bm + bn) * 16 * 4;
-    auto kernel = big ? (lhs_transposed ? gemm_f32_ring_128x128_at_kernel : gemm_f32_ring_128x128_kernel)
-                      : (lhs_transposed ? gemm_f32_ring_64x64_at_kernel : gemm_f32_ring_64x64_kernel);
+    auto kernel = big ? (rhs_packed ? gemm_f32_ring_128x128_bt_kernel
+                                    : lhs_transposed ? gemm_f32_ring_128x128_at_kernel : gemm_f32_ring_128x128_kernel)
+                      : (rhs_packed ? gemm_f32_ring_64x64_bt_kernel
+                                    : lhs_transposed ? gemm_f32_ring_64x64_at_kernel : gemm_f32_ring_64x64_kernel);
     hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                         static_cast<int>(lds_bytes));
     if (rc != hipSuccess) return rc;
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(tiles)), dim3(big ? 512 : 256), lds_bytes, stream, args);
     return hipGetLastError();
+}
+
+
+// out(cols×rows) = in(rows×cols)ᵀ through a 32×33 LDS tile (PackedB::from_row_major, pure.rs:1299-1316, and back).
+__global__ __launch_bounds__(256) void transpose_f32_kernel(int rows, int cols, const float *in, float *out)
+{
+    __shared__ float tile[32][33];
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 × 8
+    const int c0 = blockIdx.x * 32, r0 = blockIdx.y * 32;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int r = r0 + ty + 8 * i, c = c0 + tx;
+        if (r < rows && c < cols) tile[ty + 8 * i][tx] = in[static_cast<size_t>(r) * cols + c];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int c = c0 + ty + 8 * i, r = r0 + tx;
+        if (r < rows && c < cols) out[static_cast<size_t>(c) * rows + r] = tile[tx][ty + 8 * i];
+    }
 }
 
 }  // namespace
@@ -558,9 +601,49 @@ hipError_t launch_gemm_f32(size_t m, size_t n, size_t k, bool lhs_transposed, co
         // rounds; 64×64 tiles otherwise, which spread small problems and leave a shorter tail.
         const size_t tiles128 = ((m + 127) / 128) * ((n + 127) / 128);
         const bool big = tiles128 >= 512 && (tiles128 >= 3072 || tiles128 % 768 == 0 || tiles128 % 768 >= 384);
-        return launch_ring(args, lhs_transposed, big, stream);
+        return launch_ring(args, lhs_transposed, false, big, stream);
     }
     return launch_tile<64, 64, 2, 2>(args, lhs_transposed, vec, stream);
+}
+
+hipError_t launch_transpose_f32(size_t rows, size_t cols, const float *in, float *out, hipStream_t stream)
+{
+    if (rows == 0 || cols == 0) return hipSuccess;
+    const dim3 grid(static_cast<unsigned>((cols + 31) / 32), static_cast<unsigned>((rows + 31) / 32));
+    hipLaunchKernelGGL(transpose_f32_kernel, grid, dim3(256), 0, stream, static_cast<int>(rows), static_cast<int>(cols), in,
+                       out);
+    return hipGetLastError();
+}
+
+hipError_t launch_gemm_f32_packed(size_t m, size_t n, size_t k, const float *lhs, const float *packed_rhs, float *out,
+                                  const GemmEpilogue &epilogue, hipStream_t stream)
+{
+    if (m == 0 || n == 0) return hipSuccess;
+    const bool ring_ok = k >= 16 && k % 16 == 0 && aligned16(lhs) && aligned16(packed_rhs) && m * k * 4 < (1ull << 31) &&
+                         k * n * 4 < (1ull << 31);
+    if (!ring_ok) {
+        // Ragged k: unpack into the stream's workspace and take the general path.
+        void *workspace = nullptr;
+        hipError_t rc = stream_workspace(stream, k * n * sizeof(float), &workspace);
+        if (rc != hipSuccess) return rc;
+        rc = launch_transpose_f32(n, k, packed_rhs, static_cast<float *>(workspace), stream);
+        if (rc != hipSuccess) return rc;
+        return launch_gemm_f32(m, n, k, false, lhs, static_cast<const float *>(workspace), out, epilogue, stream);
+    }
+    GemmF32Args args;
+    args.A = lhs;
+    args.B = packed_rhs;
+    args.C = out;
+    args.bias = epilogue.bias;
+    args.residual = epilogue.residual;
+    args.M = static_cast<int>(m);
+    args.N = static_cast<int>(n);
+    args.K = static_cast<int>(k);
+    args.scale = epilogue.scale;
+    args.activation = epilogue.activation;
+    const size_t tiles128 = ((m + 127) / 128) * ((n + 127) / 128);
+    const bool big = tiles128 >= 512 && (tiles128 >= 3072 || tiles128 % 768 == 0 || tiles128 % 768 >= 384);
+    return launch_ring(args, false, true, big, stream);
 }
 
 }  // namespace sthip

@@ -340,6 +340,41 @@ int st_hip_gemm_bias_act_f32(size_t m, size_t n, size_t k, int activation, const
     return lease.download(out, d_out, out_len * sizeof(float));
 }
 
+int st_hip_gemm_prepacked_bias_act_f32(size_t m, size_t n, size_t k, int activation, const float *lhs, size_t lhs_len,
+                                       const float *packed_rhs, size_t packed_len, const float *bias, size_t bias_len,
+                                       const float *residual, size_t residual_len, float *out, size_t out_len)
+{
+    ST_HIP_CHECK(ensure_init());
+    ST_HIP_CHECK(validate_gemm_dimensions(m, n, k, lhs_len, packed_len, out_len));
+    if (bias != nullptr || bias_len != 0) ST_HIP_CHECK(validate_gemm_epilogue(m, n, bias_len, false, 0));
+    if (residual != nullptr) ST_HIP_CHECK(validate_gemm_epilogue(m, n, n, true, residual_len));
+    ST_HIP_CHECK(validate_activation(activation, true));
+    ST_HIP_CHECK(reject_null(lhs, lhs_len, "gemm"));
+    ST_HIP_CHECK(reject_null(packed_rhs, packed_len, "gemm"));
+    ST_HIP_CHECK(reject_null(bias, bias_len, "gemm"));
+    ST_HIP_CHECK(reject_null(out, out_len, "gemm"));
+    if (out_len == 0) return ST_HIP_OK;
+    ST_HIP_CHECK(validate_kernel_dims(m, n, k));
+
+    Lease lease;
+    ST_HIP_CHECK(lease.status());
+    void *d_lhs, *d_rhs, *d_out, *d_bias = nullptr, *d_residual = nullptr;
+    ST_HIP_CHECK(lease.upload(0, lhs, lhs_len * sizeof(float), &d_lhs));
+    ST_HIP_CHECK(lease.upload(1, packed_rhs, packed_len * sizeof(float), &d_rhs));
+    ST_HIP_CHECK(lease.buffer(2, out_len * sizeof(float), &d_out));
+    if (bias) ST_HIP_CHECK(lease.upload(3, bias, bias_len * sizeof(float), &d_bias));
+    if (residual) ST_HIP_CHECK(lease.upload(4, residual, residual_len * sizeof(float), &d_residual));
+    GemmEpilogue epilogue;
+    epilogue.bias = static_cast<const float *>(d_bias);
+    epilogue.residual = static_cast<const float *>(d_residual);
+    epilogue.activation = activation;
+    ST_HIP_CHECK(launch_status(launch_gemm_f32_packed(m, n, k, static_cast<const float *>(d_lhs),
+                                                      static_cast<const float *>(d_rhs), static_cast<float *>(d_out),
+                                                      epilogue, lease.stream()),
+                               "gemm_prepacked launch"));
+    return lease.download(out, d_out, out_len * sizeof(float));
+}
+
 int st_hip_gemm_bf16_f32acc(size_t m, size_t n, size_t k, const uint16_t *lhs, size_t lhs_len,
                             const uint16_t *rhs, size_t rhs_len, float *out, size_t out_len)
 {
@@ -527,6 +562,33 @@ int st_hip_gemm_bias_act_f32_dev(size_t m, size_t n, size_t k, int activation, c
     epilogue.activation = activation;
     return launch_status(launch_gemm_f32(m, n, k, false, lhs, rhs, out, epilogue, as_stream(stream)),
                          "gemm_bias_act_f32 launch");
+}
+
+int st_hip_gemm_prepacked_bias_act_f32_dev(size_t m, size_t n, size_t k, int activation, const float *lhs,
+                                           const float *packed_rhs, const float *bias, const float *residual, float *out,
+                                           void *stream)
+{
+    ST_HIP_CHECK(ensure_init());
+    ST_HIP_CHECK(validate_activation(activation, true));
+    ST_HIP_CHECK(validate_kernel_dims(m, n, k));
+    if (m == 0 || n == 0) return ST_HIP_OK;
+    if (!out || (k != 0 && (!lhs || !packed_rhs)))
+        return fail(ST_HIP_ERR_INVALID, "gemm received a null pointer; provide contiguous row-major buffers");
+    GemmEpilogue epilogue;
+    epilogue.bias = bias;
+    epilogue.residual = residual;
+    epilogue.activation = activation;
+    return launch_status(launch_gemm_f32_packed(m, n, k, lhs, packed_rhs, out, epilogue, as_stream(stream)),
+                         "gemm_prepacked launch");
+}
+
+int st_hip_pack_rhs_f32_dev(size_t k, size_t n, const float *rhs, float *packed, void *stream)
+{
+    ST_HIP_CHECK(ensure_init());
+    ST_HIP_CHECK(validate_kernel_dims(1, n, k));
+    if (k == 0 || n == 0) return ST_HIP_OK;
+    if (!rhs || !packed) return fail(ST_HIP_ERR_INVALID, "pack_rhs received a null pointer");
+    return launch_status(launch_transpose_f32(k, n, rhs, packed, as_stream(stream)), "pack_rhs launch");
 }
 
 int st_hip_gemm_bf16_f32acc_dev(size_t m, size_t n, size_t k, const uint16_t *lhs, const uint16_t *rhs, float *out,

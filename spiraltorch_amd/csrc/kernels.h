@@ -19,6 +19,12 @@ hipError_t launch_gemm_f32(size_t m, size_t n, size_t k, bool lhs_transposed, co
                            const float *rhs, float *out, const GemmEpilogue &epilogue,
                            hipStream_t stream);
 
+// Same with B prepacked as n×k (column-major packing, crates/st-tensor/src/pure.rs:1285-1323).
+hipError_t launch_gemm_f32_packed(size_t m, size_t n, size_t k, const float *lhs, const float *packed_rhs,
+                                  float *out, const GemmEpilogue &epilogue, hipStream_t stream);
+// out(cols×rows) = in(rows×cols) transposed.
+hipError_t launch_transpose_f32(size_t rows, size_t cols, const float *in, float *out, hipStream_t stream);
+
 // bf16 operands, f32 accumulation; writes out_f32 and/or out_bf16 (either may be null).
 hipError_t launch_gemm_bf16(size_t m, size_t n, size_t k, const uint16_t *lhs, const uint16_t *rhs,
                             float *out_f32, uint16_t *out_bf16, const GemmEpilogue &epilogue,

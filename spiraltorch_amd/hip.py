@@ -137,6 +137,18 @@ def gemm_bias_activation_f32(m: int, n: int, k: int, activation: GemmActivation,
         _ptr(res), 0 if res is None else res.size, _ptr(out), out.size))
 
 
+def gemm_prepacked_bias_activation_f32(m: int, n: int, k: int, activation, lhs, packed_rhs, bias, residual,
+                                       out) -> None:
+    """out = act((lhs @ B + bias) + residual) with B given prepacked as its (n, k) transpose — the PackedB path
+    of pure.rs:2559-2757; `bias` and `residual` may be None, `activation` may be 0."""
+    lhs, packed, out = _f32(lhs, "lhs"), _f32(packed_rhs, "packed_rhs"), _out(out, "out")
+    b = None if bias is None else _f32(bias, "bias")
+    res = None if residual is None else _f32(residual, "residual")
+    _check(_lib.load().st_hip_gemm_prepacked_bias_act_f32(
+        m, n, k, int(activation), _ptr(lhs), lhs.size, _ptr(packed), packed.size, _ptr(b),
+        0 if b is None else b.size, _ptr(res), 0 if res is None else res.size, _ptr(out), out.size))
+
+
 def gemm_bf16_f32acc(m: int, n: int, k: int, lhs_bf16, rhs_bf16, out) -> None:
     lhs, rhs, out = _u16(lhs_bf16, "lhs"), _u16(rhs_bf16, "rhs"), _out(out, "out")
     _check(_lib.load().st_hip_gemm_bf16_f32acc(m, n, k, _ptr(lhs), lhs.size, _ptr(rhs), rhs.size, _ptr(out),
@@ -290,6 +302,17 @@ def gemm_f32_dev(m, n, k, scale, lhs_transposed, lhs, rhs, out, stream=None) -> 
 def gemm_bias_act_f32_dev(m, n, k, activation, lhs, rhs, bias, residual, out, stream=None) -> None:
     _check(_lib.load().st_hip_gemm_bias_act_f32_dev(m, n, k, int(activation), _dev(lhs), _dev(rhs), _dev(bias),
                                                     _dev(residual), _dev(out), _stream_ptr(stream)))
+
+
+def gemm_prepacked_bias_act_f32_dev(m, n, k, activation, lhs, packed_rhs, bias, residual, out, stream=None) -> None:
+    _check(_lib.load().st_hip_gemm_prepacked_bias_act_f32_dev(m, n, k, int(activation), _dev(lhs), _dev(packed_rhs),
+                                                              _dev(bias), _dev(residual), _dev(out),
+                                                              _stream_ptr(stream)))
+
+
+def pack_rhs_f32_dev(k, n, rhs, packed, stream=None) -> None:
+    """packed (n, k) = rhs (k, n) transposed, on the device."""
+    _check(_lib.load().st_hip_pack_rhs_f32_dev(k, n, _dev(rhs), _dev(packed), _stream_ptr(stream)))
 
 
 def gemm_bf16_f32acc_dev(m, n, k, lhs, rhs, out, stream=None) -> None:

@@ -52,6 +52,28 @@ def _validate_finite(label: str, data: np.ndarray) -> None:
         raise TensorError("NonFiniteValue", f"non-finite value encountered in {label}: {bad}", label=label)
 
 
+class PackedB:
+    """Right-hand operand packed once for repeated matmuls (pure.rs:1285-1400): column-major, i.e. the (cols, inner)
+    row-major transpose of the (inner, cols) matrix."""
+
+    def __init__(self, inner: int, cols: int, buf: np.ndarray):
+        self._inner, self._cols, self._buf = int(inner), int(cols), buf
+
+    @classmethod
+    def from_tensor(cls, tensor: "Tensor") -> "PackedB":
+        """PackedB::from_row_major, pure.rs:1299-1316: packed[c*rows + r] = data[r*cols + c]."""
+        return cls(tensor.rows, tensor.cols, np.ascontiguousarray(tensor.numpy().T).reshape(-1))
+
+    def inner(self) -> int:
+        return self._inner
+
+    def cols(self) -> int:
+        return self._cols
+
+    def as_slice(self) -> np.ndarray:
+        return self._buf
+
+
 class Tensor:
     """2-D row-major float32 matrix held on the host (pure.rs:1406-1411)."""
 
@@ -161,6 +183,33 @@ class Tensor:
                              backend: Optional[str] = None) -> "Tensor":
         _resolve_backend(backend)
         return self._fused(other, bias, residual, hip.GemmActivation.Gelu, "matmul_bias_add_gelu_output")
+
+    def matmul_prepacked(self, packed: "PackedB", *, backend: Optional[str] = None) -> "Tensor":
+        """C = A·B with B prepacked — pure.rs:2559-2575."""
+        return self._prepacked(packed, None, "matmul_prepacked_output", backend)
+
+    def matmul_prepacked_bias(self, packed: "PackedB", bias, *, backend: Optional[str] = None) -> "Tensor":
+        """C = A·B + bias with B prepacked — pure.rs:2577-2757 (what Linear::forward calls, linear.rs:96-104)."""
+        bias = np.ascontiguousarray(np.asarray(bias, dtype=np.float32)).reshape(-1)
+        if self.cols == packed.inner() and bias.size != packed.cols():
+            raise TensorError("DataLength", f"expected {packed.cols()} values, got {bias.size}",
+                              expected=packed.cols(), got=bias.size)
+        _validate_finite("matmul_prepacked_bias_bias", bias)
+        return self._prepacked(packed, bias, "matmul_prepacked_bias_output", backend)
+
+    def _prepacked(self, packed: "PackedB", bias, label: str, backend: Optional[str]) -> "Tensor":
+        _resolve_backend(backend)
+        if self.cols != packed.inner():
+            raise TensorError("ShapeMismatch", f"left {self.shape()} right {(packed.inner(), packed.cols())}",
+                              left=self.shape(), right=(packed.inner(), packed.cols()))
+        out = Tensor.zeros(self.rows, packed.cols())
+        try:
+            hip.gemm_prepacked_bias_activation_f32(self.rows, packed.cols(), self.cols, 0, self._data,
+                                                   packed.as_slice(), bias, None, out._data)
+        except hip.HipErr as err:
+            raise _backend_failure(err) from err
+        _validate_finite(label, out._data)
+        return out
 
     # ---- attention -------------------------------------------------------------------------------
     def scaled_dot_attention(self, keys: "Tensor", values: "Tensor", *, contexts: int, sequence: int,

@@ -158,6 +158,33 @@ def test_ring_kernel_128_tiles_ragged_edges(hip, oracle):
     assert_close(out, np.maximum(pre, 0), F32_REL, F32_ABS, "bias+residual+relu")
 
 
+@pytest.mark.parametrize("m,n,k", [(2, 2, 3), (33, 65, 17), (64, 64, 64), (132, 136, 48), (1000, 260, 32),
+                                   (16384, 512, 64), (3000, 2820, 16)])
+def test_prepacked_rhs(hip, oracle, m, n, k):
+    """B prepacked as its (n, k) transpose (PackedB): same results as the row-major GEMM, with and without
+    bias / residual / GELU; ragged k takes the unpack-to-workspace path."""
+    rng = np.random.default_rng(m + 3 * n + 7 * k)
+    a = rng.uniform(-1, 1, m * k).astype(np.float32)
+    b = rng.uniform(-1, 1, k * n).astype(np.float32)
+    packed = np.ascontiguousarray(b.reshape(k, n).T).ravel()
+    bias = rng.uniform(-1, 1, n).astype(np.float32)
+    res = rng.uniform(-1, 1, m * n).astype(np.float32)
+    out = np.zeros(m * n, np.float32)
+    plain = oracle.gemm_f32(m, n, k, a, b, threads=8)
+    hip.gemm_prepacked_bias_activation_f32(m, n, k, 0, a, packed, None, None, out)
+    assert_close(out, plain, F32_REL, F32_ABS, "prepacked")
+    hip.gemm_prepacked_bias_activation_f32(m, n, k, 0, a, packed, bias, None, out)
+    assert_close(out, (plain.astype(np.float64).reshape(m, n) + bias).ravel(), F32_REL, F32_ABS, "prepacked + bias")
+    hip.gemm_prepacked_bias_activation_f32(m, n, k, hip.GemmActivation.Gelu, a, packed, bias, res, out)
+    want = oracle.gemm_bias_act_f32(m, n, k, oracle.ACT_GELU, a, b, bias, res, threads=8)
+    assert_close(out, want, F32_REL, F32_ABS, "prepacked + bias + residual + gelu")
+    # packing on the device gives the same matrix
+    d_b, d_p = hip.DeviceBuffer.from_array(b), hip.DeviceBuffer(b.nbytes)
+    hip.pack_rhs_f32_dev(k, n, d_b, d_p)
+    hip.device_synchronize()
+    assert (d_p.to_array(np.float32, k * n) == packed).all()
+
+
 def test_tensor_mirror_matches_the_reference_api(hip, oracle):
     from spiraltorch_amd import Tensor, TensorError
     a = Tensor(2, 3, [1, 2, 3, 4, 5, 6])
@@ -165,6 +192,14 @@ def test_tensor_mirror_matches_the_reference_api(hip, oracle):
     assert a.matmul(b, backend="hip").data().tolist() == [58, 64, 139, 154]
     assert a.matmul(b).shape() == (2, 2)
     assert a.matmul_scaled(b, 0.5, backend="hip").data().tolist() == [29, 32, 69.5, 77]
+    from spiraltorch_amd import PackedB
+    packed = PackedB.from_tensor(b)
+    assert packed.as_slice().tolist() == [7, 9, 11, 8, 10, 12] and (packed.inner(), packed.cols()) == (3, 2)
+    assert a.matmul_prepacked(packed, backend="hip").data().tolist() == [58, 64, 139, 154]
+    assert a.matmul_prepacked_bias(packed, [1, -1]).data().tolist() == [59, 63, 140, 153]
+    with pytest.raises(TensorError) as bad:
+        a.matmul_prepacked_bias(packed, [1, 2, 3])
+    assert bad.value.kind == "DataLength"
     at = Tensor(3, 2, [1, 4, 2, 5, 3, 6])
     assert at.matmul_lhs_transpose_scaled(b, 1.0, backend="hip").data().tolist() == [58, 64, 139, 154]
     assert a.matmul_bias_relu(b, [-60, 1], backend="hip").data().tolist() == [0, 65, 79, 155]
