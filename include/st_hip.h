@@ -130,6 +130,20 @@ int st_hip_conv2d_bias_act_f32(size_t batch, size_t c_in, size_t h, size_t w, si
                                size_t weight_len, const float *bias, size_t bias_len, float *out,
                                size_t out_len);
 
+/* Conv2d::backward, crates/st-nn/src/layers/conv.rs:780-813 with col2im :860-916: from the forward input
+ * (N, C_in, H, W), the OIHW weight and grad_output (N, C_out, OH, OW) computes
+ *   grad_input  (N, C_in, H, W)       = col2im(G · W)
+ *   grad_weight (C_out, C_in·KH·KW)   = (Gᵀ · patches) / batch
+ *   grad_bias   (C_out)               = column sums of G / batch
+ * where G is grad_output viewed per pixel.  An empty batch is a no-op (:787-789).  Needs c_out·kh·kw <= 8192. */
+int st_hip_conv2d_backward_f32(size_t batch, size_t c_in, size_t h, size_t w, size_t c_out, size_t kh,
+                               size_t kw, size_t stride_h, size_t stride_w, size_t pad_h, size_t pad_w,
+                               size_t dil_h, size_t dil_w, const float *input, size_t input_len,
+                               const float *weight, size_t weight_len, const float *grad_output,
+                               size_t grad_output_len, float *grad_input, size_t grad_input_len,
+                               float *grad_weight, size_t grad_weight_len, float *grad_bias,
+                               size_t grad_bias_len);
+
 /* Tensor::scaled_dot_attention_with_backend — crates/st-tensor/src/pure.rs:4083-4354 with the CPU
  * kernel of :11845-11919.  q,k,v,out are (contexts·sequence, head_dim); z_bias (contexts, sequence)
  * or NULL; attn_bias (contexts·sequence, sequence) or NULL.  `causal` != 0 limits query i to keys
@@ -169,6 +183,23 @@ int st_hip_conv2d_bias_act_f32_dev(size_t batch, size_t c_in, size_t h, size_t w
                                    size_t pad_h, size_t pad_w, size_t dil_h, size_t dil_w,
                                    int activation, const float *input, const float *weight,
                                    const float *bias, float *out, void *stream);
+/* The three gradients of Conv2d::backward one by one (conv.rs:791-809); grad_weight and grad_bias are
+ * multiplied by `scale` (the reference passes 1/batch). */
+int st_hip_conv2d_grad_input_f32_dev(size_t batch, size_t c_in, size_t h, size_t w, size_t c_out,
+                                     size_t kh, size_t kw, size_t stride_h, size_t stride_w,
+                                     size_t pad_h, size_t pad_w, size_t dil_h, size_t dil_w,
+                                     const float *grad_output, const float *weight,
+                                     float *grad_input, void *stream);
+int st_hip_conv2d_grad_weight_f32_dev(size_t batch, size_t c_in, size_t h, size_t w, size_t c_out,
+                                      size_t kh, size_t kw, size_t stride_h, size_t stride_w,
+                                      size_t pad_h, size_t pad_w, size_t dil_h, size_t dil_w,
+                                      const float *input, const float *grad_output, float scale,
+                                      float *grad_weight, void *stream);
+int st_hip_conv2d_grad_bias_f32_dev(size_t batch, size_t c_in, size_t h, size_t w, size_t c_out,
+                                    size_t kh, size_t kw, size_t stride_h, size_t stride_w,
+                                    size_t pad_h, size_t pad_w, size_t dil_h, size_t dil_w,
+                                    const float *grad_output, float scale, float *grad_bias,
+                                    void *stream);
 int st_hip_attention_f32_dev(size_t contexts, size_t sequence, size_t head_dim, float scale,
                              int causal, const float *q, const float *k, const float *v,
                              const float *z_bias, const float *attn_bias, float *out, void *stream);

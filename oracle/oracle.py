@@ -58,6 +58,7 @@ def load() -> ctypes.CDLL:
     lib.st_oracle_gemm_bf16_f32acc.argtypes = [S, S, S, P, P, P, I]
     lib.st_oracle_conv2d_output_hw.argtypes = [S] * 10 + [POINTER(S), POINTER(S)]
     lib.st_oracle_conv2d_bias_act_f32.argtypes = [S] * 13 + [I, P, P, P, P, I]
+    lib.st_oracle_conv2d_backward_f32.argtypes = [S] * 13 + [P, P, P, F, P, P, P]
     lib.st_oracle_attention_f32.argtypes = [S, S, S, F, I, P, P, P, P, P, P, I]
     lib.st_oracle_attention_f64.argtypes = [S, S, S, c_double, I, P, P, P, P, P, P]
     lib.st_oracle_layer_norm_f32.argtypes = [S, S, P, P, P, P, F, P]
@@ -139,6 +140,20 @@ def conv2d_bias_act_f32(batch, c_in, h, w, c_out, kernel, stride, padding, dilat
                                                 padding[0], padding[1], dilation[0], dilation[1], activation, _p(x),
                                                 _p(weight), _p(bias), _p(out), threads))
     return out
+
+
+def conv2d_backward_f32(batch, c_in, h, w, c_out, kernel, stride, padding, dilation, input, weight, grad_output,
+                        weight_scale=None):
+    """Returns (grad_input, grad_weight, grad_bias); weight_scale defaults to the reference's 1/batch."""
+    x, wgt, g = _f32(input), _f32(weight), _f32(grad_output)
+    scale = (1.0 / batch if batch else 1.0) if weight_scale is None else weight_scale
+    grad_input = np.zeros(batch * c_in * h * w, dtype=np.float32)
+    grad_weight = np.zeros(c_out * c_in * kernel[0] * kernel[1], dtype=np.float32)
+    grad_bias = np.zeros(c_out, dtype=np.float32)
+    _check(load().st_oracle_conv2d_backward_f32(batch, c_in, h, w, c_out, kernel[0], kernel[1], stride[0], stride[1],
+                                                padding[0], padding[1], dilation[0], dilation[1], _p(x), _p(wgt),
+                                                _p(g), scale, _p(grad_input), _p(grad_weight), _p(grad_bias)))
+    return grad_input, grad_weight, grad_bias
 
 
 def attention_f32(contexts, sequence, head_dim, scale, q, k, v, z_bias=None, attn_bias=None, causal=False,

@@ -254,6 +254,89 @@ int st_oracle_conv2d_bias_act_f32(size_t batch, size_t c_in, size_t h, size_t w,
     return ST_ORACLE_OK;
 }
 
+/* Conv2d backward, crates/st-nn/src/layers/conv.rs:750-813 and :860-916:
+ *   G (batch·OH·OW, C_out) is grad_output re-laid per pixel (:750-778);
+ *   grad_weight = (Gᵀ · patches) · weight_scale  — matmul_lhs_transpose_scaled (:791-795), k = pixel index ascending;
+ *   grad_bias   = (column sums of G) · weight_scale (:796-799);
+ *   grad_input  = col2im(G · W): grad_patches[p][s] = Σ_o G[p][o]·W[o][s] (o ascending), scattered with += in the
+ *   loop order of col2im (:880-912).  The reference passes weight_scale = 1/batch.  Any output may be NULL. */
+int st_oracle_conv2d_backward_f32(size_t batch, size_t c_in, size_t h, size_t w, size_t c_out,
+                                  size_t kh, size_t kw, size_t stride_h, size_t stride_w,
+                                  size_t pad_h, size_t pad_w, size_t dil_h, size_t dil_w,
+                                  const float *input, const float *weight, const float *grad_output,
+                                  float weight_scale, float *grad_input, float *grad_weight, float *grad_bias)
+{
+    size_t oh, ow;
+    if (c_in == 0 || c_out == 0) return ST_ORACLE_BAD_ARGUMENT;
+    int rc = st_oracle_conv2d_output_hw(h, w, kh, kw, stride_h, stride_w, pad_h, pad_w, dil_h, dil_w, &oh, &ow);
+    if (rc != ST_ORACLE_OK) return rc;
+    const size_t span = c_in * kh * kw, spatial = oh * ow;
+    if (grad_input) memset(grad_input, 0, batch * c_in * h * w * sizeof(float));
+    if (grad_weight) memset(grad_weight, 0, c_out * span * sizeof(float));
+    if (grad_bias) memset(grad_bias, 0, c_out * sizeof(float));
+    float *patch = (float *)malloc((span ? span : 1) * sizeof(float));
+    float *grad_patch = (float *)malloc((span ? span : 1) * sizeof(float));
+    if (!patch || !grad_patch) { free(patch); free(grad_patch); return ST_ORACLE_BAD_ARGUMENT; }
+    for (size_t b = 0; b < batch; ++b)
+        for (size_t oy = 0; oy < oh; ++oy)
+            for (size_t ox = 0; ox < ow; ++ox) {
+                const size_t sp = oy * ow + ox;
+                const float *g = grad_output + b * c_out * spatial + sp;  /* G[p][o] = g[o*spatial] */
+                if (grad_weight && input) {
+                    size_t s = 0;
+                    const float *image = input + b * c_in * h * w;
+                    for (size_t ic = 0; ic < c_in; ++ic)
+                        for (size_t ky = 0; ky < kh; ++ky)
+                            for (size_t kx = 0; kx < kw; ++kx, ++s) {
+                                const long long iy = (long long)(oy * stride_h + ky * dil_h) - (long long)pad_h;
+                                const long long ix = (long long)(ox * stride_w + kx * dil_w) - (long long)pad_w;
+                                patch[s] = (iy < 0 || ix < 0 || iy >= (long long)h || ix >= (long long)w)
+                                               ? 0.0f
+                                               : image[ic * h * w + (size_t)iy * w + (size_t)ix];
+                            }
+                    for (size_t o = 0; o < c_out; ++o) {
+                        const float go = g[o * spatial];
+                        float *row = grad_weight + o * span;
+                        for (s = 0; s < span; ++s) {
+                            const float prod = go * patch[s];
+                            row[s] = row[s] + prod;
+                        }
+                    }
+                }
+                if (grad_bias)
+                    for (size_t o = 0; o < c_out; ++o) grad_bias[o] = grad_bias[o] + g[o * spatial];
+                if (grad_input) {
+                    for (size_t s = 0; s < span; ++s) grad_patch[s] = 0.0f;
+                    for (size_t o = 0; o < c_out; ++o) {
+                        const float go = g[o * spatial];
+                        const float *wrow = weight + o * span;
+                        for (size_t s = 0; s < span; ++s) {
+                            const float prod = go * wrow[s];
+                            grad_patch[s] = grad_patch[s] + prod;
+                        }
+                    }
+                    float *gin = grad_input + b * c_in * h * w;
+                    size_t s = 0;
+                    for (size_t ic = 0; ic < c_in; ++ic)
+                        for (size_t ky = 0; ky < kh; ++ky)
+                            for (size_t kx = 0; kx < kw; ++kx, ++s) {
+                                const long long iy = (long long)(oy * stride_h + ky * dil_h) - (long long)pad_h;
+                                const long long ix = (long long)(ox * stride_w + kx * dil_w) - (long long)pad_w;
+                                if (iy < 0 || ix < 0 || iy >= (long long)h || ix >= (long long)w) continue;
+                                float *dst = gin + ic * h * w + (size_t)iy * w + (size_t)ix;
+                                *dst = *dst + grad_patch[s];
+                            }
+                }
+            }
+    if (grad_weight)
+        for (size_t i = 0; i < c_out * span; ++i) grad_weight[i] = grad_weight[i] * weight_scale;
+    if (grad_bias)
+        for (size_t o = 0; o < c_out; ++o) grad_bias[o] = grad_bias[o] * weight_scale;
+    free(patch);
+    free(grad_patch);
+    return ST_ORACLE_OK;
+}
+
 /* ------------------------------------------------------------------------------------------------
  * Attention.  crates/st-tensor/src/pure.rs:11845-11919 (fused_attention_cpu): normalised online
  * softmax, one key at a time, a finite check after every scalar step.  `causal` restricts the key

@@ -65,6 +65,16 @@ int st_oracle_conv2d_bias_act_f32(size_t batch, size_t c_in, size_t h, size_t w,
                                   int activation, const float *input, const float *weight,
                                   const float *bias, float *out, int threads);
 
+/* Conv2d backward (crates/st-nn/src/layers/conv.rs:750-813, 860-916): grad_input (N, C_in, H, W),
+ * grad_weight (C_out, C_in·KH·KW) and grad_bias (C_out), the latter two multiplied by weight_scale
+ * (the reference passes 1/batch).  Outputs may be NULL; `input` is only needed for grad_weight. */
+int st_oracle_conv2d_backward_f32(size_t batch, size_t c_in, size_t h, size_t w, size_t c_out,
+                                  size_t kh, size_t kw, size_t stride_h, size_t stride_w,
+                                  size_t pad_h, size_t pad_w, size_t dil_h, size_t dil_w,
+                                  const float *input, const float *weight, const float *grad_output,
+                                  float weight_scale, float *grad_input, float *grad_weight,
+                                  float *grad_bias);
+
 /* q,k,v,out: (contexts·sequence, head_dim); z_bias (contexts, sequence) or NULL; attn_bias
  * (contexts·sequence, sequence) or NULL; causal != 0 restricts query i to keys 0..=i. */
 int st_oracle_attention_f32(size_t contexts, size_t sequence, size_t head_dim, float scale,

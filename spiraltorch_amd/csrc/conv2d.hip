@@ -41,7 +41,13 @@ struct ConvArgs {
 // FULLK: c_in*kh*kw is a multiple of the 16-wide k-tile and weight rows are 16-byte aligned, so the loop
 // carries no k bounds checks; weight rows past c_out are clamped to the last row (what they contribute
 // only reaches output channels that are never stored).
-template <int BM, int BN, int BK, int WM, int WN, bool VEC, bool FULLK>
+//
+// TRANSPOSED turns the gather into that of the convolution's adjoint (gradient with respect to the input, the
+// col2im of crates/st-nn/src/layers/conv.rs:860-916 written as a gather): the "image" is grad_output with
+// s.c_in = C_out channels of s.h × s.w = OH × OW values, the output pixels (s.oh × s.ow = H × W) are input
+// positions, and tap (ky, kx) of output pixel (y, x) reads grad_output at ((y + pad - ky·dil) / stride, ...) when
+// that division is exact and in range.  The weight matrix is then W[ic][(oc, ky, kx)].
+template <int BM, int BN, int BK, int WM, int WN, bool VEC, bool FULLK, bool TRANSPOSED>
 __global__ __launch_bounds__(64 * WM * WN) void conv2d_f32_kernel(ConvArgs p)
 {
     // WM×WN wavefronts, each owning (BM/WM) output channels × (BN/WN) pixels.  As in the f32 GEMM, many
@@ -89,7 +95,7 @@ __global__ __launch_bounds__(64 * WM * WN) void conv2d_f32_kernel(ConvArgs p)
         const int ic = k / khw, rem = k - ic * khw;
         const int ky = rem / s.kw, kx = rem - ky * s.kw;
         const int dy = ky * s.dil_h, dx = kx * s.dil_w;
-        lut[k] = make_int2(ic * H * W + dy * W + dx, dy | (dx << 16));
+        lut[k] = make_int2(TRANSPOSED ? ic * H * W : ic * H * W + dy * W + dx, dy | (dx << 16));
     }
 
     // Every thread gathers one pixel column of the patch tile, rows (tid / BN) + B_ROW_STEP * r.
@@ -98,8 +104,8 @@ __global__ __launch_bounds__(64 * WM * WN) void conv2d_f32_kernel(ConvArgs p)
     const int px = px0 + px_local;
     const bool px_valid = px < p.spatial;
     const int oy = px / s.ow, ox = px - oy * s.ow;
-    const int iy0 = oy * s.stride_h - s.pad_h;
-    const int ix0 = ox * s.stride_w - s.pad_w;
+    const int iy0 = TRANSPOSED ? oy + s.pad_h : oy * s.stride_h - s.pad_h;
+    const int ix0 = TRANSPOSED ? ox + s.pad_w : ox * s.stride_w - s.pad_w;
     const int base = iy0 * W + ix0;
     const float *img = p.input + static_cast<size_t>(image) * s.c_in * H * W;
 
@@ -149,11 +155,19 @@ __global__ __launch_bounds__(64 * WM * WN) void conv2d_f32_kernel(ConvArgs p)
             float v = 0.0f;
             if (px_valid && (FULLK || k < K)) {
                 const int2 e = lut[k];
-                const int iy = iy0 + (e.y & 0xffff);
-                const int ix = ix0 + (e.y >> 16);
-                if (static_cast<unsigned>(iy) < static_cast<unsigned>(H) &&
-                    static_cast<unsigned>(ix) < static_cast<unsigned>(W))
-                    v = img[base + e.x];
+                if (TRANSPOSED) {
+                    const int ty = iy0 - (e.y & 0xffff), tx = ix0 - (e.y >> 16);
+                    if (ty >= 0 && tx >= 0) {
+                        const int sy = ty / s.stride_h, sx = tx / s.stride_w;
+                        if (sy * s.stride_h == ty && sx * s.stride_w == tx && sy < H && sx < W) v = img[e.x + sy * W + sx];
+                    }
+                } else {
+                    const int iy = iy0 + (e.y & 0xffff);
+                    const int ix = ix0 + (e.y >> 16);
+                    if (static_cast<unsigned>(iy) < static_cast<unsigned>(H) &&
+                        static_cast<unsigned>(ix) < static_cast<unsigned>(W))
+                        v = img[base + e.x];
+                }
             }
             rb[r] = v;
         }
@@ -488,7 +502,7 @@ hipError_t launch_ring(ConvArgs args, hipStream_t stream)
     return hipGetLastError();
 }
 
-template <int BM, int BN, int BK, int WM, int WN>
+template <int BM, int BN, int BK, int WM, int WN, bool TRANSPOSED = false>
 hipError_t launch_tile(ConvArgs args, bool vec, hipStream_t stream)
 {
     args.tiles_oc = (args.s.c_out + BM - 1) / BM;
@@ -510,11 +524,11 @@ hipError_t launch_tile(ConvArgs args, bool vec, hipStream_t stream)
         return hipSuccess;
     };
     if (vec && args.K % BK == 0)
-        rc = launch(conv2d_f32_kernel<BM, BN, BK, WM, WN, true, true>);
+        rc = launch(conv2d_f32_kernel<BM, BN, BK, WM, WN, true, true, TRANSPOSED>);
     else if (vec)
-        rc = launch(conv2d_f32_kernel<BM, BN, BK, WM, WN, true, false>);
+        rc = launch(conv2d_f32_kernel<BM, BN, BK, WM, WN, true, false, TRANSPOSED>);
     else
-        rc = launch(conv2d_f32_kernel<BM, BN, BK, WM, WN, false, false>);
+        rc = launch(conv2d_f32_kernel<BM, BN, BK, WM, WN, false, false, TRANSPOSED>);
     if (rc != hipSuccess) return rc;
     return hipGetLastError();
 }
@@ -551,6 +565,30 @@ hipError_t launch_conv2d_f32(const ConvShape &shape, int activation, const float
     if (ring_ok) return shape.c_out > 64 ? launch_ring<128>(args, stream) : launch_ring<64>(args, stream);
     if (shape.c_out > 64) return launch_tile<128, 64, 16, 4, 2>(args, vec, stream);
     return launch_tile<64, 64, 16, 2, 2>(args, vec, stream);
+}
+
+// Adjoint gather for strides other than 1: `shape` describes the virtual forward problem (see TRANSPOSED above).
+hipError_t launch_conv2d_adjoint_f32(const ConvShape &shape, const float *grad_output, const float *weight_ic_major,
+                                     float *grad_input, hipStream_t stream)
+{
+    if (shape.batch == 0 || shape.c_out == 0 || shape.oh == 0 || shape.ow == 0) return hipSuccess;
+    ConvArgs args;
+    args.input = grad_output;
+    args.weight = weight_ic_major;
+    args.bias = nullptr;
+    args.out = grad_input;
+    args.s = shape;
+    args.K = shape.c_in * shape.kh * shape.kw;
+    args.spatial = shape.oh * shape.ow;
+    args.tiles_px = args.tiles_oc = 0;
+    args.xcd_swizzle = 0;
+    args.activation = ST_HIP_ACT_NONE;
+    if ((shape.kh - 1) * static_cast<long long>(shape.dil_h) > 0x7fff ||
+        (shape.kw - 1) * static_cast<long long>(shape.dil_w) > 0x7fff || args.K > kConvMaxReduction)
+        return hipErrorInvalidValue;
+    const bool vec = (args.K % 4 == 0) && ((reinterpret_cast<uintptr_t>(weight_ic_major) & 15u) == 0);
+    if (shape.c_out > 64) return launch_tile<128, 64, 16, 4, 2, true>(args, vec, stream);
+    return launch_tile<64, 64, 16, 2, 2, true>(args, vec, stream);
 }
 
 }  // namespace sthip

@@ -1,0 +1,303 @@
+// Conv2d backward on gfx950: gradients with respect to the input, the weight and the bias.
+//
+// Reference: Conv2d::backward → accumulate_from_grad_matrix, crates/st-nn/src/layers/conv.rs:780-813, with
+// G = grad_output re-laid as (batch·OH·OW, C_out) (:750-778):
+//   grad_weight = (Gᵀ · patches) · scale        (matmul_lhs_transpose_scaled, :791-795; scale = 1/batch)
+//   grad_bias   = column sums of G · scale       (:796-799)
+//   grad_input  = col2im(G · W)                  (:803-809, col2im :860-916)
+// Neither the patch matrix, nor G, nor the (pixels × C_in·KH·KW) product is materialised here:
+//   * grad_input is the adjoint convolution.  For stride 1 it IS a forward convolution of grad_output with the
+//     taps flipped and the channel roles swapped (padding dil·(k−1) − pad), so it runs on the forward kernels;
+//     other strides take the same implicit GEMM with the adjoint gather.
+//   * grad_weight is an implicit GEMM  G_b(C_out × pixels) · patches_b(pixels × C_in·KH·KW)  summed over images:
+//     C_out × C_in·KH·KW is small and the reduction long, so the images are split over workgroups, partial tiles
+//     go to the stream's workspace and a second kernel adds them in a fixed order (reproducible) and scales.
+//   * grad_bias is a per-channel sum over NCHW planes.
+#include "device_math.h"
+#include "kernels.h"
+
+namespace sthip {
+
+namespace {
+
+// dst[ic][oc][ky][kx] = src[oc][ic][flip ? KH-1-ky : ky][flip ? KW-1-kx : kx]
+__global__ __launch_bounds__(256) void conv_weight_to_adjoint_kernel(int c_out, int c_in, int kh, int kw, int flip,
+                                                                     const float *src, float *dst)
+{
+    const int total = c_out * c_in * kh * kw;
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const int kx = i % kw;
+    int rest = i / kw;
+    const int ky = rest % kh;
+    rest /= kh;
+    const int oc = rest % c_out;
+    const int ic = rest / c_out;
+    const int sy = flip ? kh - 1 - ky : ky, sx = flip ? kw - 1 - kx : kx;
+    dst[i] = src[((static_cast<size_t>(oc) * c_in + ic) * kh + sy) * kw + sx];
+}
+
+__device__ __forceinline__ float wave_sum64(float v)
+{
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) v += __shfl_xor(v, offset);
+    return v;
+}
+
+// partial[b][oc] = Σ_pixels grad_output[b][oc][pixel]; one wavefront per (b, oc) plane.
+__global__ __launch_bounds__(256) void conv_grad_bias_partial_kernel(int planes, int spatial, const float *grad_output,
+                                                                     float *partial)
+{
+    const int lane = threadIdx.x & 63;
+    const int plane = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (plane >= planes) return;
+    const float *src = grad_output + static_cast<size_t>(plane) * spatial;
+    float sum = 0.0f;
+    for (int i = lane; i < spatial; i += 64) sum += src[i];
+    sum = wave_sum64(sum);
+    if (lane == 0) partial[plane] = sum;
+}
+
+// out[i] = scale · Σ_c partial[c][i], chunks added in order.
+__global__ __launch_bounds__(256) void conv_reduce_chunks_kernel(int chunks, size_t count, const float *partial, float scale,
+                                                                 float *out)
+{
+    const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (i >= count) return;
+    float sum = 0.0f;
+    for (int c = 0; c < chunks; ++c) sum += partial[static_cast<size_t>(c) * count + i];
+    out[i] = sum * scale;
+}
+
+struct GradWeightArgs {
+    const float *input;        // (N, C_in, H, W)
+    const float *grad_output;  // (N, C_out, OH, OW)
+    float *partial;            // (chunks, C_out, S)
+    ConvShape s;
+    int S;                     // c_in * kh * kw
+    int spatial;               // oh * ow
+    int tiles_s;
+    int images_per_chunk;
+};
+
+// One workgroup: a 64 (output channels) × 64 (reduction columns s) tile of grad_weight, summed over the pixels of
+// its images.  Per 16-pixel step the G tile (64 × 16, pixel-contiguous in NCHW) and the patch tile (16 × 64, gathered:
+// thread owns one column s, whose channel/tap offset is fixed for the whole kernel) are fetched into registers while
+// the MFMAs of the previous step run, then written to the other LDS stage.
+template <bool VEC>
+__global__ __launch_bounds__(256) void conv_grad_weight_kernel(GradWeightArgs p)
+{
+    constexpr int BM = 64, BN = 64, BK = 16;
+    constexpr int A_STRIDE = BK + 4, B_STRIDE = BN + 8;
+    __shared__ __attribute__((aligned(16))) float As[2][BM * A_STRIDE];
+    __shared__ __attribute__((aligned(16))) float Bs[2][BK * B_STRIDE];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int li = lane & 31, lh = lane >> 5;
+    const ConvShape &s = p.s;
+    const int H = s.h, W = s.w;
+
+    int bid = blockIdx.x;
+    const int tile_s = bid % p.tiles_s;
+    bid /= p.tiles_s;
+    const int tiles_oc = (s.c_out + BM - 1) / BM;
+    const int tile_oc = bid % tiles_oc;
+    const int chunk = bid / tiles_oc;
+    const int oc0 = tile_oc * BM, s0 = tile_s * BN;
+    const int image0 = chunk * p.images_per_chunk;
+    const int image1 = min(s.batch, image0 + p.images_per_chunk);
+
+    // This thread's patch column and its fixed tap.
+    const int col = s0 + (tid & 63);
+    const bool col_valid = col < p.S;
+    const int khw = s.kh * s.kw;
+    const int ic = col_valid ? col / khw : 0;
+    const int rem = col_valid ? col - ic * khw : 0;
+    const int ky = rem / s.kw, kx = rem - ky * s.kw;
+    const int dy = ky * s.dil_h - s.pad_h, dx = kx * s.dil_w - s.pad_w;
+    const int tap_offset = ic * H * W;
+    const int prow0 = tid >> 6;  // patch rows prow0 + 4r of a step
+
+    // G tile: thread loads 4 consecutive pixels of one channel row.
+    const int a_row = tid >> 2, a_c4 = (tid & 3) * 4;
+    const bool a_row_valid = oc0 + a_row < s.c_out;
+
+    f32x16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+
+    const int steps_per_image = (p.spatial + BK - 1) / BK;
+    const int total_steps = (image1 - image0) * steps_per_image;
+
+    float4 ra;
+    float rb[4];
+    auto load_global = [&](int t) {
+        const int image = image0 + t / steps_per_image;
+        const int p0 = (t % steps_per_image) * BK;
+        ra = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (a_row_valid) {
+            const float *src = p.grad_output + (static_cast<size_t>(image) * s.c_out + oc0 + a_row) * p.spatial + p0 + a_c4;
+            if (VEC && p0 + a_c4 + 3 < p.spatial) {
+                ra = *reinterpret_cast<const float4 *>(src);
+            } else {
+                if (p0 + a_c4 + 0 < p.spatial) ra.x = src[0];
+                if (p0 + a_c4 + 1 < p.spatial) ra.y = src[1];
+                if (p0 + a_c4 + 2 < p.spatial) ra.z = src[2];
+                if (p0 + a_c4 + 3 < p.spatial) ra.w = src[3];
+            }
+        }
+        const float *img = p.input + static_cast<size_t>(image) * s.c_in * H * W + tap_offset;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int pix = p0 + prow0 + 4 * r;
+            float v = 0.0f;
+            if (col_valid && pix < p.spatial) {
+                const int oy = pix / s.ow, ox = pix - oy * s.ow;
+                const int iy = oy * s.stride_h + dy, ix = ox * s.stride_w + dx;
+                if (static_cast<unsigned>(iy) < static_cast<unsigned>(H) && static_cast<unsigned>(ix) < static_cast<unsigned>(W))
+                    v = img[iy * W + ix];
+            }
+            rb[r] = v;
+        }
+    };
+    auto store_lds = [&](int stage) {
+        *reinterpret_cast<float4 *>(&As[stage][a_row * A_STRIDE + a_c4]) = ra;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) Bs[stage][(prow0 + 4 * r) * B_STRIDE + (tid & 63)] = rb[r];
+    };
+    auto compute = [&](int stage) {
+        const float *as = As[stage];
+        const float *bs = Bs[stage];
+#pragma unroll
+        for (int kk = 0; kk < BK / 8; ++kk) {
+            const float4 av = *reinterpret_cast<const float4 *>(&as[(wm * 32 + li) * A_STRIDE + kk * 8 + lh * 4]);
+            float b[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) b[t] = bs[(kk * 8 + lh * 4 + t) * B_STRIDE + wn * 32 + li];
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av.x, b[0], acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av.y, b[1], acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av.z, b[2], acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av.w, b[3], acc, 0, 0, 0);
+        }
+    };
+
+    if (total_steps > 0) {
+        load_global(0);
+        store_lds(0);
+    }
+    __syncthreads();
+    for (int t = 0; t < total_steps; ++t) {
+        const bool more = t + 1 < total_steps;
+        if (more) load_global(t + 1);
+        compute(t & 1);
+        if (more) store_lds((t + 1) & 1);
+        __syncthreads();
+    }
+
+    float *dst = p.partial + static_cast<size_t>(chunk) * s.c_out * p.S;
+    const int out_col = s0 + wn * 32 + li;
+    if (out_col < p.S) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int oc = oc0 + wm * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
+            if (oc < s.c_out) dst[static_cast<size_t>(oc) * p.S + out_col] = acc[r];
+        }
+    }
+}
+
+}  // namespace
+
+hipError_t launch_conv2d_grad_input_f32(const ConvShape &shape, const float *grad_output, const float *weight,
+                                        float *grad_input, hipStream_t stream)
+{
+    if (shape.batch == 0 || shape.c_in == 0 || shape.h == 0 || shape.w == 0) return hipSuccess;
+    const size_t weight_count = static_cast<size_t>(shape.c_out) * shape.c_in * shape.kh * shape.kw;
+    const int adj_pad_h = shape.dil_h * (shape.kh - 1) - shape.pad_h;
+    const int adj_pad_w = shape.dil_w * (shape.kw - 1) - shape.pad_w;
+    const bool as_forward = shape.stride_h == 1 && shape.stride_w == 1 && adj_pad_h >= 0 && adj_pad_w >= 0;
+    void *workspace = nullptr;
+    hipError_t rc = stream_workspace(stream, weight_count * sizeof(float), &workspace);
+    if (rc != hipSuccess) return rc;
+    float *adjoint_weight = static_cast<float *>(workspace);
+    hipLaunchKernelGGL(conv_weight_to_adjoint_kernel, dim3(static_cast<unsigned>((weight_count + 255) / 256)), dim3(256), 0,
+                       stream, shape.c_out, shape.c_in, shape.kh, shape.kw, as_forward ? 1 : 0, weight, adjoint_weight);
+    rc = hipGetLastError();
+    if (rc != hipSuccess) return rc;
+    // The virtual forward problem: grad_output is the image, input positions are the output pixels.
+    ConvShape t = shape;
+    t.c_in = shape.c_out;
+    t.h = shape.oh;
+    t.w = shape.ow;
+    t.c_out = shape.c_in;
+    t.oh = shape.h;
+    t.ow = shape.w;
+    if (as_forward) {
+        t.pad_h = adj_pad_h;
+        t.pad_w = adj_pad_w;
+        return launch_conv2d_f32(t, ST_HIP_ACT_NONE, grad_output, adjoint_weight, nullptr, grad_input, stream);
+    }
+    return launch_conv2d_adjoint_f32(t, grad_output, adjoint_weight, grad_input, stream);
+}
+
+hipError_t launch_conv2d_grad_bias_f32(const ConvShape &shape, const float *grad_output, float scale, float *grad_bias,
+                                       hipStream_t stream)
+{
+    if (shape.c_out == 0) return hipSuccess;
+    const size_t planes = static_cast<size_t>(shape.batch) * shape.c_out;
+    const int spatial = shape.oh * shape.ow;
+    void *workspace = nullptr;
+    hipError_t rc = stream_workspace(stream, (planes ? planes : 1) * sizeof(float), &workspace);
+    if (rc != hipSuccess) return rc;
+    float *partial = static_cast<float *>(workspace);
+    if (planes > 0) {
+        hipLaunchKernelGGL(conv_grad_bias_partial_kernel, dim3(static_cast<unsigned>((planes + 3) / 4)), dim3(256), 0, stream,
+                           static_cast<int>(planes), spatial, grad_output, partial);
+        rc = hipGetLastError();
+        if (rc != hipSuccess) return rc;
+    }
+    hipLaunchKernelGGL(conv_reduce_chunks_kernel, dim3(static_cast<unsigned>((shape.c_out + 255) / 256)), dim3(256), 0, stream,
+                       shape.batch, static_cast<size_t>(shape.c_out), partial, scale, grad_bias);
+    return hipGetLastError();
+}
+
+hipError_t launch_conv2d_grad_weight_f32(const ConvShape &shape, const float *input, const float *grad_output, float scale,
+                                         float *grad_weight, hipStream_t stream)
+{
+    const int S = shape.c_in * shape.kh * shape.kw;
+    const size_t count = static_cast<size_t>(shape.c_out) * S;
+    if (count == 0) return hipSuccess;
+    GradWeightArgs args;
+    args.input = input;
+    args.grad_output = grad_output;
+    args.s = shape;
+    args.S = S;
+    args.spatial = shape.oh * shape.ow;
+    args.tiles_s = (S + 63) / 64;
+    const int tiles = args.tiles_s * ((shape.c_out + 63) / 64);
+    // Enough image chunks to give every compute unit a few workgroups, at most one chunk per image.
+    int chunks = (2048 + tiles - 1) / tiles;
+    if (chunks > shape.batch) chunks = shape.batch;
+    if (chunks < 1) chunks = 1;
+    args.images_per_chunk = shape.batch > 0 ? (shape.batch + chunks - 1) / chunks : 1;
+    chunks = shape.batch > 0 ? (shape.batch + args.images_per_chunk - 1) / args.images_per_chunk : 1;
+    void *workspace = nullptr;
+    hipError_t rc = stream_workspace(stream, static_cast<size_t>(chunks) * count * sizeof(float), &workspace);
+    if (rc != hipSuccess) return rc;
+    args.partial = static_cast<float *>(workspace);
+    const bool vec = args.spatial % 4 == 0 && (reinterpret_cast<uintptr_t>(grad_output) & 15u) == 0;
+    const dim3 grid(static_cast<unsigned>(static_cast<size_t>(tiles) * chunks));
+    if (vec)
+        hipLaunchKernelGGL(conv_grad_weight_kernel<true>, grid, dim3(256), 0, stream, args);
+    else
+        hipLaunchKernelGGL(conv_grad_weight_kernel<false>, grid, dim3(256), 0, stream, args);
+    rc = hipGetLastError();
+    if (rc != hipSuccess) return rc;
+    hipLaunchKernelGGL(conv_reduce_chunks_kernel, dim3(static_cast<unsigned>((count + 255) / 256)), dim3(256), 0, stream, chunks,
+                       count, args.partial, scale, grad_weight);
+    return hipGetLastError();
+}
+
+}  // namespace sthip

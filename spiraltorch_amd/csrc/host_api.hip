@@ -464,6 +464,69 @@ int st_hip_conv2d_bias_act_f32(size_t batch, size_t c_in, size_t h, size_t w, si
     return lease.download(out, d_out, out_len * sizeof(float));
 }
 
+int st_hip_conv2d_backward_f32(size_t batch, size_t c_in, size_t h, size_t w, size_t c_out, size_t kh, size_t kw,
+                               size_t stride_h, size_t stride_w, size_t pad_h, size_t pad_w, size_t dil_h, size_t dil_w,
+                               const float *input, size_t input_len, const float *weight, size_t weight_len,
+                               const float *grad_output, size_t grad_output_len, float *grad_input, size_t grad_input_len,
+                               float *grad_weight, size_t grad_weight_len, float *grad_bias, size_t grad_bias_len)
+{
+    ST_HIP_CHECK(ensure_init());
+    ConvPlan plan;
+    ST_HIP_CHECK(plan_conv(batch, c_in, h, w, c_out, kh, kw, stride_h, stride_w, pad_h, pad_w, dil_h, dil_w, &plan));
+    if (input_len != plan.input_len)
+        return fail(ST_HIP_ERR_INVALID, "input buffer length %zu does not match batch*c_in*h*w=%zu", input_len, plan.input_len);
+    if (weight_len != plan.weight_len)
+        return fail(ST_HIP_ERR_INVALID, "weight buffer length %zu does not match c_out*c_in*kh*kw=%zu", weight_len,
+                    plan.weight_len);
+    if (grad_output_len != plan.out_len)
+        return fail(ST_HIP_ERR_INVALID, "grad_output buffer length %zu does not match batch*c_out*oh*ow=%zu", grad_output_len,
+                    plan.out_len);
+    if (grad_input_len != plan.input_len)
+        return fail(ST_HIP_ERR_INVALID, "grad_input buffer length %zu does not match batch*c_in*h*w=%zu", grad_input_len,
+                    plan.input_len);
+    if (grad_weight_len != plan.weight_len)
+        return fail(ST_HIP_ERR_INVALID, "grad_weight buffer length %zu does not match c_out*c_in*kh*kw=%zu", grad_weight_len,
+                    plan.weight_len);
+    if (grad_bias_len != c_out)
+        return fail(ST_HIP_ERR_INVALID, "grad_bias buffer length %zu does not match c_out=%zu", grad_bias_len, c_out);
+    if (c_out * kh * kw > static_cast<size_t>(kConvMaxReduction))
+        return fail(ST_HIP_ERR_UNSUPPORTED, "conv2d backward reduction extent c_out*kh*kw=%zu exceeds %d", c_out * kh * kw,
+                    kConvMaxReduction);
+    ST_HIP_CHECK(reject_null(input, input_len, "conv2d backward"));
+    ST_HIP_CHECK(reject_null(weight, weight_len, "conv2d backward"));
+    ST_HIP_CHECK(reject_null(grad_output, grad_output_len, "conv2d backward"));
+    ST_HIP_CHECK(reject_null(grad_input, grad_input_len, "conv2d backward"));
+    ST_HIP_CHECK(reject_null(grad_weight, grad_weight_len, "conv2d backward"));
+    ST_HIP_CHECK(reject_null(grad_bias, grad_bias_len, "conv2d backward"));
+    if (batch == 0) return ST_HIP_OK;  // conv.rs:787-789: an empty batch leaves the parameter gradients untouched
+
+    Lease lease;
+    ST_HIP_CHECK(lease.status());
+    void *d_x, *d_w, *d_g, *d_gi, *d_gw, *d_gb;
+    ST_HIP_CHECK(lease.upload(0, input, input_len * sizeof(float), &d_x));
+    ST_HIP_CHECK(lease.upload(1, weight, weight_len * sizeof(float), &d_w));
+    ST_HIP_CHECK(lease.upload(2, grad_output, grad_output_len * sizeof(float), &d_g));
+    ST_HIP_CHECK(lease.buffer(3, grad_input_len * sizeof(float), &d_gi));
+    ST_HIP_CHECK(lease.buffer(4, grad_weight_len * sizeof(float), &d_gw));
+    ST_HIP_CHECK(lease.buffer(5, grad_bias_len * sizeof(float), &d_gb));
+    const float scale = 1.0f / static_cast<float>(batch);  // conv.rs:793,799
+    // The three kernels share the stream's workspace one after the other (stream order).
+    ST_HIP_CHECK(launch_status(launch_conv2d_grad_weight_f32(plan.shape, static_cast<const float *>(d_x),
+                                                             static_cast<const float *>(d_g), scale,
+                                                             static_cast<float *>(d_gw), lease.stream()),
+                               "conv2d grad_weight launch"));
+    ST_HIP_CHECK(launch_status(launch_conv2d_grad_bias_f32(plan.shape, static_cast<const float *>(d_g), scale,
+                                                           static_cast<float *>(d_gb), lease.stream()),
+                               "conv2d grad_bias launch"));
+    ST_HIP_CHECK(launch_status(launch_conv2d_grad_input_f32(plan.shape, static_cast<const float *>(d_g),
+                                                            static_cast<const float *>(d_w), static_cast<float *>(d_gi),
+                                                            lease.stream()),
+                               "conv2d grad_input launch"));
+    ST_HIP_CHECK(lease.download(grad_weight, d_gw, grad_weight_len * sizeof(float)));
+    ST_HIP_CHECK(lease.download(grad_bias, d_gb, grad_bias_len * sizeof(float)));
+    return lease.download(grad_input, d_gi, grad_input_len * sizeof(float));
+}
+
 int st_hip_attention_f32(size_t contexts, size_t sequence, size_t head_dim, float scale, int causal,
                          const float *q, size_t q_len, const float *k, size_t k_len, const float *v, size_t v_len,
                          const float *z_bias, size_t z_bias_len, const float *attn_bias, size_t attn_bias_len,
@@ -629,6 +692,53 @@ int st_hip_conv2d_bias_act_f32_dev(size_t batch, size_t c_in, size_t h, size_t w
         return fail(ST_HIP_ERR_INVALID, "conv2d received a null pointer; provide contiguous buffers");
     return launch_status(launch_conv2d_f32(plan.shape, activation, input, weight, bias, out, as_stream(stream)),
                          "conv2d launch");
+}
+
+int st_hip_conv2d_grad_input_f32_dev(size_t batch, size_t c_in, size_t h, size_t w, size_t c_out, size_t kh, size_t kw,
+                                     size_t stride_h, size_t stride_w, size_t pad_h, size_t pad_w, size_t dil_h,
+                                     size_t dil_w, const float *grad_output, const float *weight, float *grad_input,
+                                     void *stream)
+{
+    ST_HIP_CHECK(ensure_init());
+    ConvPlan plan;
+    ST_HIP_CHECK(plan_conv(batch, c_in, h, w, c_out, kh, kw, stride_h, stride_w, pad_h, pad_w, dil_h, dil_w, &plan));
+    if (c_out * kh * kw > static_cast<size_t>(kConvMaxReduction))
+        return fail(ST_HIP_ERR_UNSUPPORTED, "conv2d backward reduction extent c_out*kh*kw=%zu exceeds %d", c_out * kh * kw,
+                    kConvMaxReduction);
+    if (plan.input_len == 0) return ST_HIP_OK;
+    if (!grad_output || !weight || !grad_input)
+        return fail(ST_HIP_ERR_INVALID, "conv2d backward received a null pointer; provide contiguous buffers");
+    return launch_status(launch_conv2d_grad_input_f32(plan.shape, grad_output, weight, grad_input, as_stream(stream)),
+                         "conv2d grad_input launch");
+}
+
+int st_hip_conv2d_grad_weight_f32_dev(size_t batch, size_t c_in, size_t h, size_t w, size_t c_out, size_t kh, size_t kw,
+                                      size_t stride_h, size_t stride_w, size_t pad_h, size_t pad_w, size_t dil_h,
+                                      size_t dil_w, const float *input, const float *grad_output, float scale,
+                                      float *grad_weight, void *stream)
+{
+    ST_HIP_CHECK(ensure_init());
+    ConvPlan plan;
+    ST_HIP_CHECK(plan_conv(batch, c_in, h, w, c_out, kh, kw, stride_h, stride_w, pad_h, pad_w, dil_h, dil_w, &plan));
+    if (!std::isfinite(scale)) return fail(ST_HIP_ERR_INVALID, "gemm scale must be finite, received %g", static_cast<double>(scale));
+    if (!grad_weight || (batch != 0 && plan.out_len != 0 && (!input || !grad_output)))
+        return fail(ST_HIP_ERR_INVALID, "conv2d backward received a null pointer; provide contiguous buffers");
+    return launch_status(launch_conv2d_grad_weight_f32(plan.shape, input, grad_output, scale, grad_weight, as_stream(stream)),
+                         "conv2d grad_weight launch");
+}
+
+int st_hip_conv2d_grad_bias_f32_dev(size_t batch, size_t c_in, size_t h, size_t w, size_t c_out, size_t kh, size_t kw,
+                                    size_t stride_h, size_t stride_w, size_t pad_h, size_t pad_w, size_t dil_h,
+                                    size_t dil_w, const float *grad_output, float scale, float *grad_bias, void *stream)
+{
+    ST_HIP_CHECK(ensure_init());
+    ConvPlan plan;
+    ST_HIP_CHECK(plan_conv(batch, c_in, h, w, c_out, kh, kw, stride_h, stride_w, pad_h, pad_w, dil_h, dil_w, &plan));
+    if (!std::isfinite(scale)) return fail(ST_HIP_ERR_INVALID, "gemm scale must be finite, received %g", static_cast<double>(scale));
+    if (!grad_bias || (plan.out_len != 0 && !grad_output))
+        return fail(ST_HIP_ERR_INVALID, "conv2d backward received a null pointer; provide contiguous buffers");
+    return launch_status(launch_conv2d_grad_bias_f32(plan.shape, grad_output, scale, grad_bias, as_stream(stream)),
+                         "conv2d grad_bias launch");
 }
 
 int st_hip_attention_f32_dev(size_t contexts, size_t sequence, size_t head_dim, float scale, int causal,

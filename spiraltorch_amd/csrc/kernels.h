@@ -38,6 +38,18 @@ constexpr int kConvMaxReduction = 8192;
 hipError_t launch_conv2d_f32(const ConvShape &shape, int activation, const float *input,
                              const float *weight, const float *bias, float *out, hipStream_t stream);
 
+// Adjoint gather of the implicit GEMM (`shape` is the virtual forward problem: grad_output as the image, input
+// positions as output pixels, original stride/padding/dilation; weight laid out [c_in][c_out·kh·kw]).
+hipError_t launch_conv2d_adjoint_f32(const ConvShape &shape, const float *grad_output,
+                                     const float *weight_ic_major, float *grad_input, hipStream_t stream);
+// Conv2d backward (crates/st-nn/src/layers/conv.rs:780-813, 860-916); `shape` is the forward shape.
+hipError_t launch_conv2d_grad_input_f32(const ConvShape &shape, const float *grad_output, const float *weight,
+                                        float *grad_input, hipStream_t stream);
+hipError_t launch_conv2d_grad_weight_f32(const ConvShape &shape, const float *input, const float *grad_output,
+                                         float scale, float *grad_weight, hipStream_t stream);
+hipError_t launch_conv2d_grad_bias_f32(const ConvShape &shape, const float *grad_output, float scale,
+                                       float *grad_bias, hipStream_t stream);
+
 // Largest head_dim the attention kernel is instantiated for.
 constexpr int kAttentionMaxHeadDim = 256;
 hipError_t launch_attention_f32(size_t contexts, size_t sequence, size_t head_dim, float scale,

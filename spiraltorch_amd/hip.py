@@ -173,6 +173,17 @@ def conv2d_bias_activation_f32(batch, c_in, h, w, c_out, kernel, stride, padding
         0 if b is None else b.size, _ptr(out), out.size))
 
 
+def conv2d_backward_f32(batch, c_in, h, w, c_out, kernel, stride, padding, dilation, input, weight, grad_output,
+                        grad_input, grad_weight, grad_bias) -> None:
+    """Conv2d::backward (conv.rs:780-813): fills grad_input, grad_weight (scaled 1/batch) and grad_bias (1/batch)."""
+    x, wgt, g = _f32(input, "input"), _f32(weight, "weight"), _f32(grad_output, "grad_output")
+    gi, gw, gb = _out(grad_input, "grad_input"), _out(grad_weight, "grad_weight"), _out(grad_bias, "grad_bias")
+    _check(_lib.load().st_hip_conv2d_backward_f32(
+        batch, c_in, h, w, c_out, kernel[0], kernel[1], stride[0], stride[1], padding[0], padding[1], dilation[0],
+        dilation[1], _ptr(x), x.size, _ptr(wgt), wgt.size, _ptr(g), g.size, _ptr(gi), gi.size, _ptr(gw), gw.size,
+        _ptr(gb), gb.size))
+
+
 def attention_f32(contexts, sequence, head_dim, scale, causal, q, k, v, z_bias, attn_bias, out) -> None:
     q, k, v, out = _f32(q, "q"), _f32(k, "k"), _f32(v, "v"), _out(out, "out")
     zb = None if z_bias is None else _f32(z_bias, "z_bias")
@@ -330,6 +341,27 @@ def conv2d_bias_act_f32_dev(batch, c_in, h, w, c_out, kernel, stride, padding, d
     _check(_lib.load().st_hip_conv2d_bias_act_f32_dev(
         batch, c_in, h, w, c_out, kernel[0], kernel[1], stride[0], stride[1], padding[0], padding[1], dilation[0],
         dilation[1], int(activation), _dev(input), _dev(weight), _dev(bias), _dev(out), _stream_ptr(stream)))
+
+
+def conv2d_grad_input_f32_dev(batch, c_in, h, w, c_out, kernel, stride, padding, dilation, grad_output, weight,
+                              grad_input, stream=None) -> None:
+    _check(_lib.load().st_hip_conv2d_grad_input_f32_dev(
+        batch, c_in, h, w, c_out, kernel[0], kernel[1], stride[0], stride[1], padding[0], padding[1], dilation[0],
+        dilation[1], _dev(grad_output), _dev(weight), _dev(grad_input), _stream_ptr(stream)))
+
+
+def conv2d_grad_weight_f32_dev(batch, c_in, h, w, c_out, kernel, stride, padding, dilation, input, grad_output, scale,
+                               grad_weight, stream=None) -> None:
+    _check(_lib.load().st_hip_conv2d_grad_weight_f32_dev(
+        batch, c_in, h, w, c_out, kernel[0], kernel[1], stride[0], stride[1], padding[0], padding[1], dilation[0],
+        dilation[1], _dev(input), _dev(grad_output), scale, _dev(grad_weight), _stream_ptr(stream)))
+
+
+def conv2d_grad_bias_f32_dev(batch, c_in, h, w, c_out, kernel, stride, padding, dilation, grad_output, scale,
+                             grad_bias, stream=None) -> None:
+    _check(_lib.load().st_hip_conv2d_grad_bias_f32_dev(
+        batch, c_in, h, w, c_out, kernel[0], kernel[1], stride[0], stride[1], padding[0], padding[1], dilation[0],
+        dilation[1], _dev(grad_output), scale, _dev(grad_bias), _stream_ptr(stream)))
 
 
 def attention_f32_dev(contexts, sequence, head_dim, scale, causal, q, k, v, z_bias, attn_bias, out,

@@ -111,3 +111,61 @@ def test_empty_batch(oracle):
     out = oracle.conv2d_bias_act_f32(0, 2, 4, 4, 3, (3, 3), (1, 1), (1, 1), (1, 1), oracle.ACT_NONE,
                                      np.zeros(0, np.float32), np.ones(54, np.float32), None)
     assert out.size == 0
+
+
+# ---- backward -------------------------------------------------------------------------------------------
+
+def test_backward_reference_1x1_vector(oracle):
+    """conv2d_backward_matches_manual_kernel11, crates/st-nn/src/layers/conv.rs:4114-4130: weight 1.5, input
+    [1,2,3,4] on 2x2, grad_output ones -> grad_input 1.5 everywhere, grad_weight 10, grad_bias 4."""
+    gi, gw, gb = oracle.conv2d_backward_f32(1, 1, 2, 2, 1, (1, 1), (1, 1), (0, 0), (1, 1), [1, 2, 3, 4], [1.5],
+                                            [1, 1, 1, 1])
+    assert gi.tolist() == [1.5] * 4 and gw.tolist() == [10.0] and gb.tolist() == [4.0]
+
+
+def _direct_backward_f64(batch, c_in, h, w, c_out, kernel, stride, padding, dilation, x, wgt, g):
+    """Closed form of the three gradients written from the definition (not via patches)."""
+    kh, kw = kernel
+    oh = (h + 2 * padding[0] - ((kh - 1) * dilation[0] + 1)) // stride[0] + 1
+    ow = (w + 2 * padding[1] - ((kw - 1) * dilation[1] + 1)) // stride[1] + 1
+    x = np.asarray(x, np.float64).reshape(batch, c_in, h, w)
+    wgt = np.asarray(wgt, np.float64).reshape(c_out, c_in, kh, kw)
+    g = np.asarray(g, np.float64).reshape(batch, c_out, oh, ow)
+    gi, gw = np.zeros_like(x), np.zeros_like(wgt)
+    for oy in range(oh):
+        for ox in range(ow):
+            for ky in range(kh):
+                for kx in range(kw):
+                    iy = oy * stride[0] + ky * dilation[0] - padding[0]
+                    ix = ox * stride[1] + kx * dilation[1] - padding[1]
+                    if 0 <= iy < h and 0 <= ix < w:
+                        gi[:, :, iy, ix] += g[:, :, oy, ox] @ wgt[:, :, ky, kx]
+                        gw[:, :, ky, kx] += g[:, :, oy, ox].T @ x[:, :, iy, ix]
+    return gi.ravel(), gw.ravel() / batch, g.sum(axis=(0, 2, 3)) / batch
+
+
+BACKWARD_CASES = [
+    (2, 3, 8, 8, 4, (3, 3), (1, 1), (1, 1), (1, 1)), (1, 2, 7, 5, 5, (3, 2), (1, 2), (1, 1), (1, 1)),
+    (2, 2, 9, 9, 3, (3, 3), (2, 2), (1, 1), (2, 2)), (1, 1, 6, 6, 2, (1, 1), (1, 1), (0, 0), (1, 1)),
+    (3, 4, 5, 6, 2, (2, 3), (2, 1), (0, 2), (1, 1)),
+]
+
+
+@pytest.mark.parametrize("case", BACKWARD_CASES)
+def test_backward_matches_the_definition_and_the_adjoint_identity(oracle, case):
+    batch, c_in, h, w, c_out, kernel, stride, padding, dilation = case
+    rng = np.random.default_rng(sum(case[:5]))
+    oh, ow = oracle.conv2d_output_hw(h, w, kernel, stride, padding, dilation)
+    x = rng.normal(size=batch * c_in * h * w).astype(np.float32)
+    wgt = rng.normal(size=c_out * c_in * kernel[0] * kernel[1]).astype(np.float32)
+    g = rng.normal(size=batch * c_out * oh * ow).astype(np.float32)
+    gi, gw, gb = oracle.conv2d_backward_f32(*case, x, wgt, g)
+    want_gi, want_gw, want_gb = _direct_backward_f64(*case, x, wgt, g)
+    assert_close(gi, want_gi, 1e-5, 1e-5, "grad_input")
+    assert_close(gw, want_gw, 1e-5, 1e-5, "grad_weight")
+    assert_close(gb, want_gb, 1e-5, 1e-5, "grad_bias")
+    # <conv(x), g> == <x, grad_input(g)>: ties the backward to the (separately pinned) forward
+    y = oracle.conv2d_bias_act_f32(*case[:5], kernel, stride, padding, dilation, oracle.ACT_NONE, x, wgt, None)
+    lhs = float(np.dot(y.astype(np.float64), g.astype(np.float64)))
+    rhs = float(np.dot(x.astype(np.float64), gi.astype(np.float64)))
+    assert abs(lhs - rhs) <= 1e-4 * max(1.0, abs(lhs))
