@@ -113,6 +113,29 @@ def wl_conv2d(hip, inputs, timer, warmup, steps):
         (x, wt, b, geom, (batch, c_in, h, w, c_out))
 
 
+def wl_conv2d_backward(hip, inputs, timer, warmup, steps, which):
+    """Gradients of config 2's convolution: grad_input (adjoint convolution) or grad_weight (reduction over
+    batch and pixels); both cost the forward's FLOPs."""
+    batch, c_in, h, w, c_out = 32, 64, 56, 56, 128
+    x = inputs.normal(inputs.seed_for(2, 0), batch * c_in * h * w)
+    wt = inputs.normal(inputs.seed_for(2, 1), c_out * c_in * 9, 0.0, math.sqrt(2.0 / (c_in * 9)))
+    g = inputs.normal(inputs.seed_for(2, 3), batch * c_out * h * w)
+    d_x, d_w, d_g = (hip.DeviceBuffer.from_array(a) for a in (x, wt, g))
+    geom = ((3, 3), (1, 1), (1, 1), (1, 1))
+    if which == "grad_input":
+        d_out = hip.DeviceBuffer(x.nbytes)
+        step = lambda stream: hip.conv2d_grad_input_f32_dev(batch, c_in, h, w, c_out, *geom, d_g, d_w, d_out, stream)
+        bytes_ = 4 * (g.size + wt.size + x.size)
+    else:
+        d_out = hip.DeviceBuffer(wt.nbytes)
+        step = lambda stream: hip.conv2d_grad_weight_f32_dev(batch, c_in, h, w, c_out, *geom, d_x, d_g, 1.0 / batch,
+                                                             d_out, stream)
+        bytes_ = 4 * (g.size + wt.size + x.size)
+    wall, ev = timer.run(step, warmup, steps)
+    flops = 2 * batch * c_out * h * w * c_in * 9
+    return entry(f"conv2d_{which}_f32_n32_c64to128_56x56_k3s1p1", "f32", flops, bytes_, "mfma", wall, ev)
+
+
 def wl_gemm_f32(hip, inputs, timer, warmup, steps, m, n, k, name):
     a = inputs.uniform(inputs.seed_for(1, 0), m * k, -1.0, 1.0)
     b = inputs.uniform(inputs.seed_for(1, 1), k * n, -1.0, 1.0)
@@ -253,6 +276,8 @@ def main():
     side_steps = max(5, min(args.steps, 20))
     side_warm = max(2, min(args.warmup, 5))
     plan = [
+        ("conv2d_grad_input", lambda: wl_conv2d_backward(hip, inputs, timer, side_warm, side_steps, "grad_input")),
+        ("conv2d_grad_weight", lambda: wl_conv2d_backward(hip, inputs, timer, side_warm, side_steps, "grad_weight")),
         ("gemm_f32_512", lambda: wl_gemm_f32(hip, inputs, timer, side_warm, side_steps, 512, 512, 512,
                                               "gemm_f32_512x512x512")),
         ("gemm_f32_conv_equivalent", lambda: wl_gemm_f32(hip, inputs, timer, side_warm, side_steps, 100352, 128, 576,

@@ -69,6 +69,8 @@ __global__ __launch_bounds__(256) void conv_reduce_chunks_kernel(int chunks, siz
     out[i] = sum * scale;
 }
 
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+
 struct GradWeightArgs {
     const float *input;        // (N, C_in, H, W)
     const float *grad_output;  // (N, C_out, OH, OW)
@@ -77,7 +79,7 @@ struct GradWeightArgs {
     int S;                     // c_in * kh * kw
     int spatial;               // oh * ow
     int tiles_s;
-    int images_per_chunk;
+    int steps_per_chunk;       // 16-pixel steps (numbered image by image) per workgroup
 };
 
 // One workgroup: a 64 (output channels) × 64 (reduction columns s) tile of grad_weight, summed over the pixels of
@@ -107,8 +109,6 @@ __global__ __launch_bounds__(256) void conv_grad_weight_kernel(GradWeightArgs p)
     const int tile_oc = bid % tiles_oc;
     const int chunk = bid / tiles_oc;
     const int oc0 = tile_oc * BM, s0 = tile_s * BN;
-    const int image0 = chunk * p.images_per_chunk;
-    const int image1 = min(s.batch, image0 + p.images_per_chunk);
 
     // This thread's patch column and its fixed tap.
     const int col = s0 + (tid & 63);
@@ -119,7 +119,7 @@ __global__ __launch_bounds__(256) void conv_grad_weight_kernel(GradWeightArgs p)
     const int ky = rem / s.kw, kx = rem - ky * s.kw;
     const int dy = ky * s.dil_h - s.pad_h, dx = kx * s.dil_w - s.pad_w;
     const int tap_offset = ic * H * W;
-    const int prow0 = tid >> 6;  // patch rows prow0 + 4r of a step
+    const int prow0 = (tid >> 6) * 4;  // patch rows prow0 .. prow0+3 of a step: four consecutive pixels
 
     // G tile: thread loads 4 consecutive pixels of one channel row.
     const int a_row = tid >> 2, a_c4 = (tid & 3) * 4;
@@ -130,43 +130,77 @@ __global__ __launch_bounds__(256) void conv_grad_weight_kernel(GradWeightArgs p)
     for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
 
     const int steps_per_image = (p.spatial + BK - 1) / BK;
-    const int total_steps = (image1 - image0) * steps_per_image;
+    const int first_step = chunk * p.steps_per_chunk;
+    const int total_steps = max(0, min(s.batch * steps_per_image, first_step + p.steps_per_chunk) - first_step);
 
-    float4 ra;
+    // (oy, ox) of this thread's first pixel of the step being loaded, advanced by 16 pixels per step without
+    // divisions (integer division costs about twenty vector instructions, and on this chip every vector
+    // instruction takes time from the f32 matrix pipe).  Memory is addressed through per-image buffer descriptors
+    // with 32-bit offsets; anything outside (padding, pixels past the end, channels past C_out) gets an
+    // out-of-range offset and reads as zero.
+    int load_image = first_step / steps_per_image, load_step = first_step - load_image * steps_per_image;
+    int oy, ox;
+    {
+        const int first_pixel = load_step * BK + prow0;
+        oy = first_pixel / s.ow;
+        ox = first_pixel - oy * s.ow;
+    }
+    const unsigned image_bytes = static_cast<unsigned>(s.c_in) * H * W * 4u;
+    const unsigned grad_bytes = static_cast<unsigned>(s.c_out) * p.spatial * 4u;
+    constexpr unsigned kOutside = 0x80000000u;
+    const unsigned a_base = a_row_valid ? (static_cast<unsigned>(oc0 + a_row) * p.spatial + a_c4) * 4u : kOutside;
+
+    u32x4_t ra;
     float rb[4];
-    auto load_global = [&](int t) {
-        const int image = image0 + t / steps_per_image;
-        const int p0 = (t % steps_per_image) * BK;
-        ra = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (a_row_valid) {
-            const float *src = p.grad_output + (static_cast<size_t>(image) * s.c_out + oc0 + a_row) * p.spatial + p0 + a_c4;
-            if (VEC && p0 + a_c4 + 3 < p.spatial) {
-                ra = *reinterpret_cast<const float4 *>(src);
-            } else {
-                if (p0 + a_c4 + 0 < p.spatial) ra.x = src[0];
-                if (p0 + a_c4 + 1 < p.spatial) ra.y = src[1];
-                if (p0 + a_c4 + 2 < p.spatial) ra.z = src[2];
-                if (p0 + a_c4 + 3 < p.spatial) ra.w = src[3];
+    auto load_global = [&]() {
+        const int p0 = load_step * BK;
+        const __amdgpu_buffer_rsrc_t rsrc_g = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<float *>(p.grad_output + static_cast<size_t>(load_image) * s.c_out * p.spatial), 0,
+            static_cast<int>(grad_bytes), 0x00020000);
+        const __amdgpu_buffer_rsrc_t rsrc_x = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<float *>(p.input + static_cast<size_t>(load_image) * s.c_in * H * W), 0, static_cast<int>(image_bytes),
+            0x00020000);
+        if (VEC) {  // spatial % 4 == 0: a 16-byte chunk is entirely inside its channel row or entirely past it
+            const unsigned off = (p0 + a_c4 < p.spatial) ? a_base + static_cast<unsigned>(p0) * 4u : kOutside;
+            ra = __builtin_amdgcn_raw_buffer_load_b128(rsrc_g, off, 0, 0);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const unsigned off = (p0 + a_c4 + e < p.spatial) ? a_base + static_cast<unsigned>(p0 + e) * 4u : kOutside;
+                ra[e] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_g, off, 0, 0);
             }
         }
-        const float *img = p.input + static_cast<size_t>(image) * s.c_in * H * W + tap_offset;
+        int py = oy, px = ox;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const int pix = p0 + prow0 + 4 * r;
-            float v = 0.0f;
-            if (col_valid && pix < p.spatial) {
-                const int oy = pix / s.ow, ox = pix - oy * s.ow;
-                const int iy = oy * s.stride_h + dy, ix = ox * s.stride_w + dx;
-                if (static_cast<unsigned>(iy) < static_cast<unsigned>(H) && static_cast<unsigned>(ix) < static_cast<unsigned>(W))
-                    v = img[iy * W + ix];
+            const int iy = py * s.stride_h + dy, ix = px * s.stride_w + dx;
+            const bool inside = col_valid && p0 + prow0 + r < p.spatial && static_cast<unsigned>(iy) < static_cast<unsigned>(H) &&
+                                static_cast<unsigned>(ix) < static_cast<unsigned>(W);
+            const unsigned off = inside ? static_cast<unsigned>(tap_offset + iy * W + ix) * 4u : kOutside;
+            rb[r] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc_x, off, 0, 0));
+            if (++px == s.ow) {
+                px = 0;
+                ++py;
             }
-            rb[r] = v;
+        }
+        // advance to the next step (possibly the next image)
+        if (++load_step == steps_per_image) {
+            load_step = 0;
+            ++load_image;
+            oy = prow0 / s.ow;
+            ox = prow0 - oy * s.ow;
+        } else {
+            ox += BK;
+            while (ox >= s.ow) {
+                ox -= s.ow;
+                ++oy;
+            }
         }
     };
     auto store_lds = [&](int stage) {
-        *reinterpret_cast<float4 *>(&As[stage][a_row * A_STRIDE + a_c4]) = ra;
+        *reinterpret_cast<u32x4_t *>(&As[stage][a_row * A_STRIDE + a_c4]) = ra;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) Bs[stage][(prow0 + 4 * r) * B_STRIDE + (tid & 63)] = rb[r];
+        for (int r = 0; r < 4; ++r) Bs[stage][(prow0 + r) * B_STRIDE + (tid & 63)] = rb[r];
     };
     auto compute = [&](int stage) {
         const float *as = As[stage];
@@ -185,13 +219,13 @@ __global__ __launch_bounds__(256) void conv_grad_weight_kernel(GradWeightArgs p)
     };
 
     if (total_steps > 0) {
-        load_global(0);
+        load_global();
         store_lds(0);
     }
     __syncthreads();
     for (int t = 0; t < total_steps; ++t) {
         const bool more = t + 1 < total_steps;
-        if (more) load_global(t + 1);
+        if (more) load_global();
         compute(t & 1);
         if (more) store_lds((t + 1) & 1);
         __syncthreads();
@@ -269,6 +303,10 @@ hipError_t launch_conv2d_grad_weight_f32(const ConvShape &shape, const float *in
     const int S = shape.c_in * shape.kh * shape.kw;
     const size_t count = static_cast<size_t>(shape.c_out) * S;
     if (count == 0) return hipSuccess;
+    // One image of the input and of grad_output is addressed through 32-bit byte offsets.
+    if (static_cast<size_t>(shape.c_in) * shape.h * shape.w * 4 >= (1ull << 31) ||
+        static_cast<size_t>(shape.c_out) * shape.oh * shape.ow * 4 >= (1ull << 31))
+        return hipErrorInvalidValue;
     GradWeightArgs args;
     args.input = input;
     args.grad_output = grad_output;
@@ -277,26 +315,29 @@ hipError_t launch_conv2d_grad_weight_f32(const ConvShape &shape, const float *in
     args.spatial = shape.oh * shape.ow;
     args.tiles_s = (S + 63) / 64;
     const int tiles = args.tiles_s * ((shape.c_out + 63) / 64);
-    // Enough image chunks to give every compute unit a few workgroups, at most one chunk per image.
-    int chunks = (2048 + tiles - 1) / tiles;
-    if (chunks > shape.batch) chunks = shape.batch;
+    // The reduction (all 16-pixel steps of all images, numbered image by image) is cut into chunks so that the
+    // launch is a whole number of rounds of 2048 workgroups (8 per compute unit) where the problem allows it.
+    const long long steps_per_image = (args.spatial + 15) / 16;
+    const long long total_steps = steps_per_image * shape.batch;
+    long long chunks = (2048 + tiles - 1) / tiles;
+    if (chunks > total_steps) chunks = total_steps;
     if (chunks < 1) chunks = 1;
-    args.images_per_chunk = shape.batch > 0 ? (shape.batch + chunks - 1) / chunks : 1;
-    chunks = shape.batch > 0 ? (shape.batch + args.images_per_chunk - 1) / args.images_per_chunk : 1;
+    args.steps_per_chunk = static_cast<int>(total_steps > 0 ? (total_steps + chunks - 1) / chunks : 1);
+    chunks = total_steps > 0 ? (total_steps + args.steps_per_chunk - 1) / args.steps_per_chunk : 1;
     void *workspace = nullptr;
     hipError_t rc = stream_workspace(stream, static_cast<size_t>(chunks) * count * sizeof(float), &workspace);
     if (rc != hipSuccess) return rc;
     args.partial = static_cast<float *>(workspace);
     const bool vec = args.spatial % 4 == 0 && (reinterpret_cast<uintptr_t>(grad_output) & 15u) == 0;
-    const dim3 grid(static_cast<unsigned>(static_cast<size_t>(tiles) * chunks));
+    const dim3 grid(static_cast<unsigned>(static_cast<size_t>(tiles) * static_cast<size_t>(chunks)));
     if (vec)
         hipLaunchKernelGGL(conv_grad_weight_kernel<true>, grid, dim3(256), 0, stream, args);
     else
         hipLaunchKernelGGL(conv_grad_weight_kernel<false>, grid, dim3(256), 0, stream, args);
     rc = hipGetLastError();
     if (rc != hipSuccess) return rc;
-    hipLaunchKernelGGL(conv_reduce_chunks_kernel, dim3(static_cast<unsigned>((count + 255) / 256)), dim3(256), 0, stream, chunks,
-                       count, args.partial, scale, grad_weight);
+    hipLaunchKernelGGL(conv_reduce_chunks_kernel, dim3(static_cast<unsigned>((count + 255) / 256)), dim3(256), 0, stream,
+                       static_cast<int>(chunks), count, args.partial, scale, grad_weight);
     return hipGetLastError();
 }
 
