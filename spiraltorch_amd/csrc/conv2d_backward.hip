@@ -102,7 +102,10 @@ __global__ __launch_bounds__(256) void conv_grad_weight_kernel(GradWeightArgs p)
     const ConvShape &s = p.s;
     const int H = s.h, W = s.w;
 
+    // Workgroup ids go round-robin over the 8 XCDs; give each XCD a contiguous run of (chunk, tile) pairs so that
+    // the tiles that share a chunk's pixels find them in the same L2.
     int bid = blockIdx.x;
+    if ((gridDim.x & 7) == 0) bid = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
     const int tile_s = bid % p.tiles_s;
     bid /= p.tiles_s;
     const int tiles_oc = (s.c_out + BM - 1) / BM;
