@@ -529,6 +529,142 @@ __global__ __launch_bounds__(256) void gemm_f32_ring_64x64_kernel(GemmF32Args p)
 __global__ __launch_bounds__(256) void gemm_f32_ring_64x64_at_kernel(GemmF32Args p) { gemm_f32_ring_body<64, 64, 2, 2, true, false>(p); }
 __global__ __launch_bounds__(256) void gemm_f32_ring_64x64_bt_kernel(GemmF32Args p) { gemm_f32_ring_body<64, 64, 2, 2, false, true>(p); }
 
+// Small problems (fewer 64×64 tiles than compute units): 32×32 tiles, and the four wavefronts of a workgroup
+// split K between them — wavefront w takes k-tiles w, w+4, w+8, ... through a ring of its own, so the loop has
+// no barrier at all (a wavefront only waits for its own loads) — and add their partial tiles through LDS at the
+// end.  Same direct-to-LDS staging and layouts as the ring kernel above.
+__global__ __launch_bounds__(256) void gemm_f32_ring_32x32_splitk_kernel(GemmF32Args p)
+{
+    constexpr int BM = 32, BN = 32, BK = 16, RING = 3, LOADS = 4;
+    constexpr int A_BYTES = BM * BK * 4, STAGE = A_BYTES + BK * BN * 4;
+    constexpr int WAVE_BYTES = RING * STAGE;
+    __shared__ __attribute__((aligned(16))) unsigned char lds[4 * WAVE_BYTES];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int li = lane & 31, lh = lane >> 5;
+    const int M = p.M, N = p.N, K = p.K;
+    const int tile_m = blockIdx.x / p.tiles_n, tile_n = blockIdx.x % p.tiles_n;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float *>(p.A), 0, static_cast<int>(static_cast<size_t>(M) * K * 4), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float *>(p.B), 0, static_cast<int>(static_cast<size_t>(K) * N * 4), 0x00020000);
+    constexpr unsigned kOutside = 0x80000000u;
+    unsigned a_off[2], b_off[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int row = j * 16 + (lane >> 2);
+        const int chunk = (lane & 3) ^ ((row >> 2) & 3);
+        a_off[j] = (m0 + row < M) ? (static_cast<unsigned>(m0 + row) * K + chunk * 4) * 4u : kOutside;
+        const int f = j * 256 + lane * 4;
+        const int k = f / BN, col = f % BN;
+        b_off[j] = (n0 + col < N) ? (static_cast<unsigned>(k) * N + n0 + col) * 4u : kOutside;
+    }
+    const unsigned b_step = static_cast<unsigned>(BK) * N * 4u;
+    unsigned char *ring = lds + wave * WAVE_BYTES;
+
+    auto issue = [&](auto slot_tag, int t) {  // t: global k-tile index
+        constexpr int SLOT = decltype(slot_tag)::value;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_ptr)(ring + SLOT * STAGE + j * 1024), 16, a_off[j],
+                                                     t * (BK * 4), 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_void_ptr)(ring + SLOT * STAGE + A_BYTES + j * 1024), 16,
+                                                     b_off[j], t * b_step, 0, 0);
+        }
+    };
+    unsigned a_lane[2];
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) a_lane[kk] = li * 64 + (((kk * 2 + lh) ^ ((li >> 2) & 3)) * 16);
+    const unsigned b_lane = A_BYTES + (lh * 4 * BN + li) * 4;
+
+    f32x16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+    auto compute = [&](auto slot_tag) {
+        constexpr int SLOT = decltype(slot_tag)::value;
+        const unsigned char *stage = ring + SLOT * STAGE;
+        f32x4 a[2];
+        float b[2][4];
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk) {
+            a[kk] = *reinterpret_cast<const f32x4 *>(stage + a_lane[kk]);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) b[kk][t] = *reinterpret_cast<const float *>(stage + b_lane + (kk * 8 + t) * BN * 4);
+        }
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+            for (int t = 0; t < 4; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kk][t], b[kk][t], acc, 0, 0, 0);
+    };
+
+    const int steps = K / BK;
+    const int my_steps = steps > wave ? (steps - wave + 3) / 4 : 0;  // k-tiles wave, wave+4, ...
+    if (my_steps > 0) issue(std::integral_constant<int, 0>{}, wave);
+    if (my_steps > 1) issue(std::integral_constant<int, 1>{}, wave + 4);
+    ST_F32_WAIT_VMCNT(0);
+    auto step = [&](auto slot_tag, int i) {
+        constexpr int SLOT = decltype(slot_tag)::value;
+        if (i + 1 < my_steps) ST_F32_WAIT_VMCNT(LOADS);
+        else ST_F32_WAIT_VMCNT(0);
+        asm volatile("" ::: "memory");
+        // slot (i+2)%3 was last read by this same wavefront in step i-1, whose reads have returned
+        if (i + 2 < my_steps) issue(std::integral_constant<int, (SLOT + 2) % RING>{}, wave + 4 * (i + 2));
+        compute(slot_tag);
+    };
+    int i = 0;
+    for (; i + 3 <= my_steps; i += 3) {
+        step(std::integral_constant<int, 0>{}, i);
+        step(std::integral_constant<int, 1>{}, i + 1);
+        step(std::integral_constant<int, 2>{}, i + 2);
+    }
+    if (i < my_steps) step(std::integral_constant<int, 0>{}, i);
+    if (i + 1 < my_steps) step(std::integral_constant<int, 1>{}, i + 1);
+
+    // Add the four partial tiles: each wavefront writes its 32×32 accumulators to LDS, then thread t finishes
+    // row t/8, columns 4·(t%8) .. +3.
+    __syncthreads();
+    float *partial = reinterpret_cast<float *>(lds);  // [4][32][32 + 4]
+    constexpr int P_STRIDE = BN + 4;
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+        partial[(wave * 32 + (r >> 2) * 8 + lh * 4 + (r & 3)) * P_STRIDE + li] = acc[r];
+    __syncthreads();
+    const int row = tid >> 3, c4 = (tid & 7) * 4;
+    float sum[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        const f32x4 v = *reinterpret_cast<const f32x4 *>(&partial[(w * 32 + row) * P_STRIDE + c4]);
+        sum[0] += v[0]; sum[1] += v[1]; sum[2] += v[2]; sum[3] += v[3];
+    }
+    if (m0 + row < M) {
+        const bool scaled = p.scale != 1.0f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int col = n0 + c4 + e;
+            if (col >= N) continue;
+            const size_t idx = static_cast<size_t>(m0 + row) * N + col;
+            float value = sum[e];
+            if (scaled) value *= p.scale;
+            if (p.bias) value += p.bias[col];
+            if (p.residual) value += p.residual[idx];
+            p.C[idx] = apply_activation(value, p.activation);
+        }
+    }
+}
+
+hipError_t launch_splitk32(GemmF32Args args, hipStream_t stream)
+{
+    args.tiles_n = (args.N + 31) / 32;
+    args.tiles_m = (args.M + 31) / 32;
+    const size_t tiles = static_cast<size_t>(args.tiles_n) * static_cast<size_t>(args.tiles_m);
+    hipLaunchKernelGGL(gemm_f32_ring_32x32_splitk_kernel, dim3(static_cast<unsigned>(tiles)), dim3(256), 0, stream, args);
+    return hipGetLastError();
+}
+
 hipError_t launch_ring(GemmF32Args args, bool lhs_transposed, bool rhs_packed, bool big, hipStream_t stream)
 {
     const int bm = big ? 128 : 64, bn = big ? 128 : 64;
@@ -601,6 +737,9 @@ hipError_t launch_gemm_f32(size_t m, size_t n, size_t k, bool lhs_transposed, co
         // rounds; 64×64 tiles otherwise, which spread small problems and leave a shorter tail.
         const size_t tiles128 = ((m + 127) / 128) * ((n + 127) / 128);
         const bool big = tiles128 >= 512 && (tiles128 >= 3072 || tiles128 % 768 == 0 || tiles128 % 768 >= 384);
+        // Fewer 64×64 tiles than compute units: 32×32 tiles with K split over the wavefronts of a workgroup.
+        const size_t tiles64 = ((m + 63) / 64) * ((n + 63) / 64);
+        if (!lhs_transposed && tiles64 <= 256 && k >= 128) return launch_splitk32(args, stream);
         return launch_ring(args, lhs_transposed, false, big, stream);
     }
     return launch_tile<64, 64, 2, 2>(args, lhs_transposed, vec, stream);

@@ -84,7 +84,9 @@ def test_empty_output_is_a_no_op(hip):
 SHAPES = [(1, 1, 1), (2, 3, 4), (8, 12, 7), (10, 13, 9), (8, 16, 6), (4, 16, 5), (33, 65, 17), (64, 64, 64),
           (100, 130, 70), (129, 127, 31), (256, 64, 200), (5, 300, 19), (300, 5, 23),
           # whole 16-wide k-tiles and 16-byte aligned rows: the direct-to-LDS ring kernel, ragged in m and n
-          (132, 136, 48), (260, 68, 160), (96, 260, 16), (1000, 128, 32)]
+          (132, 136, 48), (260, 68, 160), (96, 260, 16), (1000, 128, 32),
+          # few tiles and a long k: 32x32 tiles with k split over the wavefronts of a workgroup
+          (100, 132, 256), (31, 36, 144), (64, 64, 2048)]
 
 
 @pytest.mark.parametrize("m,n,k", SHAPES)
