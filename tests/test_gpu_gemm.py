@@ -86,7 +86,7 @@ SHAPES = [(1, 1, 1), (2, 3, 4), (8, 12, 7), (10, 13, 9), (8, 16, 6), (4, 16, 5),
           # whole 16-wide k-tiles and 16-byte aligned rows: the direct-to-LDS ring kernel, ragged in m and n
           (132, 136, 48), (260, 68, 160), (96, 260, 16), (1000, 128, 32),
           # few tiles and a long k: 32x32 tiles with k split over the wavefronts of a workgroup
-          (100, 132, 256), (31, 36, 144), (64, 64, 2048)]
+          (100, 132, 256), (31, 36, 144), (64, 64, 640)]
 
 
 @pytest.mark.parametrize("m,n,k", SHAPES)
@@ -110,6 +110,22 @@ def test_random_shapes_match_the_oracle(hip, oracle, m, n, k):
         hip.gemm_bias_activation_f32(m, n, k, act, a, b, bias, res, out)
         assert_close(out, oracle.gemm_bias_act_f32(m, n, k, code, a, b, bias, res), F32_REL, F32_ABS,
                      f"bias+residual+{act.name}")
+
+
+def test_long_reduction_against_float64(hip):
+    """k = 4096 with U[-1,1) data: sums of magnitude ~20 whose value can land anywhere near zero, so the bound
+    is the standard one for a reordered f32 sum, a small multiple of unit roundoff times sum |a||b| (about
+    2e-4 here), checked against exact float64 — the oracle's own sequential f32 sum carries the same error."""
+    rng = np.random.default_rng(77)
+    m, n, k = 64, 96, 4096
+    a = rng.uniform(-1, 1, m * k).astype(np.float32)
+    b = rng.uniform(-1, 1, k * n).astype(np.float32)
+    out = np.zeros(m * n, np.float32)
+    hip.gemm_f32(m, n, k, a, b, out)
+    a64, b64 = a.astype(np.float64).reshape(m, k), b.astype(np.float64).reshape(k, n)
+    exact = a64 @ b64
+    bound = 1e-4 * np.abs(exact) + 1e-5 + 2e-7 * (np.abs(a64) @ np.abs(b64))
+    assert (np.abs(out.reshape(m, n) - exact) <= bound).all()
 
 
 def test_config1_512_cubed(hip, oracle):
