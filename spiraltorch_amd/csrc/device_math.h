@@ -35,13 +35,17 @@ __device__ __forceinline__ float apply_activation(float value, int activation)
     return value;
 }
 
-// Round-to-nearest-even f32 -> bf16 bit pattern; NaN stays a quiet NaN.
+// Round-to-nearest-even f32 -> bf16 bit pattern through the hardware conversion (v_cvt_pk_bf16_f32); NaN stays
+// a quiet NaN.
+typedef __bf16 bf16x2_hw __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16x2_rne(float lo, float hi)
+{
+    const bf16x2_hw v = {static_cast<__bf16>(lo), static_cast<__bf16>(hi)};
+    return __builtin_bit_cast(uint32_t, v);
+}
 __device__ __forceinline__ uint16_t f32_to_bf16_rne(float f)
 {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x0040u);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return static_cast<uint16_t>(u >> 16);
+    return __builtin_bit_cast(uint16_t, static_cast<__bf16>(f));
 }
 
 }  // namespace sthip

@@ -458,7 +458,7 @@ __device__ __forceinline__ void gemm_bf16_w8_body(const GemmBf16Args &p)
                 strip[((r >> 2) * 8 + lh * 4 + (r & 3)) * C_STRIDE + tn * 32 + li] = tile[r];
         }
         const int row_base = m0 + wm * 64 + tm * 32;
-#pragma unroll 2
+#pragma unroll
         for (int j = 0; j < 32 / ROWS_PER_PASS; ++j) {
             const int local_row = j * ROWS_PER_PASS + lane / LPR;
             const int row = row_base + local_row;
@@ -478,8 +478,8 @@ __device__ __forceinline__ void gemm_bf16_w8_body(const GemmBf16Args &p)
                 if (p.C32) *reinterpret_cast<float4 *>(p.C32 + idx) = v;
                 if (p.C16) {
                     uint2 packed;
-                    packed.x = f32_to_bf16_rne(v.x) | (static_cast<uint32_t>(f32_to_bf16_rne(v.y)) << 16);
-                    packed.y = f32_to_bf16_rne(v.z) | (static_cast<uint32_t>(f32_to_bf16_rne(v.w)) << 16);
+                    packed.x = pack_bf16x2_rne(v.x, v.y);
+                    packed.y = pack_bf16x2_rne(v.z, v.w);
                     *reinterpret_cast<uint2 *>(p.C16 + idx) = packed;
                 }
             }

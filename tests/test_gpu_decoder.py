@@ -34,6 +34,9 @@ def test_embedding_split_merge_and_rounding(hip, oracle):
     assert (d_out.to_array(np.float32, ids.size * 3) == oracle.embedding_f32(ids.size, 4, 3, ids, table)).all()
 
     vals = np.random.default_rng(0).normal(size=1000).astype(np.float32)
+    # ties (round to even in both directions), the largest finite value, infinities, denormals and signed zero
+    vals[:10] = np.array([1.00390625, 1.01171875, -1.00390625, 3.3895314e38, np.inf, -np.inf, 1e-40, -1e-45, 0.0, -0.0],
+                         np.float32)
     d16 = hip.DeviceBuffer(2000)
     hip.f32_to_bf16_dev(1000, hip.DeviceBuffer.from_array(vals), d16)
     hip.device_synchronize()
