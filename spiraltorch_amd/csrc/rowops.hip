@@ -46,6 +46,60 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(int rows, int cols, con
     }
 }
 
+// Same, for rows of at most 2048 values with 16-byte aligned rows: the row is read once, 128 bits per lane, and
+// stays in registers between the statistics and the normalisation.
+template <int CHUNKS>
+__global__ __launch_bounds__(256) void layer_norm_vec_kernel(int rows, int cols, const float *x, const float *residual,
+                                                             const float *gamma, const float *beta, float epsilon,
+                                                             float *out_f32, uint16_t *out_bf16)
+{
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const size_t offset = static_cast<size_t>(row) * cols;
+    float4 v[CHUNKS];
+    float sum = 0.0f, sumsq = 0.0f;
+#pragma unroll
+    for (int i = 0; i < CHUNKS; ++i) {
+        const int c = (lane + 64 * i) * 4;
+        v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (c < cols) {
+            v[i] = *reinterpret_cast<const float4 *>(x + offset + c);
+            if (residual) {
+                const float4 r = *reinterpret_cast<const float4 *>(residual + offset + c);
+                v[i].x += r.x; v[i].y += r.y; v[i].z += r.z; v[i].w += r.w;
+            }
+        }
+        sum += (v[i].x + v[i].y) + (v[i].z + v[i].w);
+        sumsq += (v[i].x * v[i].x + v[i].y * v[i].y) + (v[i].z * v[i].z + v[i].w * v[i].w);
+    }
+    sum = wave_sum(sum);
+    sumsq = wave_sum(sumsq);
+    const float cols_f = static_cast<float>(cols);
+    const float mean = sum / cols_f;
+    const float var = fmaxf(sumsq / cols_f - mean * mean, 0.0f);
+    const float denom = sqrtf(var + epsilon);
+#pragma unroll
+    for (int i = 0; i < CHUNKS; ++i) {
+        const int c = (lane + 64 * i) * 4;
+        if (c >= cols) continue;
+        const float4 g = *reinterpret_cast<const float4 *>(gamma + c);
+        const float4 b = *reinterpret_cast<const float4 *>(beta + c);
+        float4 o;
+        o.x = ((v[i].x - mean) / denom) * g.x + b.x;
+        o.y = ((v[i].y - mean) / denom) * g.y + b.y;
+        o.z = ((v[i].z - mean) / denom) * g.z + b.z;
+        o.w = ((v[i].w - mean) / denom) * g.w + b.w;
+        if (out_f32) *reinterpret_cast<float4 *>(out_f32 + offset + c) = o;
+        if (out_bf16) {
+            uint2 packed;
+            packed.x = pack_bf16x2_rne(o.x, o.y);
+            packed.y = pack_bf16x2_rne(o.z, o.w);
+            *reinterpret_cast<uint2 *>(out_bf16 + offset + c) = packed;
+        }
+    }
+}
+
 // token_to_index + row gather, crates/st-nn/src/layers/embedding.rs:42-100,325-330.
 __global__ __launch_bounds__(256) void embedding_kernel(int tokens, int vocab, int dim, const float *token_ids,
                                                         const float *table, float *out)
@@ -234,9 +288,23 @@ hipError_t launch_layer_norm_f32(size_t rows, size_t cols, const float *x, const
                                  hipStream_t stream)
 {
     if (rows == 0 || cols == 0) return hipSuccess;
-    hipLaunchKernelGGL(layer_norm_kernel, dim3(static_cast<unsigned>((rows + 3) / 4)), dim3(256), 0, stream,
-                       static_cast<int>(rows), static_cast<int>(cols), x, residual, gamma, beta, epsilon, out_f32,
-                       out_bf16);
+    const dim3 grid(static_cast<unsigned>((rows + 3) / 4)), block(256);
+    auto aligned = [](const void *ptr, uintptr_t a) { return (reinterpret_cast<uintptr_t>(ptr) & (a - 1)) == 0; };
+    const bool vec = cols % 4 == 0 && cols <= 2048 && aligned(x, 16) && aligned(residual, 16) && aligned(gamma, 16) &&
+                     aligned(beta, 16) && aligned(out_f32, 16) && aligned(out_bf16, 8);
+    const int r = static_cast<int>(rows), c = static_cast<int>(cols);
+    if (vec && cols <= 512)
+        hipLaunchKernelGGL(layer_norm_vec_kernel<2>, grid, block, 0, stream, r, c, x, residual, gamma, beta, epsilon, out_f32,
+                           out_bf16);
+    else if (vec && cols <= 1024)
+        hipLaunchKernelGGL(layer_norm_vec_kernel<4>, grid, block, 0, stream, r, c, x, residual, gamma, beta, epsilon, out_f32,
+                           out_bf16);
+    else if (vec)
+        hipLaunchKernelGGL(layer_norm_vec_kernel<8>, grid, block, 0, stream, r, c, x, residual, gamma, beta, epsilon, out_f32,
+                           out_bf16);
+    else
+        hipLaunchKernelGGL(layer_norm_kernel, grid, block, 0, stream, r, c, x, residual, gamma, beta, epsilon, out_f32,
+                           out_bf16);
     return hipGetLastError();
 }
 
