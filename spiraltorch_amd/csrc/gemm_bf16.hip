@@ -448,6 +448,15 @@ __device__ __forceinline__ void gemm_bf16_w8_body(const GemmBf16Args &p)
     const int col0 = n0 + wn * WTN + (lane & (LPR - 1)) * 4;  // this lane's 4 columns in the read-back phase
     float4 bias4 = make_float4(0.f, 0.f, 0.f, 0.f);
     if (p.bias) bias4 = *reinterpret_cast<const float4 *>(p.bias + col0);
+    // bf16-only output (16-byte aligned): 8 columns per lane in the read-back phase
+    constexpr int LPR8 = WTN / 8, ROWS8_PER_PASS = 64 / LPR8;
+    const bool bf16_only = p.C32 == nullptr && (reinterpret_cast<uintptr_t>(p.C16) & 15u) == 0;
+    const int col8 = n0 + wn * WTN + (lane & (LPR8 - 1)) * 8;
+    float bias8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (bf16_only && p.bias) {
+        *reinterpret_cast<float4 *>(bias8) = *reinterpret_cast<const float4 *>(p.bias + col8);
+        *reinterpret_cast<float4 *>(bias8 + 4) = *reinterpret_cast<const float4 *>(p.bias + col8 + 4);
+    }
 #pragma unroll
     for (int tm = 0; tm < 2; ++tm) {
 #pragma unroll
@@ -458,6 +467,41 @@ __device__ __forceinline__ void gemm_bf16_w8_body(const GemmBf16Args &p)
                 strip[((r >> 2) * 8 + lh * 4 + (r & 3)) * C_STRIDE + tn * 32 + li] = tile[r];
         }
         const int row_base = m0 + wm * 64 + tm * 32;
+        if (bf16_only) {
+            // bf16 is the only output: 8 columns (16 bytes) per lane, so half as many store instructions
+#pragma unroll
+            for (int j = 0; j < 32 / ROWS8_PER_PASS; ++j) {
+                const int local_row = j * ROWS8_PER_PASS + lane / LPR8;
+                const int row = row_base + local_row;
+                const float *src = &strip[local_row * C_STRIDE + (lane & (LPR8 - 1)) * 8];
+                float v[8];
+                *reinterpret_cast<float4 *>(v) = *reinterpret_cast<const float4 *>(src);
+                *reinterpret_cast<float4 *>(v + 4) = *reinterpret_cast<const float4 *>(src + 4);
+                if (row < M) {
+                    const size_t idx = static_cast<size_t>(row) * N + col8;
+                    float res[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                    if (p.residual) {
+                        *reinterpret_cast<float4 *>(res) = *reinterpret_cast<const float4 *>(p.residual + idx);
+                        *reinterpret_cast<float4 *>(res + 4) = *reinterpret_cast<const float4 *>(p.residual + idx + 4);
+                    }
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        float value = v[e];
+                        if (scaled) value *= p.scale;
+                        value += bias8[e];
+                        value += res[e];
+                        v[e] = apply_activation(value, p.activation);
+                    }
+                    u32x4 packed;
+                    packed.x = pack_bf16x2_rne(v[0], v[1]);
+                    packed.y = pack_bf16x2_rne(v[2], v[3]);
+                    packed.z = pack_bf16x2_rne(v[4], v[5]);
+                    packed.w = pack_bf16x2_rne(v[6], v[7]);
+                    *reinterpret_cast<u32x4 *>(p.C16 + idx) = packed;
+                }
+            }
+            continue;
+        }
 #pragma unroll
         for (int j = 0; j < 32 / ROWS_PER_PASS; ++j) {
             const int local_row = j * ROWS_PER_PASS + lane / LPR;
