@@ -219,6 +219,30 @@ def wl_decoder(hip, inputs, timer, warmup, steps):
     return out
 
 
+def wl_rowops(hip, inputs, timer, warmup, steps):
+    """HBM-bound tensor utilities at the decoder's activation shape (16384 x 512 f32, 32 MiB): bytes are the
+    algorithmic reads + writes of each op."""
+    rows, cols = 16384, 512
+    n = rows * cols
+    x = inputs.normal(inputs.seed_for(5, 3), n)
+    d_x, d_y = hip.DeviceBuffer.from_array(x), hip.DeviceBuffer(n * 4)
+    d_g = hip.DeviceBuffer.from_array(inputs.normal(inputs.seed_for(5, 4), n))
+    ones = hip.DeviceBuffer.from_array(np.ones(cols, np.float32))
+    d_16, d_cols = hip.DeviceBuffer(n * 2), hip.DeviceBuffer(cols * 4)
+    ops = [
+        ("layer_norm_f32_to_bf16", 6 * n, lambda st: hip.layer_norm_f32_dev(rows, cols, d_x, None, ones, ones, 1e-5, None, d_16, st)),
+        ("row_softmax_f32", 8 * n, lambda st: hip.row_softmax_f32_dev(rows, cols, d_x, d_y, st)),
+        ("gelu_backward_f32", 12 * n, lambda st: hip.gelu_backward_f32_dev(n, d_x, d_g, d_y, st)),
+        ("scale_f32", 8 * n, lambda st: hip.scale_f32_dev(n, d_x, 0.5, d_y, st)),
+        ("sum_axis0_f32", 4 * n, lambda st: hip.sum_axis0_f32_dev(rows, cols, d_x, 1.0, d_cols, st)),
+    ]
+    out = []
+    for name, bytes_, step in ops:
+        wall, ev = timer.run(step, warmup, steps)
+        out.append(entry(f"{name}_16384x512", "f32", 0, bytes_, "hbm", wall, ev))
+    return out
+
+
 def wl_calibration(hip, inputs, timer, warmup, steps):
     """Plain streaming kernel of known traffic (f32 -> bf16 rounding of 64 Mi values: 256 MiB read, 128 MiB
     written).  It anchors the FETCH_SIZE / WRITE_SIZE counters and shows the HBM rate a trivial kernel reaches."""
@@ -290,14 +314,16 @@ def main():
         ("attention_causal", lambda: wl_attention(hip, inputs, timer, 2, 5, True)),
         ("attention_bf16", lambda: wl_attention_bf16(hip, inputs, timer, side_warm, side_steps)),
         ("decoder", lambda: wl_decoder(hip, inputs, timer, 2, 5)),
+        ("rowops", lambda: wl_rowops(hip, inputs, timer, 2, 10)),
         ("calibration", lambda: wl_calibration(hip, inputs, timer, 2, 5)),
     ]
     for name, fn in plan:
         if args.only and args.only not in name:
             continue
         result = fn()
-        log(json.dumps(result))
-        others.append(result)
+        for item in (result if isinstance(result, list) else [result]):
+            log(json.dumps(item))
+            others.append(item)
 
     cpu = None
     if not args.no_cpu_baseline:

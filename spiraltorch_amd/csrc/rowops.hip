@@ -222,6 +222,71 @@ __global__ __launch_bounds__(256) void row_softmax_kernel(int rows, int cols, co
     }
 }
 
+// Same for rows of at most 2048 values with 16-byte aligned rows: one 128-bit read per lane and chunk, the row stays
+// in registers for all three phases.
+template <int CHUNKS>
+__global__ __launch_bounds__(256) void row_softmax_vec_kernel(int rows, int cols, const float *in, float *out)
+{
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const float *x = in + static_cast<size_t>(row) * cols;
+    float *y = out + static_cast<size_t>(row) * cols;
+    float v[CHUNKS][4];
+    float best = -INFINITY;
+    int best_index = 0x7fffffff;
+#pragma unroll
+    for (int i = 0; i < CHUNKS; ++i) {
+        const int c = (lane + 64 * i) * 4;
+        if (c < cols) {
+            const float4 t = *reinterpret_cast<const float4 *>(x + c);
+            v[i][0] = t.x; v[i][1] = t.y; v[i][2] = t.z; v[i][3] = t.w;
+        } else {
+            v[i][0] = v[i][1] = v[i][2] = v[i][3] = __builtin_nanf("");  // skipped like NaN entries, never stored
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float value = v[i][e];
+            if (value != value) continue;
+            if (best_index == 0x7fffffff || value > best) {  // columns visited in ascending order per lane
+                best = value;
+                best_index = c + e;
+            }
+        }
+    }
+    const float row_max = wave_max(best_index == 0x7fffffff ? -INFINITY : best);
+    int candidate = (best_index != 0x7fffffff && best == row_max) ? best_index : 0x7fffffff;
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) candidate = min(candidate, __shfl_xor(candidate, offset));
+    const bool found = candidate != 0x7fffffff;
+    const float base = (found && isfinite(row_max)) ? row_max : 0.0f;
+    float denom = 0.0f;
+#pragma unroll
+    for (int i = 0; i < CHUNKS; ++i)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float value = v[i][e];
+            const float weight = (!found || value != value) ? 0.0f : expf(value - base);
+            v[i][e] = weight;
+            denom += weight;
+        }
+    denom = wave_sum(denom);
+    const bool normal = isfinite(denom) && denom > 1.1920929e-7f;
+    const float inv = normal ? 1.0f / denom : 0.0f;
+#pragma unroll
+    for (int i = 0; i < CHUNKS; ++i) {
+        const int c = (lane + 64 * i) * 4;
+        if (c >= cols) continue;
+        float o[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            o[e] = v[i][e] * inv;
+            if (found && !normal) o[e] = (c + e == candidate) ? 1.0f : 0.0f;
+        }
+        *reinterpret_cast<float4 *>(y + c) = make_float4(o[0], o[1], o[2], o[3]);
+    }
+}
+
 // gelu_prime(z)·g, crates/st-tensor/src/pure.rs:12033-12040 and :6549-6552.
 __global__ __launch_bounds__(256) void gelu_backward_kernel(size_t count, const float *z, const float *grad, float *out)
 {
@@ -265,14 +330,59 @@ __global__ __launch_bounds__(256) void sum_axis0_partial_kernel(int rows, int co
     partial[static_cast<size_t>(blockIdx.y) * cols + c] = sum;
 }
 
-__global__ __launch_bounds__(256) void sum_axis0_final_kernel(int chunks, int cols, const float *partial, float scale,
-                                                              float *out)
+// 16-byte aligned rows: a workgroup covers 256 columns (64 lanes × 4) and its four wavefronts take every fourth
+// row of the chunk, eight independent loads in flight each; the four partial rows are added through LDS.
+__global__ __launch_bounds__(256) void sum_axis0_partial_vec_kernel(int rows, int cols, int rows_per_chunk, const float *in,
+                                                                    float *partial)
 {
-    const int c = blockIdx.x * 256 + threadIdx.x;
-    if (c >= cols) return;
+    __shared__ float4 stage[4][64];
+    const int lane = threadIdx.x & 63, sub = threadIdx.x >> 6;
+    const int c = (blockIdx.x * 64 + lane) * 4;
+    const int r0 = blockIdx.y * rows_per_chunk;
+    const int r1 = min(rows, r0 + rows_per_chunk);
+    float4 acc[2] = {make_float4(0.f, 0.f, 0.f, 0.f), make_float4(0.f, 0.f, 0.f, 0.f)};
+    if (c < cols) {
+        const float *src = in + c;
+        int r = r0 + sub;
+        for (; r + 28 < r1; r += 32) {
+            float4 t[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) t[u] = *reinterpret_cast<const float4 *>(src + static_cast<size_t>(r + 4 * u) * cols);
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                acc[u & 1].x += t[u].x; acc[u & 1].y += t[u].y; acc[u & 1].z += t[u].z; acc[u & 1].w += t[u].w;
+            }
+        }
+        for (; r < r1; r += 4) {
+            const float4 t = *reinterpret_cast<const float4 *>(src + static_cast<size_t>(r) * cols);
+            acc[0].x += t.x; acc[0].y += t.y; acc[0].z += t.z; acc[0].w += t.w;
+        }
+    }
+    stage[sub][lane] = make_float4(acc[0].x + acc[1].x, acc[0].y + acc[1].y, acc[0].z + acc[1].z, acc[0].w + acc[1].w);
+    __syncthreads();
+    if (sub == 0 && c < cols) {
+        float4 total = stage[0][lane];
+#pragma unroll
+        for (int k = 1; k < 4; ++k) {
+            total.x += stage[k][lane].x; total.y += stage[k][lane].y; total.z += stage[k][lane].z; total.w += stage[k][lane].w;
+        }
+        *reinterpret_cast<float4 *>(partial + static_cast<size_t>(blockIdx.y) * cols + c) = total;
+    }
+}
+
+// out[c] = scale · Σ_k partial[k][c]: 64 columns per workgroup, its four wavefronts take every fourth chunk.
+__global__ __launch_bounds__(256) void sum_axis0_final_wide_kernel(int chunks, int cols, const float *partial, float scale,
+                                                                   float *out)
+{
+    __shared__ float stage[4][64];
+    const int lane = threadIdx.x & 63, sub = threadIdx.x >> 6;
+    const int c = blockIdx.x * 64 + lane;
     float sum = 0.0f;
-    for (int k = 0; k < chunks; ++k) sum += partial[static_cast<size_t>(k) * cols + c];
-    out[c] = sum * scale;
+    if (c < cols)
+        for (int k = sub; k < chunks; k += 4) sum += partial[static_cast<size_t>(k) * cols + c];
+    stage[sub][lane] = sum;
+    __syncthreads();
+    if (sub == 0 && c < cols) out[c] = (((stage[0][lane] + stage[1][lane]) + stage[2][lane]) + stage[3][lane]) * scale;
 }
 
 unsigned grid_for(size_t count)
@@ -352,8 +462,17 @@ hipError_t launch_merge_heads_f32(size_t batch, size_t seq, size_t heads, size_t
 hipError_t launch_row_softmax_f32(size_t rows, size_t cols, const float *in, float *out, hipStream_t stream)
 {
     if (rows == 0 || cols == 0) return hipSuccess;
-    hipLaunchKernelGGL(row_softmax_kernel, dim3(static_cast<unsigned>((rows + 3) / 4)), dim3(256), 0, stream,
-                       static_cast<int>(rows), static_cast<int>(cols), in, out);
+    const dim3 grid(static_cast<unsigned>((rows + 3) / 4)), block(256);
+    const int r = static_cast<int>(rows), c = static_cast<int>(cols);
+    const bool vec = cols % 4 == 0 && cols <= 2048 && ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0;
+    if (vec && cols <= 512)
+        hipLaunchKernelGGL(row_softmax_vec_kernel<2>, grid, block, 0, stream, r, c, in, out);
+    else if (vec && cols <= 1024)
+        hipLaunchKernelGGL(row_softmax_vec_kernel<4>, grid, block, 0, stream, r, c, in, out);
+    else if (vec)
+        hipLaunchKernelGGL(row_softmax_vec_kernel<8>, grid, block, 0, stream, r, c, in, out);
+    else
+        hipLaunchKernelGGL(row_softmax_kernel, grid, block, 0, stream, r, c, in, out);
     return hipGetLastError();
 }
 
@@ -382,9 +501,11 @@ hipError_t launch_add_row_f32(size_t rows, size_t cols, float *data, const float
 hipError_t launch_sum_axis0_f32(size_t rows, size_t cols, const float *in, float scale, float *out, hipStream_t stream)
 {
     if (cols == 0) return hipSuccess;
-    // Enough row chunks to occupy the chip, at least 64 rows each; the partial sums live in the stream's workspace.
-    const size_t col_blocks = (cols + 255) / 256;
-    size_t chunks = (2048 + col_blocks - 1) / col_blocks;
+    const bool vec = cols % 4 == 0 && (reinterpret_cast<uintptr_t>(in) & 15u) == 0;
+    // Row chunks: enough workgroups to fill the chip, at least 64 rows each; the partial sums live in the stream's
+    // workspace and are added in a fixed order.
+    const size_t col_blocks = vec ? (cols + 255) / 256 : (cols + 255) / 256;
+    size_t chunks = (1024 + col_blocks - 1) / col_blocks;
     const size_t max_chunks = (rows + 63) / 64;
     if (chunks > max_chunks) chunks = max_chunks;
     if (chunks == 0) chunks = 1;
@@ -395,12 +516,16 @@ hipError_t launch_sum_axis0_f32(size_t rows, size_t cols, const float *in, float
     hipError_t rc = stream_workspace(stream, chunks * cols * sizeof(float), &workspace);
     if (rc != hipSuccess) return rc;
     float *partial = static_cast<float *>(workspace);
-    hipLaunchKernelGGL(sum_axis0_partial_kernel, dim3(static_cast<unsigned>(col_blocks), static_cast<unsigned>(chunks)),
-                       dim3(256), 0, stream, static_cast<int>(rows), static_cast<int>(cols),
-                       static_cast<int>(rows_per_chunk), in, partial);
+    const dim3 grid(static_cast<unsigned>(col_blocks), static_cast<unsigned>(chunks));
+    if (vec)
+        hipLaunchKernelGGL(sum_axis0_partial_vec_kernel, grid, dim3(256), 0, stream, static_cast<int>(rows),
+                           static_cast<int>(cols), static_cast<int>(rows_per_chunk), in, partial);
+    else
+        hipLaunchKernelGGL(sum_axis0_partial_kernel, grid, dim3(256), 0, stream, static_cast<int>(rows),
+                           static_cast<int>(cols), static_cast<int>(rows_per_chunk), in, partial);
     rc = hipGetLastError();
     if (rc != hipSuccess) return rc;
-    hipLaunchKernelGGL(sum_axis0_final_kernel, dim3(static_cast<unsigned>(col_blocks)), dim3(256), 0, stream,
+    hipLaunchKernelGGL(sum_axis0_final_wide_kernel, dim3(static_cast<unsigned>((cols + 63) / 64)), dim3(256), 0, stream,
                        static_cast<int>(chunks), static_cast<int>(cols), partial, scale, out);
     return hipGetLastError();
 }

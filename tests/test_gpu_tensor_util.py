@@ -11,7 +11,7 @@ def on_device(hip, *arrays):
     return [hip.DeviceBuffer.from_array(np.ascontiguousarray(a, dtype=np.float32)) for a in arrays]
 
 
-@pytest.mark.parametrize("rows,cols", [(1, 1), (2, 4), (5, 63), (7, 64), (3, 65), (33, 1000), (1024, 256), (4, 5000)])
+@pytest.mark.parametrize("rows,cols", [(1, 1), (2, 4), (5, 63), (7, 64), (3, 65), (33, 1000), (1024, 256), (4, 5000), (9, 512), (6, 516), (5, 2048), (3, 2052)])
 def test_row_softmax(hip, oracle, rows, cols):
     rng = np.random.default_rng(rows * 31 + cols)
     x = (rng.normal(size=rows * cols) * 3).astype(np.float32)
@@ -67,7 +67,7 @@ def test_scale_and_add_row(hip, oracle):
         hip.scale_f32_dev(x.size, d_x, float("nan"), d_out)
 
 
-@pytest.mark.parametrize("rows,cols", [(1, 1), (3, 2), (64, 256), (65, 257), (1000, 19), (16384, 512), (100000, 8)])
+@pytest.mark.parametrize("rows,cols", [(1, 1), (3, 2), (64, 256), (65, 257), (1000, 19), (16384, 512), (100000, 8), (37, 260), (131, 1028), (5, 4)])
 def test_sum_axis0(hip, oracle, rows, cols):
     rng = np.random.default_rng(rows + cols)
     x = rng.normal(size=rows * cols).astype(np.float32)
