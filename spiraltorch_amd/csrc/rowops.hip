@@ -370,19 +370,34 @@ __global__ __launch_bounds__(256) void sum_axis0_partial_vec_kernel(int rows, in
     }
 }
 
-// out[c] = scale · Σ_k partial[k][c]: 64 columns per workgroup, its four wavefronts take every fourth chunk.
+// out[c] = scale · Σ_k partial[k][c]: 16 columns per workgroup, sixteen groups of lanes take every sixteenth chunk
+// with four loads in flight each; the sixteen partial sums are added in a fixed order through LDS.
 __global__ __launch_bounds__(256) void sum_axis0_final_wide_kernel(int chunks, int cols, const float *partial, float scale,
                                                                    float *out)
 {
-    __shared__ float stage[4][64];
-    const int lane = threadIdx.x & 63, sub = threadIdx.x >> 6;
-    const int c = blockIdx.x * 64 + lane;
-    float sum = 0.0f;
-    if (c < cols)
-        for (int k = sub; k < chunks; k += 4) sum += partial[static_cast<size_t>(k) * cols + c];
-    stage[sub][lane] = sum;
+    __shared__ float stage[16][17];
+    const int col = threadIdx.x & 15, sub = threadIdx.x >> 4;
+    const int c = blockIdx.x * 16 + col;
+    float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (c < cols) {
+        int k = sub;
+        for (; k + 48 < chunks; k += 64) {
+            float t[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) t[u] = partial[static_cast<size_t>(k + 16 * u) * cols + c];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) sum[u] += t[u];
+        }
+        for (; k < chunks; k += 16) sum[0] += partial[static_cast<size_t>(k) * cols + c];
+    }
+    stage[sub][col] = (sum[0] + sum[1]) + (sum[2] + sum[3]);
     __syncthreads();
-    if (sub == 0 && c < cols) out[c] = (((stage[0][lane] + stage[1][lane]) + stage[2][lane]) + stage[3][lane]) * scale;
+    if (sub == 0 && c < cols) {
+        float total = stage[0][col];
+#pragma unroll
+        for (int k = 1; k < 16; ++k) total += stage[k][col];
+        out[c] = total * scale;
+    }
 }
 
 unsigned grid_for(size_t count)
@@ -502,11 +517,11 @@ hipError_t launch_sum_axis0_f32(size_t rows, size_t cols, const float *in, float
 {
     if (cols == 0) return hipSuccess;
     const bool vec = cols % 4 == 0 && (reinterpret_cast<uintptr_t>(in) & 15u) == 0;
-    // Row chunks: enough workgroups to fill the chip, at least 64 rows each; the partial sums live in the stream's
+    // Row chunks: enough workgroups to fill the chip, at least 128 rows each; the partial sums live in the stream's
     // workspace and are added in a fixed order.
-    const size_t col_blocks = vec ? (cols + 255) / 256 : (cols + 255) / 256;
-    size_t chunks = (1024 + col_blocks - 1) / col_blocks;
-    const size_t max_chunks = (rows + 63) / 64;
+    const size_t col_blocks = (cols + 255) / 256;
+    size_t chunks = (512 + col_blocks - 1) / col_blocks;
+    const size_t max_chunks = (rows + 127) / 128;
     if (chunks > max_chunks) chunks = max_chunks;
     if (chunks == 0) chunks = 1;
     const size_t rows_per_chunk = (rows + chunks - 1) / chunks;
@@ -525,7 +540,7 @@ hipError_t launch_sum_axis0_f32(size_t rows, size_t cols, const float *in, float
                            static_cast<int>(cols), static_cast<int>(rows_per_chunk), in, partial);
     rc = hipGetLastError();
     if (rc != hipSuccess) return rc;
-    hipLaunchKernelGGL(sum_axis0_final_wide_kernel, dim3(static_cast<unsigned>((cols + 63) / 64)), dim3(256), 0, stream,
+    hipLaunchKernelGGL(sum_axis0_final_wide_kernel, dim3(static_cast<unsigned>((cols + 15) / 16)), dim3(256), 0, stream,
                        static_cast<int>(chunks), static_cast<int>(cols), partial, scale, out);
     return hipGetLastError();
 }
