@@ -211,6 +211,84 @@ class Tensor:
         _validate_finite(label, out._data)
         return out
 
+    # ---- tensor utilities ------------------------------------------------------------------------
+    def _on_device(self, run, out_values: int, *arrays) -> np.ndarray:
+        """Uploads `arrays`, calls run(device buffers..., output buffer) and downloads `out_values` floats."""
+        try:
+            buffers = [hip.DeviceBuffer.from_array(a) for a in arrays]
+            out = hip.DeviceBuffer(max(out_values, 1) * 4)
+            run(*buffers, out)
+            hip.device_synchronize()
+            return out.to_array(np.float32, out_values)
+        except hip.HipErr as err:
+            raise _backend_failure(err) from err
+
+    def row_softmax(self, *, backend: Optional[str] = None) -> "Tensor":
+        """Row-wise softmax — Tensor::row_softmax_with_backend, pure.rs:3282-3330 (inputs must be finite)."""
+        _resolve_backend(backend)
+        _validate_finite("row_softmax_input", self._data)
+        if self._data.size == 0:
+            return Tensor.zeros(self.rows, self.cols)
+        out = self._on_device(lambda x, y: hip.row_softmax_f32_dev(self.rows, self.cols, x, y), self._data.size,
+                              self._data)
+        _validate_finite("row_softmax_output", out)
+        return Tensor(self.rows, self.cols, out)
+
+    def gelu_backward(self, grad_output: "Tensor", *, backend: Optional[str] = None) -> "Tensor":
+        """gelu'(self) ⊙ grad_output — Tensor::gelu_backward_with_backend, pure.rs:6459-6560."""
+        _resolve_backend(backend)
+        if self.shape() != grad_output.shape():
+            raise TensorError("ShapeMismatch", f"left {self.shape()} right {grad_output.shape()}",
+                              left=self.shape(), right=grad_output.shape())
+        if self._data.size == 0:
+            return Tensor.zeros(self.rows, self.cols)
+        out = self._on_device(lambda z, g, y: hip.gelu_backward_f32_dev(self._data.size, z, g, y), self._data.size,
+                              self._data, grad_output._data)
+        return Tensor(self.rows, self.cols, out)
+
+    def scale(self, value: float, *, backend: Optional[str] = None) -> "Tensor":
+        """self · value — Tensor::scale_with_backend, pure.rs:5517-5620 (value must be finite)."""
+        _resolve_backend(backend)
+        if not np.isfinite(value):
+            raise TensorError("NonFiniteValue", f"non-finite value encountered in scale_factor: {value}",
+                              label="scale_factor")
+        if self._data.size == 0:
+            return Tensor.zeros(self.rows, self.cols)
+        out = self._on_device(lambda x, y: hip.scale_f32_dev(self._data.size, x, float(value), y), self._data.size,
+                              self._data)
+        return Tensor(self.rows, self.cols, out)
+
+    def add_row_inplace(self, bias, *, backend: Optional[str] = None) -> None:
+        """self[r, :] += bias — Tensor::add_row_inplace_with_backend, pure.rs:6201-6290."""
+        _resolve_backend(backend)
+        bias = np.ascontiguousarray(np.asarray(bias, dtype=np.float32)).reshape(-1)
+        if bias.size != self.cols:
+            raise TensorError("DataLength", f"expected {self.cols} values, got {bias.size}", expected=self.cols,
+                              got=bias.size)
+        if self._data.size == 0:
+            return
+        try:
+            data, row = hip.DeviceBuffer.from_array(self._data), hip.DeviceBuffer.from_array(bias)
+            hip.add_row_f32_dev(self.rows, self.cols, data, row)
+            hip.device_synchronize()
+            self._data[:] = data.to_array(np.float32, self._data.size)
+        except hip.HipErr as err:
+            raise _backend_failure(err) from err
+
+    def sum_axis0(self, *, backend: Optional[str] = None) -> np.ndarray:
+        """Column sums — Tensor::sum_axis0_with_backend, pure.rs:7009-7116."""
+        return self.sum_axis0_scaled(1.0, backend=backend)
+
+    def sum_axis0_scaled(self, scale: float, *, backend: Optional[str] = None) -> np.ndarray:
+        """scale · column sums — Tensor::sum_axis0_scaled_with_backend, pure.rs:7118-7230."""
+        _resolve_backend(backend)
+        if self.cols == 0:
+            return np.zeros(0, dtype=np.float32)
+        if self.rows == 0:
+            return np.zeros(self.cols, dtype=np.float32)
+        return self._on_device(lambda x, y: hip.sum_axis0_f32_dev(self.rows, self.cols, x, float(scale), y),
+                               self.cols, self._data)
+
     # ---- attention -------------------------------------------------------------------------------
     def scaled_dot_attention(self, keys: "Tensor", values: "Tensor", *, contexts: int, sequence: int,
                              scale: float, z_bias: Optional["Tensor"] = None,
@@ -241,8 +319,9 @@ class Tensor:
 
 
 class Conv2d:
-    """Conv2d layer of crates/st-nn/src/layers/conv.rs:607-969 (forward only), with the optional fused
-    activation the reference composes as a separate Relu layer."""
+    """Conv2d layer of crates/st-nn/src/layers/conv.rs:607-1013 (forward and backward), with the optional fused
+    activation the reference composes as a separate Relu layer.  `backward` accumulates into `weight_gradient` and
+    `bias_gradient` the way Parameter::accumulate_euclidean does (crates/st-nn/src/module.rs:329-350)."""
 
     def __init__(self, name: str, in_channels: int, out_channels: int, kernel, stride, padding, dilation,
                  input_hw, activation: int = hip.ACT_NONE):
@@ -268,6 +347,8 @@ class Conv2d:
             seed = np.float32(max(np.fmod(np.float32(seed * np.float32(1.57)), np.float32(0.15)), np.float32(5e-3)))
         self.weight = Tensor(self.out_channels, span, ramp)
         self.bias = Tensor.zeros(1, self.out_channels)
+        self.weight_gradient: Optional[Tensor] = None
+        self.bias_gradient: Optional[Tensor] = None
         self.output_hw()  # validates the configuration once (conv.rs:662)
 
     def output_hw(self) -> Tuple[int, int]:
@@ -291,3 +372,41 @@ class Conv2d:
         except hip.HipErr as err:
             raise _backend_failure(err) from err
         return out
+
+    def backward(self, input: Tensor, grad_output: Tensor) -> Tensor:
+        """Conv2d::backward (conv.rs:971-992, 780-811): returns the input gradient and accumulates the weight and
+        bias gradients, both scaled by 1/batch.  Defined for activation None, as in the reference."""
+        if self.activation != hip.ACT_NONE:
+            raise TensorError("BackendFailure", "backward is defined for a Conv2d without fused activation",
+                              backend="hip")
+        h, w = self.input_hw
+        if input.cols != self.in_channels * h * w:
+            raise TensorError("ShapeMismatch", f"left {(1, input.cols)} right {(1, self.in_channels * h * w)}",
+                              left=(1, input.cols), right=(1, self.in_channels * h * w))
+        oh, ow = self.output_hw()
+        if grad_output.shape() != (input.rows, self.out_channels * oh * ow):
+            raise TensorError("ShapeMismatch",
+                              f"left {grad_output.shape()} right {(input.rows, self.out_channels * oh * ow)}",
+                              left=grad_output.shape(), right=(input.rows, self.out_channels * oh * ow))
+        grad_input = Tensor.zeros(input.rows, input.cols)
+        if input.rows == 0:
+            return grad_input
+        grad_weight = Tensor.zeros(*self.weight.shape())
+        grad_bias = Tensor.zeros(1, self.out_channels)
+        try:
+            hip.conv2d_backward_f32(input.rows, self.in_channels, h, w, self.out_channels, self.kernel, self.stride,
+                                    self.padding, self.dilation, input.data(), self.weight.data(), grad_output.data(),
+                                    grad_input.data(), grad_weight.data(), grad_bias.data())
+        except hip.HipErr as err:
+            raise _backend_failure(err) from err
+        for name, update in (("weight_gradient", grad_weight), ("bias_gradient", grad_bias)):
+            existing = getattr(self, name)
+            if existing is None:
+                setattr(self, name, update)
+            else:
+                existing.data()[:] += update.data()
+        return grad_input
+
+    def zero_accumulators(self) -> None:
+        self.weight_gradient = None
+        self.bias_gradient = None

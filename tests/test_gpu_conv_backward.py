@@ -87,3 +87,24 @@ def test_validation(hip):
     hip.conv2d_backward_f32(0, 1, 2, 2, 1, (1, 1), (1, 1), (0, 0), (1, 1), np.zeros(0, np.float32), np.array([1.5], np.float32),
                             np.zeros(0, np.float32), np.zeros(0, np.float32), gw, gb)
     assert gw.tolist() == [7.0]
+
+
+def test_conv2d_layer_backward_accumulates(hip, oracle):
+    import spiraltorch_amd as st
+    rng = np.random.default_rng(5)
+    conv = st.Conv2d("c", 3, 4, (3, 3), (1, 1), (1, 1), (1, 1), (6, 5))
+    batch = 2
+    x = st.Tensor(batch, 3 * 6 * 5, rng.normal(size=batch * 90).astype(np.float32))
+    g = st.Tensor(batch, 4 * 6 * 5, rng.normal(size=batch * 120).astype(np.float32))
+    gi, gw, gb = oracle.conv2d_backward_f32(batch, 3, 6, 5, 4, (3, 3), (1, 1), (1, 1), (1, 1), x.data(),
+                                            conv.weight.data(), g.data())
+    got = conv.backward(x, g)
+    assert_close(got.data(), gi, F32_REL, F32_ABS, "grad_input")
+    assert_close(conv.weight_gradient.data(), gw, F32_REL, F32_ABS, "grad_weight")
+    assert_close(conv.bias_gradient.data(), gb, F32_REL, F32_ABS, "grad_bias")
+    conv.backward(x, g)  # second call accumulates
+    assert_close(conv.weight_gradient.data(), 2 * np.asarray(gw), F32_REL, 2 * F32_ABS, "grad_weight twice")
+    assert_close(conv.bias_gradient.data(), 2 * np.asarray(gb), F32_REL, 2 * F32_ABS, "grad_bias twice")
+    with pytest.raises(st.TensorError, match="ShapeMismatch"):
+        conv.backward(x, st.Tensor.zeros(batch, 7))
+    assert conv.backward(st.Tensor.zeros(0, 90), st.Tensor.zeros(0, 120)).shape() == (0, 90)

@@ -86,3 +86,33 @@ def test_sum_axis0(hip, oracle, rows, cols):
     hip.sum_axis0_f32_dev(rows, cols, d_x, -0.25, again)
     hip.device_synchronize()
     assert (again.to_array(np.float32, cols) == got).all(), "column sums must be reproducible"
+
+
+def test_tensor_mirror_methods(hip, oracle):
+    import spiraltorch_amd as st
+    rng = np.random.default_rng(77)
+    rows, cols = 37, 260
+    x = st.Tensor(rows, cols, rng.normal(size=rows * cols).astype(np.float32))
+    g = st.Tensor(rows, cols, rng.normal(size=rows * cols).astype(np.float32))
+    assert_close(x.row_softmax().data(), oracle.row_softmax_f32(rows, cols, x.data()), F32_REL, F32_ABS, "row_softmax")
+    assert_close(x.gelu_backward(g).data(), oracle.gelu_backward_f32(x.data(), g.data()), F32_REL, F32_ABS,
+                 "gelu_backward")
+    assert (x.scale(0.5).data() == oracle.scale_f32(x.data(), 0.5)).all()
+    bias = rng.normal(size=cols).astype(np.float32)
+    want = oracle.add_row_f32(rows, cols, x.data(), bias)
+    y = st.Tensor(rows, cols, x.data().copy())
+    y.add_row_inplace(bias)
+    assert (y.data() == want).all()
+    sums = x.sum_axis0_scaled(0.25)
+    assert_close(sums, oracle.sum_axis0_f32(rows, cols, x.data(), 0.25), F32_REL, F32_ABS + 1e-5, "sum_axis0_scaled")
+    assert_close(x.sum_axis0(), x.numpy().astype(np.float64).sum(axis=0), F32_REL, F32_ABS + 1e-5, "sum_axis0")
+    with pytest.raises(st.TensorError, match="ShapeMismatch"):
+        x.gelu_backward(st.Tensor.zeros(rows, cols + 1))
+    with pytest.raises(st.TensorError, match="NonFiniteValue"):
+        x.scale(float("inf"))
+    with pytest.raises(st.TensorError, match="DataLength"):
+        y.add_row_inplace(bias[:-1])
+    bad = st.Tensor(1, 2, [1.0, float("nan")])
+    with pytest.raises(st.TensorError, match="NonFiniteValue"):
+        bad.row_softmax()
+    assert st.Tensor.zeros(0, 5).sum_axis0().tolist() == [0.0] * 5
