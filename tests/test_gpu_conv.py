@@ -68,6 +68,33 @@ def test_random_shapes(hip, oracle, shape):
     assert_close(got, oracle.conv2d_bias_act_f32(*shape, oracle.ACT_RELU, x, wt, None), F32_REL, F32_ABS, "no bias")
 
 
+FAMILY_SHAPES = [
+    (2, 16, 20, 20, 70, (3, 3), (1, 1), (1, 1), (1, 1)),    # ragged channel strip, 13 pixel blocks, ragged last block
+    (1, 130, 12, 12, 40, (3, 3), (1, 1), (1, 1), (1, 1)),   # three weight slices (64 + 64 + 2 channels), idle wavefronts
+    (1, 4, 60, 60, 33, (3, 3), (1, 1), (1, 1), (1, 1)),     # several pixel chunks per image
+    (5, 8, 13, 12, 64, (3, 3), (2, 2), (0, 0), (1, 1)),     # stride 2
+    (2, 6, 15, 14, 32, (3, 3), (1, 2), (2, 3), (2, 1)),     # dilation, wide padding, odd channel pairs
+    (2, 32, 9, 9, 16, (1, 9), (1, 1), (0, 4), (1, 1)),      # nine taps in one row
+    (64, 2, 42, 42, 128, (3, 3), (1, 1), (1, 1), (1, 1)),   # 56 blocks per workgroup: seven per wavefront
+    (64, 2, 44, 32, 128, (3, 3), (1, 1), (1, 1), (1, 1)),   # 44 blocks: six and five per wavefront
+]
+
+
+@pytest.mark.parametrize("family", ["strip", "ring", "tile"])
+@pytest.mark.parametrize("shape", FAMILY_SHAPES)
+def test_kernel_families(hip, oracle, monkeypatch, family, shape):
+    """Each kernel family (chosen by shape in normal use) forced on shapes that exercise its edges."""
+    monkeypatch.setenv("ST_HIP_CONV_KERNEL", family)
+    batch, c_in, h, w, c_out, kernel, stride, padding, dilation = shape
+    rng = np.random.default_rng(batch * 1000 + c_in * 10 + c_out)
+    x = rng.normal(size=batch * c_in * h * w).astype(np.float32)
+    wt = rng.normal(0, np.sqrt(2.0 / (c_in * 9)), c_out * c_in * 9).astype(np.float32)
+    b = rng.uniform(-0.1, 0.1, c_out).astype(np.float32)
+    got = run(hip, *shape, 1, x, wt, b)
+    want = oracle.conv2d_bias_act_f32(*shape, oracle.ACT_RELU, x, wt, b, threads=8)
+    assert_close(got, want, F32_REL, F32_ABS, f"conv {shape} family={family}")
+
+
 def test_conv2d_layer_mirror(hip, oracle):
     from spiraltorch_amd import Conv2d, Tensor, TensorError
     conv = Conv2d("conv_gpu", 3, 8, (3, 3), (1, 1), (1, 1), (1, 1), (8, 8))
