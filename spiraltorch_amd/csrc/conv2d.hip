@@ -484,14 +484,17 @@ __global__ __launch_bounds__(256) void conv2d_f32_ring64_kernel(ConvArgs p) { co
 
 // ---- strip kernel: 32 output channels × a long run of pixels per workgroup, no LDS traffic for the image --------
 //
-// A workgroup owns 32 output channels and up to 56 blocks of 32 consecutive output pixels of one image; each of
-// its eight wavefronts owns up to seven of those blocks (seven 32×32 accumulators).  With only 32 output channels
-// per workgroup every gathered image value feeds exactly one MFMA, so it is loaded from global memory (L1/L2)
-// straight into the B operand register: one buffer load per MFMA, with per-lane byte offsets for the nine taps of
-// each block computed once (bit 31 set for padding taps, which the buffer range check turns into 0.0).  The 32
-// weight rows of a 64-channel slice live in LDS for the whole slice, read as three 128-bit loads per channel
-// pair.  There is no barrier in the loop and no per-tile prologue/epilogue; the work of a workgroup is cut to the
-// wavefront, so the chip's 1024 SIMDs finish together when blocks divide evenly.
+// A workgroup of 16 wavefronts owns 32 output channels and a run of 32-pixel blocks of one image.  Its weights
+// (32 rows × c_in × 9 taps) are staged into LDS once and stay there; after that single barrier the wavefronts
+// never synchronise again: each takes the next unclaimed block from a counter in LDS, runs the whole reduction
+// for that 32×32 block, stores it and takes another.  With only 32 output channels per workgroup every gathered
+// image value feeds exactly one MFMA, so it is loaded from global memory (L1/L2) straight into the B operand
+// register: one buffer load per MFMA, all nine taps of the next channel pair requested before the MFMAs of the
+// current pair (measured: f32 MFMAs interleaved one-to-one with independent buffer loads still run at the
+// matrix pipe's full rate).  The nine per-lane byte offsets of a block are computed once, with bit 31 set for
+// padding taps, which the buffer range check turns into 0.0.  Because blocks finish at different times, the
+// output stores of one block overlap the arithmetic of the others, and the unit of load balancing is a single
+// block on a single SIMD.
 //
 // k runs in the pairs {(ic, tap), (ic+1, tap)}: lanes 0-31 supply channel 2j, lanes 32-63 channel 2j+1.
 struct StripArgs {
@@ -502,7 +505,7 @@ struct StripArgs {
     ConvShape s;
     int spatial;           // oh * ow
     int blocks_per_image;  // ceil(spatial / 32)
-    int chunks;            // pixel chunks per image
+    int chunks;            // workgroups per image and channel strip
     int blocks_per_chunk;
     int oc_strips;         // ceil(c_out / 32)
     int total;             // workgroups
@@ -510,200 +513,23 @@ struct StripArgs {
     int activation;
 };
 
-constexpr int kStripTaps = 9, kStripTapPitch = 12, kStripMaxBlocks = 7, kStripChannels = 64;
-constexpr int kStripLdsBytes = kStripChannels * 32 * kStripTapPitch * 4;
+constexpr int kStripTaps = 9, kStripThreads = 1024;
+// 32 rows × c_in channels × 9 taps of f32 weights + the counter must fit 160 KiB of LDS: up to 104 channels with the
+// taps of a channel padded to 12 words (128-bit reads), up to 142 channels packed.
+constexpr int kStripMaxChannelsPadded = 104, kStripMaxChannels = 142;
 
-// Everything a wavefront with NB pixel blocks does (NB = 0: it only helps staging the weights).  A separate
-// instantiation per block count keeps the offsets and accumulators of absent blocks out of the register budget.
-template <int NB>
-__device__ __forceinline__ void strip_wave(const StripArgs &p, float *lds_w, int image, int oc0, int my_first, int tid)
-{
-    constexpr int DEPTH = NB >= kStripMaxBlocks ? 2 : 4;  // taps whose loads are in flight ahead of the MFMAs, plus one
-    constexpr int NBR = NB > 0 ? NB : 1;
-    const ConvShape &s = p.s;
-    const int lane = tid & 63, lh = lane >> 5, li = lane & 31;
-    const int K = s.c_in * kStripTaps;
-    const unsigned channel_bytes = static_cast<unsigned>(s.h) * s.w * 4u;
-    const unsigned pair_bytes = 2 * channel_bytes;
+inline int strip_pitch(int c_in) { return c_in <= kStripMaxChannelsPadded ? 12 : 9; }
+inline size_t strip_lds_bytes(int c_in) { return static_cast<size_t>(c_in) * 32 * strip_pitch(c_in) * 4 + 16; }
 
-    unsigned off[kStripTaps][NBR];
-    f32x16 acc[NBR];
-    if constexpr (NB > 0) {
-#pragma unroll
-        for (int blk = 0; blk < NB; ++blk) {
-            const int px = (my_first + blk) * 32 + li;
-            const bool valid = px < p.spatial;
-            const int oy = px / s.ow, ox = px - oy * s.ow;
-            const int iy0 = oy * s.stride_h - s.pad_h, ix0 = ox * s.stride_w - s.pad_w;
-#pragma unroll
-            for (int tap = 0; tap < kStripTaps; ++tap) {
-                const int ky = tap / s.kw, kx = tap - ky * s.kw;
-                const int iy = iy0 + ky * s.dil_h, ix = ix0 + kx * s.dil_w;
-                const bool inside = valid && static_cast<unsigned>(iy) < static_cast<unsigned>(s.h) &&
-                                    static_cast<unsigned>(ix) < static_cast<unsigned>(s.w);
-                off[tap][blk] = inside ? lh * channel_bytes + static_cast<unsigned>(iy * s.w + ix) * 4u : 0x80000000u;
-            }
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[blk][r] = 0.0f;
-        }
-    }
-    const size_t image_elems = static_cast<size_t>(s.c_in) * s.h * s.w;
-    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<float *>(p.input + static_cast<size_t>(image) * image_elems), 0, static_cast<int>(image_elems * 4), 0x00020000);
-    const float *a_lane = lds_w + (lh * 32 + li) * kStripTapPitch;
-    // One load per channel pair warms the caches for the pair after next: lane i of each half touches the i-th
-    // 128-byte line of the image rows this wavefront's pixels read (first-touch HBM latency is several times the
-    // distance the operand loads run ahead).
-    unsigned warm_off = 0x80000000u;
-    if constexpr (NB > 0) {
-        const int last_px = min(p.spatial, (my_first + NB) * 32) - 1;
-        const int iy_lo = max(0, (my_first * 32 / s.ow) * s.stride_h - s.pad_h);
-        const int iy_hi = min(s.h - 1, (last_px / s.ow) * s.stride_h - s.pad_h + (s.kh - 1) * s.dil_h);
-        const unsigned begin = static_cast<unsigned>(iy_lo) * s.w * 4u + li * 128u;
-        if (iy_hi >= iy_lo && begin < static_cast<unsigned>(iy_hi + 1) * s.w * 4u) warm_off = lh * channel_bytes + begin;
-    }
-
-    for (int c0 = 0; c0 < s.c_in; c0 += kStripChannels) {
-        const int channels = min(kStripChannels, s.c_in - c0);
-        // (Every wavefront of the workgroup passes these two barriers once per slice, whatever its NB.)
-        __syncthreads();  // all wavefronts are done with the previous slice's weights
-        const int row_values = channels * kStripTaps;
-        const float *slice = p.weight + static_cast<size_t>(c0) * kStripTaps;
-        if (row_values % 4 == 0 && K % 4 == 0 && (reinterpret_cast<uintptr_t>(p.weight) & 15u) == 0) {
-            // 128-bit reads, nine in flight per lane before the first is scattered into LDS.
-            constexpr int BATCH = 9;
-            const int per_row = row_values >> 2, total = 32 * per_row;
-            for (int first = 0; first < total; first += 512 * BATCH) {
-                float4 held[BATCH];
-#pragma unroll
-                for (int j = 0; j < BATCH; ++j) {
-                    const int v = first + j * 512 + tid;
-                    const int oc = v / per_row, q = v - oc * per_row;
-                    held[j] = (v < total && oc0 + oc < s.c_out)
-                                  ? *reinterpret_cast<const float4 *>(slice + static_cast<size_t>(oc0 + oc) * K + 4 * q)
-                                  : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-                }
-#pragma unroll
-                for (int j = 0; j < BATCH; ++j) {
-                    const int v = first + j * 512 + tid;
-                    if (v >= total) continue;
-                    const int oc = v / per_row, q = v - oc * per_row;
-                    const float values[4] = {held[j].x, held[j].y, held[j].z, held[j].w};
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const int r = 4 * q + e;
-                        const int ic = r / kStripTaps, tap = r - ic * kStripTaps;
-                        lds_w[(ic * 32 + oc) * kStripTapPitch + tap] = values[e];
-                    }
-                }
-            }
-        } else {
-            for (int e = tid; e < 32 * row_values; e += 512) {
-                const int oc = e / row_values, r = e - oc * row_values;
-                const int ic = r / kStripTaps, tap = r - ic * kStripTaps;
-                lds_w[(ic * 32 + oc) * kStripTapPitch + tap] =
-                    oc0 + oc < s.c_out ? slice[static_cast<size_t>(oc0 + oc) * K + r] : 0.0f;
-            }
-        }
-        __syncthreads();
-        if constexpr (NB > 0) {
-            const unsigned slice_bytes = static_cast<unsigned>(c0) * channel_bytes;
-            const int pairs = channels >> 1;
-            float b[DEPTH][NB];
-            f32x4 a[3];
-            auto load_b = [&](float (&dst)[NB], int tap, unsigned soff) {
-#pragma unroll
-                for (int blk = 0; blk < NB; ++blk)
-                    dst[blk] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, off[tap][blk], soff, 0));
-            };
-            auto load_a = [&](int q, int pair) {
-                a[q] = *reinterpret_cast<const f32x4 *>(a_lane + pair * (64 * kStripTapPitch) + 4 * q);
-            };
-            // One channel pair: nine taps.  The loads of tap t+DEPTH-1 are requested before the MFMAs of tap t, and
-            // each quarter of the weight registers is refilled for the next pair once its last tap has been issued.
-            // PHASE is the ring position of tap 0 (9 taps do not divide a ring of 2).
-            auto pair_body = [&](auto phase_tag, int pair) {
-                constexpr int PHASE = decltype(phase_tag)::value;
-                // (readfirstlane keeps the loop-carried scalar offsets in SGPRs; left to itself the compiler moves
-                // them to a VGPR and wraps every buffer load in a uniformity loop.)
-                const unsigned soff = __builtin_amdgcn_readfirstlane(slice_bytes + static_cast<unsigned>(pair) * pair_bytes);
-                const int following = pair + 1 < pairs ? pair + 1 : 0;  // past the end: re-read the first pair (unused)
-                const unsigned soff_next = __builtin_amdgcn_readfirstlane(slice_bytes + static_cast<unsigned>(following) * pair_bytes);
-                const int warm_pair = pair + 2 < pairs ? pair + 2 : 0;
-                const unsigned warm = __builtin_amdgcn_raw_buffer_load_b32(
-                    rsrc, warm_off, __builtin_amdgcn_readfirstlane(slice_bytes + static_cast<unsigned>(warm_pair) * pair_bytes), 0);
-#pragma unroll
-                for (int tap = 0; tap < kStripTaps; ++tap) {
-                    constexpr int AHEAD = DEPTH - 1;
-                    if (tap + AHEAD < kStripTaps) load_b(b[(PHASE + tap + AHEAD) % DEPTH], tap + AHEAD, soff);
-                    else load_b(b[(PHASE + tap + AHEAD) % DEPTH], tap + AHEAD - kStripTaps, soff_next);
-                    // (Scheduling fences: without them the compiler sinks each load to just before its use to save
-                    // registers, which leaves the loads no time to complete.)
-                    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                    for (int blk = 0; blk < NB; ++blk)
-                        acc[blk] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[tap >> 2][tap & 3], b[(PHASE + tap) % DEPTH][blk], acc[blk], 0, 0, 0);
-                    __builtin_amdgcn_sched_barrier(0);
-                    if (tap == 3) load_a(0, following);
-                    if (tap == 7) load_a(1, following);
-                    if (tap == 8) load_a(2, following);
-                }
-                asm volatile("" ::"v"(warm));  // keeps the warming load; every later load has been waited for by now
-            };
-            load_a(0, 0);
-            load_a(1, 0);
-            load_a(2, 0);
-#pragma unroll
-            for (int t = 0; t < DEPTH - 1; ++t) load_b(b[t], t, slice_bytes);
-            if constexpr (DEPTH == 3) {
-                for (int pair = 0; pair < pairs; ++pair) pair_body(std::integral_constant<int, 0>{}, pair);
-            } else if constexpr (DEPTH == 2) {
-                int pair = 0;
-                for (; pair + 2 <= pairs; pair += 2) {
-                    pair_body(std::integral_constant<int, 0>{}, pair);
-                    pair_body(std::integral_constant<int, 1>{}, pair + 1);
-                }
-                if (pair < pairs) pair_body(std::integral_constant<int, 0>{}, pair);
-            } else {
-                static_assert(DEPTH == 4);
-                int pair = 0;
-                for (; pair + 4 <= pairs; pair += 4) {
-                    pair_body(std::integral_constant<int, 0>{}, pair);
-                    pair_body(std::integral_constant<int, 1>{}, pair + 1);
-                    pair_body(std::integral_constant<int, 2>{}, pair + 2);
-                    pair_body(std::integral_constant<int, 3>{}, pair + 3);
-                }
-                if (pair < pairs) pair_body(std::integral_constant<int, 0>{}, pair);
-                if (pair + 1 < pairs) pair_body(std::integral_constant<int, 1>{}, pair + 1);
-                if (pair + 2 < pairs) pair_body(std::integral_constant<int, 2>{}, pair + 2);
-            }
-        }
-    }
-
-    if constexpr (NB > 0) {
-        float *out_image = p.out + static_cast<size_t>(image) * s.c_out * p.spatial;
-#pragma unroll
-        for (int blk = 0; blk < NB; ++blk) {
-            const int px = (my_first + blk) * 32 + li;
-            if (px >= p.spatial) continue;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int oc = oc0 + (r >> 2) * 8 + lh * 4 + (r & 3);
-                if (oc >= s.c_out) continue;
-                float value = acc[blk][r];
-                if (p.bias) value += p.bias[oc];
-                out_image[static_cast<size_t>(oc) * p.spatial + px] = apply_activation(value, p.activation);
-            }
-        }
-    }
-}
-
-__global__ __launch_bounds__(512) void conv2d_f32_strip_kernel(StripArgs p)
+template <int PITCH>
+__device__ __forceinline__ void conv2d_f32_strip_body(const StripArgs &p)
 {
     extern __shared__ __align__(16) unsigned char strip_lds[];
     float *lds_w = reinterpret_cast<float *>(strip_lds);
-    const int tid = threadIdx.x;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const ConvShape &s = p.s;
+    const int K = s.c_in * kStripTaps;
+    unsigned *counter = reinterpret_cast<unsigned *>(strip_lds + static_cast<size_t>(s.c_in) * 32 * PITCH * 4);
+    const int tid = threadIdx.x, lane = tid & 63, lh = lane >> 5, li = lane & 31;
     int bid = blockIdx.x;
     if (p.xcd_swizzle) bid = (bid & 7) * (p.total >> 3) + (bid >> 3);  // the workgroups of an image share an XCD's L2
     const int per_image = p.chunks * p.oc_strips;
@@ -713,39 +539,178 @@ __global__ __launch_bounds__(512) void conv2d_f32_strip_kernel(StripArgs p)
     const int oc0 = strip * 32;
     const int first = chunk * p.blocks_per_chunk;
     const int nblocks = min(p.blocks_per_chunk, p.blocks_per_image - first);
-    const int base = nblocks >> 3, rem = nblocks & 7;
-    const int my_count = base + (wave < rem ? 1 : 0);  // the same in all lanes of the wavefront: a scalar branch
-    const int my_first = first + wave * base + min(wave, rem);
-    switch (my_count) {
-    case 0: strip_wave<0>(p, lds_w, image, oc0, my_first, tid); break;
-    case 1: strip_wave<1>(p, lds_w, image, oc0, my_first, tid); break;
-    case 2: strip_wave<2>(p, lds_w, image, oc0, my_first, tid); break;
-    case 3: strip_wave<3>(p, lds_w, image, oc0, my_first, tid); break;
-    case 4: strip_wave<4>(p, lds_w, image, oc0, my_first, tid); break;
-    case 5: strip_wave<5>(p, lds_w, image, oc0, my_first, tid); break;
-    case 6: strip_wave<6>(p, lds_w, image, oc0, my_first, tid); break;
-    default: strip_wave<7>(p, lds_w, image, oc0, my_first, tid); break;
+
+    // Weights of the strip: LDS index of (oc, ic, tap) is (ic*32 + oc)*PITCH + tap, so that a lane's nine taps of a
+    // channel are consecutive and the 32 lanes of a half-wavefront sit PITCH words apart (no bank conflicts for 9 or 12).
+    if (K % 4 == 0 && (reinterpret_cast<uintptr_t>(p.weight) & 15u) == 0) {
+        constexpr int BATCH = 5;  // 128-bit reads in flight per lane before the first is scattered into LDS
+        const int per_row = K >> 2, total = 32 * per_row;
+        for (int base = 0; base < total; base += kStripThreads * BATCH) {
+            float4 held[BATCH];
+#pragma unroll
+            for (int j = 0; j < BATCH; ++j) {
+                const int v = base + j * kStripThreads + tid;
+                const int oc = v / per_row, q = v - oc * per_row;
+                held[j] = (v < total && oc0 + oc < s.c_out)
+                              ? *reinterpret_cast<const float4 *>(p.weight + static_cast<size_t>(oc0 + oc) * K + 4 * q)
+                              : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            }
+#pragma unroll
+            for (int j = 0; j < BATCH; ++j) {
+                const int v = base + j * kStripThreads + tid;
+                if (v >= total) continue;
+                const int oc = v / per_row, q = v - oc * per_row;
+                const float values[4] = {held[j].x, held[j].y, held[j].z, held[j].w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int r = 4 * q + e;
+                    const int ic = r / kStripTaps, tap = r - ic * kStripTaps;
+                    lds_w[(ic * 32 + oc) * PITCH + tap] = values[e];
+                }
+            }
+        }
+    } else {
+        for (int e = tid; e < 32 * K; e += kStripThreads) {
+            const int oc = e / K, r = e - oc * K;
+            const int ic = r / kStripTaps, tap = r - ic * kStripTaps;
+            lds_w[(ic * 32 + oc) * PITCH + tap] = oc0 + oc < s.c_out ? p.weight[static_cast<size_t>(oc0 + oc) * K + r] : 0.0f;
+        }
+    }
+    if (tid == 0) *counter = 0;
+    __syncthreads();
+
+    const unsigned channel_bytes = static_cast<unsigned>(s.h) * s.w * 4u;
+    const unsigned pair_bytes = 2 * channel_bytes;
+    const int pairs = s.c_in >> 1;
+    const size_t image_elems = static_cast<size_t>(s.c_in) * s.h * s.w;
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float *>(p.input + static_cast<size_t>(image) * image_elems), 0, static_cast<int>(image_elems * 4), 0x00020000);
+    const float *a_lane = lds_w + (lh * 32 + li) * PITCH;
+    float *out_image = p.out + static_cast<size_t>(image) * s.c_out * p.spatial;
+    float bias[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int oc = oc0 + (r >> 2) * 8 + lh * 4 + (r & 3);
+        bias[r] = (p.bias && oc < s.c_out) ? p.bias[oc] : 0.0f;
+    }
+
+    // Stagger: the four wavefronts that share a SIMD start a quarter of a block's duration apart.  Blocks all take
+    // the same time, so without this every wavefront of the chip would reach its load-latency and store phases at
+    // the same moment with nothing left to cover them; a sleeping wavefront costs nothing while the others keep the
+    // SIMD's matrix pipe full.  (One s_sleep(127) is 127·64 cycles; a block is pairs·9 MFMAs of 64 cycles, times four
+    // wavefronts.)
+    {
+        // Bits 3:0 of the hardware-id register (register 4): this wavefront's slot on its SIMD.
+        const int slot = static_cast<int>(__builtin_amdgcn_s_getreg(4 | (0 << 6) | (3 << 11))) & 3;
+        const int naps = (slot * pairs * kStripTaps + 63) / 127;
+        for (int i = 0; i < naps; ++i) __builtin_amdgcn_s_sleep(127);
+    }
+
+    for (;;) {
+        unsigned claimed = 0;
+        if (lane == 0) claimed = atomicAdd(counter, 1u);
+        const int blk = __builtin_amdgcn_readfirstlane(claimed);
+        if (blk >= nblocks) break;
+
+        const int px = (first + blk) * 32 + li;
+        const bool valid = px < p.spatial;
+        unsigned off[kStripTaps];
+        {
+            const int oy = px / s.ow, ox = px - oy * s.ow;
+            const int iy0 = oy * s.stride_h - s.pad_h, ix0 = ox * s.stride_w - s.pad_w;
+#pragma unroll
+            for (int tap = 0; tap < kStripTaps; ++tap) {
+                const int ky = tap / s.kw, kx = tap - ky * s.kw;
+                const int iy = iy0 + ky * s.dil_h, ix = ix0 + kx * s.dil_w;
+                const bool inside = valid && static_cast<unsigned>(iy) < static_cast<unsigned>(s.h) &&
+                                    static_cast<unsigned>(ix) < static_cast<unsigned>(s.w);
+                off[tap] = inside ? lh * channel_bytes + static_cast<unsigned>(iy * s.w + ix) * 4u : 0x80000000u;
+            }
+        }
+        f32x16 acc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+
+        auto load_b = [&](float (&dst)[kStripTaps], int pair) {
+            // (readfirstlane keeps the scalar offset in an SGPR; left to itself the compiler may move the
+            // loop-carried value to a VGPR and wrap every buffer load in a uniformity loop.)
+            const unsigned soff = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(pair) * pair_bytes);
+#pragma unroll
+            for (int tap = 0; tap < kStripTaps; ++tap)
+                dst[tap] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, off[tap], soff, 0));
+        };
+        auto load_a = [&](float (&dst)[kStripTaps], int pair) {
+            const float *src = a_lane + pair * (64 * PITCH);
+            if constexpr (PITCH == 12) {  // 16-byte aligned rows: three 128-bit reads
+#pragma unroll
+                for (int q = 0; q < 3; ++q) {
+                    const f32x4 v = *reinterpret_cast<const f32x4 *>(src + 4 * q);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (4 * q + e < kStripTaps) dst[4 * q + e] = v[e];
+                }
+            } else {
+#pragma unroll
+                for (int tap = 0; tap < kStripTaps; ++tap) dst[tap] = src[tap];
+            }
+        };
+        // One channel pair: the operands of the next pair are requested, then nine MFMAs run on this pair's.
+        // (Scheduling fences: without them the compiler sinks each load to just before its use to save registers,
+        // which leaves the loads no time to complete.)
+        auto pair_body = [&](const float (&a_use)[kStripTaps], const float (&b_use)[kStripTaps], float (&a_next)[kStripTaps],
+                             float (&b_next)[kStripTaps], int pair) {
+            const int following = pair + 1 < pairs ? pair + 1 : pair;  // past the end: re-read this pair (unused)
+            load_b(b_next, following);
+            load_a(a_next, following);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int tap = 0; tap < kStripTaps; ++tap)
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a_use[tap], b_use[tap], acc, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        float a0[kStripTaps], a1[kStripTaps], b0[kStripTaps], b1[kStripTaps];
+        load_b(b0, 0);
+        load_a(a0, 0);
+        int pair = 0;
+        for (; pair + 2 <= pairs; pair += 2) {
+            pair_body(a0, b0, a1, b1, pair);
+            pair_body(a1, b1, a0, b0, pair + 1);
+        }
+        if (pair < pairs) pair_body(a0, b0, a1, b1, pair);
+
+        if (valid) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int oc = oc0 + (r >> 2) * 8 + lh * 4 + (r & 3);
+                if (oc < s.c_out)
+                    out_image[static_cast<size_t>(oc) * p.spatial + px] = apply_activation(acc[r] + bias[r], p.activation);
+            }
+        }
     }
 }
+
+// (A kernel template loses its host-side launch stub with this compiler when its body uses some builtins, hence
+// plain kernels around the templated body.)
+__global__ __launch_bounds__(kStripThreads) void conv2d_f32_strip12_kernel(StripArgs p) { conv2d_f32_strip_body<12>(p); }
+__global__ __launch_bounds__(kStripThreads) void conv2d_f32_strip9_kernel(StripArgs p) { conv2d_f32_strip_body<9>(p); }
 
 // Splits `shape` into strip workgroups.  False when the shape does not fit the kernel, or (unless `forced`) when
 // the split would leave more than a fifth of the chip's SIMD time idle.
 bool plan_strip(const ConvShape &shape, bool forced, StripArgs &args)
 {
-    if (shape.kh * shape.kw != kStripTaps || shape.c_in % 2 != 0) return false;
+    if (shape.kh * shape.kw != kStripTaps || shape.c_in % 2 != 0 || shape.c_in > kStripMaxChannels) return false;
     const long long spatial = static_cast<long long>(shape.oh) * shape.ow;
     const long long blocks = (spatial + 31) / 32;
     const long long strips = (shape.c_out + 31) / 32;
-    long long chunks = (blocks + 55) / 56;
+    long long chunks = 1;
     while (shape.batch * strips * chunks < 256 && blocks / (chunks + 1) >= 16) ++chunks;
     const long long per_chunk = (blocks + chunks - 1) / chunks;
     chunks = (blocks + per_chunk - 1) / per_chunk;
     const long long total = shape.batch * strips * chunks;
     if (total > 0x7fffffff) return false;
-    // Cost in units of one 32×32 block per SIMD: workgroups take a compute unit each, two wavefronts per SIMD.
+    // Cost in 32×32 blocks per SIMD: one workgroup per compute unit at a time, its blocks spread over four SIMDs.
     const long long rounds = (total + 255) / 256;
-    const long long per_wave = (per_chunk + 7) / 8;
-    const double cost = static_cast<double>(rounds) * 2.0 * per_wave;
+    const double cost = static_cast<double>(rounds) * static_cast<double>((per_chunk + 3) / 4);
     const double ideal = static_cast<double>(shape.batch) * strips * blocks / 1024.0;
     if (!forced && ideal < 0.8 * cost) return false;
     args.spatial = static_cast<int>(spatial);
@@ -760,10 +725,12 @@ bool plan_strip(const ConvShape &shape, bool forced, StripArgs &args)
 
 hipError_t launch_strip(StripArgs args, hipStream_t stream)
 {
-    hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void *>(conv2d_f32_strip_kernel),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, kStripLdsBytes);
+    const size_t lds_bytes = strip_lds_bytes(args.s.c_in);
+    auto kernel = strip_pitch(args.s.c_in) == 12 ? conv2d_f32_strip12_kernel : conv2d_f32_strip9_kernel;
+    hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        static_cast<int>(lds_bytes));
     if (rc != hipSuccess) return rc;
-    hipLaunchKernelGGL(conv2d_f32_strip_kernel, dim3(static_cast<unsigned>(args.total)), dim3(512), kStripLdsBytes, stream, args);
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(args.total)), dim3(kStripThreads), lds_bytes, stream, args);
     return hipGetLastError();
 }
 
@@ -856,8 +823,13 @@ hipError_t launch_conv2d_f32(const ConvShape &shape, int activation, const float
     const bool force_ring = forced && std::strcmp(forced, "ring") == 0;
     const bool force_tile = forced && std::strcmp(forced, "tile") == 0;
     if (ring_ok && !force_tile) {
+        // The ring kernel has the better steady state (several rounds of 128×64 tiles per compute unit); the strip
+        // kernel, balanced to the single SIMD, wins when the ring kernel's tiles would fill the chip fewer than
+        // 1.75 times (1024 resident tiles) and for 64 or fewer output channels.
+        const long long ring_tiles = static_cast<long long>(shape.batch) * ((args.spatial + 63) / 64) * ((shape.c_out + 127) / 128);
+        const bool prefer_strip = force_strip || shape.c_out <= 64 || ring_tiles < 1792;
         StripArgs strip;
-        if (!force_ring && plan_strip(shape, force_strip, strip)) {
+        if (!force_ring && prefer_strip && plan_strip(shape, force_strip, strip)) {
             strip.input = input;
             strip.weight = weight;
             strip.bias = bias;
