@@ -58,15 +58,34 @@ __global__ __launch_bounds__(256) void conv_grad_bias_partial_kernel(int planes,
     if (lane == 0) partial[plane] = sum;
 }
 
-// out[i] = scale · Σ_c partial[c][i], chunks added in order.
+// out[i] = scale · Σ_c partial[c][i] in a fixed order: 16 outputs per workgroup, sixteen groups of lanes take every
+// sixteenth chunk (four loads in flight each) and their partial sums are added through LDS.
 __global__ __launch_bounds__(256) void conv_reduce_chunks_kernel(int chunks, size_t count, const float *partial, float scale,
                                                                  float *out)
 {
-    const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
-    if (i >= count) return;
-    float sum = 0.0f;
-    for (int c = 0; c < chunks; ++c) sum += partial[static_cast<size_t>(c) * count + i];
-    out[i] = sum * scale;
+    __shared__ float stage[16][17];
+    const int col = threadIdx.x & 15, sub = threadIdx.x >> 4;
+    const size_t i = static_cast<size_t>(blockIdx.x) * 16 + col;
+    float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (i < count) {
+        int c = sub;
+        for (; c + 48 < chunks; c += 64) {
+            float t[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) t[u] = partial[static_cast<size_t>(c + 16 * u) * count + i];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) sum[u] += t[u];
+        }
+        for (; c < chunks; c += 16) sum[0] += partial[static_cast<size_t>(c) * count + i];
+    }
+    stage[sub][col] = (sum[0] + sum[1]) + (sum[2] + sum[3]);
+    __syncthreads();
+    if (sub == 0 && i < count) {
+        float total = stage[0][col];
+#pragma unroll
+        for (int k = 1; k < 16; ++k) total += stage[k][col];
+        out[i] = total * scale;
+    }
 }
 
 typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
@@ -90,9 +109,11 @@ template <bool VEC>
 __global__ __launch_bounds__(256) void conv_grad_weight_kernel(GradWeightArgs p)
 {
     constexpr int BM = 64, BN = 64, BK = 16;
-    constexpr int A_STRIDE = BK + 4, B_STRIDE = BN + 8;
+    // Both tiles are kept pixel-contiguous (row = channel or patch column, 16 pixels + 4 words of padding), so that a
+    // lane's four k-values of either operand are one conflict-free 128-bit LDS read.
+    constexpr int A_STRIDE = BK + 4, B_STRIDE = BK + 4;
     __shared__ __attribute__((aligned(16))) float As[2][BM * A_STRIDE];
-    __shared__ __attribute__((aligned(16))) float Bs[2][BK * B_STRIDE];
+    __shared__ __attribute__((aligned(16))) float Bs[2][BN * B_STRIDE];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -202,22 +223,19 @@ __global__ __launch_bounds__(256) void conv_grad_weight_kernel(GradWeightArgs p)
     };
     auto store_lds = [&](int stage) {
         *reinterpret_cast<u32x4_t *>(&As[stage][a_row * A_STRIDE + a_c4]) = ra;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) Bs[stage][(prow0 + r) * B_STRIDE + (tid & 63)] = rb[r];
+        f32x4 packed;
+        packed[0] = rb[0]; packed[1] = rb[1]; packed[2] = rb[2]; packed[3] = rb[3];
+        *reinterpret_cast<f32x4 *>(&Bs[stage][(tid & 63) * B_STRIDE + prow0]) = packed;
     };
     auto compute = [&](int stage) {
         const float *as = As[stage];
         const float *bs = Bs[stage];
 #pragma unroll
         for (int kk = 0; kk < BK / 8; ++kk) {
-            const float4 av = *reinterpret_cast<const float4 *>(&as[(wm * 32 + li) * A_STRIDE + kk * 8 + lh * 4]);
-            float b[4];
+            const f32x4 av = *reinterpret_cast<const f32x4 *>(&as[(wm * 32 + li) * A_STRIDE + kk * 8 + lh * 4]);
+            const f32x4 bv = *reinterpret_cast<const f32x4 *>(&bs[(wn * 32 + li) * B_STRIDE + kk * 8 + lh * 4]);
 #pragma unroll
-            for (int t = 0; t < 4; ++t) b[t] = bs[(kk * 8 + lh * 4 + t) * B_STRIDE + wn * 32 + li];
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av.x, b[0], acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av.y, b[1], acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av.z, b[2], acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av.w, b[3], acc, 0, 0, 0);
+            for (int t = 0; t < 4; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[t], bv[t], acc, 0, 0, 0);
         }
     };
 
@@ -295,7 +313,7 @@ hipError_t launch_conv2d_grad_bias_f32(const ConvShape &shape, const float *grad
         rc = hipGetLastError();
         if (rc != hipSuccess) return rc;
     }
-    hipLaunchKernelGGL(conv_reduce_chunks_kernel, dim3(static_cast<unsigned>((shape.c_out + 255) / 256)), dim3(256), 0, stream,
+    hipLaunchKernelGGL(conv_reduce_chunks_kernel, dim3(static_cast<unsigned>((shape.c_out + 15) / 16)), dim3(256), 0, stream,
                        shape.batch, static_cast<size_t>(shape.c_out), partial, scale, grad_bias);
     return hipGetLastError();
 }
@@ -339,7 +357,7 @@ hipError_t launch_conv2d_grad_weight_f32(const ConvShape &shape, const float *in
         hipLaunchKernelGGL(conv_grad_weight_kernel<false>, grid, dim3(256), 0, stream, args);
     rc = hipGetLastError();
     if (rc != hipSuccess) return rc;
-    hipLaunchKernelGGL(conv_reduce_chunks_kernel, dim3(static_cast<unsigned>((count + 255) / 256)), dim3(256), 0, stream,
+    hipLaunchKernelGGL(conv_reduce_chunks_kernel, dim3(static_cast<unsigned>((count + 15) / 16)), dim3(256), 0, stream,
                        static_cast<int>(chunks), count, args.partial, scale, grad_weight);
     return hipGetLastError();
 }
