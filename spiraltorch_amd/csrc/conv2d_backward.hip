@@ -117,7 +117,7 @@ __global__ __launch_bounds__(256) void conv_grad_weight_kernel(GradWeightArgs p)
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: the pixel bookkeeping below stays off the VALU
     const int wm = wave >> 1, wn = wave & 1;
     const int li = lane & 31, lh = lane >> 5;
     const ConvShape &s = p.s;
@@ -143,7 +143,7 @@ __global__ __launch_bounds__(256) void conv_grad_weight_kernel(GradWeightArgs p)
     const int ky = rem / s.kw, kx = rem - ky * s.kw;
     const int dy = ky * s.dil_h - s.pad_h, dx = kx * s.dil_w - s.pad_w;
     const int tap_offset = ic * H * W;
-    const int prow0 = (tid >> 6) * 4;  // patch rows prow0 .. prow0+3 of a step: four consecutive pixels
+    const int prow0 = wave * 4;  // patch rows prow0 .. prow0+3 of a step: four consecutive pixels, the same for all lanes
 
     // G tile: thread loads 4 consecutive pixels of one channel row.
     const int a_row = tid >> 2, a_c4 = (tid & 3) * 4;
@@ -194,7 +194,25 @@ __global__ __launch_bounds__(256) void conv_grad_weight_kernel(GradWeightArgs p)
                 ra[e] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_g, off, 0, 0);
             }
         }
+        // The four pixels are the same for every lane of the wavefront (lanes differ in their tap), so whether they
+        // sit in one image row is a scalar question.  If they do, and no lane's tap straddles the left or right
+        // border, the four values are one 128-bit load (dword-aligned is enough for buffer loads).
+        const bool one_row = s.stride_w == 1 && ox + 3 < s.ow && p0 + prow0 + 3 < p.spatial;
+        bool vector_done = false;
+        if (one_row) {
+            const int iy = oy * s.stride_h + dy, ix0 = ox + dx;
+            const bool row_ok = col_valid && static_cast<unsigned>(iy) < static_cast<unsigned>(H);
+            const bool full = row_ok && ix0 >= 0 && ix0 + 3 < W;
+            if (__builtin_amdgcn_ballot_w64(row_ok && !full) == 0) {
+                const unsigned off = full ? static_cast<unsigned>(tap_offset + iy * W + ix0) * 4u : kOutside;
+                const u32x4_t raw = __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, off, 0, 0);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) rb[r] = __uint_as_float(raw[r]);
+                vector_done = true;
+            }
+        }
         int py = oy, px = ox;
+        if (!vector_done)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int iy = py * s.stride_h + dy, ix = px * s.stride_w + dx;
