@@ -287,7 +287,8 @@ def main():
     args = parser.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (every op shards into independent "
-              "units; see DESIGN.md). Run with --gpus 1.", file=sys.stderr)
+              "units: GEMM by row blocks, conv by image, attention by context, the decoder by batch). "
+              "Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
 
     from spiraltorch_amd import hip, inputs
