@@ -13,8 +13,11 @@
 // column, so the running maximum and sum are per-lane scalars and the probabilities leave the first
 // product's accumulators already in the register layout the second product's B operand needs (no
 // shuffle, no LDS round trip).  The accumulator of a 32x32 tile hands lane half h the keys
-// {8a + 4h + c}; the second product wants eight consecutive k-indices per lane, so V is staged
-// transposed with key bits 2 and 3 swapped, which makes those eight keys one 128-bit LDS read.
+// {8a + 4h + c}; the second product wants eight k-indices per lane, so its Vᵀ operand takes keys
+// 16j + 4h + {0..3} and 16j + 8 + 4h + {0..3}: V is staged exactly as it is stored (rows = keys, one 128-bit
+// LDS write per 128-bit load) and those two groups of four keys are fetched with the transposing LDS read
+// (ds_read_b64_tr_b16).  (Transposing while staging — eight 16-bit scattered writes per load — spent two thirds
+// of the LDS cycles on bank conflicts.)
 #include "device_math.h"
 #include "kernels.h"
 
@@ -42,6 +45,7 @@ constexpr float kLog2e16 = 1.4426950408889634f;
 typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef s16x4 __attribute__((address_space(3))) *lds_s16x4_ptr;
 
 __device__ __forceinline__ unsigned pack_bf16x2(float lo, float hi)
 {
@@ -54,14 +58,14 @@ __global__ __launch_bounds__(256) void attention_bf16_kernel(AttnBf16Args p)
 {
     constexpr int BKV = 64;
     constexpr int KS = D + 8;      // K row stride (elements): 16 bytes of padding keep 128-bit reads conflict-free
-    constexpr int VTS = BKV + 8;   // Vt row stride: rows are head-dim indices, columns (permuted) keys
-    constexpr int K_ELEMS = BKV * KS, V_ELEMS = D * VTS;
+    constexpr int VS = D + 8;      // V row stride: V is staged as it is stored (rows = keys) and read transposed
+    constexpr int K_ELEMS = BKV * KS, V_ELEMS = BKV * VS;
     constexpr int KC = D / 16;     // k-blocks of K·Qᵀ
     constexpr int DT = D / 32;     // 32-row tiles of Oᵀ
     constexpr int LOADS = BKV * D / 8 / 256;
     extern __shared__ __attribute__((aligned(16))) uint16_t attn16_lds[];
     uint16_t *Ks = attn16_lds;                // [2][K_ELEMS]
-    uint16_t *Vt = attn16_lds + 2 * K_ELEMS;  // [2][V_ELEMS]
+    uint16_t *Vs = attn16_lds + 2 * K_ELEMS;  // [2][V_ELEMS]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -138,27 +142,26 @@ __global__ __launch_bounds__(256) void attention_bf16_kernel(AttnBf16Args p)
     };
     auto store_lds = [&](int stage) {
         uint16_t *ks = Ks + stage * K_ELEMS;
-        uint16_t *vt = Vt + stage * V_ELEMS;
+        uint16_t *vs = Vs + stage * V_ELEMS;
 #pragma unroll
         for (int r = 0; r < LOADS; ++r) {
             const int f = tid + 256 * r;
             const int row = f / (D / 8), c8 = (f % (D / 8)) * 8;
             *reinterpret_cast<u32x4_t *>(&ks[row * KS + c8]) = rk[r];
-            const int pos = (row & ~12) | ((row & 4) << 1) | ((row & 8) >> 1);  // key bits 2 and 3 swapped
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                vt[(c8 + 2 * e + 0) * VTS + pos] = static_cast<uint16_t>(rv[r][e] & 0xffffu);
-                vt[(c8 + 2 * e + 1) * VTS + pos] = static_cast<uint16_t>(rv[r][e] >> 16);
-            }
+            *reinterpret_cast<u32x4_t *>(&vs[row * VS + c8]) = rv[r];
         }
     };
+    // Transpose-read lane roles (ds_read_b64_tr_b16): within each 16-lane group lane i16 supplies the address of
+    // row i16/4 and 4-column chunk i16%4 of a 4×16 block and receives column i16 of it (4 rows).
+    const int i16 = lane & 15, c16 = (lane >> 4) & 1;
+    const int v_read = (lh * 4 + (i16 >> 2)) * VS + c16 * 16 + (i16 & 3) * 4;
 
     const float scale_log2e = p.scale * kLog2e16;
     // NT = number of 32-key tiles of this stage this wavefront works on (1 or 2).
     auto compute = [&](auto nt_tag, int stage, int key0) {
         constexpr int NT = decltype(nt_tag)::value;
         const uint16_t *ks = Ks + stage * K_ELEMS;
-        const uint16_t *vt = Vt + stage * V_ELEMS;
+        const uint16_t *vs = Vs + stage * V_ELEMS;
         f32x16 sacc[NT];
 #pragma unroll
         for (int t = 0; t < NT; ++t)
@@ -218,7 +221,9 @@ __global__ __launch_bounds__(256) void attention_bf16_kernel(AttnBf16Args p)
                 tile_sum += pr;
             }
         run_sum += tile_sum;
-        // Oᵀ += Vᵀ·Pᵀ, 16 keys per MFMA: accumulator registers 8j .. 8j+7 are this lane's k-indices 8·lh .. 8·lh+7.
+        // Oᵀ += Vᵀ·Pᵀ, 16 keys per MFMA: accumulator registers 8j .. 8j+7 are this lane's k-indices 8·lh .. 8·lh+7,
+        // which are keys 16j + 4·lh + {0..3} and 16j + 8 + 4·lh + {0..3}; the Vᵀ operand is gathered to match with
+        // two transposing reads (4 keys × 16 head-dim columns per 16-lane group each).
 #pragma unroll
         for (int t = 0; t < NT; ++t)
 #pragma unroll
@@ -229,8 +234,12 @@ __global__ __launch_bounds__(256) void attention_bf16_kernel(AttnBf16Args p)
                 const bf16x8 pf = __builtin_bit_cast(bf16x8, packed);
                 bf16x8 vf[DT];
 #pragma unroll
-                for (int dt = 0; dt < DT; ++dt)
-                    vf[dt] = *reinterpret_cast<const bf16x8 *>(&vt[(dt * 32 + li) * VTS + t * 32 + j * 16 + lh * 8]);
+                for (int dt = 0; dt < DT; ++dt) {
+                    const uint16_t *src = &vs[(t * 32 + j * 16) * VS + v_read + dt * 32];
+                    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(src));
+                    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(src + 8 * VS));
+                    vf[dt] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+                }
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[dt], pf, oacc[dt], 0, 0, 0);
             }
@@ -273,7 +282,7 @@ __global__ __launch_bounds__(256) void attention_bf16_kernel(AttnBf16Args p)
 template <int D, bool CAUSAL>
 hipError_t launch_variant(const AttnBf16Args &args, hipStream_t stream)
 {
-    constexpr size_t lds_bytes = 2 * (static_cast<size_t>(64) * (D + 8) + static_cast<size_t>(D) * (64 + 8)) * sizeof(uint16_t);
+    constexpr size_t lds_bytes = 2 * (static_cast<size_t>(64) * (D + 8) + static_cast<size_t>(64) * (D + 8)) * sizeof(uint16_t);
     auto kernel = attention_bf16_kernel<D, CAUSAL>;
     hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
