@@ -54,7 +54,7 @@ __device__ __forceinline__ unsigned pack_bf16x2(float lo, float hi)
 }
 
 template <int D, bool CAUSAL>
-__global__ __launch_bounds__(256) void attention_bf16_kernel(AttnBf16Args p)
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 64 ? 4 : 2, D == 64 ? 4 : 2))) void attention_bf16_kernel(AttnBf16Args p)
 {
     constexpr int BKV = 64;
     constexpr int KS = D + 8;      // K row stride (elements): 16 bytes of padding keep 128-bit reads conflict-free
@@ -118,7 +118,13 @@ __global__ __launch_bounds__(256) void attention_bf16_kernel(AttnBf16Args p)
     // Qᵀ fragments (B operand): lane (li, lh) holds Q[my_q][16c + 8·lh .. +7].
     bf16x8 qf[KC];
 #pragma unroll
-    for (int c = 0; c < KC; ++c) qf[c] = __builtin_bit_cast(bf16x8, fetch8(rsrc_q, my_q, c * 16 + lh * 8));
+    for (int c = 0; c < KC; ++c) {
+        // A negative scale is moved into Q (sign bits flipped) so that the scale applied below is never negative
+        // and the running maximum can be taken over the raw dot products.
+        u32x4_t raw = fetch8(rsrc_q, my_q, c * 16 + lh * 8);
+        if (p.scale < 0.0f) raw ^= 0x80008000u;
+        qf[c] = __builtin_bit_cast(bf16x8, raw);
+    }
 
     f32x16 oacc[DT];
 #pragma unroll
@@ -156,7 +162,9 @@ __global__ __launch_bounds__(256) void attention_bf16_kernel(AttnBf16Args p)
     const int i16 = lane & 15, c16 = (lane >> 4) & 1;
     const int v_read = (lh * 4 + (i16 >> 2)) * VS + c16 * 16 + (i16 & 3) * 4;
 
-    const float scale_log2e = p.scale * kLog2e16;
+    // (Floored at a tiny positive value so that a zero scale still turns masked (-inf) logits into weight 0
+    // instead of -inf·0.)
+    const float scale_log2e = fmaxf(fabsf(p.scale) * kLog2e16, 1e-30f);
     // NT = number of 32-key tiles of this stage this wavefront works on (1 or 2).
     auto compute = [&](auto nt_tag, int stage, int key0) {
         constexpr int NT = decltype(nt_tag)::value;
@@ -175,7 +183,9 @@ __global__ __launch_bounds__(256) void attention_bf16_kernel(AttnBf16Args p)
 #pragma unroll
             for (int t = 0; t < NT; ++t) sacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[t], qf[c], sacc[t], 0, 0, 0);
         }
-        // logits in log2 units; masking only where a tile crosses the sequence end or the diagonal
+        // The running maximum is kept in units of the raw dot product (scale >= 0 here), so the scale costs no pass
+        // of its own: p = exp2(dot·scale·log2e − max·scale·log2e) is one fused multiply-add and one exp2.  Masking
+        // only where a tile crosses the sequence end or the diagonal.
         const bool need_mask = (key0 + NT * 32 > S) || (CAUSAL && key0 + NT * 32 - 1 > wq0);
         float tile_max = -INFINITY;
         if (need_mask) {
@@ -184,7 +194,7 @@ __global__ __launch_bounds__(256) void attention_bf16_kernel(AttnBf16Args p)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int key = key0 + t * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
-                    float v = sacc[t][r] * scale_log2e;
+                    float v = sacc[t][r];
                     if (key >= S || (CAUSAL && key > my_q)) v = -INFINITY;
                     sacc[t][r] = v;
                     tile_max = fmaxf(tile_max, v);
@@ -193,17 +203,14 @@ __global__ __launch_bounds__(256) void attention_bf16_kernel(AttnBf16Args p)
 #pragma unroll
             for (int t = 0; t < NT; ++t)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const float v = sacc[t][r] * scale_log2e;
-                    sacc[t][r] = v;
-                    tile_max = fmaxf(tile_max, v);
-                }
+                for (int r = 0; r < 16; ++r) tile_max = fmaxf(tile_max, sacc[t][r]);
         }
         tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32));
         const float new_max = fmaxf(run_max, tile_max);
         const float safe_max = new_max == -INFINITY ? 0.0f : new_max;
+        const float shift = -safe_max * scale_log2e;
         if (__any(new_max != run_max)) {  // wavefront-uniform: some query's maximum moved
-            const float alpha = __builtin_amdgcn_exp2f(run_max - safe_max);  // run_max = -inf -> 0
+            const float alpha = __builtin_amdgcn_exp2f(fmaf(run_max, scale_log2e, shift));  // run_max = -inf -> 0
             run_sum *= alpha;
 #pragma unroll
             for (int t = 0; t < DT; ++t)
@@ -216,7 +223,7 @@ __global__ __launch_bounds__(256) void attention_bf16_kernel(AttnBf16Args p)
         for (int t = 0; t < NT; ++t)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const float pr = __builtin_amdgcn_exp2f(sacc[t][r] - safe_max);
+                const float pr = __builtin_amdgcn_exp2f(fmaf(sacc[t][r], scale_log2e, shift));
                 sacc[t][r] = pr;
                 tile_sum += pr;
             }

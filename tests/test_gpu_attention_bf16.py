@@ -51,6 +51,18 @@ def test_fused_qkv_layout(hip, oracle, batch, heads, seq, dim, causal):
     assert_close(got, want, BF16_REL, ABS, f"bf16 attention b{batch} h{heads} s{seq} d{dim} causal={causal}")
 
 
+@pytest.mark.parametrize("scale", [-0.2, 0.0, 3.0])
+@pytest.mark.parametrize("causal", [False, True])
+def test_unusual_scales(hip, oracle, scale, causal):
+    """Negative, zero and large scales (the kernel folds |scale| into the exponent and moves the sign into Q)."""
+    batch, heads, seq, dim = 1, 2, 97, 64
+    rng = np.random.default_rng(int(scale * 10) + 100 + causal)
+    qkv_bits = inputs.to_bf16((rng.normal(size=batch * seq * 3 * heads * dim) * 0.5).astype(np.float32))
+    got = run_fused(hip, batch, heads, seq, dim, scale, qkv_bits, causal)
+    want = oracle_fused(oracle, batch, heads, seq, dim, scale, qkv_bits, causal)
+    assert_close(got, want, BF16_REL, ABS, f"bf16 attention scale={scale} causal={causal}")
+
+
 def test_contiguous_contexts_and_row_sums(hip, oracle):
     """heads = 1, ld = head_dim is the (contexts*seq, head_dim) layout of the f32 entry point; V = 1 must give
     rows that sum to one (every output element equals 1 up to the bf16 rounding of the result)."""
