@@ -165,6 +165,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 64 ? 4
     // (Floored at a tiny positive value so that a zero scale still turns masked (-inf) logits into weight 0
     // instead of -inf·0.)
     const float scale_log2e = fmaxf(fabsf(p.scale) * kLog2e16, 1e-30f);
+    const float lag = 8.0f / scale_log2e;  // 2^8 in units of the raw dot product
     // NT = number of 32-key tiles of this stage this wavefront works on (1 or 2).
     auto compute = [&](auto nt_tag, int stage, int key0) {
         constexpr int NT = decltype(nt_tag)::value;
@@ -206,11 +207,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 64 ? 4
                 for (int r = 0; r < 16; ++r) tile_max = fmaxf(tile_max, sacc[t][r]);
         }
         tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32));
-        const float new_max = fmaxf(run_max, tile_max);
-        const float safe_max = new_max == -INFINITY ? 0.0f : new_max;
-        const float shift = -safe_max * scale_log2e;
-        if (__any(new_max != run_max)) {  // wavefront-uniform: some query's maximum moved
-            const float alpha = __builtin_amdgcn_exp2f(fmaf(run_max, scale_log2e, shift));  // run_max = -inf -> 0
+        // The reference maximum in the exponent is allowed to lag the true running maximum by up to 2^8 (weights then
+        // reach 256 instead of 1, harmless in f32 and bf16); the accumulators are rescaled only when some query's
+        // maximum has moved by more than that, which after the first key tiles is rare.
+        if (__any(tile_max > run_max + lag)) {  // wavefront-uniform
+            const float new_max = fmaxf(run_max, tile_max);
+            const float new_safe = new_max == -INFINITY ? 0.0f : new_max;
+            const float alpha = __builtin_amdgcn_exp2f((run_max - new_safe) * scale_log2e);  // run_max = -inf -> 0
             run_sum *= alpha;
 #pragma unroll
             for (int t = 0; t < DT; ++t)
@@ -218,6 +221,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 64 ? 4
                 for (int r = 0; r < 16; ++r) oacc[t][r] *= alpha;
             run_max = new_max;
         }
+        const float safe_max = run_max == -INFINITY ? 0.0f : run_max;
+        const float shift = -safe_max * scale_log2e;
         float tile_sum = 0.0f;
 #pragma unroll
         for (int t = 0; t < NT; ++t)
