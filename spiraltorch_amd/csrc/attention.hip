@@ -337,6 +337,11 @@ __global__ __launch_bounds__(256) void attention_f32_fast_kernel(AttnArgs p)
     for (int c = 0; c < CHUNKS; ++c) {
         const float4 v = fetch4(rsrc_q, my_q, c * 8 + lh * 4);
         qf[c][0] = v.x; qf[c][1] = v.y; qf[c][2] = v.z; qf[c][3] = v.w;
+        // A negative scale is moved into Q so that the scale applied below is never negative and the running
+        // maximum can be taken over the raw dot products.
+        if (p.scale < 0.0f) {
+            qf[c][0] = -qf[c][0]; qf[c][1] = -qf[c][1]; qf[c][2] = -qf[c][2]; qf[c][3] = -qf[c][3];
+        }
     }
 
     f32x16 oacc[DT];
@@ -374,7 +379,11 @@ __global__ __launch_bounds__(256) void attention_f32_fast_kernel(AttnArgs p)
         }
     };
 
-    const float scale_log2e = p.scale * kLog2e;
+    // The maximum is kept in units of the raw dot product and the scale is folded into the exponent:
+    // p = exp2(fma(dot, scale·log2e, −max·scale·log2e)).  (Floored at a tiny positive value so that a zero scale
+    // still turns masked (−inf) logits into weight 0 instead of −inf·0.)
+    const float scale_log2e = fmaxf(fabsf(p.scale) * kLog2e, 1e-30f);
+    const float lag = 8.0f / scale_log2e;  // 2^8 in units of the raw dot product, see below
     // NT = number of 32-key tiles of this stage this wavefront works on (1 or 2).
     auto compute = [&](auto nt_tag, int stage, int key0) {
         constexpr int NT = decltype(nt_tag)::value;
@@ -406,7 +415,7 @@ __global__ __launch_bounds__(256) void attention_f32_fast_kernel(AttnArgs p)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int key = key0 + t * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
-                    float v = sacc[t][r] * scale_log2e;
+                    float v = sacc[t][r];
                     if (key >= S || (CAUSAL && key > my_q)) v = -INFINITY;
                     sacc[t][r] = v;
                     tile_max = fmaxf(tile_max, v);
@@ -415,17 +424,16 @@ __global__ __launch_bounds__(256) void attention_f32_fast_kernel(AttnArgs p)
 #pragma unroll
             for (int t = 0; t < NT; ++t)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const float v = sacc[t][r] * scale_log2e;
-                    sacc[t][r] = v;
-                    tile_max = fmaxf(tile_max, v);
-                }
+                for (int r = 0; r < 16; ++r) tile_max = fmaxf(tile_max, sacc[t][r]);
         }
         tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32));
-        const float new_max = fmaxf(run_max, tile_max);
-        const float safe_max = new_max == -INFINITY ? 0.0f : new_max;
-        if (__any(new_max != run_max)) {  // wavefront-uniform: some row's maximum moved
-            const float alpha = __builtin_amdgcn_exp2f(run_max - safe_max);  // run_max = -inf -> 0
+        // The reference maximum in the exponent may lag the true running maximum by up to 2^8 (weights then reach
+        // 256 instead of 1, which changes nothing in f32 but the exponent); the accumulators are rescaled only when
+        // some row's maximum has moved by more than that, which after the first key tiles is rare.
+        if (__any(tile_max > run_max + lag)) {  // wavefront-uniform
+            const float new_max = fmaxf(run_max, tile_max);
+            const float new_safe = new_max == -INFINITY ? 0.0f : new_max;
+            const float alpha = __builtin_amdgcn_exp2f((run_max - new_safe) * scale_log2e);  // run_max = -inf -> 0
             run_sum *= alpha;
 #pragma unroll
             for (int t = 0; t < DT; ++t)
@@ -433,12 +441,14 @@ __global__ __launch_bounds__(256) void attention_f32_fast_kernel(AttnArgs p)
                 for (int r = 0; r < 16; ++r) oacc[t][r] *= alpha;
             run_max = new_max;
         }
+        const float safe_max = run_max == -INFINITY ? 0.0f : run_max;
+        const float shift = -safe_max * scale_log2e;
         float tile_sum = 0.0f;
 #pragma unroll
         for (int t = 0; t < NT; ++t)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const float pr = __builtin_amdgcn_exp2f(sacc[t][r] - safe_max);
+                const float pr = __builtin_amdgcn_exp2f(fmaf(sacc[t][r], scale_log2e, shift));
                 sacc[t][r] = pr;
                 tile_sum += pr;
             }

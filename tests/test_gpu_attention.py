@@ -47,6 +47,21 @@ def test_random_cases(hip, oracle, contexts, seq, dim, causal, biased):
     assert_close(ones, np.ones_like(ones), F32_REL, F32_ABS, "row sums")
 
 
+@pytest.mark.parametrize("scale", [-0.3, 0.0, 2.5])
+@pytest.mark.parametrize("causal", [False, True])
+def test_unusual_scales(hip, oracle, scale, causal):
+    """Negative, zero and large scales on the fast path (|scale| is folded into the exponent, the sign into Q; a large
+    scale makes running maxima jump by more than the lag the kernel tolerates before rescaling)."""
+    contexts, seq, dim = 2, 150, 64
+    rng = np.random.default_rng(int(scale * 10) + 50 + causal)
+    q, k, v = (rng.normal(size=contexts * seq * dim).astype(np.float32) for _ in range(3))
+    got = run(hip, contexts, seq, dim, scale, q, k, v, None, None, causal)
+    want = oracle.attention_f32(contexts, seq, dim, scale, q, k, v, None, None, causal, threads=8)
+    assert_close(got, want, F32_REL, F32_ABS, f"attention scale={scale} causal={causal}")
+    ones = run(hip, contexts, seq, dim, scale, q, k, np.ones_like(v), None, None, causal)
+    assert_close(ones, np.ones_like(ones), F32_REL, F32_ABS, "row sums")
+
+
 def test_invariants(hip, oracle):
     rng = np.random.default_rng(5)
     contexts, seq, dim = 3, 150, 64
