@@ -54,7 +54,7 @@ __device__ __forceinline__ unsigned pack_bf16x2(float lo, float hi)
 }
 
 template <int D, bool CAUSAL>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 64 ? 4 : 2, D == 64 ? 4 : 2))) void attention_bf16_kernel(AttnBf16Args p)
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 64 ? (CAUSAL ? 4 : 3) : 2, D == 64 ? (CAUSAL ? 4 : 3) : 2))) void attention_bf16_kernel(AttnBf16Args p)
 {
     constexpr int BKV = 64;
     constexpr int KS = D + 8;      // K row stride (elements): 16 bytes of padding keep 128-bit reads conflict-free
