@@ -101,19 +101,20 @@ struct GradWeightArgs {
     int steps_per_chunk;       // 16-pixel steps (numbered image by image) per workgroup
 };
 
-// One workgroup: a 64 (output channels) × 64 (reduction columns s) tile of grad_weight, summed over the pixels of
-// its images.  Per 16-pixel step the G tile (64 × 16, pixel-contiguous in NCHW) and the patch tile (16 × 64, gathered:
-// thread owns one column s, whose channel/tap offset is fixed for the whole kernel) are fetched into registers while
-// the MFMAs of the previous step run, then written to the other LDS stage.
-template <bool VEC>
-__global__ __launch_bounds__(256) void conv_grad_weight_kernel(GradWeightArgs p)
+// One workgroup: a (64·TM output channels) × (64·TN reduction columns s) tile of grad_weight, summed over the pixels
+// of its images; four wavefronts in a 2×2 arrangement, each owning TM×TN 32×32 accumulators.  Per 16-pixel step the G
+// tile (pixel-contiguous in NCHW) and the patch tile (gathered: a thread owns TN columns s, whose channel/tap offsets
+// are fixed for the whole kernel) are fetched into registers while the MFMAs of the previous step run, then written to
+// the other LDS stage.  The big tile (TM = 2, TN = 3: 128 × 192, three of which span a 3×3 layer's 576 columns exactly
+// for 64 input channels) reads 5 fragments per 24 MFMAs instead of 2 per 4.
+template <bool VEC, int TM, int TN>
+__device__ __forceinline__ void conv_grad_weight_body(const GradWeightArgs &p, float *As, float *Bs)
 {
-    constexpr int BM = 64, BN = 64, BK = 16;
+    constexpr int BM = 64 * TM, BN = 64 * TN, BK = 16;
     // Both tiles are kept pixel-contiguous (row = channel or patch column, 16 pixels + 4 words of padding), so that a
     // lane's four k-values of either operand are one conflict-free 128-bit LDS read.
     constexpr int A_STRIDE = BK + 4, B_STRIDE = BK + 4;
-    __shared__ __attribute__((aligned(16))) float As[2][BM * A_STRIDE];
-    __shared__ __attribute__((aligned(16))) float Bs[2][BN * B_STRIDE];
+    constexpr int A_STAGE = BM * A_STRIDE, B_STAGE = BN * B_STRIDE;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -134,34 +135,41 @@ __global__ __launch_bounds__(256) void conv_grad_weight_kernel(GradWeightArgs p)
     const int chunk = bid / tiles_oc;
     const int oc0 = tile_oc * BM, s0 = tile_s * BN;
 
-    // This thread's patch column and its fixed tap.
-    const int col = s0 + (tid & 63);
-    const bool col_valid = col < p.S;
+    // This thread's patch columns (lane + 64·j) and their fixed taps.
     const int khw = s.kh * s.kw;
-    const int ic = col_valid ? col / khw : 0;
-    const int rem = col_valid ? col - ic * khw : 0;
-    const int ky = rem / s.kw, kx = rem - ky * s.kw;
-    const int dy = ky * s.dil_h - s.pad_h, dx = kx * s.dil_w - s.pad_w;
-    const int tap_offset = ic * H * W;
+    bool col_valid[TN];
+    int dy[TN], dx[TN], tap_offset[TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const int col = s0 + j * 64 + lane;
+        col_valid[j] = col < p.S;
+        const int ic = col_valid[j] ? col / khw : 0;
+        const int rem = col_valid[j] ? col - ic * khw : 0;
+        const int ky = rem / s.kw, kx = rem - ky * s.kw;
+        dy[j] = ky * s.dil_h - s.pad_h;
+        dx[j] = kx * s.dil_w - s.pad_w;
+        tap_offset[j] = ic * H * W;
+    }
     const int prow0 = wave * 4;  // patch rows prow0 .. prow0+3 of a step: four consecutive pixels, the same for all lanes
 
-    // G tile: thread loads 4 consecutive pixels of one channel row.
+    // G tile: a thread loads 4 consecutive pixels of the channel rows a_row + 64·i.
     const int a_row = tid >> 2, a_c4 = (tid & 3) * 4;
-    const bool a_row_valid = oc0 + a_row < s.c_out;
 
-    f32x16 acc;
+    f32x16 acc[TM][TN];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
     const int steps_per_image = (p.spatial + BK - 1) / BK;
     const int first_step = chunk * p.steps_per_chunk;
     const int total_steps = max(0, min(s.batch * steps_per_image, first_step + p.steps_per_chunk) - first_step);
 
-    // (oy, ox) of this thread's first pixel of the step being loaded, advanced by 16 pixels per step without
-    // divisions (integer division costs about twenty vector instructions, and on this chip every vector
-    // instruction takes time from the f32 matrix pipe).  Memory is addressed through per-image buffer descriptors
-    // with 32-bit offsets; anything outside (padding, pixels past the end, channels past C_out) gets an
-    // out-of-range offset and reads as zero.
+    // (oy, ox) of this wavefront's first pixel of the step being loaded, advanced by 16 pixels per step without
+    // divisions.  Memory is addressed through per-image buffer descriptors with 32-bit offsets; anything outside
+    // (padding, pixels past the end, channels past C_out) gets an out-of-range offset and reads as zero.
     int load_image = first_step / steps_per_image, load_step = first_step - load_image * steps_per_image;
     int oy, ox;
     {
@@ -172,10 +180,13 @@ __global__ __launch_bounds__(256) void conv_grad_weight_kernel(GradWeightArgs p)
     const unsigned image_bytes = static_cast<unsigned>(s.c_in) * H * W * 4u;
     const unsigned grad_bytes = static_cast<unsigned>(s.c_out) * p.spatial * 4u;
     constexpr unsigned kOutside = 0x80000000u;
-    const unsigned a_base = a_row_valid ? (static_cast<unsigned>(oc0 + a_row) * p.spatial + a_c4) * 4u : kOutside;
+    unsigned a_base[TM];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+        a_base[i] = oc0 + a_row + 64 * i < s.c_out ? (static_cast<unsigned>(oc0 + a_row + 64 * i) * p.spatial + a_c4) * 4u : kOutside;
 
-    u32x4_t ra;
-    float rb[4];
+    u32x4_t ra[TM];
+    float rb[TN][4];
     auto load_global = [&]() {
         const int p0 = load_step * BK;
         const __amdgpu_buffer_rsrc_t rsrc_g = __builtin_amdgcn_make_buffer_rsrc(
@@ -184,45 +195,53 @@ __global__ __launch_bounds__(256) void conv_grad_weight_kernel(GradWeightArgs p)
         const __amdgpu_buffer_rsrc_t rsrc_x = __builtin_amdgcn_make_buffer_rsrc(
             const_cast<float *>(p.input + static_cast<size_t>(load_image) * s.c_in * H * W), 0, static_cast<int>(image_bytes),
             0x00020000);
-        if (VEC) {  // spatial % 4 == 0: a 16-byte chunk is entirely inside its channel row or entirely past it
-            const unsigned off = (p0 + a_c4 < p.spatial) ? a_base + static_cast<unsigned>(p0) * 4u : kOutside;
-            ra = __builtin_amdgcn_raw_buffer_load_b128(rsrc_g, off, 0, 0);
-        } else {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const unsigned off = (p0 + a_c4 + e < p.spatial) ? a_base + static_cast<unsigned>(p0 + e) * 4u : kOutside;
-                ra[e] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_g, off, 0, 0);
+        for (int i = 0; i < TM; ++i) {
+            if (VEC) {  // spatial % 4 == 0: a 16-byte chunk is entirely inside its channel row or entirely past it
+                const unsigned off = (p0 + a_c4 < p.spatial) ? a_base[i] + static_cast<unsigned>(p0) * 4u : kOutside;
+                ra[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_g, off, 0, 0);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const unsigned off = (p0 + a_c4 + e < p.spatial) ? a_base[i] + static_cast<unsigned>(p0 + e) * 4u : kOutside;
+                    ra[i][e] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_g, off, 0, 0);
+                }
             }
         }
-        // The four pixels are the same for every lane of the wavefront (lanes differ in their tap), so whether they
+        // The four pixels are the same for every lane of the wavefront (lanes differ in their taps), so whether they
         // sit in one image row is a scalar question.  If they do, and no lane's tap straddles the left or right
         // border, the four values are one 128-bit load (dword-aligned is enough for buffer loads).
         const bool one_row = s.stride_w == 1 && ox + 3 < s.ow && p0 + prow0 + 3 < p.spatial;
-        bool vector_done = false;
-        if (one_row) {
-            const int iy = oy * s.stride_h + dy, ix0 = ox + dx;
-            const bool row_ok = col_valid && static_cast<unsigned>(iy) < static_cast<unsigned>(H);
-            const bool full = row_ok && ix0 >= 0 && ix0 + 3 < W;
-            if (__builtin_amdgcn_ballot_w64(row_ok && !full) == 0) {
-                const unsigned off = full ? static_cast<unsigned>(tap_offset + iy * W + ix0) * 4u : kOutside;
-                const u32x4_t raw = __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, off, 0, 0);
 #pragma unroll
-                for (int r = 0; r < 4; ++r) rb[r] = __uint_as_float(raw[r]);
-                vector_done = true;
+        for (int j = 0; j < TN; ++j) {
+            bool vector_done = false;
+            if (one_row) {
+                const int iy = oy * s.stride_h + dy[j], ix0 = ox + dx[j];
+                const bool row_ok = col_valid[j] && static_cast<unsigned>(iy) < static_cast<unsigned>(H);
+                const bool full = row_ok && ix0 >= 0 && ix0 + 3 < W;
+                if (__builtin_amdgcn_ballot_w64(row_ok && !full) == 0) {
+                    const unsigned off = full ? static_cast<unsigned>(tap_offset[j] + iy * W + ix0) * 4u : kOutside;
+                    const u32x4_t raw = __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, off, 0, 0);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) rb[j][r] = __uint_as_float(raw[r]);
+                    vector_done = true;
+                }
             }
-        }
-        int py = oy, px = ox;
-        if (!vector_done)
+            if (!vector_done) {
+                int py = oy, px = ox;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int iy = py * s.stride_h + dy, ix = px * s.stride_w + dx;
-            const bool inside = col_valid && p0 + prow0 + r < p.spatial && static_cast<unsigned>(iy) < static_cast<unsigned>(H) &&
-                                static_cast<unsigned>(ix) < static_cast<unsigned>(W);
-            const unsigned off = inside ? static_cast<unsigned>(tap_offset + iy * W + ix) * 4u : kOutside;
-            rb[r] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc_x, off, 0, 0));
-            if (++px == s.ow) {
-                px = 0;
-                ++py;
+                for (int r = 0; r < 4; ++r) {
+                    const int iy = py * s.stride_h + dy[j], ix = px * s.stride_w + dx[j];
+                    const bool inside = col_valid[j] && p0 + prow0 + r < p.spatial &&
+                                        static_cast<unsigned>(iy) < static_cast<unsigned>(H) &&
+                                        static_cast<unsigned>(ix) < static_cast<unsigned>(W);
+                    const unsigned off = inside ? static_cast<unsigned>(tap_offset[j] + iy * W + ix) * 4u : kOutside;
+                    rb[j][r] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc_x, off, 0, 0));
+                    if (++px == s.ow) {
+                        px = 0;
+                        ++py;
+                    }
+                }
             }
         }
         // advance to the next step (possibly the next image)
@@ -240,20 +259,35 @@ __global__ __launch_bounds__(256) void conv_grad_weight_kernel(GradWeightArgs p)
         }
     };
     auto store_lds = [&](int stage) {
-        *reinterpret_cast<u32x4_t *>(&As[stage][a_row * A_STRIDE + a_c4]) = ra;
-        f32x4 packed;
-        packed[0] = rb[0]; packed[1] = rb[1]; packed[2] = rb[2]; packed[3] = rb[3];
-        *reinterpret_cast<f32x4 *>(&Bs[stage][(tid & 63) * B_STRIDE + prow0]) = packed;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+            *reinterpret_cast<u32x4_t *>(&As[stage * A_STAGE + (a_row + 64 * i) * A_STRIDE + a_c4]) = ra[i];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            f32x4 packed;
+            packed[0] = rb[j][0]; packed[1] = rb[j][1]; packed[2] = rb[j][2]; packed[3] = rb[j][3];
+            *reinterpret_cast<f32x4 *>(&Bs[stage * B_STAGE + (j * 64 + lane) * B_STRIDE + prow0]) = packed;
+        }
     };
     auto compute = [&](int stage) {
-        const float *as = As[stage];
-        const float *bs = Bs[stage];
+        const float *as = As + stage * A_STAGE;
+        const float *bs = Bs + stage * B_STAGE;
 #pragma unroll
         for (int kk = 0; kk < BK / 8; ++kk) {
-            const f32x4 av = *reinterpret_cast<const f32x4 *>(&as[(wm * 32 + li) * A_STRIDE + kk * 8 + lh * 4]);
-            const f32x4 bv = *reinterpret_cast<const f32x4 *>(&bs[(wn * 32 + li) * B_STRIDE + kk * 8 + lh * 4]);
+            f32x4 av[TM], bv[TN];
 #pragma unroll
-            for (int t = 0; t < 4; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[t], bv[t], acc, 0, 0, 0);
+            for (int i = 0; i < TM; ++i)
+                av[i] = *reinterpret_cast<const f32x4 *>(&as[(wm * 32 * TM + i * 32 + li) * A_STRIDE + kk * 8 + lh * 4]);
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                bv[j] = *reinterpret_cast<const f32x4 *>(&bs[(wn * 32 * TN + j * 32 + li) * B_STRIDE + kk * 8 + lh * 4]);
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i][t], bv[j][t], acc[i][j], 0, 0, 0);
         }
     };
 
@@ -271,14 +305,34 @@ __global__ __launch_bounds__(256) void conv_grad_weight_kernel(GradWeightArgs p)
     }
 
     float *dst = p.partial + static_cast<size_t>(chunk) * s.c_out * p.S;
-    const int out_col = s0 + wn * 32 + li;
-    if (out_col < p.S) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int oc = oc0 + wm * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
-            if (oc < s.c_out) dst[static_cast<size_t>(oc) * p.S + out_col] = acc[r];
-        }
+    for (int j = 0; j < TN; ++j) {
+        const int out_col = s0 + wn * 32 * TN + j * 32 + li;
+        if (out_col >= p.S) continue;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int oc = oc0 + wm * 32 * TM + i * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
+                if (oc < s.c_out) dst[static_cast<size_t>(oc) * p.S + out_col] = acc[i][j][r];
+            }
     }
+}
+
+template <bool VEC>
+__global__ __launch_bounds__(256) void conv_grad_weight_kernel(GradWeightArgs p)
+{
+    __shared__ __attribute__((aligned(16))) float As[2 * 64 * 20];
+    __shared__ __attribute__((aligned(16))) float Bs[2 * 64 * 20];
+    conv_grad_weight_body<VEC, 1, 1>(p, As, Bs);
+}
+
+template <bool VEC>
+__global__ __launch_bounds__(256) void conv_grad_weight_big_kernel(GradWeightArgs p)
+{
+    __shared__ __attribute__((aligned(16))) float As[2 * 128 * 20];
+    __shared__ __attribute__((aligned(16))) float Bs[2 * 192 * 20];
+    conv_grad_weight_body<VEC, 2, 3>(p, As, Bs);
 }
 
 }  // namespace
@@ -352,13 +406,19 @@ hipError_t launch_conv2d_grad_weight_f32(const ConvShape &shape, const float *in
     args.s = shape;
     args.S = S;
     args.spatial = shape.oh * shape.ow;
-    args.tiles_s = (S + 63) / 64;
-    const int tiles = args.tiles_s * ((shape.c_out + 63) / 64);
+    // 128 × 192 tiles when they waste little (every output channel and column a tile covers beyond the matrix is
+    // arithmetic thrown away), 64 × 64 tiles otherwise.
+    const long long big_cover = static_cast<long long>((shape.c_out + 127) / 128 * 128) * ((S + 191) / 192 * 192);
+    const bool big = big_cover * 10 <= static_cast<long long>(count) * 12;
+    const int bm = big ? 128 : 64, bn = big ? 192 : 64;
+    args.tiles_s = (S + bn - 1) / bn;
+    const int tiles = args.tiles_s * ((shape.c_out + bm - 1) / bm);
     // The reduction (all 16-pixel steps of all images, numbered image by image) is cut into chunks so that the
-    // launch is a whole number of rounds of 2048 workgroups (8 per compute unit) where the problem allows it.
+    // launch is about one round of resident workgroups (8 small or 2 big tiles per compute unit).
     const long long steps_per_image = (args.spatial + 15) / 16;
     const long long total_steps = steps_per_image * shape.batch;
-    long long chunks = (2048 + tiles - 1) / tiles;
+    const long long slots = big ? 512 : 2048;
+    long long chunks = slots / tiles;  // rounded down: one workgroup too many would run as a round of its own
     if (chunks > total_steps) chunks = total_steps;
     if (chunks < 1) chunks = 1;
     args.steps_per_chunk = static_cast<int>(total_steps > 0 ? (total_steps + chunks - 1) / chunks : 1);
@@ -369,7 +429,11 @@ hipError_t launch_conv2d_grad_weight_f32(const ConvShape &shape, const float *in
     args.partial = static_cast<float *>(workspace);
     const bool vec = args.spatial % 4 == 0 && (reinterpret_cast<uintptr_t>(grad_output) & 15u) == 0;
     const dim3 grid(static_cast<unsigned>(static_cast<size_t>(tiles) * static_cast<size_t>(chunks)));
-    if (vec)
+    if (big && vec)
+        hipLaunchKernelGGL(conv_grad_weight_big_kernel<true>, grid, dim3(256), 0, stream, args);
+    else if (big)
+        hipLaunchKernelGGL(conv_grad_weight_big_kernel<false>, grid, dim3(256), 0, stream, args);
+    else if (vec)
         hipLaunchKernelGGL(conv_grad_weight_kernel<true>, grid, dim3(256), 0, stream, args);
     else
         hipLaunchKernelGGL(conv_grad_weight_kernel<false>, grid, dim3(256), 0, stream, args);

@@ -19,6 +19,9 @@ CASES = [
     (2, 5, 10, 11, 6, (3, 3), (1, 1), (3, 3), (1, 1)),     # padding larger than the kernel reach: adjoint gather
     (2, 4, 16, 16, 8, (5, 5), (1, 1), (2, 2), (1, 1)),
     (8, 64, 14, 14, 64, (1, 1), (1, 1), (0, 0), (1, 1)),
+    (2, 64, 9, 10, 128, (3, 3), (1, 1), (1, 1), (1, 1)),   # 128 × 192 grad_weight tiles, exact fit (S = 576)
+    (3, 21, 11, 7, 120, (3, 3), (1, 1), (1, 1), (1, 1)),   # 128 × 192 tiles with ragged channels and columns (S = 189)
+    (2, 22, 9, 9, 250, (3, 3), (2, 1), (1, 0), (1, 1)),    # two channel tiles, strided rows (per-element gather)
 ]
 
 
