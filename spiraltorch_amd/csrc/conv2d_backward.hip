@@ -99,6 +99,7 @@ struct GradWeightArgs {
     int spatial;               // oh * ow
     int tiles_s;
     int steps_per_chunk;       // 16-pixel steps (numbered image by image) per workgroup
+    int workgroups;            // tiles × chunks; the launch grid is this rounded up to a multiple of 8
 };
 
 // One workgroup: a (64·TM output channels) × (64·TN reduction columns s) tile of grad_weight, summed over the pixels
@@ -126,8 +127,9 @@ __device__ __forceinline__ void conv_grad_weight_body(const GradWeightArgs &p, f
 
     // Workgroup ids go round-robin over the 8 XCDs; give each XCD a contiguous run of (chunk, tile) pairs so that
     // the tiles that share a chunk's pixels find them in the same L2.
-    int bid = blockIdx.x;
-    if ((gridDim.x & 7) == 0) bid = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+    // (The grid is padded to a multiple of 8; the padding workgroups leave at once.)
+    int bid = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+    if (bid >= p.workgroups) return;
     const int tile_s = bid % p.tiles_s;
     bid /= p.tiles_s;
     const int tiles_oc = (s.c_out + BM - 1) / BM;
@@ -428,7 +430,10 @@ hipError_t launch_conv2d_grad_weight_f32(const ConvShape &shape, const float *in
     if (rc != hipSuccess) return rc;
     args.partial = static_cast<float *>(workspace);
     const bool vec = args.spatial % 4 == 0 && (reinterpret_cast<uintptr_t>(grad_output) & 15u) == 0;
-    const dim3 grid(static_cast<unsigned>(static_cast<size_t>(tiles) * static_cast<size_t>(chunks)));
+    const size_t workgroups = static_cast<size_t>(tiles) * static_cast<size_t>(chunks);
+    if (workgroups > 0x7ffffff0u) return hipErrorInvalidConfiguration;
+    args.workgroups = static_cast<int>(workgroups);
+    const dim3 grid(static_cast<unsigned>((workgroups + 7) / 8 * 8));
     if (big && vec)
         hipLaunchKernelGGL(conv_grad_weight_big_kernel<true>, grid, dim3(256), 0, stream, args);
     else if (big)
