@@ -14,6 +14,12 @@
 // per-element cost is two adds, two range checks and one load.
 //
 // MFMA usage is the same as the f32 GEMM (32x32x2 f32, k issued as the pairs {s, s+4}).
+//
+// Three kernel families share this formulation, chosen by shape in launch_conv2d_f32: the general tile kernel
+// described above (any shape), the ring kernel (weights and patch rows go memory -> LDS directly; the better steady
+// state for layers that give the chip several rounds of tiles) and the strip kernel (weights resident in LDS, image
+// values loaded straight into the MFMA operand registers, blocks claimed dynamically; the better balance when the
+// tiles of a layer quantise badly over the chip, and for narrow layers).
 #include "device_math.h"
 #include "kernels.h"
 
