@@ -86,6 +86,8 @@ __global__ __launch_bounds__(256) void layer_norm_vec_kernel(int rows, int cols,
         const float4 g = *reinterpret_cast<const float4 *>(gamma + c);
         const float4 b = *reinterpret_cast<const float4 *>(beta + c);
         float4 o;
+        // (a true division, not a multiply by the reciprocal: the last bit decides some of the bf16 roundings
+        // downstream, and the decoder is compared with a CPU stack that divides)
         o.x = ((v[i].x - mean) / denom) * g.x + b.x;
         o.y = ((v[i].y - mean) / denom) * g.y + b.y;
         o.z = ((v[i].z - mean) / denom) * g.z + b.z;
@@ -266,7 +268,7 @@ __global__ __launch_bounds__(256) void row_softmax_vec_kernel(int rows, int cols
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             const float value = v[i][e];
-            const float weight = (!found || value != value) ? 0.0f : expf(value - base);
+            const float weight = (!found || value != value) ? 0.0f : __expf(value - base);  // exp2 of a scaled argument
             v[i][e] = weight;
             denom += weight;
         }
@@ -298,6 +300,58 @@ __global__ __launch_bounds__(256) void gelu_backward_kernel(size_t count, const 
         const float t = tanhf(inner);
         const float prime = 0.5f * (1.0f + t) + (((0.5f * x) * (1.0f - t * t)) * 0.7978846f) * (1.0f + (3.0f * 0.044715f) * x2);
         out[i] = prime * grad[i];
+    }
+}
+
+// 128-bit forms of the element-wise kernels (count a multiple of 4, 16-byte aligned pointers): one float4 per
+// thread and as many workgroups as that takes, which is the access pattern that streams fastest on this chip.
+__global__ __launch_bounds__(256) void gelu_backward_vec_kernel(size_t count4, const float4 *z, const float4 *grad, float4 *out)
+{
+    const size_t stride = static_cast<size_t>(gridDim.x) * 256;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < count4; i += stride) {
+        const float4 x4 = z[i], g4 = grad[i];
+        const float xs[4] = {x4.x, x4.y, x4.z, x4.w}, gs[4] = {g4.x, g4.y, g4.z, g4.w};
+        float r[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float x = xs[e];
+            const float x2 = x * x;
+            const float inner = 0.7978846f * (x + (0.044715f * x) * x2);
+            const float t = tanhf(inner);
+            const float prime = 0.5f * (1.0f + t) + (((0.5f * x) * (1.0f - t * t)) * 0.7978846f) * (1.0f + (3.0f * 0.044715f) * x2);
+            r[e] = prime * gs[e];
+        }
+        out[i] = make_float4(r[0], r[1], r[2], r[3]);
+    }
+}
+
+__global__ __launch_bounds__(256) void scale_vec_kernel(size_t count4, const float4 *in, float scale, float4 *out)
+{
+    const size_t stride = static_cast<size_t>(gridDim.x) * 256;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < count4; i += stride) {
+        const float4 v = in[i];
+        out[i] = make_float4(v.x * scale, v.y * scale, v.z * scale, v.w * scale);
+    }
+}
+
+// cols a multiple of 4: a float4 never straddles a row
+__global__ __launch_bounds__(256) void add_row_vec_kernel(size_t count4, int cols4, float4 *data, const float4 *bias)
+{
+    const size_t stride = static_cast<size_t>(gridDim.x) * 256;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < count4; i += stride) {
+        float4 v = data[i];
+        const float4 b = bias[i % static_cast<size_t>(cols4)];
+        v.x += b.x; v.y += b.y; v.z += b.z; v.w += b.w;
+        data[i] = v;
+    }
+}
+
+__global__ __launch_bounds__(256) void f32_to_bf16_vec_kernel(size_t count4, const float4 *in, uint2 *out)
+{
+    const size_t stride = static_cast<size_t>(gridDim.x) * 256;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < count4; i += stride) {
+        const float4 v = in[i];
+        out[i] = make_uint2(pack_bf16x2_rne(v.x, v.y), pack_bf16x2_rne(v.z, v.w));
     }
 }
 
@@ -400,6 +454,14 @@ __global__ __launch_bounds__(256) void sum_axis0_final_wide_kernel(int chunks, i
     }
 }
 
+unsigned grid_vec_for(size_t count4)
+{
+    const size_t blocks = (count4 + 255) / 256;
+    return static_cast<unsigned>(blocks < 0x7fffffffull ? (blocks ? blocks : 1) : 0x7fffffffull);
+}
+
+bool aligned16(const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
+
 unsigned grid_for(size_t count)
 {
     const size_t blocks = (count + 255) / 256;
@@ -445,6 +507,11 @@ hipError_t launch_embedding_f32(size_t tokens, size_t vocab, size_t dim, const f
 hipError_t launch_f32_to_bf16(size_t count, const float *in, uint16_t *out, hipStream_t stream)
 {
     if (count == 0) return hipSuccess;
+    if (count % 4 == 0 && aligned16(in) && (reinterpret_cast<uintptr_t>(out) & 7u) == 0) {
+        hipLaunchKernelGGL(f32_to_bf16_vec_kernel, dim3(grid_vec_for(count / 4)), dim3(256), 0, stream, count / 4,
+                           reinterpret_cast<const float4 *>(in), reinterpret_cast<uint2 *>(out));
+        return hipGetLastError();
+    }
     hipLaunchKernelGGL(f32_to_bf16_kernel, dim3(grid_for(count)), dim3(256), 0, stream, count, in, out);
     return hipGetLastError();
 }
@@ -494,6 +561,12 @@ hipError_t launch_row_softmax_f32(size_t rows, size_t cols, const float *in, flo
 hipError_t launch_gelu_backward_f32(size_t count, const float *z, const float *grad, float *out, hipStream_t stream)
 {
     if (count == 0) return hipSuccess;
+    if (count % 4 == 0 && aligned16(z) && aligned16(grad) && aligned16(out)) {
+        hipLaunchKernelGGL(gelu_backward_vec_kernel, dim3(grid_vec_for(count / 4)), dim3(256), 0, stream, count / 4,
+                           reinterpret_cast<const float4 *>(z), reinterpret_cast<const float4 *>(grad),
+                           reinterpret_cast<float4 *>(out));
+        return hipGetLastError();
+    }
     hipLaunchKernelGGL(gelu_backward_kernel, dim3(grid_for(count)), dim3(256), 0, stream, count, z, grad, out);
     return hipGetLastError();
 }
@@ -501,6 +574,11 @@ hipError_t launch_gelu_backward_f32(size_t count, const float *z, const float *g
 hipError_t launch_scale_f32(size_t count, const float *in, float scale, float *out, hipStream_t stream)
 {
     if (count == 0) return hipSuccess;
+    if (count % 4 == 0 && aligned16(in) && aligned16(out)) {
+        hipLaunchKernelGGL(scale_vec_kernel, dim3(grid_vec_for(count / 4)), dim3(256), 0, stream, count / 4,
+                           reinterpret_cast<const float4 *>(in), scale, reinterpret_cast<float4 *>(out));
+        return hipGetLastError();
+    }
     hipLaunchKernelGGL(scale_kernel, dim3(grid_for(count)), dim3(256), 0, stream, count, in, scale, out);
     return hipGetLastError();
 }
@@ -508,6 +586,11 @@ hipError_t launch_scale_f32(size_t count, const float *in, float scale, float *o
 hipError_t launch_add_row_f32(size_t rows, size_t cols, float *data, const float *bias, hipStream_t stream)
 {
     if (rows == 0 || cols == 0) return hipSuccess;
+    if (cols % 4 == 0 && aligned16(data) && aligned16(bias)) {
+        hipLaunchKernelGGL(add_row_vec_kernel, dim3(grid_vec_for(rows * cols / 4)), dim3(256), 0, stream, rows * cols / 4,
+                           static_cast<int>(cols / 4), reinterpret_cast<float4 *>(data), reinterpret_cast<const float4 *>(bias));
+        return hipGetLastError();
+    }
     hipLaunchKernelGGL(add_row_kernel, dim3(grid_for(rows * cols)), dim3(256), 0, stream, rows * cols,
                        static_cast<int>(cols), data, bias);
     return hipGetLastError();

@@ -10,7 +10,9 @@ pytestmark = pytest.mark.gpu
 def test_layer_norm(hip, oracle):
     from spiraltorch_amd import inputs
     rng = np.random.default_rng(4)
-    for rows, cols in ((1, 1), (5, 48), (130, 512), (7, 1000), (9, 1536), (3, 2048), (4, 2052), (6, 4100)):
+    # (16384 rows and more: two rows per wavefront, odd row counts leave the last wavefront half empty)
+    for rows, cols in ((1, 1), (5, 48), (130, 512), (7, 1000), (9, 1536), (3, 2048), (4, 2052), (6, 4100), (16384, 512),
+                       (16387, 256), (16389, 1024)):
         x = rng.normal(1.0, 2.0, rows * cols).astype(np.float32)
         res = rng.normal(size=rows * cols).astype(np.float32)
         g, b = rng.normal(size=cols).astype(np.float32), rng.normal(size=cols).astype(np.float32)

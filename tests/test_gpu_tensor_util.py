@@ -11,7 +11,8 @@ def on_device(hip, *arrays):
     return [hip.DeviceBuffer.from_array(np.ascontiguousarray(a, dtype=np.float32)) for a in arrays]
 
 
-@pytest.mark.parametrize("rows,cols", [(1, 1), (2, 4), (5, 63), (7, 64), (3, 65), (33, 1000), (1024, 256), (4, 5000), (9, 512), (6, 516), (5, 2048), (3, 2052)])
+@pytest.mark.parametrize("rows,cols", [(1, 1), (2, 4), (5, 63), (7, 64), (3, 65), (33, 1000), (1024, 256), (4, 5000), (9, 512), (6, 516), (5, 2048), (3, 2052),
+                                       (16384, 512), (16387, 128), (16389, 1024)])
 def test_row_softmax(hip, oracle, rows, cols):
     rng = np.random.default_rng(rows * 31 + cols)
     x = (rng.normal(size=rows * cols) * 3).astype(np.float32)
@@ -38,11 +39,16 @@ def test_row_softmax_reference_input_and_edge_rows(hip, oracle, golden):
     assert got[12:16].tolist() == [0.0] * 4 and got[16:20].tolist() == [0.0, 1.0, 0.0, 0.0]
 
 
-def test_gelu_backward(hip, oracle, golden):
+@pytest.mark.parametrize("multiple_of_four", [False, True])
+def test_gelu_backward(hip, oracle, golden, multiple_of_four):
+    # a count that is a multiple of four takes the 128-bit kernel, any other the scalar one
     c = golden["gelu_backward"]
     rng = np.random.default_rng(8)
-    z = np.concatenate([np.array(c["z"], np.float32), (rng.normal(size=100003) * 2).astype(np.float32)])
-    g = np.concatenate([np.array(c["grad"], np.float32), rng.normal(size=100003).astype(np.float32)])
+    extra = 100003
+    while ((len(c["z"]) + extra) % 4 == 0) != multiple_of_four:
+        extra += 1
+    z = np.concatenate([np.array(c["z"], np.float32), (rng.normal(size=extra) * 2).astype(np.float32)])
+    g = np.concatenate([np.array(c["grad"], np.float32), rng.normal(size=extra).astype(np.float32)])
     d_z, d_g = on_device(hip, z, g)
     d_out = hip.DeviceBuffer(z.nbytes)
     hip.gelu_backward_f32_dev(z.size, d_z, d_g, d_out)
@@ -50,9 +56,10 @@ def test_gelu_backward(hip, oracle, golden):
     assert_close(d_out.to_array(np.float32, z.size), oracle.gelu_backward_f32(z, g), F32_REL, F32_ABS, "gelu_backward")
 
 
-def test_scale_and_add_row(hip, oracle):
+@pytest.mark.parametrize("rows,cols", [(301, 77), (512, 256), (33, 1028), (7, 4)])
+def test_scale_and_add_row(hip, oracle, rows, cols):
+    # (column counts that are multiples of four take the 128-bit kernels)
     rng = np.random.default_rng(12)
-    rows, cols = 301, 77
     x = rng.normal(size=rows * cols).astype(np.float32)
     bias = rng.normal(size=cols).astype(np.float32)
     d_x, d_b = on_device(hip, x, bias)
@@ -65,6 +72,27 @@ def test_scale_and_add_row(hip, oracle):
     assert (d_x.to_array(np.float32, x.size) == oracle.add_row_f32(rows, cols, x, bias)).all()
     with pytest.raises(hip.HipErr, match="scale_factor"):
         hip.scale_f32_dev(x.size, d_x, float("nan"), d_out)
+
+
+def test_elementwise_kernels_on_unaligned_pointers(hip, oracle):
+    """Pointers that are only 4-byte aligned must take the scalar kernels and give the same values."""
+    rng = np.random.default_rng(13)
+    rows, cols = 64, 256
+    n = rows * cols
+    x = rng.normal(size=n + 1).astype(np.float32)
+    g = rng.normal(size=n + 1).astype(np.float32)
+    bias = rng.normal(size=cols + 1).astype(np.float32)
+    d_x, d_g, d_b = on_device(hip, x, g, bias)
+    d_out = hip.DeviceBuffer((n + 1) * 4)
+    hip.scale_f32_dev(n, d_x.at(4), 1.5, d_out.at(4))
+    hip.device_synchronize()
+    assert (d_out.to_array(np.float32, n + 1)[1:] == oracle.scale_f32(x[1:], 1.5)).all()
+    hip.gelu_backward_f32_dev(n, d_x.at(4), d_g.at(4), d_out.at(4))
+    hip.device_synchronize()
+    assert_close(d_out.to_array(np.float32, n + 1)[1:], oracle.gelu_backward_f32(x[1:], g[1:]), F32_REL, F32_ABS, "gelu_backward")
+    hip.add_row_f32_dev(rows, cols, d_x.at(4), d_b.at(4))
+    hip.device_synchronize()
+    assert (d_x.to_array(np.float32, n + 1)[1:] == oracle.add_row_f32(rows, cols, x[1:], bias[1:])).all()
 
 
 @pytest.mark.parametrize("rows,cols", [(1, 1), (3, 2), (64, 256), (65, 257), (1000, 19), (16384, 512), (100000, 8), (37, 260), (131, 1028), (5, 4)])
