@@ -79,6 +79,15 @@ __global__ __launch_bounds__(256) void layer_norm_vec_kernel(int rows, int cols,
     const float mean = sum / cols_f;
     const float var = fmaxf(sumsq / cols_f - mean * mean, 0.0f);
     const float denom = sqrtf(var + epsilon);
+    // (v - mean) / denom for every element, with one real division per row: the product with the correctly rounded
+    // reciprocal, corrected once by its exact remainder (two fused multiply-adds), is the correctly rounded quotient
+    // again, i.e. bit for bit what the division gives; only the last bit matters here, because it decides some of
+    // the bf16 roundings downstream and the decoder is compared with a CPU stack that divides.
+    const float inv = 1.0f / denom;
+    auto quotient = [&](float a) {
+        const float q = a * inv;
+        return fmaf(fmaf(-q, denom, a), inv, q);
+    };
 #pragma unroll
     for (int i = 0; i < CHUNKS; ++i) {
         const int c = (lane + 64 * i) * 4;
@@ -86,12 +95,10 @@ __global__ __launch_bounds__(256) void layer_norm_vec_kernel(int rows, int cols,
         const float4 g = *reinterpret_cast<const float4 *>(gamma + c);
         const float4 b = *reinterpret_cast<const float4 *>(beta + c);
         float4 o;
-        // (a true division, not a multiply by the reciprocal: the last bit decides some of the bf16 roundings
-        // downstream, and the decoder is compared with a CPU stack that divides)
-        o.x = ((v[i].x - mean) / denom) * g.x + b.x;
-        o.y = ((v[i].y - mean) / denom) * g.y + b.y;
-        o.z = ((v[i].z - mean) / denom) * g.z + b.z;
-        o.w = ((v[i].w - mean) / denom) * g.w + b.w;
+        o.x = quotient(v[i].x - mean) * g.x + b.x;
+        o.y = quotient(v[i].y - mean) * g.y + b.y;
+        o.z = quotient(v[i].z - mean) * g.z + b.z;
+        o.w = quotient(v[i].w - mean) * g.w + b.w;
         if (out_f32) *reinterpret_cast<float4 *>(out_f32 + offset + c) = o;
         if (out_bf16) {
             uint2 packed;
