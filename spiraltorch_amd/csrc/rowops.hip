@@ -127,6 +127,25 @@ __global__ __launch_bounds__(256) void embedding_kernel(int tokens, int vocab, i
     for (int c = threadIdx.x; c < dim; c += 256) dst[c] = src[c];
 }
 
+// Same gather, 128 bits per thread (dim a multiple of 4, 16-byte aligned table and output): thread i of the launch
+// copies chunk i % (dim/4) of token i / (dim/4).
+__global__ __launch_bounds__(256) void embedding_vec_kernel(size_t chunks, int vocab, int dim4, const float *token_ids,
+                                                            const float4 *table, float4 *out)
+{
+    const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (i >= chunks) return;
+    const size_t token = i / static_cast<size_t>(dim4);
+    const int c = static_cast<int>(i - token * dim4);
+    const float value = token_ids[token];
+    int index = 0;
+    if (isfinite(value)) {
+        const float rounded = roundf(value);
+        if (rounded > 0.0f) index = rounded >= static_cast<float>(vocab) ? vocab - 1 : static_cast<int>(rounded);
+        if (index > vocab - 1) index = vocab - 1;
+    }
+    out[i] = table[static_cast<size_t>(index) * dim4 + c];
+}
+
 __global__ __launch_bounds__(256) void f32_to_bf16_kernel(size_t count, const float *in, uint16_t *out)
 {
     const size_t stride = static_cast<size_t>(gridDim.x) * 256;
@@ -506,6 +525,13 @@ hipError_t launch_embedding_f32(size_t tokens, size_t vocab, size_t dim, const f
                                 float *out, hipStream_t stream)
 {
     if (tokens == 0 || dim == 0) return hipSuccess;
+    const size_t chunks = tokens * (dim / 4);
+    if (dim % 4 == 0 && aligned16(table) && aligned16(out) && (chunks + 255) / 256 < 0x7fffffffull) {
+        hipLaunchKernelGGL(embedding_vec_kernel, dim3(static_cast<unsigned>((chunks + 255) / 256)), dim3(256), 0, stream, chunks,
+                           static_cast<int>(vocab), static_cast<int>(dim / 4), token_ids,
+                           reinterpret_cast<const float4 *>(table), reinterpret_cast<float4 *>(out));
+        return hipGetLastError();
+    }
     hipLaunchKernelGGL(embedding_kernel, dim3(static_cast<unsigned>(tokens)), dim3(256), 0, stream,
                        static_cast<int>(tokens), static_cast<int>(vocab), static_cast<int>(dim), token_ids, table, out);
     return hipGetLastError();

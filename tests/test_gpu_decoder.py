@@ -34,6 +34,13 @@ def test_embedding_split_merge_and_rounding(hip, oracle):
     hip.embedding_f32_dev(ids.size, 4, 3, hip.DeviceBuffer.from_array(ids), hip.DeviceBuffer.from_array(table), d_out)
     hip.device_synchronize()
     assert (d_out.to_array(np.float32, ids.size * 3) == oracle.embedding_f32(ids.size, 4, 3, ids, table)).all()
+    # rows that are a multiple of four wide take the 128-bit gather
+    wide = np.arange(4 * 72, dtype=np.float32).reshape(4, 72)
+    many = np.concatenate([ids, np.random.default_rng(3).uniform(-1, 5, 500).astype(np.float32)])
+    d_wide = hip.DeviceBuffer(many.size * 72 * 4)
+    hip.embedding_f32_dev(many.size, 4, 72, hip.DeviceBuffer.from_array(many), hip.DeviceBuffer.from_array(wide), d_wide)
+    hip.device_synchronize()
+    assert (d_wide.to_array(np.float32, many.size * 72) == oracle.embedding_f32(many.size, 4, 72, many, wide)).all()
 
     vals = np.random.default_rng(0).normal(size=1000).astype(np.float32)
     # ties (round to even in both directions), the largest finite value, infinities, denormals and signed zero
