@@ -95,6 +95,30 @@ def test_kernel_families(hip, oracle, monkeypatch, family, shape):
     assert_close(got, want, F32_REL, F32_ABS, f"conv {shape} family={family}")
 
 
+def test_strip_kernel_store_paths_agree(hip, oracle, monkeypatch):
+    """The strip kernel stores 128 bits per lane through an LDS tile when the output is 16-byte aligned and the
+    plane size is a multiple of four, 32 bits per lane otherwise: same values either way."""
+    monkeypatch.setenv("ST_HIP_CONV_KERNEL", "strip")
+    shape = (3, 16, 20, 20, 70, (3, 3), (1, 1), (1, 1), (1, 1))
+    batch, c_in, h, w, c_out, kernel, stride, padding, dilation = shape
+    rng = np.random.default_rng(77)
+    x = rng.normal(size=batch * c_in * h * w).astype(np.float32)
+    wt = rng.normal(0, 0.1, c_out * c_in * 9).astype(np.float32)
+    b = rng.uniform(-0.1, 0.1, c_out).astype(np.float32)
+    n_out = batch * c_out * 20 * 20
+    d_x, d_w, d_b = (hip.DeviceBuffer.from_array(a) for a in (x, wt, b))
+    d_out = hip.DeviceBuffer((n_out + 1) * 4)
+    hip.conv2d_bias_act_f32_dev(*shape, 1, d_x, d_w, d_b, d_out)
+    hip.device_synchronize()
+    aligned = d_out.to_array(np.float32, n_out + 1)[:n_out].copy()
+    d_out.zero()
+    hip.conv2d_bias_act_f32_dev(*shape, 1, d_x, d_w, d_b, d_out.at(4))
+    hip.device_synchronize()
+    shifted = d_out.to_array(np.float32, n_out + 1)[1:]
+    assert (aligned == shifted).all()
+    assert_close(aligned, oracle.conv2d_bias_act_f32(*shape, oracle.ACT_RELU, x, wt, b, threads=8), F32_REL, F32_ABS, "strip stores")
+
+
 def test_conv2d_layer_mirror(hip, oracle):
     from spiraltorch_amd import Conv2d, Tensor, TensorError
     conv = Conv2d("conv_gpu", 3, 8, (3, 3), (1, 1), (1, 1), (1, 1), (8, 8))
