@@ -598,14 +598,6 @@ __device__ __forceinline__ void conv2d_f32_strip_body(const StripArgs &p)
         const_cast<float *>(p.input + static_cast<size_t>(image) * image_elems), 0, static_cast<int>(image_elems * 4), 0x00020000);
     const float *a_lane = lds_w + (lh * 32 + li) * PITCH;
     float *out_image = p.out + static_cast<size_t>(image) * s.c_out * p.spatial;
-    float bias[WIDE ? 1 : 16];
-    if constexpr (!WIDE) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int oc = oc0 + (r >> 2) * 8 + lh * 4 + (r & 3);
-            bias[r] = (p.bias && oc < s.c_out) ? p.bias[oc] : 0.0f;
-        }
-    }
     // 128-bit store path (WIDE): the wavefront's 32 × 32 results go through an LDS tile of its own, 16 channels at a time,
     // and leave as rows of four pixels per lane (lane -> channel row lane/8 (+8), pixels 4·(lane%8) .. +3).
     float *stage = reinterpret_cast<float *>(strip_lds + static_cast<size_t>(s.c_in) * 32 * PITCH * 4 + 16) +
@@ -681,12 +673,13 @@ __device__ __forceinline__ void conv2d_f32_strip_body(const StripArgs &p)
                 for (int tap = 0; tap < kStripTaps; ++tap) dst[tap] = src[tap];
             }
         };
-        // One channel pair: the operands of the next pair are requested, then nine MFMAs run on this pair's.
-        // (Scheduling fences: without them the compiler sinks each load to just before its use to save registers,
-        // which leaves the loads no time to complete.)
+        // One channel pair: the operands of the pair after next are requested, then nine MFMAs run on this pair's;
+        // three register sets in rotation (one pair ahead leaves the loads too little time: 157 -> 149 µs at
+        // config 2; a fourth set spills).  Scheduling fences: without them the compiler sinks each load to just
+        // before its use to save registers, which leaves the loads no time to complete.
         auto pair_body = [&](const float (&a_use)[kStripTaps], const float (&b_use)[kStripTaps], float (&a_next)[kStripTaps],
                              float (&b_next)[kStripTaps], int pair) {
-            const int following = pair + 1 < pairs ? pair + 1 : pair;  // past the end: re-read this pair (unused)
+            const int following = pair + 2 < pairs ? pair + 2 : pairs - 1;  // past the end: a re-read (unused)
             load_b(b_next, following);
             load_a(a_next, following);
             __builtin_amdgcn_sched_barrier(0);
@@ -695,15 +688,19 @@ __device__ __forceinline__ void conv2d_f32_strip_body(const StripArgs &p)
                 acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a_use[tap], b_use[tap], acc, 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
         };
-        float a0[kStripTaps], a1[kStripTaps], b0[kStripTaps], b1[kStripTaps];
+        float a0[kStripTaps], a1[kStripTaps], a2[kStripTaps], b0[kStripTaps], b1[kStripTaps], b2[kStripTaps];
         load_b(b0, 0);
         load_a(a0, 0);
+        load_b(b1, pairs > 1 ? 1 : 0);
+        load_a(a1, pairs > 1 ? 1 : 0);
         int pair = 0;
-        for (; pair + 2 <= pairs; pair += 2) {
-            pair_body(a0, b0, a1, b1, pair);
+        for (; pair + 3 <= pairs; pair += 3) {
+            pair_body(a0, b0, a2, b2, pair);
             pair_body(a1, b1, a0, b0, pair + 1);
+            pair_body(a2, b2, a1, b1, pair + 2);
         }
-        if (pair < pairs) pair_body(a0, b0, a1, b1, pair);
+        if (pair < pairs) pair_body(a0, b0, a2, b2, pair);
+        if (pair + 1 < pairs) pair_body(a1, b1, a0, b0, pair + 1);
 
         if constexpr (WIDE) {
             const int px4 = (first + blk) * 32 + (lane & 7) * 4;
@@ -731,9 +728,9 @@ __device__ __forceinline__ void conv2d_f32_strip_body(const StripArgs &p)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int oc = oc0 + (r >> 2) * 8 + lh * 4 + (r & 3);
-                if (oc < s.c_out)
+                if (oc < s.c_out)  // (the bias is re-read per block: sixteen registers are worth more in the main loop)
                     out_image[static_cast<size_t>(oc) * p.spatial + px] =
-                        apply_activation(acc[r] + bias[WIDE ? 0 : r], p.activation);
+                        apply_activation(acc[r] + (p.bias ? p.bias[oc] : 0.0f), p.activation);
             }
         }
     }
