@@ -366,8 +366,11 @@ __global__ __launch_bounds__(256) void conv_grad_weight_kernel(GradWeightArgs p)
     conv_grad_weight_body<VEC, 1, 1>(p, As, Bs);
 }
 
+// Three workgroups per compute unit (3 × 51,200 B of LDS, three wavefronts per SIMD): the occupancy attribute makes
+// the compiler fit 170 registers (it does, 160 without spilling) instead of spreading the accumulators over the
+// accumulation registers at two wavefronts per SIMD.
 template <bool VEC>
-__global__ __launch_bounds__(256) void conv_grad_weight_big_kernel(GradWeightArgs p)
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void conv_grad_weight_big_kernel(GradWeightArgs p)
 {
     __shared__ __attribute__((aligned(16))) float As[2 * 128 * 20];
     __shared__ __attribute__((aligned(16))) float Bs[2 * 192 * 20];
@@ -453,10 +456,10 @@ hipError_t launch_conv2d_grad_weight_f32(const ConvShape &shape, const float *in
     args.tiles_s = (S + bn - 1) / bn;
     const int tiles = args.tiles_s * ((shape.c_out + bm - 1) / bm);
     // The reduction (all 16-pixel steps of all images, numbered image by image) is cut into chunks so that the
-    // launch is about one round of resident workgroups (8 small or 2 big tiles per compute unit).
+    // launch is about one round of resident workgroups (8 small or 3 big tiles per compute unit).
     const long long steps_per_image = (args.spatial + 15) / 16;
     const long long total_steps = steps_per_image * shape.batch;
-    const long long slots = big ? 512 : 2048;
+    const long long slots = big ? 768 : 2048;
     long long chunks = slots / tiles;  // rounded down: one workgroup too many would run as a round of its own
     if (chunks > total_steps) chunks = total_steps;
     if (chunks < 1) chunks = 1;
