@@ -633,11 +633,12 @@ hipError_t launch_sum_axis0_f32(size_t rows, size_t cols, const float *in, float
 {
     if (cols == 0) return hipSuccess;
     const bool vec = cols % 4 == 0 && (reinterpret_cast<uintptr_t>(in) & 15u) == 0;
-    // Row chunks: enough workgroups to fill the chip, at least 128 rows each; the partial sums live in the stream's
-    // workspace and are added in a fixed order.
+    // Row chunks: about four workgroups per compute unit, at least 64 rows each (measured best on 16384 × 512: 9.0 µs
+    // with 128-row chunks, 6.8 µs with 64, 9.0 µs with 32); the partial sums live in the stream's workspace and are
+    // added in a fixed order.
     const size_t col_blocks = (cols + 255) / 256;
-    size_t chunks = (512 + col_blocks - 1) / col_blocks;
-    const size_t max_chunks = (rows + 127) / 128;
+    size_t chunks = (1024 + col_blocks - 1) / col_blocks;
+    const size_t max_chunks = (rows + 63) / 64;
     if (chunks > max_chunks) chunks = max_chunks;
     if (chunks == 0) chunks = 1;
     const size_t rows_per_chunk = (rows + chunks - 1) / chunks;
