@@ -39,7 +39,7 @@ MEASURED_TRAFFIC_BYTES = {
     "conv2d_bias_relu_f32_n32_c64to128_56x56_k3s1p1": (14304 * 2 + 50176) * 1024,
     "conv2d_grad_input_f32_n32_c64to128_56x56_k3s1p1": (30742 * 2 + 25088) * 1024,
     "gemm_bf16_f32acc_4096x4096x4096": (98558 * 2 + 65536) * 1024,
-    "gemm_bf16_f32acc_16x4096x4096": (16927 * 2 + 4096) * 1024,
+    "gemm_bf16_f32acc_16x4096x4096": (16927 * 2 + 2048) * 1024,
     "attention_f32_b8_h16_s2048_d64_noncausal": (98387 * 2 + 65536) * 1024,
     "attention_f32_b8_h16_s2048_d64_causal": (371670 * 2 + 65544) * 1024,
 }
