@@ -132,9 +132,12 @@ def test_fused_epilogue_and_bf16_output(hip, oracle, m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k,ragged", [(8192, 1024, 128, 0), (8192, 2048, 64, 0), (16384, 512, 192, 0),
-                                          (8192 - 37, 2048, 128, 1), (16384 - 5, 768, 64, 1)])
+                                          (8192 - 37, 2048, 128, 1), (16384 - 5, 768, 64, 1),
+                                          # few tiles: the same kernels serve every shape they can address
+                                          (65, 128, 64, 1), (300, 384, 192, 1), (257, 256, 64, 1), (512, 512, 512, 0),
+                                          (100, 1152, 320, 1)])
 def test_large_tile_kernels_with_epilogue(hip, oracle, m, n, k, ragged):
-    """Shapes that take the 256x256 and 256x128 tile kernels (>= 128 tiles), with bias + residual + GELU and
+    """Shapes that take the 256x256 and 256x128 tile kernels, with bias + residual + GELU and
     both output types; m may be ragged."""
     from spiraltorch_amd import inputs
     rng = np.random.default_rng(m + n + k)
