@@ -311,6 +311,7 @@ def main():
         ("conv2d_grad_weight", lambda: wl_conv2d_backward(hip, inputs, timer, side_warm, side_steps, "grad_weight")),
         ("gemm_f32_512", lambda: wl_gemm_f32(hip, inputs, timer, side_warm, side_steps, 512, 512, 512,
                                               "gemm_f32_512x512x512")),
+        ("gemm_f32_4096", lambda: wl_gemm_f32(hip, inputs, timer, 2, 5, 4096, 4096, 4096, "gemm_f32_4096x4096x4096")),
         ("gemm_f32_conv_equivalent", lambda: wl_gemm_f32(hip, inputs, timer, side_warm, side_steps, 100352, 128, 576,
                                                          "gemm_f32_100352x128x576_conv_equivalent")),
         ("gemm_bf16_4096", lambda: wl_gemm_bf16(hip, inputs, timer, side_warm, side_steps, 4096, 4096, 4096,
