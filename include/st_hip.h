@@ -130,6 +130,27 @@ int st_hip_conv2d_bias_act_f32(size_t batch, size_t c_in, size_t h, size_t w, si
                                size_t weight_len, const float *bias, size_t bias_len, float *out,
                                size_t out_len);
 
+/* Which kernel the dispatcher runs for a convolution.  The choice is made from the shape alone (plus 16-byte
+ * alignment of the weight and output pointers, assumed here); st_hip_conv2d_planned_kernel reports it for the forward
+ * pass (direction 0) or for grad_input of that forward shape (direction 1) as one of ST_HIP_CONV_KERNEL_*.
+ * st_hip_conv2d_force_family is a process-wide diagnostic switch (the parity tests use it to run every family on
+ * small shapes): with a family forced, a convolution whose shape that family cannot serve fails with
+ * ST_HIP_ERR_UNSUPPORTED instead of silently running another kernel, and the query reports 0 for it.  No reference
+ * counterpart (the reference has one CPU path, conv.rs:2559-2599). */
+enum { ST_HIP_CONV_FAMILY_AUTO = 0, ST_HIP_CONV_FAMILY_TILE = 1, ST_HIP_CONV_FAMILY_RING = 2, ST_HIP_CONV_FAMILY_STRIP = 3 };
+enum {
+    ST_HIP_CONV_KERNEL_TILE = 1,         /* register-staged general kernel                                  */
+    ST_HIP_CONV_KERNEL_RING = 2,         /* direct-to-LDS ring kernel                                       */
+    ST_HIP_CONV_KERNEL_STRIP12 = 3,      /* strip kernel, weight rows padded to 12 words, 32-bit stores     */
+    ST_HIP_CONV_KERNEL_STRIP12_WIDE = 4, /* the same with 128-bit stores through LDS                        */
+    ST_HIP_CONV_KERNEL_STRIP9 = 5,       /* strip kernel, packed weight rows (more than 104 input channels) */
+    ST_HIP_CONV_KERNEL_ADJOINT = 6       /* grad_input only: adjoint gather (stride != 1 or padding > reach) */
+};
+int st_hip_conv2d_force_family(int family);
+int st_hip_conv2d_planned_kernel(size_t batch, size_t c_in, size_t h, size_t w, size_t c_out, size_t kh,
+                                 size_t kw, size_t stride_h, size_t stride_w, size_t pad_h, size_t pad_w,
+                                 size_t dil_h, size_t dil_w, int direction, int *kernel);
+
 /* Conv2d::backward, crates/st-nn/src/layers/conv.rs:780-813 with col2im :860-916: from the forward input
  * (N, C_in, H, W), the OIHW weight and grad_output (N, C_out, OH, OW) computes
  *   grad_input  (N, C_in, H, W)       = col2im(G · W)

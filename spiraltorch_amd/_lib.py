@@ -74,6 +74,8 @@ SIGNATURES = {
     "st_hip_gemm_bf16_f32acc": (c_int, [c_size_t, c_size_t, c_size_t, c_void_p, c_size_t, c_void_p, c_size_t,
                                         c_void_p, c_size_t]),
     "st_hip_conv2d_output_hw": (c_int, [c_size_t] * 10 + [POINTER(c_size_t), POINTER(c_size_t)]),
+    "st_hip_conv2d_force_family": (c_int, [c_int]),
+    "st_hip_conv2d_planned_kernel": (c_int, [c_size_t] * 13 + [c_int, POINTER(c_int)]),
     "st_hip_conv2d_bias_act_f32": (c_int, [c_size_t] * 13 + [c_int, c_void_p, c_size_t, c_void_p, c_size_t,
                                                              c_void_p, c_size_t, c_void_p, c_size_t]),
     "st_hip_attention_f32": (c_int, [c_size_t, c_size_t, c_size_t, c_float, c_int, c_void_p, c_size_t, c_void_p,

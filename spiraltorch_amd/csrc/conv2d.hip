@@ -23,8 +23,7 @@
 #include "device_math.h"
 #include "kernels.h"
 
-#include <cstdlib>
-#include <cstring>
+#include <atomic>
 #include <type_traits>
 
 namespace sthip {
@@ -771,14 +770,13 @@ bool plan_strip(const ConvShape &shape, bool forced, StripArgs &args)
     return true;
 }
 
-hipError_t launch_strip(StripArgs args, hipStream_t stream)
+hipError_t launch_strip(StripArgs args, int which, hipStream_t stream)
 {
     size_t lds_bytes = strip_lds_bytes(args.s.c_in);
-    const bool wide = strip_pitch(args.s.c_in) == 12 && args.spatial % 4 == 0 &&
-                      (reinterpret_cast<uintptr_t>(args.out) & 15u) == 0 && lds_bytes + kStripStageBytes <= 160 * 1024;
-    if (wide) lds_bytes += kStripStageBytes;
-    auto kernel = wide ? conv2d_f32_strip12_wide_kernel
-                  : strip_pitch(args.s.c_in) == 12 ? conv2d_f32_strip12_kernel : conv2d_f32_strip9_kernel;
+    if (which == ST_HIP_CONV_KERNEL_STRIP12_WIDE) lds_bytes += kStripStageBytes;
+    auto kernel = which == ST_HIP_CONV_KERNEL_STRIP12_WIDE ? conv2d_f32_strip12_wide_kernel
+                  : which == ST_HIP_CONV_KERNEL_STRIP12    ? conv2d_f32_strip12_kernel
+                                                           : conv2d_f32_strip9_kernel;
     hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                         static_cast<int>(lds_bytes));
     if (rc != hipSuccess) return rc;
@@ -839,7 +837,57 @@ hipError_t launch_tile(ConvArgs args, bool vec, hipStream_t stream)
     return hipGetLastError();
 }
 
+// Kernel family forced by st_hip_conv2d_force_family (a diagnostic hook: the parity tests use it to run every family
+// on small shapes); ST_HIP_CONV_FAMILY_AUTO in normal use.
+std::atomic<int> g_forced_family{ST_HIP_CONV_FAMILY_AUTO};
+
+// The dispatcher's decision for `shape`: one of ST_HIP_CONV_KERNEL_*, or 0 when a forced family cannot serve the
+// shape.  `strip` is filled when a strip kernel is chosen.
+int choose_conv_kernel(const ConvShape &shape, bool weight_aligned, bool out_aligned, int forced, StripArgs &strip)
+{
+    const int K = shape.c_in * shape.kh * shape.kw;
+    const int spatial = shape.oh * shape.ow;
+    const bool vec = (K % 4 == 0) && weight_aligned;
+    // Both direct-load kernels address one image through 32-bit byte offsets with the top bits spare.
+    const bool image_ok = static_cast<size_t>(shape.c_in) * shape.h * shape.w * 4 < (1ull << 30);
+    // 8 wavefronts of 32×32 per 128×64 tile measured best for wide layers (128×128 tiles, 32-deep k-tiles and
+    // 4-wavefront layouts were all 10-20 % slower on the 64->128 channel 56×56 case).
+    const bool ring_ok = vec && K % 16 == 0 && shape.kh * shape.kw <= 32 && image_ok &&
+                         (static_cast<size_t>(shape.pad_h) * shape.w + shape.pad_w) * 4 < (1ull << 30) &&
+                         (static_cast<size_t>(shape.oh + 64) * shape.stride_h * shape.w + static_cast<size_t>(shape.ow) * shape.stride_w) * 4 < (1ull << 30) &&
+                         static_cast<size_t>(shape.c_out) * K * 4 < (1ull << 31);
+    auto strip_kernel = [&]() {
+        if (strip_pitch(shape.c_in) != 12) return ST_HIP_CONV_KERNEL_STRIP9;
+        const bool wide = spatial % 4 == 0 && out_aligned &&
+                          strip_lds_bytes(shape.c_in) + kStripStageBytes <= 160 * 1024;
+        return wide ? ST_HIP_CONV_KERNEL_STRIP12_WIDE : ST_HIP_CONV_KERNEL_STRIP12;
+    };
+    switch (forced) {
+    case ST_HIP_CONV_FAMILY_TILE: return ST_HIP_CONV_KERNEL_TILE;
+    case ST_HIP_CONV_FAMILY_RING: return ring_ok ? ST_HIP_CONV_KERNEL_RING : 0;
+    case ST_HIP_CONV_FAMILY_STRIP: return image_ok && plan_strip(shape, true, strip) ? strip_kernel() : 0;
+    default: break;
+    }
+    if (!ring_ok) return ST_HIP_CONV_KERNEL_TILE;
+    // The ring kernel has the better steady state (several rounds of 128×64 tiles per compute unit); the strip
+    // kernel, balanced to the single SIMD, wins when the ring kernel's tiles would fill the chip fewer than
+    // 1.75 times (1024 resident tiles) and for 64 or fewer output channels.
+    const long long ring_tiles = static_cast<long long>(shape.batch) * ((spatial + 63) / 64) * ((shape.c_out + 127) / 128);
+    const bool prefer_strip = shape.c_out <= 64 || ring_tiles < 1792;
+    if (prefer_strip && plan_strip(shape, false, strip)) return strip_kernel();
+    return ST_HIP_CONV_KERNEL_RING;
+}
+
 }  // namespace
+
+void set_conv_forced_family(int family) { g_forced_family.store(family, std::memory_order_relaxed); }
+
+int planned_conv_kernel(const ConvShape &shape, bool weight_aligned, bool out_aligned)
+{
+    if (shape.kh * shape.kw * static_cast<long long>(shape.c_in) > kConvMaxReduction) return 0;
+    StripArgs strip;
+    return choose_conv_kernel(shape, weight_aligned, out_aligned, g_forced_family.load(std::memory_order_relaxed), strip);
+}
 
 hipError_t launch_conv2d_f32(const ConvShape &shape, int activation, const float *input, const float *weight,
                              const float *bias, float *out, hipStream_t stream)
@@ -860,40 +908,32 @@ hipError_t launch_conv2d_f32(const ConvShape &shape, int activation, const float
     if ((shape.kh - 1) * static_cast<long long>(shape.dil_h) > 0x7fff ||
         (shape.kw - 1) * static_cast<long long>(shape.dil_w) > 0x7fff || args.K > kConvMaxReduction)
         return hipErrorInvalidValue;
-    const bool vec = (args.K % 4 == 0) && ((reinterpret_cast<uintptr_t>(weight) & 15u) == 0);
-    // 8 wavefronts of 32×32 per 128×64 tile measured best for wide layers (128×128 tiles, 32-deep k-tiles and
-    // 4-wavefront layouts were all 10-20 % slower on the 64->128 channel 56×56 case).
-    const bool ring_ok = vec && args.K % 16 == 0 && shape.kh * shape.kw <= 32 &&
-                         static_cast<size_t>(shape.c_in) * shape.h * shape.w * 4 < (1ull << 30) &&
-                         (static_cast<size_t>(shape.pad_h) * shape.w + shape.pad_w) * 4 < (1ull << 30) &&
-                         (static_cast<size_t>(shape.oh + 64) * shape.stride_h * shape.w + static_cast<size_t>(shape.ow) * shape.stride_w) * 4 < (1ull << 30) &&
-                         static_cast<size_t>(shape.c_out) * args.K * 4 < (1ull << 31);
-    // ST_HIP_CONV_KERNEL=strip|ring|tile overrides the choice between the kernel families for shapes that fit the
-    // named family (the parity tests use it to run every family on small shapes).
-    const char *forced = std::getenv("ST_HIP_CONV_KERNEL");
-    const bool force_strip = forced && std::strcmp(forced, "strip") == 0;
-    const bool force_ring = forced && std::strcmp(forced, "ring") == 0;
-    const bool force_tile = forced && std::strcmp(forced, "tile") == 0;
-    if (ring_ok && !force_tile) {
-        // The ring kernel has the better steady state (several rounds of 128×64 tiles per compute unit); the strip
-        // kernel, balanced to the single SIMD, wins when the ring kernel's tiles would fill the chip fewer than
-        // 1.75 times (1024 resident tiles) and for 64 or fewer output channels.
-        const long long ring_tiles = static_cast<long long>(shape.batch) * ((args.spatial + 63) / 64) * ((shape.c_out + 127) / 128);
-        const bool prefer_strip = force_strip || shape.c_out <= 64 || ring_tiles < 1792;
-        StripArgs strip;
-        if (!force_ring && prefer_strip && plan_strip(shape, force_strip, strip)) {
-            strip.input = input;
-            strip.weight = weight;
-            strip.bias = bias;
-            strip.out = out;
-            strip.s = shape;
-            strip.activation = activation;
-            return launch_strip(strip, stream);
-        }
+    const bool weight_aligned = (reinterpret_cast<uintptr_t>(weight) & 15u) == 0;
+    const bool out_aligned = (reinterpret_cast<uintptr_t>(out) & 15u) == 0;
+    StripArgs strip;
+    const int kernel = choose_conv_kernel(shape, weight_aligned, out_aligned,
+                                          g_forced_family.load(std::memory_order_relaxed), strip);
+    switch (kernel) {
+    case ST_HIP_CONV_KERNEL_STRIP12:
+    case ST_HIP_CONV_KERNEL_STRIP12_WIDE:
+    case ST_HIP_CONV_KERNEL_STRIP9:
+        strip.input = input;
+        strip.weight = weight;
+        strip.bias = bias;
+        strip.out = out;
+        strip.s = shape;
+        strip.activation = activation;
+        return launch_strip(strip, kernel, stream);
+    case ST_HIP_CONV_KERNEL_RING:
         return shape.c_out > 64 ? launch_ring<128>(args, stream) : launch_ring<64>(args, stream);
+    case ST_HIP_CONV_KERNEL_TILE: {
+        const bool vec = (args.K % 4 == 0) && weight_aligned;
+        if (shape.c_out > 64) return launch_tile<128, 64, 16, 4, 2>(args, vec, stream);
+        return launch_tile<64, 64, 16, 2, 2>(args, vec, stream);
     }
-    if (shape.c_out > 64) return launch_tile<128, 64, 16, 4, 2>(args, vec, stream);
-    return launch_tile<64, 64, 16, 2, 2>(args, vec, stream);
+    default:
+        return hipErrorInvalidConfiguration;  // a forced family that cannot serve the shape (entry points check first)
+    }
 }
 
 // Adjoint gather for strides other than 1: `shape` describes the virtual forward problem (see TRANSPOSED above).

@@ -379,24 +379,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
 
 }  // namespace
 
-hipError_t launch_conv2d_grad_input_f32(const ConvShape &shape, const float *grad_output, const float *weight,
-                                        float *grad_input, hipStream_t stream)
+namespace {
+// grad_input as a forward problem: grad_output is the image, input positions are the output pixels.  True when the
+// forward kernels can run it (stride 1 and a non-negative adjoint padding); `t` is that problem either way, with
+// the original stride/padding when the adjoint gather has to run instead.
+bool grad_input_as_forward(const ConvShape &shape, ConvShape &t)
 {
-    if (shape.batch == 0 || shape.c_in == 0 || shape.h == 0 || shape.w == 0) return hipSuccess;
-    const size_t weight_count = static_cast<size_t>(shape.c_out) * shape.c_in * shape.kh * shape.kw;
     const int adj_pad_h = shape.dil_h * (shape.kh - 1) - shape.pad_h;
     const int adj_pad_w = shape.dil_w * (shape.kw - 1) - shape.pad_w;
     const bool as_forward = shape.stride_h == 1 && shape.stride_w == 1 && adj_pad_h >= 0 && adj_pad_w >= 0;
-    void *workspace = nullptr;
-    hipError_t rc = stream_workspace(stream, weight_count * sizeof(float), &workspace);
-    if (rc != hipSuccess) return rc;
-    float *adjoint_weight = static_cast<float *>(workspace);
-    hipLaunchKernelGGL(conv_weight_to_adjoint_kernel, dim3(static_cast<unsigned>((weight_count + 255) / 256)), dim3(256), 0,
-                       stream, shape.c_out, shape.c_in, shape.kh, shape.kw, as_forward ? 1 : 0, weight, adjoint_weight);
-    rc = hipGetLastError();
-    if (rc != hipSuccess) return rc;
-    // The virtual forward problem: grad_output is the image, input positions are the output pixels.
-    ConvShape t = shape;
+    t = shape;
     t.c_in = shape.c_out;
     t.h = shape.oh;
     t.w = shape.ow;
@@ -406,8 +398,35 @@ hipError_t launch_conv2d_grad_input_f32(const ConvShape &shape, const float *gra
     if (as_forward) {
         t.pad_h = adj_pad_h;
         t.pad_w = adj_pad_w;
-        return launch_conv2d_f32(t, ST_HIP_ACT_NONE, grad_output, adjoint_weight, nullptr, grad_input, stream);
     }
+    return as_forward;
+}
+}  // namespace
+
+int planned_conv_grad_input_kernel(const ConvShape &shape)
+{
+    ConvShape t;
+    if (!grad_input_as_forward(shape, t)) return ST_HIP_CONV_KERNEL_ADJOINT;
+    return planned_conv_kernel(t, true, true);
+}
+
+hipError_t launch_conv2d_grad_input_f32(const ConvShape &shape, const float *grad_output, const float *weight,
+                                        float *grad_input, hipStream_t stream)
+{
+    if (shape.batch == 0 || shape.c_in == 0 || shape.h == 0 || shape.w == 0) return hipSuccess;
+    const size_t weight_count = static_cast<size_t>(shape.c_out) * shape.c_in * shape.kh * shape.kw;
+    ConvShape t;
+    const bool as_forward = grad_input_as_forward(shape, t);
+    void *workspace = nullptr;
+    hipError_t rc = stream_workspace(stream, weight_count * sizeof(float), &workspace);
+    if (rc != hipSuccess) return rc;
+    float *adjoint_weight = static_cast<float *>(workspace);
+    hipLaunchKernelGGL(conv_weight_to_adjoint_kernel, dim3(static_cast<unsigned>((weight_count + 255) / 256)), dim3(256), 0,
+                       stream, shape.c_out, shape.c_in, shape.kh, shape.kw, as_forward ? 1 : 0, weight, adjoint_weight);
+    rc = hipGetLastError();
+    if (rc != hipSuccess) return rc;
+    if (as_forward)
+        return launch_conv2d_f32(t, ST_HIP_ACT_NONE, grad_output, adjoint_weight, nullptr, grad_input, stream);
     return launch_conv2d_adjoint_f32(t, grad_output, adjoint_weight, grad_input, stream);
 }
 

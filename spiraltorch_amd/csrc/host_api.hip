@@ -244,6 +244,20 @@ int plan_conv(size_t batch, size_t c_in, size_t h, size_t w, size_t c_out, size_
     return ST_HIP_OK;
 }
 
+// With a kernel family forced (st_hip_conv2d_force_family), a shape that family cannot serve is an error rather
+// than a silent switch to another kernel.
+int check_conv_family(const ConvShape &shape, int direction, const void *weight, const void *out)
+{
+    const bool weight_aligned = (reinterpret_cast<uintptr_t>(weight) & 15u) == 0;
+    const bool out_aligned = (reinterpret_cast<uintptr_t>(out) & 15u) == 0;
+    const int kernel = direction == 0 ? planned_conv_kernel(shape, weight_aligned, out_aligned)
+                                      : planned_conv_grad_input_kernel(shape);
+    if (kernel == 0)
+        return fail(ST_HIP_ERR_UNSUPPORTED, "the forced conv2d kernel family cannot serve this shape (%s)",
+                    direction == 0 ? "forward" : "grad_input");
+    return ST_HIP_OK;
+}
+
 struct AttentionPlan {
     size_t rows, qkv_len, z_len, bias_len;
 };
@@ -424,6 +438,26 @@ int st_hip_conv2d_output_hw(size_t h, size_t w, size_t kh, size_t kw, size_t str
     return ST_HIP_OK;
 }
 
+int st_hip_conv2d_force_family(int family)
+{
+    if (family < ST_HIP_CONV_FAMILY_AUTO || family > ST_HIP_CONV_FAMILY_STRIP)
+        return fail(ST_HIP_ERR_INVALID, "unknown conv2d kernel family %d", family);
+    set_conv_forced_family(family);
+    return ST_HIP_OK;
+}
+
+int st_hip_conv2d_planned_kernel(size_t batch, size_t c_in, size_t h, size_t w, size_t c_out, size_t kh, size_t kw,
+                                 size_t stride_h, size_t stride_w, size_t pad_h, size_t pad_w, size_t dil_h,
+                                 size_t dil_w, int direction, int *kernel)
+{
+    if (!kernel) return fail(ST_HIP_ERR_INVALID, "conv2d planned_kernel received a null out-pointer");
+    if (direction != 0 && direction != 1) return fail(ST_HIP_ERR_INVALID, "unknown conv2d direction %d", direction);
+    ConvPlan plan;
+    ST_HIP_CHECK(plan_conv(batch, c_in, h, w, c_out, kh, kw, stride_h, stride_w, pad_h, pad_w, dil_h, dil_w, &plan));
+    *kernel = direction == 0 ? planned_conv_kernel(plan.shape, true, true) : planned_conv_grad_input_kernel(plan.shape);
+    return ST_HIP_OK;
+}
+
 int st_hip_conv2d_bias_act_f32(size_t batch, size_t c_in, size_t h, size_t w, size_t c_out, size_t kh, size_t kw,
                                size_t stride_h, size_t stride_w, size_t pad_h, size_t pad_w, size_t dil_h,
                                size_t dil_w, int activation, const float *input, size_t input_len,
@@ -457,6 +491,7 @@ int st_hip_conv2d_bias_act_f32(size_t batch, size_t c_in, size_t h, size_t w, si
     ST_HIP_CHECK(lease.upload(1, weight, weight_len * sizeof(float), &d_w));
     ST_HIP_CHECK(lease.buffer(2, out_len * sizeof(float), &d_out));
     if (bias) ST_HIP_CHECK(lease.upload(3, bias, bias_len * sizeof(float), &d_bias));
+    ST_HIP_CHECK(check_conv_family(plan.shape, 0, d_w, d_out));
     ST_HIP_CHECK(launch_status(launch_conv2d_f32(plan.shape, activation, static_cast<const float *>(d_in),
                                                  static_cast<const float *>(d_w), static_cast<const float *>(d_bias),
                                                  static_cast<float *>(d_out), lease.stream()),
@@ -499,6 +534,7 @@ int st_hip_conv2d_backward_f32(size_t batch, size_t c_in, size_t h, size_t w, si
     ST_HIP_CHECK(reject_null(grad_weight, grad_weight_len, "conv2d backward"));
     ST_HIP_CHECK(reject_null(grad_bias, grad_bias_len, "conv2d backward"));
     if (batch == 0) return ST_HIP_OK;  // conv.rs:787-789: an empty batch leaves the parameter gradients untouched
+    ST_HIP_CHECK(check_conv_family(plan.shape, 1, nullptr, nullptr));
 
     Lease lease;
     ST_HIP_CHECK(lease.status());
@@ -690,6 +726,7 @@ int st_hip_conv2d_bias_act_f32_dev(size_t batch, size_t c_in, size_t h, size_t w
     if (plan.out_len == 0) return ST_HIP_OK;
     if (!input || !weight || !out)
         return fail(ST_HIP_ERR_INVALID, "conv2d received a null pointer; provide contiguous buffers");
+    ST_HIP_CHECK(check_conv_family(plan.shape, 0, weight, out));
     return launch_status(launch_conv2d_f32(plan.shape, activation, input, weight, bias, out, as_stream(stream)),
                          "conv2d launch");
 }
@@ -708,6 +745,7 @@ int st_hip_conv2d_grad_input_f32_dev(size_t batch, size_t c_in, size_t h, size_t
     if (plan.input_len == 0) return ST_HIP_OK;
     if (!grad_output || !weight || !grad_input)
         return fail(ST_HIP_ERR_INVALID, "conv2d backward received a null pointer; provide contiguous buffers");
+    ST_HIP_CHECK(check_conv_family(plan.shape, 1, nullptr, nullptr));
     return launch_status(launch_conv2d_grad_input_f32(plan.shape, grad_output, weight, grad_input, as_stream(stream)),
                          "conv2d grad_input launch");
 }

@@ -38,6 +38,12 @@ constexpr int kConvMaxReduction = 8192;
 hipError_t launch_conv2d_f32(const ConvShape &shape, int activation, const float *input,
                              const float *weight, const float *bias, float *out, hipStream_t stream);
 
+// Which kernel launch_conv2d_f32 would run for `shape` (one of ST_HIP_CONV_KERNEL_*; 0 when the family forced with
+// set_conv_forced_family cannot serve it), and the same for launch_conv2d_grad_input_f32 on the forward `shape`.
+int planned_conv_kernel(const ConvShape &shape, bool weight_aligned, bool out_aligned);
+int planned_conv_grad_input_kernel(const ConvShape &shape);
+void set_conv_forced_family(int family);
+
 // Adjoint gather of the implicit GEMM (`shape` is the virtual forward problem: grad_output as the image, input
 // positions as output pixels, original stride/padding/dilation; weight laid out [c_in][c_out·kh·kw]).
 hipError_t launch_conv2d_adjoint_f32(const ConvShape &shape, const float *grad_output,

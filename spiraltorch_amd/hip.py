@@ -163,6 +163,26 @@ def conv2d_output_hw(h, w, kernel, stride, padding, dilation):
     return oh.value, ow.value
 
 
+CONV_FAMILIES = {"auto": 0, "tile": 1, "ring": 2, "strip": 3}
+CONV_KERNELS = {0: None, 1: "tile", 2: "ring", 3: "strip12", 4: "strip12_wide", 5: "strip9", 6: "adjoint"}
+
+
+def conv2d_force_family(family: str) -> None:
+    """Process-wide diagnostic switch: "auto" (the dispatcher decides), "tile", "ring" or "strip".  With a family
+    forced, a shape it cannot serve raises HipErr instead of running another kernel."""
+    _check(_lib.load().st_hip_conv2d_force_family(CONV_FAMILIES[family]))
+
+
+def conv2d_planned_kernel(batch, c_in, h, w, c_out, kernel, stride, padding, dilation, direction="forward"):
+    """Name of the kernel the dispatcher runs for this shape ("forward" or "grad_input"); None when the forced
+    family cannot serve it."""
+    which = ctypes.c_int()
+    _check(_lib.load().st_hip_conv2d_planned_kernel(
+        batch, c_in, h, w, c_out, kernel[0], kernel[1], stride[0], stride[1], padding[0], padding[1], dilation[0],
+        dilation[1], {"forward": 0, "grad_input": 1}[direction], ctypes.byref(which)))
+    return CONV_KERNELS[which.value]
+
+
 def conv2d_bias_activation_f32(batch, c_in, h, w, c_out, kernel, stride, padding, dilation, activation,
                                input, weight, bias, out) -> None:
     x, wgt, out = _f32(input, "input"), _f32(weight, "weight"), _out(out, "out")

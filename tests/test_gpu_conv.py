@@ -68,37 +68,103 @@ def test_random_shapes(hip, oracle, shape):
     assert_close(got, oracle.conv2d_bias_act_f32(*shape, oracle.ACT_RELU, x, wt, None), F32_REL, F32_ABS, "no bias")
 
 
-FAMILY_SHAPES = [
-    (2, 16, 20, 20, 70, (3, 3), (1, 1), (1, 1), (1, 1)),    # ragged channel strip, 13 pixel blocks, ragged last block
-    (1, 130, 12, 12, 40, (3, 3), (1, 1), (1, 1), (1, 1)),   # three weight slices (64 + 64 + 2 channels), idle wavefronts
-    (1, 4, 60, 60, 33, (3, 3), (1, 1), (1, 1), (1, 1)),     # several pixel chunks per image
-    (5, 8, 13, 12, 64, (3, 3), (2, 2), (0, 0), (1, 1)),     # stride 2
-    (2, 6, 15, 14, 32, (3, 3), (1, 2), (2, 3), (2, 1)),     # dilation, wide padding, odd channel pairs
-    (2, 32, 9, 9, 16, (1, 9), (1, 1), (0, 4), (1, 1)),      # nine taps in one row
-    (64, 2, 42, 42, 128, (3, 3), (1, 1), (1, 1), (1, 1)),   # 56 blocks per workgroup: seven per wavefront
-    (64, 2, 44, 32, 128, (3, 3), (1, 1), (1, 1), (1, 1)),   # 44 blocks: six and five per wavefront
+G33 = ((3, 3), (1, 1), (1, 1), (1, 1))
+FAMILY_SHAPES = {
+    # name: (batch, c_in, h, w, c_out, kernel, stride, padding, dilation)
+    "ragged_strip": (2, 16, 20, 20, 70, *G33),           # ragged channel strip, 13 pixel blocks, ragged last block
+    "c130": (1, 130, 12, 12, 40, *G33),                  # packed weight rows, K % 4 != 0: scalar weight staging
+    "chunks_c4": (1, 4, 60, 60, 33, *G33),               # several pixel chunks per image
+    "stride2_c8": (5, 8, 13, 12, 64, (3, 3), (2, 2), (0, 0), (1, 1)),
+    "dilated_c6": (2, 6, 15, 14, 32, (3, 3), (1, 2), (2, 3), (2, 1)),   # dilation, wide padding, three channel pairs
+    "row_of_nine": (2, 32, 9, 9, 16, (1, 9), (1, 1), (0, 4), (1, 1)),    # nine taps in one row
+    "blocks56": (64, 2, 42, 42, 128, *G33),              # 56 blocks per workgroup: seven per wavefront
+    "blocks44": (64, 2, 44, 32, 128, *G33),              # 44 blocks: six and five per wavefront
+    "c112": (2, 112, 14, 14, 40, *G33),                  # packed rows (more than 104 channels), ragged second strip
+    "c128_odd_plane": (3, 128, 11, 13, 70, *G33),        # packed rows, plane of 143 pixels (not a multiple of 4)
+    "c96": (2, 96, 12, 12, 64, *G33),                    # padded rows but no LDS left for the 128-bit store path
+    "stride2_c32": (2, 32, 21, 21, 48, (3, 3), (2, 2), (1, 1), (1, 1)),  # stride 2, plane of 121 pixels
+    "dilated_c48": (2, 48, 19, 17, 33, (3, 3), (1, 1), (2, 2), (2, 2)),  # dilation 2, plane of 323 pixels
+    "chunks_c16": (1, 16, 64, 64, 32, *G33),             # 128 blocks of one image split over several workgroups
+    "fuzz_c64_p0": (3, 64, 33, 33, 160, (3, 3), (1, 1), (0, 0), (1, 1)),  # no padding, two channel tiles
+    "ring64": (2, 16, 20, 20, 40, *G33),                 # 64-row ring tiles
+    "ring_5x5": (2, 16, 15, 15, 130, (5, 5), (1, 1), (2, 2), (1, 1)),    # 25 taps, ragged channel tile
+}
+# (shape, forced family, the kernel that has to run)
+FAMILY_CASES = [
+    ("ragged_strip", "strip", "strip12_wide"), ("c130", "strip", "strip9"), ("chunks_c4", "strip", "strip12_wide"),
+    ("stride2_c8", "strip", "strip12"), ("dilated_c6", "strip", "strip12"), ("row_of_nine", "strip", "strip12"),
+    ("blocks56", "strip", "strip12_wide"), ("blocks44", "strip", "strip12_wide"), ("c112", "strip", "strip9"),
+    ("c128_odd_plane", "strip", "strip9"), ("c96", "strip", "strip12"), ("stride2_c32", "strip", "strip12"),
+    ("dilated_c48", "strip", "strip12"), ("chunks_c16", "strip", "strip12_wide"), ("fuzz_c64_p0", "strip", "strip12"),
+    ("ragged_strip", "ring", "ring"), ("row_of_nine", "ring", "ring"), ("c112", "ring", "ring"),
+    ("c128_odd_plane", "ring", "ring"), ("stride2_c32", "ring", "ring"), ("dilated_c48", "ring", "ring"),
+    ("chunks_c16", "ring", "ring"), ("fuzz_c64_p0", "ring", "ring"), ("ring64", "ring", "ring"),
+    ("ring_5x5", "ring", "ring"),
+    ("ragged_strip", "tile", "tile"), ("c130", "tile", "tile"), ("chunks_c4", "tile", "tile"),
+    ("stride2_c8", "tile", "tile"), ("dilated_c6", "tile", "tile"), ("row_of_nine", "tile", "tile"),
+    ("blocks56", "tile", "tile"), ("c112", "tile", "tile"), ("stride2_c32", "tile", "tile"),
+    ("dilated_c48", "tile", "tile"), ("ring_5x5", "tile", "tile"),
 ]
 
 
-@pytest.mark.parametrize("family", ["strip", "ring", "tile"])
-@pytest.mark.parametrize("shape", FAMILY_SHAPES)
-def test_kernel_families(hip, oracle, monkeypatch, family, shape):
-    """Each kernel family (chosen by shape in normal use) forced on shapes that exercise its edges."""
-    monkeypatch.setenv("ST_HIP_CONV_KERNEL", family)
-    batch, c_in, h, w, c_out, kernel, stride, padding, dilation = shape
+@pytest.fixture
+def force_family(hip):
+    """Forces a conv kernel family for one test and gives the choice back to the dispatcher afterwards."""
+    yield hip.conv2d_force_family
+    hip.conv2d_force_family("auto")
+
+
+@pytest.mark.parametrize("name,family,kernel", FAMILY_CASES)
+def test_kernel_families(hip, oracle, force_family, name, family, kernel):
+    """Each kernel family (chosen by shape in normal use) forced on shapes that exercise its edges; the dispatcher
+    is asked which kernel it runs, so a case cannot pass on another family's kernel."""
+    shape = FAMILY_SHAPES[name]
+    force_family(family)
+    assert hip.conv2d_planned_kernel(*shape) == kernel
+    batch, c_in, h, w, c_out, kernel_hw, stride, padding, dilation = shape
     rng = np.random.default_rng(batch * 1000 + c_in * 10 + c_out)
     x = rng.normal(size=batch * c_in * h * w).astype(np.float32)
-    wt = rng.normal(0, np.sqrt(2.0 / (c_in * 9)), c_out * c_in * 9).astype(np.float32)
+    wt = rng.normal(0, np.sqrt(2.0 / (c_in * 9)), c_out * c_in * kernel_hw[0] * kernel_hw[1]).astype(np.float32)
     b = rng.uniform(-0.1, 0.1, c_out).astype(np.float32)
     got = run(hip, *shape, 1, x, wt, b)
     want = oracle.conv2d_bias_act_f32(*shape, oracle.ACT_RELU, x, wt, b, threads=8)
-    assert_close(got, want, F32_REL, F32_ABS, f"conv {shape} family={family}")
+    assert_close(got, want, F32_REL, F32_ABS, f"conv {name} {shape} family={family}")
 
 
-def test_strip_kernel_store_paths_agree(hip, oracle, monkeypatch):
+def test_forced_family_that_cannot_serve_is_an_error(hip, force_family):
+    """A forced family never silently falls back: the ring kernel needs c_in*kh*kw % 16 == 0, the strip kernel nine
+    taps and an even channel count."""
+    shape = (1, 4, 8, 8, 8, *G33)
+    x, wt = np.zeros(4 * 64, np.float32), np.zeros(8 * 36, np.float32)
+    out = np.full(8 * 64, 13.0, np.float32)
+    force_family("ring")
+    assert hip.conv2d_planned_kernel(*shape) is None
+    with pytest.raises(hip.HipErr, match="forced conv2d kernel family cannot serve"):
+        hip.conv2d_bias_activation_f32(*shape, 0, x, wt, None, out)
+    force_family("strip")
+    odd = (1, 3, 8, 8, 8, *G33)
+    assert hip.conv2d_planned_kernel(*odd) is None
+    with pytest.raises(hip.HipErr, match="forced conv2d kernel family cannot serve"):
+        hip.conv2d_bias_activation_f32(*odd, 0, np.zeros(3 * 64, np.float32), np.zeros(8 * 27, np.float32), None, out)
+    assert (out == 13.0).all()
+    with pytest.raises(hip.HipErr, match="unknown conv2d kernel family"):
+        hip._check(hip._lib.load().st_hip_conv2d_force_family(9))
+
+
+def test_dispatcher_choices(hip):
+    """What runs without forcing: config 2 and its grad_input on the strip kernels, many-tile layers on the ring
+    kernel, reductions that are not a multiple of 16 on the general kernel."""
+    assert hip.conv2d_planned_kernel(32, 64, 56, 56, 128, *G33) == "strip12_wide"
+    assert hip.conv2d_planned_kernel(32, 64, 56, 56, 128, *G33, direction="grad_input") == "strip9"
+    assert hip.conv2d_planned_kernel(64, 64, 56, 56, 256, *G33) == "ring"
+    assert hip.conv2d_planned_kernel(8, 3, 32, 32, 16, *G33) == "tile"
+    assert hip.conv2d_planned_kernel(2, 8, 9, 9, 4, (3, 3), (2, 2), (1, 1), (1, 1), direction="grad_input") == "adjoint"
+
+
+def test_strip_kernel_store_paths_agree(hip, oracle, force_family):
     """The strip kernel stores 128 bits per lane through an LDS tile when the output is 16-byte aligned and the
     plane size is a multiple of four, 32 bits per lane otherwise: same values either way."""
-    monkeypatch.setenv("ST_HIP_CONV_KERNEL", "strip")
+    force_family("strip")
     shape = (3, 16, 20, 20, 70, (3, 3), (1, 1), (1, 1), (1, 1))
     batch, c_in, h, w, c_out, kernel, stride, padding, dilation = shape
     rng = np.random.default_rng(77)
