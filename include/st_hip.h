@@ -211,6 +211,19 @@ int st_hip_conv2d_grad_input_f32_dev(size_t batch, size_t c_in, size_t h, size_t
                                      size_t pad_h, size_t pad_w, size_t dil_h, size_t dil_w,
                                      const float *grad_output, const float *weight,
                                      float *grad_input, void *stream);
+/* No counterpart in the reference.  st_hip_conv2d_grad_input_f32_dev for callers that cannot allocate device
+ * memory (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): same arguments, same
+ * kernels and bit-identical results, but the flipped weights the kernels read go to a static device array of
+ * ST_HIP_NOALLOC_SCRATCH_BYTES instead of the stream's grow-on-demand workspace, and the call performs no hipMalloc /
+ * hipFree on any path.  c_out*c_in*kh*kw*4 bytes must fit the array, otherwise ST_HIP_ERR_UNSUPPORTED (nothing is
+ * launched).  Every call on a GPU shares that GPU's array: calls that overlap on one GPU (different streams or
+ * threads) race; calls on one stream are ordered and safe.  st_hip_init must have succeeded first. */
+#define ST_HIP_NOALLOC_SCRATCH_BYTES (16u << 20)
+int st_hip_conv2d_grad_input_f32_noalloc_dev(size_t batch, size_t c_in, size_t h, size_t w, size_t c_out,
+                                             size_t kh, size_t kw, size_t stride_h, size_t stride_w,
+                                             size_t pad_h, size_t pad_w, size_t dil_h, size_t dil_w,
+                                             const float *grad_output, const float *weight,
+                                             float *grad_input, void *stream);
 int st_hip_conv2d_grad_weight_f32_dev(size_t batch, size_t c_in, size_t h, size_t w, size_t c_out,
                                       size_t kh, size_t kw, size_t stride_h, size_t stride_w,
                                       size_t pad_h, size_t pad_w, size_t dil_h, size_t dil_w,

@@ -102,6 +102,7 @@ SIGNATURES = {
     "st_hip_pack_rhs_f32_dev": (c_int, [c_size_t, c_size_t, c_void_p, c_void_p, c_void_p]),
     "st_hip_conv2d_backward_f32": (c_int, [c_size_t] * 13 + [c_void_p, c_size_t] * 6),
     "st_hip_conv2d_grad_input_f32_dev": (c_int, [c_size_t] * 13 + [c_void_p, c_void_p, c_void_p, c_void_p]),
+    "st_hip_conv2d_grad_input_f32_noalloc_dev": (c_int, [c_size_t] * 13 + [c_void_p, c_void_p, c_void_p, c_void_p]),
     "st_hip_conv2d_grad_weight_f32_dev": (c_int, [c_size_t] * 13 + [c_void_p, c_void_p, c_float, c_void_p, c_void_p]),
     "st_hip_conv2d_grad_bias_f32_dev": (c_int, [c_size_t] * 13 + [c_void_p, c_float, c_void_p, c_void_p]),
     "st_hip_row_softmax_f32_dev": (c_int, [c_size_t, c_size_t, c_void_p, c_void_p, c_void_p]),

@@ -16,7 +16,41 @@
 #include "device_math.h"
 #include "kernels.h"
 
+#include <mutex>
+
 namespace sthip {
+
+// Scratch of the allocation-free grad_input entry point: the flipped, channel-swapped weights live here instead of
+// in memory from hipMalloc.  Each GPU the library runs on holds its own copy of the array until the process ends.
+// In host code the array's name is only a stand-in for the symbol: its device address on the current GPU comes from
+// hipGetSymbolAddress (noalloc_scratch below), and only that pointer is ever passed to a kernel.
+static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex scratch_mutex;
+void *scratch_ptr[kMaxDevices] = {};
+
+}  // namespace
+
+// Device address of `scratch` on the current GPU, resolved once per device.
+hipError_t noalloc_scratch(void **out)
+{
+    int device = 0;
+    hipError_t rc = hipGetDevice(&device);
+    if (rc != hipSuccess) return rc;
+    if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    if (scratch_ptr[device] == nullptr) {
+        void *ptr = nullptr;
+        rc = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (rc != hipSuccess) return rc;
+        scratch_ptr[device] = ptr;
+    }
+    *out = scratch_ptr[device];
+    return hipSuccess;
+}
 
 namespace {
 
@@ -411,16 +445,20 @@ int planned_conv_grad_input_kernel(const ConvShape &shape)
 }
 
 hipError_t launch_conv2d_grad_input_f32(const ConvShape &shape, const float *grad_output, const float *weight,
-                                        float *grad_input, hipStream_t stream)
+                                        float *grad_input, hipStream_t stream, float *weight_scratch)
 {
     if (shape.batch == 0 || shape.c_in == 0 || shape.h == 0 || shape.w == 0) return hipSuccess;
     const size_t weight_count = static_cast<size_t>(shape.c_out) * shape.c_in * shape.kh * shape.kw;
     ConvShape t;
     const bool as_forward = grad_input_as_forward(shape, t);
-    void *workspace = nullptr;
-    hipError_t rc = stream_workspace(stream, weight_count * sizeof(float), &workspace);
-    if (rc != hipSuccess) return rc;
-    float *adjoint_weight = static_cast<float *>(workspace);
+    hipError_t rc;
+    float *adjoint_weight = weight_scratch;  // room for weight_count values, owned by the caller
+    if (adjoint_weight == nullptr) {
+        void *workspace = nullptr;
+        rc = stream_workspace(stream, weight_count * sizeof(float), &workspace);
+        if (rc != hipSuccess) return rc;
+        adjoint_weight = static_cast<float *>(workspace);
+    }
     hipLaunchKernelGGL(conv_weight_to_adjoint_kernel, dim3(static_cast<unsigned>((weight_count + 255) / 256)), dim3(256), 0,
                        stream, shape.c_out, shape.c_in, shape.kh, shape.kw, as_forward ? 1 : 0, weight, adjoint_weight);
     rc = hipGetLastError();

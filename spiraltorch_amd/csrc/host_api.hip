@@ -750,6 +750,33 @@ int st_hip_conv2d_grad_input_f32_dev(size_t batch, size_t c_in, size_t h, size_t
                          "conv2d grad_input launch");
 }
 
+int st_hip_conv2d_grad_input_f32_noalloc_dev(size_t batch, size_t c_in, size_t h, size_t w, size_t c_out, size_t kh,
+                                             size_t kw, size_t stride_h, size_t stride_w, size_t pad_h, size_t pad_w,
+                                             size_t dil_h, size_t dil_w, const float *grad_output, const float *weight,
+                                             float *grad_input, void *stream)
+{
+    ST_HIP_CHECK(ensure_init());
+    ConvPlan plan;
+    ST_HIP_CHECK(plan_conv(batch, c_in, h, w, c_out, kh, kw, stride_h, stride_w, pad_h, pad_w, dil_h, dil_w, &plan));
+    if (c_out * kh * kw > static_cast<size_t>(kConvMaxReduction))
+        return fail(ST_HIP_ERR_UNSUPPORTED, "conv2d backward reduction extent c_out*kh*kw=%zu exceeds %d", c_out * kh * kw,
+                    kConvMaxReduction);
+    if (plan.weight_len > kNoAllocScratchBytes / sizeof(float))
+        return fail(ST_HIP_ERR_UNSUPPORTED,
+                    "conv2d grad_input without allocation: the weights (%zu bytes) exceed the static scratch of %zu bytes; "
+                    "use st_hip_conv2d_grad_input_f32_dev",
+                    plan.weight_len * sizeof(float), kNoAllocScratchBytes);
+    if (plan.input_len == 0) return ST_HIP_OK;
+    if (!grad_output || !weight || !grad_input)
+        return fail(ST_HIP_ERR_INVALID, "conv2d backward received a null pointer; provide contiguous buffers");
+    ST_HIP_CHECK(check_conv_family(plan.shape, 1, nullptr, nullptr));
+    void *scratch_ptr = nullptr;
+    ST_HIP_TRY(noalloc_scratch(&scratch_ptr), "hipGetSymbolAddress(scratch)");
+    return launch_status(launch_conv2d_grad_input_f32(plan.shape, grad_output, weight, grad_input, as_stream(stream),
+                                                      static_cast<float *>(scratch_ptr)),
+                         "conv2d grad_input launch");
+}
+
 int st_hip_conv2d_grad_weight_f32_dev(size_t batch, size_t c_in, size_t h, size_t w, size_t c_out, size_t kh, size_t kw,
                                       size_t stride_h, size_t stride_w, size_t pad_h, size_t pad_w, size_t dil_h,
                                       size_t dil_w, const float *input, const float *grad_output, float scale,

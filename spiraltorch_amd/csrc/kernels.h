@@ -49,8 +49,12 @@ void set_conv_forced_family(int family);
 hipError_t launch_conv2d_adjoint_f32(const ConvShape &shape, const float *grad_output,
                                      const float *weight_ic_major, float *grad_input, hipStream_t stream);
 // Conv2d backward (crates/st-nn/src/layers/conv.rs:780-813, 860-916); `shape` is the forward shape.
+// The re-laid weights (c_out·c_in·kh·kw values) go to `weight_scratch` when given, else to the stream's workspace.
 hipError_t launch_conv2d_grad_input_f32(const ConvShape &shape, const float *grad_output, const float *weight,
-                                        float *grad_input, hipStream_t stream);
+                                        float *grad_input, hipStream_t stream, float *weight_scratch = nullptr);
+// Static device array behind st_hip_conv2d_grad_input_f32_noalloc_dev: its size, and its address on the current GPU.
+constexpr size_t kNoAllocScratchBytes = ST_HIP_NOALLOC_SCRATCH_BYTES;
+hipError_t noalloc_scratch(void **out);
 hipError_t launch_conv2d_grad_weight_f32(const ConvShape &shape, const float *input, const float *grad_output,
                                          float scale, float *grad_weight, hipStream_t stream);
 hipError_t launch_conv2d_grad_bias_f32(const ConvShape &shape, const float *grad_output, float scale,

@@ -73,6 +73,11 @@ int ensure_init()
                     "HIP not enabled (device 0 is %s; this library carries gfx950 code only)",
                     devices[0].gcnArchName);
     }
+    // Set-up of the allocation-free entry point: the device address of its static scratch array on the current
+    // GPU (other GPUs resolve theirs on their first call with that device current).
+    void *scratch_address = nullptr;
+    rc = noalloc_scratch(&scratch_address);
+    if (rc != hipSuccess) return hip_fail(rc, "hipGetSymbolAddress(scratch)");
     rt.devices.swap(devices);
     rt.ready = true;
     return ST_HIP_OK;

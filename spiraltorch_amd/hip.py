@@ -370,6 +370,18 @@ def conv2d_grad_input_f32_dev(batch, c_in, h, w, c_out, kernel, stride, padding,
         dilation[1], _dev(grad_output), _dev(weight), _dev(grad_input), _stream_ptr(stream)))
 
 
+NOALLOC_SCRATCH_BYTES = 16 << 20
+
+
+def conv2d_grad_input_f32_noalloc_dev(batch, c_in, h, w, c_out, kernel, stride, padding, dilation, grad_output, weight,
+                                      grad_input, stream=None) -> None:
+    """conv2d_grad_input_f32_dev that allocates nothing: the re-laid weights go to a static device array of
+    NOALLOC_SCRATCH_BYTES (larger weights raise HipErr).  Calls that overlap on one GPU race on that array."""
+    _check(_lib.load().st_hip_conv2d_grad_input_f32_noalloc_dev(
+        batch, c_in, h, w, c_out, kernel[0], kernel[1], stride[0], stride[1], padding[0], padding[1], dilation[0],
+        dilation[1], _dev(grad_output), _dev(weight), _dev(grad_input), _stream_ptr(stream)))
+
+
 def conv2d_grad_weight_f32_dev(batch, c_in, h, w, c_out, kernel, stride, padding, dilation, input, grad_output, scale,
                                grad_weight, stream=None) -> None:
     _check(_lib.load().st_hip_conv2d_grad_weight_f32_dev(
