@@ -199,6 +199,14 @@ int st_hip_gemm_bf16_bias_act_dev(size_t m, size_t n, size_t k, int activation,
                                   const uint16_t *lhs, const uint16_t *rhs, const float *bias,
                                   const float *residual, float *out_f32, uint16_t *out_bf16,
                                   void *stream);
+/* The same with B prepacked as its n×k transpose — PackedB's column-major layout (crates/st-tensor/src/pure.rs:
+ * 1285-1323; what Linear::forward passes, crates/st-nn/src/layers/linear.rs:96-104), in bf16 storage — and the packing
+ * itself on the device.  With both operands k-contiguous neither needs transposing on its way to the matrix cores. */
+int st_hip_gemm_bf16_prepacked_bias_act_dev(size_t m, size_t n, size_t k, int activation,
+                                            const uint16_t *lhs, const uint16_t *packed_rhs,
+                                            const float *bias, const float *residual, float *out_f32,
+                                            uint16_t *out_bf16, void *stream);
+int st_hip_pack_rhs_bf16_dev(size_t k, size_t n, const uint16_t *rhs, uint16_t *packed, void *stream);
 int st_hip_conv2d_bias_act_f32_dev(size_t batch, size_t c_in, size_t h, size_t w, size_t c_out,
                                    size_t kh, size_t kw, size_t stride_h, size_t stride_w,
                                    size_t pad_h, size_t pad_w, size_t dil_h, size_t dil_w,

@@ -88,6 +88,9 @@ SIGNATURES = {
     "st_hip_gemm_bf16_f32acc_dev": (c_int, [c_size_t, c_size_t, c_size_t, c_void_p, c_void_p, c_void_p, c_void_p]),
     "st_hip_gemm_bf16_bias_act_dev": (c_int, [c_size_t, c_size_t, c_size_t, c_int, c_void_p, c_void_p, c_void_p,
                                               c_void_p, c_void_p, c_void_p, c_void_p]),
+    "st_hip_gemm_bf16_prepacked_bias_act_dev": (c_int, [c_size_t, c_size_t, c_size_t, c_int, c_void_p, c_void_p,
+                                                        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "st_hip_pack_rhs_bf16_dev": (c_int, [c_size_t, c_size_t, c_void_p, c_void_p, c_void_p]),
     "st_hip_conv2d_bias_act_f32_dev": (c_int, [c_size_t] * 13 + [c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                                                  c_void_p]),
     "st_hip_attention_f32_dev": (c_int, [c_size_t, c_size_t, c_size_t, c_float, c_int, c_void_p, c_void_p, c_void_p,

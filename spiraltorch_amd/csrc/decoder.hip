@@ -112,12 +112,21 @@ int st_hip_decoder_create(const st_hip_decoder_config *config, const float *host
         hipError_t rc = hipMemcpy(blob, host_weights, weight_len * sizeof(float), hipMemcpyHostToDevice);
         if (rc != hipSuccess) status = hip_fail(rc, "hipMemcpy(H2D)");
     }
-    auto to_bf16 = [&](uint16_t **dst, const float *src, size_t count) {
+    // GEMM weights: (in, out) f32 -> bf16 -> packed (out, in), the layout in which neither GEMM operand needs
+    // transposing on its way to the matrix cores (PackedB, crates/st-tensor/src/pure.rs:1285-1323; the reference's
+    // Linear packs its weight once per parameter the same way, crates/st-nn/src/module.rs:674).
+    std::vector<void *> staging;
+    auto to_bf16 = [&](uint16_t **dst, const float *src, size_t in, size_t out) {
         if (status != ST_HIP_OK) return;
-        status = dec->alloc(dst, count);
+        status = dec->alloc(dst, in * out);
         if (status != ST_HIP_OK) return;
-        hipError_t rc = launch_f32_to_bf16(count, src, *dst, nullptr);
-        if (rc != hipSuccess) status = hip_fail(rc, "f32_to_bf16 launch");
+        void *rounded = nullptr;
+        hipError_t rc = hipMalloc(&rounded, (in * out ? in * out : 1) * sizeof(uint16_t));
+        if (rc != hipSuccess) { status = hip_fail(rc, "hipMalloc"); return; }
+        staging.push_back(rounded);
+        rc = launch_f32_to_bf16(in * out, src, static_cast<uint16_t *>(rounded), nullptr);
+        if (rc == hipSuccess) rc = launch_transpose_u16(in, out, static_cast<const uint16_t *>(rounded), *dst, nullptr);
+        if (rc != hipSuccess) status = hip_fail(rc, "weight packing launch");
     };
     float *p = blob;
     dec->embed = p; p += vocab * d;
@@ -126,20 +135,20 @@ int st_hip_decoder_create(const st_hip_decoder_config *config, const float *host
         LayerWeights &w = dec->layers[l];
         w.ln1_g = p; p += d;
         w.ln1_b = p; p += d;
-        to_bf16(&w.w_qkv, p, d * 3 * d); p += d * 3 * d;
+        to_bf16(&w.w_qkv, p, d, 3 * d); p += d * 3 * d;
         w.b_qkv = p; p += 3 * d;
-        to_bf16(&w.w_o, p, d * d); p += d * d;
+        to_bf16(&w.w_o, p, d, d); p += d * d;
         w.b_o = p; p += d;
         w.ln2_g = p; p += d;
         w.ln2_b = p; p += d;
-        to_bf16(&w.w_fc1, p, d * ff); p += d * ff;
+        to_bf16(&w.w_fc1, p, d, ff); p += d * ff;
         w.b_fc1 = p; p += ff;
-        to_bf16(&w.w_fc2, p, ff * d); p += ff * d;
+        to_bf16(&w.w_fc2, p, ff, d); p += ff * d;
         w.b_fc2 = p; p += d;
     }
     dec->lnf_g = p; p += d;
     dec->lnf_b = p; p += d;
-    to_bf16(&dec->w_head, p, d * vocab); p += d * vocab;
+    to_bf16(&dec->w_head, p, d, vocab); p += d * vocab;
     dec->b_head = p;
 
     if (status == ST_HIP_OK) status = dec->alloc(&dec->x, tokens * d);
@@ -158,9 +167,10 @@ int st_hip_decoder_create(const st_hip_decoder_config *config, const float *host
     if (status == ST_HIP_OK) status = dec->alloc(&dec->h16, tokens * d);
     if (status == ST_HIP_OK) status = dec->alloc(&dec->attn16, tokens * d);
     if (status == ST_HIP_OK) status = dec->alloc(&dec->u16, tokens * ff);
-    if (status == ST_HIP_OK) {
+    {
         hipError_t rc = hipDeviceSynchronize();
-        if (rc != hipSuccess) status = hip_fail(rc, "hipDeviceSynchronize");
+        if (rc != hipSuccess && status == ST_HIP_OK) status = hip_fail(rc, "hipDeviceSynchronize");
+        for (void *ptr : staging) (void)hipFree(ptr);
     }
     if (status != ST_HIP_OK) {
         delete dec;
@@ -195,14 +205,14 @@ int st_hip_decoder_forward_dev(void *decoder, const float *tokens, float *logits
         ep.bias = w.b_qkv;
         if (dec.fused_attention) {
             // q, k, v leave the projection as bf16 and are consumed in place, head by head.
-            ST_LAUNCH(launch_gemm_bf16(T, 3 * d, d, dec.h16, w.w_qkv, nullptr, dec.qkv16, ep, stream), "qkv gemm launch");
+            ST_LAUNCH(launch_gemm_bf16(T, 3 * d, d, dec.h16, w.w_qkv, nullptr, dec.qkv16, ep, stream, true), "qkv gemm launch");
             ST_LAUNCH(launch_attention_bf16(c.batch, heads, c.seq, hd, scale, true, dec.qkv16, dec.qkv16 + d,
                                             dec.qkv16 + 2 * d, 3 * d, dec.attn16, d, stream),
                       "attention launch");
         } else {
             // Head sizes the bf16 kernel does not cover: same rounding points (q, k, v rounded to bf16,
             // attention output rounded to bf16), carried out by the f32 attention kernel.
-            ST_LAUNCH(launch_gemm_bf16(T, 3 * d, d, dec.h16, w.w_qkv, dec.qkv, nullptr, ep, stream), "qkv gemm launch");
+            ST_LAUNCH(launch_gemm_bf16(T, 3 * d, d, dec.h16, w.w_qkv, dec.qkv, nullptr, ep, stream, true), "qkv gemm launch");
             ST_LAUNCH(launch_split_heads_f32(c.batch, c.seq, heads, hd, dec.qkv, dec.q, dec.k, dec.v, true, stream),
                       "split_heads launch");
             ST_LAUNCH(launch_attention_f32(c.batch * heads, c.seq, hd, scale, true, dec.q, dec.k, dec.v, nullptr,
@@ -214,23 +224,23 @@ int st_hip_decoder_forward_dev(void *decoder, const float *tokens, float *logits
         ep = GemmEpilogue();
         ep.bias = w.b_o;
         ep.residual = dec.x;
-        ST_LAUNCH(launch_gemm_bf16(T, d, d, dec.attn16, w.w_o, dec.x2, nullptr, ep, stream), "out-proj gemm launch");
+        ST_LAUNCH(launch_gemm_bf16(T, d, d, dec.attn16, w.w_o, dec.x2, nullptr, ep, stream, true), "out-proj gemm launch");
         ST_LAUNCH(launch_layer_norm_f32(T, d, dec.x2, nullptr, w.ln2_g, w.ln2_b, c.ln_eps, nullptr, dec.h16, stream),
                   "layer_norm launch");
         ep = GemmEpilogue();
         ep.bias = w.b_fc1;
         ep.activation = ST_HIP_ACT_GELU;
-        ST_LAUNCH(launch_gemm_bf16(T, ff, d, dec.h16, w.w_fc1, nullptr, dec.u16, ep, stream), "fc1 gemm launch");
+        ST_LAUNCH(launch_gemm_bf16(T, ff, d, dec.h16, w.w_fc1, nullptr, dec.u16, ep, stream, true), "fc1 gemm launch");
         ep = GemmEpilogue();
         ep.bias = w.b_fc2;
         ep.residual = dec.x2;
-        ST_LAUNCH(launch_gemm_bf16(T, d, ff, dec.u16, w.w_fc2, dec.x, nullptr, ep, stream), "fc2 gemm launch");
+        ST_LAUNCH(launch_gemm_bf16(T, d, ff, dec.u16, w.w_fc2, dec.x, nullptr, ep, stream, true), "fc2 gemm launch");
     }
     ST_LAUNCH(launch_layer_norm_f32(T, d, dec.x, nullptr, dec.lnf_g, dec.lnf_b, c.ln_eps, nullptr, dec.h16, stream),
               "layer_norm launch");
     GemmEpilogue head;
     head.bias = dec.b_head;
-    ST_LAUNCH(launch_gemm_bf16(T, c.vocab, d, dec.h16, dec.w_head, logits, nullptr, head, stream), "head gemm launch");
+    ST_LAUNCH(launch_gemm_bf16(T, c.vocab, d, dec.h16, dec.w_head, logits, nullptr, head, stream, true), "head gemm launch");
 #undef ST_LAUNCH
     return ST_HIP_OK;
 }

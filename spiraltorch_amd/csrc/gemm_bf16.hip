@@ -241,6 +241,106 @@ typedef __attribute__((address_space(3))) void *lds_void_ptr;
 // s_waitcnt vmcnt(n) only (expcnt and lgkmcnt left at their maxima), gfx9 encoding.
 #define ST_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (7 << 4) | (15 << 8) | ((((n) >> 4) & 3) << 14))
 
+// Epilogue of the 256-row kernels: a wavefront's 32·TM × WTN accumulators leave through its own 32-row f32 strip in LDS
+// so that bias/residual loads and the stores are 128-bit and row-contiguous.  `row_first` / `col_base`: the
+// wavefront's first row and column of C.
+template <int WTN, int TM = 2>
+__device__ __forceinline__ void gemm_bf16_epilogue(const GemmBf16Args &p, const f32x16 (&acc)[TM][WTN / 32], float *strip,
+                                                   int row_first, int col_base, int lane)
+{
+    constexpr int TN = WTN / 32;
+    constexpr int C_STRIDE = WTN + 4;
+    const int li = lane & 31, lh = lane >> 5;
+    const int M = p.M, N = p.N;
+    const bool scaled = p.scale != 1.0f;
+    constexpr int LPR = WTN / 4;        // lanes per strip row in the read-back phase (4 columns each)
+    constexpr int ROWS_PER_PASS = 64 / LPR;
+    const int col0 = col_base + (lane & (LPR - 1)) * 4;  // this lane's 4 columns in the read-back phase
+    float4 bias4 = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (p.bias) bias4 = *reinterpret_cast<const float4 *>(p.bias + col0);
+    // bf16-only output (16-byte aligned): 8 columns per lane in the read-back phase
+    constexpr int LPR8 = WTN / 8, ROWS8_PER_PASS = 64 / LPR8;
+    const bool bf16_only = p.C32 == nullptr && (reinterpret_cast<uintptr_t>(p.C16) & 15u) == 0;
+    const int col8 = col_base + (lane & (LPR8 - 1)) * 8;
+    float bias8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (bf16_only && p.bias) {
+        *reinterpret_cast<float4 *>(bias8) = *reinterpret_cast<const float4 *>(p.bias + col8);
+        *reinterpret_cast<float4 *>(bias8 + 4) = *reinterpret_cast<const float4 *>(p.bias + col8 + 4);
+    }
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) {
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn) {
+            const f32x16 tile = acc[tm][tn];
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                strip[((r >> 2) * 8 + lh * 4 + (r & 3)) * C_STRIDE + tn * 32 + li] = tile[r];
+        }
+        const int row_base = row_first + tm * 32;
+        if (bf16_only) {
+            // bf16 is the only output: 8 columns (16 bytes) per lane, so half as many store instructions
+#pragma unroll
+            for (int j = 0; j < 32 / ROWS8_PER_PASS; ++j) {
+                const int local_row = j * ROWS8_PER_PASS + lane / LPR8;
+                const int row = row_base + local_row;
+                const float *src = &strip[local_row * C_STRIDE + (lane & (LPR8 - 1)) * 8];
+                float v[8];
+                *reinterpret_cast<float4 *>(v) = *reinterpret_cast<const float4 *>(src);
+                *reinterpret_cast<float4 *>(v + 4) = *reinterpret_cast<const float4 *>(src + 4);
+                if (row < M) {
+                    const size_t idx = static_cast<size_t>(row) * N + col8;
+                    float res[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                    if (p.residual) {
+                        *reinterpret_cast<float4 *>(res) = *reinterpret_cast<const float4 *>(p.residual + idx);
+                        *reinterpret_cast<float4 *>(res + 4) = *reinterpret_cast<const float4 *>(p.residual + idx + 4);
+                    }
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        float value = v[e];
+                        if (scaled) value *= p.scale;
+                        value += bias8[e];
+                        value += res[e];
+                        v[e] = apply_activation(value, p.activation);
+                    }
+                    u32x4 packed;
+                    packed.x = pack_bf16x2_rne(v[0], v[1]);
+                    packed.y = pack_bf16x2_rne(v[2], v[3]);
+                    packed.z = pack_bf16x2_rne(v[4], v[5]);
+                    packed.w = pack_bf16x2_rne(v[6], v[7]);
+                    *reinterpret_cast<u32x4 *>(p.C16 + idx) = packed;
+                }
+            }
+            continue;
+        }
+#pragma unroll
+        for (int j = 0; j < 32 / ROWS_PER_PASS; ++j) {
+            const int local_row = j * ROWS_PER_PASS + lane / LPR;
+            const int row = row_base + local_row;
+            float4 v = *reinterpret_cast<const float4 *>(&strip[local_row * C_STRIDE + (lane & (LPR - 1)) * 4]);
+            if (row < M) {
+                const size_t idx = static_cast<size_t>(row) * N + col0;
+                if (scaled) { v.x *= p.scale; v.y *= p.scale; v.z *= p.scale; v.w *= p.scale; }
+                v.x += bias4.x; v.y += bias4.y; v.z += bias4.z; v.w += bias4.w;
+                if (p.residual) {
+                    const float4 rr = *reinterpret_cast<const float4 *>(p.residual + idx);
+                    v.x += rr.x; v.y += rr.y; v.z += rr.z; v.w += rr.w;
+                }
+                v.x = apply_activation(v.x, p.activation);
+                v.y = apply_activation(v.y, p.activation);
+                v.z = apply_activation(v.z, p.activation);
+                v.w = apply_activation(v.w, p.activation);
+                if (p.C32) *reinterpret_cast<float4 *>(p.C32 + idx) = v;
+                if (p.C16) {
+                    uint2 packed;
+                    packed.x = pack_bf16x2_rne(v.x, v.y);
+                    packed.y = pack_bf16x2_rne(v.z, v.w);
+                    *reinterpret_cast<uint2 *>(p.C16 + idx) = packed;
+                }
+            }
+        }
+    }
+}
+
 // Eight wavefronts, two per SIMD (each owns a 64 × BN/2 tile of C), so that one can issue MFMAs while the
 // other waits on LDS, memory or the barrier.  Wavefronts 0 .. BN/64-1 stage
 // B (fetch, transpose, store), wavefronts 4-7 issue the direct-to-LDS loads of A.  BN = 256 is the main
@@ -439,100 +539,212 @@ __device__ __forceinline__ void gemm_bf16_w8_body(const GemmBf16Args &p)
     }
     iteration(std::false_type{}, std::false_type{}, std::false_type{}, t);
 
-    // ---- epilogue through LDS ---------------------------------------------------------------------
     __syncthreads();
-    float *strip = reinterpret_cast<float *>(lds_bytes) + wave * (32 * C_STRIDE);
-    const bool scaled = p.scale != 1.0f;
-    constexpr int LPR = WTN / 4;        // lanes per strip row in the read-back phase (4 columns each)
-    constexpr int ROWS_PER_PASS = 64 / LPR;
-    const int col0 = n0 + wn * WTN + (lane & (LPR - 1)) * 4;  // this lane's 4 columns in the read-back phase
-    float4 bias4 = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (p.bias) bias4 = *reinterpret_cast<const float4 *>(p.bias + col0);
-    // bf16-only output (16-byte aligned): 8 columns per lane in the read-back phase
-    constexpr int LPR8 = WTN / 8, ROWS8_PER_PASS = 64 / LPR8;
-    const bool bf16_only = p.C32 == nullptr && (reinterpret_cast<uintptr_t>(p.C16) & 15u) == 0;
-    const int col8 = n0 + wn * WTN + (lane & (LPR8 - 1)) * 8;
-    float bias8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    if (bf16_only && p.bias) {
-        *reinterpret_cast<float4 *>(bias8) = *reinterpret_cast<const float4 *>(p.bias + col8);
-        *reinterpret_cast<float4 *>(bias8 + 4) = *reinterpret_cast<const float4 *>(p.bias + col8 + 4);
-    }
-#pragma unroll
-    for (int tm = 0; tm < 2; ++tm) {
-#pragma unroll
-        for (int tn = 0; tn < TN; ++tn) {
-            const f32x16 tile = acc[tm][tn];
-#pragma unroll
-            for (int r = 0; r < 16; ++r)
-                strip[((r >> 2) * 8 + lh * 4 + (r & 3)) * C_STRIDE + tn * 32 + li] = tile[r];
-        }
-        const int row_base = m0 + wm * 64 + tm * 32;
-        if (bf16_only) {
-            // bf16 is the only output: 8 columns (16 bytes) per lane, so half as many store instructions
-#pragma unroll
-            for (int j = 0; j < 32 / ROWS8_PER_PASS; ++j) {
-                const int local_row = j * ROWS8_PER_PASS + lane / LPR8;
-                const int row = row_base + local_row;
-                const float *src = &strip[local_row * C_STRIDE + (lane & (LPR8 - 1)) * 8];
-                float v[8];
-                *reinterpret_cast<float4 *>(v) = *reinterpret_cast<const float4 *>(src);
-                *reinterpret_cast<float4 *>(v + 4) = *reinterpret_cast<const float4 *>(src + 4);
-                if (row < M) {
-                    const size_t idx = static_cast<size_t>(row) * N + col8;
-                    float res[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-                    if (p.residual) {
-                        *reinterpret_cast<float4 *>(res) = *reinterpret_cast<const float4 *>(p.residual + idx);
-                        *reinterpret_cast<float4 *>(res + 4) = *reinterpret_cast<const float4 *>(p.residual + idx + 4);
-                    }
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        float value = v[e];
-                        if (scaled) value *= p.scale;
-                        value += bias8[e];
-                        value += res[e];
-                        v[e] = apply_activation(value, p.activation);
-                    }
-                    u32x4 packed;
-                    packed.x = pack_bf16x2_rne(v[0], v[1]);
-                    packed.y = pack_bf16x2_rne(v[2], v[3]);
-                    packed.z = pack_bf16x2_rne(v[4], v[5]);
-                    packed.w = pack_bf16x2_rne(v[6], v[7]);
-                    *reinterpret_cast<u32x4 *>(p.C16 + idx) = packed;
-                }
-            }
-            continue;
-        }
-#pragma unroll
-        for (int j = 0; j < 32 / ROWS_PER_PASS; ++j) {
-            const int local_row = j * ROWS_PER_PASS + lane / LPR;
-            const int row = row_base + local_row;
-            float4 v = *reinterpret_cast<const float4 *>(&strip[local_row * C_STRIDE + (lane & (LPR - 1)) * 4]);
-            if (row < M) {
-                const size_t idx = static_cast<size_t>(row) * N + col0;
-                if (scaled) { v.x *= p.scale; v.y *= p.scale; v.z *= p.scale; v.w *= p.scale; }
-                v.x += bias4.x; v.y += bias4.y; v.z += bias4.z; v.w += bias4.w;
-                if (p.residual) {
-                    const float4 rr = *reinterpret_cast<const float4 *>(p.residual + idx);
-                    v.x += rr.x; v.y += rr.y; v.z += rr.z; v.w += rr.w;
-                }
-                v.x = apply_activation(v.x, p.activation);
-                v.y = apply_activation(v.y, p.activation);
-                v.z = apply_activation(v.z, p.activation);
-                v.w = apply_activation(v.w, p.activation);
-                if (p.C32) *reinterpret_cast<float4 *>(p.C32 + idx) = v;
-                if (p.C16) {
-                    uint2 packed;
-                    packed.x = pack_bf16x2_rne(v.x, v.y);
-                    packed.y = pack_bf16x2_rne(v.z, v.w);
-                    *reinterpret_cast<uint2 *>(p.C16 + idx) = packed;
-                }
-            }
-        }
-    }
+    gemm_bf16_epilogue<WTN>(p, acc, reinterpret_cast<float *>(lds_bytes) + wave * (32 * C_STRIDE), m0 + wm * 64, n0 + wn * WTN,
+                            lane);
 }
 
 __global__ __launch_bounds__(512) void gemm_bf16_256w8_kernel(GemmBf16Args p) { gemm_bf16_w8_body<256>(p); }
 __global__ __launch_bounds__(512) void gemm_bf16_256x128w8_kernel(GemmBf16Args p) { gemm_bf16_w8_body<128>(p); }
+
+// -------------------------------------------------------------------------------------------------
+// Packed-B kernel: B is given prepacked as Bᵀ (n×k row-major, k contiguous — PackedB's column-major layout,
+// crates/st-tensor/src/pure.rs:1285-1323).  Same 256×BN×64 tiles, LDS layout, swizzle and epilogue as the kernel
+// above, but B needs no transposition: both operands go global memory -> LDS with buffer_load ... lds, every
+// wavefront issuing an eighth of the loads of each, and the main loop carries no vector-ALU work at all (the LDS
+// destination of each load is wavefront-uniform and computed on the scalar unit).
+//
+// Issue order is pinned: within a 16-wide k sub-step a wavefront alternates one MFMA with one memory instruction
+// (a fragment read of the next sub-step, or a direct load of a later k-tile).  An MFMA occupies the matrix pipe
+// for 32 cycles but issues in a few, so the memory instruction rides in its shadow; left to the compiler's own
+// order (all reads of a sub-step in a burst right before the MFMAs that use them) both wavefronts of a SIMD sit
+// in their read bursts at the same time and the pipe idles (4096³, all-zero operands so that the clock stays at
+// 2.4 GHz: 1.22 µs per k-tile against 0.92 with the order pinned; a loop of MFMAs alone needs 0.94).
+//
+// WAVES = 4 (one wavefront per SIMD, 128×128 of C each, a third less LDS read traffic) is instantiable but
+// measured slower (0.997 µs per k-tile on zeros, no gain on random data) and is not built.
+// -------------------------------------------------------------------------------------------------
+#define ST_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
+
+template <int BN, int WAVES>
+__device__ __forceinline__ void gemm_bf16_packed_body(const GemmBf16Args &p)
+{
+    static_assert(BN == 256 || BN == 128, "tile width");
+    static_assert(WAVES == 8 || WAVES == 4, "wavefronts per workgroup");
+    constexpr int BM = 256, BK = 64;
+    constexpr int WTM = 2 * BM / WAVES;      // wavefront tile: WAVES/2 × 2 wavefronts
+    constexpr int WTN = BN / 2;
+    constexpr int TM = WTM / 32, TN = WTN / 32;  // 32×32 MFMA tiles per wavefront
+    constexpr int NA = 32 / WAVES;           // direct loads per wavefront and k-tile: A ...
+    constexpr int NB = BN / 8 / WAVES;       // ... and B (one load fills 8 rows of a stage)
+    constexpr int STAGE = 32768;             // bytes: 256 rows × 128 B, for A and for Bᵀ alike
+    constexpr int B_REGION = 3 * STAGE;      // [A0][A1][A2][B0][B1]
+    constexpr int C_STRIDE = WTN + 4;        // floats, epilogue strip
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_bytes[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;  // WAVES/2 × 2 wavefronts, WTM × WTN each
+    const int li = lane & 31, lh = lane >> 5;
+    const int M = p.M, N = p.N, K = p.K;
+
+    int logical = blockIdx.x;
+    if (p.swizzle) logical = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+    constexpr int GROUP_M = 4;
+    const int width = GROUP_M * p.tiles_n;
+    const int group = logical / width;
+    const int first_m = group * GROUP_M;
+    const int group_size = min(p.tiles_m - first_m, GROUP_M);
+    const int tile_m = first_m + (logical % width) % group_size;
+    const int tile_n = (logical % width) / group_size;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t *>(p.A), 0, static_cast<int>(static_cast<unsigned>(M) * static_cast<unsigned>(K) * 2u), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t *>(p.B), 0, static_cast<int>(static_cast<unsigned>(K) * static_cast<unsigned>(N) * 2u), 0x00020000);
+
+    // Direct loads: instruction r of wavefront w fills rows (r*WAVES + w)*8 .. +7 of a stage (1 KB of LDS, lane l at
+    // chunk position l&7 of row l>>3), so lane l fetches logical chunk (l&7) ^ swz(row), swz(r) = ((r>>1) ^ (r>>4)) & 7.
+    constexpr int NMAX = NA > NB ? NA : NB;
+    unsigned a_off[NA], b_off[NB];
+    {
+        const int row_in = wave * 8 + (lane >> 3);
+        const int sw_base = ((wave * 4 + (lane >> 4)) ^ (wave >> 1)) & 7;
+#pragma unroll
+        for (int r = 0; r < NMAX; ++r) {
+            const int chunk = ((lane & 7) ^ sw_base ^ ((r * WAVES / 2) & 7)) & 7;
+            if (r < NA) a_off[r] = (static_cast<unsigned>(m0 + r * WAVES * 8 + row_in) * K + chunk * 8) * 2u;
+            if (r < NB) b_off[r] = (static_cast<unsigned>(n0 + r * WAVES * 8 + row_in) * K + chunk * 8) * 2u;
+        }
+    }
+    const int lds_row_block = wave * 1024;  // wavefront-uniform part of every load's LDS destination
+    auto load_a1 = [&](int stage, int r, unsigned k_off) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_ptr)(lds_bytes + stage * STAGE + r * (WAVES * 1024) + lds_row_block),
+                                                 16, a_off[r], k_off, 0, 0);
+    };
+    auto load_b1 = [&](int stage, int r, unsigned k_off) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            rsrc_b, (lds_void_ptr)(lds_bytes + B_REGION + stage * STAGE + r * (WAVES * 1024) + lds_row_block), 16, b_off[r], k_off, 0, 0);
+    };
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int a = 0; a < TM; ++a)
+#pragma unroll
+        for (int b = 0; b < TN; ++b)
+            acc[a][b] = f32x16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+
+    // Fragment addresses: row*128 + ((q ^ swz(row)) << 4) with q = 2*kk + lh; for row = base + t*32 + li the
+    // swizzle is sw0 ^ 2t, so the four values of (2kk) ^ (2t) select one of four precomputed addresses.
+    unsigned a_frag[4], b_frag[4];
+    {
+        const int sw0 = ((li >> 1) ^ (li >> 4)) & 7;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            a_frag[c] = (wm * WTM + li) * 128 + ((lh ^ sw0 ^ ((wm * WTM / 16) & 7) ^ (2 * c)) & 7) * 16;
+            b_frag[c] = B_REGION + (wn * WTN + li) * 128 + ((lh ^ sw0 ^ ((wn * WTN / 16) & 7) ^ (2 * c)) & 7) * 16;
+        }
+    }
+    bf16x8 fa[2][TM], fb[2][TN];
+    auto read_a = [&](int buf, int a_stage, int kk, int t) {
+        fa[buf][t] = *reinterpret_cast<const bf16x8 *>(lds_bytes + a_frag[kk ^ t] + a_stage * STAGE + t * 4096);
+    };
+    auto read_b = [&](int buf, int b_stage, int kk, int t) {
+        fb[buf][t] = *reinterpret_cast<const bf16x8 *>(lds_bytes + b_frag[kk ^ t] + b_stage * STAGE + t * 4096);
+    };
+    auto mfma = [&](int buf, int tm, int tn) {
+        acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[buf][tm], fb[buf][tn], acc[tm][tn], 0, 0, 0);
+    };
+    // One sub-step: the TM×TN MFMAs on fragment buffer `buf`, each followed by a slot for memory instructions: the
+    // first TM + TN slots issue the fragment reads of the sub-step after it (into the other buffer, in the order
+    // that sub-step uses them: A0, B0 .. B(TN-1), A1 ..), the last `loads` slots one direct load each (`load(i)`).
+    auto substep = [&](int buf, bool reads, int a_stage_r, int b_stage_r, int kk_r, auto &&load, int loads) {
+        constexpr int SLOTS = TM * TN;
+        static_assert(TM + TN <= SLOTS, "a sub-step has a slot for each fragment read");
+#pragma unroll
+        for (int slot = 0; slot < SLOTS; ++slot) {
+            mfma(buf, slot / TN, slot % TN);
+            ST_SCHED_FENCE();
+            if (reads) {
+                if (slot == 0) read_a(buf ^ 1, a_stage_r, kk_r, 0);
+                else if (slot <= TN) read_b(buf ^ 1, b_stage_r, kk_r, slot - 1);
+                else if (slot < TM + TN) read_a(buf ^ 1, a_stage_r, kk_r, slot - TN);
+            }
+            if (slot >= SLOTS - loads) load(slot - (SLOTS - loads));
+            ST_SCHED_FENCE();
+        }
+    };
+    auto no_load = [](int) {};
+
+    // One k-tile t.  On entry fragment buffer 0 holds sub-step 0 of tile t; B(t+1) and A(t+1) are in flight or
+    // landed.  Sub-step 0 requests A(t+2) (its stage was freed by the previous barrier); sub-step 3, after this
+    // tile's barrier, requests B(t+2) into the B stage this tile was read from.  The wait before the barrier lets
+    // the newest NA loads (A(t+2)) stay in flight; every load therefore has at least a whole k-tile to land.
+    int a_stage = 0;  // t % 3
+    auto iteration = [&](auto more_tag, auto load_tag, int t) {
+        constexpr bool MORE = decltype(more_tag)::value;  // a tile t+1 exists
+        constexpr bool LOAD = decltype(load_tag)::value;  // a tile t+2 exists
+        const int b_stage = t & 1;
+        const int a_next = a_stage == 2 ? 0 : a_stage + 1;
+        const int a_load = a_next == 2 ? 0 : a_next + 1;
+        const unsigned k_load = static_cast<unsigned>(t + 2) * (BK * 2u);
+        auto load_a_t2 = [&](int i) { load_a1(a_load, i, k_load); };
+        auto load_b_t2 = [&](int i) { load_b1(b_stage, i, k_load); };
+        if constexpr (LOAD) substep(0, true, a_stage, b_stage, 1, load_a_t2, NA);
+        else substep(0, true, a_stage, b_stage, 1, no_load, 0);
+        substep(1, true, a_stage, b_stage, 2, no_load, 0);
+        substep(0, true, a_stage, b_stage, 3, no_load, 0);
+        if constexpr (MORE) {
+            if constexpr (LOAD) ST_WAIT_VMCNT(NA); else ST_WAIT_VMCNT(0);
+        }
+        // Bare barrier: __syncthreads() would add a wait for every outstanding load.  This wavefront's LDS reads
+        // of tile t have returned (lgkmcnt) before anyone may overwrite the stages they came from.
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if constexpr (LOAD) substep(1, MORE, a_next, b_stage ^ 1, 0, load_b_t2, NB);
+        else substep(1, MORE, a_next, b_stage ^ 1, 0, no_load, 0);
+        a_stage = a_next;
+    };
+
+    const int steps = K / BK;
+#pragma unroll
+    for (int r = 0; r < NA; ++r) load_a1(0, r, 0u);
+#pragma unroll
+    for (int r = 0; r < NB; ++r) load_b1(0, r, 0u);
+    if (steps > 1) {
+#pragma unroll
+        for (int r = 0; r < NA; ++r) load_a1(1, r, BK * 2u);
+#pragma unroll
+        for (int r = 0; r < NB; ++r) load_b1(1, r, BK * 2u);
+        ST_WAIT_VMCNT(NA + NB);
+    } else {
+        ST_WAIT_VMCNT(0);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) read_a(0, 0, 0, tm);
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) read_b(0, 0, 0, tn);
+    int t = 0;
+    for (; t + 2 < steps; ++t) iteration(std::true_type{}, std::true_type{}, t);
+    if (t + 1 < steps) {
+        iteration(std::true_type{}, std::false_type{}, t);
+        ++t;
+    }
+    iteration(std::false_type{}, std::false_type{}, t);
+
+    __syncthreads();
+    gemm_bf16_epilogue<WTN, TM>(p, acc, reinterpret_cast<float *>(lds_bytes) + wave * (32 * C_STRIDE), m0 + wm * WTM,
+                                n0 + wn * WTN, lane);
+}
+
+__global__ __launch_bounds__(512) void gemm_bf16_256w8_packed_kernel(GemmBf16Args p) { gemm_bf16_packed_body<256, 8>(p); }
+__global__ __launch_bounds__(512) void gemm_bf16_256x128w8_packed_kernel(GemmBf16Args p) { gemm_bf16_packed_body<128, 8>(p); }
+
 
 // -------------------------------------------------------------------------------------------------
 // Skinny kernel (M <= 64, decode-like): HBM-bound on B, so the job is to keep many bytes of B in flight
@@ -705,11 +917,9 @@ __global__ __launch_bounds__(256) void gemm_bf16_skinny_reduce_kernel(SkinnyArgs
     if (p.C16) p.C16[idx] = f32_to_bf16_rne(value);
 }
 
-hipError_t launch_skinny(const GemmBf16Args &args, hipStream_t stream)
+// The split of a skinny problem over workgroups; fills the shape fields of `sk` and returns the bytes of partial sums.
+size_t plan_skinny(const GemmBf16Args &args, SkinnyArgs &sk)
 {
-    SkinnyArgs sk;
-    sk.A = args.A;
-    sk.B = args.B;
     sk.M = args.M;
     sk.N = args.N;
     sk.K = args.K;
@@ -721,11 +931,20 @@ hipError_t launch_skinny(const GemmBf16Args &args, hipStream_t stream)
     splits = std::max(1, std::min(splits, k_tiles / 4 > 0 ? k_tiles / 4 : 1));
     sk.tiles_per_split = (k_tiles + splits - 1) / splits;
     sk.k_splits = (k_tiles + sk.tiles_per_split - 1) / sk.tiles_per_split;
-    const size_t bytes = static_cast<size_t>(sk.k_splits) * args.M * args.N * sizeof(float);
+    return static_cast<size_t>(sk.k_splits) * args.M * args.N * sizeof(float);
+}
+
+// `workspace_offset`: bytes at the front of the stream's workspace that the caller is using (an unpacked B).
+hipError_t launch_skinny(const GemmBf16Args &args, hipStream_t stream, size_t workspace_offset)
+{
+    SkinnyArgs sk;
+    sk.A = args.A;
+    sk.B = args.B;
+    const size_t bytes = plan_skinny(args, sk);
     void *workspace = nullptr;
-    hipError_t rc = stream_workspace(stream, bytes, &workspace);  // hipMallocAsync/hipFreeAsync per call cost more than the kernel
-    sk.partial = static_cast<float *>(workspace);
+    hipError_t rc = stream_workspace(stream, workspace_offset + bytes, &workspace);  // hipMallocAsync/hipFreeAsync per call cost more than the kernel
     if (rc != hipSuccess) return rc;
+    sk.partial = reinterpret_cast<float *>(static_cast<unsigned char *>(workspace) + workspace_offset);
     sk.C32 = args.C32;
     sk.C16 = args.C16;
     sk.bias = args.bias;
@@ -752,8 +971,51 @@ hipError_t launch_skinny(const GemmBf16Args &args, hipStream_t stream)
     return hipGetLastError();
 }
 
+// out(cols×rows) = in(rows×cols)ᵀ for 16-bit elements, 64×64 tiles through LDS, 128-bit global accesses when the
+// shape allows (PackedB::from_row_major, crates/st-tensor/src/pure.rs:1299-1316, for bf16 storage).
+__global__ __launch_bounds__(256) void transpose_u16_kernel(int rows, int cols, int vec, const uint16_t *in, uint16_t *out)
+{
+    __shared__ uint16_t tile[64][66];
+    const int t = threadIdx.x;
+    const int c0 = blockIdx.x * 64, r0 = blockIdx.y * 64;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int r = (t >> 3) + 32 * i, c8 = (t & 7) * 8;
+        uint16_t e[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (r0 + r < rows) {
+            const uint16_t *src = in + static_cast<size_t>(r0 + r) * cols + c0 + c8;
+            if (vec && c0 + c8 + 8 <= cols) {
+                *reinterpret_cast<uint4 *>(e) = *reinterpret_cast<const uint4 *>(src);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    if (c0 + c8 + j < cols) e[j] = src[j];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) tile[r][c8 + j] = e[j];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int c = (t >> 3) + 32 * i, r8 = (t & 7) * 8;
+        if (c0 + c >= cols) continue;
+        uint16_t e[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) e[j] = tile[r8 + j][c];
+        uint16_t *dst = out + static_cast<size_t>(c0 + c) * rows + r0 + r8;
+        if (vec && r0 + r8 + 8 <= rows) {
+            *reinterpret_cast<uint4 *>(dst) = *reinterpret_cast<const uint4 *>(e);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                if (r0 + r8 + j < rows) dst[j] = e[j];
+        }
+    }
+}
+
 template <int BN>
-hipError_t launch_256(GemmBf16Args args, hipStream_t stream)
+hipError_t launch_256(GemmBf16Args args, bool packed, hipStream_t stream)
 {
     args.tiles_m = (args.M + 255) / 256;
     args.tiles_n = args.N / BN;
@@ -762,7 +1024,8 @@ hipError_t launch_256(GemmBf16Args args, hipStream_t stream)
     args.swizzle = (tiles % 8 == 0) ? 1 : 0;
     constexpr size_t lds_bytes = 5 * 32768;  // three A stages + two B stages
     static_assert(lds_bytes >= 8 * 32 * (128 + 4) * sizeof(float), "eight epilogue strips must fit in the stage buffers");
-    auto kernel = BN == 256 ? gemm_bf16_256w8_kernel : gemm_bf16_256x128w8_kernel;
+    auto kernel = BN == 256 ? (packed ? gemm_bf16_256w8_packed_kernel : gemm_bf16_256w8_kernel)
+                            : (packed ? gemm_bf16_256x128w8_packed_kernel : gemm_bf16_256x128w8_kernel);
     hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
     if (rc != hipSuccess) return rc;
@@ -802,9 +1065,19 @@ bool aligned16(const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u
 
 }  // namespace
 
+hipError_t launch_transpose_u16(size_t rows, size_t cols, const uint16_t *in, uint16_t *out, hipStream_t stream)
+{
+    if (rows == 0 || cols == 0) return hipSuccess;
+    const int vec = rows % 8 == 0 && cols % 8 == 0 && aligned16(in) && aligned16(out) ? 1 : 0;
+    const dim3 grid(static_cast<unsigned>((cols + 63) / 64), static_cast<unsigned>((rows + 63) / 64));
+    hipLaunchKernelGGL(transpose_u16_kernel, grid, dim3(256), 0, stream, static_cast<int>(rows), static_cast<int>(cols), vec,
+                       in, out);
+    return hipGetLastError();
+}
+
 hipError_t launch_gemm_bf16(size_t m, size_t n, size_t k, const uint16_t *lhs, const uint16_t *rhs,
                             float *out_f32, uint16_t *out_bf16, const GemmEpilogue &epilogue,
-                            hipStream_t stream)
+                            hipStream_t stream, bool rhs_packed)
 {
     if (m == 0 || n == 0) return hipSuccess;
     GemmBf16Args args;
@@ -827,18 +1100,34 @@ hipError_t launch_gemm_bf16(size_t m, size_t n, size_t k, const uint16_t *lhs, c
     const bool fits_buffer = m * k * 2 < (1ull << 31) && k * n * 2 < (1ull << 31);
     const bool epilogue_aligned = aligned16(out_f32) && aligned16(epilogue.bias) && aligned16(epilogue.residual) &&
                                   (reinterpret_cast<uintptr_t>(out_bf16) & 7u) == 0;
-    if (m <= 64 && vec && k >= 256 && k % 64 == 0 && n % 128 == 0 && fits_buffer)
-        return launch_skinny(args, stream);
+    const bool fits_256 = vec && k >= 64 && k % 64 == 0 && n % 128 == 0 && fits_buffer && epilogue_aligned;
+    const bool skinny = m <= 64 && vec && k >= 256 && k % 64 == 0 && n % 128 == 0 && fits_buffer;
+    size_t workspace_offset = 0;
+    if (rhs_packed && (!fits_256 || skinny) && k > 0) {
+        // Shapes the packed 256-row kernels do not take: unpack B into the front of the stream's workspace (sized for
+        // the skinny kernel's partial sums behind it as well, so that it does not move) and go on with B as k×n.
+        workspace_offset = (k * n * sizeof(uint16_t) + 255) & ~static_cast<size_t>(255);
+        SkinnyArgs probe;
+        const size_t behind = skinny ? plan_skinny(args, probe) : 0;
+        void *workspace = nullptr;
+        hipError_t rc = stream_workspace(stream, workspace_offset + behind, &workspace);
+        if (rc != hipSuccess) return rc;
+        rc = launch_transpose_u16(n, k, rhs, static_cast<uint16_t *>(workspace), stream);
+        if (rc != hipSuccess) return rc;
+        args.B = static_cast<const uint16_t *>(workspace);
+        rhs_packed = false;
+    }
+    if (skinny) return launch_skinny(args, stream, workspace_offset);
     // The 256-row kernels serve every shape they can address: measured against the 128×128 tile kernel they win
     // from a single tile up (256×256×4096: 58 vs 74 µs; 1024³: 21 vs 30 µs; 16384×256×512: 17 vs 24 µs).
-    if (vec && k >= 64 && k % 64 == 0 && n % 128 == 0 && fits_buffer && epilogue_aligned) {
+    if (fits_256) {
         // One workgroup per compute unit at a time: the launch runs in rounds of 256 tiles.  Halving the tile
         // width costs about 15 % in the main loop (more LDS traffic per flop), so do it only when it fills
         // rounds that the 256-wide tiling would leave partly empty (or when N is not a multiple of 256).
         auto fill = [](size_t tiles) { return static_cast<double>(tiles) / static_cast<double>((tiles + 255) / 256 * 256); };
         const size_t row_tiles = (m + 255) / 256;
-        if (n % 256 != 0 || fill(row_tiles * (n / 128)) > 1.15 * fill(row_tiles * (n / 256))) return launch_256<128>(args, stream);
-        return launch_256<256>(args, stream);
+        if (n % 256 != 0 || fill(row_tiles * (n / 128)) > 1.15 * fill(row_tiles * (n / 256))) return launch_256<128>(args, rhs_packed, stream);
+        return launch_256<256>(args, rhs_packed, stream);
     }
     return launch_tile<128, 128, 32>(args, vec, stream);
 }

@@ -714,6 +714,33 @@ int st_hip_gemm_bf16_bias_act_dev(size_t m, size_t n, size_t k, int activation, 
                          "gemm_bf16 launch");
 }
 
+int st_hip_gemm_bf16_prepacked_bias_act_dev(size_t m, size_t n, size_t k, int activation, const uint16_t *lhs,
+                                            const uint16_t *packed_rhs, const float *bias, const float *residual,
+                                            float *out_f32, uint16_t *out_bf16, void *stream)
+{
+    ST_HIP_CHECK(ensure_init());
+    ST_HIP_CHECK(validate_activation(activation, true));
+    ST_HIP_CHECK(validate_kernel_dims(m, n, k));
+    if (m == 0 || n == 0) return ST_HIP_OK;
+    if ((!out_f32 && !out_bf16) || (k != 0 && (!lhs || !packed_rhs)))
+        return fail(ST_HIP_ERR_INVALID, "gemm received a null pointer; provide contiguous row-major buffers");
+    GemmEpilogue epilogue;
+    epilogue.bias = bias;
+    epilogue.residual = residual;
+    epilogue.activation = activation;
+    return launch_status(launch_gemm_bf16(m, n, k, lhs, packed_rhs, out_f32, out_bf16, epilogue, as_stream(stream), true),
+                         "gemm_bf16 prepacked launch");
+}
+
+int st_hip_pack_rhs_bf16_dev(size_t k, size_t n, const uint16_t *rhs, uint16_t *packed, void *stream)
+{
+    ST_HIP_CHECK(ensure_init());
+    ST_HIP_CHECK(validate_kernel_dims(1, n, k));
+    if (k == 0 || n == 0) return ST_HIP_OK;
+    if (!rhs || !packed) return fail(ST_HIP_ERR_INVALID, "pack_rhs received a null pointer");
+    return launch_status(launch_transpose_u16(k, n, rhs, packed, as_stream(stream)), "pack_rhs launch");
+}
+
 int st_hip_conv2d_bias_act_f32_dev(size_t batch, size_t c_in, size_t h, size_t w, size_t c_out, size_t kh, size_t kw,
                                    size_t stride_h, size_t stride_w, size_t pad_h, size_t pad_w, size_t dil_h,
                                    size_t dil_w, int activation, const float *input, const float *weight,

@@ -25,10 +25,13 @@ hipError_t launch_gemm_f32_packed(size_t m, size_t n, size_t k, const float *lhs
 // out(cols×rows) = in(rows×cols) transposed.
 hipError_t launch_transpose_f32(size_t rows, size_t cols, const float *in, float *out, hipStream_t stream);
 
-// bf16 operands, f32 accumulation; writes out_f32 and/or out_bf16 (either may be null).
+// bf16 operands, f32 accumulation; writes out_f32 and/or out_bf16 (either may be null).  `rhs_packed`: rhs is the
+// n×k transpose of B (PackedB's layout, crates/st-tensor/src/pure.rs:1285-1323) instead of k×n.
 hipError_t launch_gemm_bf16(size_t m, size_t n, size_t k, const uint16_t *lhs, const uint16_t *rhs,
                             float *out_f32, uint16_t *out_bf16, const GemmEpilogue &epilogue,
-                            hipStream_t stream);
+                            hipStream_t stream, bool rhs_packed = false);
+// out(cols×rows) = in(rows×cols) transposed, 16-bit elements.
+hipError_t launch_transpose_u16(size_t rows, size_t cols, const uint16_t *in, uint16_t *out, hipStream_t stream);
 
 struct ConvShape {
     int batch, c_in, h, w, c_out, kh, kw, stride_h, stride_w, pad_h, pad_w, dil_h, dil_w, oh, ow;

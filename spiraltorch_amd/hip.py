@@ -356,6 +356,19 @@ def gemm_bf16_bias_act_dev(m, n, k, activation, lhs, rhs, bias, residual, out_f3
                                                      _stream_ptr(stream)))
 
 
+def gemm_bf16_prepacked_bias_act_dev(m, n, k, activation, lhs, packed_rhs, bias, residual, out_f32, out_bf16,
+                                     stream=None) -> None:
+    """gemm_bf16_bias_act_dev with B given as its (n, k) transpose (the PackedB layout)."""
+    _check(_lib.load().st_hip_gemm_bf16_prepacked_bias_act_dev(m, n, k, int(activation), _dev(lhs), _dev(packed_rhs),
+                                                               _dev(bias), _dev(residual), _dev(out_f32),
+                                                               _dev(out_bf16), _stream_ptr(stream)))
+
+
+def pack_rhs_bf16_dev(k, n, rhs, packed, stream=None) -> None:
+    """packed (n, k) = rhs (k, n) transposed, bf16 bit patterns, on the device."""
+    _check(_lib.load().st_hip_pack_rhs_bf16_dev(k, n, _dev(rhs), _dev(packed), _stream_ptr(stream)))
+
+
 def conv2d_bias_act_f32_dev(batch, c_in, h, w, c_out, kernel, stride, padding, dilation, activation, input, weight,
                             bias, out, stream=None) -> None:
     _check(_lib.load().st_hip_conv2d_bias_act_f32_dev(

@@ -158,6 +158,66 @@ def test_large_tile_kernels_with_epilogue(hip, oracle, m, n, k, ragged):
         assert (got16 == inputs.to_bf16(got32)).all(), "bf16 output must be the RNE rounding of the f32 output"
 
 
+PACKED_SHAPES = [
+    # m, n, k — the packed 256-row kernels (k % 64 == 0, n % 128 == 0), full and ragged in m, one to many k-tiles
+    (256, 256, 64), (512, 512, 512), (300, 384, 192), (8192 - 37, 2048, 128), (16384, 512, 192), (257, 256, 1024),
+    (100, 1152, 320), (4096, 128, 4096),
+    # shapes they do not take: unpacked on the device first (general kernel, skinny split-k kernel)
+    (33, 40, 72), (130, 136, 264), (5, 7, 9), (16, 384, 320), (64, 128, 1024), (1, 8, 8),
+]
+
+
+@pytest.mark.parametrize("m,n,k", PACKED_SHAPES)
+def test_prepacked_rhs(hip, oracle, m, n, k):
+    """B given as its (n, k) transpose (PackedB's layout): packed on the device, checked against the oracle on the
+    unpacked operands and, with the epilogue, bit for bit against the k×n entry point."""
+    from spiraltorch_amd import inputs
+    rng = np.random.default_rng(m * 31 + n * 7 + k)
+    a, b = bf16_pair(rng, m, n, k, std=0.5)
+    bias = rng.normal(size=n).astype(np.float32)
+    res = rng.normal(size=m * n).astype(np.float32)
+    d = {name: hip.DeviceBuffer.from_array(v) for name, v in (("a", a), ("b", b), ("bias", bias), ("res", res))}
+    d_packed = hip.DeviceBuffer(k * n * 2)
+    hip.pack_rhs_bf16_dev(k, n, d["b"], d_packed)
+    hip.device_synchronize()
+    assert (d_packed.to_array(np.uint16, k * n).reshape(n, k) == b.reshape(k, n).T).all()
+    plain = hip.DeviceBuffer(m * n * 4)
+    hip.gemm_bf16_prepacked_bias_act_dev(m, n, k, 0, d["a"], d_packed, None, None, plain, None)
+    hip.device_synchronize()
+    check(plain.to_array(np.float32, m * n), oracle.gemm_bf16_f32acc(m, n, k, a, b, threads=8), f"prepacked {m}x{n}x{k}")
+    want32, want16 = hip.DeviceBuffer(m * n * 4), hip.DeviceBuffer(m * n * 2)
+    got32, got16 = hip.DeviceBuffer(m * n * 4), hip.DeviceBuffer(m * n * 2)
+    hip.gemm_bf16_bias_act_dev(m, n, k, 2, d["a"], d["b"], d["bias"], d["res"], want32, want16)
+    hip.gemm_bf16_prepacked_bias_act_dev(m, n, k, 2, d["a"], d_packed, d["bias"], d["res"], got32, got16)
+    hip.device_synchronize()
+    assert (got32.to_array(np.float32, m * n) == want32.to_array(np.float32, m * n)).all()
+    assert (got16.to_array(np.uint16, m * n) == want16.to_array(np.uint16, m * n)).all()
+
+
+def test_config4_4096_cubed_prepacked(hip, oracle):
+    """BASELINE config 4 with B prepacked: 24 sampled rows against the oracle, the rest of the matrix bit for bit
+    against the k×n kernel (checked itself above), and exact power-of-two linearity."""
+    from spiraltorch_amd import inputs
+    n = 4096
+    a = inputs.to_bf16(inputs.normal(inputs.seed_for(4, 0), n * n, 0.0, 0.02))
+    b = inputs.to_bf16(inputs.normal(inputs.seed_for(4, 1), n * n, 0.0, 0.02))
+    d_a, d_b = hip.DeviceBuffer.from_array(a), hip.DeviceBuffer.from_array(b)
+    d_packed, d_out, d_ref = hip.DeviceBuffer(n * n * 2), hip.DeviceBuffer(n * n * 4), hip.DeviceBuffer(n * n * 4)
+    hip.pack_rhs_bf16_dev(n, n, d_b, d_packed)
+    hip.gemm_bf16_prepacked_bias_act_dev(n, n, n, 0, d_a, d_packed, None, None, d_out, None)
+    hip.gemm_bf16_f32acc_dev(n, n, n, d_a, d_b, d_ref)
+    hip.device_synchronize()
+    out = d_out.to_array(np.float32, (n, n))
+    rows = [0, 1, 31, 32, 255, 256, 257, 1023, 2048, 3000, 4094, 4095] + list(range(1500, 1512))
+    want = oracle.gemm_bf16_f32acc(len(rows), n, n, a.reshape(n, n)[rows].ravel(), b, threads=8)
+    check(out[rows].ravel(), want, "4096^3 prepacked, sampled rows")
+    assert (out == d_ref.to_array(np.float32, (n, n))).all()
+    d_a2 = hip.DeviceBuffer.from_array(inputs.to_bf16(2 * inputs.from_bf16(a)))
+    hip.gemm_bf16_prepacked_bias_act_dev(n, n, n, 0, d_a2, d_packed, None, None, d_ref, None)
+    hip.device_synchronize()
+    assert (d_ref.to_array(np.float32, (n, n)) == 2 * out).all()
+
+
 def test_validation(hip):
     out = np.full(4, 13.0, np.float32)
     with pytest.raises(hip.HipErr, match="lhs buffer length 4 does not match m\\*k=6"):
