@@ -216,21 +216,20 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmBf16Args p)
 
 
 // -------------------------------------------------------------------------------------------------
-// Large-problem kernel: 256×256×64 tiles, K a multiple of 64, N a multiple of 256 (M may be ragged:
-// rows past the end read as zero through the buffer descriptor's range check and are never stored).
+// Large-problem kernels: 256×256×64 (or 256×128×64) tiles, eight wavefronts (two per SIMD, 64 × BN/2 of C each), K a
+// multiple of 64, N a multiple of 128 (M may be ragged: rows past the end read as zero through the buffer
+// descriptor's range check and are never stored).  Two forms, by the layout of B: packed (n×k) and row-major (k×n).
 //
-// LDS is the scarce resource of this kernel (per k-tile a compute unit writes 64 KB and reads 128 KB of
-// it while the matrix pipes need 2048 cycles), so both operands are laid out for 128-bit, conflict-free
-// reads and neither is padded:
+// LDS is the scarce resource (per k-tile a compute unit writes 64 KB and reads 192 KB of it while the matrix pipes
+// need 2048 cycles; measured rates: 160 B/clk for 128-bit reads, 70 B/clk for 128-bit writes, 120 B/clk for a 2:1
+// mix), so both operands are laid out for 128-bit, conflict-free reads and neither is padded:
 //   * every operand row holds the tile's 64 k-values (128 B = 8 chunks of 16 B); chunk q of row r is
 //     stored at chunk position q ^ swz(r), swz(r) = ((r >> 1) ^ (r >> 4)) & 7, which spreads the 16 rows
-//     a 128-bit read touches per cycle, and the rows 8 apart that the B writes touch, over all banks;
-//   * A (k-contiguous in memory) goes from global memory straight into LDS with buffer_load ... lds;
-//     the swizzle is applied by choosing which 16 bytes each lane fetches.  A has three stages so these
-//     loads get two k-tiles of latency budget;
-//   * B (n-contiguous in memory) is fetched as 8×8 blocks (8 k-rows × 16 B per thread), transposed in
-//     registers with 32 v_perm_b32 and stored as rows of Bᵀ, so its fragments are 128-bit reads too
-//     (the LDS transpose read, ds_read_b64_tr_b16, moves a third of the bytes per cycle).
+//     a 128-bit read touches per cycle, and the rows the B writes touch, over all banks;
+//   * a k-contiguous operand (A; packed B) goes from global memory straight into LDS with buffer_load ... lds;
+//     the swizzle is applied by choosing which 16 bytes each lane fetches.  A has three stages, B two;
+//   * a row-major B is transposed in registers (v_perm_b32) and stored as rows of Bᵀ, so its fragments are
+//     128-bit reads too (the LDS transpose read, ds_read_b64_tr_b16, moves a third of the bytes per cycle).
 // Fragment reads run one 16-wide k sub-step ahead of the MFMAs and cross the tile boundary; there is one
 // barrier per k-tile.  The epilogue goes through LDS (each wavefront owns a 32-row f32 strip) so that
 // bias/residual loads and the stores are 128-bit and row-contiguous.
@@ -340,212 +339,6 @@ __device__ __forceinline__ void gemm_bf16_epilogue(const GemmBf16Args &p, const 
         }
     }
 }
-
-// Eight wavefronts, two per SIMD (each owns a 64 × BN/2 tile of C), so that one can issue MFMAs while the
-// other waits on LDS, memory or the barrier.  Wavefronts 0 .. BN/64-1 stage
-// B (fetch, transpose, store), wavefronts 4-7 issue the direct-to-LDS loads of A.  BN = 256 is the main
-// shape; BN = 128 halves the tile for problems whose 256-wide tiling would leave compute units idle.
-template <int BN>
-__device__ __forceinline__ void gemm_bf16_w8_body(const GemmBf16Args &p)
-{
-    static_assert(BN == 256 || BN == 128, "tile width");
-    constexpr int BM = 256, BK = 64;
-    constexpr int WTN = BN / 2;              // wavefront tile width
-    constexpr int TN = WTN / 32;             // 32-column MFMA tiles per wavefront
-    constexpr int B_THREADS = BN;            // threads that stage B: 8 k-groups × BN/8 column groups
-    constexpr int STAGE = 32768;             // bytes: 256 rows × 128 B, for A and for Bᵀ alike
-    constexpr int B_REGION = 3 * STAGE;      // [A0][A1][A2][B0][B1]
-    constexpr int C_STRIDE = WTN + 4;        // floats, epilogue strip
-    extern __shared__ __attribute__((aligned(16))) unsigned char lds_bytes[];
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;  // 4 × 2 wavefronts, 64 × WTN each
-    const int li = lane & 31, lh = lane >> 5;
-    const bool stages_b = wave < B_THREADS / 64;  // wavefront-uniform roles
-    const bool loads_a = wave >= 4;
-    const int lw = wave & 3;         // index within the role
-    const int M = p.M, N = p.N, K = p.K;
-
-    int logical = blockIdx.x;
-    if (p.swizzle) logical = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
-    constexpr int GROUP_M = 4;
-    const int width = GROUP_M * p.tiles_n;
-    const int group = logical / width;
-    const int first_m = group * GROUP_M;
-    const int group_size = min(p.tiles_m - first_m, GROUP_M);
-    const int tile_m = first_m + (logical % width) % group_size;
-    const int tile_n = (logical % width) / group_size;
-    const int m0 = tile_m * BM, n0 = tile_n * BN;
-
-    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint16_t *>(p.A), 0, static_cast<int>(static_cast<unsigned>(M) * static_cast<unsigned>(K) * 2u), 0x00020000);
-    const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint16_t *>(p.B), 0, static_cast<int>(static_cast<unsigned>(K) * static_cast<unsigned>(N) * 2u), 0x00020000);
-
-    // ---- A: direct global->LDS.  Instruction r of wavefront w fills rows r*32 + w*8 .. +7; lane l lands at
-    // chunk position l&7 of row (l>>3), so it must fetch logical chunk (l&7) ^ swz(row).
-    unsigned a_off[8];
-    {
-        const int row_in = lw * 8 + (lane >> 3);
-        const int sw_base = ((lw * 4 + (lane >> 4)) ^ (lw >> 1)) & 7;
-#pragma unroll
-        for (int r = 0; r < 8; ++r) {
-            const int chunk = ((lane & 7) ^ sw_base ^ ((2 * r) & 7)) & 7;
-            a_off[r] = (static_cast<unsigned>(m0 + r * 32 + row_in) * K + chunk * 8) * 2u;
-        }
-    }
-    // ---- B: thread (kg, nc) owns k-rows kg*8 .. +7 and columns nc*8 .. +7 of the tile.
-    const int kg = (tid & (B_THREADS - 1)) / (BN / 8), nc = tid & (BN / 8 - 1);
-    unsigned b_off = (static_cast<unsigned>(kg * 8) * N + n0 + nc * 8) * 2u;
-    const unsigned b_row_step = static_cast<unsigned>(N) * 2u;
-    const unsigned b_tile_step = static_cast<unsigned>(BK) * N * 2u;
-    // Store instruction s writes column s ^ (nc & 1): odd and even lanes then hit rows of different parity
-    // and, with the swizzle, a 16-lane group covers all 64 banks.
-    const unsigned sel_even = (nc & 1) ? 0x07060302u : 0x05040100u;  // column parity 0 for even lanes
-    const unsigned sel_odd = (nc & 1) ? 0x05040100u : 0x07060302u;
-    unsigned b_store[8];
-#pragma unroll
-    for (int sidx = 0; sidx < 8; ++sidx) {
-        const int col = nc * 8 + (sidx ^ (nc & 1));
-        const int pc = (kg ^ ((col >> 1) ^ (col >> 4))) & 7;
-        b_store[sidx] = B_REGION + col * 128 + pc * 16;
-    }
-
-    f32x16 acc[2][TN];
-#pragma unroll
-    for (int a = 0; a < 2; ++a)
-#pragma unroll
-        for (int b = 0; b < TN; ++b)
-            acc[a][b] = f32x16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-
-    u32x4 rb[8];
-    unsigned k_bytes = 0;  // byte offset of the next k-tile to request, within a row of A
-    auto load_a = [&](int stage) {
-#pragma unroll
-        for (int r = 0; r < 8; ++r)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_ptr)(lds_bytes + stage * STAGE + (r * 4 + lw) * 1024),
-                                                     16, a_off[r] + k_bytes, 0, 0, 0);
-    };
-    auto load_b = [&]() {
-#pragma unroll
-        for (int r = 0; r < 8; ++r) rb[r] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, b_off + r * b_row_step, 0, 0);
-        b_off += b_tile_step;
-    };
-    auto store_b = [&](int stage) {
-        // out[c].dword[j] = {rb[2j] element c, rb[2j+1] element c}; element c sits in dword c>>1, half c&1.
-#pragma unroll
-        for (int sidx = 0; sidx < 8; ++sidx) {
-            const int d = sidx >> 1;  // (sidx ^ 1) >> 1 == sidx >> 1: both lane parities read the same dword
-            const unsigned sel = (sidx & 1) ? sel_odd : sel_even;
-            u32x4 out;
-            out.x = __builtin_amdgcn_perm(rb[1][d], rb[0][d], sel);
-            out.y = __builtin_amdgcn_perm(rb[3][d], rb[2][d], sel);
-            out.z = __builtin_amdgcn_perm(rb[5][d], rb[4][d], sel);
-            out.w = __builtin_amdgcn_perm(rb[7][d], rb[6][d], sel);
-            *reinterpret_cast<u32x4 *>(lds_bytes + b_store[sidx] + stage * STAGE) = out;
-        }
-    };
-
-    // Fragment addresses: row*128 + ((q ^ swz(row)) << 4) with q = 2*kk + lh; for row = base + t*32 + li the
-    // swizzle is sw0 ^ 2t, so the four values of (2kk) ^ (2t) select one of four precomputed addresses.
-    unsigned a_frag[4], b_frag[4];
-    {
-        const int sw0 = ((li >> 1) ^ (li >> 4)) & 7;
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            a_frag[c] = (wm * 64 + li) * 128 + ((lh ^ sw0 ^ ((wm & 1) * 4) ^ (2 * c)) & 7) * 16;
-            b_frag[c] = B_REGION + (wn * WTN + li) * 128 + ((lh ^ sw0 ^ ((wn * WTN / 16) & 7) ^ (2 * c)) & 7) * 16;
-        }
-    }
-    bf16x8 fa[2][2], fb[2][TN];
-    auto read_frags = [&](int buf, int a_stage, int b_stage, int kk) {
-#pragma unroll
-        for (int t2 = 0; t2 < 2; ++t2)
-            fa[buf][t2] = *reinterpret_cast<const bf16x8 *>(lds_bytes + a_frag[kk ^ t2] + a_stage * STAGE + t2 * 4096);
-#pragma unroll
-        for (int t4 = 0; t4 < TN; ++t4)
-            fb[buf][t4] = *reinterpret_cast<const bf16x8 *>(lds_bytes + b_frag[kk ^ t4] + b_stage * STAGE + t4 * 4096);
-    };
-    auto mfma_step = [&](int buf) {
-#pragma unroll
-        for (int tm = 0; tm < 2; ++tm)
-#pragma unroll
-            for (int tn = 0; tn < TN; ++tn)
-                acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[buf][tm], fb[buf][tn], acc[tm][tn], 0, 0, 0);
-    };
-
-    // One k-tile t.  On entry: fragment buffer 0 holds sub-step 0 of tile t; rb holds B(t+1); the direct loads
-    // of A(t+1) are in flight.  STORE: B(t+1) is transposed into the other B stage; LOAD: B(t+2) and A(t+2)
-    // are requested; NEXT: sub-step 0 of tile t+1 is fetched after the barrier.
-    int a_stage = 0;  // t % 3
-    auto iteration = [&](auto store_tag, auto load_tag, auto next_tag, int t) {
-        constexpr bool STORE = decltype(store_tag)::value;
-        constexpr bool LOAD = decltype(load_tag)::value;
-        constexpr bool NEXT = decltype(next_tag)::value;
-        const int b_stage = t & 1;
-        const int a_next = a_stage == 2 ? 0 : a_stage + 1;
-        read_frags(1, a_stage, b_stage, 1);
-        mfma_step(0);
-        if (stages_b) {
-            if constexpr (STORE) store_b(b_stage ^ 1);
-            if constexpr (LOAD) load_b();
-        } else if (loads_a) {
-            if constexpr (LOAD) load_a(a_next == 2 ? 0 : a_next + 1);
-        }
-        if constexpr (LOAD) k_bytes += BK * 2u;
-        read_frags(0, a_stage, b_stage, 2);
-        mfma_step(1);
-        read_frags(1, a_stage, b_stage, 3);
-        mfma_step(0);
-        // A(t+1) must have landed before the barrier publishes it; this iteration's 8 requests may stay
-        // in flight.  (The B wavefronts' loads are register loads; the compiler waits where they are used.)
-        if constexpr (NEXT) {
-            if (loads_a) {
-                if constexpr (LOAD) ST_WAIT_VMCNT(8); else ST_WAIT_VMCNT(0);
-            }
-        }
-        __syncthreads();
-        if constexpr (NEXT) read_frags(0, a_next, b_stage ^ 1, 0);
-        mfma_step(1);
-        a_stage = a_next;
-    };
-
-    const int steps = K / BK;
-    if (stages_b) {
-        load_b();
-        store_b(0);
-        if (steps > 1) load_b();
-    } else if (loads_a) {
-        load_a(0);
-        if (steps > 1) {
-            k_bytes += BK * 2u;
-            load_a(1);
-            k_bytes -= BK * 2u;
-            ST_WAIT_VMCNT(8);
-        } else {
-            ST_WAIT_VMCNT(0);
-        }
-    }
-    k_bytes += (steps > 1 ? 2u : 1u) * BK * 2u;
-    __syncthreads();
-    read_frags(0, 0, 0, 0);
-    int t = 0;
-    for (; t + 2 < steps; ++t) iteration(std::true_type{}, std::true_type{}, std::true_type{}, t);
-    if (t + 1 < steps) {
-        iteration(std::true_type{}, std::false_type{}, std::true_type{}, t);
-        ++t;
-    }
-    iteration(std::false_type{}, std::false_type{}, std::false_type{}, t);
-
-    __syncthreads();
-    gemm_bf16_epilogue<WTN>(p, acc, reinterpret_cast<float *>(lds_bytes) + wave * (32 * C_STRIDE), m0 + wm * 64, n0 + wn * WTN,
-                            lane);
-}
-
-__global__ __launch_bounds__(512) void gemm_bf16_256w8_kernel(GemmBf16Args p) { gemm_bf16_w8_body<256>(p); }
-__global__ __launch_bounds__(512) void gemm_bf16_256x128w8_kernel(GemmBf16Args p) { gemm_bf16_w8_body<128>(p); }
 
 // -------------------------------------------------------------------------------------------------
 // Packed-B kernel: B is given prepacked as Bᵀ (n×k row-major, k contiguous — PackedB's column-major layout,
@@ -741,6 +534,230 @@ __device__ __forceinline__ void gemm_bf16_packed_body(const GemmBf16Args &p)
     gemm_bf16_epilogue<WTN, TM>(p, acc, reinterpret_cast<float *>(lds_bytes) + wave * (32 * C_STRIDE), m0 + wm * WTM,
                                 n0 + wn * WTN, lane);
 }
+
+// -------------------------------------------------------------------------------------------------
+// Row-major-B kernel in the same pinned style.  B (k×n, n contiguous) has to reach LDS as rows of Bᵀ, so it goes
+// through registers: every thread owns KR k-rows × 4 columns of the k-tile (KR × 64-bit loads, a wavefront
+// instruction reading 512 contiguous bytes of one k-row), transposes them with v_perm_b32 and writes 4 pieces of
+// Bᵀ rows (128-bit for KR = 8, 64-bit for KR = 4) into the stage the previous barrier freed.  The loads of B(t+2)
+// are issued in sub-step 2 of tile t and consumed in sub-step 1 of tile t+1; all of it — 4 direct loads of A,
+// KR loads, 2·KR permutes and 4 LDS writes per wavefront and k-tile — rides in the slots behind the MFMAs.
+// -------------------------------------------------------------------------------------------------
+template <int BN>
+__device__ __forceinline__ void gemm_bf16_rowmajor_body(const GemmBf16Args &p)
+{
+    static_assert(BN == 256 || BN == 128, "tile width");
+    constexpr int BM = 256, BK = 64;
+    constexpr int WTN = BN / 2;
+    constexpr int TN = WTN / 32;
+    constexpr int SLOTS = 2 * TN;            // MFMAs (and memory slots) per sub-step
+    constexpr int KR = BN / 32;              // k-rows of B per thread: 512 threads × KR × 4 columns = 64 × BN
+    constexpr int STAGE = 32768;
+    constexpr int B_REGION = 3 * STAGE;      // [A0][A1][A2][B0][B1]
+    constexpr int C_STRIDE = WTN + 4;
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_bytes[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int li = lane & 31, lh = lane >> 5;
+    const int M = p.M, N = p.N, K = p.K;
+
+    int logical = blockIdx.x;
+    if (p.swizzle) logical = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+    constexpr int GROUP_M = 4;
+    const int width = GROUP_M * p.tiles_n;
+    const int group = logical / width;
+    const int first_m = group * GROUP_M;
+    const int group_size = min(p.tiles_m - first_m, GROUP_M);
+    const int tile_m = first_m + (logical % width) % group_size;
+    const int tile_n = (logical % width) / group_size;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t *>(p.A), 0, static_cast<int>(static_cast<unsigned>(M) * static_cast<unsigned>(K) * 2u), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t *>(p.B), 0, static_cast<int>(static_cast<unsigned>(K) * static_cast<unsigned>(N) * 2u), 0x00020000);
+
+    // A: as in the packed kernel (instruction r of wavefront w fills rows r*64 + w*8 .. +7 of a stage).
+    unsigned a_off[4];
+    {
+        const int row_in = wave * 8 + (lane >> 3);
+        const int sw_base = ((wave * 4 + (lane >> 4)) ^ (wave >> 1)) & 7;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int chunk = ((lane & 7) ^ sw_base ^ ((4 * r) & 7)) & 7;
+            a_off[r] = (static_cast<unsigned>(m0 + r * 64 + row_in) * K + chunk * 8) * 2u;
+        }
+    }
+    const int lds_row_block = wave * 1024;
+    auto load_a1 = [&](int stage, int r, unsigned k_off) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_ptr)(lds_bytes + stage * STAGE + r * 8192 + lds_row_block), 16,
+                                                 a_off[r], k_off, 0, 0);
+    };
+
+    // B: thread (kg, nc) owns k-rows kg*KR .. +KR-1 and columns nc*4 .. +3 of the k-tile.
+    const int nc = tid & (BN / 4 - 1), kg = tid / (BN / 4);
+    unsigned b_voff[KR];
+#pragma unroll
+    for (int j = 0; j < KR; ++j) b_voff[j] = (static_cast<unsigned>(kg * KR + j) * N + n0 + nc * 4) * 2u;
+    const unsigned b_tile_step = static_cast<unsigned>(BK) * N * 2u;
+    uint2 rb[KR];
+    auto load_b1 = [&](int j, unsigned tile) {
+        const unsigned soff = __builtin_amdgcn_readfirstlane(tile * b_tile_step);
+        const auto v = __builtin_amdgcn_raw_buffer_load_b64(rsrc_b, b_voff[j], soff, 0);
+        rb[j] = make_uint2(v[0], v[1]);
+    };
+    // Store instruction s writes column s ^ (nc & 1): odd and even lanes then hit rows of different parity and, with
+    // the swizzle, the lanes of one LDS pass cover all banks.
+    const unsigned sel_even = (nc & 1) ? 0x07060302u : 0x05040100u;
+    const unsigned sel_odd = (nc & 1) ? 0x05040100u : 0x07060302u;
+    unsigned b_store[4];
+#pragma unroll
+    for (int sidx = 0; sidx < 4; ++sidx) {
+        const int col = nc * 4 + (sidx ^ (nc & 1));
+        const int swz = ((col >> 1) ^ (col >> 4)) & 7;
+        if (KR == 8) b_store[sidx] = B_REGION + col * 128 + ((kg ^ swz) & 7) * 16;
+        else b_store[sidx] = B_REGION + col * 128 + (((kg >> 1) ^ swz) & 7) * 16 + (kg & 1) * 8;
+    }
+    // Piece `sidx` of the transposed block: the KR k-values of one column as KR/2 dwords.
+    auto store_b1 = [&](int sidx, int stage) {
+        const unsigned sel = (sidx & 1) ? sel_odd : sel_even;
+        unsigned out[KR / 2];
+#pragma unroll
+        for (int i = 0; i < KR / 2; ++i) {
+            const unsigned hi = (sidx >> 1) ? rb[2 * i + 1].y : rb[2 * i + 1].x;
+            const unsigned lo = (sidx >> 1) ? rb[2 * i].y : rb[2 * i].x;
+            out[i] = __builtin_amdgcn_perm(hi, lo, sel);
+        }
+        if constexpr (KR == 8) {
+            u32x4 v;
+            v.x = out[0]; v.y = out[1]; v.z = out[2]; v.w = out[3];
+            *reinterpret_cast<u32x4 *>(lds_bytes + b_store[sidx] + stage * STAGE) = v;
+        } else {
+            *reinterpret_cast<uint2 *>(lds_bytes + b_store[sidx] + stage * STAGE) = make_uint2(out[0], out[1]);
+        }
+    };
+
+    f32x16 acc[2][TN];
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < TN; ++b)
+            acc[a][b] = f32x16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+
+    unsigned a_frag[4], b_frag[4];
+    {
+        const int sw0 = ((li >> 1) ^ (li >> 4)) & 7;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            a_frag[c] = (wm * 64 + li) * 128 + ((lh ^ sw0 ^ ((wm & 1) * 4) ^ (2 * c)) & 7) * 16;
+            b_frag[c] = B_REGION + (wn * WTN + li) * 128 + ((lh ^ sw0 ^ ((wn * WTN / 16) & 7) ^ (2 * c)) & 7) * 16;
+        }
+    }
+    bf16x8 fa[2][2], fb[2][TN];
+    auto read_a = [&](int buf, int a_stage, int kk, int t) {
+        fa[buf][t] = *reinterpret_cast<const bf16x8 *>(lds_bytes + a_frag[kk ^ t] + a_stage * STAGE + t * 4096);
+    };
+    auto read_b = [&](int buf, int b_stage, int kk, int t) {
+        fb[buf][t] = *reinterpret_cast<const bf16x8 *>(lds_bytes + b_frag[kk ^ t] + b_stage * STAGE + t * 4096);
+    };
+    // One sub-step: the 2×TN MFMAs on fragment buffer `buf`, each followed by a slot: a fragment read of the sub-step
+    // after it in the first 2 + TN slots (A0, B0 .. B(TN-1), A1), then whatever `extra(slot)` issues.
+    auto substep = [&](int buf, bool reads, int a_stage_r, int b_stage_r, int kk_r, auto &&extra) {
+#pragma unroll
+        for (int slot = 0; slot < SLOTS; ++slot) {
+            acc[slot / TN][slot % TN] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[buf][slot / TN], fb[buf][slot % TN],
+                                                                              acc[slot / TN][slot % TN], 0, 0, 0);
+            ST_SCHED_FENCE();
+            if (reads) {
+                if (slot == 0) read_a(buf ^ 1, a_stage_r, kk_r, 0);
+                else if (slot <= TN) read_b(buf ^ 1, b_stage_r, kk_r, slot - 1);
+                else if (slot < 2 + TN) read_a(buf ^ 1, a_stage_r, kk_r, slot - TN);
+            }
+            extra(slot);
+            ST_SCHED_FENCE();
+        }
+    };
+    auto nothing = [](int) {};
+
+    // One k-tile t.  On entry: fragment buffer 0 holds sub-step 0 of tile t, rb holds (or is receiving) B(t+1),
+    // A(t+1) is in flight or landed.
+    int a_stage = 0;  // t % 3
+    auto iteration = [&](auto more_tag, auto load_tag, int t) {
+        constexpr bool MORE = decltype(more_tag)::value;  // a tile t+1 exists
+        constexpr bool LOAD = decltype(load_tag)::value;  // a tile t+2 exists
+        const int b_stage = t & 1;
+        const int a_next = a_stage == 2 ? 0 : a_stage + 1;
+        const int a_load = a_next == 2 ? 0 : a_next + 1;
+        const unsigned k_load = static_cast<unsigned>(t + 2) * (BK * 2u);
+        // sub-step 0: A(t+2) into the stage the previous barrier freed
+        substep(0, true, a_stage, b_stage, 1, [&](int slot) {
+            if (LOAD && slot >= SLOTS - 4) load_a1(a_load, slot - (SLOTS - 4), k_load);
+        });
+        // sub-step 1: B(t+1) from the registers into the other B stage
+        substep(1, true, a_stage, b_stage, 2, [&](int slot) {
+            if (!MORE) return;
+            if (SLOTS == 8) {
+                if (slot & 1) store_b1(slot >> 1, b_stage ^ 1);
+            } else {
+                store_b1(slot, b_stage ^ 1);
+            }
+        });
+        // sub-step 2: B(t+2) into the registers
+        substep(0, true, a_stage, b_stage, 3, [&](int slot) {
+            if (LOAD && slot < KR) load_b1(slot, static_cast<unsigned>(t + 2));
+        });
+        if constexpr (MORE) {
+            if constexpr (LOAD) ST_WAIT_VMCNT(4 + KR); else ST_WAIT_VMCNT(0);
+        }
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wavefront's LDS reads and writes are done
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        substep(1, MORE, a_next, b_stage ^ 1, 0, nothing);
+        a_stage = a_next;
+    };
+
+    const int steps = K / BK;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) load_a1(0, r, 0u);
+#pragma unroll
+    for (int j = 0; j < KR; ++j) load_b1(j, 0u);
+    if (steps > 1) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) load_a1(1, r, BK * 2u);
+    }
+#pragma unroll
+    for (int sidx = 0; sidx < 4; ++sidx) store_b1(sidx, 0);
+    if (steps > 1) {
+#pragma unroll
+        for (int j = 0; j < KR; ++j) load_b1(j, 1u);
+        ST_WAIT_VMCNT(4 + KR);
+    } else {
+        ST_WAIT_VMCNT(0);
+    }
+    __syncthreads();
+    read_a(0, 0, 0, 0);
+    read_a(0, 0, 0, 1);
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) read_b(0, 0, 0, tn);
+    int t = 0;
+    for (; t + 2 < steps; ++t) iteration(std::true_type{}, std::true_type{}, t);
+    if (t + 1 < steps) {
+        iteration(std::true_type{}, std::false_type{}, t);
+        ++t;
+    }
+    iteration(std::false_type{}, std::false_type{}, t);
+
+    __syncthreads();
+    gemm_bf16_epilogue<WTN>(p, acc, reinterpret_cast<float *>(lds_bytes) + wave * (32 * C_STRIDE), m0 + wm * 64, n0 + wn * WTN,
+                            lane);
+}
+
+__global__ __launch_bounds__(512) void gemm_bf16_256rm_kernel(GemmBf16Args p) { gemm_bf16_rowmajor_body<256>(p); }
+__global__ __launch_bounds__(512) void gemm_bf16_256x128rm_kernel(GemmBf16Args p) { gemm_bf16_rowmajor_body<128>(p); }
 
 __global__ __launch_bounds__(512) void gemm_bf16_256w8_packed_kernel(GemmBf16Args p) { gemm_bf16_packed_body<256, 8>(p); }
 __global__ __launch_bounds__(512) void gemm_bf16_256x128w8_packed_kernel(GemmBf16Args p) { gemm_bf16_packed_body<128, 8>(p); }
@@ -1024,8 +1041,8 @@ hipError_t launch_256(GemmBf16Args args, bool packed, hipStream_t stream)
     args.swizzle = (tiles % 8 == 0) ? 1 : 0;
     constexpr size_t lds_bytes = 5 * 32768;  // three A stages + two B stages
     static_assert(lds_bytes >= 8 * 32 * (128 + 4) * sizeof(float), "eight epilogue strips must fit in the stage buffers");
-    auto kernel = BN == 256 ? (packed ? gemm_bf16_256w8_packed_kernel : gemm_bf16_256w8_kernel)
-                            : (packed ? gemm_bf16_256x128w8_packed_kernel : gemm_bf16_256x128w8_kernel);
+    auto kernel = BN == 256 ? (packed ? gemm_bf16_256w8_packed_kernel : gemm_bf16_256rm_kernel)
+                            : (packed ? gemm_bf16_256x128w8_packed_kernel : gemm_bf16_256x128rm_kernel);
     hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
     if (rc != hipSuccess) return rc;
