@@ -11,8 +11,11 @@ non-causal, the decoder stack) under `workloads`, each with its own roofline fig
 
 Timing: W untimed warm-up steps, then exactly K steps bracketed by a device synchronisation on both
 sides (wall clock) and by HIP events recorded on the stream the kernels are launched on (kernel time).
-The CPU baseline times the C restatement of the reference's CPU path (oracle/) on the host cores of the
-same box; it is a reported baseline, never part of `value`.
+The defaults (W = 50, K = 200) time the kernels in the sustained regime: under bf16 MFMA load on random
+data the chip settles at a lower clock than it starts with (and a cold chip ramps up), so a handful of
+steps measures neither.  Every workload carries a `cpu_baseline`: the C restatement of the reference's
+CPU path (oracle/) timed on the host cores of the same box, on a bounded sample that is stated with it;
+a reported baseline, never part of `value`.
 """
 from __future__ import annotations
 
@@ -151,14 +154,23 @@ def wl_gemm_f32(hip, inputs, timer, warmup, steps, m, n, k, name):
     return entry(name, "f32", 2 * m * n * k, 4 * (m * k + k * n + m * n), "mfma", wall, ev)
 
 
-def wl_gemm_bf16(hip, inputs, timer, warmup, steps, m, n, k, name, bound):
+def wl_gemm_bf16(hip, inputs, timer, warmup, steps, m, n, k, name, bound, packed=False):
+    """bf16 operands, f32 accumulation and output.  `packed`: B handed over as its (n, k) transpose (PackedB's
+    layout), packed once outside the timed region as a weight would be."""
     a = inputs.to_bf16(inputs.normal(inputs.seed_for(4, 0 if m == n else 2), m * k, 0.0, 0.02))
     b = inputs.to_bf16(inputs.normal(inputs.seed_for(4, 1), k * n, 0.0, 0.02))
     d_a, d_b = hip.DeviceBuffer.from_array(a), hip.DeviceBuffer.from_array(b)
     d_c = hip.DeviceBuffer(m * n * 4)
+    if packed:
+        d_packed = hip.DeviceBuffer(k * n * 2)
+        hip.pack_rhs_bf16_dev(k, n, d_b, d_packed)
+        hip.device_synchronize()
 
-    def step(stream):
-        hip.gemm_bf16_f32acc_dev(m, n, k, d_a, d_b, d_c, stream)
+        def step(stream):
+            hip.gemm_bf16_prepacked_bias_act_dev(m, n, k, 0, d_a, d_packed, None, None, d_c, None, stream)
+    else:
+        def step(stream):
+            hip.gemm_bf16_f32acc_dev(m, n, k, d_a, d_b, d_c, stream)
 
     wall, ev = timer.run(step, warmup, steps)
     return entry(name, "bf16", 2 * m * n * k, 2 * (m * k + k * n) + 4 * m * n, bound, wall, ev)
@@ -178,6 +190,25 @@ def wl_attention(hip, inputs, timer, warmup, steps, causal):
     flops = 4 * dim * contexts * (seq * (seq + 1) // 2 if causal else seq * seq)
     name = "attention_f32_b8_h16_s2048_d64_" + ("causal" if causal else "noncausal")
     return entry(name, "f32", flops, 4 * 4 * count, "mfma", wall, ev)
+
+
+def wl_attention_bias(hip, inputs, timer, warmup, steps, contexts, seq):
+    """Attention with a per-query bias matrix, the form the reference's only in-tree Rust caller uses (one context
+    per head with an attn_bias kernel matrix, crates/st-nn/src/z_rba/attention.rs:586-595): general kernel."""
+    dim = 64
+    count = contexts * seq * dim
+    q, k, v = (inputs.normal(inputs.seed_for(3, i), count) for i in range(3))
+    bias = inputs.normal(inputs.seed_for(3, 5), contexts * seq * seq, 0.0, 0.5)
+    d_q, d_k, d_v, d_b = (hip.DeviceBuffer.from_array(a) for a in (q, k, v, bias))
+    d_o = hip.DeviceBuffer(count * 4)
+
+    def step(stream):
+        hip.attention_f32_dev(contexts, seq, dim, 0.125, False, d_q, d_k, d_v, None, d_b, d_o, stream)
+
+    wall, ev = timer.run(step, warmup, steps)
+    flops = 4 * dim * contexts * seq * seq
+    return entry(f"attention_f32_attn_bias_c{contexts}_s{seq}_d64", "f32", flops, 4 * (4 * count + bias.size), "mfma",
+                 wall, ev)
 
 
 def wl_attention_bf16(hip, inputs, timer, warmup, steps):
@@ -260,32 +291,82 @@ def wl_calibration(hip, inputs, timer, warmup, steps):
     return entry("calibration_f32_to_bf16_64mi", "f32", 0, count * 6, "hbm", wall, ev)
 
 
-# ---- CPU baseline ---------------------------------------------------------------------------------------
+# ---- CPU baselines: the C restatement of the reference's CPU path, timed on the host cores of this box ------------
 
-def cpu_baseline_conv(conv_inputs, passes=7):
-    """Times the C restatement of Conv2d::forward_cpu (single-threaded, as the reference's contraction is)
-    on full passes of config 2: about ten seconds of CPU work; the median pass is reported."""
+def _cpu(flops, seconds, cores, sample):
+    return {"value": round(flops / seconds / 1e9, 3), "unit": "GFLOP/s", "cores": cores, "kind": "port", "sample": sample}
+
+
+def cpu_baseline_conv(conv_inputs, passes=5):
+    """Conv2d::forward_cpu, single-threaded as the reference's contraction is (conv.rs:297-323), on full passes
+    of config 2; the median pass is reported."""
     from oracle import oracle
     x, wt, b, geom, (batch, c_in, h, w, c_out) = conv_inputs
-    oracle.load()
     seconds = []
     for _ in range(passes):
         t0 = time.perf_counter()
         oracle.conv2d_bias_act_f32(batch, c_in, h, w, c_out, *geom, oracle.ACT_RELU, x, wt, b, threads=1)
         seconds.append(time.perf_counter() - t0)
     median = sorted(seconds)[len(seconds) // 2]
-    flops = 2 * batch * c_out * h * w * c_in * 9
-    return {"value": round(flops / median / 1e9, 3), "unit": "GFLOP/s", "cores": 1, "kind": "port",
-            "sample": f"{passes} full passes of config 2 ({batch} images each) through oracle/st_oracle.c, single "
-                      f"thread, {sum(seconds):.1f} s in all, median pass {median:.2f} s; host has "
-                      f"{os.cpu_count()} logical CPUs"}
+    return _cpu(2 * batch * c_out * h * w * c_in * 9, median, 1,
+                f"{passes} full passes of config 2 ({batch} images each), single thread, {sum(seconds):.1f} s in all, "
+                f"median pass {median:.2f} s; host has {os.cpu_count()} logical CPUs")
+
+
+def cpu_baselines(inputs):
+    """One bounded sample per remaining configuration; returns {workload name: cpu_baseline}."""
+    from oracle import oracle
+    cores = min(16, os.cpu_count() or 1)
+    out = {}
+
+    def timed(fn, repeat=1):
+        best = None
+        for _ in range(repeat):
+            t0 = time.perf_counter()
+            fn()
+            dt = time.perf_counter() - t0
+            best = dt if best is None else min(best, dt)
+        return best
+
+    # config 1: all cores over row tiles, as rayon does in cpu_dense.rs:226-236
+    a = inputs.uniform(inputs.seed_for(1, 0), 512 * 512, -1.0, 1.0)
+    b = inputs.uniform(inputs.seed_for(1, 1), 512 * 512, -1.0, 1.0)
+    sec = timed(lambda: oracle.gemm_f32(512, 512, 512, a, b, threads=cores), repeat=20)
+    out["gemm_f32_512x512x512"] = _cpu(2 * 512 ** 3, sec, cores, f"full 512^3, best of 20 passes, {cores} threads over row tiles")
+    # config 3: single thread as fused_attention_cpu is (pure.rs:11860-11916); 2 of 128 contexts, scaled
+    q, k, v = (inputs.normal(inputs.seed_for(3, i), 2 * 2048 * 64) for i in range(3))
+    for causal in (False, True):
+        sec = timed(lambda: oracle.attention_f32(2, 2048, 64, 0.125, q, k, v, causal=causal))
+        flops = 4 * 64 * 2 * (2048 * 2049 // 2 if causal else 2048 * 2048)
+        out["attention_f32_b8_h16_s2048_d64_" + ("causal" if causal else "noncausal")] = _cpu(
+            flops, sec, 1, f"2 of 128 contexts, single thread, {sec:.2f} s (the full config would take {sec * 64:.0f} s)")
+    # config 4: all cores over rows; 128 of 4096 rows of A for the square shape, the whole skinny shape
+    a16 = inputs.to_bf16(inputs.normal(inputs.seed_for(4, 0), 128 * 4096, 0.0, 0.02))
+    b16 = inputs.to_bf16(inputs.normal(inputs.seed_for(4, 1), 4096 * 4096, 0.0, 0.02))
+    sec = timed(lambda: oracle.gemm_bf16_f32acc(128, 4096, 4096, a16, b16, threads=cores), repeat=3)
+    square = _cpu(2 * 128 * 4096 * 4096, sec, cores, f"128 of 4096 rows of A, best of 3, {cores} threads ({sec:.2f} s; full: {sec * 32:.0f} s)")
+    out["gemm_bf16_f32acc_4096x4096x4096"] = square
+    out["gemm_bf16_f32acc_4096x4096x4096_prepacked_rhs"] = square
+    sec = timed(lambda: oracle.gemm_bf16_f32acc(16, 4096, 4096, a16[:16 * 4096], b16, threads=cores), repeat=5)
+    out["gemm_bf16_f32acc_16x4096x4096"] = _cpu(2 * 16 * 4096 * 4096, sec, cores, f"full shape, best of 5, {cores} threads")
+    # config 5: one layer (+ embedding, final norm, head) on one of 16 sequences, single thread, scaled
+    vocab, d, heads, ff, seq = 256, 512, 8, 2048, 1024
+    weights = inputs.normal(inputs.seed_for(5, 0), oracle.decoder_weight_count(vocab, d, heads, 1, ff), 0.0, 0.02)
+    tokens = inputs.tokens(inputs.seed_for(5, 1), seq, vocab)
+    sec = timed(lambda: oracle.decoder_forward(vocab, d, heads, 1, ff, 1, seq, 1e-5, weights, tokens))
+    hd = d // heads
+    layer = 3 * 2 * seq * d * d + 2 * seq * d * d + 4 * hd * heads * (seq * (seq + 1) // 2) + 2 * 2 * seq * d * ff
+    out["decoder_bf16_v256_d512_h8_l6_ff2048_b16_s1024"] = _cpu(
+        layer + 2 * seq * d * vocab, sec, 1,
+        f"1 of 6 layers on 1 of 16 sequences, single thread, {sec:.2f} s (the full config would take about {sec * 96:.0f} s)")
+    return out
 
 
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
-    parser.add_argument("--steps", type=int, default=50)
-    parser.add_argument("--warmup", type=int, default=10)
+    parser.add_argument("--steps", type=int, default=200)
+    parser.add_argument("--warmup", type=int, default=50)
     parser.add_argument("--no-cpu-baseline", action="store_true")
     parser.add_argument("--only", default=None, help="run only the headline plus workloads whose name contains this")
     args = parser.parse_args()
@@ -304,39 +385,52 @@ def main():
     headline, conv_inputs = wl_conv2d(hip, inputs, timer, args.warmup, args.steps)
     log(json.dumps(headline))
     others = []
-    side_steps = max(5, min(args.steps, 20))
-    side_warm = max(2, min(args.warmup, 5))
+    # Side workloads: the same sustained protocol, scaled down for the kernels that last a millisecond.
+    warm, steps = max(2, min(args.warmup, 50)), max(5, min(args.steps, 200))
+    long_warm, long_steps = max(2, warm // 5), max(5, steps // 5)
     plan = [
-        ("conv2d_grad_input", lambda: wl_conv2d_backward(hip, inputs, timer, side_warm, side_steps, "grad_input")),
-        ("conv2d_grad_weight", lambda: wl_conv2d_backward(hip, inputs, timer, side_warm, side_steps, "grad_weight")),
-        ("gemm_f32_512", lambda: wl_gemm_f32(hip, inputs, timer, side_warm, side_steps, 512, 512, 512,
-                                              "gemm_f32_512x512x512")),
-        ("gemm_f32_4096", lambda: wl_gemm_f32(hip, inputs, timer, 2, 5, 4096, 4096, 4096, "gemm_f32_4096x4096x4096")),
-        ("gemm_f32_conv_equivalent", lambda: wl_gemm_f32(hip, inputs, timer, side_warm, side_steps, 100352, 128, 576,
+        ("conv2d_grad_input", lambda: wl_conv2d_backward(hip, inputs, timer, warm, steps, "grad_input")),
+        ("conv2d_grad_weight", lambda: wl_conv2d_backward(hip, inputs, timer, warm, steps, "grad_weight")),
+        ("gemm_f32_512", lambda: wl_gemm_f32(hip, inputs, timer, warm, steps, 512, 512, 512, "gemm_f32_512x512x512")),
+        ("gemm_f32_4096", lambda: wl_gemm_f32(hip, inputs, timer, long_warm, long_steps, 4096, 4096, 4096,
+                                               "gemm_f32_4096x4096x4096")),
+        ("gemm_f32_conv_equivalent", lambda: wl_gemm_f32(hip, inputs, timer, warm, steps, 100352, 128, 576,
                                                          "gemm_f32_100352x128x576_conv_equivalent")),
-        ("gemm_bf16_4096", lambda: wl_gemm_bf16(hip, inputs, timer, side_warm, side_steps, 4096, 4096, 4096,
+        ("gemm_bf16_4096", lambda: wl_gemm_bf16(hip, inputs, timer, warm, steps, 4096, 4096, 4096,
                                                 "gemm_bf16_f32acc_4096x4096x4096", "mfma")),
-        ("gemm_bf16_skinny", lambda: wl_gemm_bf16(hip, inputs, timer, side_warm, side_steps, 16, 4096, 4096,
+        ("gemm_bf16_4096_prepacked", lambda: wl_gemm_bf16(hip, inputs, timer, warm, steps, 4096, 4096, 4096,
+                                                          "gemm_bf16_f32acc_4096x4096x4096_prepacked_rhs", "mfma", True)),
+        ("gemm_bf16_skinny", lambda: wl_gemm_bf16(hip, inputs, timer, warm, steps, 16, 4096, 4096,
                                                   "gemm_bf16_f32acc_16x4096x4096", "hbm")),
-        ("attention_noncausal", lambda: wl_attention(hip, inputs, timer, 2, 5, False)),
-        ("attention_causal", lambda: wl_attention(hip, inputs, timer, 2, 5, True)),
-        ("attention_bf16", lambda: wl_attention_bf16(hip, inputs, timer, side_warm, side_steps)),
-        ("decoder", lambda: wl_decoder(hip, inputs, timer, 2, 5)),
-        ("rowops", lambda: wl_rowops(hip, inputs, timer, 2, 10)),
-        ("calibration", lambda: wl_calibration(hip, inputs, timer, 2, 5)),
+        ("attention_noncausal", lambda: wl_attention(hip, inputs, timer, long_warm, long_steps, False)),
+        ("attention_causal", lambda: wl_attention(hip, inputs, timer, long_warm, long_steps, True)),
+        ("attention_bias", lambda: [wl_attention_bias(hip, inputs, timer, warm, steps, 1, 2048),
+                                    wl_attention_bias(hip, inputs, timer, long_warm, long_steps, 16, 1024)]),
+        ("attention_bf16", lambda: wl_attention_bf16(hip, inputs, timer, warm, steps)),
+        ("decoder", lambda: wl_decoder(hip, inputs, timer, long_warm, long_steps)),
+        ("rowops", lambda: wl_rowops(hip, inputs, timer, warm, steps)),
+        ("calibration", lambda: wl_calibration(hip, inputs, timer, long_warm, long_steps)),
     ]
     for name, fn in plan:
         if args.only and args.only not in name:
             continue
         result = fn()
         for item in (result if isinstance(result, list) else [result]):
-            log(json.dumps(item))
             others.append(item)
 
     cpu = None
     if not args.no_cpu_baseline:
         cpu = cpu_baseline_conv(conv_inputs)
         log(json.dumps(cpu))
+        per_workload = cpu_baselines(inputs)
+        for item in others:
+            if item["workload"] in per_workload:
+                item["cpu_baseline"] = per_workload[item["workload"]]
+            elif item["workload"].startswith("conv2d_grad"):
+                item["cpu_baseline"] = dict(cpu, sample="the forward pass of the same layer (the reference's backward runs "
+                                                         "the same contraction sizes): " + cpu["sample"])
+    for item in others:
+        log(json.dumps(item))
 
     line = {
         "metric": "GFLOP/s and % of MFMA roofline (GEMM, conv, attention) on 1 MI355X; value = fused conv2d+bias+ReLU",
