@@ -62,6 +62,16 @@ typedef struct {
 } st_hip_device_props;
 int st_hip_device_properties(int index, st_hip_device_props *out);
 
+/* st_backend_hip::probe() — lib.rs:188-207 (HipProbe: available, initialized, devices, error): tries init() and
+ * reports instead of failing.  `error` receives the init failure text (empty when initialised); returns 0 always. */
+typedef struct {
+    int available;    /* a HIP runtime and at least one device answered */
+    int initialized;  /* init() succeeded: device 0 is a gfx950 this library can run on */
+    int device_count;
+    char error[256];
+} st_hip_probe_result;
+int st_hip_probe(st_hip_probe_result *out);
+
 /* Copies the calling thread's last error text (NUL-terminated, truncated to len) and returns its full
  * length.  Precedent: spiraltorch_last_error_* in bindings/spiraltorch-sys/src/lib.rs:149-185. */
 size_t st_hip_last_error_message(char *buf, size_t len);
@@ -72,6 +82,11 @@ int st_hip_free(void *device_ptr);
 int st_hip_memcpy_h2d(void *device_dst, const void *host_src, size_t bytes, void *stream);
 int st_hip_memcpy_d2h(void *host_dst, const void *device_src, size_t bytes, void *stream);
 int st_hip_memset_zero(void *device_dst, size_t bytes, void *stream);
+/* Host<->device copies made through this library since start (or since the last call with reset != 0):
+ * {host-to-device copies, bytes, device-to-host copies, bytes}.  For callers and tests that check that tensors
+ * stay resident between operators (the per-call traffic of crates/st-backend-hip/src/real.rs:718-756 is what a
+ * resident tensor removes); the 16-byte status words of st_hip_count_nonfinite_f32_dev are not counted. */
+int st_hip_transfer_counters(uint64_t counters[4], int reset);
 int st_hip_stream_create(void **stream);
 int st_hip_stream_synchronize(void *stream);
 int st_hip_stream_destroy(void *stream);
@@ -92,6 +107,11 @@ int st_hip_event_destroy(void *event);
 int st_hip_gemm_f32(size_t m, size_t n, size_t k, float scale, int lhs_transposed,
                     const float *lhs, size_t lhs_len, const float *rhs, size_t rhs_len,
                     float *out, size_t out_len);
+
+/* gemm_f32_raw — lib.rs:760-799: the raw-pointer form (host pointers, lengths implied by m, n, k).  Null pointers
+ * are rejected ("gemm received a null pointer; provide contiguous row-major buffers", lib.rs:779-783), dimension
+ * products are checked for overflow ("gemm dimensions overflow while constructing lhs slice" ...). */
+int st_hip_gemm_f32_raw(size_t m, size_t n, size_t k, const float *lhs, const float *rhs, float *out);
 
 /* gemm_bias_activation_f32 — lib.rs:700-720; epilogue semantics of lib.rs:572-605:
  * out = act((lhs·rhs + bias[col]) + residual).  residual may be NULL (residual_len ignored).
@@ -269,6 +289,14 @@ int st_hip_attention_bf16_dev(size_t batch, size_t heads, size_t sequence, size_
  * add_row:       data[r][c] += bias[c] in place, pure.rs:6196-6290.
  * sum_axis0:     out[c] = (sum over rows of in[r][c]) * scale, pure.rs:6999-7210 (scale 1 is sum_axis0). */
 int st_hip_row_softmax_f32_dev(size_t rows, size_t cols, const float *in, float *out, void *stream);
+/* gelu: out = gelu(in), Gelu::forward, crates/st-nn/src/layers/gelu.rs:78-94 (tanh form of pure.rs:12026-12031). */
+int st_hip_gelu_f32_dev(size_t count, const float *in, float *out, void *stream);
+/* The finite check the reference makes on every operator result (validate_finite_tensor_util_slice,
+ * crates/st-tensor/src/pure.rs:5521-5533; call sites :2169, :4537, :4206-4210), for a tensor that lives on the
+ * device: counts the non-finite values of `data` and reports the first one's index and value.  Synchronous on
+ * `stream`; moves 16 bytes each way, whatever `count` is. */
+int st_hip_count_nonfinite_f32_dev(size_t count, const float *data, uint64_t *nonfinite,
+                                   uint64_t *first_index, float *first_value, void *stream);
 int st_hip_gelu_backward_f32_dev(size_t count, const float *z, const float *grad, float *out,
                                  void *stream);
 int st_hip_scale_f32_dev(size_t count, const float *in, float scale, float *out, void *stream);

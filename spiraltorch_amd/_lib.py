@@ -32,6 +32,10 @@ class DeviceProps(ctypes.Structure):
     ]
 
 
+class ProbeResult(ctypes.Structure):
+    _fields_ = [("available", c_int), ("initialized", c_int), ("device_count", c_int), ("error", ctypes.c_char * 256)]
+
+
 class DecoderConfig(ctypes.Structure):
     _fields_ = [
         ("vocab", c_size_t),
@@ -52,12 +56,14 @@ SIGNATURES = {
     "st_hip_device_count": (c_int, []),
     "st_hip_device_name": (c_int, [c_int, c_char_p, c_size_t]),
     "st_hip_device_properties": (c_int, [c_int, POINTER(DeviceProps)]),
+    "st_hip_probe": (c_int, [POINTER(ProbeResult)]),
     "st_hip_last_error_message": (c_size_t, [c_char_p, c_size_t]),
     "st_hip_malloc": (c_int, [POINTER(c_void_p), c_size_t]),
     "st_hip_free": (c_int, [c_void_p]),
     "st_hip_memcpy_h2d": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
     "st_hip_memcpy_d2h": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
     "st_hip_memset_zero": (c_int, [c_void_p, c_size_t, c_void_p]),
+    "st_hip_transfer_counters": (c_int, [POINTER(c_uint64), c_int]),
     "st_hip_stream_create": (c_int, [POINTER(c_void_p)]),
     "st_hip_stream_synchronize": (c_int, [c_void_p]),
     "st_hip_stream_destroy": (c_int, [c_void_p]),
@@ -69,6 +75,7 @@ SIGNATURES = {
     "st_hip_event_destroy": (c_int, [c_void_p]),
     "st_hip_gemm_f32": (c_int, [c_size_t, c_size_t, c_size_t, c_float, c_int, c_void_p, c_size_t, c_void_p,
                                 c_size_t, c_void_p, c_size_t]),
+    "st_hip_gemm_f32_raw": (c_int, [c_size_t, c_size_t, c_size_t, c_void_p, c_void_p, c_void_p]),
     "st_hip_gemm_bias_act_f32": (c_int, [c_size_t, c_size_t, c_size_t, c_int, c_void_p, c_size_t, c_void_p,
                                          c_size_t, c_void_p, c_size_t, c_void_p, c_size_t, c_void_p, c_size_t]),
     "st_hip_gemm_bf16_f32acc": (c_int, [c_size_t, c_size_t, c_size_t, c_void_p, c_size_t, c_void_p, c_size_t,
@@ -109,6 +116,9 @@ SIGNATURES = {
     "st_hip_conv2d_grad_weight_f32_dev": (c_int, [c_size_t] * 13 + [c_void_p, c_void_p, c_float, c_void_p, c_void_p]),
     "st_hip_conv2d_grad_bias_f32_dev": (c_int, [c_size_t] * 13 + [c_void_p, c_float, c_void_p, c_void_p]),
     "st_hip_row_softmax_f32_dev": (c_int, [c_size_t, c_size_t, c_void_p, c_void_p, c_void_p]),
+    "st_hip_gelu_f32_dev": (c_int, [c_size_t, c_void_p, c_void_p, c_void_p]),
+    "st_hip_count_nonfinite_f32_dev": (c_int, [c_size_t, c_void_p, POINTER(c_uint64), POINTER(c_uint64),
+                                               POINTER(c_float), c_void_p]),
     "st_hip_gelu_backward_f32_dev": (c_int, [c_size_t, c_void_p, c_void_p, c_void_p, c_void_p]),
     "st_hip_scale_f32_dev": (c_int, [c_size_t, c_void_p, c_float, c_void_p, c_void_p]),
     "st_hip_add_row_f32_dev": (c_int, [c_size_t, c_size_t, c_void_p, c_void_p, c_void_p]),

@@ -101,16 +101,20 @@ class Lease {
     int upload(int slot, const void *host, size_t bytes, void **device)
     {
         ST_HIP_CHECK(buffer(slot, bytes, device));
-        if (bytes)
+        if (bytes) {
+            count_transfer(true, bytes);
             ST_HIP_TRY(hipMemcpyAsync(*device, host, bytes, hipMemcpyHostToDevice, ws_->stream),
                        "hipMemcpyAsync(H2D)");
+        }
         return ST_HIP_OK;
     }
     int download(void *host, const void *device, size_t bytes)
     {
-        if (bytes)
+        if (bytes) {
+            count_transfer(false, bytes);
             ST_HIP_TRY(hipMemcpyAsync(host, device, bytes, hipMemcpyDeviceToHost, ws_->stream),
                        "hipMemcpyAsync(D2H)");
+        }
         ST_HIP_TRY(hipStreamSynchronize(ws_->stream), "hipStreamSynchronize");
         return ST_HIP_OK;
     }
@@ -318,6 +322,18 @@ int st_hip_gemm_f32(size_t m, size_t n, size_t k, float scale, int lhs_transpose
                                                epilogue, lease.stream()),
                                "gemm_f32 launch"));
     return lease.download(out, d_out, out_len * sizeof(float));
+}
+
+int st_hip_gemm_f32_raw(size_t m, size_t n, size_t k, const float *lhs, const float *rhs, float *out)
+{
+    // crates/st-backend-hip/src/lib.rs:779-798: null check first, then the slice lengths, then gemm_f32.
+    if (!lhs || !rhs || !out)
+        return fail(ST_HIP_ERR_INVALID, "gemm received a null pointer; provide contiguous row-major buffers");
+    size_t lhs_len, rhs_len, out_len;
+    if (!checked_mul(m, k, &lhs_len)) return fail(ST_HIP_ERR_INVALID, "gemm dimensions overflow while constructing lhs slice");
+    if (!checked_mul(k, n, &rhs_len)) return fail(ST_HIP_ERR_INVALID, "gemm dimensions overflow while constructing rhs slice");
+    if (!checked_mul(m, n, &out_len)) return fail(ST_HIP_ERR_INVALID, "gemm dimensions overflow while constructing output slice");
+    return st_hip_gemm_f32(m, n, k, 1.0f, 0, lhs, lhs_len, rhs, rhs_len, out, out_len);
 }
 
 int st_hip_gemm_bias_act_f32(size_t m, size_t n, size_t k, int activation, const float *lhs, size_t lhs_len,
@@ -890,6 +906,45 @@ int st_hip_row_softmax_f32_dev(size_t rows, size_t cols, const float *in, float 
     if (rows == 0 || cols == 0) return ST_HIP_OK;
     if (!in || !out) return fail(ST_HIP_ERR_INVALID, "row_softmax received a null pointer");
     return launch_status(launch_row_softmax_f32(rows, cols, in, out, as_stream(stream)), "row_softmax launch");
+}
+
+int st_hip_gelu_f32_dev(size_t count, const float *in, float *out, void *stream)
+{
+    ST_HIP_CHECK(ensure_init());
+    if (count == 0) return ST_HIP_OK;
+    if (!in || !out) return fail(ST_HIP_ERR_INVALID, "gelu received a null pointer");
+    return launch_status(launch_gelu_f32(count, in, out, as_stream(stream)), "gelu launch");
+}
+
+int st_hip_count_nonfinite_f32_dev(size_t count, const float *data, uint64_t *nonfinite, uint64_t *first_index,
+                                   float *first_value, void *stream)
+{
+    ST_HIP_CHECK(ensure_init());
+    if (!nonfinite) return fail(ST_HIP_ERR_INVALID, "count_nonfinite received a null out-pointer");
+    *nonfinite = 0;
+    if (first_index) *first_index = 0;
+    if (first_value) *first_value = 0.0f;
+    if (count == 0) return ST_HIP_OK;
+    if (!data) return fail(ST_HIP_ERR_INVALID, "count_nonfinite received a null pointer");
+    hipStream_t s = as_stream(stream);
+    void *workspace = nullptr;
+    ST_HIP_TRY(stream_workspace(s, 16, &workspace), "hipMalloc");
+    unsigned long long *status = static_cast<unsigned long long *>(workspace);
+    const unsigned long long init[2] = {0ull, ~0ull};
+    ST_HIP_TRY(hipMemcpyAsync(status, init, sizeof init, hipMemcpyHostToDevice, s), "hipMemcpyAsync(H2D)");
+    ST_HIP_CHECK(launch_status(launch_nonfinite_probe_f32(count, data, status, s), "count_nonfinite launch"));
+    unsigned long long result[2] = {0, 0};
+    ST_HIP_TRY(hipMemcpyAsync(result, status, sizeof result, hipMemcpyDeviceToHost, s), "hipMemcpyAsync(D2H)");
+    ST_HIP_TRY(hipStreamSynchronize(s), "hipStreamSynchronize");
+    *nonfinite = result[0];
+    if (result[0] != 0) {
+        if (first_index) *first_index = result[1];
+        if (first_value) {
+            ST_HIP_TRY(hipMemcpyAsync(first_value, data + result[1], sizeof(float), hipMemcpyDeviceToHost, s), "hipMemcpyAsync(D2H)");
+            ST_HIP_TRY(hipStreamSynchronize(s), "hipStreamSynchronize");
+        }
+    }
+    return ST_HIP_OK;
 }
 
 int st_hip_gelu_backward_f32_dev(size_t count, const float *z, const float *grad, float *out, void *stream)

@@ -92,6 +92,9 @@ hipError_t launch_merge_heads_f32(size_t batch, size_t seq, size_t heads, size_t
 
 // Element-wise and row-wise tensor utilities (all f32, row-major).
 hipError_t launch_row_softmax_f32(size_t rows, size_t cols, const float *in, float *out, hipStream_t stream);
+hipError_t launch_gelu_f32(size_t count, const float *in, float *out, hipStream_t stream);
+// status[0] += number of non-finite values of data, status[1] = min(status[1], index of one).
+hipError_t launch_nonfinite_probe_f32(size_t count, const float *data, unsigned long long *status, hipStream_t stream);
 hipError_t launch_gelu_backward_f32(size_t count, const float *z, const float *grad, float *out, hipStream_t stream);
 hipError_t launch_scale_f32(size_t count, const float *in, float scale, float *out, hipStream_t stream);
 hipError_t launch_add_row_f32(size_t rows, size_t cols, float *data, const float *bias, hipStream_t stream);
@@ -101,5 +104,7 @@ hipError_t launch_sum_axis0_f32(size_t rows, size_t cols, const float *in, float
 // partials).  Work on a stream is ordered, so two launches on the same stream never use it at the same time.
 hipError_t stream_workspace(hipStream_t stream, size_t bytes, void **out);
 void release_stream_workspace(hipStream_t stream);
+// Host<->device copies made by the library, for tests that check where tensors live.
+void count_transfer(bool to_device, size_t bytes);
 
 }  // namespace sthip

@@ -315,6 +315,31 @@ __global__ __launch_bounds__(256) void row_softmax_vec_kernel(int rows, int cols
     }
 }
 
+// Gelu::forward, crates/st-nn/src/layers/gelu.rs:78-94 (the tanh form of crates/st-tensor/src/pure.rs:12026-12031).
+__global__ __launch_bounds__(256) void gelu_forward_kernel(size_t count, const float *in, float *out)
+{
+    const size_t stride = static_cast<size_t>(gridDim.x) * 256;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < count; i += stride) out[i] = gelu_tanh(in[i]);
+}
+
+// status[0] = number of non-finite values, status[1] = smallest index of one (status[1] must start at ~0).
+// The first workgroup resets nothing: the caller clears the two words before the launch.
+__global__ __launch_bounds__(256) void nonfinite_probe_kernel(size_t count, const float *data, unsigned long long *status)
+{
+    const size_t stride = static_cast<size_t>(gridDim.x) * 256;
+    unsigned long long found = 0, first = ~0ull;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < count; i += stride) {
+        if (!isfinite(data[i])) {
+            ++found;
+            if (i < first) first = i;
+        }
+    }
+    if (found) {
+        atomicAdd(&status[0], found);
+        atomicMin(&status[1], first);
+    }
+}
+
 // gelu_prime(z)·g, crates/st-tensor/src/pure.rs:12033-12040 and :6549-6552.
 __global__ __launch_bounds__(256) void gelu_backward_kernel(size_t count, const float *z, const float *grad, float *out)
 {
@@ -588,6 +613,19 @@ hipError_t launch_row_softmax_f32(size_t rows, size_t cols, const float *in, flo
         hipLaunchKernelGGL(row_softmax_vec_kernel<8>, grid, block, 0, stream, r, c, in, out);
     else
         hipLaunchKernelGGL(row_softmax_kernel, grid, block, 0, stream, r, c, in, out);
+    return hipGetLastError();
+}
+
+hipError_t launch_gelu_f32(size_t count, const float *in, float *out, hipStream_t stream)
+{
+    if (count == 0) return hipSuccess;
+    hipLaunchKernelGGL(gelu_forward_kernel, dim3(grid_for(count)), dim3(256), 0, stream, count, in, out);
+    return hipGetLastError();
+}
+
+hipError_t launch_nonfinite_probe_f32(size_t count, const float *data, unsigned long long *status, hipStream_t stream)
+{
+    hipLaunchKernelGGL(nonfinite_probe_kernel, dim3(count ? grid_for(count) : 1), dim3(256), 0, stream, count, data, status);
     return hipGetLastError();
 }
 

@@ -1,6 +1,7 @@
 // Runtime half of the C ABI: init/probe, error text, device buffers, streams and events.
 // Mirrors crates/st-backend-hip/src/lib.rs:148-207 (init once, shared by all threads) and the RAII
 // wrappers of crates/st-backend-hip/src/real.rs:190-220,649-697, flattened to C handles.
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -81,6 +82,16 @@ int ensure_init()
     rt.devices.swap(devices);
     rt.ready = true;
     return ST_HIP_OK;
+}
+
+namespace {
+std::atomic<unsigned long long> g_transfers[4];  // h2d copies, h2d bytes, d2h copies, d2h bytes
+}  // namespace
+
+void count_transfer(bool to_device, size_t bytes)
+{
+    g_transfers[to_device ? 0 : 2].fetch_add(1, std::memory_order_relaxed);
+    g_transfers[to_device ? 1 : 3].fetch_add(bytes, std::memory_order_relaxed);
 }
 
 namespace {
@@ -178,6 +189,23 @@ int st_hip_device_properties(int index, st_hip_device_props *out)
     return ST_HIP_OK;
 }
 
+int st_hip_probe(st_hip_probe_result *out)
+{
+    if (!out) return fail(ST_HIP_ERR_INVALID, "st_hip_probe received a null out-pointer");
+    std::memset(out, 0, sizeof *out);
+    int count = 0;
+    const hipError_t rc = hipGetDeviceCount(&count);
+    if (rc != hipSuccess) (void)hipGetLastError();
+    out->available = rc == hipSuccess && count > 0;
+    out->device_count = rc == hipSuccess ? count : 0;
+    if (ensure_init() == ST_HIP_OK) {
+        out->initialized = 1;
+    } else {
+        snprintf(out->error, sizeof out->error, "%s", g_last_error.c_str());
+    }
+    return ST_HIP_OK;
+}
+
 size_t st_hip_last_error_message(char *buf, size_t len)
 {
     if (buf && len > 0) snprintf(buf, len, "%s", g_last_error.c_str());
@@ -203,6 +231,7 @@ int st_hip_free(void *device_ptr)
 int st_hip_memcpy_h2d(void *device_dst, const void *host_src, size_t bytes, void *stream)
 {
     if (bytes == 0) return ST_HIP_OK;
+    count_transfer(true, bytes);
     ST_HIP_TRY(hipMemcpyAsync(device_dst, host_src, bytes, hipMemcpyHostToDevice, as_stream(stream)),
                "hipMemcpyAsync(H2D)");
     ST_HIP_TRY(hipStreamSynchronize(as_stream(stream)), "hipStreamSynchronize");
@@ -212,6 +241,7 @@ int st_hip_memcpy_h2d(void *device_dst, const void *host_src, size_t bytes, void
 int st_hip_memcpy_d2h(void *host_dst, const void *device_src, size_t bytes, void *stream)
 {
     if (bytes == 0) return ST_HIP_OK;
+    count_transfer(false, bytes);
     ST_HIP_TRY(hipMemcpyAsync(host_dst, device_src, bytes, hipMemcpyDeviceToHost, as_stream(stream)),
                "hipMemcpyAsync(D2H)");
     ST_HIP_TRY(hipStreamSynchronize(as_stream(stream)), "hipStreamSynchronize");
@@ -222,6 +252,14 @@ int st_hip_memset_zero(void *device_dst, size_t bytes, void *stream)
 {
     if (bytes == 0) return ST_HIP_OK;
     ST_HIP_TRY(hipMemsetAsync(device_dst, 0, bytes, as_stream(stream)), "hipMemsetAsync");
+    return ST_HIP_OK;
+}
+
+int st_hip_transfer_counters(uint64_t counters[4], int reset)
+{
+    if (!counters) return fail(ST_HIP_ERR_INVALID, "st_hip_transfer_counters received a null out-pointer");
+    for (int i = 0; i < 4; ++i)
+        counters[i] = reset ? g_transfers[i].exchange(0, std::memory_order_relaxed) : g_transfers[i].load(std::memory_order_relaxed);
     return ST_HIP_OK;
 }
 

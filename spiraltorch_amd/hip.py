@@ -84,6 +84,20 @@ def hip_available() -> bool:
         return False
 
 
+def probe() -> dict:
+    """`probe()` of crates/st-backend-hip/src/lib.rs:188-207: tries init() and reports (HipProbe's fields)."""
+    result = _lib.ProbeResult()
+    _check(_lib.load().st_hip_probe(ctypes.byref(result)))
+    error = result.error.decode("utf-8", "replace")
+    return {"available": bool(result.available), "initialized": bool(result.initialized),
+            "devices": device_info() if result.initialized else [], "error": error or None}
+
+
+def runtime():
+    """`runtime()` of lib.rs:164-166: the initialised runtime (here: its device list), or None before init()."""
+    return device_info() if hip_available() else None
+
+
 def device_count() -> int:
     return int(_lib.load().st_hip_device_count())
 
@@ -118,6 +132,12 @@ def gemm_scaled_f32(m: int, n: int, k: int, scale: float, lhs, rhs, out) -> None
 def gemm_f32(m: int, n: int, k: int, lhs, rhs, out) -> None:
     """lib.rs:607-616."""
     gemm_scaled_f32(m, n, k, 1.0, lhs, rhs, out)
+
+
+def gemm_f32_raw(m: int, n: int, k: int, lhs_address, rhs_address, out_address) -> None:
+    """`gemm_f32_raw` of lib.rs:760-799: raw host addresses (ints or None), lengths implied by m, n, k."""
+    as_ptr = lambda a: None if not a else ctypes.c_void_p(int(a))
+    _check(_lib.load().st_hip_gemm_f32_raw(m, n, k, as_ptr(lhs_address), as_ptr(rhs_address), as_ptr(out_address)))
 
 
 def gemm_lhs_transpose_scaled_f32(m: int, n: int, k: int, scale: float, lhs, rhs, out) -> None:
@@ -426,6 +446,26 @@ def attention_bf16_dev(batch, heads, sequence, head_dim, scale, causal, q, k, v,
 
 def row_softmax_f32_dev(rows, cols, src, dst, stream=None) -> None:
     _check(_lib.load().st_hip_row_softmax_f32_dev(rows, cols, _dev(src), _dev(dst), _stream_ptr(stream)))
+
+
+def gelu_f32_dev(count, src, dst, stream=None) -> None:
+    _check(_lib.load().st_hip_gelu_f32_dev(count, _dev(src), _dev(dst), _stream_ptr(stream)))
+
+
+def count_nonfinite_f32_dev(count, data, stream=None):
+    """(number of non-finite values, index of the first, its value) of a device buffer; synchronous."""
+    found, first = ctypes.c_uint64(), ctypes.c_uint64()
+    value = ctypes.c_float()
+    _check(_lib.load().st_hip_count_nonfinite_f32_dev(count, _dev(data), ctypes.byref(found), ctypes.byref(first),
+                                                      ctypes.byref(value), _stream_ptr(stream)))
+    return int(found.value), int(first.value), float(value.value)
+
+
+def transfer_counters(reset: bool = False) -> dict:
+    """Host<->device copies made through the library: copies and bytes in each direction."""
+    raw = (ctypes.c_uint64 * 4)()
+    _check(_lib.load().st_hip_transfer_counters(raw, int(reset)))
+    return {"h2d_copies": int(raw[0]), "h2d_bytes": int(raw[1]), "d2h_copies": int(raw[2]), "d2h_bytes": int(raw[3])}
 
 
 def gelu_backward_f32_dev(count, z, grad, out, stream=None) -> None:

@@ -46,18 +46,13 @@ def _backend_failure(err: hip.HipErr) -> TensorError:
     return TensorError("BackendFailure", err.message, backend="hip")
 
 
-def _validate_finite(label: str, data: np.ndarray) -> None:
-    if not np.isfinite(data).all():
-        bad = data[~np.isfinite(data)].ravel()[0]
-        raise TensorError("NonFiniteValue", f"non-finite value encountered in {label}: {bad}", label=label)
-
-
 class PackedB:
     """Right-hand operand packed once for repeated matmuls (pure.rs:1285-1400): column-major, i.e. the (cols, inner)
-    row-major transpose of the (inner, cols) matrix."""
+    row-major transpose of the (inner, cols) matrix.  Its device copy is made on first use and kept."""
 
     def __init__(self, inner: int, cols: int, buf: np.ndarray):
         self._inner, self._cols, self._buf = int(inner), int(cols), buf
+        self._dev: Optional[hip.DeviceBuffer] = None
 
     @classmethod
     def from_tensor(cls, tensor: "Tensor") -> "PackedB":
@@ -73,20 +68,34 @@ class PackedB:
     def as_slice(self) -> np.ndarray:
         return self._buf
 
+    def _device(self) -> hip.DeviceBuffer:
+        if self._dev is None:
+            self._dev = hip.DeviceBuffer.from_array(self._buf)
+        return self._dev
+
 
 class Tensor:
-    """2-D row-major float32 matrix held on the host (pure.rs:1406-1411)."""
+    """2-D row-major float32 matrix (pure.rs:1406-1411) with a device-resident twin.
+
+    A tensor built from host values is uploaded the first time an operator needs it and the device copy is kept;
+    an operator's result is born on the device and is downloaded only when its values are read (`data()`,
+    `numpy()`).  A chain of operators therefore costs one upload per input and one download at the end, instead of
+    the reference HIP backend's three allocations and three copies per call
+    (crates/st-backend-hip/src/real.rs:718-756).  `data()` returns a read-only view; `data_mut()` returns a writable
+    one and drops the device copy."""
 
     def __init__(self, rows: int, cols: int, data=None):
         if data is None:
             buf = np.zeros(rows * cols, dtype=np.float32)
         else:
-            buf = np.ascontiguousarray(np.asarray(data, dtype=np.float32)).reshape(-1)
+            buf = np.array(data, dtype=np.float32).reshape(-1)
             if buf.size != rows * cols:
                 raise TensorError("DataLength", f"expected {rows * cols} values, got {buf.size}",
                                   expected=rows * cols, got=buf.size)
         self.rows, self.cols = int(rows), int(cols)
-        self._data = buf
+        self._host: Optional[np.ndarray] = buf
+        self._dev: Optional[hip.DeviceBuffer] = None
+        self._finite: Optional[bool] = None  # None: not examined yet
 
     @classmethod
     def zeros(cls, rows: int, cols: int) -> "Tensor":
@@ -99,14 +108,95 @@ class Tensor:
             raise TensorError("InvalidDimensions", "expected a 2-D array", rows=a.ndim, cols=2)
         return cls(a.shape[0], a.shape[1], a)
 
+    @classmethod
+    def _on_device_result(cls, rows: int, cols: int) -> "Tensor":
+        """A result tensor that exists only on the device so far."""
+        out = cls.__new__(cls)
+        out.rows, out.cols = int(rows), int(cols)
+        out._host = None
+        out._dev = hip.DeviceBuffer(max(out.rows * out.cols, 1) * 4)
+        out._finite = None
+        return out
+
     def shape(self) -> Tuple[int, int]:
         return (self.rows, self.cols)
 
+    def __len__(self) -> int:
+        return self.rows * self.cols
+
+    def is_device_resident(self) -> bool:
+        return self._dev is not None
+
+    def _host_values(self) -> np.ndarray:
+        if self._host is None:
+            try:
+                self._host = self._dev.to_array(np.float32, self.rows * self.cols)
+            except hip.HipErr as err:
+                raise _backend_failure(err) from err
+        return self._host
+
     def data(self) -> np.ndarray:
-        return self._data
+        """The values, row-major, as a read-only array (downloaded once if they live on the device)."""
+        view = self._host_values().view()
+        view.flags.writeable = False
+        return view
+
+    def data_mut(self) -> np.ndarray:
+        """Writable values (Tensor::data_mut): the device copy is dropped and re-made on the next use."""
+        values = self._host_values()
+        self._dev = None
+        self._finite = None
+        return values
 
     def numpy(self) -> np.ndarray:
-        return self._data.reshape(self.rows, self.cols)
+        return self.data().reshape(self.rows, self.cols)
+
+    def _device(self) -> hip.DeviceBuffer:
+        if self._dev is None:
+            try:
+                self._dev = hip.DeviceBuffer.from_array(self._host)
+            except hip.HipErr as err:
+                raise _backend_failure(err) from err
+        return self._dev
+
+    def _require_finite(self, label: str) -> None:
+        """validate_finite_tensor_util_slice (pure.rs:5521-5533) on an operand, wherever it lives; the answer is
+        remembered, so an operator's validated result is not examined again when it feeds the next operator."""
+        if self._finite is None:
+            if self._host is not None:
+                bad = self._host[~np.isfinite(self._host)]
+                self._finite = bad.size == 0
+                if not self._finite:
+                    raise TensorError("NonFiniteValue", f"non-finite value encountered in {label}: {bad[0]}", label=label)
+            else:
+                self._validate_result(label)
+        elif not self._finite:
+            raise TensorError("NonFiniteValue", f"non-finite value encountered in {label}", label=label)
+
+    def _validate_result(self, label: str) -> "Tensor":
+        """The post-operator finite check (pure.rs:2169, 4537) on the device: sixteen bytes come back, not the tensor."""
+        try:
+            found, _, value = hip.count_nonfinite_f32_dev(self.rows * self.cols, self._dev)
+        except hip.HipErr as err:
+            raise _backend_failure(err) from err
+        self._finite = found == 0
+        if found:
+            raise TensorError("NonFiniteValue", f"non-finite value encountered in {label}: {value}", label=label)
+        return self
+
+    @staticmethod
+    def _row_vector(values, expected: int) -> "Tensor":
+        """A bias given as a Tensor is used (and kept on the device) as it is; anything else becomes a 1×n Tensor."""
+        if isinstance(values, Tensor):
+            if values.rows * values.cols != expected:
+                raise TensorError("DataLength", f"expected {expected} values, got {values.rows * values.cols}",
+                                  expected=expected, got=values.rows * values.cols)
+            return values
+        flat = np.ascontiguousarray(np.asarray(values, dtype=np.float32)).reshape(-1)
+        if flat.size != expected:
+            raise TensorError("DataLength", f"expected {expected} values, got {flat.size}", expected=expected,
+                              got=flat.size)
+        return Tensor(1, expected, flat)
 
     # ---- dense matmul family ---------------------------------------------------------------------
     def _check_inner(self, other: "Tensor") -> None:
@@ -123,13 +213,12 @@ class Tensor:
         """C = (A·B)·scale — pure.rs:2200-2369."""
         _resolve_backend(backend)
         self._check_inner(other)
-        out = Tensor.zeros(self.rows, other.cols)
+        out = Tensor._on_device_result(self.rows, other.cols)
         try:
-            hip.gemm_scaled_f32(self.rows, other.cols, self.cols, scale, self._data, other._data, out._data)
+            hip.gemm_f32_dev(self.rows, other.cols, self.cols, scale, False, self._device(), other._device(), out._dev)
         except hip.HipErr as err:
             raise _backend_failure(err) from err
-        _validate_finite(f"{_op}_output", out._data)  # pure.rs:2169
-        return out
+        return out._validate_result(f"{_op}_output")  # pure.rs:2169
 
     def matmul_lhs_transpose_scaled(self, other: "Tensor", scale: float, *,
                                     backend: Optional[str] = None) -> "Tensor":
@@ -138,32 +227,26 @@ class Tensor:
         if self.rows != other.rows:
             raise TensorError("ShapeMismatch", f"left {self.shape()} right {other.shape()}",
                               left=self.shape(), right=other.shape())
-        out = Tensor.zeros(self.cols, other.cols)
+        out = Tensor._on_device_result(self.cols, other.cols)
         try:
-            hip.gemm_lhs_transpose_scaled_f32(self.cols, other.cols, self.rows, scale, self._data, other._data,
-                                              out._data)
+            hip.gemm_f32_dev(self.cols, other.cols, self.rows, scale, True, self._device(), other._device(), out._dev)
         except hip.HipErr as err:
             raise _backend_failure(err) from err
-        _validate_finite("matmul_lhs_transpose_scaled_output", out._data)
-        return out
+        return out._validate_result("matmul_lhs_transpose_scaled_output")
 
     def _fused(self, other: "Tensor", bias, residual: Optional["Tensor"], activation, label: str) -> "Tensor":
         self._check_inner(other)
-        bias = np.ascontiguousarray(np.asarray(bias, dtype=np.float32)).reshape(-1)
-        if bias.size != other.cols:
-            raise TensorError("DataLength", f"expected {other.cols} values, got {bias.size}",
-                              expected=other.cols, got=bias.size)
+        bias = Tensor._row_vector(bias, other.cols)
         if residual is not None and residual.shape() != (self.rows, other.cols):
             raise TensorError("ShapeMismatch", f"left {residual.shape()} right {(self.rows, other.cols)}",
                               left=residual.shape(), right=(self.rows, other.cols))
-        out = Tensor.zeros(self.rows, other.cols)
+        out = Tensor._on_device_result(self.rows, other.cols)
         try:
-            hip.gemm_bias_activation_f32(self.rows, other.cols, self.cols, activation, self._data, other._data, bias,
-                                         None if residual is None else residual._data, out._data)
+            hip.gemm_bias_act_f32_dev(self.rows, other.cols, self.cols, activation, self._device(), other._device(),
+                                      bias._device(), None if residual is None else residual._device(), out._dev)
         except hip.HipErr as err:
             raise _backend_failure(err) from err
-        _validate_finite(label, out._data)  # pure.rs:4537
-        return out
+        return out._validate_result(label)  # pure.rs:4537
 
     def matmul_bias_relu(self, other: "Tensor", bias, *, backend: Optional[str] = None) -> "Tensor":
         """relu(A·B + bias) — pure.rs:4411-4550."""
@@ -190,11 +273,9 @@ class Tensor:
 
     def matmul_prepacked_bias(self, packed: "PackedB", bias, *, backend: Optional[str] = None) -> "Tensor":
         """C = A·B + bias with B prepacked — pure.rs:2577-2757 (what Linear::forward calls, linear.rs:96-104)."""
-        bias = np.ascontiguousarray(np.asarray(bias, dtype=np.float32)).reshape(-1)
-        if self.cols == packed.inner() and bias.size != packed.cols():
-            raise TensorError("DataLength", f"expected {packed.cols()} values, got {bias.size}",
-                              expected=packed.cols(), got=bias.size)
-        _validate_finite("matmul_prepacked_bias_bias", bias)
+        if self.cols == packed.inner():
+            bias = Tensor._row_vector(bias, packed.cols())
+            bias._require_finite("matmul_prepacked_bias_bias")
         return self._prepacked(packed, bias, "matmul_prepacked_bias_output", backend)
 
     def _prepacked(self, packed: "PackedB", bias, label: str, backend: Optional[str]) -> "Tensor":
@@ -202,37 +283,41 @@ class Tensor:
         if self.cols != packed.inner():
             raise TensorError("ShapeMismatch", f"left {self.shape()} right {(packed.inner(), packed.cols())}",
                               left=self.shape(), right=(packed.inner(), packed.cols()))
-        out = Tensor.zeros(self.rows, packed.cols())
+        out = Tensor._on_device_result(self.rows, packed.cols())
         try:
-            hip.gemm_prepacked_bias_activation_f32(self.rows, packed.cols(), self.cols, 0, self._data,
-                                                   packed.as_slice(), bias, None, out._data)
+            hip.gemm_prepacked_bias_act_f32_dev(self.rows, packed.cols(), self.cols, 0, self._device(),
+                                                packed._device(), None if bias is None else bias._device(), None,
+                                                out._dev)
         except hip.HipErr as err:
             raise _backend_failure(err) from err
-        _validate_finite(label, out._data)
-        return out
+        return out._validate_result(label)
 
     # ---- tensor utilities ------------------------------------------------------------------------
-    def _on_device(self, run, out_values: int, *arrays) -> np.ndarray:
-        """Uploads `arrays`, calls run(device buffers..., output buffer) and downloads `out_values` floats."""
+    def _elementwise(self, run, rows: int, cols: int) -> "Tensor":
+        out = Tensor._on_device_result(rows, cols)
         try:
-            buffers = [hip.DeviceBuffer.from_array(a) for a in arrays]
-            out = hip.DeviceBuffer(max(out_values, 1) * 4)
-            run(*buffers, out)
-            hip.device_synchronize()
-            return out.to_array(np.float32, out_values)
+            run(out._dev)
         except hip.HipErr as err:
             raise _backend_failure(err) from err
+        return out
 
     def row_softmax(self, *, backend: Optional[str] = None) -> "Tensor":
         """Row-wise softmax — Tensor::row_softmax_with_backend, pure.rs:3282-3330 (inputs must be finite)."""
         _resolve_backend(backend)
-        _validate_finite("row_softmax_input", self._data)
-        if self._data.size == 0:
+        self._require_finite("row_softmax_input")
+        if len(self) == 0:
             return Tensor.zeros(self.rows, self.cols)
-        out = self._on_device(lambda x, y: hip.row_softmax_f32_dev(self.rows, self.cols, x, y), self._data.size,
-                              self._data)
-        _validate_finite("row_softmax_output", out)
-        return Tensor(self.rows, self.cols, out)
+        out = self._elementwise(lambda y: hip.row_softmax_f32_dev(self.rows, self.cols, self._device(), y), self.rows,
+                                self.cols)
+        return out._validate_result("row_softmax_output")
+
+    def gelu(self, *, backend: Optional[str] = None) -> "Tensor":
+        """gelu(self) — Gelu::forward, crates/st-nn/src/layers/gelu.rs:78-94."""
+        _resolve_backend(backend)
+        if len(self) == 0:
+            return Tensor.zeros(self.rows, self.cols)
+        out = self._elementwise(lambda y: hip.gelu_f32_dev(len(self), self._device(), y), self.rows, self.cols)
+        return out._validate_result("gelu_output")
 
     def gelu_backward(self, grad_output: "Tensor", *, backend: Optional[str] = None) -> "Tensor":
         """gelu'(self) ⊙ grad_output — Tensor::gelu_backward_with_backend, pure.rs:6459-6560."""
@@ -240,11 +325,10 @@ class Tensor:
         if self.shape() != grad_output.shape():
             raise TensorError("ShapeMismatch", f"left {self.shape()} right {grad_output.shape()}",
                               left=self.shape(), right=grad_output.shape())
-        if self._data.size == 0:
+        if len(self) == 0:
             return Tensor.zeros(self.rows, self.cols)
-        out = self._on_device(lambda z, g, y: hip.gelu_backward_f32_dev(self._data.size, z, g, y), self._data.size,
-                              self._data, grad_output._data)
-        return Tensor(self.rows, self.cols, out)
+        return self._elementwise(lambda y: hip.gelu_backward_f32_dev(len(self), self._device(), grad_output._device(), y),
+                                 self.rows, self.cols)
 
     def scale(self, value: float, *, backend: Optional[str] = None) -> "Tensor":
         """self · value — Tensor::scale_with_backend, pure.rs:5517-5620 (value must be finite)."""
@@ -252,42 +336,39 @@ class Tensor:
         if not np.isfinite(value):
             raise TensorError("NonFiniteValue", f"non-finite value encountered in scale_factor: {value}",
                               label="scale_factor")
-        if self._data.size == 0:
+        if len(self) == 0:
             return Tensor.zeros(self.rows, self.cols)
-        out = self._on_device(lambda x, y: hip.scale_f32_dev(self._data.size, x, float(value), y), self._data.size,
-                              self._data)
-        return Tensor(self.rows, self.cols, out)
+        return self._elementwise(lambda y: hip.scale_f32_dev(len(self), self._device(), float(value), y), self.rows,
+                                 self.cols)
 
     def add_row_inplace(self, bias, *, backend: Optional[str] = None) -> None:
         """self[r, :] += bias — Tensor::add_row_inplace_with_backend, pure.rs:6201-6290."""
         _resolve_backend(backend)
-        bias = np.ascontiguousarray(np.asarray(bias, dtype=np.float32)).reshape(-1)
-        if bias.size != self.cols:
-            raise TensorError("DataLength", f"expected {self.cols} values, got {bias.size}", expected=self.cols,
-                              got=bias.size)
-        if self._data.size == 0:
+        bias = Tensor._row_vector(bias, self.cols)
+        if len(self) == 0:
             return
         try:
-            data, row = hip.DeviceBuffer.from_array(self._data), hip.DeviceBuffer.from_array(bias)
-            hip.add_row_f32_dev(self.rows, self.cols, data, row)
-            hip.device_synchronize()
-            self._data[:] = data.to_array(np.float32, self._data.size)
+            hip.add_row_f32_dev(self.rows, self.cols, self._device(), bias._device())
         except hip.HipErr as err:
             raise _backend_failure(err) from err
+        self._host = None   # the device copy is now the tensor
+        self._finite = None
 
     def sum_axis0(self, *, backend: Optional[str] = None) -> np.ndarray:
         """Column sums — Tensor::sum_axis0_with_backend, pure.rs:7009-7116."""
         return self.sum_axis0_scaled(1.0, backend=backend)
 
     def sum_axis0_scaled(self, scale: float, *, backend: Optional[str] = None) -> np.ndarray:
-        """scale · column sums — Tensor::sum_axis0_scaled_with_backend, pure.rs:7118-7230."""
+        """scale · column sums — Tensor::sum_axis0_scaled_with_backend, pure.rs:7118-7230 (a Vec<f32> there, a host
+        array here)."""
         _resolve_backend(backend)
         if self.cols == 0:
             return np.zeros(0, dtype=np.float32)
         if self.rows == 0:
             return np.zeros(self.cols, dtype=np.float32)
-        return self._on_device(lambda x, y: hip.sum_axis0_f32_dev(self.rows, self.cols, x, float(scale), y),
-                               self.cols, self._data)
+        out = self._elementwise(lambda y: hip.sum_axis0_f32_dev(self.rows, self.cols, self._device(), float(scale), y),
+                                1, self.cols)
+        return np.array(out.data())
 
     # ---- attention -------------------------------------------------------------------------------
     def scaled_dot_attention(self, keys: "Tensor", values: "Tensor", *, contexts: int, sequence: int,
@@ -308,14 +389,23 @@ class Tensor:
         if attn_bias is not None and attn_bias.shape() != (expected_rows, sequence):
             raise TensorError("ShapeMismatch", f"left {attn_bias.shape()} right {(expected_rows, sequence)}",
                               left=attn_bias.shape(), right=(expected_rows, sequence))
-        out = Tensor.zeros(expected_rows, self.cols)
+        # Finite checks in the order of pure.rs:4148-4157.
+        if not np.isfinite(scale):
+            raise TensorError("NonFiniteValue", f"non-finite value encountered in scaled_dot_attention_scale: {scale}",
+                              label="scaled_dot_attention_scale")
+        for t, name in ((self, "query"), (keys, "key"), (values, "value"), (z_bias, "z_bias"), (attn_bias, "attn_bias")):
+            if t is not None:
+                t._require_finite(f"scaled_dot_attention_{name}")
+        if expected_rows == 0 or self.cols == 0:
+            return Tensor.zeros(expected_rows, self.cols)  # pure.rs:4171-4193
+        out = Tensor._on_device_result(expected_rows, self.cols)
         try:
-            hip.attention_f32(contexts, sequence, self.cols, scale, causal, self._data, keys._data, values._data,
-                              None if z_bias is None else z_bias._data,
-                              None if attn_bias is None else attn_bias._data, out._data)
+            hip.attention_f32_dev(contexts, sequence, self.cols, scale, causal, self._device(), keys._device(),
+                                  values._device(), None if z_bias is None else z_bias._device(),
+                                  None if attn_bias is None else attn_bias._device(), out._dev)
         except hip.HipErr as err:
             raise _backend_failure(err) from err
-        return out
+        return out._validate_result("scaled_dot_attention_output")  # pure.rs:4206-4210
 
 
 class Conv2d:
@@ -364,11 +454,13 @@ class Conv2d:
             raise TensorError("ShapeMismatch", f"left {input.shape()} right {(input.rows, self.in_channels * h * w)}",
                               left=input.shape(), right=(input.rows, self.in_channels * h * w))
         oh, ow = self.output_hw()
-        out = Tensor.zeros(input.rows, self.out_channels * oh * ow)
+        if input.rows == 0:
+            return Tensor.zeros(0, self.out_channels * oh * ow)  # conv.rs:4132-4137
+        out = Tensor._on_device_result(input.rows, self.out_channels * oh * ow)
         try:
-            hip.conv2d_bias_activation_f32(input.rows, self.in_channels, h, w, self.out_channels, self.kernel,
-                                           self.stride, self.padding, self.dilation, self.activation, input.data(),
-                                           self.weight.data(), self.bias.data(), out.data())
+            hip.conv2d_bias_act_f32_dev(input.rows, self.in_channels, h, w, self.out_channels, self.kernel, self.stride,
+                                        self.padding, self.dilation, self.activation, input._device(),
+                                        self.weight._device(), self.bias._device(), out._dev)
         except hip.HipErr as err:
             raise _backend_failure(err) from err
         return out
@@ -388,15 +480,18 @@ class Conv2d:
             raise TensorError("ShapeMismatch",
                               f"left {grad_output.shape()} right {(input.rows, self.out_channels * oh * ow)}",
                               left=grad_output.shape(), right=(input.rows, self.out_channels * oh * ow))
-        grad_input = Tensor.zeros(input.rows, input.cols)
         if input.rows == 0:
-            return grad_input
-        grad_weight = Tensor.zeros(*self.weight.shape())
-        grad_bias = Tensor.zeros(1, self.out_channels)
+            return Tensor.zeros(0, input.cols)
+        grad_input = Tensor._on_device_result(input.rows, input.cols)
+        grad_weight = Tensor._on_device_result(*self.weight.shape())
+        grad_bias = Tensor._on_device_result(1, self.out_channels)
+        shape = (input.rows, self.in_channels, h, w, self.out_channels, self.kernel, self.stride, self.padding,
+                 self.dilation)
+        scale = 1.0 / input.rows  # conv.rs:793,799
         try:
-            hip.conv2d_backward_f32(input.rows, self.in_channels, h, w, self.out_channels, self.kernel, self.stride,
-                                    self.padding, self.dilation, input.data(), self.weight.data(), grad_output.data(),
-                                    grad_input.data(), grad_weight.data(), grad_bias.data())
+            hip.conv2d_grad_weight_f32_dev(*shape, input._device(), grad_output._device(), scale, grad_weight._dev)
+            hip.conv2d_grad_bias_f32_dev(*shape, grad_output._device(), scale, grad_bias._dev)
+            hip.conv2d_grad_input_f32_dev(*shape, grad_output._device(), self.weight._device(), grad_input._dev)
         except hip.HipErr as err:
             raise _backend_failure(err) from err
         for name, update in (("weight_gradient", grad_weight), ("bias_gradient", grad_bias)):
@@ -404,7 +499,7 @@ class Conv2d:
             if existing is None:
                 setattr(self, name, update)
             else:
-                existing.data()[:] += update.data()
+                existing.data_mut()[:] += update.data()
         return grad_input
 
     def zero_accumulators(self) -> None:

@@ -144,3 +144,96 @@ def test_tensor_mirror_methods(hip, oracle):
     with pytest.raises(st.TensorError, match="NonFiniteValue"):
         bad.row_softmax()
     assert st.Tensor.zeros(0, 5).sum_axis0().tolist() == [0.0] * 5
+
+
+def test_operator_chains_stay_on_the_device(hip, oracle):
+    """Linear -> GELU -> Linear through the Tensor mirror (Linear::forward = matmul_prepacked_bias,
+    crates/st-nn/src/layers/linear.rs:96-104; Gelu::forward, layers/gelu.rs:78-94): every input is uploaded once,
+    intermediate results never leave the device, and only the final values are downloaded."""
+    import spiraltorch_amd as st
+    rng = np.random.default_rng(3)
+    batch, d_in, d_hidden, d_out = 96, 64, 160, 48
+    x = st.Tensor(batch, d_in, rng.normal(size=batch * d_in).astype(np.float32))
+    w1 = st.Tensor(d_in, d_hidden, rng.normal(0, 0.2, d_in * d_hidden).astype(np.float32))
+    w2 = st.Tensor(d_hidden, d_out, rng.normal(0, 0.2, d_hidden * d_out).astype(np.float32))
+    b1 = st.Tensor(1, d_hidden, rng.normal(size=d_hidden).astype(np.float32))
+    b2 = st.Tensor(1, d_out, rng.normal(size=d_out).astype(np.float32))
+    p1, p2 = st.PackedB.from_tensor(w1), st.PackedB.from_tensor(w2)
+
+    hip.transfer_counters(reset=True)
+    hidden = x.matmul_prepacked_bias(p1, b1)
+    activated = hidden.gelu()
+    y = activated.matmul_prepacked_bias(p2, b2)
+    on_device = hip.transfer_counters()
+    assert on_device["h2d_copies"] == 5                       # x, packed w1, b1, packed w2, b2: once each
+    assert on_device["h2d_bytes"] == 4 * (x.data().size + w1.data().size + w2.data().size + d_hidden + d_out)
+    assert on_device["d2h_copies"] == 0 and on_device["d2h_bytes"] == 0
+    assert hidden.is_device_resident() and activated.is_device_resident()
+    values = y.data()
+    after = hip.transfer_counters()
+    assert after["d2h_copies"] == 1 and after["d2h_bytes"] == 4 * batch * d_out
+    y.data()                                                  # cached: no second download
+    assert hip.transfer_counters()["d2h_copies"] == 1
+
+    want_hidden = oracle.gemm_bias_act_f32(batch, d_hidden, d_in, oracle.ACT_GELU, x.data(), w1.data(), b1.data())
+    want = oracle.gemm_f32(batch, d_out, d_hidden, want_hidden, w2.data()).reshape(batch, d_out) + b2.data()
+    assert_close(values, want, F32_REL, 2 * F32_ABS, "Linear -> GELU -> Linear")
+
+    # a second pass over the same tensors uploads nothing at all
+    hip.transfer_counters(reset=True)
+    again = x.matmul_prepacked_bias(p1, b1).gelu().matmul_prepacked_bias(p2, b2)
+    assert hip.transfer_counters()["h2d_copies"] == 0
+    assert (again.data() == values).all()
+
+    # writing through data_mut() drops the device copy: the next operator sees the new values
+    x.data_mut()[:] = 0.0
+    zeroed = x.matmul_prepacked_bias(p1, b1)
+    assert_close(zeroed.data(), np.tile(b1.data(), batch), 0, 1e-6, "after data_mut")
+    with pytest.raises(ValueError):
+        x.data()[0] = 1.0                                     # data() is read-only
+
+
+def test_nonfinite_results_are_caught_on_the_device(hip):
+    """The reference's output finite check (pure.rs:2169), without bringing the tensor back."""
+    import spiraltorch_amd as st
+    a = st.Tensor(4, 4, np.full(16, 3e38, np.float32))
+    hip.transfer_counters(reset=True)
+    with pytest.raises(st.TensorError) as err:
+        a.matmul(st.Tensor(4, 4, np.full(16, 10.0, np.float32)))
+    assert err.value.kind == "NonFiniteValue" and err.value.fields["label"] == "matmul_output"
+    assert "inf" in err.value.message
+    assert hip.transfer_counters()["d2h_copies"] == 0
+    rng = np.random.default_rng(0)
+    values = rng.normal(size=1000).astype(np.float32)
+    buf = hip.DeviceBuffer.from_array(values)
+    assert hip.count_nonfinite_f32_dev(1000, buf) == (0, 0, 0.0)
+    values[[17, 500]] = [np.nan, -np.inf]
+    buf = hip.DeviceBuffer.from_array(values)
+    found, first, value = hip.count_nonfinite_f32_dev(1000, buf)
+    assert (found, first) == (2, 17) and np.isnan(value)
+    assert hip.count_nonfinite_f32_dev(0, None)[0] == 0
+
+
+def test_gelu_forward_matches_the_oracle(hip, oracle):
+    import spiraltorch_amd as st
+    x = st.Tensor(3, 50, np.linspace(-6, 6, 150).astype(np.float32))
+    want = np.array([oracle.gelu(float(v)) for v in x.data()])
+    assert_close(x.gelu().data(), want, F32_REL, F32_ABS, "gelu")
+
+
+def test_raw_gemm_and_probe(hip):
+    """gemm_f32_raw and probe() of crates/st-backend-hip/src/lib.rs:188-207, 760-799."""
+    a = np.arange(1, 7, dtype=np.float32)
+    b = np.arange(7, 13, dtype=np.float32)
+    out = np.zeros(4, np.float32)
+    hip.gemm_f32_raw(2, 2, 3, a.ctypes.data, b.ctypes.data, out.ctypes.data)
+    assert out.tolist() == [58, 64, 139, 154]                 # lib.rs:1107-1112
+    with pytest.raises(hip.HipErr, match="gemm received a null pointer; provide contiguous row-major buffers"):
+        hip.gemm_f32_raw(2, 2, 3, a.ctypes.data, None, out.ctypes.data)
+    with pytest.raises(hip.HipErr, match="gemm dimensions overflow while constructing lhs slice"):
+        hip.gemm_f32_raw(2 ** 40, 2, 2 ** 40, a.ctypes.data, b.ctypes.data, out.ctypes.data)
+    assert out.tolist() == [58, 64, 139, 154]
+    report = hip.probe()
+    assert report["available"] and report["initialized"] and report["error"] is None
+    assert len(report["devices"]) == hip.device_count() >= 1
+    assert hip.runtime() is not None
