@@ -114,7 +114,10 @@ class Tensor:
         out = cls.__new__(cls)
         out.rows, out.cols = int(rows), int(cols)
         out._host = None
-        out._dev = hip.DeviceBuffer(max(out.rows * out.cols, 1) * 4)
+        try:
+            out._dev = hip.DeviceBuffer(max(out.rows * out.cols, 1) * 4)
+        except hip.HipErr as err:
+            raise _backend_failure(err) from err
         out._finite = None
         return out
 
