@@ -255,8 +255,9 @@ __global__ __launch_bounds__(256) void attention_f32_kernel(AttnArgs p)
 // Same transposed formulation as the general kernel above, tuned for the matrix pipe:
 //   * 64 keys (two 32-key tiles) per softmax step: the two QKᵀ accumulations are independent MFMA
 //     chains, and the max / exchange / rescale bookkeeping is paid once per 64 keys;
-//   * V is staged TRANSPOSED (Vt[d][key]) so that the four keys a lane needs for four consecutive
-//     PV steps are one 128-bit LDS read (8 reads per 64 keys and 32 output rows, instead of 64);
+//   * V is staged exactly as stored (rows = keys, 128-bit writes); the PV operand is one conflict-free 32-bit
+//     read per MFMA at an immediate offset.  (Staging V transposed saved three of four reads, but its 32-bit
+//     scatter writes spent more than half of the LDS cycles on bank conflicts.)
 //   * the output accumulator is rescaled only when some lane's running maximum actually moved
 //     (wavefront-uniform test) — after the first few key tiles it almost never does;
 //   * exp2 is the bare v_exp_f32 (arguments are <= 0; results below 2^-126 may flush to zero);
@@ -266,19 +267,21 @@ __global__ __launch_bounds__(256) void attention_f32_kernel(AttnArgs p)
 // -------------------------------------------------------------------------------------------------
 typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
 
+// (Up to head_dim 64 two workgroups fit a compute unit, i.e. two wavefronts per SIMD: the register allocation is
+// held to that; the 128-wide form has LDS for one workgroup only.)
 template <int DPAD, bool CAUSAL>
-__global__ __launch_bounds__(256) void attention_f32_fast_kernel(AttnArgs p)
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DPAD <= 64 ? 2 : 1))) void attention_f32_fast_kernel(AttnArgs p)
 {
     constexpr int BKV = 64;
     constexpr int KS = DPAD + 4;   // K row stride (floats)
-    constexpr int VTS = BKV + 4;   // Vt row stride (floats): rows are head-dim indices, columns keys
-    constexpr int K_ELEMS = BKV * KS, V_ELEMS = DPAD * VTS;
+    constexpr int VS = DPAD + 8;   // V row stride (floats): four rows are 32 banks apart (see the PV reads)
+    constexpr int K_ELEMS = BKV * KS, V_ELEMS = BKV * VS;
     constexpr int CHUNKS = DPAD / 8;
     constexpr int DT = DPAD / 32;
     constexpr int LOADS = BKV * DPAD / 4 / 256;
     extern __shared__ __attribute__((aligned(16))) float attn_lds[];
     float *Ks = attn_lds;                // [2][K_ELEMS]
-    float *Vt = attn_lds + 2 * K_ELEMS;  // [2][V_ELEMS]
+    float *Vs = attn_lds + 2 * K_ELEMS;  // [2][V_ELEMS]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -286,34 +289,24 @@ __global__ __launch_bounds__(256) void attention_f32_fast_kernel(AttnArgs p)
     const int li = lane & 31, lh = lane >> 5;
     const int S = p.S, D = p.D;
 
-    // Workgroup -> (context, query tile).  Workgroup ids are dealt round-robin to the 8 XCDs, so id & 7 picks
-    // the XCD; each XCD keeps its own slice of the contexts (their K/V stay in that XCD's L2).  Under the
-    // causal mask a query tile's cost grows with its index, so every XCD runs its tiles longest-first
-    // across ALL of its contexts (tile q_tiles-1 of every context, then q_tiles-2, ...): the short tiles at
-    // the end fill the gaps the long ones leave.
-    int ctx, q_tile;
+    // Workgroup -> (context, query tiles).  Workgroup ids are dealt round-robin to the 8 XCDs, so id & 7 picks the
+    // XCD; each XCD keeps its own slice of the contexts and walks it context by context, so the workgroups that run
+    // together read the same K/V and those stay in that XCD's L2.  Under the causal mask a query tile's cost grows
+    // with its index, so a workgroup takes a PAIR of tiles, j and q_tiles-1-j, one after the other: every workgroup
+    // then does the same amount of work (q_tiles+1 key tiles), which balances the chip without spreading each
+    // context's tiles over the whole launch (longest-first across all contexts balanced as well, but re-read K/V
+    // from memory three times over).
+    const int per_ctx = CAUSAL ? (p.q_tiles + 1) / 2 : p.q_tiles;  // workgroups per context
+    int ctx, unit;
     if (p.swizzle) {
         const int per_xcd = p.contexts >> 3;
         const int xcd = blockIdx.x & 7, i = blockIdx.x >> 3;
-        if (CAUSAL) {
-            q_tile = p.q_tiles - 1 - i / per_xcd;
-            ctx = xcd * per_xcd + i % per_xcd;
-        } else {
-            ctx = xcd * per_xcd + i / p.q_tiles;
-            q_tile = i % p.q_tiles;
-        }
+        ctx = xcd * per_xcd + i / per_ctx;
+        unit = i % per_ctx;
     } else {
-        if (CAUSAL) {
-            q_tile = p.q_tiles - 1 - blockIdx.x / p.contexts;
-            ctx = blockIdx.x % p.contexts;
-        } else {
-            ctx = blockIdx.x / p.q_tiles;
-            q_tile = blockIdx.x % p.q_tiles;
-        }
+        ctx = blockIdx.x / per_ctx;
+        unit = blockIdx.x % per_ctx;
     }
-    const int q0 = q_tile * kBQ;
-    const int wq0 = q0 + wave * 32;
-    const int my_q = wq0 + li;
     const size_t ctx_elem0 = static_cast<size_t>(ctx) * S * D;
     const unsigned ctx_bytes = static_cast<unsigned>(S) * static_cast<unsigned>(D) * 4u;
     const __amdgpu_buffer_rsrc_t rsrc_q =
@@ -331,6 +324,12 @@ __global__ __launch_bounds__(256) void attention_f32_fast_kernel(AttnArgs p)
         return v;
     };
 
+    const int passes = (CAUSAL && unit != p.q_tiles - 1 - unit) ? 2 : 1;
+    for (int pass = 0; pass < passes; ++pass) {
+    const int q_tile = CAUSAL ? (pass == 0 ? p.q_tiles - 1 - unit : unit) : unit;  // the long tile first
+    const int q0 = q_tile * kBQ;
+    const int wq0 = q0 + wave * 32;
+    const int my_q = wq0 + li;
     // Q fragments: qf[c][s] = Q[my_q][8c + 4h + s]; rows past the end read as zero.
     float qf[CHUNKS][4];
 #pragma unroll
@@ -366,16 +365,13 @@ __global__ __launch_bounds__(256) void attention_f32_fast_kernel(AttnArgs p)
     };
     auto store_lds = [&](int stage) {
         float *ks = Ks + stage * K_ELEMS;
-        float *vt = Vt + stage * V_ELEMS;
+        float *vs = Vs + stage * V_ELEMS;
 #pragma unroll
         for (int r = 0; r < LOADS; ++r) {
             const int f = tid + 256 * r;
             const int row = f / (DPAD / 4), c4 = (f % (DPAD / 4)) * 4;
             *reinterpret_cast<float4 *>(&ks[row * KS + c4]) = rk[r];
-            vt[(c4 + 0) * VTS + row] = rv[r].x;
-            vt[(c4 + 1) * VTS + row] = rv[r].y;
-            vt[(c4 + 2) * VTS + row] = rv[r].z;
-            vt[(c4 + 3) * VTS + row] = rv[r].w;
+            *reinterpret_cast<float4 *>(&vs[row * VS + c4]) = rv[r];
         }
     };
 
@@ -388,7 +384,7 @@ __global__ __launch_bounds__(256) void attention_f32_fast_kernel(AttnArgs p)
     auto compute = [&](auto nt_tag, int stage, int key0) {
         constexpr int NT = decltype(nt_tag)::value;
         const float *ks = Ks + stage * K_ELEMS;
-        const float *vt = Vt + stage * V_ELEMS;
+        const float *vs = Vs + stage * V_ELEMS;
         f32x16 sacc[NT];
 #pragma unroll
         for (int t = 0; t < NT; ++t)
@@ -453,22 +449,26 @@ __global__ __launch_bounds__(256) void attention_f32_fast_kernel(AttnArgs p)
                 tile_sum += pr;
             }
         run_sum += tile_sum;
-        // Oᵀ += Vᵀ·Pᵀ: for register group g the lane needs keys 8g + 4h .. +3 of its head-dim row: one 128-bit read.
+        // Oᵀ += Vᵀ·Pᵀ with V as stored (rows = keys): probability register r of lane half h belongs to key
+        // (r/4)*8 + 4h + r%4, so the A operand of that MFMA is V[that key][32·dt + li] — one 32-bit read whose 64
+        // lanes cover 32 consecutive floats of two rows four apart, 32 banks apart with the row stride above: no
+        // bank conflicts, nothing transposed on the way into LDS, and every address is this lane's base plus an
+        // immediate.
+        const float *v_lane = vs + (lh * 4) * VS + li;
 #pragma unroll
         for (int t = 0; t < NT; ++t)
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                float4 vv[DT];
+                float vv[DT][4];
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt)
-                    vv[dt] = *reinterpret_cast<const float4 *>(&vt[(dt * 32 + li) * VTS + t * 32 + g * 8 + lh * 4]);
 #pragma unroll
-                for (int dt = 0; dt < DT; ++dt) {
-                    oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv[dt].x, sacc[t][g * 4 + 0], oacc[dt], 0, 0, 0);
-                    oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv[dt].y, sacc[t][g * 4 + 1], oacc[dt], 0, 0, 0);
-                    oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv[dt].z, sacc[t][g * 4 + 2], oacc[dt], 0, 0, 0);
-                    oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv[dt].w, sacc[t][g * 4 + 3], oacc[dt], 0, 0, 0);
-                }
+                    for (int e = 0; e < 4; ++e) vv[dt][e] = v_lane[(t * 32 + g * 8 + e) * VS + dt * 32];
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv[dt][e], sacc[t][g * 4 + e], oacc[dt], 0, 0, 0);
             }
     };
 
@@ -503,17 +503,18 @@ __global__ __launch_bounds__(256) void attention_f32_fast_kernel(AttnArgs p)
                                                                         oacc[t][g * 4 + 2] * inv, oacc[t][g * 4 + 3] * inv);
             }
     }
+    }  // pass
 }
 
 template <int DPAD, bool CAUSAL>
 hipError_t launch_fast(const AttnArgs &args, hipStream_t stream)
 {
-    constexpr size_t lds_bytes = 2 * (static_cast<size_t>(64) * (DPAD + 4) + static_cast<size_t>(DPAD) * (64 + 4)) * sizeof(float);
+    constexpr size_t lds_bytes = 2 * static_cast<size_t>(64) * ((DPAD + 4) + (DPAD + 8)) * sizeof(float);
     auto kernel = attention_f32_fast_kernel<DPAD, CAUSAL>;
     hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
     if (rc != hipSuccess) return rc;
-    const size_t blocks = static_cast<size_t>(args.contexts) * args.q_tiles;
+    const size_t blocks = static_cast<size_t>(args.contexts) * (CAUSAL ? (args.q_tiles + 1) / 2 : args.q_tiles);
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), lds_bytes, stream, args);
     return hipGetLastError();
 }

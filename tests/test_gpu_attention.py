@@ -29,6 +29,8 @@ CASES = [
     (1, 40, 16, True, True), (4, 64, 64, False, False), (2, 129, 64, True, False), (3, 200, 32, False, False),
     (2, 257, 64, False, True), (1, 300, 128, True, False), (1, 130, 80, False, False), (2, 96, 256, True, False),
     (1, 70, 200, False, True), (5, 128, 64, True, True), (8, 384, 64, True, False),
+    # causal query tiles are taken in pairs (j, last - j): five tiles (the middle one alone), four tiles, one XCD slice each
+    (8, 600, 64, True, False), (16, 512, 32, True, False), (3, 1100, 64, True, False),
 ]
 
 
