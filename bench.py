@@ -39,12 +39,17 @@ PEAK_HBM_GBS = 8000.0
 # scaled x2.0 and WRITE_SIZE x1.0, the factors a streaming kernel of known size gives on this chip).  The
 # summaries live in profiles/dominant_kernels_counters.md; workloads not listed there report null.
 MEASURED_TRAFFIC_BYTES = {
-    "conv2d_bias_relu_f32_n32_c64to128_56x56_k3s1p1": (14304 * 2 + 50176) * 1024,
-    "conv2d_grad_input_f32_n32_c64to128_56x56_k3s1p1": (30742 * 2 + 25088) * 1024,
-    "gemm_bf16_f32acc_4096x4096x4096": (98558 * 2 + 65536) * 1024,
-    "gemm_bf16_f32acc_16x4096x4096": (16927 * 2 + 2048) * 1024,
-    "attention_f32_b8_h16_s2048_d64_noncausal": (98387 * 2 + 65536) * 1024,
-    "attention_f32_b8_h16_s2048_d64_causal": (371670 * 2 + 65544) * 1024,
+    "conv2d_bias_relu_f32_n32_c64to128_56x56_k3s1p1": (14305 * 2 + 50176) * 1024,
+    "conv2d_grad_input_f32_n32_c64to128_56x56_k3s1p1": (30664 * 2 + 25088) * 1024,
+    "conv2d_grad_weight_f32_n32_c64to128_56x56_k3s1p1": ((44175 + 36161) * 2 + 72288 + 288) * 1024,
+    "gemm_bf16_f32acc_4096x4096x4096": (98736 * 2 + 65536) * 1024,
+    "gemm_bf16_f32acc_4096x4096x4096_prepacked_rhs": (98536 * 2 + 65536) * 1024,
+    "gemm_bf16_f32acc_16x4096x4096": ((16927 + 1045) * 2 + 2048 + 256) * 1024,
+    "attention_f32_b8_h16_s2048_d64_noncausal": (98379 * 2 + 65536) * 1024,
+    "attention_f32_b8_h16_s2048_d64_causal": (137761 * 2 + 65540) * 1024,
+    "gemm_f32_100352x128x576_conv_equivalent": (139548 * 2 + 50176) * 1024,
+    "gemm_f32_4096x4096x4096": (196753 * 2 + 65536) * 1024,
+    "attention_bf16_b16_h8_s1024_d64_causal": (24968 * 2 + 16384) * 1024,
 }
 
 
