@@ -100,8 +100,9 @@ hipError_t launch_scale_f32(size_t count, const float *in, float scale, float *o
 hipError_t launch_add_row_f32(size_t rows, size_t cols, float *data, const float *bias, hipStream_t stream);
 hipError_t launch_sum_axis0_f32(size_t rows, size_t cols, const float *in, float scale, float *out, hipStream_t stream);
 
-// One grow-only device buffer per stream for kernels that need scratch memory (split-k partial sums, column-sum
-// partials).  Work on a stream is ordered, so two launches on the same stream never use it at the same time.
+// One grow-only device buffer per (stream, host thread) for kernels that need scratch memory (split-k partial sums,
+// column-sum partials).  A thread's work on a stream is ordered, so two of its launches never use the buffer at the
+// same time, and threads that share a stream (the NULL stream) do not share scratch.
 hipError_t stream_workspace(hipStream_t stream, size_t bytes, void **out);
 void release_stream_workspace(hipStream_t stream);
 // Host<->device copies made by the library, for tests that check where tensors live.

@@ -7,6 +7,7 @@
 #include <cstring>
 #include <mutex>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include "common.h"
@@ -95,8 +96,13 @@ void count_transfer(bool to_device, size_t bytes)
 }
 
 namespace {
+// Scratch is keyed by (stream, host thread): launches on one stream from one thread are ordered, so they never use
+// the buffer at the same time; two host threads that share a stream (every caller that passes none shares the
+// NULL stream) each get a buffer of their own, so one thread growing its scratch can never free memory that a
+// kernel the other thread has just been handed is about to use.
 struct WorkspaceEntry {
     hipStream_t stream;
+    std::thread::id owner;
     void *ptr;
     size_t capacity;
 };
@@ -106,25 +112,32 @@ std::vector<WorkspaceEntry> workspace_entries;
 
 hipError_t stream_workspace(hipStream_t stream, size_t bytes, void **out)
 {
+    const std::thread::id me = std::this_thread::get_id();
     std::lock_guard<std::mutex> lock(workspace_mutex);
     for (WorkspaceEntry &e : workspace_entries) {
-        if (e.stream != stream) continue;
-        if (e.capacity < bytes) {
-            // Grow: earlier launches on this stream may still be using the old buffer.
+        if (e.stream != stream || e.owner != me) continue;
+        if (e.capacity < bytes || e.ptr == nullptr) {
+            // Grow: earlier launches of this thread on this stream may still be using the old buffer.
             hipError_t rc = hipStreamSynchronize(stream);
             if (rc != hipSuccess) return rc;
-            rc = hipFree(e.ptr);
-            if (rc != hipSuccess) return rc;
+            if (e.ptr) {
+                rc = hipFree(e.ptr);
+                if (rc != hipSuccess) return rc;
+            }
             e.ptr = nullptr;
             e.capacity = 0;
-            rc = hipMalloc(&e.ptr, bytes);
-            if (rc != hipSuccess) return rc;
-            e.capacity = bytes;
+            const size_t wanted = bytes ? bytes : 256;
+            rc = hipMalloc(&e.ptr, wanted);
+            if (rc != hipSuccess) {
+                e.ptr = nullptr;
+                return rc;
+            }
+            e.capacity = wanted;
         }
         *out = e.ptr;
         return hipSuccess;
     }
-    WorkspaceEntry fresh{stream, nullptr, bytes ? bytes : 256};
+    WorkspaceEntry fresh{stream, me, nullptr, bytes ? bytes : 256};
     hipError_t rc = hipMalloc(&fresh.ptr, fresh.capacity);
     if (rc != hipSuccess) return rc;
     workspace_entries.push_back(fresh);
@@ -136,11 +149,10 @@ hipError_t stream_workspace(hipStream_t stream, size_t bytes, void **out)
 void release_stream_workspace(hipStream_t stream)
 {
     std::lock_guard<std::mutex> lock(workspace_mutex);
-    for (size_t i = 0; i < workspace_entries.size(); ++i) {
+    for (size_t i = workspace_entries.size(); i-- > 0;) {
         if (workspace_entries[i].stream != stream) continue;
         (void)hipFree(workspace_entries[i].ptr);
         workspace_entries.erase(workspace_entries.begin() + static_cast<long>(i));
-        return;
     }
 }
 

@@ -237,3 +237,42 @@ def test_raw_gemm_and_probe(hip):
     assert report["available"] and report["initialized"] and report["error"] is None
     assert len(report["devices"]) == hip.device_count() >= 1
     assert hip.runtime() is not None
+
+
+def test_threads_sharing_the_null_stream_do_not_share_scratch(hip, oracle):
+    """Kernels with scratch memory (here the split-k bf16 GEMM and the column sums) called from several host
+    threads on the NULL stream, with sizes that make every thread's scratch grow: each result stays right."""
+    import threading
+    from spiraltorch_amd import inputs
+    failures = []
+
+    def work(index):
+        try:
+            rng = np.random.default_rng(index)
+            for round_ in range(6):
+                m, n, k = 8 + 8 * index, 128 * (1 + (round_ + index) % 4), 256 * (1 + round_ % 3)
+                a = inputs.to_bf16(rng.normal(0, 0.5, m * k).astype(np.float32))
+                b = inputs.to_bf16(rng.normal(0, 0.5, k * n).astype(np.float32))
+                d_a, d_b, d_c = hip.DeviceBuffer.from_array(a), hip.DeviceBuffer.from_array(b), hip.DeviceBuffer(m * n * 4)
+                hip.gemm_bf16_f32acc_dev(m, n, k, d_a, d_b, d_c)
+                rows, cols = 300 + 100 * round_, 64 * (index + 1)
+                x = rng.normal(size=rows * cols).astype(np.float32)
+                d_x, d_s = hip.DeviceBuffer.from_array(x), hip.DeviceBuffer(cols * 4)
+                hip.sum_axis0_f32_dev(rows, cols, d_x, 1.0, d_s)
+                hip.device_synchronize()
+                got = d_c.to_array(np.float32, m * n)
+                want = oracle.gemm_bf16_f32acc(m, n, k, a, b)
+                if np.abs(got - want).max() > 1e-3 * max(1.0, np.abs(want).max()):
+                    failures.append(("gemm", index, round_))
+                sums = d_s.to_array(np.float32, cols)
+                if np.abs(sums - x.reshape(rows, cols).astype(np.float64).sum(axis=0)).max() > 1e-3:
+                    failures.append(("sum", index, round_))
+        except Exception as err:  # noqa: BLE001
+            failures.append((index, repr(err)))
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not failures, failures
