@@ -250,7 +250,8 @@ __global__ __launch_bounds__(256) void attention_f32_kernel(AttnArgs p)
 }
 
 // -------------------------------------------------------------------------------------------------
-// Fast path: no additive biases, head_dim a multiple of 4, 16-byte aligned operands.
+// Fast path: head_dim a multiple of 4, 16-byte aligned operands; BIAS adds z_bias / attn_bias where their rows can
+// be read 128 bits at a time (sequence a multiple of 4), otherwise biased calls take the general kernel above.
 //
 // Same transposed formulation as the general kernel above, tuned for the matrix pipe:
 //   * 64 keys (two 32-key tiles) per softmax step: the two QKᵀ accumulations are independent MFMA
@@ -269,7 +270,7 @@ typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
 
 // (Up to head_dim 64 two workgroups fit a compute unit, i.e. two wavefronts per SIMD: the register allocation is
 // held to that; the 128-wide form has LDS for one workgroup only.)
-template <int DPAD, bool CAUSAL>
+template <int DPAD, bool CAUSAL, bool BIAS>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DPAD <= 64 ? 2 : 1))) void attention_f32_fast_kernel(AttnArgs p)
 {
     constexpr int BKV = 64;
@@ -379,7 +380,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DPAD <= 64 
     // p = exp2(fma(dot, scale·log2e, −max·scale·log2e)).  (Floored at a tiny positive value so that a zero scale
     // still turns masked (−inf) logits into weight 0 instead of −inf·0.)
     const float scale_log2e = fmaxf(fabsf(p.scale) * kLog2e, 1e-30f);
-    const float lag = 8.0f / scale_log2e;  // 2^8 in units of the raw dot product, see below
+    // With additive biases the logits are formed explicitly (dot·scale·log2e + bias·log2e) before the maximum is
+    // taken, so everything after that works in log2 units: the factor applied in the exponent is then 1.
+    const float exp_scale = BIAS ? 1.0f : scale_log2e;
+    const float lag = 8.0f / exp_scale;  // 2^8 in the units the maximum is kept in, see below
+    const float *zb_ctx = BIAS && p.z_bias ? p.z_bias + static_cast<size_t>(ctx) * S : nullptr;
+    const float *ab_row = BIAS && p.attn_bias && my_q < S
+                              ? p.attn_bias + (static_cast<size_t>(ctx) * S + my_q) * static_cast<size_t>(S) : nullptr;
     // NT = number of 32-key tiles of this stage this wavefront works on (1 or 2).
     auto compute = [&](auto nt_tag, int stage, int key0) {
         constexpr int NT = decltype(nt_tag)::value;
@@ -389,6 +396,27 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DPAD <= 64 
 #pragma unroll
         for (int t = 0; t < NT; ++t)
             sacc[t] = f32x16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        // Biases of this lane's query for the keys its registers hold (four consecutive keys per register group: one
+        // 128-bit load each; S is a multiple of 4 on this path, so a group is inside the sequence or past it as a
+        // whole), requested before the QKᵀ MFMAs so that they arrive behind them.
+        float4 bias4[BIAS ? NT : 1][4];
+        if constexpr (BIAS) {
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int key = key0 + t * 32 + g * 8 + lh * 4;
+                    float4 b = make_float4(0.f, 0.f, 0.f, 0.f);
+                    if (key < S) {
+                        if (ab_row) b = *reinterpret_cast<const float4 *>(ab_row + key);
+                        if (zb_ctx) {
+                            const float4 z = *reinterpret_cast<const float4 *>(zb_ctx + key);
+                            b.x += z.x; b.y += z.y; b.z += z.z; b.w += z.w;
+                        }
+                    }
+                    bias4[t][g] = b;
+                }
+        }
 #pragma unroll
         for (int c = 0; c < CHUNKS; ++c) {
             float4 kv[NT];
@@ -401,6 +429,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DPAD <= 64 
                 sacc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(kv[t].z, qf[c][2], sacc[t], 0, 0, 0);
                 sacc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(kv[t].w, qf[c][3], sacc[t], 0, 0, 0);
             }
+        }
+        if constexpr (BIAS) {
+            // logit = (dot·scale + z_bias) + attn_bias of pure.rs:11870-11880, in log2 units
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const float b[4] = {bias4[t][g].x, bias4[t][g].y, bias4[t][g].z, bias4[t][g].w};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) sacc[t][g * 4 + e] = fmaf(sacc[t][g * 4 + e], scale_log2e, b[e] * kLog2e);
+                }
         }
         // logits in log2 units; the masking code only runs where a tile crosses the sequence end or the diagonal
         const bool need_mask = (key0 + NT * 32 > S) || (CAUSAL && key0 + NT * 32 - 1 > wq0);
@@ -429,7 +468,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DPAD <= 64 
         if (__any(tile_max > run_max + lag)) {  // wavefront-uniform
             const float new_max = fmaxf(run_max, tile_max);
             const float new_safe = new_max == -INFINITY ? 0.0f : new_max;
-            const float alpha = __builtin_amdgcn_exp2f((run_max - new_safe) * scale_log2e);  // run_max = -inf -> 0
+            const float alpha = __builtin_amdgcn_exp2f((run_max - new_safe) * exp_scale);  // run_max = -inf -> 0
             run_sum *= alpha;
 #pragma unroll
             for (int t = 0; t < DT; ++t)
@@ -438,13 +477,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DPAD <= 64 
             run_max = new_max;
         }
         const float safe_max = run_max == -INFINITY ? 0.0f : run_max;
-        const float shift = -safe_max * scale_log2e;
+        const float shift = -safe_max * exp_scale;
         float tile_sum = 0.0f;
 #pragma unroll
         for (int t = 0; t < NT; ++t)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const float pr = __builtin_amdgcn_exp2f(fmaf(sacc[t][r], scale_log2e, shift));
+                const float pr = __builtin_amdgcn_exp2f(fmaf(sacc[t][r], exp_scale, shift));
                 sacc[t][r] = pr;
                 tile_sum += pr;
             }
@@ -506,11 +545,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DPAD <= 64 
     }  // pass
 }
 
-template <int DPAD, bool CAUSAL>
+template <int DPAD, bool CAUSAL, bool BIAS = false>
 hipError_t launch_fast(const AttnArgs &args, hipStream_t stream)
 {
     constexpr size_t lds_bytes = 2 * static_cast<size_t>(64) * ((DPAD + 4) + (DPAD + 8)) * sizeof(float);
-    auto kernel = attention_f32_fast_kernel<DPAD, CAUSAL>;
+    auto kernel = attention_f32_fast_kernel<DPAD, CAUSAL, BIAS>;
     hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
     if (rc != hipSuccess) return rc;
@@ -579,6 +618,12 @@ hipError_t launch_attention_f32(size_t contexts, size_t sequence, size_t head_di
         if (head_dim <= 32) return causal ? launch_fast<32, true>(args, stream) : launch_fast<32, false>(args, stream);
         if (head_dim <= 64) return causal ? launch_fast<64, true>(args, stream) : launch_fast<64, false>(args, stream);
         return causal ? launch_fast<128, true>(args, stream) : launch_fast<128, false>(args, stream);
+    }
+    // The same kernel with the additive biases folded in, where their rows can be read 128 bits at a time.
+    const bool bias_vec = sequence % 4 == 0 && aligned(z_bias) && aligned(attn_bias);
+    if (bias && bias_vec && vec && fits_buffer && head_dim <= 64) {
+        if (head_dim <= 32) return causal ? launch_fast<32, true, true>(args, stream) : launch_fast<32, false, true>(args, stream);
+        return causal ? launch_fast<64, true, true>(args, stream) : launch_fast<64, false, true>(args, stream);
     }
     if (head_dim <= 32) return launch_dpad<32, 64>(args, causal, bias, vec, stream);
     if (head_dim <= 64) return launch_dpad<64, 64>(args, causal, bias, vec, stream);

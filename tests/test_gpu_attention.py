@@ -64,6 +64,32 @@ def test_unusual_scales(hip, oracle, scale, causal):
     assert_close(ones, np.ones_like(ones), F32_REL, F32_ABS, "row sums")
 
 
+@pytest.mark.parametrize("contexts,seq,dim,causal,which,scale", [
+    (4, 256, 64, False, "both", 0.125), (2, 300, 32, True, "both", 0.2), (8, 132, 64, False, "attn", 0.125),
+    (3, 64, 48, True, "z", 0.15), (1, 1024, 64, False, "attn", 0.125), (2, 200, 64, True, "both", -0.3),
+    (2, 96, 20, False, "both", 0.0),
+])
+def test_biases_in_the_matrix_core_kernel(hip, oracle, contexts, seq, dim, causal, which, scale):
+    """Sequences that are a multiple of four with head_dim <= 64 keep the flash-style kernel when z_bias / attn_bias
+    are given (the shape of the reference's own caller, crates/st-nn/src/z_rba/attention.rs:586-595: one context,
+    an attn_bias kernel matrix): logit = (dot*scale + z_bias[key]) + attn_bias[query][key], pure.rs:11870-11880."""
+    rng = np.random.default_rng(contexts * 100 + seq + dim)
+    q, k, v = (rng.normal(size=contexts * seq * dim).astype(np.float32) for _ in range(3))
+    zb = rng.normal(size=contexts * seq).astype(np.float32) if which in ("z", "both") else None
+    ab = rng.normal(0, 2.0, size=contexts * seq * seq).astype(np.float32) if which in ("attn", "both") else None
+    got = run(hip, contexts, seq, dim, scale, q, k, v, zb, ab, causal)
+    want = oracle.attention_f32(contexts, seq, dim, scale, q, k, v, zb, ab, causal, threads=8)
+    assert_close(got, want, F32_REL, F32_ABS, f"biased attention {contexts}x{seq}x{dim} {which} causal={causal}")
+    ones = run(hip, contexts, seq, dim, scale, q, k, np.ones_like(v), zb, ab, causal)
+    assert_close(ones, np.ones_like(ones), F32_REL, F32_ABS, "row sums")
+    if which == "attn" and not causal:
+        # a -1e30 bias above the diagonal is the reference's way of masking: same values as the causal flag
+        mask = np.where(np.triu(np.ones((seq, seq), bool), 1), np.float32(-1e30), np.float32(0))
+        masked = run(hip, contexts, seq, dim, scale, q, k, v, None,
+                     np.ascontiguousarray(np.tile(mask.reshape(1, seq, seq), (contexts, 1, 1)), np.float32).ravel())
+        assert_close(masked, run(hip, contexts, seq, dim, scale, q, k, v, causal=True), F32_REL, F32_ABS, "mask == causal")
+
+
 def test_invariants(hip, oracle):
     rng = np.random.default_rng(5)
     contexts, seq, dim = 3, 150, 64
