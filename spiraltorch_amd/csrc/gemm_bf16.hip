@@ -240,77 +240,91 @@ typedef __attribute__((address_space(3))) void *lds_void_ptr;
 // s_waitcnt vmcnt(n) only (expcnt and lgkmcnt left at their maxima), gfx9 encoding.
 #define ST_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (7 << 4) | (15 << 8) | ((((n) >> 4) & 3) << 14))
 
-// Epilogue of the 256-row kernels: a wavefront's 32·TM × WTN accumulators leave through its own 32-row f32 strip in LDS
-// so that bias/residual loads and the stores are 128-bit and row-contiguous.  `row_first` / `col_base`: the
-// wavefront's first row and column of C.
+// Epilogue of the 256-row kernels.  The main loops form the product transposed (the MFMA's first operand is the Bᵀ
+// fragment), so accumulator register 4g + j of lane (li, lh) in tile (tm, tn) is
+//     C[row_first + 32·tm + li][col_base + 32·tn + 8g + 4·lh + j]:
+// four neighbouring columns of one row, i.e. one 128-bit (f32) or 64-bit (bf16) LDS write.  Every wavefront sends its
+// accumulators through a strip of LDS of its own and reads them back row-contiguous, so that the global stores (and
+// the residual loads) are 128-bit and cover whole 256- or 512-byte row segments.
+//   * bf16 is the only output and there is no residual: scale, bias and activation are applied in the accumulator
+//     layout, the values are rounded to bf16 first and all 32·TM rows go through LDS in one pass (row = WTN·2 bytes,
+//     unpadded; the 8-byte chunk q of row r sits at chunk q ^ swz(r), which spreads the 32 rows a write instruction
+//     touches, and the rows a read instruction touches, over all banks);
+//   * otherwise: f32 strips of 32 rows (row stride WTN + 4 floats), bias / residual / activation after the read-back.
+// `lds`: start of the workgroup's LDS (the operand stages are dead by now); `wave`: this wavefront's index.
 template <int WTN, int TM = 2>
-__device__ __forceinline__ void gemm_bf16_epilogue(const GemmBf16Args &p, const f32x16 (&acc)[TM][WTN / 32], float *strip,
-                                                   int row_first, int col_base, int lane)
+__device__ __forceinline__ void gemm_bf16_epilogue(const GemmBf16Args &p, const f32x16 (&acc)[TM][WTN / 32], unsigned char *lds,
+                                                   int wave, int row_first, int col_base, int lane)
 {
     constexpr int TN = WTN / 32;
-    constexpr int C_STRIDE = WTN + 4;
     const int li = lane & 31, lh = lane >> 5;
     const int M = p.M, N = p.N;
     const bool scaled = p.scale != 1.0f;
+    const bool bf16_only = p.C32 == nullptr && (reinterpret_cast<uintptr_t>(p.C16) & 15u) == 0;
+    if (bf16_only && p.residual == nullptr) {
+        constexpr int ROW_BYTES = WTN * 2;
+        constexpr int LPR8 = WTN / 8, ROWS8_PER_PASS = 64 / LPR8;  // read-back: 16 bytes (8 columns) per lane
+        unsigned char *strip = lds + wave * (TM * 32 * ROW_BYTES);
+        auto swz = [](int row) { return WTN == 128 ? (row & 31) : ((row >> 1) & 15); };
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                float4 bias4 = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (p.bias) bias4 = *reinterpret_cast<const float4 *>(p.bias + col_base + tn * 32 + g * 8 + lh * 4);
+                const int q = tn * 8 + g * 2 + lh;
+#pragma unroll
+                for (int tm = 0; tm < TM; ++tm) {
+                    float v0 = acc[tm][tn][4 * g + 0], v1 = acc[tm][tn][4 * g + 1];
+                    float v2 = acc[tm][tn][4 * g + 2], v3 = acc[tm][tn][4 * g + 3];
+                    if (scaled) { v0 *= p.scale; v1 *= p.scale; v2 *= p.scale; v3 *= p.scale; }
+                    v0 = apply_activation(v0 + bias4.x, p.activation);
+                    v1 = apply_activation(v1 + bias4.y, p.activation);
+                    v2 = apply_activation(v2 + bias4.z, p.activation);
+                    v3 = apply_activation(v3 + bias4.w, p.activation);
+                    uint2 packed;
+                    packed.x = pack_bf16x2_rne(v0, v1);
+                    packed.y = pack_bf16x2_rne(v2, v3);
+                    const int row = tm * 32 + li;
+                    *reinterpret_cast<uint2 *>(strip + row * ROW_BYTES + ((q ^ swz(row)) << 3)) = packed;
+                }
+            }
+        }
+        const int piece = lane & (LPR8 - 1);
+#pragma unroll
+        for (int j = 0; j < TM * 32 / ROWS8_PER_PASS; ++j) {
+            const int local_row = j * ROWS8_PER_PASS + lane / LPR8;
+            const int row = row_first + local_row;
+            const unsigned char *src = strip + local_row * ROW_BYTES;
+            const uint2 lo = *reinterpret_cast<const uint2 *>(src + (((2 * piece) ^ swz(local_row)) << 3));
+            const uint2 hi = *reinterpret_cast<const uint2 *>(src + (((2 * piece + 1) ^ swz(local_row)) << 3));
+            if (row < M) {
+                u32x4 packed;
+                packed.x = lo.x; packed.y = lo.y; packed.z = hi.x; packed.w = hi.y;
+                *reinterpret_cast<u32x4 *>(p.C16 + static_cast<size_t>(row) * N + col_base + piece * 8) = packed;
+            }
+        }
+        return;
+    }
+
+    constexpr int C_STRIDE = WTN + 4;
+    float *strip = reinterpret_cast<float *>(lds) + wave * (32 * C_STRIDE);
     constexpr int LPR = WTN / 4;        // lanes per strip row in the read-back phase (4 columns each)
     constexpr int ROWS_PER_PASS = 64 / LPR;
     const int col0 = col_base + (lane & (LPR - 1)) * 4;  // this lane's 4 columns in the read-back phase
     float4 bias4 = make_float4(0.f, 0.f, 0.f, 0.f);
     if (p.bias) bias4 = *reinterpret_cast<const float4 *>(p.bias + col0);
-    // bf16-only output (16-byte aligned): 8 columns per lane in the read-back phase
-    constexpr int LPR8 = WTN / 8, ROWS8_PER_PASS = 64 / LPR8;
-    const bool bf16_only = p.C32 == nullptr && (reinterpret_cast<uintptr_t>(p.C16) & 15u) == 0;
-    const int col8 = col_base + (lane & (LPR8 - 1)) * 8;
-    float bias8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    if (bf16_only && p.bias) {
-        *reinterpret_cast<float4 *>(bias8) = *reinterpret_cast<const float4 *>(p.bias + col8);
-        *reinterpret_cast<float4 *>(bias8 + 4) = *reinterpret_cast<const float4 *>(p.bias + col8 + 4);
-    }
 #pragma unroll
     for (int tm = 0; tm < TM; ++tm) {
 #pragma unroll
         for (int tn = 0; tn < TN; ++tn) {
             const f32x16 tile = acc[tm][tn];
 #pragma unroll
-            for (int r = 0; r < 16; ++r)
-                strip[((r >> 2) * 8 + lh * 4 + (r & 3)) * C_STRIDE + tn * 32 + li] = tile[r];
+            for (int g = 0; g < 4; ++g)
+                *reinterpret_cast<float4 *>(&strip[li * C_STRIDE + tn * 32 + g * 8 + lh * 4]) =
+                    make_float4(tile[4 * g], tile[4 * g + 1], tile[4 * g + 2], tile[4 * g + 3]);
         }
         const int row_base = row_first + tm * 32;
-        if (bf16_only) {
-            // bf16 is the only output: 8 columns (16 bytes) per lane, so half as many store instructions
-#pragma unroll
-            for (int j = 0; j < 32 / ROWS8_PER_PASS; ++j) {
-                const int local_row = j * ROWS8_PER_PASS + lane / LPR8;
-                const int row = row_base + local_row;
-                const float *src = &strip[local_row * C_STRIDE + (lane & (LPR8 - 1)) * 8];
-                float v[8];
-                *reinterpret_cast<float4 *>(v) = *reinterpret_cast<const float4 *>(src);
-                *reinterpret_cast<float4 *>(v + 4) = *reinterpret_cast<const float4 *>(src + 4);
-                if (row < M) {
-                    const size_t idx = static_cast<size_t>(row) * N + col8;
-                    float res[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-                    if (p.residual) {
-                        *reinterpret_cast<float4 *>(res) = *reinterpret_cast<const float4 *>(p.residual + idx);
-                        *reinterpret_cast<float4 *>(res + 4) = *reinterpret_cast<const float4 *>(p.residual + idx + 4);
-                    }
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        float value = v[e];
-                        if (scaled) value *= p.scale;
-                        value += bias8[e];
-                        value += res[e];
-                        v[e] = apply_activation(value, p.activation);
-                    }
-                    u32x4 packed;
-                    packed.x = pack_bf16x2_rne(v[0], v[1]);
-                    packed.y = pack_bf16x2_rne(v[2], v[3]);
-                    packed.z = pack_bf16x2_rne(v[4], v[5]);
-                    packed.w = pack_bf16x2_rne(v[6], v[7]);
-                    *reinterpret_cast<u32x4 *>(p.C16 + idx) = packed;
-                }
-            }
-            continue;
-        }
 #pragma unroll
         for (int j = 0; j < 32 / ROWS_PER_PASS; ++j) {
             const int local_row = j * ROWS_PER_PASS + lane / LPR;
@@ -448,7 +462,7 @@ __device__ __forceinline__ void gemm_bf16_packed_body(const GemmBf16Args &p)
         fb[buf][t] = *reinterpret_cast<const bf16x8 *>(lds_bytes + b_frag[kk ^ t] + b_stage * STAGE + t * 4096);
     };
     auto mfma = [&](int buf, int tm, int tn) {
-        acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[buf][tm], fb[buf][tn], acc[tm][tn], 0, 0, 0);
+        acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[buf][tn], fa[buf][tm], acc[tm][tn], 0, 0, 0);
     };
     // One sub-step: the TM×TN MFMAs on fragment buffer `buf`, each followed by a slot for memory instructions: the
     // first TM + TN slots issue the fragment reads of the sub-step after it (into the other buffer, in the order
@@ -531,8 +545,7 @@ __device__ __forceinline__ void gemm_bf16_packed_body(const GemmBf16Args &p)
     iteration(std::false_type{}, std::false_type{}, t);
 
     __syncthreads();
-    gemm_bf16_epilogue<WTN, TM>(p, acc, reinterpret_cast<float *>(lds_bytes) + wave * (32 * C_STRIDE), m0 + wm * WTM,
-                                n0 + wn * WTN, lane);
+    gemm_bf16_epilogue<WTN, TM>(p, acc, lds_bytes, wave, m0 + wm * WTM, n0 + wn * WTN, lane);
 }
 
 // -------------------------------------------------------------------------------------------------
@@ -668,7 +681,7 @@ __device__ __forceinline__ void gemm_bf16_rowmajor_body(const GemmBf16Args &p)
     auto substep = [&](int buf, bool reads, int a_stage_r, int b_stage_r, int kk_r, auto &&extra) {
 #pragma unroll
         for (int slot = 0; slot < SLOTS; ++slot) {
-            acc[slot / TN][slot % TN] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[buf][slot / TN], fb[buf][slot % TN],
+            acc[slot / TN][slot % TN] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[buf][slot % TN], fa[buf][slot / TN],
                                                                               acc[slot / TN][slot % TN], 0, 0, 0);
             ST_SCHED_FENCE();
             if (reads) {
@@ -752,8 +765,7 @@ __device__ __forceinline__ void gemm_bf16_rowmajor_body(const GemmBf16Args &p)
     iteration(std::false_type{}, std::false_type{}, t);
 
     __syncthreads();
-    gemm_bf16_epilogue<WTN>(p, acc, reinterpret_cast<float *>(lds_bytes) + wave * (32 * C_STRIDE), m0 + wm * 64, n0 + wn * WTN,
-                            lane);
+    gemm_bf16_epilogue<WTN>(p, acc, lds_bytes, wave, m0 + wm * 64, n0 + wn * WTN, lane);
 }
 
 __global__ __launch_bounds__(512) void gemm_bf16_256rm_kernel(GemmBf16Args p) { gemm_bf16_rowmajor_body<256>(p); }
