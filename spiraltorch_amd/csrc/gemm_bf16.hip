@@ -252,70 +252,107 @@ typedef __attribute__((address_space(3))) void *lds_void_ptr;
 //     touches, and the rows a read instruction touches, over all banks);
 //   * otherwise: f32 strips of 32 rows (row stride WTN + 4 floats), bias / residual / activation after the read-back.
 // `lds`: start of the workgroup's LDS (the operand stages are dead by now); `wave`: this wavefront's index.
-template <int WTN, int TM = 2>
-__device__ __forceinline__ void gemm_bf16_epilogue(const GemmBf16Args &p, const f32x16 (&acc)[TM][WTN / 32], unsigned char *lds,
-                                                   int wave, int row_first, int col_base, int lane)
+// Everything the epilogue decides per launch (activation, bias, residual) is a template parameter of the bodies below
+// and is dispatched once per wavefront: with those decisions made per element the epilogue compiled to several
+// hundred basic blocks whose loads, conversions and stores could not be scheduled across each other.
+template <int ACT>
+__device__ __forceinline__ float activate(float value)
+{
+    if constexpr (ACT == ST_HIP_ACT_RELU) return value > 0.0f ? value : 0.0f;
+    else if constexpr (ACT == ST_HIP_ACT_GELU) return gelu_tanh(value);
+    else return value;
+}
+
+template <int WTN, int TM, int ACT, bool FULL>
+__device__ __forceinline__ void gemm_bf16_epilogue_bf16(const GemmBf16Args &p, const f32x16 (&acc)[TM][WTN / 32],
+                                                        unsigned char *lds, int wave, int row_first, int col_base, int lane)
 {
     constexpr int TN = WTN / 32;
     const int li = lane & 31, lh = lane >> 5;
     const int M = p.M, N = p.N;
-    const bool scaled = p.scale != 1.0f;
-    const bool bf16_only = p.C32 == nullptr && (reinterpret_cast<uintptr_t>(p.C16) & 15u) == 0;
-    if (bf16_only && p.residual == nullptr) {
-        constexpr int ROW_BYTES = WTN * 2;
-        constexpr int LPR8 = WTN / 8, ROWS8_PER_PASS = 64 / LPR8;  // read-back: 16 bytes (8 columns) per lane
-        unsigned char *strip = lds + wave * (TM * 32 * ROW_BYTES);
-        auto swz = [](int row) { return WTN == 128 ? (row & 31) : ((row >> 1) & 15); };
+    const float scale = p.scale;
+    constexpr int ROW_BYTES = WTN * 2;
+    constexpr int LPR8 = WTN / 8, ROWS8_PER_PASS = 64 / LPR8;  // read-back: 16 bytes (8 columns) per lane
+    unsigned char *strip = lds + wave * (TM * 32 * ROW_BYTES);
+    auto swz = [](int row) { return WTN == 128 ? (row & 31) : ((row >> 1) & 15); };
+    // Without a bias the addend is -0.0f, which leaves every value (either zero included) as it is.
+    float4 bias4[TN][4];
 #pragma unroll
-        for (int tn = 0; tn < TN; ++tn) {
+    for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                float4 bias4 = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (p.bias) bias4 = *reinterpret_cast<const float4 *>(p.bias + col_base + tn * 32 + g * 8 + lh * 4);
-                const int q = tn * 8 + g * 2 + lh;
+        for (int g = 0; g < 4; ++g) bias4[tn][g] = make_float4(-0.0f, -0.0f, -0.0f, -0.0f);
+    if (p.bias) {
 #pragma unroll
-                for (int tm = 0; tm < TM; ++tm) {
-                    float v0 = acc[tm][tn][4 * g + 0], v1 = acc[tm][tn][4 * g + 1];
-                    float v2 = acc[tm][tn][4 * g + 2], v3 = acc[tm][tn][4 * g + 3];
-                    if (scaled) { v0 *= p.scale; v1 *= p.scale; v2 *= p.scale; v3 *= p.scale; }
-                    v0 = apply_activation(v0 + bias4.x, p.activation);
-                    v1 = apply_activation(v1 + bias4.y, p.activation);
-                    v2 = apply_activation(v2 + bias4.z, p.activation);
-                    v3 = apply_activation(v3 + bias4.w, p.activation);
-                    uint2 packed;
-                    packed.x = pack_bf16x2_rne(v0, v1);
-                    packed.y = pack_bf16x2_rne(v2, v3);
-                    const int row = tm * 32 + li;
-                    *reinterpret_cast<uint2 *>(strip + row * ROW_BYTES + ((q ^ swz(row)) << 3)) = packed;
-                }
-            }
-        }
-        const int piece = lane & (LPR8 - 1);
+        for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
-        for (int j = 0; j < TM * 32 / ROWS8_PER_PASS; ++j) {
-            const int local_row = j * ROWS8_PER_PASS + lane / LPR8;
-            const int row = row_first + local_row;
-            const unsigned char *src = strip + local_row * ROW_BYTES;
-            const uint2 lo = *reinterpret_cast<const uint2 *>(src + (((2 * piece) ^ swz(local_row)) << 3));
-            const uint2 hi = *reinterpret_cast<const uint2 *>(src + (((2 * piece + 1) ^ swz(local_row)) << 3));
-            if (row < M) {
-                u32x4 packed;
-                packed.x = lo.x; packed.y = lo.y; packed.z = hi.x; packed.w = hi.y;
-                *reinterpret_cast<u32x4 *>(p.C16 + static_cast<size_t>(row) * N + col_base + piece * 8) = packed;
-            }
-        }
-        return;
+            for (int g = 0; g < 4; ++g)
+                bias4[tn][g] = *reinterpret_cast<const float4 *>(p.bias + col_base + tn * 32 + g * 8 + lh * 4);
     }
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int q = tn * 8 + g * 2 + lh;
+#pragma unroll
+            for (int tm = 0; tm < TM; ++tm) {
+                float v0 = acc[tm][tn][4 * g + 0] * scale, v1 = acc[tm][tn][4 * g + 1] * scale;
+                float v2 = acc[tm][tn][4 * g + 2] * scale, v3 = acc[tm][tn][4 * g + 3] * scale;
+                v0 += bias4[tn][g].x; v1 += bias4[tn][g].y; v2 += bias4[tn][g].z; v3 += bias4[tn][g].w;
+                uint2 packed;
+                packed.x = pack_bf16x2_rne(activate<ACT>(v0), activate<ACT>(v1));
+                packed.y = pack_bf16x2_rne(activate<ACT>(v2), activate<ACT>(v3));
+                const int row = tm * 32 + li;
+                *reinterpret_cast<uint2 *>(strip + row * ROW_BYTES + ((q ^ swz(row)) << 3)) = packed;
+            }
+        }
+    }
+    const int piece = lane & (LPR8 - 1);
+#pragma unroll
+    for (int j = 0; j < TM * 32 / ROWS8_PER_PASS; ++j) {
+        const int local_row = j * ROWS8_PER_PASS + lane / LPR8;
+        const int row = row_first + local_row;
+        const unsigned char *src = strip + local_row * ROW_BYTES;
+        const uint2 lo = *reinterpret_cast<const uint2 *>(src + (((2 * piece) ^ swz(local_row)) << 3));
+        const uint2 hi = *reinterpret_cast<const uint2 *>(src + (((2 * piece + 1) ^ swz(local_row)) << 3));
+        if (FULL || row < M) {
+            u32x4 packed;
+            packed.x = lo.x; packed.y = lo.y; packed.z = hi.x; packed.w = hi.y;
+            *reinterpret_cast<u32x4 *>(p.C16 + static_cast<size_t>(row) * N + col_base + piece * 8) = packed;
+        }
+    }
+}
 
+template <int WTN, int TM, int ACT, bool RES, bool OUT32, bool OUT16, bool FULL>
+__device__ __forceinline__ void gemm_bf16_epilogue_f32(const GemmBf16Args &p, const f32x16 (&acc)[TM][WTN / 32],
+                                                       unsigned char *lds, int wave, int row_first, int col_base, int lane)
+{
+    constexpr int TN = WTN / 32;
+    const int li = lane & 31, lh = lane >> 5;
+    const int M = p.M, N = p.N;
+    const float scale = p.scale;
     constexpr int C_STRIDE = WTN + 4;
     float *strip = reinterpret_cast<float *>(lds) + wave * (32 * C_STRIDE);
     constexpr int LPR = WTN / 4;        // lanes per strip row in the read-back phase (4 columns each)
     constexpr int ROWS_PER_PASS = 64 / LPR;
+    constexpr int PASSES = 32 / ROWS_PER_PASS;
     const int col0 = col_base + (lane & (LPR - 1)) * 4;  // this lane's 4 columns in the read-back phase
-    float4 bias4 = make_float4(0.f, 0.f, 0.f, 0.f);
+    float4 bias4 = make_float4(-0.0f, -0.0f, -0.0f, -0.0f);  // x + -0.0f == x for every x
     if (p.bias) bias4 = *reinterpret_cast<const float4 *>(p.bias + col0);
+    float *const c32 = p.C32;
+    uint16_t *const c16 = p.C16;
 #pragma unroll
     for (int tm = 0; tm < TM; ++tm) {
+        const int row_base = row_first + tm * 32;
+        // The residual rows of this strip are requested before the accumulators go through LDS.
+        float4 rr[PASSES];
+        if constexpr (RES) {
+#pragma unroll
+            for (int j = 0; j < PASSES; ++j) {
+                const int row = row_base + j * ROWS_PER_PASS + lane / LPR;
+                rr[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (FULL || row < M) rr[j] = *reinterpret_cast<const float4 *>(p.residual + static_cast<size_t>(row) * N + col0);
+            }
+        }
 #pragma unroll
         for (int tn = 0; tn < TN; ++tn) {
             const f32x16 tile = acc[tm][tn];
@@ -324,34 +361,66 @@ __device__ __forceinline__ void gemm_bf16_epilogue(const GemmBf16Args &p, const 
                 *reinterpret_cast<float4 *>(&strip[li * C_STRIDE + tn * 32 + g * 8 + lh * 4]) =
                     make_float4(tile[4 * g], tile[4 * g + 1], tile[4 * g + 2], tile[4 * g + 3]);
         }
-        const int row_base = row_first + tm * 32;
 #pragma unroll
-        for (int j = 0; j < 32 / ROWS_PER_PASS; ++j) {
+        for (int j = 0; j < PASSES; ++j) {
             const int local_row = j * ROWS_PER_PASS + lane / LPR;
             const int row = row_base + local_row;
             float4 v = *reinterpret_cast<const float4 *>(&strip[local_row * C_STRIDE + (lane & (LPR - 1)) * 4]);
-            if (row < M) {
+            if (FULL || row < M) {
                 const size_t idx = static_cast<size_t>(row) * N + col0;
-                if (scaled) { v.x *= p.scale; v.y *= p.scale; v.z *= p.scale; v.w *= p.scale; }
+                v.x *= scale; v.y *= scale; v.z *= scale; v.w *= scale;
                 v.x += bias4.x; v.y += bias4.y; v.z += bias4.z; v.w += bias4.w;
-                if (p.residual) {
-                    const float4 rr = *reinterpret_cast<const float4 *>(p.residual + idx);
-                    v.x += rr.x; v.y += rr.y; v.z += rr.z; v.w += rr.w;
-                }
-                v.x = apply_activation(v.x, p.activation);
-                v.y = apply_activation(v.y, p.activation);
-                v.z = apply_activation(v.z, p.activation);
-                v.w = apply_activation(v.w, p.activation);
-                if (p.C32) *reinterpret_cast<float4 *>(p.C32 + idx) = v;
-                if (p.C16) {
+                if constexpr (RES) { v.x += rr[j].x; v.y += rr[j].y; v.z += rr[j].z; v.w += rr[j].w; }
+                v.x = activate<ACT>(v.x);
+                v.y = activate<ACT>(v.y);
+                v.z = activate<ACT>(v.z);
+                v.w = activate<ACT>(v.w);
+                if constexpr (OUT32) *reinterpret_cast<float4 *>(c32 + idx) = v;
+                if constexpr (OUT16) {
                     uint2 packed;
                     packed.x = pack_bf16x2_rne(v.x, v.y);
                     packed.y = pack_bf16x2_rne(v.z, v.w);
-                    *reinterpret_cast<uint2 *>(p.C16 + idx) = packed;
+                    *reinterpret_cast<uint2 *>(c16 + idx) = packed;
                 }
             }
         }
     }
+}
+
+template <int WTN, int TM, int ACT, bool FULL>
+__device__ __forceinline__ void gemm_bf16_epilogue_act(const GemmBf16Args &p, const f32x16 (&acc)[TM][WTN / 32],
+                                                       unsigned char *lds, int wave, int row_first, int col_base, int lane)
+{
+    const bool bf16_only = p.C32 == nullptr && (reinterpret_cast<uintptr_t>(p.C16) & 15u) == 0;
+    if (bf16_only && p.residual == nullptr) {
+        gemm_bf16_epilogue_bf16<WTN, TM, ACT, FULL>(p, acc, lds, wave, row_first, col_base, lane);
+    } else if (p.residual) {
+        if (p.C32 && p.C16) gemm_bf16_epilogue_f32<WTN, TM, ACT, true, true, true, FULL>(p, acc, lds, wave, row_first, col_base, lane);
+        else if (p.C32) gemm_bf16_epilogue_f32<WTN, TM, ACT, true, true, false, FULL>(p, acc, lds, wave, row_first, col_base, lane);
+        else gemm_bf16_epilogue_f32<WTN, TM, ACT, true, false, true, FULL>(p, acc, lds, wave, row_first, col_base, lane);
+    } else {
+        if (p.C32 && p.C16) gemm_bf16_epilogue_f32<WTN, TM, ACT, false, true, true, FULL>(p, acc, lds, wave, row_first, col_base, lane);
+        else if (p.C32) gemm_bf16_epilogue_f32<WTN, TM, ACT, false, true, false, FULL>(p, acc, lds, wave, row_first, col_base, lane);
+        else gemm_bf16_epilogue_f32<WTN, TM, ACT, false, false, true, FULL>(p, acc, lds, wave, row_first, col_base, lane);
+    }
+}
+
+template <int WTN, int TM, int ACT>
+__device__ __forceinline__ void gemm_bf16_epilogue_rows(const GemmBf16Args &p, const f32x16 (&acc)[TM][WTN / 32],
+                                                        unsigned char *lds, int wave, int row_first, int col_base, int lane)
+{
+    // Only the last row of tiles can hang over the end of a ragged M; every other wavefront runs without row checks.
+    if (row_first + TM * 32 <= p.M) gemm_bf16_epilogue_act<WTN, TM, ACT, true>(p, acc, lds, wave, row_first, col_base, lane);
+    else gemm_bf16_epilogue_act<WTN, TM, ACT, false>(p, acc, lds, wave, row_first, col_base, lane);
+}
+
+template <int WTN, int TM = 2>
+__device__ __forceinline__ void gemm_bf16_epilogue(const GemmBf16Args &p, const f32x16 (&acc)[TM][WTN / 32], unsigned char *lds,
+                                                   int wave, int row_first, int col_base, int lane)
+{
+    if (p.activation == ST_HIP_ACT_GELU) gemm_bf16_epilogue_rows<WTN, TM, ST_HIP_ACT_GELU>(p, acc, lds, wave, row_first, col_base, lane);
+    else if (p.activation == ST_HIP_ACT_RELU) gemm_bf16_epilogue_rows<WTN, TM, ST_HIP_ACT_RELU>(p, acc, lds, wave, row_first, col_base, lane);
+    else gemm_bf16_epilogue_rows<WTN, TM, ST_HIP_ACT_NONE>(p, acc, lds, wave, row_first, col_base, lane);
 }
 
 // -------------------------------------------------------------------------------------------------
