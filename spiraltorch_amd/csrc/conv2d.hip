@@ -233,22 +233,23 @@ __global__ __launch_bounds__(64 * WM * WN) void conv2d_f32_kernel(ConvArgs p)
     }
 
     float *out_image = p.out + static_cast<size_t>(image) * s.c_out * p.spatial;
+    with_epilogue_ops(p.activation, false, [&](auto &&act, auto) {
 #pragma unroll
-    for (int tn = 0; tn < TN; ++tn) {
-        const int col = px0 + wn * WTN + tn * 32 + li;
-        if (col >= p.spatial) continue;
+        for (int tn = 0; tn < TN; ++tn) {
+            const int col = px0 + wn * WTN + tn * 32 + li;
+            if (col >= p.spatial) continue;
 #pragma unroll
-        for (int tm = 0; tm < TM; ++tm) {
+            for (int tm = 0; tm < TM; ++tm) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int oc = oc0 + wm * WTM + tm * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
-                if (oc >= s.c_out) continue;
-                float value = acc[tm][tn][r];
-                if (p.bias) value += p.bias[oc];
-                out_image[static_cast<size_t>(oc) * p.spatial + col] = apply_activation(value, p.activation);
+                for (int r = 0; r < 16; ++r) {
+                    const int oc = oc0 + wm * WTM + tm * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
+                    if (oc >= s.c_out) continue;
+                    const float value = acc[tm][tn][r] + (p.bias ? p.bias[oc] : -0.0f);  // x + -0.0f == x
+                    out_image[static_cast<size_t>(oc) * p.spatial + col] = act(value);
+                }
             }
         }
-    }
+    });
 }
 
 // -------------------------------------------------------------------------------------------------
@@ -464,22 +465,23 @@ __device__ __forceinline__ void conv2d_f32_ring_body(const ConvArgs &p)
     if (t + 1 < steps) step(std::integral_constant<int, 1>{}, t + 1);
 
     float *out_image = p.out + static_cast<size_t>(image) * s.c_out * p.spatial;
+    with_epilogue_ops(p.activation, false, [&](auto &&act, auto) {
 #pragma unroll
-    for (int tn = 0; tn < TN; ++tn) {
-        const int col = px0 + wn * WTN + tn * 32 + li;
-        if (col >= p.spatial) continue;
+        for (int tn = 0; tn < TN; ++tn) {
+            const int col = px0 + wn * WTN + tn * 32 + li;
+            if (col >= p.spatial) continue;
 #pragma unroll
-        for (int tm = 0; tm < TM; ++tm) {
+            for (int tm = 0; tm < TM; ++tm) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int oc = oc0 + wm * WTM + tm * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
-                if (oc >= s.c_out) continue;
-                float value = acc[tm][tn][r];
-                if (p.bias) value += p.bias[oc];
-                out_image[static_cast<size_t>(oc) * p.spatial + col] = apply_activation(value, p.activation);
+                for (int r = 0; r < 16; ++r) {
+                    const int oc = oc0 + wm * WTM + tm * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
+                    if (oc >= s.c_out) continue;
+                    const float value = acc[tm][tn][r] + (p.bias ? p.bias[oc] : -0.0f);  // x + -0.0f == x
+                    out_image[static_cast<size_t>(oc) * p.spatial + col] = act(value);
+                }
             }
         }
-    }
+    });
 }
 
 // (A kernel template whose body uses the LDS-load builtins loses its host-side launch stub with this
@@ -701,37 +703,41 @@ __device__ __forceinline__ void conv2d_f32_strip_body(const StripArgs &p)
         if (pair < pairs) pair_body(a0, b0, a2, b2, pair);
         if (pair + 1 < pairs) pair_body(a1, b1, a0, b0, pair + 1);
 
-        if constexpr (WIDE) {
-            const int px4 = (first + blk) * 32 + (lane & 7) * 4;
+        // The activation is wavefront-uniform: GELU takes a copy of the store code of its own, ReLU and none share a
+        // branch-free one (decided per element, the stores of a block were cut into a dozen basic blocks).
+        auto store_block = [&](auto &&act) {
+            if constexpr (WIDE) {
+                const int px4 = (first + blk) * 32 + (lane & 7) * 4;
 #pragma unroll
-            for (int h = 0; h < 2; ++h) {
+                for (int h = 0; h < 2; ++h) {
 #pragma unroll
-                for (int rr = 0; rr < 8; ++rr) {
-                    const int r = h * 8 + rr;
-                    stage[(((r >> 2) & 1) * 8 + lh * 4 + (r & 3)) * kStripStagePitch + li] = acc[r];
-                }
+                    for (int rr = 0; rr < 8; ++rr) {
+                        const int r = h * 8 + rr;
+                        stage[(((r >> 2) & 1) * 8 + lh * 4 + (r & 3)) * kStripStagePitch + li] = acc[r];
+                    }
 #pragma unroll
-                for (int q = 0; q < 2; ++q) {
-                    const int row = q * 8 + (lane >> 3);
-                    const f32x4 v = *reinterpret_cast<const f32x4 *>(stage + row * kStripStagePitch + (lane & 7) * 4);
-                    const int oc = oc0 + h * 16 + row;
-                    if (oc < s.c_out && px4 < p.spatial) {
+                    for (int q = 0; q < 2; ++q) {
+                        const int row = q * 8 + (lane >> 3);
+                        const f32x4 v = *reinterpret_cast<const f32x4 *>(stage + row * kStripStagePitch + (lane & 7) * 4);
+                        const int oc = oc0 + h * 16 + row;
                         f32x4 o;
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) o[e] = apply_activation(v[e] + bias_wide[h][q], p.activation);
-                        *reinterpret_cast<f32x4 *>(out_image + static_cast<size_t>(oc) * p.spatial + px4) = o;
+                        for (int e = 0; e < 4; ++e) o[e] = act(v[e] + bias_wide[h][q]);
+                        if (oc < s.c_out && px4 < p.spatial)
+                            *reinterpret_cast<f32x4 *>(out_image + static_cast<size_t>(oc) * p.spatial + px4) = o;
                     }
                 }
-            }
-        } else if (valid) {
+            } else if (valid) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int oc = oc0 + (r >> 2) * 8 + lh * 4 + (r & 3);
-                if (oc < s.c_out)  // (the bias is re-read per block: sixteen registers are worth more in the main loop)
-                    out_image[static_cast<size_t>(oc) * p.spatial + px] =
-                        apply_activation(acc[r] + (p.bias ? p.bias[oc] : 0.0f), p.activation);
+                for (int r = 0; r < 16; ++r) {
+                    const int oc = oc0 + (r >> 2) * 8 + lh * 4 + (r & 3);
+                    if (oc < s.c_out)  // (the bias is re-read per block: sixteen registers are worth more in the main loop)
+                        out_image[static_cast<size_t>(oc) * p.spatial + px] = act(acc[r] + (p.bias ? p.bias[oc] : 0.0f));
+                }
             }
-        }
+        };
+        if (p.activation == ST_HIP_ACT_GELU) store_block([](float v) { return gelu_tanh(v); });
+        else store_block([relu = p.activation == ST_HIP_ACT_RELU](float v) { return relu_or_identity(v, relu); });
     }
 }
 

@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
+#include <type_traits>
 
 #include "st_hip.h"
 
@@ -33,6 +34,30 @@ __device__ __forceinline__ float apply_activation(float value, int activation)
     if (activation == ST_HIP_ACT_RELU) return value > 0.0f ? value : 0.0f;
     if (activation == ST_HIP_ACT_GELU) return gelu_tanh(value);
     return value;
+}
+
+// ReLU when `relu` (a wavefront-uniform flag), else the value itself, without a branch: compare, select, select.
+__device__ __forceinline__ float relu_or_identity(float value, bool relu)
+{
+    const float rectified = value > 0.0f ? value : 0.0f;
+    return relu ? rectified : value;
+}
+
+// Runs `body(act, has_residual)` with the activation as a callable and the presence of a residual as a compile-time
+// constant, chosen once from the (wavefront-uniform) launch arguments: an epilogue that decides them per element
+// compiles to a chain of scalar branches around every store.
+template <class Body>
+__device__ __forceinline__ void with_epilogue_ops(int activation, bool has_residual, Body &&body)
+{
+    auto gelu = [](float v) { return gelu_tanh(v); };
+    auto cheap = [relu = activation == ST_HIP_ACT_RELU](float v) { return relu_or_identity(v, relu); };
+    if (activation == ST_HIP_ACT_GELU) {
+        if (has_residual) body(gelu, std::true_type{});
+        else body(gelu, std::false_type{});
+    } else {
+        if (has_residual) body(cheap, std::true_type{});
+        else body(cheap, std::false_type{});
+    }
 }
 
 // Round-to-nearest-even f32 -> bf16 bit pattern through the hardware conversion (v_cvt_pk_bf16_f32); NaN stays
