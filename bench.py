@@ -161,24 +161,41 @@ def wl_gemm_f32(hip, inputs, timer, warmup, steps, m, n, k, name):
 
 def wl_gemm_bf16(hip, inputs, timer, warmup, steps, m, n, k, name, bound, packed=False):
     """bf16 operands, f32 accumulation and output.  `packed`: B handed over as its (n, k) transpose (PackedB's
-    layout), packed once outside the timed region as a weight would be."""
+    layout), packed once outside the timed region as a weight would be.
+
+    The HBM-bound (skinny) shapes cycle through ten copies of B, 320 MiB in all: a single 32 MiB B stays in the
+    256 MiB memory-side cache from one launch to the next, and a loop over it measures that cache, not HBM (a decode
+    loop reads a different weight matrix with every GEMM).  The cache-resident time is reported beside it."""
     a = inputs.to_bf16(inputs.normal(inputs.seed_for(4, 0 if m == n else 2), m * k, 0.0, 0.02))
     b = inputs.to_bf16(inputs.normal(inputs.seed_for(4, 1), k * n, 0.0, 0.02))
-    d_a, d_b = hip.DeviceBuffer.from_array(a), hip.DeviceBuffer.from_array(b)
+    d_a = hip.DeviceBuffer.from_array(a)
     d_c = hip.DeviceBuffer(m * n * 4)
+    copies = 10 if bound == "hbm" else 1
     if packed:
-        d_packed = hip.DeviceBuffer(k * n * 2)
-        hip.pack_rhs_bf16_dev(k, n, d_b, d_packed)
+        d_b = hip.DeviceBuffer.from_array(b)
+        rhs = []
+        for _ in range(copies):
+            rhs.append(hip.DeviceBuffer(k * n * 2))
+            hip.pack_rhs_bf16_dev(k, n, d_b, rhs[-1])
         hip.device_synchronize()
-
-        def step(stream):
-            hip.gemm_bf16_prepacked_bias_act_dev(m, n, k, 0, d_a, d_packed, None, None, d_c, None, stream)
     else:
-        def step(stream):
-            hip.gemm_bf16_f32acc_dev(m, n, k, d_a, d_b, d_c, stream)
+        rhs = [hip.DeviceBuffer.from_array(b) for _ in range(copies)]
+    turn = [0]
+
+    def step(stream, rotate=True):
+        d_rhs = rhs[turn[0] % copies if rotate else 0]
+        turn[0] += 1
+        if packed:
+            hip.gemm_bf16_prepacked_bias_act_dev(m, n, k, 0, d_a, d_rhs, None, None, d_c, None, stream)
+        else:
+            hip.gemm_bf16_f32acc_dev(m, n, k, d_a, d_rhs, d_c, stream)
 
     wall, ev = timer.run(step, warmup, steps)
-    return entry(name, "bf16", 2 * m * n * k, 2 * (m * k + k * n) + 4 * m * n, bound, wall, ev)
+    extra = None
+    if copies > 1:
+        _, resident = timer.run(lambda stream: step(stream, rotate=False), warmup, steps)
+        extra = {"rhs_copies_cycled": copies, "kernel_ms_per_step_rhs_cache_resident": round(resident, 5)}
+    return entry(name, "bf16", 2 * m * n * k, 2 * (m * k + k * n) + 4 * m * n, bound, wall, ev, extra)
 
 
 def wl_attention(hip, inputs, timer, warmup, steps, causal):
@@ -354,6 +371,7 @@ def cpu_baselines(inputs):
     out["gemm_bf16_f32acc_4096x4096x4096_prepacked_rhs"] = square
     sec = timed(lambda: oracle.gemm_bf16_f32acc(16, 4096, 4096, a16[:16 * 4096], b16, threads=cores), repeat=5)
     out["gemm_bf16_f32acc_16x4096x4096"] = _cpu(2 * 16 * 4096 * 4096, sec, cores, f"full shape, best of 5, {cores} threads")
+    out["gemm_bf16_f32acc_16x4096x4096_prepacked_rhs"] = out["gemm_bf16_f32acc_16x4096x4096"]
     # config 5: one layer (+ embedding, final norm, head) on one of 16 sequences, single thread, scaled
     vocab, d, heads, ff, seq = 256, 512, 8, 2048, 1024
     weights = inputs.normal(inputs.seed_for(5, 0), oracle.decoder_weight_count(vocab, d, heads, 1, ff), 0.0, 0.02)
@@ -407,6 +425,8 @@ def main():
                                                           "gemm_bf16_f32acc_4096x4096x4096_prepacked_rhs", "mfma", True)),
         ("gemm_bf16_skinny", lambda: wl_gemm_bf16(hip, inputs, timer, warm, steps, 16, 4096, 4096,
                                                   "gemm_bf16_f32acc_16x4096x4096", "hbm")),
+        ("gemm_bf16_skinny_prepacked", lambda: wl_gemm_bf16(hip, inputs, timer, warm, steps, 16, 4096, 4096,
+                                                            "gemm_bf16_f32acc_16x4096x4096_prepacked_rhs", "hbm", True)),
         ("attention_noncausal", lambda: wl_attention(hip, inputs, timer, long_warm, long_steps, False)),
         ("attention_causal", lambda: wl_attention(hip, inputs, timer, long_warm, long_steps, True)),
         ("attention_bias", lambda: [wl_attention_bias(hip, inputs, timer, warm, steps, 1, 2048),

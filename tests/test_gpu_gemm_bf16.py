@@ -194,6 +194,41 @@ def test_prepacked_rhs(hip, oracle, m, n, k):
     assert (got16.to_array(np.uint16, m * n) == want16.to_array(np.uint16, m * n)).all()
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 1024, 128), (16, 4096, 4096), (17, 1024, 384), (32, 2048, 1152), (5, 1040, 2176),
+                                   (9, 1024, 896), (31, 4096, 1024),
+                                   # not taken by that kernel (m > 32, k not a multiple of 128): unpacked first
+                                   (64, 1024, 4096), (48, 4096, 512), (5, 1040, 2080)])
+def test_skinny_prepacked_single_launch(hip, oracle, m, n, k):
+    """Decode-like shapes on a prepacked B (m <= 32, at least 64 strips of 16 columns, k a multiple of 128) take the
+    single-launch kernel whose eight wavefronts each stream a k-range and add their tiles in a fixed order."""
+    from spiraltorch_amd import inputs
+    rng = np.random.default_rng(m * 13 + n * 3 + k)
+    a, b = bf16_pair(rng, m, n, k, std=0.5)
+    bias = rng.normal(size=n).astype(np.float32)
+    res = rng.normal(size=m * n).astype(np.float32)
+    d = {name: hip.DeviceBuffer.from_array(v) for name, v in (("a", a), ("bias", bias), ("res", res))}
+    d_packed = hip.DeviceBuffer.from_array(np.ascontiguousarray(b.reshape(k, n).T))
+    out = hip.DeviceBuffer(m * n * 4)
+    hip.gemm_bf16_prepacked_bias_act_dev(m, n, k, 0, d["a"], d_packed, None, None, out, None)
+    hip.device_synchronize()
+    base = oracle.gemm_bf16_f32acc(m, n, k, a, b, threads=8)
+    first = out.to_array(np.float32, m * n)
+    check(first, base, f"skinny prepacked {m}x{n}x{k}")
+    hip.gemm_bf16_prepacked_bias_act_dev(m, n, k, 0, d["a"], d_packed, None, None, out, None)
+    hip.device_synchronize()
+    assert (out.to_array(np.float32, m * n) == first).all(), "the k-range sums must be added in a fixed order"
+    d16 = hip.DeviceBuffer(m * n * 2)
+    pre = (base.astype(np.float64).reshape(m, n) + bias).ravel() + res
+    for act in (0, 1, 2):
+        hip.gemm_bf16_prepacked_bias_act_dev(m, n, k, act, d["a"], d_packed, d["bias"], d["res"], out, d16)
+        hip.device_synchronize()
+        want = pre if act == 0 else np.maximum(pre, 0) if act == 1 else \
+            0.5 * pre * (1.0 + np.tanh(0.7978846 * (pre + 0.044715 * pre ** 3)))
+        got32 = out.to_array(np.float32, m * n)
+        assert_close(got32, want, 1e-4, 2e-5 * max(1.0, float(np.abs(base).max())), f"skinny prepacked epilogue act={act}")
+        assert (d16.to_array(np.uint16, m * n) == inputs.to_bf16(got32)).all()
+
+
 def test_config4_4096_cubed_prepacked(hip, oracle):
     """BASELINE config 4 with B prepacked: 24 sampled rows against the oracle, the rest of the matrix bit for bit
     against the k×n kernel (checked itself above), and exact power-of-two linearity."""
