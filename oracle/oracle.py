@@ -54,6 +54,7 @@ def load() -> ctypes.CDLL:
     lib = ctypes.CDLL(LIBRARY_PATH)
     S, P, F, I = c_size_t, c_void_p, c_float, c_int
     lib.st_oracle_gemm_f32.argtypes = [S, S, S, F, I, P, P, P, I]
+    lib.st_oracle_gemm_f32_packed_naive.argtypes = [S, S, S, P, P, P]
     lib.st_oracle_gemm_bias_act_f32.argtypes = [S, S, S, I, P, P, P, P, P, I]
     lib.st_oracle_gemm_bf16_f32acc.argtypes = [S, S, S, P, P, P, I]
     lib.st_oracle_conv2d_output_hw.argtypes = [S] * 10 + [POINTER(S), POINTER(S)]
@@ -99,6 +100,15 @@ def gemm_f32(m, n, k, lhs, rhs, scale=1.0, lhs_transposed=False, threads=1) -> n
     assert lhs.size == m * k and rhs.size == k * n
     out = np.zeros(m * n, dtype=np.float32)
     _check(load().st_oracle_gemm_f32(m, n, k, scale, int(lhs_transposed), _p(lhs), _p(rhs), _p(out), threads))
+    return out
+
+
+def gemm_f32_packed_naive(m, n, k, lhs, packed_rhs) -> np.ndarray:
+    """`packed_rhs` is the (n, k) transpose of B (PackedB's layout)."""
+    lhs, packed_rhs = _f32(lhs), _f32(packed_rhs)
+    assert lhs.size == m * k and packed_rhs.size == k * n
+    out = np.zeros(m * n, dtype=np.float32)
+    _check(load().st_oracle_gemm_f32_packed_naive(m, n, k, _p(lhs), _p(packed_rhs), _p(out)))
     return out
 
 

@@ -9,6 +9,8 @@
  *
  * Pinning status (checked in tests/test_oracle_*.py):
  *   gemm / scaled / lhs-transposed / bias+act   — reference known-answer vectors + float64 closed form
+ *   packed naive gemm (dot_unrolled tail)       — bit-equal to the sequential gemm on the 4-column blocks, an
+ *                                                 order-revealing vector (2^24 and ones) and float64 on the tail
  *   conv2d                                      — reference layout vector + float64 direct convolution
  *   attention                                   — reference vectors vs float64 two-pass softmax, invariants
  *   layer-norm, gelu, embedding, bf16 rounding  — textbook closed forms
@@ -71,6 +73,62 @@ int st_oracle_gemm_f32(size_t m, size_t n, size_t k, float scale, int lhs_transp
             float *dst = out + (size_t)row * n;
             for (size_t col = 0; col < n; ++col) dst[col] = dst[col] * scale;
         }
+    }
+    return ST_ORACLE_OK;
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * The naive CPU path on a prepacked rhs (PackedB, n×k with k contiguous): crates/st-tensor/src/pure.rs:11688-11758
+ * (matmul_naive_packed_row).  Columns are taken four at a time (PACKED_MATMUL_COL_BLOCK, :11567), each with one
+ * accumulator that adds its k products strictly in order — the same sequence as st_oracle_gemm_f32 —; the
+ * cols % 4 columns left over go through dot_unrolled (:11664-11686): four partial sums over k ≡ 0,1,2,3 (mod 4),
+ * added as ((acc0 + acc1) + acc2) + acc3, then the k % 4 tail products in order.
+ * ---------------------------------------------------------------------------------------------- */
+static float dot_unrolled(const float *lhs, const float *rhs, size_t len)
+{
+    float acc0 = 0.0f, acc1 = 0.0f, acc2 = 0.0f, acc3 = 0.0f;
+    const size_t chunks = len / 4;
+    for (size_t i = 0; i < chunks; ++i) {
+        const size_t base = i * 4;
+        const float p0 = lhs[base] * rhs[base];
+        const float p1 = lhs[base + 1] * rhs[base + 1];
+        const float p2 = lhs[base + 2] * rhs[base + 2];
+        const float p3 = lhs[base + 3] * rhs[base + 3];
+        acc0 = acc0 + p0;
+        acc1 = acc1 + p1;
+        acc2 = acc2 + p2;
+        acc3 = acc3 + p3;
+    }
+    float sum = acc0 + acc1;
+    sum = sum + acc2;
+    sum = sum + acc3;
+    for (size_t i = chunks * 4; i < len; ++i) {
+        const float prod = lhs[i] * rhs[i];
+        sum = sum + prod;
+    }
+    return sum;
+}
+
+int st_oracle_gemm_f32_packed_naive(size_t m, size_t n, size_t k, const float *lhs, const float *packed_rhs,
+                                    float *out)
+{
+    if (mul_overflows(m, k) || mul_overflows(k, n) || mul_overflows(m, n)) return ST_ORACLE_BAD_ARGUMENT;
+    for (size_t row = 0; row < m; ++row) {
+        const float *lhs_row = lhs + row * k;
+        float *dst = out + row * n;
+        size_t col = 0;
+        for (; col + 4 <= n; col += 4) {
+            for (size_t j = 0; j < 4; ++j) {
+                const float *column = packed_rhs + (col + j) * k;
+                float acc = 0.0f;
+                for (size_t p = 0; p < k; ++p) {
+                    const float prod = lhs_row[p] * column[p];
+                    acc = acc + prod;
+                }
+                dst[col + j] = acc;
+            }
+        }
+        for (; col < n; ++col) dst[col] = dot_unrolled(lhs_row, packed_rhs + col * k, k);
     }
     return ST_ORACLE_OK;
 }

@@ -43,6 +43,11 @@ enum {
 int st_oracle_gemm_f32(size_t m, size_t n, size_t k, float scale, int lhs_transposed,
                        const float *lhs, const float *rhs, float *out, int threads);
 
+/* The naive path on a prepacked rhs (n×k): sequential sums for the columns taken four at a time, the four-way
+ * unrolled dot product for the cols % 4 columns left over (crates/st-tensor/src/pure.rs:11664-11758). */
+int st_oracle_gemm_f32_packed_naive(size_t m, size_t n, size_t k, const float *lhs, const float *packed_rhs,
+                                    float *out);
+
 /* out = act((lhs·rhs + bias[col]) + residual), residual may be NULL; activation NONE/RELU/GELU. */
 int st_oracle_gemm_bias_act_f32(size_t m, size_t n, size_t k, int activation, const float *lhs,
                                 const float *rhs, const float *bias, const float *residual,

@@ -191,6 +191,8 @@ def test_prepacked_rhs(hip, oracle, m, n, k):
     plain = oracle.gemm_f32(m, n, k, a, b, threads=8)
     hip.gemm_prepacked_bias_activation_f32(m, n, k, 0, a, packed, None, None, out)
     assert_close(out, plain, F32_REL, F32_ABS, "prepacked")
+    if m * n * k <= 1 << 22:  # the reference's naive packed order (four partial sums on the n % 4 tail columns)
+        assert_close(out, oracle.gemm_f32_packed_naive(m, n, k, a, packed), F32_REL, F32_ABS, "prepacked vs packed-naive order")
     hip.gemm_prepacked_bias_activation_f32(m, n, k, 0, a, packed, bias, None, out)
     assert_close(out, (plain.astype(np.float64).reshape(m, n) + bias).ravel(), F32_REL, F32_ABS, "prepacked + bias")
     hip.gemm_prepacked_bias_activation_f32(m, n, k, hip.GemmActivation.Gelu, a, packed, bias, res, out)

@@ -113,3 +113,46 @@ def test_bf16_rounding_and_gemm(oracle):
     b = inputs.to_bf16(rng.normal(0, 0.02, (40, 11)).astype(np.float32))
     want = inputs.from_bf16(a).reshape(9, 40).astype(np.float64) @ inputs.from_bf16(b).reshape(40, 11).astype(np.float64)
     assert_close(oracle.gemm_bf16_f32acc(9, 11, 40, a, b), want, 1e-5, 1e-7, "bf16 gemm")
+
+
+def test_packed_naive_blocks_are_the_sequential_sum(oracle):
+    """matmul_naive_packed_row (pure.rs:11688-11758) adds the k products of a 4-column block strictly in order: on
+    n % 4 == 0 it must agree bit for bit with the sequential GEMM, whatever the data."""
+    rng = np.random.default_rng(5)
+    m, n, k = 7, 12, 203
+    a = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+    b = rng.uniform(-1, 1, (k, n)).astype(np.float32)
+    packed = np.ascontiguousarray(b.T)
+    assert (oracle.gemm_f32_packed_naive(m, n, k, a, packed) == oracle.gemm_f32(m, n, k, a, b)).all()
+
+
+def test_packed_naive_tail_columns_use_four_partial_sums(oracle):
+    """dot_unrolled (pure.rs:11664-11686): with lhs = [2^24, 1, 1, 1, 1, 1, 1, 1, 1, 1] and a column of ones the
+    sequential f32 sum stays at 2^24 (every +1 is lost), while four partial sums over k mod 4 give
+    acc0 = 2^24 (+1 lost twice), acc1 = 3, acc2 = 2, acc3 = 2, then ((acc0 + acc1) + acc2) + acc3 = 2^24 + 7 -> the
+    f32 neighbours are 2 apart: 2^24+3 -> 2^24+4 (ties to even), +2 -> 2^24+6, +2 -> 2^24+8."""
+    k = 10
+    lhs = np.ones(k, np.float32)
+    lhs[0] = 2.0 ** 24
+    for n in (1, 2, 3):  # every column is a tail column
+        packed = np.ones((n, k), np.float32)
+        out = oracle.gemm_f32_packed_naive(1, n, k, lhs, packed)
+        assert out.tolist() == [2.0 ** 24 + 8] * n
+        assert oracle.gemm_f32(1, n, k, lhs, np.ones((k, n), np.float32)).tolist() == [2.0 ** 24] * n
+    # n = 5: the first four columns are a block (sequential), the fifth is a tail column
+    out = oracle.gemm_f32_packed_naive(1, 5, k, lhs, np.ones((5, k), np.float32))
+    assert out.tolist() == [2.0 ** 24] * 4 + [2.0 ** 24 + 8]
+
+
+@pytest.mark.parametrize("m,n,k", [(3, 5, 7), (4, 7, 64), (2, 9, 131), (1, 3, 3)])
+def test_packed_naive_against_float64(oracle, m, n, k):
+    rng = np.random.default_rng(m + 10 * n + 100 * k)
+    a = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+    b = rng.uniform(-1, 1, (k, n)).astype(np.float32)
+    want = a.astype(np.float64) @ b.astype(np.float64)
+    got = oracle.gemm_f32_packed_naive(m, n, k, a, np.ascontiguousarray(b.T))
+    assert_close(got, want, 1e-5, 1e-5, f"packed naive {m}x{n}x{k}")
+    # and a transposed packing (k x n handed over as if it were n x k) must fail that check
+    if n != k:
+        wrong = oracle.gemm_f32_packed_naive(m, n, k, a, b)
+        assert np.abs(wrong - want.ravel()).max() > 1e-3
