@@ -37,6 +37,37 @@ def test_python_binding_covers_every_declared_symbol():
     assert sorted(_lib.SIGNATURES) == declared_symbols()
 
 
+def test_rust_binding_matches_the_header():
+    """The Rust crate's extern block (spiraltorch_amd/rust/st-backend-hip/src/ffi.rs) is generated from the header;
+    it must be the generator's current output, name every declared symbol once, and every ffi:: call in the crate's
+    hand-written sources must name a declared symbol with the declared number of arguments."""
+    import subprocess
+    import sys
+    rust = os.path.join(ROOT, "spiraltorch_amd", "rust")
+    subprocess.run([sys.executable, os.path.join(rust, "gen_ffi.py"), "--check"], check=True)
+    ffi = open(os.path.join(rust, "st-backend-hip", "src", "ffi.rs")).read()
+    bound = re.findall(r"pub fn (st_hip_\w+)\(([^)]*)\)", ffi)
+    assert sorted(name for name, _ in bound) == declared_symbols()
+    arity = {name: (0 if not args.strip() else args.count(":")) for name, args in bound}
+    for source in ("lib.rs", "device.rs"):
+        text = open(os.path.join(rust, "st-backend-hip", "src", source)).read()
+        for match in re.finditer(r"ffi::(st_hip_\w+)\(", text):
+            name = match.group(1)
+            assert name in arity, f"{source} calls {name}, which the header does not declare"
+            depth, i, commas, empty = 1, match.end(), 0, True
+            while depth:
+                ch = text[i]
+                depth += ch in "([{"
+                depth -= ch in ")]}"
+                if depth == 1 and ch == ",":
+                    commas += 1
+                if depth >= 1 and not ch.isspace() and not (depth == 0):
+                    empty = empty and ch == ")"
+                i += 1
+            passed = 0 if empty else commas + 1
+            assert passed == arity[name], f"{source}: {name} called with {passed} arguments, declared with {arity[name]}"
+
+
 def test_product_never_touches_the_oracle():
     offenders = []
     for base, _, files in os.walk(os.path.join(ROOT, "spiraltorch_amd")):
