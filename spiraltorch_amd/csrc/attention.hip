@@ -38,6 +38,12 @@ struct AttnArgs {
     int q_tiles;
     int swizzle;
     float scale;
+    // Keys split over workgroups (non-causal fast kernel only): workgroup (…, split) covers keys_per_split keys
+    // (a multiple of 64) and leaves its un-normalised output rows in part_o[split][context·S + query][D] and their
+    // (reference maximum, sum) in part_ml[split][context·S + query][2]; attention_merge_splits_kernel combines them.
+    int key_splits, keys_per_split;
+    float *part_o;
+    float *part_ml;
 };
 
 constexpr int kBQ = 128;
@@ -299,14 +305,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DPAD <= 64 
     // from memory three times over).
     const int per_ctx = CAUSAL ? (p.q_tiles + 1) / 2 : p.q_tiles;  // workgroups per context
     int ctx, unit;
+    int split = 0;
     if (p.swizzle) {
         const int per_xcd = p.contexts >> 3;
         const int xcd = blockIdx.x & 7, i = blockIdx.x >> 3;
         ctx = xcd * per_xcd + i / per_ctx;
         unit = i % per_ctx;
     } else {
-        ctx = blockIdx.x / per_ctx;
-        unit = blockIdx.x % per_ctx;
+        int id = blockIdx.x;
+        if constexpr (!CAUSAL) {  // the splits of one query tile are neighbours: they share its Q rows in the L2
+            split = id % p.key_splits;
+            id /= p.key_splits;
+        }
+        ctx = id / per_ctx;
+        unit = id % per_ctx;
     }
     const size_t ctx_elem0 = static_cast<size_t>(ctx) * S * D;
     const unsigned ctx_bytes = static_cast<unsigned>(S) * static_cast<unsigned>(D) * 4u;
@@ -351,8 +363,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DPAD <= 64 
     float run_max = -INFINITY;
     float run_sum = 0.0f;
 
-    const int key_end = CAUSAL ? min(S, q0 + kBQ) : S;
-    const int stages = (key_end + BKV - 1) / BKV;
+    const int key_first = CAUSAL ? 0 : split * p.keys_per_split;
+    const int key_end = CAUSAL ? min(S, q0 + kBQ) : min(S, key_first + p.keys_per_split);
+    const int stages = (key_end - key_first + BKV - 1) / BKV;
 
     float4 rk[LOADS], rv[LOADS];
     auto load_global = [&](int key0) {
@@ -512,14 +525,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DPAD <= 64 
     };
 
     if (stages > 0) {
-        load_global(0);
+        load_global(key_first);
         store_lds(0);
     }
     __syncthreads();
     for (int t = 0; t < stages; ++t) {
         const bool more = t + 1 < stages;
-        if (more) load_global((t + 1) * BKV);
-        const int key0 = t * BKV;
+        if (more) load_global(key_first + (t + 1) * BKV);
+        const int key0 = key_first + t * BKV;
         // Tiles entirely past the sequence end or (causal) entirely above this wavefront's rows are skipped.
         const int limit = CAUSAL ? min(S, wq0 + 32) : S;
         if (key0 + 32 < limit) compute(std::integral_constant<int, 2>{}, t & 1, key0);
@@ -529,6 +542,25 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DPAD <= 64 
     }
 
     const float total = run_sum + __shfl_xor(run_sum, 32);
+    if constexpr (!CAUSAL) {
+        if (p.key_splits > 1) {
+            if (my_q < S) {
+                const size_t row = (static_cast<size_t>(split) * p.contexts + ctx) * S + my_q;
+                float *orow = p.part_o + row * D;
+#pragma unroll
+                for (int t = 0; t < DT; ++t)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const int d = t * 32 + g * 8 + lh * 4;
+                        if (d < D)
+                            *reinterpret_cast<float4 *>(orow + d) =
+                                make_float4(oacc[t][g * 4 + 0], oacc[t][g * 4 + 1], oacc[t][g * 4 + 2], oacc[t][g * 4 + 3]);
+                    }
+                if (lh == 0) *reinterpret_cast<float2 *>(p.part_ml + row * 2) = make_float2(run_max, total);
+            }
+            return;
+        }
+    }
     const float inv = total > 0.0f ? 1.0f / total : 0.0f;
     if (my_q < S) {
         float *orow = p.out + ctx_elem0 + static_cast<size_t>(my_q) * D;
@@ -545,16 +577,99 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DPAD <= 64 
     }  // pass
 }
 
+// Combines the key splits of the fast kernel: with m = max over splits of their reference maxima,
+// out = Σ_s 2^((m_s − m)·exp_scale)·O_s / Σ_s 2^((m_s − m)·exp_scale)·l_s, splits added in order.  One thread per four
+// output values.
+__global__ __launch_bounds__(256) void attention_merge_splits_kernel(AttnArgs p, float exp_scale)
+{
+    const int D = p.D;
+    const int quads = D / 4;
+    const size_t rows = static_cast<size_t>(p.contexts) * p.S;
+    const size_t id = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (id >= rows * quads) return;
+    const size_t row = id / quads;
+    const int d = static_cast<int>(id % quads) * 4;
+    // Eight splits at a time, all their loads requested before the first is used (a plain loop over the splits is a
+    // chain of dependent memory round trips); splits past the end repeat the last one with weight zero.
+    const int last = p.key_splits - 1;
+    float top = -INFINITY;
+    for (int s0 = 0; s0 < p.key_splits; s0 += 8) {
+        float m[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) m[j] = p.part_ml[(min(s0 + j, last) * rows + row) * 2];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) top = fmaxf(top, m[j]);
+    }
+    const float safe_top = top == -INFINITY ? 0.0f : top;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    float denom = 0.0f;
+    for (int s0 = 0; s0 < p.key_splits; s0 += 8) {
+        float2 ml[8];
+        float4 o[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const size_t at = min(s0 + j, last) * rows + row;
+            ml[j] = *reinterpret_cast<const float2 *>(p.part_ml + at * 2);
+            o[j] = *reinterpret_cast<const float4 *>(p.part_o + at * D + d);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            // a split with no weight: 2^-inf = 0
+            const float w = s0 + j <= last ? __builtin_amdgcn_exp2f((ml[j].x - safe_top) * exp_scale) : 0.0f;
+            acc.x = fmaf(w, o[j].x, acc.x); acc.y = fmaf(w, o[j].y, acc.y);
+            acc.z = fmaf(w, o[j].z, acc.z); acc.w = fmaf(w, o[j].w, acc.w);
+            denom = fmaf(w, ml[j].y, denom);
+        }
+    }
+    const float inv = denom > 0.0f ? 1.0f / denom : 0.0f;
+    *reinterpret_cast<float4 *>(p.out + row * D + d) = make_float4(acc.x * inv, acc.y * inv, acc.z * inv, acc.w * inv);
+}
+
 template <int DPAD, bool CAUSAL, bool BIAS = false>
-hipError_t launch_fast(const AttnArgs &args, hipStream_t stream)
+hipError_t launch_fast(AttnArgs args, hipStream_t stream)
 {
     constexpr size_t lds_bytes = 2 * static_cast<size_t>(64) * ((DPAD + 4) + (DPAD + 8)) * sizeof(float);
     auto kernel = attention_f32_fast_kernel<DPAD, CAUSAL, BIAS>;
     hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
     if (rc != hipSuccess) return rc;
-    const size_t blocks = static_cast<size_t>(args.contexts) * (CAUSAL ? (args.q_tiles + 1) / 2 : args.q_tiles);
+    size_t blocks = static_cast<size_t>(args.contexts) * (CAUSAL ? (args.q_tiles + 1) / 2 : args.q_tiles);
+    args.key_splits = 1;
+    args.keys_per_split = args.S;
+    args.part_o = args.part_ml = nullptr;
+    if constexpr (!CAUSAL) {
+        // Few query tiles (the reference's own caller attends within one context: crates/st-nn/src/z_rba/attention.rs:586):
+        // split the keys over workgroups until the launch offers about two workgroups per compute unit, 128 keys at least
+        // per split, and merge the partial rows in a second kernel.
+        constexpr size_t kTargetBlocks = 512;
+        if (blocks * 2 <= kTargetBlocks && args.S >= 256) {
+            const size_t want = (kTargetBlocks + blocks - 1) / blocks;
+            const size_t most = static_cast<size_t>(args.S) / 128;
+            const size_t splits = std::min(want, most);
+            const size_t per = ((static_cast<size_t>(args.S) + splits - 1) / splits + 63) / 64 * 64;
+            args.keys_per_split = static_cast<int>(per);
+            args.key_splits = static_cast<int>((static_cast<size_t>(args.S) + per - 1) / per);
+        }
+        if (args.key_splits > 1) {
+            const size_t rows = static_cast<size_t>(args.contexts) * args.S;
+            const size_t o_bytes = static_cast<size_t>(args.key_splits) * rows * args.D * sizeof(float);
+            const size_t ml_bytes = static_cast<size_t>(args.key_splits) * rows * 2 * sizeof(float);
+            void *workspace = nullptr;
+            rc = stream_workspace(stream, o_bytes + ml_bytes, &workspace);
+            if (rc != hipSuccess) return rc;
+            args.part_o = static_cast<float *>(workspace);
+            args.part_ml = reinterpret_cast<float *>(static_cast<unsigned char *>(workspace) + o_bytes);
+            args.swizzle = 0;
+            blocks *= static_cast<size_t>(args.key_splits);
+        }
+    }
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), lds_bytes, stream, args);
+    rc = hipGetLastError();
+    if (rc != hipSuccess || args.key_splits == 1) return rc;
+    const float scale_log2e = fmaxf(fabsf(args.scale) * kLog2e, 1e-30f);
+    const size_t work = static_cast<size_t>(args.contexts) * args.S * (args.D / 4);
+    hipLaunchKernelGGL(attention_merge_splits_kernel, dim3(static_cast<unsigned>((work + 255) / 256)), dim3(256), 0, stream, args,
+                       BIAS ? 1.0f : scale_log2e);
     return hipGetLastError();
 }
 
@@ -609,6 +724,9 @@ hipError_t launch_attention_f32(size_t contexts, size_t sequence, size_t head_di
     if (blocks > 0x7fffffffu) return hipErrorInvalidConfiguration;
     args.swizzle = (contexts % 8 == 0) ? 1 : 0;  // each XCD gets whole contexts
     args.scale = scale;
+    args.key_splits = 1;
+    args.keys_per_split = args.S;
+    args.part_o = args.part_ml = nullptr;
     const bool bias = z_bias != nullptr || attn_bias != nullptr;
     auto aligned = [](const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; };
     const bool vec = (head_dim % 4 == 0) && aligned(q) && aligned(k) && aligned(v) && aligned(out);

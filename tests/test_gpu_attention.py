@@ -49,6 +49,26 @@ def test_random_cases(hip, oracle, contexts, seq, dim, causal, biased):
     assert_close(ones, np.ones_like(ones), F32_REL, F32_ABS, "row sums")
 
 
+@pytest.mark.parametrize("contexts,seq,dim,biased,scale", [
+    (1, 2048, 64, True, 0.125), (1, 2048, 64, False, 0.125), (3, 1000, 32, True, 0.2), (2, 300, 128, False, -0.4),
+    (1, 512, 64, False, 3.0), (5, 260, 64, True, 0.0), (1, 4096, 16, False, 0.25), (7, 384, 64, False, 0.125)])
+def test_keys_split_over_workgroups(hip, oracle, contexts, seq, dim, biased, scale):
+    """Non-causal calls with few query tiles (the reference's own caller attends within one context) split the keys
+    over workgroups and merge the partial rows: same values as the oracle, rows still sum to one, and a softmax so
+    peaked (scale 3) that one split holds nearly all of a row's weight."""
+    rng = np.random.default_rng(contexts * 31 + seq + dim)
+    q, k, v = (rng.normal(size=contexts * seq * dim).astype(np.float32) for _ in range(3))
+    zb = rng.normal(size=contexts * seq).astype(np.float32) if biased else None
+    ab = rng.normal(0, 2.0, size=contexts * seq * seq).astype(np.float32) if biased else None
+    got = run(hip, contexts, seq, dim, scale, q, k, v, zb, ab, False)
+    want = oracle.attention_f32(contexts, seq, dim, scale, q, k, v, zb, ab, False, threads=8)
+    assert_close(got, want, F32_REL, F32_ABS, f"split keys {contexts}x{seq}x{dim} bias={biased} scale={scale}")
+    ones = run(hip, contexts, seq, dim, scale, q, k, np.ones_like(v), zb, ab, False)
+    assert_close(ones, np.ones_like(ones), F32_REL, F32_ABS, "row sums")
+    again = run(hip, contexts, seq, dim, scale, q, k, v, zb, ab, False)
+    assert (again == got).all(), "the splits are merged in a fixed order"
+
+
 @pytest.mark.parametrize("scale", [-0.3, 0.0, 2.5])
 @pytest.mark.parametrize("causal", [False, True])
 def test_unusual_scales(hip, oracle, scale, causal):
