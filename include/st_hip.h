@@ -226,6 +226,19 @@ int st_hip_gemm_bf16_prepacked_bias_act_dev(size_t m, size_t n, size_t k, int ac
                                             const uint16_t *lhs, const uint16_t *packed_rhs,
                                             const float *bias, const float *residual, float *out_f32,
                                             uint16_t *out_bf16, void *stream);
+/* Linear + residual + LayerNorm of a pre-norm transformer block in one call (block order of
+ * crates/st-vision/src/models/vit.rs:256-265; Linear::forward, crates/st-nn/src/layers/linear.rs:87-107; layer_norm,
+ * crates/st-tensor/src/pure.rs:4008-4058): out_f32 = (lhs·rhs + bias) + residual, the rows the next residual add needs,
+ * and out_ln_bf16 = layer_norm(out_f32; gamma, beta, epsilon) rounded nearest-even to bf16, the operand of the next
+ * projection.  bf16 lhs (m×k), rhs prepacked as its (n, k) transpose, f32 accumulation; bias (n) and residual (m×n)
+ * may be NULL, gamma and beta (n) may not.  n = 512 with k a multiple of 64 up to 1024 and 16-byte aligned buffers is
+ * a single kernel whose workgroups own whole rows; any other shape runs the GEMM and the layer-norm kernel one after
+ * the other.  Both routes give the same bits. */
+int st_hip_gemm_bf16_prepacked_residual_layer_norm_dev(size_t m, size_t n, size_t k, const uint16_t *lhs,
+                                                      const uint16_t *packed_rhs, const float *bias,
+                                                      const float *residual, const float *gamma, const float *beta,
+                                                      float epsilon, float *out_f32, uint16_t *out_ln_bf16,
+                                                      void *stream);
 int st_hip_pack_rhs_bf16_dev(size_t k, size_t n, const uint16_t *rhs, uint16_t *packed, void *stream);
 int st_hip_conv2d_bias_act_f32_dev(size_t batch, size_t c_in, size_t h, size_t w, size_t c_out,
                                    size_t kh, size_t kw, size_t stride_h, size_t stride_w,

@@ -97,6 +97,9 @@ SIGNATURES = {
                                               c_void_p, c_void_p, c_void_p, c_void_p]),
     "st_hip_gemm_bf16_prepacked_bias_act_dev": (c_int, [c_size_t, c_size_t, c_size_t, c_int, c_void_p, c_void_p,
                                                         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "st_hip_gemm_bf16_prepacked_residual_layer_norm_dev": (c_int, [c_size_t, c_size_t, c_size_t, c_void_p, c_void_p, c_void_p,
+                                                                    c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p,
+                                                                    c_void_p]),
     "st_hip_pack_rhs_bf16_dev": (c_int, [c_size_t, c_size_t, c_void_p, c_void_p, c_void_p]),
     "st_hip_conv2d_bias_act_f32_dev": (c_int, [c_size_t] * 13 + [c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                                                  c_void_p]),

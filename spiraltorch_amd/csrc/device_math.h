@@ -43,6 +43,11 @@ __device__ __forceinline__ float relu_or_identity(float value, bool relu)
     return relu ? rectified : value;
 }
 
+// Sum and sum of squares of four neighbouring row values, with the association written out: the layer-norm kernel and
+// the GEMM epilogue that normalises rows must add a row's values in the same order to give the same statistics.
+__device__ __forceinline__ float sum4(const float4 &v) { return (v.x + v.y) + (v.z + v.w); }
+__device__ __forceinline__ float sumsq4(const float4 &v) { return fmaf(v.x, v.x, v.y * v.y) + fmaf(v.z, v.z, v.w * v.w); }
+
 // Runs `body(act, has_residual)` with the activation as a callable and the presence of a residual as a compile-time
 // constant, chosen once from the (wavefront-uniform) launch arguments: an epilogue that decides them per element
 // compiles to a chain of scalar branches around every store.

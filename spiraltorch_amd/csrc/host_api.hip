@@ -748,6 +748,23 @@ int st_hip_gemm_bf16_prepacked_bias_act_dev(size_t m, size_t n, size_t k, int ac
                          "gemm_bf16 prepacked launch");
 }
 
+int st_hip_gemm_bf16_prepacked_residual_layer_norm_dev(size_t m, size_t n, size_t k, const uint16_t *lhs,
+                                                      const uint16_t *packed_rhs, const float *bias, const float *residual,
+                                                      const float *gamma, const float *beta, float epsilon, float *out_f32,
+                                                      uint16_t *out_ln_bf16, void *stream)
+{
+    ST_HIP_CHECK(ensure_init());
+    ST_HIP_CHECK(validate_kernel_dims(m, n, k));
+    if (!std::isfinite(epsilon) || epsilon < 0.0f)
+        return fail(ST_HIP_ERR_INVALID, "layer_norm epsilon must be finite and non-negative, received %g", static_cast<double>(epsilon));
+    if (m == 0 || n == 0) return ST_HIP_OK;
+    if (!out_f32 || !out_ln_bf16 || !gamma || !beta || (k != 0 && (!lhs || !packed_rhs)))
+        return fail(ST_HIP_ERR_INVALID, "gemm + layer_norm received a null pointer; provide contiguous row-major buffers");
+    return launch_status(launch_gemm_bf16_residual_layer_norm(m, n, k, lhs, packed_rhs, bias, residual, gamma, beta, epsilon,
+                                                              out_f32, out_ln_bf16, as_stream(stream)),
+                         "gemm_bf16 + layer_norm launch");
+}
+
 int st_hip_pack_rhs_bf16_dev(size_t k, size_t n, const uint16_t *rhs, uint16_t *packed, void *stream)
 {
     ST_HIP_CHECK(ensure_init());

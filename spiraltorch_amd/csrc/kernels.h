@@ -30,6 +30,11 @@ hipError_t launch_transpose_f32(size_t rows, size_t cols, const float *in, float
 hipError_t launch_gemm_bf16(size_t m, size_t n, size_t k, const uint16_t *lhs, const uint16_t *rhs,
                             float *out_f32, uint16_t *out_bf16, const GemmEpilogue &epilogue,
                             hipStream_t stream, bool rhs_packed = false);
+// out_f32 = (lhs·rhs + bias) + residual and out_ln = layer_norm(out_f32) rounded to bf16, rhs packed n×k: Linear + residual +
+// LayerNorm of a transformer block (crates/st-vision/src/models/vit.rs:256-265) in one launch where the shape allows.
+hipError_t launch_gemm_bf16_residual_layer_norm(size_t m, size_t n, size_t k, const uint16_t *lhs, const uint16_t *packed_rhs,
+                                                const float *bias, const float *residual, const float *gamma, const float *beta,
+                                                float epsilon, float *out_f32, uint16_t *out_ln, hipStream_t stream);
 // out(cols×rows) = in(rows×cols) transposed, 16-bit elements.
 hipError_t launch_transpose_u16(size_t rows, size_t cols, const uint16_t *in, uint16_t *out, hipStream_t stream);
 

@@ -70,8 +70,8 @@ __global__ __launch_bounds__(256) void layer_norm_vec_kernel(int rows, int cols,
                 v[i].x += r.x; v[i].y += r.y; v[i].z += r.z; v[i].w += r.w;
             }
         }
-        sum += (v[i].x + v[i].y) + (v[i].z + v[i].w);
-        sumsq += (v[i].x * v[i].x + v[i].y * v[i].y) + (v[i].z * v[i].z + v[i].w * v[i].w);
+        sum += sum4(v[i]);
+        sumsq += sumsq4(v[i]);
     }
     sum = wave_sum(sum);
     sumsq = wave_sum(sumsq);

@@ -384,6 +384,15 @@ def gemm_bf16_prepacked_bias_act_dev(m, n, k, activation, lhs, packed_rhs, bias,
                                                                _dev(out_bf16), _stream_ptr(stream)))
 
 
+def gemm_bf16_prepacked_residual_layer_norm_dev(m, n, k, lhs, packed_rhs, bias, residual, gamma, beta, epsilon, out_f32,
+                                                out_ln_bf16, stream=None) -> None:
+    """out_f32 = (lhs @ rhs + bias) + residual and out_ln_bf16 = layer_norm(out_f32) rounded to bf16: Linear + residual +
+    LayerNorm of a pre-norm transformer block (crates/st-vision/src/models/vit.rs:256-265) in one call."""
+    _check(_lib.load().st_hip_gemm_bf16_prepacked_residual_layer_norm_dev(
+        m, n, k, _dev(lhs), _dev(packed_rhs), _dev(bias), _dev(residual), _dev(gamma), _dev(beta), float(epsilon),
+        _dev(out_f32), _dev(out_ln_bf16), _stream_ptr(stream)))
+
+
 def pack_rhs_bf16_dev(k, n, rhs, packed, stream=None) -> None:
     """packed (n, k) = rhs (k, n) transposed, bf16 bit patterns, on the device."""
     _check(_lib.load().st_hip_pack_rhs_bf16_dev(k, n, _dev(rhs), _dev(packed), _stream_ptr(stream)))

@@ -229,6 +229,54 @@ def test_skinny_prepacked_single_launch(hip, oracle, m, n, k):
         assert (d16.to_array(np.uint16, m * n) == inputs.to_bf16(got32)).all()
 
 
+@pytest.mark.parametrize("m,n,k", [(64, 512, 64), (1000, 512, 512), (16384, 512, 192), (130, 512, 2048), (1, 512, 128),
+                                   # other widths: the GEMM and the layer-norm kernel one after the other
+                                   (300, 384, 128), (33, 512, 96), (70, 1024, 256)])
+def test_gemm_residual_layer_norm(hip, oracle, m, n, k):
+    """Linear + residual + LayerNorm in one call: the rows before normalisation against the oracle's GEMM (+ bias +
+    residual), the normalised bf16 rows against the oracle's layer-norm of those rows (within one bf16 step: the
+    row statistics are summed in another order), and against the separate GEMM and layer-norm kernels."""
+    from spiraltorch_amd import inputs
+    rng = np.random.default_rng(m + 3 * n + 5 * k)
+    a, b = bf16_pair(rng, m, n, k, std=0.5)
+    bias = rng.normal(size=n).astype(np.float32)
+    res = rng.normal(size=m * n).astype(np.float32)
+    gamma = rng.normal(1.0, 0.2, size=n).astype(np.float32)
+    beta = rng.normal(0.0, 0.2, size=n).astype(np.float32)
+    eps = 1e-5
+    d = {name: hip.DeviceBuffer.from_array(v) for name, v in (("a", a), ("bias", bias), ("res", res), ("g", gamma), ("b", beta))}
+    d_packed = hip.DeviceBuffer.from_array(np.ascontiguousarray(b.reshape(k, n).T))
+    x32, ln16 = hip.DeviceBuffer(m * n * 4), hip.DeviceBuffer(m * n * 2)
+    hip.gemm_bf16_prepacked_residual_layer_norm_dev(m, n, k, d["a"], d_packed, d["bias"], d["res"], d["g"], d["b"], eps, x32, ln16)
+    hip.device_synchronize()
+    base = oracle.gemm_bf16_f32acc(m, n, k, a, b, threads=8)
+    want_x = ((base.reshape(m, n) + bias).astype(np.float32).ravel() + res).astype(np.float32)
+    got_x = x32.to_array(np.float32, m * n)
+    assert_close(got_x, want_x, 1e-4, 1e-4, f"rows before normalisation {m}x{n}x{k}")
+    # the normalisation is checked on the rows the GPU produced, so that only the layer-norm itself is compared
+    want_ln = oracle.layer_norm_f32(m, n, got_x, gamma, beta, eps)
+    got_ln = inputs.from_bf16(ln16.to_array(np.uint16, m * n))
+    step = np.maximum(np.abs(want_ln), 2.0 ** -120) * 2.0 ** -7  # one bf16 step is at most 2^-7 relative
+    assert (np.abs(got_ln - want_ln) <= step + 1e-6).all(), "normalised rows differ from the oracle by more than one bf16 step"
+    # separate kernels on the same operands
+    y32, y16 = hip.DeviceBuffer(m * n * 4), hip.DeviceBuffer(m * n * 2)
+    hip.gemm_bf16_prepacked_bias_act_dev(m, n, k, 0, d["a"], d_packed, d["bias"], d["res"], y32, None)
+    hip.layer_norm_f32_dev(m, n, y32, None, d["g"], d["b"], eps, None, y16)
+    hip.device_synchronize()
+    assert (y32.to_array(np.float32, m * n) == got_x).all(), "both kernels add the k products in the same order"
+    sep = y16.to_array(np.uint16, m * n)
+    assert (sep == ln16.to_array(np.uint16, m * n)).all(), "fused and separate normalisation add a row in the same order"
+    # without bias and residual
+    hip.gemm_bf16_prepacked_residual_layer_norm_dev(m, n, k, d["a"], d_packed, None, None, d["g"], d["b"], eps, x32, ln16)
+    hip.device_synchronize()
+    plain = x32.to_array(np.float32, m * n)
+    assert_close(plain, base, 1e-4, 1e-4, "no bias, no residual")
+    want_ln = oracle.layer_norm_f32(m, n, plain, gamma, beta, eps)
+    got_ln = inputs.from_bf16(ln16.to_array(np.uint16, m * n))
+    step = np.maximum(np.abs(want_ln), 2.0 ** -120) * 2.0 ** -7
+    assert (np.abs(got_ln - want_ln) <= step + 1e-6).all()
+
+
 def test_config4_4096_cubed_prepacked(hip, oracle):
     """BASELINE config 4 with B prepacked: 24 sampled rows against the oracle, the rest of the matrix bit for bit
     against the k×n kernel (checked itself above), and exact power-of-two linearity."""
