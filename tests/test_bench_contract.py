@@ -38,5 +38,5 @@ def test_entries_carry_measured_traffic_only_where_a_profile_has_it():
     item = bench.entry(name, "f32", 14_797_504_512, 77_365_760, "mfma", 0.16, 0.16)
     assert item["roofline"]["traffic"] == bench.MEASURED_TRAFFIC_BYTES[name]
     assert 1.0 < item["roofline"]["traffic"] / 77_365_760 < 1.2  # measured HBM bytes close to the algorithmic bytes
-    assert bench.entry("gemm_f32_512x512x512", "f32", 1, 1, "mfma", 1.0, 1.0)["roofline"]["traffic"] is None
+    assert bench.entry("decoder_bf16_v256_d512_h8_l6_ff2048_b16_s1024", "bf16", 1, 1, "mfma", 1.0, 1.0)["roofline"]["traffic"] is None
     json.dumps(item)  # serialisable
