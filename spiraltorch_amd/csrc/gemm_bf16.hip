@@ -1654,7 +1654,8 @@ hipError_t launch_gemm_bf16_residual_layer_norm(size_t m, size_t n, size_t k, co
     // Measured at m = 16384 (one 64-row workgroup per compute unit): 27.3 µs against 18.2 + 10.2 µs for the two kernels at
     // k = 512, 51.2 against 37.9 + 10.1 µs at k = 2048 — a 64-row tile streams the whole of B through every compute unit,
     // which costs more than the saved pass over the rows once k is long.
-    if (n == 512 && k >= 64 && k % 64 == 0 && k <= 1024 && fits_buffer && aligned) {
+    // (m <= 64 stays with the GEMM dispatcher, which splits k over the chip for such shapes.)
+    if (n == 512 && m > 64 && k >= 64 && k % 64 == 0 && k <= 1024 && fits_buffer && aligned) {
         RowLnArgs row;
         row.g.A = lhs;
         row.g.B = packed_rhs;
