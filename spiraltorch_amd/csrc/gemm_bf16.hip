@@ -36,6 +36,12 @@ struct GemmBf16Args {
     int swizzle;  // 1: remap workgroup ids so each XCD (id % 8) works on a compact block of tiles
     float scale;
     int activation;
+    // Split-k form of the 256-row kernels (launches of few tiles with a long k): workgroup (tile, split) covers
+    // tiles_per_split k-tiles and leaves its raw sums in partial[split][M][N]; gemm_bf16_skinny_reduce_kernel adds the
+    // splits in order and applies the epilogue.
+    int k_splits = 1;
+    int tiles_per_split = 0;
+    float *partial = nullptr;
 };
 
 typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
@@ -423,6 +429,24 @@ __device__ __forceinline__ void gemm_bf16_epilogue(const GemmBf16Args &p, const 
     else gemm_bf16_epilogue_rows<WTN, TM, ST_HIP_ACT_NONE>(p, acc, lds, wave, row_first, col_base, lane);
 }
 
+// Epilogue of a 256-row kernel's workgroup: the launch's own, or — when k is split over workgroups — the raw sums of
+// this split into its plane of the partial buffer (the reduction kernel applies scale, bias, residual and activation).
+template <int WTN, int TM>
+__device__ __forceinline__ void gemm_bf16_finish(const GemmBf16Args &p, int split, const f32x16 (&acc)[TM][WTN / 32],
+                                                 unsigned char *lds, int wave, int row_first, int col_base, int lane)
+{
+    GemmBf16Args q = p;
+    if (p.k_splits > 1) {
+        q.C32 = p.partial + static_cast<size_t>(split) * p.M * p.N;
+        q.C16 = nullptr;
+        q.bias = nullptr;
+        q.residual = nullptr;
+        q.scale = 1.0f;
+        q.activation = ST_HIP_ACT_NONE;
+    }
+    gemm_bf16_epilogue<WTN, TM>(q, acc, lds, wave, row_first, col_base, lane);
+}
+
 // -------------------------------------------------------------------------------------------------
 // Packed-B kernel: B is given prepacked as Bᵀ (n×k row-major, k contiguous — PackedB's column-major layout,
 // crates/st-tensor/src/pure.rs:1285-1323).  Same 256×BN×64 tiles, LDS layout, swizzle and epilogue as the kernel
@@ -467,6 +491,9 @@ __device__ __forceinline__ void gemm_bf16_packed_body(const GemmBf16Args &p)
 
     int logical = blockIdx.x;
     if (p.swizzle) logical = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+    const int tiles = p.tiles_m * p.tiles_n;
+    const int split = logical / tiles;  // 0 unless k is split over workgroups
+    logical -= split * tiles;
     constexpr int GROUP_M = 4;
     const int width = GROUP_M * p.tiles_n;
     const int group = logical / width;
@@ -475,6 +502,7 @@ __device__ __forceinline__ void gemm_bf16_packed_body(const GemmBf16Args &p)
     const int tile_m = first_m + (logical % width) % group_size;
     const int tile_n = (logical % width) / group_size;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int tile0 = split * p.tiles_per_split;  // first k-tile of this workgroup
 
     const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint16_t *>(p.A), 0, static_cast<int>(static_cast<unsigned>(M) * static_cast<unsigned>(K) * 2u), 0x00020000);
@@ -488,11 +516,12 @@ __device__ __forceinline__ void gemm_bf16_packed_body(const GemmBf16Args &p)
     {
         const int row_in = wave * 8 + (lane >> 3);
         const int sw_base = ((wave * 4 + (lane >> 4)) ^ (wave >> 1)) & 7;
+        const unsigned k_first = static_cast<unsigned>(tile0) * BK;
 #pragma unroll
         for (int r = 0; r < NMAX; ++r) {
             const int chunk = ((lane & 7) ^ sw_base ^ ((r * WAVES / 2) & 7)) & 7;
-            if (r < NA) a_off[r] = (static_cast<unsigned>(m0 + r * WAVES * 8 + row_in) * K + chunk * 8) * 2u;
-            if (r < NB) b_off[r] = (static_cast<unsigned>(n0 + r * WAVES * 8 + row_in) * K + chunk * 8) * 2u;
+            if (r < NA) a_off[r] = (static_cast<unsigned>(m0 + r * WAVES * 8 + row_in) * K + k_first + chunk * 8) * 2u;
+            if (r < NB) b_off[r] = (static_cast<unsigned>(n0 + r * WAVES * 8 + row_in) * K + k_first + chunk * 8) * 2u;
         }
     }
     const int lds_row_block = wave * 1024;  // wavefront-uniform part of every load's LDS destination
@@ -586,7 +615,7 @@ __device__ __forceinline__ void gemm_bf16_packed_body(const GemmBf16Args &p)
         a_stage = a_next;
     };
 
-    const int steps = K / BK;
+    const int steps = p.k_splits > 1 ? min(p.tiles_per_split, K / BK - tile0) : K / BK;
 #pragma unroll
     for (int r = 0; r < NA; ++r) load_a1(0, r, 0u);
 #pragma unroll
@@ -614,7 +643,7 @@ __device__ __forceinline__ void gemm_bf16_packed_body(const GemmBf16Args &p)
     iteration(std::false_type{}, std::false_type{}, t);
 
     __syncthreads();
-    gemm_bf16_epilogue<WTN, TM>(p, acc, lds_bytes, wave, m0 + wm * WTM, n0 + wn * WTN, lane);
+    gemm_bf16_finish<WTN, TM>(p, split, acc, lds_bytes, wave, m0 + wm * WTM, n0 + wn * WTN, lane);
 }
 
 // -------------------------------------------------------------------------------------------------
@@ -897,6 +926,9 @@ __device__ __forceinline__ void gemm_bf16_rowmajor_body(const GemmBf16Args &p)
 
     int logical = blockIdx.x;
     if (p.swizzle) logical = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+    const int tiles = p.tiles_m * p.tiles_n;
+    const int split = logical / tiles;  // 0 unless k is split over workgroups
+    logical -= split * tiles;
     constexpr int GROUP_M = 4;
     const int width = GROUP_M * p.tiles_n;
     const int group = logical / width;
@@ -905,6 +937,7 @@ __device__ __forceinline__ void gemm_bf16_rowmajor_body(const GemmBf16Args &p)
     const int tile_m = first_m + (logical % width) % group_size;
     const int tile_n = (logical % width) / group_size;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int tile0 = split * p.tiles_per_split;  // first k-tile of this workgroup
 
     const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint16_t *>(p.A), 0, static_cast<int>(static_cast<unsigned>(M) * static_cast<unsigned>(K) * 2u), 0x00020000);
@@ -916,10 +949,11 @@ __device__ __forceinline__ void gemm_bf16_rowmajor_body(const GemmBf16Args &p)
     {
         const int row_in = wave * 8 + (lane >> 3);
         const int sw_base = ((wave * 4 + (lane >> 4)) ^ (wave >> 1)) & 7;
+        const unsigned k_first = static_cast<unsigned>(tile0) * BK;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int chunk = ((lane & 7) ^ sw_base ^ ((4 * r) & 7)) & 7;
-            a_off[r] = (static_cast<unsigned>(m0 + r * 64 + row_in) * K + chunk * 8) * 2u;
+            a_off[r] = (static_cast<unsigned>(m0 + r * 64 + row_in) * K + k_first + chunk * 8) * 2u;
         }
     }
     const int lds_row_block = wave * 1024;
@@ -936,7 +970,7 @@ __device__ __forceinline__ void gemm_bf16_rowmajor_body(const GemmBf16Args &p)
     const unsigned b_tile_step = static_cast<unsigned>(BK) * N * 2u;
     uint2 rb[KR];
     auto load_b1 = [&](int j, unsigned tile) {
-        const unsigned soff = __builtin_amdgcn_readfirstlane(tile * b_tile_step);
+        const unsigned soff = __builtin_amdgcn_readfirstlane((tile + static_cast<unsigned>(tile0)) * b_tile_step);
         const auto v = __builtin_amdgcn_raw_buffer_load_b64(rsrc_b, b_voff[j], soff, 0);
         rb[j] = make_uint2(v[0], v[1]);
     };
@@ -1051,7 +1085,7 @@ __device__ __forceinline__ void gemm_bf16_rowmajor_body(const GemmBf16Args &p)
         a_stage = a_next;
     };
 
-    const int steps = K / BK;
+    const int steps = p.k_splits > 1 ? min(p.tiles_per_split, K / BK - tile0) : K / BK;
 #pragma unroll
     for (int r = 0; r < 4; ++r) load_a1(0, r, 0u);
 #pragma unroll
@@ -1083,7 +1117,7 @@ __device__ __forceinline__ void gemm_bf16_rowmajor_body(const GemmBf16Args &p)
     iteration(std::false_type{}, std::false_type{}, t);
 
     __syncthreads();
-    gemm_bf16_epilogue<WTN>(p, acc, lds_bytes, wave, m0 + wm * 64, n0 + wn * WTN, lane);
+    gemm_bf16_finish<WTN, 2>(p, split, acc, lds_bytes, wave, m0 + wm * 64, n0 + wn * WTN, lane);
 }
 
 __global__ __launch_bounds__(512) void gemm_bf16_256rm_kernel(GemmBf16Args p) { gemm_bf16_rowmajor_body<256>(p); }
@@ -1505,12 +1539,45 @@ __global__ __launch_bounds__(256) void transpose_u16_kernel(int rows, int cols, 
 }
 
 template <int BN>
-hipError_t launch_256(GemmBf16Args args, bool packed, hipStream_t stream)
+hipError_t launch_256(GemmBf16Args args, bool packed, hipStream_t stream, size_t workspace_offset)
 {
     args.tiles_m = (args.M + 255) / 256;
     args.tiles_n = args.N / BN;
-    const size_t tiles = static_cast<size_t>(args.tiles_m) * static_cast<size_t>(args.tiles_n);
+    size_t tiles = static_cast<size_t>(args.tiles_m) * static_cast<size_t>(args.tiles_n);
     if (tiles > 0x7fffffffu) return hipErrorInvalidConfiguration;
+    // Few tiles and a long k (a batch of a hundred rows against a 4096² weight is 32 tiles of 64 k-tiles each): split k
+    // over workgroups until the launch fills the chip — at least four k-tiles per split, and only as far as the partial
+    // sums (written once, read once) stay below the operands' own bytes, or the split costs more than it spreads.
+    const size_t k_tiles = static_cast<size_t>(args.K) / 64;
+    size_t splits = 1;
+    if (tiles * 2 <= 256 && k_tiles >= 8) {
+        splits = std::min<size_t>(256 / tiles, k_tiles / 4);
+        const size_t operand_bytes = (static_cast<size_t>(args.M) * args.K + static_cast<size_t>(args.K) * args.N) * 2;
+        const size_t plane_bytes = static_cast<size_t>(args.M) * args.N * sizeof(float);
+        while (splits > 1 && splits * plane_bytes * 2 > operand_bytes) --splits;
+    }
+    SkinnyArgs reduce{};
+    if (splits > 1) {
+        args.tiles_per_split = static_cast<int>((k_tiles + splits - 1) / splits);
+        args.k_splits = static_cast<int>((k_tiles + args.tiles_per_split - 1) / args.tiles_per_split);
+        const size_t bytes = static_cast<size_t>(args.k_splits) * args.M * args.N * sizeof(float);
+        void *workspace = nullptr;
+        hipError_t rc = stream_workspace(stream, workspace_offset + bytes, &workspace);
+        if (rc != hipSuccess) return rc;
+        args.partial = reinterpret_cast<float *>(static_cast<unsigned char *>(workspace) + workspace_offset);
+        reduce.partial = args.partial;
+        reduce.C32 = args.C32;
+        reduce.C16 = args.C16;
+        reduce.bias = args.bias;
+        reduce.residual = args.residual;
+        reduce.M = args.M;
+        reduce.N = args.N;
+        reduce.K = args.K;
+        reduce.k_splits = args.k_splits;
+        reduce.scale = args.scale;
+        reduce.activation = args.activation;
+        tiles *= static_cast<size_t>(args.k_splits);
+    }
     args.swizzle = (tiles % 8 == 0) ? 1 : 0;
     constexpr size_t lds_bytes = 5 * 32768;  // three A stages + two B stages
     static_assert(lds_bytes >= 8 * 32 * (128 + 4) * sizeof(float), "eight epilogue strips must fit in the stage buffers");
@@ -1520,6 +1587,11 @@ hipError_t launch_256(GemmBf16Args args, bool packed, hipStream_t stream)
                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
     if (rc != hipSuccess) return rc;
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(tiles)), dim3(512), lds_bytes, stream, args);
+    rc = hipGetLastError();
+    if (rc != hipSuccess || args.k_splits == 1) return rc;
+    const size_t plane = static_cast<size_t>(args.M) * args.N;
+    hipLaunchKernelGGL(gemm_bf16_skinny_reduce_kernel, dim3(static_cast<unsigned>((plane + 255) / 256)), dim3(256), 0, stream,
+                       reduce);
     return hipGetLastError();
 }
 
@@ -1634,8 +1706,9 @@ hipError_t launch_gemm_bf16(size_t m, size_t n, size_t k, const uint16_t *lhs, c
         // rounds that the 256-wide tiling would leave partly empty (or when N is not a multiple of 256).
         auto fill = [](size_t tiles) { return static_cast<double>(tiles) / static_cast<double>((tiles + 255) / 256 * 256); };
         const size_t row_tiles = (m + 255) / 256;
-        if (n % 256 != 0 || fill(row_tiles * (n / 128)) > 1.15 * fill(row_tiles * (n / 256))) return launch_256<128>(args, rhs_packed, stream);
-        return launch_256<256>(args, rhs_packed, stream);
+        if (n % 256 != 0 || fill(row_tiles * (n / 128)) > 1.15 * fill(row_tiles * (n / 256)))
+            return launch_256<128>(args, rhs_packed, stream, workspace_offset);
+        return launch_256<256>(args, rhs_packed, stream, workspace_offset);
     }
     return launch_tile<128, 128, 32>(args, vec, stream);
 }

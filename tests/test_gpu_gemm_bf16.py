@@ -278,6 +278,45 @@ def test_gemm_residual_layer_norm(hip, oracle, m, n, k):
     assert (np.abs(got_ln - want_ln) <= step + 1e-6).all()
 
 
+@pytest.mark.parametrize("m,n,k", [(100, 4096, 4096), (256, 1024, 4096), (130, 2048, 2048), (65, 128, 8192), (4096, 128, 4096),
+                                   (300, 384, 1984)])
+def test_few_tiles_with_a_long_k_split_k(hip, oracle, m, n, k):
+    """Launches of few 256-row tiles with many k-tiles split k over workgroups (raw partial sums, added in split order by
+    a second kernel that applies the epilogue): both layouts of B, the fused epilogue with both output types, and the
+    same bits from call to call and from either layout."""
+    from spiraltorch_amd import inputs
+    rng = np.random.default_rng(m + 7 * n + 3 * k)
+    a, b = bf16_pair(rng, m, n, k, std=0.5)
+    bias = rng.normal(size=n).astype(np.float32)
+    res = rng.normal(size=m * n).astype(np.float32)
+    d = {name: hip.DeviceBuffer.from_array(v) for name, v in (("a", a), ("b", b), ("bias", bias), ("res", res))}
+    d_packed = hip.DeviceBuffer.from_array(np.ascontiguousarray(b.reshape(k, n).T))
+    out = hip.DeviceBuffer(m * n * 4)
+    hip.gemm_bf16_f32acc_dev(m, n, k, d["a"], d["b"], out)
+    hip.device_synchronize()
+    base = oracle.gemm_bf16_f32acc(m, n, k, a, b, threads=8)
+    plain = out.to_array(np.float32, m * n)
+    check(plain, base, f"row-major {m}x{n}x{k}")
+    hip.gemm_bf16_prepacked_bias_act_dev(m, n, k, 0, d["a"], d_packed, None, None, out, None)
+    hip.device_synchronize()
+    assert (out.to_array(np.float32, m * n) == plain).all(), "both layouts split k the same way"
+    hip.gemm_bf16_f32acc_dev(m, n, k, d["a"], d["b"], out)
+    hip.device_synchronize()
+    assert (out.to_array(np.float32, m * n) == plain).all(), "the splits are added in a fixed order"
+    d16 = hip.DeviceBuffer(m * n * 2)
+    pre = (base.astype(np.float64).reshape(m, n) + bias).ravel() + res
+    want = 0.5 * pre * (1.0 + np.tanh(0.7978846 * (pre + 0.044715 * pre ** 3)))
+    for packed in (False, True):
+        if packed:
+            hip.gemm_bf16_prepacked_bias_act_dev(m, n, k, 2, d["a"], d_packed, d["bias"], d["res"], out, d16)
+        else:
+            hip.gemm_bf16_bias_act_dev(m, n, k, 2, d["a"], d["b"], d["bias"], d["res"], out, d16)
+        hip.device_synchronize()
+        got32 = out.to_array(np.float32, m * n)
+        assert_close(got32, want, 1e-4, 2e-5 * max(1.0, float(np.abs(base).max())), f"split-k epilogue packed={packed}")
+        assert (d16.to_array(np.uint16, m * n) == inputs.to_bf16(got32)).all()
+
+
 def test_config4_4096_cubed_prepacked(hip, oracle):
     """BASELINE config 4 with B prepacked: 24 sampled rows against the oracle, the rest of the matrix bit for bit
     against the k×n kernel (checked itself above), and exact power-of-two linearity."""
