@@ -41,7 +41,10 @@ struct AttnArgs {
     // Keys split over workgroups (non-causal fast kernel only): workgroup (…, split) covers keys_per_split keys
     // (a multiple of 64) and leaves its un-normalised output rows in part_o[split][context·S + query][D] and their
     // (reference maximum, sum) in part_ml[split][context·S + query][2]; attention_merge_splits_kernel combines them.
+    // Causal calls split per query tile: tile j sees (j + 1)·128 keys, i.e. j / r + 1 chunks of keys_per_split = 128·r
+    // keys; causal_items is the number of (tile, chunk) workgroups per context and key_splits the most chunks a tile has.
     int key_splits, keys_per_split;
+    int causal_items;
     float *part_o;
     float *part_ml;
 };
@@ -306,6 +309,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DPAD <= 64 
     const int per_ctx = CAUSAL ? (p.q_tiles + 1) / 2 : p.q_tiles;  // workgroups per context
     int ctx, unit;
     int split = 0;
+    int split_tile = -1;  // causal with split keys: this workgroup's query tile (no pairing then)
     if (p.swizzle) {
         const int per_xcd = p.contexts >> 3;
         const int xcd = blockIdx.x & 7, i = blockIdx.x >> 3;
@@ -313,12 +317,28 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DPAD <= 64 
         unit = i % per_ctx;
     } else {
         int id = blockIdx.x;
-        if constexpr (!CAUSAL) {  // the splits of one query tile are neighbours: they share its Q rows in the L2
-            split = id % p.key_splits;
-            id /= p.key_splits;
+        if (CAUSAL && p.key_splits > 1) {
+            // (tile, chunk) items of a context, tiles from the last (most chunks) to the first
+            ctx = id / p.causal_items;
+            int rest = id - ctx * p.causal_items;
+            const int r = p.keys_per_split / kBQ;
+            int j = p.q_tiles - 1;
+            for (;; --j) {
+                const int chunks = j / r + 1;
+                if (rest < chunks) break;
+                rest -= chunks;
+            }
+            split_tile = j;
+            split = rest;
+            unit = 0;
+        } else {
+            if constexpr (!CAUSAL) {  // the splits of one query tile are neighbours: they share its Q rows in the L2
+                split = id % p.key_splits;
+                id /= p.key_splits;
+            }
+            ctx = id / per_ctx;
+            unit = id % per_ctx;
         }
-        ctx = id / per_ctx;
-        unit = id % per_ctx;
     }
     const size_t ctx_elem0 = static_cast<size_t>(ctx) * S * D;
     const unsigned ctx_bytes = static_cast<unsigned>(S) * static_cast<unsigned>(D) * 4u;
@@ -337,9 +357,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DPAD <= 64 
         return v;
     };
 
-    const int passes = (CAUSAL && unit != p.q_tiles - 1 - unit) ? 2 : 1;
+    const int passes = (CAUSAL && split_tile < 0 && unit != p.q_tiles - 1 - unit) ? 2 : 1;
     for (int pass = 0; pass < passes; ++pass) {
-    const int q_tile = CAUSAL ? (pass == 0 ? p.q_tiles - 1 - unit : unit) : unit;  // the long tile first
+    const int q_tile = !CAUSAL ? unit : split_tile >= 0 ? split_tile : (pass == 0 ? p.q_tiles - 1 - unit : unit);  // the long tile first
     const int q0 = q_tile * kBQ;
     const int wq0 = q0 + wave * 32;
     const int my_q = wq0 + li;
@@ -363,8 +383,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DPAD <= 64 
     float run_max = -INFINITY;
     float run_sum = 0.0f;
 
-    const int key_first = CAUSAL ? 0 : split * p.keys_per_split;
-    const int key_end = CAUSAL ? min(S, q0 + kBQ) : min(S, key_first + p.keys_per_split);
+    const bool split_keys = !CAUSAL || split_tile >= 0;
+    const int key_first = split_keys ? split * p.keys_per_split : 0;
+    const int key_end = min(CAUSAL ? min(S, q0 + kBQ) : S, split_keys ? key_first + p.keys_per_split : S);
     const int stages = (key_end - key_first + BKV - 1) / BKV;
 
     float4 rk[LOADS], rv[LOADS];
@@ -542,7 +563,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DPAD <= 64 
     }
 
     const float total = run_sum + __shfl_xor(run_sum, 32);
-    if constexpr (!CAUSAL) {
+    {
         if (p.key_splits > 1) {
             if (my_q < S) {
                 const size_t row = (static_cast<size_t>(split) * p.contexts + ctx) * S + my_q;
@@ -580,7 +601,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DPAD <= 64 
 // Combines the key splits of the fast kernel: with m = max over splits of their reference maxima,
 // out = Σ_s 2^((m_s − m)·exp_scale)·O_s / Σ_s 2^((m_s − m)·exp_scale)·l_s, splits added in order.  One thread per four
 // output values.
-__global__ __launch_bounds__(256) void attention_merge_splits_kernel(AttnArgs p, float exp_scale)
+__global__ __launch_bounds__(256) void attention_merge_splits_kernel(AttnArgs p, float exp_scale, int causal_r)
 {
     const int D = p.D;
     const int quads = D / 4;
@@ -591,9 +612,11 @@ __global__ __launch_bounds__(256) void attention_merge_splits_kernel(AttnArgs p,
     const int d = static_cast<int>(id % quads) * 4;
     // Eight splits at a time, all their loads requested before the first is used (a plain loop over the splits is a
     // chain of dependent memory round trips); splits past the end repeat the last one with weight zero.
-    const int last = p.key_splits - 1;
+    // causal: the query tile of this row has (tile / r) + 1 chunks of keys; the planes beyond were never written
+    const int splits = causal_r > 0 ? (static_cast<int>(row % static_cast<size_t>(p.S)) / kBQ) / causal_r + 1 : p.key_splits;
+    const int last = splits - 1;
     float top = -INFINITY;
-    for (int s0 = 0; s0 < p.key_splits; s0 += 8) {
+    for (int s0 = 0; s0 < splits; s0 += 8) {
         float m[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) m[j] = p.part_ml[(min(s0 + j, last) * rows + row) * 2];
@@ -603,7 +626,7 @@ __global__ __launch_bounds__(256) void attention_merge_splits_kernel(AttnArgs p,
     const float safe_top = top == -INFINITY ? 0.0f : top;
     float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
     float denom = 0.0f;
-    for (int s0 = 0; s0 < p.key_splits; s0 += 8) {
+    for (int s0 = 0; s0 < splits; s0 += 8) {
         float2 ml[8];
         float4 o[8];
 #pragma unroll
@@ -636,7 +659,35 @@ hipError_t launch_fast(AttnArgs args, hipStream_t stream)
     size_t blocks = static_cast<size_t>(args.contexts) * (CAUSAL ? (args.q_tiles + 1) / 2 : args.q_tiles);
     args.key_splits = 1;
     args.keys_per_split = args.S;
+    args.causal_items = 0;
     args.part_o = args.part_ml = nullptr;
+    int causal_r = 0;
+    if constexpr (CAUSAL) {
+        // Few contexts: pairs of query tiles leave most of the chip idle (8 contexts of 2048: 64 workgroups, slower than
+        // the non-causal call that does twice the work).  Split every tile's keys into chunks of 128·r instead, with the
+        // largest r that still gives about two workgroups per compute unit; all (tile, chunk) items then cost the same.
+        constexpr size_t kTargetBlocks = 512;
+        if (blocks * 2 <= kTargetBlocks && args.S >= 256) {
+            const size_t tiles = static_cast<size_t>(args.q_tiles);
+            auto items = [&](size_t r) {
+                size_t total = 0;
+                for (size_t j = 0; j < tiles; ++j) total += j / r + 1;
+                return total;
+            };
+            size_t r = tiles;
+            while (r > 1 && static_cast<size_t>(args.contexts) * items(r) < kTargetBlocks) --r;
+            const size_t per_context = items(r);
+            // (r == tiles would be one chunk per tile: nothing to merge, and the kernel tells the two forms apart by
+            // key_splits > 1 — such launches keep the pairing.)
+            if (r < tiles && static_cast<size_t>(args.contexts) * per_context > blocks) {
+                causal_r = static_cast<int>(r);
+                args.keys_per_split = static_cast<int>(r) * kBQ;
+                args.key_splits = static_cast<int>((tiles - 1) / r + 1);
+                args.causal_items = static_cast<int>(per_context);
+                blocks = static_cast<size_t>(args.contexts) * per_context;
+            }
+        }
+    }
     if constexpr (!CAUSAL) {
         // Few query tiles (the reference's own caller attends within one context: crates/st-nn/src/z_rba/attention.rs:586):
         // split the keys over workgroups until the launch offers about two workgroups per compute unit, 128 keys at least
@@ -650,18 +701,18 @@ hipError_t launch_fast(AttnArgs args, hipStream_t stream)
             args.keys_per_split = static_cast<int>(per);
             args.key_splits = static_cast<int>((static_cast<size_t>(args.S) + per - 1) / per);
         }
-        if (args.key_splits > 1) {
-            const size_t rows = static_cast<size_t>(args.contexts) * args.S;
-            const size_t o_bytes = static_cast<size_t>(args.key_splits) * rows * args.D * sizeof(float);
-            const size_t ml_bytes = static_cast<size_t>(args.key_splits) * rows * 2 * sizeof(float);
-            void *workspace = nullptr;
-            rc = stream_workspace(stream, o_bytes + ml_bytes, &workspace);
-            if (rc != hipSuccess) return rc;
-            args.part_o = static_cast<float *>(workspace);
-            args.part_ml = reinterpret_cast<float *>(static_cast<unsigned char *>(workspace) + o_bytes);
-            args.swizzle = 0;
-            blocks *= static_cast<size_t>(args.key_splits);
-        }
+        if (args.key_splits > 1) blocks *= static_cast<size_t>(args.key_splits);
+    }
+    if (args.key_splits > 1) {
+        const size_t rows = static_cast<size_t>(args.contexts) * args.S;
+        const size_t o_bytes = static_cast<size_t>(args.key_splits) * rows * args.D * sizeof(float);
+        const size_t ml_bytes = static_cast<size_t>(args.key_splits) * rows * 2 * sizeof(float);
+        void *workspace = nullptr;
+        rc = stream_workspace(stream, o_bytes + ml_bytes, &workspace);
+        if (rc != hipSuccess) return rc;
+        args.part_o = static_cast<float *>(workspace);
+        args.part_ml = reinterpret_cast<float *>(static_cast<unsigned char *>(workspace) + o_bytes);
+        args.swizzle = 0;
     }
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), lds_bytes, stream, args);
     rc = hipGetLastError();
@@ -669,7 +720,7 @@ hipError_t launch_fast(AttnArgs args, hipStream_t stream)
     const float scale_log2e = fmaxf(fabsf(args.scale) * kLog2e, 1e-30f);
     const size_t work = static_cast<size_t>(args.contexts) * args.S * (args.D / 4);
     hipLaunchKernelGGL(attention_merge_splits_kernel, dim3(static_cast<unsigned>((work + 255) / 256)), dim3(256), 0, stream, args,
-                       BIAS ? 1.0f : scale_log2e);
+                       BIAS ? 1.0f : scale_log2e, causal_r);
     return hipGetLastError();
 }
 
@@ -726,6 +777,7 @@ hipError_t launch_attention_f32(size_t contexts, size_t sequence, size_t head_di
     args.scale = scale;
     args.key_splits = 1;
     args.keys_per_split = args.S;
+    args.causal_items = 0;
     args.part_o = args.part_ml = nullptr;
     const bool bias = z_bias != nullptr || attn_bias != nullptr;
     auto aligned = [](const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; };

@@ -31,6 +31,8 @@ CASES = [
     (1, 70, 200, False, True), (5, 128, 64, True, True), (8, 384, 64, True, False),
     # causal query tiles are taken in pairs (j, last - j): five tiles (the middle one alone), four tiles, one XCD slice each
     (8, 600, 64, True, False), (16, 512, 32, True, False), (3, 1100, 64, True, False),
+    # 256 paired causal workgroups: too many to split the keys, one chunk per tile would be nothing to merge
+    (256, 256, 64, True, False), (255, 256, 32, True, False),
 ]
 
 
@@ -67,6 +69,28 @@ def test_keys_split_over_workgroups(hip, oracle, contexts, seq, dim, biased, sca
     assert_close(ones, np.ones_like(ones), F32_REL, F32_ABS, "row sums")
     again = run(hip, contexts, seq, dim, scale, q, k, v, zb, ab, False)
     assert (again == got).all(), "the splits are merged in a fixed order"
+
+
+@pytest.mark.parametrize("contexts,seq,dim,biased,scale", [
+    (8, 2048, 128, False, 0.0884), (4, 4096, 64, False, 0.125), (12, 1000, 64, False, 0.125), (1, 2048, 64, True, 0.125),
+    (3, 300, 32, True, -0.2), (2, 260, 64, False, 2.0), (5, 640, 16, False, 0.25)])
+def test_causal_keys_split_per_query_tile(hip, oracle, contexts, seq, dim, biased, scale):
+    """Causal calls with few contexts give every query tile one workgroup per chunk of its keys (tile j sees (j+1)*128
+    keys) instead of pairing tiles: rows early in a tile see none of a late chunk's keys (a partial row of weight zero),
+    the last chunk of a tile is cut by the diagonal, and the merge adds a different number of chunks per tile."""
+    rng = np.random.default_rng(contexts * 17 + seq + dim)
+    q, k, v = (rng.normal(size=contexts * seq * dim).astype(np.float32) for _ in range(3))
+    zb = rng.normal(size=contexts * seq).astype(np.float32) if biased else None
+    ab = rng.normal(0, 2.0, size=contexts * seq * seq).astype(np.float32) if biased else None
+    got = run(hip, contexts, seq, dim, scale, q, k, v, zb, ab, True)
+    want = oracle.attention_f32(contexts, seq, dim, scale, q, k, v, zb, ab, True, threads=8)
+    assert_close(got, want, F32_REL, F32_ABS, f"causal split {contexts}x{seq}x{dim} bias={biased} scale={scale}")
+    ones = run(hip, contexts, seq, dim, scale, q, k, np.ones_like(v), zb, ab, True)
+    assert_close(ones, np.ones_like(ones), F32_REL, F32_ABS, "row sums")
+    first = got.reshape(contexts, seq, dim)[:, 0, :]
+    assert_close(first, v.reshape(contexts, seq, dim)[:, 0, :], 1e-6, 1e-6, "causal row 0 is V[0]")
+    again = run(hip, contexts, seq, dim, scale, q, k, v, zb, ab, True)
+    assert (again == got).all()
 
 
 @pytest.mark.parametrize("contexts,seq,dim,biased", [(6, 300, 128, False), (2, 384, 128, True)])
