@@ -466,19 +466,21 @@ __device__ __forceinline__ void gemm_bf16_finish(const GemmBf16Args &p, int spli
 // -------------------------------------------------------------------------------------------------
 #define ST_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
 
-template <int BN, int WAVES>
+template <int BN, int WAVES, int BM = 256>
 __device__ __forceinline__ void gemm_bf16_packed_body(const GemmBf16Args &p)
 {
     static_assert(BN == 256 || BN == 128, "tile width");
     static_assert(WAVES == 8 || WAVES == 4, "wavefronts per workgroup");
-    constexpr int BM = 256, BK = 64;
+    static_assert(BM == 256 || (BM == 128 && BN == 128 && WAVES == 4), "tile height");
+    constexpr int BK = 64;
     constexpr int WTM = 2 * BM / WAVES;      // wavefront tile: WAVES/2 × 2 wavefronts
     constexpr int WTN = BN / 2;
     constexpr int TM = WTM / 32, TN = WTN / 32;  // 32×32 MFMA tiles per wavefront
-    constexpr int NA = 32 / WAVES;           // direct loads per wavefront and k-tile: A ...
+    constexpr int NA = BM / 8 / WAVES;       // direct loads per wavefront and k-tile: A ...
     constexpr int NB = BN / 8 / WAVES;       // ... and B (one load fills 8 rows of a stage)
-    constexpr int STAGE = 32768;             // bytes: 256 rows × 128 B, for A and for Bᵀ alike
-    constexpr int B_REGION = 3 * STAGE;      // [A0][A1][A2][B0][B1]
+    constexpr int A_STAGE = BM * 128;        // bytes: BM rows × 128 B
+    constexpr int B_STAGE = BM == 256 ? 32768 : BN * 128;  // (the 256-row forms give Bᵀ 256 rows' room whatever BN is)
+    constexpr int B_REGION = 3 * A_STAGE;    // [A0][A1][A2][B0][B1]
     constexpr int C_STRIDE = WTN + 4;        // floats, epilogue strip
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_bytes[];
 
@@ -526,12 +528,12 @@ __device__ __forceinline__ void gemm_bf16_packed_body(const GemmBf16Args &p)
     }
     const int lds_row_block = wave * 1024;  // wavefront-uniform part of every load's LDS destination
     auto load_a1 = [&](int stage, int r, unsigned k_off) {
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_ptr)(lds_bytes + stage * STAGE + r * (WAVES * 1024) + lds_row_block),
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_ptr)(lds_bytes + stage * A_STAGE + r * (WAVES * 1024) + lds_row_block),
                                                  16, a_off[r], k_off, 0, 0);
     };
     auto load_b1 = [&](int stage, int r, unsigned k_off) {
         __builtin_amdgcn_raw_ptr_buffer_load_lds(
-            rsrc_b, (lds_void_ptr)(lds_bytes + B_REGION + stage * STAGE + r * (WAVES * 1024) + lds_row_block), 16, b_off[r], k_off, 0, 0);
+            rsrc_b, (lds_void_ptr)(lds_bytes + B_REGION + stage * B_STAGE + r * (WAVES * 1024) + lds_row_block), 16, b_off[r], k_off, 0, 0);
     };
 
     f32x16 acc[TM][TN];
@@ -554,10 +556,10 @@ __device__ __forceinline__ void gemm_bf16_packed_body(const GemmBf16Args &p)
     }
     bf16x8 fa[2][TM], fb[2][TN];
     auto read_a = [&](int buf, int a_stage, int kk, int t) {
-        fa[buf][t] = *reinterpret_cast<const bf16x8 *>(lds_bytes + a_frag[kk ^ t] + a_stage * STAGE + t * 4096);
+        fa[buf][t] = *reinterpret_cast<const bf16x8 *>(lds_bytes + a_frag[kk ^ t] + a_stage * A_STAGE + t * 4096);
     };
     auto read_b = [&](int buf, int b_stage, int kk, int t) {
-        fb[buf][t] = *reinterpret_cast<const bf16x8 *>(lds_bytes + b_frag[kk ^ t] + b_stage * STAGE + t * 4096);
+        fb[buf][t] = *reinterpret_cast<const bf16x8 *>(lds_bytes + b_frag[kk ^ t] + b_stage * B_STAGE + t * 4096);
     };
     auto mfma = [&](int buf, int tm, int tn) {
         acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[buf][tn], fa[buf][tm], acc[tm][tn], 0, 0, 0);
@@ -1125,6 +1127,10 @@ __global__ __launch_bounds__(512) void gemm_bf16_256x128rm_kernel(GemmBf16Args p
 
 __global__ __launch_bounds__(512) void gemm_bf16_256w8_packed_kernel(GemmBf16Args p) { gemm_bf16_packed_body<256, 8>(p); }
 __global__ __launch_bounds__(512) void gemm_bf16_256x128w8_packed_kernel(GemmBf16Args p) { gemm_bf16_packed_body<128, 8>(p); }
+// 128×128 tiles, four wavefronts (64×64 of C each), 80 KB of LDS: two workgroups per compute unit.  Every MFMA needs a
+// fragment read of its own (the 256-row forms need three for four), so its main loop is LDS-bound; it serves launches
+// that would otherwise leave most compute units without a tile (1024³ is 16 tiles of 256×256).
+__global__ __launch_bounds__(256, 2) void gemm_bf16_128x128w4_packed_kernel(GemmBf16Args p) { gemm_bf16_packed_body<128, 4, 128>(p); }
 
 
 // -------------------------------------------------------------------------------------------------
@@ -1538,6 +1544,20 @@ __global__ __launch_bounds__(256) void transpose_u16_kernel(int rows, int cols, 
     }
 }
 
+// Few tiles and a long k (a batch of a hundred rows against a 4096² weight is 32 tiles of 64 k-tiles each): split k
+// over workgroups until the launch fills the chip — at least four k-tiles per split, and only as far as the partial
+// sums (written once, read once) stay below the operands' own bytes, or the split costs more than it spreads.
+size_t choose_k_splits(size_t m, size_t n, size_t k, size_t tiles)
+{
+    const size_t k_tiles = k / 64;
+    if (tiles * 2 > 256 || k_tiles < 8) return 1;
+    size_t splits = std::min<size_t>(256 / tiles, k_tiles / 4);
+    const size_t operand_bytes = (m * k + k * n) * 2;
+    const size_t plane_bytes = m * n * sizeof(float);
+    while (splits > 1 && splits * plane_bytes * 2 > operand_bytes) --splits;
+    return std::max<size_t>(splits, 1);
+}
+
 template <int BN>
 hipError_t launch_256(GemmBf16Args args, bool packed, hipStream_t stream, size_t workspace_offset)
 {
@@ -1545,17 +1565,8 @@ hipError_t launch_256(GemmBf16Args args, bool packed, hipStream_t stream, size_t
     args.tiles_n = args.N / BN;
     size_t tiles = static_cast<size_t>(args.tiles_m) * static_cast<size_t>(args.tiles_n);
     if (tiles > 0x7fffffffu) return hipErrorInvalidConfiguration;
-    // Few tiles and a long k (a batch of a hundred rows against a 4096² weight is 32 tiles of 64 k-tiles each): split k
-    // over workgroups until the launch fills the chip — at least four k-tiles per split, and only as far as the partial
-    // sums (written once, read once) stay below the operands' own bytes, or the split costs more than it spreads.
     const size_t k_tiles = static_cast<size_t>(args.K) / 64;
-    size_t splits = 1;
-    if (tiles * 2 <= 256 && k_tiles >= 8) {
-        splits = std::min<size_t>(256 / tiles, k_tiles / 4);
-        const size_t operand_bytes = (static_cast<size_t>(args.M) * args.K + static_cast<size_t>(args.K) * args.N) * 2;
-        const size_t plane_bytes = static_cast<size_t>(args.M) * args.N * sizeof(float);
-        while (splits > 1 && splits * plane_bytes * 2 > operand_bytes) --splits;
-    }
+    const size_t splits = choose_k_splits(args.M, args.N, args.K, tiles);
     SkinnyArgs reduce{};
     if (splits > 1) {
         args.tiles_per_split = static_cast<int>((k_tiles + splits - 1) / splits);
@@ -1592,6 +1603,23 @@ hipError_t launch_256(GemmBf16Args args, bool packed, hipStream_t stream, size_t
     const size_t plane = static_cast<size_t>(args.M) * args.N;
     hipLaunchKernelGGL(gemm_bf16_skinny_reduce_kernel, dim3(static_cast<unsigned>((plane + 255) / 256)), dim3(256), 0, stream,
                        reduce);
+    return hipGetLastError();
+}
+
+hipError_t launch_128(GemmBf16Args args, hipStream_t stream)
+{
+    args.tiles_m = (args.M + 127) / 128;
+    args.tiles_n = args.N / 128;
+    const size_t tiles = static_cast<size_t>(args.tiles_m) * static_cast<size_t>(args.tiles_n);
+    if (tiles > 0x7fffffffu) return hipErrorInvalidConfiguration;
+    args.swizzle = (tiles % 8 == 0) ? 1 : 0;
+    constexpr size_t lds_bytes = 5 * 16384;  // three A stages + two B stages of 128 rows
+    static_assert(lds_bytes >= 4 * 32 * (64 + 4) * sizeof(float), "four epilogue strips must fit in the stage buffers");
+    auto kernel = gemm_bf16_128x128w4_packed_kernel;
+    hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
+    if (rc != hipSuccess) return rc;
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(tiles)), dim3(256), lds_bytes, stream, args);
     return hipGetLastError();
 }
 
@@ -1706,8 +1734,14 @@ hipError_t launch_gemm_bf16(size_t m, size_t n, size_t k, const uint16_t *lhs, c
         // rounds that the 256-wide tiling would leave partly empty (or when N is not a multiple of 256).
         auto fill = [](size_t tiles) { return static_cast<double>(tiles) / static_cast<double>((tiles + 255) / 256 * 256); };
         const size_t row_tiles = (m + 255) / 256;
-        if (n % 256 != 0 || fill(row_tiles * (n / 128)) > 1.15 * fill(row_tiles * (n / 256)))
-            return launch_256<128>(args, rhs_packed, stream, workspace_offset);
+        const bool narrow = n % 256 != 0 || fill(row_tiles * (n / 128)) > 1.15 * fill(row_tiles * (n / 256));
+        // A packed B whose 256-row tiling would leave most compute units without a tile, and whose k is not worth
+        // splitting: 128×128 tiles, two workgroups per compute unit (1024³: 16 tiles of 256×256, 64 of 128×128).
+        const size_t tiles_256 = row_tiles * (n / (narrow ? 128 : 256));
+        const size_t tiles_128 = ((m + 127) / 128) * (n / 128);
+        if (rhs_packed && tiles_256 < 192 && tiles_128 >= 2 * tiles_256 && choose_k_splits(m, n, k, tiles_256) == 1)
+            return launch_128(args, stream);
+        if (narrow) return launch_256<128>(args, rhs_packed, stream, workspace_offset);
         return launch_256<256>(args, rhs_packed, stream, workspace_offset);
     }
     return launch_tile<128, 128, 32>(args, vec, stream);
