@@ -905,16 +905,18 @@ __global__ __launch_bounds__(512) void gemm_bf16_rowcomplete_kernel(RowLnArgs q)
 // are issued in sub-step 2 of tile t and consumed in sub-step 1 of tile t+1; all of it — 4 direct loads of A,
 // KR loads, 2·KR permutes and 4 LDS writes per wavefront and k-tile — rides in the slots behind the MFMAs.
 // -------------------------------------------------------------------------------------------------
-template <int BN>
+template <int BN, int BM = 256>
 __device__ __forceinline__ void gemm_bf16_rowmajor_body(const GemmBf16Args &p)
 {
     static_assert(BN == 256 || BN == 128, "tile width");
-    constexpr int BM = 256, BK = 64;
+    static_assert(BM == 256 || (BM == 128 && BN == 128), "tile height");
+    constexpr int BK = 64;
+    constexpr int WAVES = BM / 32;           // a wavefront owns 64 rows × BN/2 columns of C
     constexpr int WTN = BN / 2;
     constexpr int TN = WTN / 32;
     constexpr int SLOTS = 2 * TN;            // MFMAs (and memory slots) per sub-step
-    constexpr int KR = BN / 32;              // k-rows of B per thread: 512 threads × KR × 4 columns = 64 × BN
-    constexpr int STAGE = 32768;
+    constexpr int KR = BN / (4 * WAVES);     // k-rows of B per thread: threads × KR × 4 columns = 64 × BN
+    constexpr int STAGE = BM * 128;          // bytes per stage of A; a stage of B (BN × 128) never needs more
     constexpr int B_REGION = 3 * STAGE;      // [A0][A1][A2][B0][B1]
     constexpr int C_STRIDE = WTN + 4;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_bytes[];
@@ -946,7 +948,7 @@ __device__ __forceinline__ void gemm_bf16_rowmajor_body(const GemmBf16Args &p)
     const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint16_t *>(p.B), 0, static_cast<int>(static_cast<unsigned>(K) * static_cast<unsigned>(N) * 2u), 0x00020000);
 
-    // A: as in the packed kernel (instruction r of wavefront w fills rows r*64 + w*8 .. +7 of a stage).
+    // A: as in the packed kernel (instruction r of wavefront w fills rows r*8*WAVES + w*8 .. +7 of a stage).
     unsigned a_off[4];
     {
         const int row_in = wave * 8 + (lane >> 3);
@@ -954,13 +956,13 @@ __device__ __forceinline__ void gemm_bf16_rowmajor_body(const GemmBf16Args &p)
         const unsigned k_first = static_cast<unsigned>(tile0) * BK;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const int chunk = ((lane & 7) ^ sw_base ^ ((4 * r) & 7)) & 7;
-            a_off[r] = (static_cast<unsigned>(m0 + r * 64 + row_in) * K + k_first + chunk * 8) * 2u;
+            const int chunk = ((lane & 7) ^ sw_base ^ ((r * WAVES / 2) & 7)) & 7;
+            a_off[r] = (static_cast<unsigned>(m0 + r * 8 * WAVES + row_in) * K + k_first + chunk * 8) * 2u;
         }
     }
     const int lds_row_block = wave * 1024;
     auto load_a1 = [&](int stage, int r, unsigned k_off) {
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_ptr)(lds_bytes + stage * STAGE + r * 8192 + lds_row_block), 16,
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_ptr)(lds_bytes + stage * STAGE + r * (1024 * WAVES) + lds_row_block), 16,
                                                  a_off[r], k_off, 0, 0);
     };
 
@@ -1074,7 +1076,14 @@ __device__ __forceinline__ void gemm_bf16_rowmajor_body(const GemmBf16Args &p)
         });
         // sub-step 2: B(t+2) into the registers
         substep(0, true, a_stage, b_stage, 3, [&](int slot) {
-            if (LOAD && slot < KR) load_b1(slot, static_cast<unsigned>(t + 2));
+            if constexpr (KR > SLOTS) {
+                if (LOAD) {
+#pragma unroll
+                    for (int j = 0; j < KR / SLOTS; ++j) load_b1(slot * (KR / SLOTS) + j, static_cast<unsigned>(t + 2));
+                }
+            } else {
+                if (LOAD && slot < KR) load_b1(slot, static_cast<unsigned>(t + 2));
+            }
         });
         if constexpr (MORE) {
             if constexpr (LOAD) ST_WAIT_VMCNT(4 + KR); else ST_WAIT_VMCNT(0);
@@ -1124,6 +1133,7 @@ __device__ __forceinline__ void gemm_bf16_rowmajor_body(const GemmBf16Args &p)
 
 __global__ __launch_bounds__(512) void gemm_bf16_256rm_kernel(GemmBf16Args p) { gemm_bf16_rowmajor_body<256>(p); }
 __global__ __launch_bounds__(512) void gemm_bf16_256x128rm_kernel(GemmBf16Args p) { gemm_bf16_rowmajor_body<128>(p); }
+__global__ __launch_bounds__(256, 2) void gemm_bf16_128x128w4_rm_kernel(GemmBf16Args p) { gemm_bf16_rowmajor_body<128, 128>(p); }
 
 __global__ __launch_bounds__(512) void gemm_bf16_256w8_packed_kernel(GemmBf16Args p) { gemm_bf16_packed_body<256, 8>(p); }
 __global__ __launch_bounds__(512) void gemm_bf16_256x128w8_packed_kernel(GemmBf16Args p) { gemm_bf16_packed_body<128, 8>(p); }
@@ -1606,7 +1616,7 @@ hipError_t launch_256(GemmBf16Args args, bool packed, hipStream_t stream, size_t
     return hipGetLastError();
 }
 
-hipError_t launch_128(GemmBf16Args args, hipStream_t stream)
+hipError_t launch_128(GemmBf16Args args, bool packed, hipStream_t stream)
 {
     args.tiles_m = (args.M + 127) / 128;
     args.tiles_n = args.N / 128;
@@ -1615,7 +1625,7 @@ hipError_t launch_128(GemmBf16Args args, hipStream_t stream)
     args.swizzle = (tiles % 8 == 0) ? 1 : 0;
     constexpr size_t lds_bytes = 5 * 16384;  // three A stages + two B stages of 128 rows
     static_assert(lds_bytes >= 4 * 32 * (64 + 4) * sizeof(float), "four epilogue strips must fit in the stage buffers");
-    auto kernel = gemm_bf16_128x128w4_packed_kernel;
+    auto kernel = packed ? gemm_bf16_128x128w4_packed_kernel : gemm_bf16_128x128w4_rm_kernel;
     hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
     if (rc != hipSuccess) return rc;
@@ -1735,12 +1745,12 @@ hipError_t launch_gemm_bf16(size_t m, size_t n, size_t k, const uint16_t *lhs, c
         auto fill = [](size_t tiles) { return static_cast<double>(tiles) / static_cast<double>((tiles + 255) / 256 * 256); };
         const size_t row_tiles = (m + 255) / 256;
         const bool narrow = n % 256 != 0 || fill(row_tiles * (n / 128)) > 1.15 * fill(row_tiles * (n / 256));
-        // A packed B whose 256-row tiling would leave most compute units without a tile, and whose k is not worth
-        // splitting: 128×128 tiles, two workgroups per compute unit (1024³: 16 tiles of 256×256, 64 of 128×128).
+        // A 256-row tiling that would leave most compute units without a tile, and a k not worth splitting: 128×128
+        // tiles, two workgroups per compute unit (1024³: 16 tiles of 256×256, 64 of 128×128).
         const size_t tiles_256 = row_tiles * (n / (narrow ? 128 : 256));
         const size_t tiles_128 = ((m + 127) / 128) * (n / 128);
-        if (rhs_packed && tiles_256 < 192 && tiles_128 >= 2 * tiles_256 && choose_k_splits(m, n, k, tiles_256) == 1)
-            return launch_128(args, stream);
+        if (tiles_256 < 192 && tiles_128 >= 2 * tiles_256 && choose_k_splits(m, n, k, tiles_256) == 1)
+            return launch_128(args, rhs_packed, stream);
         if (narrow) return launch_256<128>(args, rhs_packed, stream, workspace_offset);
         return launch_256<256>(args, rhs_packed, stream, workspace_offset);
     }

@@ -319,36 +319,43 @@ def test_few_tiles_with_a_long_k_split_k(hip, oracle, m, n, k):
 
 @pytest.mark.parametrize("m,n,k", [(1024, 1024, 1024), (300, 1024, 512), (130, 2048, 256), (1000, 1280, 192), (2048, 2048, 64),
                                    (513, 384, 448)])
-def test_prepacked_mid_size_128_row_tiles(hip, oracle, m, n, k):
-    """A packed B whose 256-row tiling leaves most compute units idle runs 128×128 tiles, two workgroups per compute
-    unit: plain product against the oracle (ragged last row tiles included), every activation with bias and residual
-    into both output types, and bf16-only output."""
+def test_mid_size_128_row_tiles(hip, oracle, m, n, k):
+    """A launch whose 256-row tiling leaves most compute units idle runs 128×128 tiles, two workgroups per compute
+    unit, for either layout of B: plain product against the oracle (ragged last row tiles included), every activation
+    with bias and residual into both output types, bf16-only output, and the same bits from both layouts."""
     from spiraltorch_amd import inputs
     rng = np.random.default_rng(5 * m + 3 * n + k)
     a, b = bf16_pair(rng, m, n, k, std=0.5)
     bias = rng.normal(size=n).astype(np.float32)
     res = rng.normal(size=m * n).astype(np.float32)
-    d = {name: hip.DeviceBuffer.from_array(v) for name, v in (("a", a), ("bias", bias), ("res", res))}
+    d = {name: hip.DeviceBuffer.from_array(v) for name, v in (("a", a), ("b", b), ("bias", bias), ("res", res))}
     d_packed = hip.DeviceBuffer.from_array(np.ascontiguousarray(b.reshape(k, n).T))
     out = hip.DeviceBuffer(m * n * 4)
     d16 = hip.DeviceBuffer(m * n * 2)
     base = oracle.gemm_bf16_f32acc(m, n, k, a, b, threads=8)
-    hip.gemm_bf16_prepacked_bias_act_dev(m, n, k, 0, d["a"], d_packed, None, None, out, None)
-    hip.device_synchronize()
-    check(out.to_array(np.float32, m * n), base, f"128-row tiles {m}x{n}x{k}")
     pre = (base.astype(np.float64).reshape(m, n) + bias).ravel() + res
-    for activation, want in ((0, pre), (1, np.maximum(pre, 0.0)),
-                             (2, 0.5 * pre * (1.0 + np.tanh(0.7978846 * (pre + 0.044715 * pre ** 3))))):
-        hip.gemm_bf16_prepacked_bias_act_dev(m, n, k, activation, d["a"], d_packed, d["bias"], d["res"], out, d16)
-        hip.device_synchronize()
-        got32 = out.to_array(np.float32, m * n)
-        assert_close(got32, want, 1e-4, 2e-5 * max(1.0, float(np.abs(base).max())), f"activation {activation}")
-        assert (d16.to_array(np.uint16, m * n) == inputs.to_bf16(got32)).all()
-    hip.gemm_bf16_prepacked_bias_act_dev(m, n, k, 1, d["a"], d_packed, d["bias"], None, None, d16)
-    hip.device_synchronize()
-    want16 = np.maximum((base.astype(np.float64).reshape(m, n) + bias).ravel(), 0.0)
-    got16 = inputs.from_bf16(d16.to_array(np.uint16, m * n))
-    assert_close(got16, want16, 2 ** -7, 2e-5 * max(1.0, float(np.abs(base).max())), "bf16-only output")
+    bits = {}
+    for packed in (True, False):
+        def run(activation, bias_, res_, out32, out16):
+            if packed:
+                hip.gemm_bf16_prepacked_bias_act_dev(m, n, k, activation, d["a"], d_packed, bias_, res_, out32, out16)
+            else:
+                hip.gemm_bf16_bias_act_dev(m, n, k, activation, d["a"], d["b"], bias_, res_, out32, out16)
+            hip.device_synchronize()
+        run(0, None, None, out, None)
+        bits[packed] = out.to_array(np.float32, m * n)
+        check(bits[packed], base, f"128-row tiles {m}x{n}x{k} packed={packed}")
+        for activation, want in ((0, pre), (1, np.maximum(pre, 0.0)),
+                                 (2, 0.5 * pre * (1.0 + np.tanh(0.7978846 * (pre + 0.044715 * pre ** 3))))):
+            run(activation, d["bias"], d["res"], out, d16)
+            got32 = out.to_array(np.float32, m * n)
+            assert_close(got32, want, 1e-4, 2e-5 * max(1.0, float(np.abs(base).max())), f"activation {activation}")
+            assert (d16.to_array(np.uint16, m * n) == inputs.to_bf16(got32)).all()
+        run(1, d["bias"], None, None, d16)
+        want16 = np.maximum((base.astype(np.float64).reshape(m, n) + bias).ravel(), 0.0)
+        got16 = inputs.from_bf16(d16.to_array(np.uint16, m * n))
+        assert_close(got16, want16, 2 ** -7, 2e-5 * max(1.0, float(np.abs(base).max())), "bf16-only output")
+    assert (bits[True] == bits[False]).all(), "both layouts accumulate in the same order"
 
 
 def test_config4_4096_cubed_prepacked(hip, oracle):
