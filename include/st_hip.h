@@ -231,9 +231,9 @@ int st_hip_gemm_bf16_prepacked_bias_act_dev(size_t m, size_t n, size_t k, int ac
  * crates/st-tensor/src/pure.rs:4008-4058): out_f32 = (lhs·rhs + bias) + residual, the rows the next residual add needs,
  * and out_ln_bf16 = layer_norm(out_f32; gamma, beta, epsilon) rounded nearest-even to bf16, the operand of the next
  * projection.  bf16 lhs (m×k), rhs prepacked as its (n, k) transpose, f32 accumulation; bias (n) and residual (m×n)
- * may be NULL, gamma and beta (n) may not.  n = 512 with m > 64, k a multiple of 64 up to 1024 and 16-byte aligned
- * buffers is a single kernel whose workgroups own whole rows; any other shape runs the GEMM and the layer-norm kernel
- * one after the other.  The single kernel adds the k products and a row's statistics in the order the tiled GEMM and
+ * may be NULL, gamma and beta (n) may not.  n = 512 with m > 64, k a multiple of 64 up to 1024, 16-byte aligned
+ * buffers and no split of k in the plain GEMM's launch plan (few rows with a long k are split there) is a single
+ * kernel whose workgroups own whole rows; any other shape runs the GEMM and the layer-norm kernel one after the other.  The single kernel adds the k products and a row's statistics in the order the tiled GEMM and
  * the layer-norm kernel use, so for its shapes it returns, bit for bit, what those two return. */
 int st_hip_gemm_bf16_prepacked_residual_layer_norm_dev(size_t m, size_t n, size_t k, const uint16_t *lhs,
                                                       const uint16_t *packed_rhs, const float *bias,

@@ -1568,6 +1568,26 @@ size_t choose_k_splits(size_t m, size_t n, size_t k, size_t tiles)
     return std::max<size_t>(splits, 1);
 }
 
+// The 256-row tiling of an m×n×k product (n a multiple of 128): tile width, tile count and k-splits.
+// One workgroup per compute unit at a time: the launch runs in rounds of 256 tiles.  Halving the tile width costs
+// about 15 % in the main loop (more LDS traffic per flop), so do it only when it fills rounds that the 256-wide
+// tiling would leave partly empty (or when n is not a multiple of 256).
+struct TilePlan {
+    bool narrow;
+    size_t tiles;
+    size_t k_splits;
+};
+TilePlan plan_tiles(size_t m, size_t n, size_t k)
+{
+    auto fill = [](size_t tiles) { return static_cast<double>(tiles) / static_cast<double>((tiles + 255) / 256 * 256); };
+    const size_t row_tiles = (m + 255) / 256;
+    TilePlan plan;
+    plan.narrow = n % 256 != 0 || fill(row_tiles * (n / 128)) > 1.15 * fill(row_tiles * (n / 256));
+    plan.tiles = row_tiles * (n / (plan.narrow ? 128 : 256));
+    plan.k_splits = choose_k_splits(m, n, k, plan.tiles);
+    return plan;
+}
+
 template <int BN>
 hipError_t launch_256(GemmBf16Args args, bool packed, hipStream_t stream, size_t workspace_offset)
 {
@@ -1739,17 +1759,13 @@ hipError_t launch_gemm_bf16(size_t m, size_t n, size_t k, const uint16_t *lhs, c
     // The 256-row kernels serve every shape they can address: measured against the 128×128 tile kernel they win
     // from a single tile up (256×256×4096: 58 vs 74 µs; 1024³: 21 vs 30 µs; 16384×256×512: 17 vs 24 µs).
     if (fits_256) {
-        // One workgroup per compute unit at a time: the launch runs in rounds of 256 tiles.  Halving the tile
-        // width costs about 15 % in the main loop (more LDS traffic per flop), so do it only when it fills
-        // rounds that the 256-wide tiling would leave partly empty (or when N is not a multiple of 256).
-        auto fill = [](size_t tiles) { return static_cast<double>(tiles) / static_cast<double>((tiles + 255) / 256 * 256); };
-        const size_t row_tiles = (m + 255) / 256;
-        const bool narrow = n % 256 != 0 || fill(row_tiles * (n / 128)) > 1.15 * fill(row_tiles * (n / 256));
+        const TilePlan plan = plan_tiles(m, n, k);
+        const bool narrow = plan.narrow;
         // A 256-row tiling that would leave most compute units without a tile, and a k not worth splitting: 128×128
         // tiles, two workgroups per compute unit (1024³: 16 tiles of 256×256, 64 of 128×128).
-        const size_t tiles_256 = row_tiles * (n / (narrow ? 128 : 256));
+        const size_t tiles_256 = plan.tiles;
         const size_t tiles_128 = ((m + 127) / 128) * (n / 128);
-        if (tiles_256 < 192 && tiles_128 >= 2 * tiles_256 && choose_k_splits(m, n, k, tiles_256) == 1)
+        if (tiles_256 < 192 && tiles_128 >= 2 * tiles_256 && plan.k_splits == 1)
             return launch_128(args, rhs_packed, stream);
         if (narrow) return launch_256<128>(args, rhs_packed, stream, workspace_offset);
         return launch_256<256>(args, rhs_packed, stream, workspace_offset);
@@ -1771,8 +1787,9 @@ hipError_t launch_gemm_bf16_residual_layer_norm(size_t m, size_t n, size_t k, co
     // Measured at m = 16384 (one 64-row workgroup per compute unit): 27.3 µs against 18.2 + 10.2 µs for the two kernels at
     // k = 512, 51.2 against 37.9 + 10.1 µs at k = 2048 — a 64-row tile streams the whole of B through every compute unit,
     // which costs more than the saved pass over the rows once k is long.
-    // (m <= 64 stays with the GEMM dispatcher, which splits k over the chip for such shapes.)
-    if (n == 512 && m > 64 && k >= 64 && k % 64 == 0 && k <= 1024 && fits_buffer && aligned) {
+    // (m <= 64 stays with the GEMM dispatcher, which splits k over the chip for such shapes, and so does every shape of
+    // few row tiles and a long k that the dispatcher would split: the split sums add up in another order.)
+    if (n == 512 && m > 64 && k >= 64 && k % 64 == 0 && k <= 1024 && fits_buffer && aligned && plan_tiles(m, n, k).k_splits == 1) {
         RowLnArgs row;
         row.g.A = lhs;
         row.g.B = packed_rhs;

@@ -48,63 +48,84 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(int rows, int cols, con
 
 // Same, for rows of at most 2048 values with 16-byte aligned rows: the row is read once, 128 bits per lane, and
 // stays in registers between the statistics and the normalisation.
-template <int CHUNKS>
+template <int CHUNKS, int ROWS>
 __global__ __launch_bounds__(256) void layer_norm_vec_kernel(int rows, int cols, const float *x, const float *residual,
                                                              const float *gamma, const float *beta, float epsilon,
                                                              float *out_f32, uint16_t *out_bf16)
 {
+    // A wavefront takes ROWS consecutive rows and has all their loads in flight before the first reduction: with one
+    // short row per wavefront the launch is bound by the latency of that one load, not by bandwidth.
     const int lane = threadIdx.x & 63;
-    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (row >= rows) return;
-    const size_t offset = static_cast<size_t>(row) * cols;
-    float4 v[CHUNKS];
-    float sum = 0.0f, sumsq = 0.0f;
+    const int row0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * ROWS;
+    if (row0 >= rows) return;
+    float4 v[ROWS][CHUNKS];
 #pragma unroll
-    for (int i = 0; i < CHUNKS; ++i) {
-        const int c = (lane + 64 * i) * 4;
-        v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (c < cols) {
-            v[i] = *reinterpret_cast<const float4 *>(x + offset + c);
-            if (residual) {
-                const float4 r = *reinterpret_cast<const float4 *>(residual + offset + c);
-                v[i].x += r.x; v[i].y += r.y; v[i].z += r.z; v[i].w += r.w;
+    for (int r = 0; r < ROWS; ++r) {
+        const size_t offset = static_cast<size_t>(row0 + r) * cols;
+#pragma unroll
+        for (int i = 0; i < CHUNKS; ++i) {
+            const int c = (lane + 64 * i) * 4;
+            v[r][i] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (c < cols && row0 + r < rows) {
+                v[r][i] = *reinterpret_cast<const float4 *>(x + offset + c);
+                if (residual) {
+                    const float4 q = *reinterpret_cast<const float4 *>(residual + offset + c);
+                    v[r][i].x += q.x; v[r][i].y += q.y; v[r][i].z += q.z; v[r][i].w += q.w;
+                }
             }
         }
-        sum += sum4(v[i]);
-        sumsq += sumsq4(v[i]);
     }
-    sum = wave_sum(sum);
-    sumsq = wave_sum(sumsq);
-    const float cols_f = static_cast<float>(cols);
-    const float mean = sum / cols_f;
-    const float var = fmaxf(sumsq / cols_f - mean * mean, 0.0f);
-    const float denom = sqrtf(var + epsilon);
-    // (v - mean) / denom for every element, with one real division per row: the product with the correctly rounded
-    // reciprocal, corrected once by its exact remainder (two fused multiply-adds), is the correctly rounded quotient
-    // again, i.e. bit for bit what the division gives; only the last bit matters here, because it decides some of
-    // the bf16 roundings downstream and the decoder is compared with a CPU stack that divides.
-    const float inv = 1.0f / denom;
-    auto quotient = [&](float a) {
-        const float q = a * inv;
-        return fmaf(fmaf(-q, denom, a), inv, q);
-    };
+    float4 g[CHUNKS], b[CHUNKS];
 #pragma unroll
     for (int i = 0; i < CHUNKS; ++i) {
         const int c = (lane + 64 * i) * 4;
-        if (c >= cols) continue;
-        const float4 g = *reinterpret_cast<const float4 *>(gamma + c);
-        const float4 b = *reinterpret_cast<const float4 *>(beta + c);
-        float4 o;
-        o.x = quotient(v[i].x - mean) * g.x + b.x;
-        o.y = quotient(v[i].y - mean) * g.y + b.y;
-        o.z = quotient(v[i].z - mean) * g.z + b.z;
-        o.w = quotient(v[i].w - mean) * g.w + b.w;
-        if (out_f32) *reinterpret_cast<float4 *>(out_f32 + offset + c) = o;
-        if (out_bf16) {
-            uint2 packed;
-            packed.x = pack_bf16x2_rne(o.x, o.y);
-            packed.y = pack_bf16x2_rne(o.z, o.w);
-            *reinterpret_cast<uint2 *>(out_bf16 + offset + c) = packed;
+        g[i] = b[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (c < cols) {
+            g[i] = *reinterpret_cast<const float4 *>(gamma + c);
+            b[i] = *reinterpret_cast<const float4 *>(beta + c);
+        }
+    }
+    const float cols_f = static_cast<float>(cols);
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+        if (row0 + r >= rows) break;
+        const size_t offset = static_cast<size_t>(row0 + r) * cols;
+        float sum = 0.0f, sumsq = 0.0f;
+#pragma unroll
+        for (int i = 0; i < CHUNKS; ++i) {
+            sum += sum4(v[r][i]);
+            sumsq += sumsq4(v[r][i]);
+        }
+        sum = wave_sum(sum);
+        sumsq = wave_sum(sumsq);
+        const float mean = sum / cols_f;
+        const float var = fmaxf(sumsq / cols_f - mean * mean, 0.0f);
+        const float denom = sqrtf(var + epsilon);
+        // (v - mean) / denom for every element, with one real division per row: the product with the correctly rounded
+        // reciprocal, corrected once by its exact remainder (two fused multiply-adds), is the correctly rounded quotient
+        // again, i.e. bit for bit what the division gives; only the last bit matters here, because it decides some of
+        // the bf16 roundings downstream and the decoder is compared with a CPU stack that divides.
+        const float inv = 1.0f / denom;
+        auto quotient = [&](float a) {
+            const float q = a * inv;
+            return fmaf(fmaf(-q, denom, a), inv, q);
+        };
+#pragma unroll
+        for (int i = 0; i < CHUNKS; ++i) {
+            const int c = (lane + 64 * i) * 4;
+            if (c >= cols) continue;
+            float4 o;
+            o.x = quotient(v[r][i].x - mean) * g[i].x + b[i].x;
+            o.y = quotient(v[r][i].y - mean) * g[i].y + b[i].y;
+            o.z = quotient(v[r][i].z - mean) * g[i].z + b[i].z;
+            o.w = quotient(v[r][i].w - mean) * g[i].w + b[i].w;
+            if (out_f32) *reinterpret_cast<float4 *>(out_f32 + offset + c) = o;
+            if (out_bf16) {
+                uint2 packed;
+                packed.x = pack_bf16x2_rne(o.x, o.y);
+                packed.y = pack_bf16x2_rne(o.z, o.w);
+                *reinterpret_cast<uint2 *>(out_bf16 + offset + c) = packed;
+            }
         }
     }
 }
@@ -531,15 +552,24 @@ hipError_t launch_layer_norm_f32(size_t rows, size_t cols, const float *x, const
     const bool vec = cols % 4 == 0 && cols <= 2048 && aligned(x, 16) && aligned(residual, 16) && aligned(gamma, 16) &&
                      aligned(beta, 16) && aligned(out_f32, 16) && aligned(out_bf16, 8);
     const int r = static_cast<int>(rows), c = static_cast<int>(cols);
-    if (vec && cols <= 512)
-        hipLaunchKernelGGL(layer_norm_vec_kernel<2>, grid, block, 0, stream, r, c, x, residual, gamma, beta, epsilon, out_f32,
-                           out_bf16);
+    // Two rows per wavefront once there are enough rows to fill the chip that way.
+    const bool two_rows = rows >= 8192;
+    const dim3 grid2(static_cast<unsigned>((rows + 7) / 8));
+    if (vec && cols <= 512 && two_rows)
+        hipLaunchKernelGGL((layer_norm_vec_kernel<2, 2>), grid2, block, 0, stream, r, c, x, residual, gamma, beta, epsilon,
+                           out_f32, out_bf16);
+    else if (vec && cols <= 512)
+        hipLaunchKernelGGL((layer_norm_vec_kernel<2, 1>), grid, block, 0, stream, r, c, x, residual, gamma, beta, epsilon,
+                           out_f32, out_bf16);
+    else if (vec && cols <= 1024 && two_rows)
+        hipLaunchKernelGGL((layer_norm_vec_kernel<4, 2>), grid2, block, 0, stream, r, c, x, residual, gamma, beta, epsilon,
+                           out_f32, out_bf16);
     else if (vec && cols <= 1024)
-        hipLaunchKernelGGL(layer_norm_vec_kernel<4>, grid, block, 0, stream, r, c, x, residual, gamma, beta, epsilon, out_f32,
-                           out_bf16);
+        hipLaunchKernelGGL((layer_norm_vec_kernel<4, 1>), grid, block, 0, stream, r, c, x, residual, gamma, beta, epsilon,
+                           out_f32, out_bf16);
     else if (vec)
-        hipLaunchKernelGGL(layer_norm_vec_kernel<8>, grid, block, 0, stream, r, c, x, residual, gamma, beta, epsilon, out_f32,
-                           out_bf16);
+        hipLaunchKernelGGL((layer_norm_vec_kernel<8, 1>), grid, block, 0, stream, r, c, x, residual, gamma, beta, epsilon,
+                           out_f32, out_bf16);
     else
         hipLaunchKernelGGL(layer_norm_kernel, grid, block, 0, stream, r, c, x, residual, gamma, beta, epsilon, out_f32,
                            out_bf16);

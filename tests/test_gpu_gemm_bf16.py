@@ -229,7 +229,7 @@ def test_skinny_prepacked_single_launch(hip, oracle, m, n, k):
         assert (d16.to_array(np.uint16, m * n) == inputs.to_bf16(got32)).all()
 
 
-@pytest.mark.parametrize("m,n,k", [(65, 512, 64), (1000, 512, 512), (16384, 512, 192), (130, 512, 2048), (1, 512, 128),
+@pytest.mark.parametrize("m,n,k", [(65, 512, 64), (1000, 512, 512), (16384, 512, 192), (130, 512, 2048), (1, 512, 128), (65, 512, 1024), (300, 512, 1024),
                                    (64, 512, 512), (256, 512, 1024),
                                    # other widths: the GEMM and the layer-norm kernel one after the other
                                    (300, 384, 128), (33, 512, 96), (70, 1024, 256)])
