@@ -358,6 +358,36 @@ def test_mid_size_128_row_tiles(hip, oracle, m, n, k):
     assert (bits[True] == bits[False]).all(), "both layouts accumulate in the same order"
 
 
+@pytest.mark.parametrize("m,n,k,activation", [(16384, 1536, 512, 0), (16384, 2048, 512, 2), (8192, 4352, 64, 1), (2304, 3968, 128, 2),
+                                              (4096, 2176, 320, 0), (512, 66048, 192, 1)])
+def test_prepacked_bf16_output_over_several_rounds_of_tiles(hip, oracle, m, n, k, activation):
+    """More 256×128 tiles than compute units, bf16 the only output, M a multiple of 256: the persistent kernel (a ninth
+    wavefront loads, eight compute and store).  Bit for bit the bf16 rounding of what the same call returns when it
+    also asks for the f32 output (which takes the one-tile-per-workgroup kernel), and sampled rows against the oracle."""
+    from spiraltorch_amd import inputs
+    rng = np.random.default_rng(m + 3 * n + 7 * k)
+    a, b = bf16_pair(rng, m, n, k, std=0.5)
+    bias = rng.normal(size=n).astype(np.float32)
+    d_a, d_bias = hip.DeviceBuffer.from_array(a), hip.DeviceBuffer.from_array(bias)
+    d_packed = hip.DeviceBuffer.from_array(np.ascontiguousarray(b.reshape(k, n).T))
+    d32, d16, d16_ref = hip.DeviceBuffer(m * n * 4), hip.DeviceBuffer(m * n * 2), hip.DeviceBuffer(m * n * 2)
+    for use_bias in (True, False):
+        hip.gemm_bf16_prepacked_bias_act_dev(m, n, k, activation, d_a, d_packed, d_bias if use_bias else None, None, d32, d16_ref)
+        hip.gemm_bf16_prepacked_bias_act_dev(m, n, k, activation, d_a, d_packed, d_bias if use_bias else None, None, None, d16)
+        hip.device_synchronize()
+        got = d16.to_array(np.uint16, m * n)
+        assert (got == d16_ref.to_array(np.uint16, m * n)).all(), f"bias={use_bias}"
+    rows = sorted(set([0, 1, 255, 256, m // 2 + 3, m - 257, m - 1]))
+    base = oracle.gemm_bf16_f32acc(len(rows), n, k, a.reshape(m, k)[rows].ravel(), b, threads=8).astype(np.float64).reshape(len(rows), n)
+    want = base  # the last call ran without a bias
+    if activation == 1:
+        want = np.maximum(want, 0.0)
+    elif activation == 2:
+        want = 0.5 * want * (1.0 + np.tanh(0.7978846 * (want + 0.044715 * want ** 3)))
+    got_rows = inputs.from_bf16(got.reshape(m, n)[rows].ravel())
+    assert_close(got_rows, want.ravel(), 2 ** -7, 2e-5 * max(1.0, float(np.abs(base).max())), "sampled rows")
+
+
 def test_config4_4096_cubed_prepacked(hip, oracle):
     """BASELINE config 4 with B prepacked: 24 sampled rows against the oracle, the rest of the matrix bit for bit
     against the k×n kernel (checked itself above), and exact power-of-two linearity."""
