@@ -44,17 +44,17 @@ MEASURED_TRAFFIC_BYTES = {
     "conv2d_grad_weight_f32_n32_c64to128_56x56_k3s1p1": ((44170 + 36161) * 2 + 72288 + 288) * 1024,
     "gemm_bf16_f32acc_4096x4096x4096": (98511 * 2 + 65536) * 1024,
     "gemm_bf16_f32acc_4096x4096x4096_prepacked_rhs": (98406 * 2 + 65536) * 1024,
-    "gemm_bf16_f32acc_16x4096x4096": ((16926 + 1041) * 2 + 2048 + 256) * 1024,
-    "gemm_bf16_f32acc_16x4096x4096_prepacked_rhs": (16923 * 2 + 256) * 1024,
+    "gemm_bf16_f32acc_16x4096x4096": ((16927 + 1045) * 2 + 2048 + 256) * 1024,
+    "gemm_bf16_f32acc_16x4096x4096_prepacked_rhs": (16924 * 2 + 256) * 1024,
     "attention_f32_b8_h16_s2048_d64_noncausal": (98379 * 2 + 65536) * 1024,
     "attention_f32_b8_h16_s2048_d64_causal": (138815 * 2 + 65537) * 1024,
-    "attention_f32_attn_bias_c1_s2048_d64": ((10827 + 4256) * 2 + 8448 + 512) * 1024,
-    "attention_f32_attn_bias_c16_s1024_d64": ((49227 + 8480) * 2 + 16896 + 4096) * 1024,
+    "attention_f32_attn_bias_c1_s2048_d64": ((10840 + 4260) * 2 + 8448 + 512) * 1024,
+    "attention_f32_attn_bias_c16_s1024_d64": ((49240 + 8484) * 2 + 16896 + 4096) * 1024,
     "gemm_f32_100352x128x576_conv_equivalent": (136982 * 2 + 50176) * 1024,
     "gemm_f32_4096x4096x4096": (196708 * 2 + 65536) * 1024,
     "gemm_f32_512x512x512": (4646 * 2 + 1024) * 1024,
-    "attention_bf16_b16_h8_s1024_d64_causal": (24981 * 2 + 16384) * 1024,
-    "layer_norm_f32_to_bf16_16384x512": (16421 * 2 + 16384) * 1024,
+    "attention_bf16_b16_h8_s1024_d64_causal": (25124 * 2 + 16384) * 1024,
+    "layer_norm_f32_to_bf16_16384x512": (16432 * 2 + 16384) * 1024,
     "row_softmax_f32_16384x512": (16408 * 2 + 32768) * 1024,
     "gelu_backward_f32_16384x512": (32788 * 2 + 32768) * 1024,
     "scale_f32_16384x512": (16394 * 2 + 32768) * 1024,
