@@ -270,9 +270,7 @@ __device__ __forceinline__ float activate(float value)
     else return value;
 }
 
-// (EARLY_BIAS: all of the wavefront's bias values are requested up front — one latency instead of eight, at 4·TN·4
-// registers.)
-template <int WTN, int TM, int ACT, bool FULL, bool EARLY_BIAS = true>
+template <int WTN, int TM, int ACT, bool FULL>
 __device__ __forceinline__ void gemm_bf16_epilogue_bf16(const GemmBf16Args &p, const f32x16 (&acc)[TM][WTN / 32],
                                                         unsigned char *lds, int wave, int row_first, int col_base, int lane)
 {
@@ -290,7 +288,7 @@ __device__ __forceinline__ void gemm_bf16_epilogue_bf16(const GemmBf16Args &p, c
     for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
         for (int g = 0; g < 4; ++g) bias4[tn][g] = make_float4(-0.0f, -0.0f, -0.0f, -0.0f);
-    if (EARLY_BIAS && p.bias) {
+    if (p.bias) {
 #pragma unroll
         for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
@@ -302,7 +300,6 @@ __device__ __forceinline__ void gemm_bf16_epilogue_bf16(const GemmBf16Args &p, c
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             const int q = tn * 8 + g * 2 + lh;
-            if (!EARLY_BIAS && p.bias) bias4[tn][g] = *reinterpret_cast<const float4 *>(p.bias + col_base + tn * 32 + g * 8 + lh * 4);
 #pragma unroll
             for (int tm = 0; tm < TM; ++tm) {
                 float v0 = acc[tm][tn][4 * g + 0] * scale, v1 = acc[tm][tn][4 * g + 1] * scale;
