@@ -176,7 +176,7 @@ int st_hip_conv2d_planned_kernel(size_t batch, size_t c_in, size_t h, size_t w, 
  *   grad_input  (N, C_in, H, W)       = col2im(G · W)
  *   grad_weight (C_out, C_in·KH·KW)   = (Gᵀ · patches) / batch
  *   grad_bias   (C_out)               = column sums of G / batch
- * where G is grad_output viewed per pixel.  An empty batch is a no-op (:787-789).  Needs c_out·kh·kw <= 8192. */
+ * where G is grad_output viewed per pixel.  An empty batch is a no-op (:787-789). */
 int st_hip_conv2d_backward_f32(size_t batch, size_t c_in, size_t h, size_t w, size_t c_out, size_t kh,
                                size_t kw, size_t stride_h, size_t stride_w, size_t pad_h, size_t pad_w,
                                size_t dil_h, size_t dil_w, const float *input, size_t input_len,

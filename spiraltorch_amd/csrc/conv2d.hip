@@ -74,7 +74,8 @@ __global__ __launch_bounds__(64 * WM * WN) void conv2d_f32_kernel(ConvArgs p)
 
     extern __shared__ __attribute__((aligned(16))) unsigned char conv_lds[];
     const int K = p.K;
-    const int k_padded = (K + 15) & ~15;
+    // The offset table holds one segment of the reduction (kConvTableEntries entries) at a time.
+    const int k_padded = (min(K, kConvTableEntries) + 15) & ~15;
     int2 *lut = reinterpret_cast<int2 *>(conv_lds);
     float *As = reinterpret_cast<float *>(conv_lds + static_cast<size_t>(k_padded) * sizeof(int2));
     float *Bs = As + 2 * A_ELEMS;
@@ -98,12 +99,16 @@ __global__ __launch_bounds__(64 * WM * WN) void conv2d_f32_kernel(ConvArgs p)
     const ConvShape &s = p.s;
     const int H = s.h, W = s.w;
     const int khw = s.kh * s.kw;
-    for (int k = tid; k < K; k += T) {
-        const int ic = k / khw, rem = k - ic * khw;
-        const int ky = rem / s.kw, kx = rem - ky * s.kw;
-        const int dy = ky * s.dil_h, dx = kx * s.dil_w;
-        lut[k] = make_int2(TRANSPOSED ? ic * H * W : ic * H * W + dy * W + dx, dy | (dx << 16));
-    }
+    int seg0 = 0;  // first reduction index of the segment the table describes
+    auto fill_table = [&]() {
+        const int seg_end = min(K, seg0 + kConvTableEntries);
+        for (int k = seg0 + tid; k < seg_end; k += T) {
+            const int ic = k / khw, rem = k - ic * khw;
+            const int ky = rem / s.kw, kx = rem - ky * s.kw;
+            const int dy = ky * s.dil_h, dx = kx * s.dil_w;
+            lut[k - seg0] = make_int2(TRANSPOSED ? ic * H * W : ic * H * W + dy * W + dx, dy | (dx << 16));
+        }
+    };
 
     // Every thread gathers one pixel column of the patch tile, rows (tid / BN) + B_ROW_STEP * r.
     const int px_local = tid % BN;
@@ -161,7 +166,7 @@ __global__ __launch_bounds__(64 * WM * WN) void conv2d_f32_kernel(ConvArgs p)
             const int k = k0 + krow0 + B_ROW_STEP * r;
             float v = 0.0f;
             if (px_valid && (FULLK || k < K)) {
-                const int2 e = lut[k];
+                const int2 e = lut[k - seg0];
                 if (TRANSPOSED) {
                     const int ty = iy0 - (e.y & 0xffff), tx = ix0 - (e.y >> 16);
                     if (ty >= 0 && tx >= 0) {
@@ -219,17 +224,23 @@ __global__ __launch_bounds__(64 * WM * WN) void conv2d_f32_kernel(ConvArgs p)
         }
     };
 
-    __syncthreads();  // offset table complete
-    const int steps = (K + BK - 1) / BK;
-    load_global(0);
-    store_lds(0);
-    __syncthreads();
-    for (int t = 0; t < steps; ++t) {
-        const bool more = t + 1 < steps;
-        if (more) load_global((t + 1) * BK);
-        compute(t & 1);
-        if (more) store_lds((t + 1) & 1);
+    // Segment by segment (one for every layer up to kConvTableEntries reduction terms): table, then its k-tiles
+    // through the two-stage pipeline; the accumulators run on across segments, in reduction order.
+    static_assert(kConvTableEntries % BK == 0, "segments hold whole k-tiles");
+    for (; seg0 < K; seg0 += kConvTableEntries) {
+        fill_table();
+        __syncthreads();  // offset table complete (and the previous segment's last tile has been consumed)
+        const int steps = (min(K - seg0, kConvTableEntries) + BK - 1) / BK;
+        load_global(seg0);
+        store_lds(0);
         __syncthreads();
+        for (int t = 0; t < steps; ++t) {
+            const bool more = t + 1 < steps;
+            if (more) load_global(seg0 + (t + 1) * BK);
+            compute(t & 1);
+            if (more) store_lds((t + 1) & 1);
+            __syncthreads();
+        }
     }
 
     float *out_image = p.out + static_cast<size_t>(image) * s.c_out * p.spatial;
@@ -811,7 +822,7 @@ hipError_t launch_tile(ConvArgs args, bool vec, hipStream_t stream)
     const size_t tiles = static_cast<size_t>(args.tiles_oc) * args.tiles_px * static_cast<size_t>(args.s.batch);
     if (tiles > 0x7fffffffu) return hipErrorInvalidConfiguration;
     args.xcd_swizzle = (args.s.batch % 8 == 0) ? 1 : 0;
-    const size_t k_padded = (static_cast<size_t>(args.K) + 15) & ~static_cast<size_t>(15);
+    const size_t k_padded = (static_cast<size_t>(std::min(args.K, kConvTableEntries)) + 15) & ~static_cast<size_t>(15);
     const size_t lds_bytes = k_padded * sizeof(int2) +
                              2 * (static_cast<size_t>(BM) * (BK + 4) + static_cast<size_t>(BK) * (BN + 8)) * sizeof(float);
     const dim3 grid(static_cast<unsigned>(tiles));
@@ -881,7 +892,6 @@ void set_conv_forced_family(int family) { g_forced_family.store(family, std::mem
 
 int planned_conv_kernel(const ConvShape &shape, bool weight_aligned, bool out_aligned)
 {
-    if (shape.kh * shape.kw * static_cast<long long>(shape.c_in) > kConvMaxReduction) return 0;
     StripArgs strip;
     return choose_conv_kernel(shape, weight_aligned, out_aligned, g_forced_family.load(std::memory_order_relaxed), strip);
 }
@@ -903,7 +913,7 @@ hipError_t launch_conv2d_f32(const ConvShape &shape, int activation, const float
     args.activation = activation;
     // The offset table packs ky*dh and kx*dw into 16 bits each.
     if ((shape.kh - 1) * static_cast<long long>(shape.dil_h) > 0x7fff ||
-        (shape.kw - 1) * static_cast<long long>(shape.dil_w) > 0x7fff || args.K > kConvMaxReduction)
+        (shape.kw - 1) * static_cast<long long>(shape.dil_w) > 0x7fff)
         return hipErrorInvalidValue;
     const bool weight_aligned = (reinterpret_cast<uintptr_t>(weight) & 15u) == 0;
     const bool out_aligned = (reinterpret_cast<uintptr_t>(out) & 15u) == 0;
@@ -950,7 +960,7 @@ hipError_t launch_conv2d_adjoint_f32(const ConvShape &shape, const float *grad_o
     args.xcd_swizzle = 0;
     args.activation = ST_HIP_ACT_NONE;
     if ((shape.kh - 1) * static_cast<long long>(shape.dil_h) > 0x7fff ||
-        (shape.kw - 1) * static_cast<long long>(shape.dil_w) > 0x7fff || args.K > kConvMaxReduction)
+        (shape.kw - 1) * static_cast<long long>(shape.dil_w) > 0x7fff)
         return hipErrorInvalidValue;
     const bool vec = (args.K % 4 == 0) && ((reinterpret_cast<uintptr_t>(weight_ic_major) & 15u) == 0);
     if (shape.c_out > 64) return launch_tile<128, 64, 16, 4, 2, true>(args, vec, stream);

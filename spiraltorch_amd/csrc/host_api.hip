@@ -236,9 +236,6 @@ int plan_conv(size_t batch, size_t c_in, size_t h, size_t w, size_t c_out, size_
         return fail(ST_HIP_ERR_INVALID, "conv2d dimensions overflow");
     if (chw > kMaxDim || ochw > kMaxDim || span > kMaxDim)
         return fail(ST_HIP_ERR_UNSUPPORTED, "conv2d per-image extent exceeds i32");
-    if (span > static_cast<size_t>(kConvMaxReduction))
-        return fail(ST_HIP_ERR_UNSUPPORTED, "conv2d reduction extent c_in*kh*kw=%zu exceeds %d", span,
-                    kConvMaxReduction);
     ConvShape &s = plan->shape;
     s.batch = static_cast<int>(batch); s.c_in = static_cast<int>(c_in); s.h = static_cast<int>(h);
     s.w = static_cast<int>(w); s.c_out = static_cast<int>(c_out); s.kh = static_cast<int>(kh);
@@ -540,9 +537,8 @@ int st_hip_conv2d_backward_f32(size_t batch, size_t c_in, size_t h, size_t w, si
                     plan.weight_len);
     if (grad_bias_len != c_out)
         return fail(ST_HIP_ERR_INVALID, "grad_bias buffer length %zu does not match c_out=%zu", grad_bias_len, c_out);
-    if (c_out * kh * kw > static_cast<size_t>(kConvMaxReduction))
-        return fail(ST_HIP_ERR_UNSUPPORTED, "conv2d backward reduction extent c_out*kh*kw=%zu exceeds %d", c_out * kh * kw,
-                    kConvMaxReduction);
+    if (c_out * kh * kw > static_cast<size_t>(kMaxDim))
+        return fail(ST_HIP_ERR_UNSUPPORTED, "conv2d backward reduction extent c_out*kh*kw=%zu exceeds i32", c_out * kh * kw);
     ST_HIP_CHECK(reject_null(input, input_len, "conv2d backward"));
     ST_HIP_CHECK(reject_null(weight, weight_len, "conv2d backward"));
     ST_HIP_CHECK(reject_null(grad_output, grad_output_len, "conv2d backward"));
@@ -799,9 +795,8 @@ int st_hip_conv2d_grad_input_f32_dev(size_t batch, size_t c_in, size_t h, size_t
     ST_HIP_CHECK(ensure_init());
     ConvPlan plan;
     ST_HIP_CHECK(plan_conv(batch, c_in, h, w, c_out, kh, kw, stride_h, stride_w, pad_h, pad_w, dil_h, dil_w, &plan));
-    if (c_out * kh * kw > static_cast<size_t>(kConvMaxReduction))
-        return fail(ST_HIP_ERR_UNSUPPORTED, "conv2d backward reduction extent c_out*kh*kw=%zu exceeds %d", c_out * kh * kw,
-                    kConvMaxReduction);
+    if (c_out * kh * kw > static_cast<size_t>(kMaxDim))
+        return fail(ST_HIP_ERR_UNSUPPORTED, "conv2d backward reduction extent c_out*kh*kw=%zu exceeds i32", c_out * kh * kw);
     if (plan.input_len == 0) return ST_HIP_OK;
     if (!grad_output || !weight || !grad_input)
         return fail(ST_HIP_ERR_INVALID, "conv2d backward received a null pointer; provide contiguous buffers");
@@ -818,9 +813,8 @@ int st_hip_conv2d_grad_input_f32_noalloc_dev(size_t batch, size_t c_in, size_t h
     ST_HIP_CHECK(ensure_init());
     ConvPlan plan;
     ST_HIP_CHECK(plan_conv(batch, c_in, h, w, c_out, kh, kw, stride_h, stride_w, pad_h, pad_w, dil_h, dil_w, &plan));
-    if (c_out * kh * kw > static_cast<size_t>(kConvMaxReduction))
-        return fail(ST_HIP_ERR_UNSUPPORTED, "conv2d backward reduction extent c_out*kh*kw=%zu exceeds %d", c_out * kh * kw,
-                    kConvMaxReduction);
+    if (c_out * kh * kw > static_cast<size_t>(kMaxDim))
+        return fail(ST_HIP_ERR_UNSUPPORTED, "conv2d backward reduction extent c_out*kh*kw=%zu exceeds i32", c_out * kh * kw);
     if (plan.weight_len > kNoAllocScratchBytes / sizeof(float))
         return fail(ST_HIP_ERR_UNSUPPORTED,
                     "conv2d grad_input without allocation: the weights (%zu bytes) exceed the static scratch of %zu bytes; "

@@ -41,8 +41,9 @@ hipError_t launch_transpose_u16(size_t rows, size_t cols, const uint16_t *in, ui
 struct ConvShape {
     int batch, c_in, h, w, c_out, kh, kw, stride_h, stride_w, pad_h, pad_w, dil_h, dil_w, oh, ow;
 };
-// Largest c_in*kh*kw the implicit-GEMM kernel's LDS offset table holds.
-constexpr int kConvMaxReduction = 8192;
+// Entries of the general implicit-GEMM kernel's LDS offset table: longer reductions (c_in*kh*kw) go through it in
+// segments of this many terms.
+constexpr int kConvTableEntries = 8192;
 hipError_t launch_conv2d_f32(const ConvShape &shape, int activation, const float *input,
                              const float *weight, const float *bias, float *out, hipStream_t stream);
 

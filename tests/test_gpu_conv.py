@@ -68,6 +68,28 @@ def test_random_shapes(hip, oracle, shape):
     assert_close(got, oracle.conv2d_bias_act_f32(*shape, oracle.ACT_RELU, x, wt, None), F32_REL, F32_ABS, "no bias")
 
 
+@pytest.mark.parametrize("shape", [
+    (1, 192, 12, 12, 40, (7, 7), (1, 1), (3, 3), (1, 1)),    # 9408 terms: two table segments (ConvNeXt-style 7×7)
+    (2, 170, 9, 9, 70, (7, 7), (2, 2), (3, 3), (1, 1)),      # 8330 terms, k % 16 != 0, strided
+    (1, 384, 8, 8, 33, (7, 7), (1, 1), (3, 3), (1, 1)),      # 18816 terms: three segments
+    (1, 1030, 6, 6, 20, (3, 3), (1, 1), (1, 1), (1, 1)),     # 9270 terms, k % 4 != 0: scalar weight staging
+])
+def test_reductions_longer_than_the_offset_table(hip, oracle, shape):
+    """c_in·kh·kw beyond the 8192 entries of the general kernel's LDS offset table: the table is rebuilt segment by
+    segment while the accumulators run on.  He-scaled weights; compared against the oracle with the bound a
+    reordered f32 sum of that length supports (a small multiple of unit roundoff times sum |x||w|)."""
+    batch, c_in, h, w, c_out, kernel, stride, padding, dilation = shape
+    rng = np.random.default_rng(c_in * 31 + c_out)
+    x = rng.normal(size=batch * c_in * h * w).astype(np.float32)
+    wt = rng.normal(0, np.sqrt(2.0 / (c_in * kernel[0] * kernel[1])), c_out * c_in * kernel[0] * kernel[1]).astype(np.float32)
+    b = rng.uniform(-0.1, 0.1, c_out).astype(np.float32)
+    got = run(hip, *shape, 1, x, wt, b)
+    want = oracle.conv2d_bias_act_f32(*shape, oracle.ACT_RELU, x, wt, b)
+    magnitude = oracle.conv2d_bias_act_f32(*shape, oracle.ACT_NONE, np.abs(x), np.abs(wt), None)
+    assert_close(got, want, F32_REL, F32_ABS + 2 * 2.0 ** -24 * float(magnitude.max()), f"conv {shape}")
+    assert float(np.abs(got).max()) > 0.1  # the comparison is not about zeros
+
+
 G33 = ((3, 3), (1, 1), (1, 1), (1, 1))
 FAMILY_SHAPES = {
     # name: (batch, c_in, h, w, c_out, kernel, stride, padding, dilation)

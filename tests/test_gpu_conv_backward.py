@@ -23,6 +23,8 @@ CASES = [
     (2, 64, 9, 10, 128, (3, 3), (1, 1), (1, 1), (1, 1)),   # 128 × 192 grad_weight tiles, exact fit (S = 576)
     (3, 21, 11, 7, 120, (3, 3), (1, 1), (1, 1), (1, 1)),   # 128 × 192 tiles with ragged channels and columns (S = 189)
     (2, 22, 9, 9, 250, (3, 3), (2, 1), (1, 0), (1, 1)),    # two channel tiles, strided rows (per-element gather)
+    (1, 24, 10, 10, 192, (7, 7), (1, 1), (3, 3), (1, 1)),  # c_out*kh*kw = 9408: more than one offset-table segment
+    (1, 20, 11, 11, 180, (7, 7), (2, 2), (3, 3), (1, 1)),  # the same through the adjoint gather (stride 2), 8820 terms
 ]
 
 
@@ -37,7 +39,10 @@ def test_backward_matches_the_oracle(hip, oracle, case):
     gi, gw, gb = (np.zeros(n, np.float32) for n in (x.size, wgt.size, c_out))
     hip.conv2d_backward_f32(*case, x, wgt, g, gi, gw, gb)
     want_gi, want_gw, want_gb = oracle.conv2d_backward_f32(*case, x, wgt, g)
-    assert_close(gi, want_gi, F32_REL, F32_ABS, f"grad_input {case}")
+    if c_out * kernel[0] * kernel[1] > 2000:
+        assert_grad_input(gi, case, g, wgt, want_gi, f"grad_input {case}")  # long reduction: bound from float64
+    else:
+        assert_close(gi, want_gi, F32_REL, F32_ABS, f"grad_input {case}")
     # grad_weight / grad_bias add batch*oh*ow terms in a different order than the oracle
     floor = 2e-7 * float(np.abs(g).max()) * float(np.abs(x).max()) * oh * ow
     assert_close(gw, want_gw, F32_REL, F32_ABS + floor, f"grad_weight {case}")
