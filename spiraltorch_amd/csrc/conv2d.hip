@@ -41,7 +41,7 @@ struct ConvArgs {
     int tiles_px, tiles_oc;
     int xcd_swizzle;
     int activation;
-    unsigned tap_bytes[32];  // ring kernel: byte offset of tap ky*kw + kx relative to a pixel's top-left tap
+    unsigned tap_bytes[64];  // ring kernel: byte offset of tap ky*kw + kx relative to a pixel's top-left tap
 };
 
 
@@ -273,7 +273,7 @@ __global__ __launch_bounds__(64 * WM * WN) void conv2d_f32_kernel(ConvArgs p)
 // gathered row belongs to is wavefront-uniform and tracked in scalar registers, so the loop's vector address
 // arithmetic is a shift, an add and a shift-add per gathered row.
 //
-// Needs: c_in*kh*kw a multiple of 16 with 16-byte aligned weight rows, kh*kw <= 32, one image smaller than
+// Needs: c_in*kh*kw a multiple of 16 with 16-byte aligned weight rows, kh*kw <= 64, one image smaller than
 // 1 GiB and the weights smaller than 2 GiB (32-bit buffer offsets).  Everything else takes the register-staged kernel above.
 //
 // LDS per stage: weights BM rows × 64 B, 16-byte chunk c of row r stored at position c ^ ((r >> 2) & 3)
@@ -332,14 +332,14 @@ __device__ __forceinline__ void conv2d_f32_ring_body(const ConvArgs &p)
     const int iy0 = oy * s.stride_h - s.pad_h;
     const int ix0 = ox * s.stride_w - s.pad_w;
     const unsigned base_bytes = static_cast<unsigned>(iy0 * W + ix0) * 4u;  // may wrap; valid taps unwrap it
-    unsigned tap_mask = 0;
+    unsigned long long tap_mask = 0;  // up to 64 taps (7×7 kernels have 49)
     for (int j = 0; j < khw; ++j) {
         const int ky = j / s.kw, kx = j - ky * s.kw;
         const bool ok = px_valid && static_cast<unsigned>(iy0 + ky * s.dil_h) < static_cast<unsigned>(H) &&
                         static_cast<unsigned>(ix0 + kx * s.dil_w) < static_cast<unsigned>(W);
-        tap_mask |= (ok ? 1u : 0u) << j;
+        tap_mask |= (ok ? 1ull : 0ull) << j;
     }
-    const unsigned tap_outside = ~tap_mask;  // bit j set: tap j of this pixel reads padding (or the pixel is past the end)
+    const unsigned long long tap_outside = ~tap_mask;  // bit j set: tap j of this pixel reads padding (or the pixel is past the end)
 
     const size_t image_elems = static_cast<size_t>(s.c_in) * H * W;
     const __amdgpu_buffer_rsrc_t rsrc_x = __builtin_amdgcn_make_buffer_rsrc(
@@ -375,7 +375,7 @@ __device__ __forceinline__ void conv2d_f32_ring_body(const ConvArgs &p)
         for (int r = 0; r < B_ROWS; ++r) {
             const int row = wave * B_ROWS + r;
             const unsigned tap_bytes = p.tap_bytes[row_tap[r]] + static_cast<unsigned>(row_ic[r]) * channel_bytes;
-            const unsigned off = ((tap_outside >> row_tap[r]) << 31) + (base_bytes + tap_bytes);
+            const unsigned off = (static_cast<unsigned>(tap_outside >> row_tap[r]) << 31) + (base_bytes + tap_bytes);
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (lds_void_ptr)(stage + A_BYTES + row * B_PITCH), 4, off, 0, 0, 0);
             row_tap[r] += step_tap;
             row_ic[r] += step_ic;
@@ -800,7 +800,7 @@ hipError_t launch_ring(ConvArgs args, hipStream_t stream)
     const size_t tiles = static_cast<size_t>(args.tiles_oc) * args.tiles_px * static_cast<size_t>(args.s.batch);
     if (tiles > 0x7fffffffu) return hipErrorInvalidConfiguration;
     args.xcd_swizzle = (args.s.batch % 8 == 0) ? 1 : 0;
-    for (int j = 0; j < 32; ++j) {
+    for (int j = 0; j < 64; ++j) {
         const int ky = j / args.s.kw, kx = j % args.s.kw;
         args.tap_bytes[j] = j < args.s.kh * args.s.kw
                                 ? static_cast<unsigned>(ky * args.s.dil_h * args.s.w + kx * args.s.dil_w) * 4u : 0u;
@@ -860,7 +860,7 @@ int choose_conv_kernel(const ConvShape &shape, bool weight_aligned, bool out_ali
     const bool image_ok = static_cast<size_t>(shape.c_in) * shape.h * shape.w * 4 < (1ull << 30);
     // 8 wavefronts of 32×32 per 128×64 tile measured best for wide layers (128×128 tiles, 32-deep k-tiles and
     // 4-wavefront layouts were all 10-20 % slower on the 64->128 channel 56×56 case).
-    const bool ring_ok = vec && K % 16 == 0 && shape.kh * shape.kw <= 32 && image_ok &&
+    const bool ring_ok = vec && K % 16 == 0 && shape.kh * shape.kw <= 64 && image_ok &&
                          (static_cast<size_t>(shape.pad_h) * shape.w + shape.pad_w) * 4 < (1ull << 30) &&
                          (static_cast<size_t>(shape.oh + 64) * shape.stride_h * shape.w + static_cast<size_t>(shape.ow) * shape.stride_w) * 4 < (1ull << 30) &&
                          static_cast<size_t>(shape.c_out) * K * 4 < (1ull << 31);

@@ -110,6 +110,8 @@ FAMILY_SHAPES = {
     "fuzz_c64_p0": (3, 64, 33, 33, 160, (3, 3), (1, 1), (0, 0), (1, 1)),  # no padding, two channel tiles
     "ring64": (2, 16, 20, 20, 40, *G33),                 # 64-row ring tiles
     "ring_5x5": (2, 16, 15, 15, 130, (5, 5), (1, 1), (2, 2), (1, 1)),    # 25 taps, ragged channel tile
+    "ring_7x7": (2, 32, 17, 15, 70, (7, 7), (1, 1), (3, 3), (1, 1)),     # 49 taps: the upper word of the tap mask
+    "ring_7x7_s2": (2, 16, 23, 23, 40, (7, 7), (2, 2), (3, 3), (1, 1)),  # 49 taps, stride 2, 64-row tiles
 }
 # (shape, forced family, the kernel that has to run)
 FAMILY_CASES = [
@@ -121,7 +123,7 @@ FAMILY_CASES = [
     ("ragged_strip", "ring", "ring"), ("row_of_nine", "ring", "ring"), ("c112", "ring", "ring"),
     ("c128_odd_plane", "ring", "ring"), ("stride2_c32", "ring", "ring"), ("dilated_c48", "ring", "ring"),
     ("chunks_c16", "ring", "ring"), ("fuzz_c64_p0", "ring", "ring"), ("ring64", "ring", "ring"),
-    ("ring_5x5", "ring", "ring"),
+    ("ring_5x5", "ring", "ring"), ("ring_7x7", "ring", "ring"), ("ring_7x7_s2", "ring", "ring"), ("ring_7x7", "tile", "tile"),
     ("ragged_strip", "tile", "tile"), ("c130", "tile", "tile"), ("chunks_c4", "tile", "tile"),
     ("stride2_c8", "tile", "tile"), ("dilated_c6", "tile", "tile"), ("row_of_nine", "tile", "tile"),
     ("blocks56", "tile", "tile"), ("c112", "tile", "tile"), ("stride2_c32", "tile", "tile"),

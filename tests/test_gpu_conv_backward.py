@@ -142,6 +142,7 @@ GRAD_INPUT_FAMILY_CASES = [
     ("ring", "ring", (2, 70, 20, 20, 16, (3, 3), (1, 1), (1, 1), (1, 1))),
     ("ring", "ring", (2, 130, 15, 15, 16, (5, 5), (1, 1), (2, 2), (1, 1))),
     ("ring", "ring", (2, 24, 14, 14, 112, (3, 3), (1, 1), (1, 1), (1, 1))),
+    ("ring", "ring", (2, 20, 13, 12, 32, (7, 7), (1, 1), (3, 3), (1, 1))),          # 49 taps
     ("tile", "tile", (2, 24, 14, 14, 112, (3, 3), (1, 1), (1, 1), (1, 1))),
     ("tile", "tile", (2, 5, 10, 11, 6, (3, 3), (1, 1), (2, 2), (1, 1))),
     ("auto", "adjoint", (2, 22, 9, 9, 250, (3, 3), (2, 1), (1, 0), (1, 1))),
