@@ -931,8 +931,14 @@ hipError_t launch_conv2d_f32(const ConvShape &shape, int activation, const float
         strip.s = shape;
         strip.activation = activation;
         return launch_strip(strip, kernel, stream);
-    case ST_HIP_CONV_KERNEL_RING:
-        return shape.c_out > 64 ? launch_ring<128>(args, stream) : launch_ring<64>(args, stream);
+    case ST_HIP_CONV_KERNEL_RING: {
+        // 128 output channels per tile unless that leaves half of the compute units without a tile (deep layers on
+        // small planes: 512 channels on 7×7 are 32 × 1 × 4 tiles); 64-channel tiles then double the workgroups and
+        // still run in one round (512→512 on 7×7: 196 → 151 µs; with 192 tiles of 128 channels, 768→768 7×7 with a
+        // 7×7 kernel, the 384 tiles of 64 are slower: 1539 → 1837 µs).
+        const long long tiles128 = static_cast<long long>(shape.batch) * ((args.spatial + 63) / 64) * ((shape.c_out + 127) / 128);
+        return shape.c_out > 64 && tiles128 > 128 ? launch_ring<128>(args, stream) : launch_ring<64>(args, stream);
+    }
     case ST_HIP_CONV_KERNEL_TILE: {
         const bool vec = (args.K % 4 == 0) && weight_aligned;
         if (shape.c_out > 64) return launch_tile<128, 64, 16, 4, 2>(args, vec, stream);
