@@ -16,6 +16,8 @@
 #include "device_math.h"
 #include "kernels.h"
 
+#include <algorithm>
+#include <cmath>
 #include <mutex>
 
 namespace sthip {
@@ -69,6 +71,47 @@ __global__ __launch_bounds__(256) void conv_weight_to_adjoint_kernel(int c_out, 
     const int ic = rest / c_out;
     const int sy = flip ? kh - 1 - ky : ky, sx = flip ? kw - 1 - kx : kx;
     dst[i] = src[((static_cast<size_t>(oc) * c_in + ic) * kh + sy) * kw + sx];
+}
+
+// col2im as a gather (crates/st-nn/src/layers/conv.rs:860-916 adds patch gradients into the input gradient patch by
+// patch; here every input position collects the entries that land on it, in the same order: output rows ascending,
+// then output columns ascending).  cols: [images][OH·OW][C_in·KH·KW], the product grad_outputᵀ · W of each image.
+// One thread per input value.
+__global__ __launch_bounds__(256) void conv_col2im_gather_kernel(ConvShape s, int images, const float *cols, float *grad_input)
+{
+    const size_t total = static_cast<size_t>(images) * s.c_in * s.h * s.w;
+    const size_t idx = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (idx >= total) return;
+    const int x = static_cast<int>(idx % s.w);
+    size_t rest = idx / s.w;
+    const int y = static_cast<int>(rest % s.h);
+    rest /= s.h;
+    const int ic = static_cast<int>(rest % s.c_in);
+    const int image = static_cast<int>(rest / s.c_in);
+    const int S = s.c_in * s.kh * s.kw;
+    const float *image_cols = cols + static_cast<size_t>(image) * s.oh * s.ow * S + static_cast<size_t>(ic) * s.kh * s.kw;
+    // Taps that can reach this position: (y + pad − ky·dil) a non-negative multiple of the stride below OH·stride.
+    // Without dilation they are every stride-th ky, so the loop steps over the others (a 16×16 kernel at stride 16 has
+    // one candidate per axis, not sixteen).
+    const int step_y = s.dil_h == 1 ? s.stride_h : 1, step_x = s.dil_w == 1 ? s.stride_w : 1;
+    int ky_last = s.kh - 1, kx_last = s.kw - 1;
+    if (s.dil_h == 1) ky_last -= ((ky_last - (y + s.pad_h)) % step_y + step_y) % step_y;
+    if (s.dil_w == 1) kx_last -= ((kx_last - (x + s.pad_w)) % step_x + step_x) % step_x;
+    float sum = 0.0f;
+    for (int ky = ky_last; ky >= 0; ky -= step_y) {  // descending ky = ascending output row
+        const int ty = y + s.pad_h - ky * s.dil_h;
+        if (ty < 0 || ty % s.stride_h != 0) continue;
+        const int oy = ty / s.stride_h;
+        if (oy >= s.oh) continue;
+        for (int kx = kx_last; kx >= 0; kx -= step_x) {
+            const int tx = x + s.pad_w - kx * s.dil_w;
+            if (tx < 0 || tx % s.stride_w != 0) continue;
+            const int ox = tx / s.stride_w;
+            if (ox >= s.ow) continue;
+            sum += image_cols[(static_cast<size_t>(oy) * s.ow + ox) * S + ky * s.kw + kx];
+        }
+    }
+    grad_input[idx] = sum;
 }
 
 __device__ __forceinline__ float wave_sum64(float v)
@@ -437,10 +480,29 @@ bool grad_input_as_forward(const ConvShape &shape, ConvShape &t)
 }
 }  // namespace
 
+namespace {
+// Strided (or over-padded) layers: the adjoint gather kernel tests every (channel, tap) for every input position,
+// although only one tap in stride_h·stride_w can contribute, and its output-channel tiles hold 64 or 128 input
+// channels — the ViT patch embedding (3 channels, 16×16 at stride 16) took 1.3 s that way.  The reference's own route,
+// the product grad_outputᵀ·W followed by col2im, does the forward's flops once: per image an f32 GEMM with the
+// transposed-A kernel (grad_output of an image is C_out × OH·OW, i.e. k × m), its result gathered into grad_input.
+// Images are processed in groups whose products fit kCol2imWorkspaceBytes.  Chosen when the gather's wasted work
+// (stride product × channel-tile padding) exceeds a factor of three; the allocation-free entry point keeps the gather.
+constexpr size_t kCol2imWorkspaceBytes = 256u << 20;
+bool grad_input_by_col2im(const ConvShape &shape)
+{
+    const double tile = shape.c_in > 64 ? 128.0 : 64.0;
+    const double padded = std::ceil(shape.c_in / tile) * tile / shape.c_in;
+    const size_t image_cols = static_cast<size_t>(shape.oh) * shape.ow * shape.c_in * shape.kh * shape.kw * sizeof(float);
+    return static_cast<double>(shape.stride_h) * shape.stride_w * padded > 3.0 && image_cols <= kCol2imWorkspaceBytes &&
+           image_cols > 0;
+}
+}  // namespace
+
 int planned_conv_grad_input_kernel(const ConvShape &shape)
 {
     ConvShape t;
-    if (!grad_input_as_forward(shape, t)) return ST_HIP_CONV_KERNEL_ADJOINT;
+    if (!grad_input_as_forward(shape, t)) return grad_input_by_col2im(shape) ? ST_HIP_CONV_KERNEL_COL2IM : ST_HIP_CONV_KERNEL_ADJOINT;
     return planned_conv_kernel(t, true, true);
 }
 
@@ -452,6 +514,32 @@ hipError_t launch_conv2d_grad_input_f32(const ConvShape &shape, const float *gra
     ConvShape t;
     const bool as_forward = grad_input_as_forward(shape, t);
     hipError_t rc;
+    if (!as_forward && weight_scratch == nullptr && grad_input_by_col2im(shape)) {
+        const size_t m = static_cast<size_t>(shape.oh) * shape.ow, S = static_cast<size_t>(shape.c_in) * shape.kh * shape.kw;
+        const size_t image_cols = m * S;
+        const size_t group = std::max<size_t>(1, std::min<size_t>(shape.batch, kCol2imWorkspaceBytes / (image_cols * sizeof(float))));
+        void *workspace = nullptr;
+        rc = stream_workspace(stream, group * image_cols * sizeof(float), &workspace);
+        if (rc != hipSuccess) return rc;
+        float *cols = static_cast<float *>(workspace);
+        const size_t image_in = static_cast<size_t>(shape.c_in) * shape.h * shape.w;
+        GemmEpilogue plain;
+        for (size_t first = 0; first < static_cast<size_t>(shape.batch); first += group) {
+            const size_t images = std::min(group, static_cast<size_t>(shape.batch) - first);
+            for (size_t i = 0; i < images; ++i) {
+                // cols_i (OH·OW × S) = G_iᵀ · W with G_i = grad_output of the image, C_out × OH·OW (k × m), W = C_out × S
+                rc = launch_gemm_f32(m, S, static_cast<size_t>(shape.c_out), true, grad_output + (first + i) * shape.c_out * m,
+                                     weight, cols + i * image_cols, plain, stream);
+                if (rc != hipSuccess) return rc;
+            }
+            const size_t total = images * image_in;
+            hipLaunchKernelGGL(conv_col2im_gather_kernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, stream,
+                               shape, static_cast<int>(images), cols, grad_input + first * image_in);
+            rc = hipGetLastError();
+            if (rc != hipSuccess) return rc;
+        }
+        return hipSuccess;
+    }
     float *adjoint_weight = weight_scratch;  // room for weight_count values, owned by the caller
     if (adjoint_weight == nullptr) {
         void *workspace = nullptr;

@@ -24,7 +24,8 @@ CASES = [
     (3, 21, 11, 7, 120, (3, 3), (1, 1), (1, 1), (1, 1)),   # 128 × 192 tiles with ragged channels and columns (S = 189)
     (2, 22, 9, 9, 250, (3, 3), (2, 1), (1, 0), (1, 1)),    # two channel tiles, strided rows (per-element gather)
     (1, 24, 10, 10, 192, (7, 7), (1, 1), (3, 3), (1, 1)),  # c_out*kh*kw = 9408: more than one offset-table segment
-    (1, 20, 11, 11, 180, (7, 7), (2, 2), (3, 3), (1, 1)),  # the same through the adjoint gather (stride 2), 8820 terms
+    (1, 20, 11, 11, 180, (7, 7), (2, 2), (3, 3), (1, 1)),  # stride 2, 8820 terms: GEMM + col2im
+    (1, 128, 11, 11, 180, (7, 7), (1, 2), (3, 3), (1, 1)), # the same through the adjoint gather (whole channel tile, stride 1×2)
 ]
 
 
@@ -98,7 +99,8 @@ HE_CASES = [
     ("ring", "ring", (3, 64, 33, 33, 160, (3, 3), (1, 1), (0, 0), (1, 1))),
     ("tile", "tile", (4, 16, 19, 26, 100, (3, 3), (1, 1), (1, 1), (1, 1))),
     ("tile", "tile", (3, 2, 38, 35, 160, (3, 3), (1, 1), (2, 0), (1, 2))),
-    ("auto", "adjoint", (3, 2, 38, 24, 128, (3, 3), (2, 1), (0, 1), (2, 1))),
+    ("auto", "col2im", (3, 2, 38, 24, 128, (3, 3), (2, 1), (0, 1), (2, 1))),
+    ("auto", "adjoint", (3, 64, 20, 18, 128, (3, 3), (2, 1), (0, 1), (2, 1))),
     ("ring", "ring", (4, 16, 28, 32, 160, (3, 3), (1, 1), (0, 0), (1, 1))),
     ("strip", "strip9", (2, 16, 30, 30, 128, (3, 3), (1, 1), (1, 1), (1, 1))),
     ("strip", "strip12", (2, 32, 17, 19, 100, (3, 3), (1, 1), (1, 1), (1, 1))),
@@ -145,8 +147,14 @@ GRAD_INPUT_FAMILY_CASES = [
     ("ring", "ring", (2, 20, 13, 12, 32, (7, 7), (1, 1), (3, 3), (1, 1))),          # 49 taps
     ("tile", "tile", (2, 24, 14, 14, 112, (3, 3), (1, 1), (1, 1), (1, 1))),
     ("tile", "tile", (2, 5, 10, 11, 6, (3, 3), (1, 1), (2, 2), (1, 1))),
-    ("auto", "adjoint", (2, 22, 9, 9, 250, (3, 3), (2, 1), (1, 0), (1, 1))),
-    ("auto", "adjoint", (2, 5, 10, 11, 6, (3, 3), (1, 1), (3, 3), (1, 1))),        # padding beyond the kernel's reach
+    ("auto", "adjoint", (2, 64, 9, 9, 250, (3, 3), (2, 1), (1, 0), (1, 1))),        # whole channel tile, stride 2×1
+    ("auto", "adjoint", (2, 128, 10, 11, 6, (3, 3), (1, 1), (3, 3), (1, 1))),       # padding beyond the kernel's reach
+    ("auto", "col2im", (2, 22, 9, 9, 250, (3, 3), (2, 1), (1, 0), (1, 1))),         # ragged channel tile: GEMM + col2im
+    ("auto", "col2im", (2, 5, 10, 11, 6, (3, 3), (1, 1), (3, 3), (1, 1))),          # padding beyond the kernel's reach
+    ("auto", "col2im", (3, 3, 32, 32, 40, (16, 16), (16, 16), (0, 0), (1, 1))),     # patch embedding: one tap per position
+    ("auto", "col2im", (2, 3, 30, 29, 16, (7, 7), (2, 2), (3, 3), (1, 1))),         # stem: 7×7 at stride 2
+    ("auto", "col2im", (2, 8, 17, 19, 12, (3, 3), (2, 3), (1, 2), (2, 1))),         # dilation along one axis, stride 2×3
+    ("auto", "col2im", (5, 16, 12, 12, 24, (2, 2), (2, 2), (0, 0), (1, 1))),        # 2×2 at stride 2 (down-sampling)
 ]
 
 

@@ -11,7 +11,7 @@ CALLS = [
     # batch, c_in, h, w, c_out, kernel, stride, padding, dilation — run in this order on one stream
     (4, 64, 28, 28, 128, *G33),                            # strip kernel on 128 'input' channels
     (2, 16, 14, 14, 32, *G33),                             # smaller: reuses the front of the array
-    (2, 22, 9, 9, 250, (3, 3), (2, 1), (1, 0), (1, 1)),    # strided: adjoint gather
+    (2, 64, 9, 9, 250, (3, 3), (2, 1), (1, 0), (1, 1)),    # strided: adjoint gather in both entry points
     (1, 3, 8, 8, 4, (5, 5), (1, 1), (2, 2), (1, 1)),       # smaller again, general kernel
 ]
 
