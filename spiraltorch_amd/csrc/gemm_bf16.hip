@@ -86,7 +86,13 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmBf16Args p)
     const int wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const int li = lane & 31, lh = lane >> 5;
-    const int M = p.M, N = p.N, K = p.K;
+    const int M = p.M, N = p.N;
+    // This workgroup's k range [k_lo, K): slice blockIdx.y of a k-sliced launch (few tiles, long k), whose raw sums go
+    // to plane blockIdx.y of C32 (the launch passes the workspace of partial planes as C32 and no epilogue);
+    // K below is the END of the range, p.K stays the row stride of A.
+    const int k_lo = static_cast<int>(blockIdx.y) * p.tiles_per_split * BK;
+    const int K = p.k_splits > 1 ? min(p.K, k_lo + p.tiles_per_split * BK) : p.K;
+    float *const C32 = p.C32 ? p.C32 + static_cast<size_t>(blockIdx.y) * M * N : nullptr;
 
     int logical = blockIdx.x;
     if (p.swizzle) {
@@ -118,7 +124,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmBf16Args p)
         for (int r = 0; r < A_CHUNKS; ++r) {
             const int f = tid + 256 * r;
             const int row = f / (BK / 8), c8 = (f % (BK / 8)) * 8;
-            ra[r] = load_row8<VEC>(p.A, static_cast<size_t>(m0 + row) * K, k0 + c8, K, m0 + row < M);
+            ra[r] = load_row8<VEC>(p.A, static_cast<size_t>(m0 + row) * p.K, k0 + c8, K, m0 + row < M);
         }
 #pragma unroll
         for (int r = 0; r < B_CHUNKS; ++r) {
@@ -177,15 +183,15 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmBf16Args p)
         }
     };
 
-    const int steps = (K + BK - 1) / BK;
+    const int steps = (K - k_lo + BK - 1) / BK;
     if (steps > 0) {
-        load_global(0);
+        load_global(k_lo);
         store_lds(0);
     }
     __syncthreads();
     for (int t = 0; t < steps; ++t) {
         const bool more = t + 1 < steps;
-        if (more) load_global((t + 1) * BK);
+        if (more) load_global(k_lo + (t + 1) * BK);
         compute(t & 1);
         if (more) store_lds((t + 1) & 1);
         __syncthreads();
@@ -212,7 +218,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmBf16Args p)
                     value += bias;
                     if (p.residual) value += p.residual[idx];
                     value = apply_activation(value, p.activation);
-                    if (p.C32) p.C32[idx] = value;
+                    if (C32) C32[idx] = value;
                     if (p.C16) p.C16[idx] = f32_to_bf16_rne(value);
                 }
             }
@@ -2030,16 +2036,63 @@ hipError_t launch_rowcomplete(const RowLnArgs &args, hipStream_t stream)
     return hipGetLastError();
 }
 
-template <int BM, int BN, int BK>
-hipError_t launch_tile(GemmBf16Args args, bool vec, hipStream_t stream)
+// k-slices of the general tile kernel (128×128 tiles, 32-wide k-tiles): none while the tiles alone give every other
+// compute unit a workgroup; otherwise enough for about two workgroups per compute unit, each slice keeping at least 16
+// k-tiles, and the partial planes (written once, read once, f32) staying below the operands' bytes.
+size_t general_k_slices(size_t m, size_t n, size_t k)
 {
+    const size_t tiles = ((m + 127) / 128) * ((n + 127) / 128), k_steps = (k + 31) / 32;
+    if (tiles > 128 || k_steps < 32) return 1;
+    size_t slices = std::min<size_t>(512 / tiles, k_steps / 16);
+    while (slices > 1 && slices * m * n * 8 > (m * k + k * n) * 2) --slices;
+    return std::max<size_t>(slices, 1);
+}
+size_t general_slice_bytes(size_t m, size_t n, size_t k)
+{
+    const size_t slices = general_k_slices(m, n, k);
+    return slices > 1 ? slices * m * n * sizeof(float) : 0;
+}
+
+// `workspace_offset`: bytes at the front of the stream's workspace that the caller is using (an unpacked B).
+template <int BM, int BN, int BK>
+hipError_t launch_tile(GemmBf16Args args, bool vec, hipStream_t stream, size_t workspace_offset)
+{
+    static_assert(BM == 128 && BN == 128 && BK == 32, "general_k_slices plans for this tiling");
     args.tiles_m = (args.M + BM - 1) / BM;
     args.tiles_n = (args.N + BN - 1) / BN;
     const size_t tiles = static_cast<size_t>(args.tiles_m) * static_cast<size_t>(args.tiles_n);
     if (tiles > 0x7fffffffu) return hipErrorInvalidConfiguration;
     args.swizzle = (tiles % 8 == 0) ? 1 : 0;
     constexpr size_t lds_bytes = 2 * (static_cast<size_t>(BM) * (BK + 8) + static_cast<size_t>(BK) * (BN + 32)) * 2;
-    const dim3 grid(static_cast<unsigned>(tiles));
+    const size_t slices = general_k_slices(args.M, args.N, args.K);
+    SkinnyArgs reduce{};
+    if (slices > 1) {
+        const size_t k_steps = (static_cast<size_t>(args.K) + BK - 1) / BK;
+        args.tiles_per_split = static_cast<int>((k_steps + slices - 1) / slices);
+        args.k_splits = static_cast<int>((k_steps + args.tiles_per_split - 1) / args.tiles_per_split);
+        void *workspace = nullptr;
+        hipError_t ws = stream_workspace(stream, workspace_offset + slices * args.M * static_cast<size_t>(args.N) * sizeof(float),
+                                         &workspace);
+        if (ws != hipSuccess) return ws;
+        reduce.partial = reinterpret_cast<float *>(static_cast<unsigned char *>(workspace) + workspace_offset);
+        reduce.C32 = args.C32;
+        reduce.C16 = args.C16;
+        reduce.bias = args.bias;
+        reduce.residual = args.residual;
+        reduce.M = args.M;
+        reduce.N = args.N;
+        reduce.K = args.K;
+        reduce.k_splits = args.k_splits;
+        reduce.scale = args.scale;
+        reduce.activation = args.activation;
+        args.C32 = reduce.partial;
+        args.C16 = nullptr;
+        args.bias = nullptr;
+        args.residual = nullptr;
+        args.scale = 1.0f;
+        args.activation = ST_HIP_ACT_NONE;
+    }
+    const dim3 grid(static_cast<unsigned>(tiles), static_cast<unsigned>(args.k_splits));
     const dim3 block(256);
     hipError_t rc;
     if (vec) {
@@ -2055,6 +2108,11 @@ hipError_t launch_tile(GemmBf16Args args, bool vec, hipStream_t stream)
         if (rc != hipSuccess) return rc;
         hipLaunchKernelGGL(kernel, grid, block, lds_bytes, stream, args);
     }
+    rc = hipGetLastError();
+    if (rc != hipSuccess || args.k_splits == 1) return rc;
+    const size_t plane = static_cast<size_t>(args.M) * args.N;
+    hipLaunchKernelGGL(gemm_bf16_skinny_reduce_kernel, dim3(static_cast<unsigned>((plane + 255) / 256)), dim3(256), 0, stream,
+                       reduce);
     return hipGetLastError();
 }
 
@@ -2077,6 +2135,8 @@ hipError_t launch_gemm_bf16(size_t m, size_t n, size_t k, const uint16_t *lhs, c
                             hipStream_t stream, bool rhs_packed)
 {
     if (m == 0 || n == 0) return hipSuccess;
+    if (gemv_bf16_applies(m, n, k, lhs, rhs))
+        return launch_gemv_bf16(m, n, k, lhs, rhs, rhs_packed, out_f32, out_bf16, epilogue, stream);
     GemmBf16Args args;
     args.A = lhs;
     args.B = rhs;
@@ -2109,7 +2169,7 @@ hipError_t launch_gemm_bf16(size_t m, size_t n, size_t k, const uint16_t *lhs, c
         // the skinny kernel's partial sums behind it as well, so that it does not move) and go on with B as k×n.
         workspace_offset = (k * n * sizeof(uint16_t) + 255) & ~static_cast<size_t>(255);
         SkinnyArgs probe;
-        const size_t behind = skinny ? plan_skinny(args, probe) : 0;
+        const size_t behind = skinny ? plan_skinny(args, probe) : fits_256 ? 0 : general_slice_bytes(m, n, k);
         void *workspace = nullptr;
         hipError_t rc = stream_workspace(stream, workspace_offset + behind, &workspace);
         if (rc != hipSuccess) return rc;
@@ -2139,7 +2199,7 @@ hipError_t launch_gemm_bf16(size_t m, size_t n, size_t k, const uint16_t *lhs, c
         if (narrow) return launch_256<128>(args, rhs_packed, stream, workspace_offset);
         return launch_256<256>(args, rhs_packed, stream, workspace_offset);
     }
-    return launch_tile<128, 128, 32>(args, vec, stream);
+    return launch_tile<128, 128, 32>(args, vec, stream, workspace_offset);
 }
 
 // out_f32 = (lhs·rhs + bias) + residual, out_ln = layer_norm(out_f32; gamma, beta, epsilon) rounded to bf16; rhs packed n×k.

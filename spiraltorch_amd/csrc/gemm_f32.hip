@@ -18,6 +18,7 @@
 #include "device_math.h"
 #include "kernels.h"
 
+#include <algorithm>
 #include <type_traits>
 
 namespace sthip {
@@ -34,6 +35,10 @@ struct GemmF32Args {
     int tiles_m, tiles_n;  // the grid is one-dimensional over (tile_m, tile_n)
     float scale;
     int activation;
+    // k-sliced form (few tiles, long k): workgroup (tile, blockIdx.y) covers k in [y·slice_k, (y+1)·slice_k) and writes
+    // its raw sums to plane y of C (the launch passes the workspace of partial planes as C, scale 1 and no bias,
+    // residual or activation); gemm_f32_slice_reduce_kernel adds the planes in order and applies the epilogue.
+    int slice_k = 0;  // 0: one slice, the whole of K
 };
 
 constexpr int kBK = 16;
@@ -88,7 +93,11 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_f32_kernel(GemmF32Args p)
     const int group_rows = min(p.tiles_m - first_m, GROUP_M);
     const int tile_m = first_m + in_group % group_rows, tile_n = in_group / group_rows;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
-    const int M = p.M, N = p.N, K = p.K;
+    const int M = p.M, N = p.N;
+    // This workgroup's k range [k_lo, K): K below is the END of the range, p.K stays the row stride of A.
+    const int k_lo = p.slice_k ? static_cast<int>(blockIdx.y) * p.slice_k : 0;
+    const int K = p.slice_k ? min(p.K, k_lo + p.slice_k) : p.K;
+    float *const C = p.C + static_cast<size_t>(blockIdx.y) * M * N;
 
     f32x16 acc[TM][TN];
 #pragma unroll
@@ -110,7 +119,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_f32_kernel(GemmF32Args p)
             const int f = tid + T * r;
             if (!AT) {
                 const int row = min(m0 + (f >> 2), M - 1), c4 = (f & 3) * 4;
-                a_src[r] = p.A + static_cast<size_t>(row) * K + c4;
+                a_src[r] = p.A + static_cast<size_t>(row) * p.K + c4;
             } else {
                 const int krow = f / (BM / 4), col = min(m0 + (f % (BM / 4)) * 4, M - 4);
                 a_src[r] = p.A + static_cast<size_t>(krow) * M + col;
@@ -123,7 +132,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_f32_kernel(GemmF32Args p)
             b_src[r] = p.B + static_cast<size_t>(krow) * N + col;
         }
     }
-    const int full_steps = K / kBK;  // k-tiles that lie completely inside K
+    const int full_steps = (K - k_lo) / kBK;  // k-tiles that lie completely inside the range
 
     auto load_fast = [&](int k0) {
 #pragma unroll
@@ -144,7 +153,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_f32_kernel(GemmF32Args p)
             if (A_VECS % T != 0 && f >= A_VECS) continue;
             if (!AT) {
                 const int row = f >> 2, c4 = (f & 3) * 4;
-                ra[r] = load_row4<VEC>(p.A, static_cast<size_t>(m0 + row) * K, k0 + c4, K, m0 + row < M);
+                ra[r] = load_row4<VEC>(p.A, static_cast<size_t>(m0 + row) * p.K, k0 + c4, K, m0 + row < M);
             } else {
                 const int krow = f / (BM / 4), c4 = (f % (BM / 4)) * 4;
                 ra[r] = load_row4<VEC>(p.A, static_cast<size_t>(k0 + krow) * M, m0 + c4, M, k0 + krow < K);
@@ -212,9 +221,9 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_f32_kernel(GemmF32Args p)
         }
     };
 
-    const int steps = (K + kBK - 1) / kBK;
+    const int steps = (K - k_lo + kBK - 1) / kBK;
     if (steps > 0) {
-        if (VEC && full_steps > 0) load_fast(0); else load_checked(0);
+        if (VEC && full_steps > 0) load_fast(k_lo); else load_checked(k_lo);
         store_lds(0);
     }
     __syncthreads();
@@ -222,7 +231,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_f32_kernel(GemmF32Args p)
     if (VEC) {
         // Steady state: the next k-tile lies completely inside K, so its loads need no checks.
         for (; t + 1 < full_steps; ++t) {
-            load_fast((t + 1) * kBK);
+            load_fast(k_lo + (t + 1) * kBK);
             compute(t & 1);
             store_lds((t + 1) & 1);
             __syncthreads();
@@ -230,7 +239,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_f32_kernel(GemmF32Args p)
     }
     for (; t < steps; ++t) {
         const bool more = t + 1 < steps;
-        if (more) load_checked((t + 1) * kBK);
+        if (more) load_checked(k_lo + (t + 1) * kBK);
         compute(t & 1);
         if (more) store_lds((t + 1) & 1);
         __syncthreads();
@@ -254,7 +263,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_f32_kernel(GemmF32Args p)
                         const size_t idx = static_cast<size_t>(row) * N + col;
                         float value = tile[r] * p.scale + bias;
                         if constexpr (decltype(has_residual)::value) value += p.residual[idx];
-                        p.C[idx] = act(value);
+                        C[idx] = act(value);
                     }
                 }
             }
@@ -262,14 +271,88 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_f32_kernel(GemmF32Args p)
     });
 }
 
+// Adds the partial planes of a k-sliced launch in slice order (so the result does not depend on scheduling) and applies
+// the epilogue.  One thread per output element; eight planes are requested together so the loads overlap.
+struct SliceReduceArgs {
+    const float *partial;
+    float *C;
+    const float *bias;
+    const float *residual;
+    size_t plane;
+    int N, slices;
+    float scale;
+    int activation;
+};
+__global__ __launch_bounds__(256) void gemm_f32_slice_reduce_kernel(SliceReduceArgs p)
+{
+    const size_t idx = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (idx >= p.plane) return;
+    float value = 0.0f;
+    for (int s0 = 0; s0 < p.slices; s0 += 8) {
+        float part[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) part[j] = (s0 + j < p.slices) ? p.partial[(s0 + j) * p.plane + idx] : 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) value += part[j];
+    }
+    value = value * p.scale + (p.bias ? p.bias[idx % p.N] : -0.0f);
+    if (p.residual) value += p.residual[idx];
+    p.C[idx] = apply_activation(value, p.activation);
+}
+
+// How many k-slices a launch of `tiles` workgroups, each walking `k_steps` k-tiles, is cut into: none while the tiles
+// alone give every other compute unit a workgroup; otherwise enough for about two workgroups per compute unit, each
+// slice keeping at least `min_steps` k-tiles, and the partial planes (written once, read once) staying below the
+// operands' bytes.
+size_t choose_k_slices(size_t m, size_t n, size_t k, size_t tiles, size_t k_steps, size_t min_steps)
+{
+    if (tiles > 128 || k_steps < 2 * min_steps) return 1;
+    size_t slices = std::min<size_t>(512 / tiles, k_steps / min_steps);
+    while (slices > 1 && slices * m * n * 2 > m * k + k * n) --slices;
+    return std::max<size_t>(slices, 1);
+}
+
+// Runs `launch(args)` k-sliced: partial planes in the stream's workspace, then the reduction with the epilogue.
+template <class Launch>
+hipError_t launch_k_sliced(GemmF32Args args, size_t slices, size_t k_steps, int bk, hipStream_t stream, Launch &&launch)
+{
+    const size_t steps_per_slice = (k_steps + slices - 1) / slices;
+    slices = (k_steps + steps_per_slice - 1) / steps_per_slice;
+    const size_t plane = static_cast<size_t>(args.M) * args.N;
+    void *workspace = nullptr;
+    hipError_t rc = stream_workspace(stream, slices * plane * sizeof(float), &workspace);
+    if (rc != hipSuccess) return rc;
+    SliceReduceArgs reduce;
+    reduce.partial = static_cast<const float *>(workspace);
+    reduce.C = args.C;
+    reduce.bias = args.bias;
+    reduce.residual = args.residual;
+    reduce.plane = plane;
+    reduce.N = args.N;
+    reduce.slices = static_cast<int>(slices);
+    reduce.scale = args.scale;
+    reduce.activation = args.activation;
+    args.C = static_cast<float *>(workspace);
+    args.bias = nullptr;
+    args.residual = nullptr;
+    args.scale = 1.0f;
+    args.activation = ST_HIP_ACT_NONE;
+    args.slice_k = static_cast<int>(steps_per_slice) * bk;
+    rc = launch(args, static_cast<unsigned>(slices));
+    if (rc != hipSuccess) return rc;
+    hipLaunchKernelGGL(gemm_f32_slice_reduce_kernel, dim3(static_cast<unsigned>((plane + 255) / 256)), dim3(256), 0, stream,
+                       reduce);
+    return hipGetLastError();
+}
+
 template <int BM, int BN, int WM, int WN>
-hipError_t launch_tile(GemmF32Args args, bool lhs_transposed, bool vec, hipStream_t stream)
+hipError_t launch_tile(GemmF32Args args, bool lhs_transposed, bool vec, hipStream_t stream, unsigned slices = 1)
 {
     args.tiles_n = (args.N + BN - 1) / BN;
     args.tiles_m = (args.M + BM - 1) / BM;
     const size_t tiles = static_cast<size_t>(args.tiles_n) * static_cast<size_t>(args.tiles_m);
     if (tiles > 0x7fffffffu) return hipErrorInvalidConfiguration;
-    const dim3 grid(static_cast<unsigned>(tiles));
+    const dim3 grid(static_cast<unsigned>(tiles), slices);
     const dim3 block(64 * WM * WN);
     if (lhs_transposed) {
         if (vec)
@@ -601,10 +684,13 @@ __global__ __launch_bounds__(256) void gemm_f32_ring_32x32_splitk_kernel(GemmF32
             for (int t = 0; t < 4; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kk][t], b[kk][t], acc, 0, 0, 0);
     };
 
-    const int steps = K / BK;
-    const int my_steps = steps > wave ? (steps - wave + 3) / 4 : 0;  // k-tiles wave, wave+4, ...
-    if (my_steps > 0) issue(std::integral_constant<int, 0>{}, wave);
-    if (my_steps > 1) issue(std::integral_constant<int, 1>{}, wave + 4);
+    // k-tiles of this workgroup: all of them, or slice blockIdx.y of a k-sliced launch.
+    const int slice_steps = p.slice_k / BK;
+    const int t0 = __builtin_amdgcn_readfirstlane(static_cast<int>(blockIdx.y) * slice_steps) + wave;
+    const int steps = p.slice_k ? min(K / BK - static_cast<int>(blockIdx.y) * slice_steps, slice_steps) : K / BK;
+    const int my_steps = steps > wave ? (steps - wave + 3) / 4 : 0;  // k-tiles t0, t0+4, ...
+    if (my_steps > 0) issue(std::integral_constant<int, 0>{}, t0);
+    if (my_steps > 1) issue(std::integral_constant<int, 1>{}, t0 + 4);
     ST_F32_WAIT_VMCNT(0);
     auto step = [&](auto slot_tag, int i) {
         constexpr int SLOT = decltype(slot_tag)::value;
@@ -612,7 +698,7 @@ __global__ __launch_bounds__(256) void gemm_f32_ring_32x32_splitk_kernel(GemmF32
         else ST_F32_WAIT_VMCNT(0);
         asm volatile("" ::: "memory");
         // slot (i+2)%3 was last read by this same wavefront in step i-1, whose reads have returned
-        if (i + 2 < my_steps) issue(std::integral_constant<int, (SLOT + 2) % RING>{}, wave + 4 * (i + 2));
+        if (i + 2 < my_steps) issue(std::integral_constant<int, (SLOT + 2) % RING>{}, t0 + 4 * (i + 2));
         compute(slot_tag);
     };
     int i = 0;
@@ -640,6 +726,7 @@ __global__ __launch_bounds__(256) void gemm_f32_ring_32x32_splitk_kernel(GemmF32
         const f32x4 v = *reinterpret_cast<const f32x4 *>(&partial[(w * 32 + row) * P_STRIDE + c4]);
         sum[0] += v[0]; sum[1] += v[1]; sum[2] += v[2]; sum[3] += v[3];
     }
+    float *const C = p.C + static_cast<size_t>(blockIdx.y) * M * N;
     if (m0 + row < M) {
         with_epilogue_ops(p.activation, p.residual != nullptr, [&](auto &&act, auto has_residual) {
 #pragma unroll
@@ -649,7 +736,7 @@ __global__ __launch_bounds__(256) void gemm_f32_ring_32x32_splitk_kernel(GemmF32
                 const size_t idx = static_cast<size_t>(m0 + row) * N + col;
                 float value = sum[e] * p.scale + (p.bias ? p.bias[col] : -0.0f);
                 if constexpr (decltype(has_residual)::value) value += p.residual[idx];
-                p.C[idx] = act(value);
+                C[idx] = act(value);
             }
         });
     }
@@ -660,8 +747,16 @@ hipError_t launch_splitk32(GemmF32Args args, hipStream_t stream)
     args.tiles_n = (args.N + 31) / 32;
     args.tiles_m = (args.M + 31) / 32;
     const size_t tiles = static_cast<size_t>(args.tiles_n) * static_cast<size_t>(args.tiles_m);
-    hipLaunchKernelGGL(gemm_f32_ring_32x32_splitk_kernel, dim3(static_cast<unsigned>(tiles)), dim3(256), 0, stream, args);
-    return hipGetLastError();
+    auto launch = [&](const GemmF32Args &a, unsigned slices) {
+        hipLaunchKernelGGL(gemm_f32_ring_32x32_splitk_kernel, dim3(static_cast<unsigned>(tiles), slices), dim3(256), 0, stream, a);
+        return hipGetLastError();
+    };
+    // A long k over few tiles (64×64×100000, 256×256×16384) is cut over workgroups as well: 64 k-tiles per slice keep
+    // 16 for each wavefront's ring.
+    const size_t k_steps = static_cast<size_t>(args.K) / 16;
+    const size_t slices = choose_k_slices(args.M, args.N, args.K, tiles, k_steps, 64);
+    if (slices > 1) return launch_k_sliced(args, slices, k_steps, 16, stream, launch);
+    return launch(args, 1);
 }
 
 hipError_t launch_ring(GemmF32Args args, bool lhs_transposed, bool rhs_packed, bool big, hipStream_t stream)
@@ -709,6 +804,7 @@ hipError_t launch_gemm_f32(size_t m, size_t n, size_t k, bool lhs_transposed, co
                            const float *rhs, float *out, const GemmEpilogue &epilogue, hipStream_t stream)
 {
     if (m == 0 || n == 0) return hipSuccess;
+    if (!lhs_transposed && gemv_f32_applies(m, n, k, lhs, rhs)) return launch_gemv_f32(m, n, k, lhs, rhs, out, epilogue, stream);
     GemmF32Args args;
     args.A = lhs;
     args.B = rhs;
@@ -741,6 +837,14 @@ hipError_t launch_gemm_f32(size_t m, size_t n, size_t k, bool lhs_transposed, co
         if (!lhs_transposed && tiles64 <= 256 && k >= 128) return launch_splitk32(args, stream);
         return launch_ring(args, lhs_transposed, false, big, stream);
     }
+    // Shapes the ring kernels do not take.  Few tiles and a long k (a matrix-vector product, n < 4, is the common case):
+    // k-sliced, so that the whole chip streams A and B.
+    const size_t tiles64 = ((m + 63) / 64) * ((n + 63) / 64), k_steps = (k + kBK - 1) / kBK;
+    const size_t slices = choose_k_slices(m, n, k, tiles64, k_steps, 32);
+    if (slices > 1)
+        return launch_k_sliced(args, slices, k_steps, kBK, stream, [&](const GemmF32Args &a, unsigned count) {
+            return launch_tile<64, 64, 2, 2>(a, lhs_transposed, vec, stream, count);
+        });
     return launch_tile<64, 64, 2, 2>(args, lhs_transposed, vec, stream);
 }
 

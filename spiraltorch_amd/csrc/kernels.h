@@ -19,6 +19,15 @@ hipError_t launch_gemm_f32(size_t m, size_t n, size_t k, bool lhs_transposed, co
                            const float *rhs, float *out, const GemmEpilogue &epilogue,
                            hipStream_t stream);
 
+// Matrix times a few columns (n <= 3 for f32, n <= 7 for bf16; 16-byte aligned operands, k a multiple of the 16-byte
+// vector): a stream over A, one wavefront or workgroup per row.  The tiled launchers route here when `*_applies`.
+bool gemv_f32_applies(size_t m, size_t n, size_t k, const float *lhs, const float *rhs);
+hipError_t launch_gemv_f32(size_t m, size_t n, size_t k, const float *lhs, const float *rhs, float *out,
+                           const GemmEpilogue &epilogue, hipStream_t stream);
+bool gemv_bf16_applies(size_t m, size_t n, size_t k, const uint16_t *lhs, const uint16_t *rhs);
+hipError_t launch_gemv_bf16(size_t m, size_t n, size_t k, const uint16_t *lhs, const uint16_t *rhs, bool rhs_packed,
+                            float *out_f32, uint16_t *out_bf16, const GemmEpilogue &epilogue, hipStream_t stream);
+
 // Same with B prepacked as n×k (column-major packing, crates/st-tensor/src/pure.rs:1285-1323).
 hipError_t launch_gemm_f32_packed(size_t m, size_t n, size_t k, const float *lhs, const float *packed_rhs,
                                   float *out, const GemmEpilogue &epilogue, hipStream_t stream);

@@ -130,6 +130,92 @@ __global__ __launch_bounds__(256) void layer_norm_vec_kernel(int rows, int cols,
     }
 }
 
+// Sum / maximum / minimum over a workgroup of THREADS threads: the butterfly inside each wavefront, then the wavefronts'
+// values added (compared) in wavefront order by every thread, so all threads hold the same result and it depends on
+// nothing but the shape.  `scratch` holds THREADS/64 values and may be reused after the call returns.
+template <int THREADS, class T, class Op>
+__device__ __forceinline__ T block_reduce(T v, T *scratch, Op op)
+{
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) v = op(v, __shfl_xor(v, offset));
+    __syncthreads();  // earlier readers of scratch are done
+    if ((threadIdx.x & 63) == 0) scratch[threadIdx.x >> 6] = v;
+    __syncthreads();
+    T total = scratch[0];
+#pragma unroll
+    for (int w = 1; w < THREADS / 64; ++w) total = op(total, scratch[w]);
+    return total;
+}
+
+// Long rows (more than 2048 values, or rows that are not 16-byte aligned): one workgroup per row, two sweeps over the
+// row (statistics, then the normalisation; the second sweep is served by the caches for rows of up to a few MB).
+template <int THREADS, bool VEC>
+__global__ __launch_bounds__(THREADS) void layer_norm_long_kernel(int cols, const float *x, const float *residual,
+                                                                  const float *gamma, const float *beta, float epsilon,
+                                                                  float *out_f32, uint16_t *out_bf16)
+{
+    __shared__ float scratch[THREADS / 64];
+    const int tid = threadIdx.x;
+    const size_t offset = static_cast<size_t>(blockIdx.x) * cols;
+    constexpr int W = VEC ? 4 : 1;
+    auto load = [&](int c, float (&v)[W]) {
+        if constexpr (VEC) {
+            const float4 t = *reinterpret_cast<const float4 *>(x + offset + c);
+            v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+            if (residual) {
+                const float4 q = *reinterpret_cast<const float4 *>(residual + offset + c);
+                v[0] += q.x; v[1] += q.y; v[2] += q.z; v[3] += q.w;
+            }
+        } else {
+            v[0] = x[offset + c];
+            if (residual) v[0] += residual[offset + c];
+        }
+    };
+    float sum = 0.0f, sumsq = 0.0f;
+#pragma unroll 4
+    for (int c = tid * W; c < cols; c += THREADS * W) {
+        float v[W];
+        load(c, v);
+#pragma unroll
+        for (int e = 0; e < W; ++e) {
+            sum += v[e];
+            sumsq = fmaf(v[e], v[e], sumsq);
+        }
+    }
+    auto add = [](float a, float b) { return a + b; };
+    sum = block_reduce<THREADS>(sum, scratch, add);
+    sumsq = block_reduce<THREADS>(sumsq, scratch, add);
+    const float cols_f = static_cast<float>(cols);
+    const float mean = sum / cols_f;
+    const float var = fmaxf(sumsq / cols_f - mean * mean, 0.0f);
+    const float denom = sqrtf(var + epsilon);
+    const float inv = 1.0f / denom;
+    auto quotient = [&](float a) {  // a / denom, correctly rounded (see layer_norm_vec_kernel)
+        const float q = a * inv;
+        return fmaf(fmaf(-q, denom, a), inv, q);
+    };
+#pragma unroll 4
+    for (int c = tid * W; c < cols; c += THREADS * W) {
+        float v[W], o[W];
+        load(c, v);
+#pragma unroll
+        for (int e = 0; e < W; ++e) o[e] = quotient(v[e] - mean) * gamma[c + e] + beta[c + e];
+        if constexpr (VEC) {
+            if (out_f32) *reinterpret_cast<float4 *>(out_f32 + offset + c) = make_float4(o[0], o[1], o[2], o[3]);
+            if (out_bf16) {
+                uint2 packed;
+                packed.x = pack_bf16x2_rne(o[0], o[1]);
+                packed.y = pack_bf16x2_rne(o[2], o[3]);
+                *reinterpret_cast<uint2 *>(out_bf16 + offset + c) = packed;
+            }
+        } else {
+            if (out_f32) out_f32[offset + c] = o[0];
+            if (out_bf16) out_bf16[offset + c] = f32_to_bf16_rne(o[0]);
+        }
+    }
+}
+
+
 // token_to_index + row gather, crates/st-nn/src/layers/embedding.rs:42-100,325-330.
 __global__ __launch_bounds__(256) void embedding_kernel(int tokens, int vocab, int dim, const float *token_ids,
                                                         const float *table, float *out)
@@ -333,6 +419,71 @@ __global__ __launch_bounds__(256) void row_softmax_vec_kernel(int rows, int cols
             if (found && !normal) o[e] = (c + e == candidate) ? 1.0f : 0.0f;
         }
         *reinterpret_cast<float4 *>(y + c) = make_float4(o[0], o[1], o[2], o[3]);
+    }
+}
+
+// Long rows: one workgroup per row, three sweeps (maximum and its first position; the sum of the weights; the output).
+template <int THREADS, bool VEC>
+__global__ __launch_bounds__(THREADS) void row_softmax_long_kernel(int cols, const float *in, float *out)
+{
+    __shared__ float scratch_f[THREADS / 64];
+    __shared__ int scratch_i[THREADS / 64];
+    const int tid = threadIdx.x;
+    const float *x = in + static_cast<size_t>(blockIdx.x) * cols;
+    float *y = out + static_cast<size_t>(blockIdx.x) * cols;
+    constexpr int W = VEC ? 4 : 1;
+    auto load = [&](int c, float (&v)[W]) {
+        if constexpr (VEC) {
+            const float4 t = *reinterpret_cast<const float4 *>(x + c);
+            v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+        } else {
+            v[0] = x[c];
+        }
+    };
+    float best = -INFINITY;
+    int best_index = 0x7fffffff;
+#pragma unroll 4
+    for (int c = tid * W; c < cols; c += THREADS * W) {  // ascending columns per thread: the first occurrence wins
+        float v[W];
+        load(c, v);
+#pragma unroll
+        for (int e = 0; e < W; ++e) {
+            if (v[e] != v[e]) continue;
+            if (best_index == 0x7fffffff || v[e] > best) {
+                best = v[e];
+                best_index = c + e;
+            }
+        }
+    }
+    const float row_max = block_reduce<THREADS>(best_index == 0x7fffffff ? -INFINITY : best, scratch_f,
+                                                [](float a, float b) { return fmaxf(a, b); });
+    const int candidate = block_reduce<THREADS>((best_index != 0x7fffffff && best == row_max) ? best_index : 0x7fffffff,
+                                                scratch_i, [](int a, int b) { return min(a, b); });
+    const bool found = candidate != 0x7fffffff;
+    const float base = (found && isfinite(row_max)) ? row_max : 0.0f;
+    float denom = 0.0f;
+#pragma unroll 4
+    for (int c = tid * W; c < cols; c += THREADS * W) {
+        float v[W];
+        load(c, v);
+#pragma unroll
+        for (int e = 0; e < W; ++e) denom += (!found || v[e] != v[e]) ? 0.0f : __expf(v[e] - base);
+    }
+    denom = block_reduce<THREADS>(denom, scratch_f, [](float a, float b) { return a + b; });
+    const bool normal = isfinite(denom) && denom > 1.1920929e-7f;
+    const float inv = normal ? 1.0f / denom : 0.0f;
+#pragma unroll 4
+    for (int c = tid * W; c < cols; c += THREADS * W) {
+        float v[W], o[W];
+        load(c, v);
+#pragma unroll
+        for (int e = 0; e < W; ++e) {
+            const float weight = (!found || v[e] != v[e]) ? 0.0f : __expf(v[e] - base);
+            o[e] = weight * inv;
+            if (found && !normal) o[e] = (c + e == candidate) ? 1.0f : 0.0f;
+        }
+        if constexpr (VEC) *reinterpret_cast<float4 *>(y + c) = make_float4(o[0], o[1], o[2], o[3]);
+        else y[c] = o[0];
     }
 }
 
@@ -570,7 +721,18 @@ hipError_t launch_layer_norm_f32(size_t rows, size_t cols, const float *x, const
     else if (vec)
         hipLaunchKernelGGL((layer_norm_vec_kernel<8, 1>), grid, block, 0, stream, r, c, x, residual, gamma, beta, epsilon,
                            out_f32, out_bf16);
-    else
+    else if (cols > 2048) {
+        // A workgroup per row: 1024 threads while the rows are few, 256 once the rows alone fill the chip.
+        const bool vec_long = cols % 4 == 0 && aligned(x, 16) && aligned(residual, 16) && aligned(out_f32, 16) && aligned(out_bf16, 8);
+        const dim3 rows_grid(static_cast<unsigned>(rows));
+        if (rows < 2048) {
+            if (vec_long) hipLaunchKernelGGL((layer_norm_long_kernel<1024, true>), rows_grid, dim3(1024), 0, stream, c, x, residual, gamma, beta, epsilon, out_f32, out_bf16);
+            else hipLaunchKernelGGL((layer_norm_long_kernel<1024, false>), rows_grid, dim3(1024), 0, stream, c, x, residual, gamma, beta, epsilon, out_f32, out_bf16);
+        } else {
+            if (vec_long) hipLaunchKernelGGL((layer_norm_long_kernel<256, true>), rows_grid, dim3(256), 0, stream, c, x, residual, gamma, beta, epsilon, out_f32, out_bf16);
+            else hipLaunchKernelGGL((layer_norm_long_kernel<256, false>), rows_grid, dim3(256), 0, stream, c, x, residual, gamma, beta, epsilon, out_f32, out_bf16);
+        }
+    } else
         hipLaunchKernelGGL(layer_norm_kernel, grid, block, 0, stream, r, c, x, residual, gamma, beta, epsilon, out_f32,
                            out_bf16);
     return hipGetLastError();
@@ -641,7 +803,18 @@ hipError_t launch_row_softmax_f32(size_t rows, size_t cols, const float *in, flo
         hipLaunchKernelGGL(row_softmax_vec_kernel<4>, grid, block, 0, stream, r, c, in, out);
     else if (vec)
         hipLaunchKernelGGL(row_softmax_vec_kernel<8>, grid, block, 0, stream, r, c, in, out);
-    else
+    else if (cols > 2048) {
+        // A workgroup per row: 1024 threads while the rows are few, 256 once the rows alone fill the chip.
+        const bool vec_long = cols % 4 == 0 && ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0;
+        const dim3 rows_grid(static_cast<unsigned>(rows));
+        if (rows < 2048) {
+            if (vec_long) hipLaunchKernelGGL((row_softmax_long_kernel<1024, true>), rows_grid, dim3(1024), 0, stream, c, in, out);
+            else hipLaunchKernelGGL((row_softmax_long_kernel<1024, false>), rows_grid, dim3(1024), 0, stream, c, in, out);
+        } else {
+            if (vec_long) hipLaunchKernelGGL((row_softmax_long_kernel<256, true>), rows_grid, dim3(256), 0, stream, c, in, out);
+            else hipLaunchKernelGGL((row_softmax_long_kernel<256, false>), rows_grid, dim3(256), 0, stream, c, in, out);
+        }
+    } else
         hipLaunchKernelGGL(row_softmax_kernel, grid, block, 0, stream, r, c, in, out);
     return hipGetLastError();
 }

@@ -12,7 +12,9 @@ def test_layer_norm(hip, oracle):
     rng = np.random.default_rng(4)
     # (16384 rows and more: two rows per wavefront, odd row counts leave the last wavefront half empty)
     for rows, cols in ((1, 1), (5, 48), (130, 512), (7, 1000), (9, 1536), (3, 2048), (4, 2052), (6, 4100), (16384, 512),
-                       (16387, 256), (16389, 1024)):
+                       (16387, 256), (16389, 1024),
+                       # rows longer than 2048: a workgroup per row (1024 threads; 256 from 2048 rows on)
+                       (3, 100000), (2, 50001), (2100, 2056), (2049, 2051)):
         x = rng.normal(1.0, 2.0, rows * cols).astype(np.float32)
         res = rng.normal(size=rows * cols).astype(np.float32)
         g, b = rng.normal(size=cols).astype(np.float32), rng.normal(size=cols).astype(np.float32)
@@ -22,7 +24,16 @@ def test_layer_norm(hip, oracle):
             hip.layer_norm_f32_dev(rows, cols, d["x"], dr, d["g"], d["b"], 1e-5, o32, o16)
             hip.device_synchronize()
             got = o32.to_array(np.float32, rows * cols)
-            assert_close(got, oracle.layer_norm_f32(rows, cols, x, g, b, 1e-5, residual), F32_REL, 2e-5, "layer norm")
+            want = oracle.layer_norm_f32(rows, cols, x, g, b, 1e-5, residual)
+            if cols > 20000:
+                # Sequential f32 sums over this many values (the oracle's, like the reference's) carry more error than
+                # the bar allows; the kernel's tree of partial sums is held to float64 statistics instead.
+                assert_close(got, want, 1e-3, 1e-3, "layer norm against sequential f32 statistics")
+                v = (x.astype(np.float64) + (0 if residual is None else residual)).reshape(rows, cols)
+                mean = v.mean(axis=1, keepdims=True)
+                var = np.maximum((v * v).mean(axis=1, keepdims=True) - mean * mean, 0.0)
+                want = (((v - mean) / np.sqrt(var + 1e-5)) * g + b).ravel()
+            assert_close(got, want, F32_REL, 2e-5, "layer norm")
             assert (o16.to_array(np.uint16, rows * cols) == inputs.to_bf16(got)).all()
 
 

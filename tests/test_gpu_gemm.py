@@ -128,6 +128,53 @@ def test_long_reduction_against_float64(hip):
     assert (np.abs(out.reshape(m, n) - exact) <= bound).all()
 
 
+@pytest.mark.parametrize("m,n,k,lhs_t", [
+    (64, 64, 20000, False),    # 32x32 tiles, k cut over workgroups as well as over a workgroup's wavefronts
+    (256, 256, 8192, False),
+    (40, 36, 2064, False),     # the last slice shorter than the others
+    (4096, 1, 4096, False),    # matrix-vector: one wavefront per row of A
+    (300, 3, 2048, False),     # few rows: a workgroup per row
+    (5000, 2, 260, False),
+    (64, 1, 64, False),
+    (1000, 3, 1028, False),
+    (2050, 1, 4099, False),    # k not a multiple of 4: the general tile kernel, k-sliced
+    (300, 3, 2049, False),     # ragged k: the last slice ends inside a k-tile
+    (1030, 2, 1100, True),     # A stored transposed
+    (130, 70, 5000, True),
+])
+def test_k_sliced_launches_against_float64(hip, m, n, k, lhs_t):
+    """Few output tiles and a long k: the launch is cut along k over workgroups, the partial planes are added in slice
+    order and the epilogue runs in the reduction.  Bound as in test_long_reduction_against_float64."""
+    rng = np.random.default_rng(m + n + k)
+    a = rng.uniform(-1, 1, m * k).astype(np.float32)
+    b = rng.uniform(-1, 1, k * n).astype(np.float32)
+    bias = rng.uniform(-1, 1, n).astype(np.float32)
+    res = rng.uniform(-1, 1, m * n).astype(np.float32)
+    a64 = (a.reshape(k, m).T if lhs_t else a.reshape(m, k)).astype(np.float64)
+    b64 = b.astype(np.float64).reshape(k, n)
+    exact = a64 @ b64
+    slack = 2e-7 * (np.abs(a64) @ np.abs(b64))
+    out = np.full(m * n, np.nan, np.float32)
+    if lhs_t:
+        hip.gemm_lhs_transpose_scaled_f32(m, n, k, 0.25, a, b, out)
+        want = 0.25 * exact
+        assert (np.abs(out.reshape(m, n) - want) <= 1e-4 * np.abs(want) + 1e-5 + slack).all()
+        return
+    hip.gemm_scaled_f32(m, n, k, -0.5, a, b, out)
+    want = -0.5 * exact
+    assert (np.abs(out.reshape(m, n) - want) <= 1e-4 * np.abs(want) + 1e-5 + slack).all()
+    twice = np.zeros(m * n, np.float32)
+    hip.gemm_scaled_f32(m, n, k, -0.5, a, b, twice)
+    assert (twice == out).all(), "the slices are added in a fixed order"
+    hip.gemm_bias_activation_f32(m, n, k, hip.GemmActivation.Relu, a, b, bias, res, out)
+    want = np.maximum(exact + bias.astype(np.float64)[None, :] + res.astype(np.float64).reshape(m, n), 0.0)
+    assert (np.abs(out.reshape(m, n) - want) <= 1e-4 * np.abs(want) + 1e-5 + slack).all()
+    hip.gemm_bias_activation_f32(m, n, k, hip.GemmActivation.Gelu, a, b, bias, None, out)
+    pre = exact + bias.astype(np.float64)[None, :]
+    want = 0.5 * pre * (1.0 + np.tanh(np.sqrt(2.0 / np.pi) * (pre + 0.044715 * pre ** 3)))
+    assert (np.abs(out.reshape(m, n) - want) <= 1e-4 * np.abs(want) + 2e-5 + 2 * slack).all()
+
+
 def test_config1_512_cubed(hip, oracle):
     """BASELINE config 1: f32 C = A.B, M=N=K=512, U[-1,1) from the fixed seeds."""
     from spiraltorch_amd import inputs

@@ -279,9 +279,13 @@ def test_gemm_residual_layer_norm(hip, oracle, m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(100, 4096, 4096), (256, 1024, 4096), (130, 2048, 2048), (65, 128, 8192), (4096, 128, 4096),
-                                   (300, 384, 1984)])
+                                   (300, 384, 1984),
+                                   # shapes of the general 128x128 kernel (n not a multiple of 128), k-sliced the same way
+                                   (64, 64, 20000), (4096, 16, 4096), (4096, 1, 4100), (300, 72, 3000), (130, 136, 1064),
+                                   # at most 8 columns: a stream over A, one wavefront or workgroup per row
+                                   (4096, 8, 4096), (4096, 1, 4096), (300, 5, 4096), (1000, 7, 520), (64, 3, 64), (5000, 2, 264)])
 def test_few_tiles_with_a_long_k_split_k(hip, oracle, m, n, k):
-    """Launches of few 256-row tiles with many k-tiles split k over workgroups (raw partial sums, added in split order by
+    """Launches of few tiles with many k-tiles split k over workgroups (raw partial sums, added in split order by
     a second kernel that applies the epilogue): both layouts of B, the fused epilogue with both output types, and the
     same bits from call to call and from either layout."""
     from spiraltorch_amd import inputs
