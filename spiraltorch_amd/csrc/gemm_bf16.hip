@@ -55,6 +55,12 @@ __device__ __forceinline__ uint4 load_row8(const uint16_t *base, size_t row_offs
     const uint16_t *src = base + row_offset + col;
     if (VEC) {
         if (col < col_limit) v = *reinterpret_cast<const uint4 *>(src);
+    } else if (col + 8 <= col_limit) {
+        // Eight values inside the row at any 2-byte alignment: still one 16-byte load (global memory takes wide
+        // accesses at any alignment; the type says so, and the compiler keeps the single instruction).
+        typedef uint32_t u32x4_a2 __attribute__((ext_vector_type(4), aligned(2)));
+        const u32x4_a2 w = *reinterpret_cast<const u32x4_a2 *>(src);
+        v = make_uint4(w[0], w[1], w[2], w[3]);
     } else {
         uint16_t e[8];
 #pragma unroll
@@ -427,10 +433,90 @@ __device__ __forceinline__ void gemm_bf16_epilogue_rows(const GemmBf16Args &p, c
     else gemm_bf16_epilogue_act<WTN, TM, ACT, false>(p, acc, lds, wave, row_first, col_base, lane);
 }
 
+// Epilogue for an N that is not a multiple of 128 (a vocabulary of 50257, 1000 classes): the rows of C, of the residual
+// and the pieces of the bias start at any 4-byte (f32) or 2-byte (bf16) boundary and the last tile hangs over the end.
+// Same f32 strips through LDS as above; the four columns a lane owns are stored as one 16-byte (f32) / 8-byte (bf16)
+// access where they all exist — global memory takes those at any alignment, and the types say so — and one by one in
+// the last piece of a row.  Everything per launch is a run-time value here: this path is bound by its stores.
+template <int WTN, int TM>
+__device__ __forceinline__ void gemm_bf16_epilogue_ragged(const GemmBf16Args &p, const f32x16 (&acc)[TM][WTN / 32],
+                                                          unsigned char *lds, int wave, int row_first, int col_base, int lane)
+{
+    typedef float f32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+    typedef uint32_t u32x2_a2 __attribute__((ext_vector_type(2), aligned(2)));
+    constexpr int TN = WTN / 32;
+    const int li = lane & 31, lh = lane >> 5;
+    const int M = p.M, N = p.N;
+    const float scale = p.scale;
+    constexpr int C_STRIDE = WTN + 4;
+    float *strip = reinterpret_cast<float *>(lds) + wave * (32 * C_STRIDE);
+    constexpr int LPR = WTN / 4;
+    constexpr int ROWS_PER_PASS = 64 / LPR;
+    constexpr int PASSES = 32 / ROWS_PER_PASS;
+    const int col0 = col_base + (lane & (LPR - 1)) * 4;
+    const bool whole = col0 + 4 <= N;  // all four columns exist
+    float bias[4] = {-0.0f, -0.0f, -0.0f, -0.0f};
+    if (p.bias) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (col0 + e < N) bias[e] = p.bias[col0 + e];
+    }
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) {
+        const int row_base = row_first + tm * 32;
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn) {
+            const f32x16 tile = acc[tm][tn];
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+                *reinterpret_cast<float4 *>(&strip[li * C_STRIDE + tn * 32 + g * 8 + lh * 4]) =
+                    make_float4(tile[4 * g], tile[4 * g + 1], tile[4 * g + 2], tile[4 * g + 3]);
+        }
+#pragma unroll
+        for (int j = 0; j < PASSES; ++j) {
+            const int local_row = j * ROWS_PER_PASS + lane / LPR;
+            const int row = row_base + local_row;
+            const float4 s4 = *reinterpret_cast<const float4 *>(&strip[local_row * C_STRIDE + (lane & (LPR - 1)) * 4]);
+            if (row >= M || col0 >= N) continue;
+            const size_t idx = static_cast<size_t>(row) * N + col0;
+            float v[4] = {s4.x, s4.y, s4.z, s4.w};
+            float res[4] = {0.f, 0.f, 0.f, 0.f};
+            if (p.residual) {
+                if (whole) {
+                    const f32x4_a4 r4 = *reinterpret_cast<const f32x4_a4 *>(p.residual + idx);
+                    res[0] = r4[0]; res[1] = r4[1]; res[2] = r4[2]; res[3] = r4[3];
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (col0 + e < N) res[e] = p.residual[idx + e];
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                float value = v[e] * scale + bias[e];
+                if (p.residual) value += res[e];
+                v[e] = apply_activation(value, p.activation);
+            }
+            if (whole) {
+                if (p.C32) *reinterpret_cast<f32x4_a4 *>(p.C32 + idx) = f32x4_a4{v[0], v[1], v[2], v[3]};
+                if (p.C16) *reinterpret_cast<u32x2_a2 *>(p.C16 + idx) = u32x2_a2{pack_bf16x2_rne(v[0], v[1]), pack_bf16x2_rne(v[2], v[3])};
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    if (col0 + e >= N) continue;
+                    if (p.C32) p.C32[idx + e] = v[e];
+                    if (p.C16) p.C16[idx + e] = f32_to_bf16_rne(v[e]);
+                }
+            }
+        }
+    }
+}
+
 template <int WTN, int TM = 2>
 __device__ __forceinline__ void gemm_bf16_epilogue(const GemmBf16Args &p, const f32x16 (&acc)[TM][WTN / 32], unsigned char *lds,
                                                    int wave, int row_first, int col_base, int lane)
 {
+    if (p.N & 127) return gemm_bf16_epilogue_ragged<WTN, TM>(p, acc, lds, wave, row_first, col_base, lane);
     if (p.activation == ST_HIP_ACT_GELU) gemm_bf16_epilogue_rows<WTN, TM, ST_HIP_ACT_GELU>(p, acc, lds, wave, row_first, col_base, lane);
     else if (p.activation == ST_HIP_ACT_RELU) gemm_bf16_epilogue_rows<WTN, TM, ST_HIP_ACT_RELU>(p, acc, lds, wave, row_first, col_base, lane);
     else gemm_bf16_epilogue_rows<WTN, TM, ST_HIP_ACT_NONE>(p, acc, lds, wave, row_first, col_base, lane);
@@ -1932,9 +2018,13 @@ TilePlan plan_tiles(size_t m, size_t n, size_t k)
 {
     auto fill = [](size_t tiles) { return static_cast<double>(tiles) / static_cast<double>((tiles + 255) / 256 * 256); };
     const size_t row_tiles = (m + 255) / 256;
+    // An n that is not a multiple of 128 hangs over the last tile either way; 256-wide tiles then only cost more when
+    // they add a whole empty 128-column block to a narrow matrix.
+    const size_t cols128 = (n + 127) / 128, cols256 = (n + 255) / 256;
+    const bool wide_fits = n % 256 == 0 || (n % 128 != 0 && (cols128 % 2 == 0 || cols128 >= 16));
     TilePlan plan;
-    plan.narrow = n % 256 != 0 || fill(row_tiles * (n / 128)) > 1.15 * fill(row_tiles * (n / 256));
-    plan.tiles = row_tiles * (n / (plan.narrow ? 128 : 256));
+    plan.narrow = !wide_fits || fill(row_tiles * cols128) > 1.15 * fill(row_tiles * cols256);
+    plan.tiles = row_tiles * (plan.narrow ? cols128 : cols256);
     plan.k_splits = choose_k_splits(m, n, k, plan.tiles);
     return plan;
 }
@@ -1943,7 +2033,7 @@ template <int BN>
 hipError_t launch_256(GemmBf16Args args, bool packed, hipStream_t stream, size_t workspace_offset)
 {
     args.tiles_m = (args.M + 255) / 256;
-    args.tiles_n = args.N / BN;
+    args.tiles_n = (args.N + BN - 1) / BN;  // the packed kernels take a ragged N: rows of Bᵀ past it read as zero
     size_t tiles = static_cast<size_t>(args.tiles_m) * static_cast<size_t>(args.tiles_n);
     if (tiles > 0x7fffffffu) return hipErrorInvalidConfiguration;
     const size_t k_tiles = static_cast<size_t>(args.K) / 64;
@@ -1990,7 +2080,7 @@ hipError_t launch_256(GemmBf16Args args, bool packed, hipStream_t stream, size_t
 hipError_t launch_128(GemmBf16Args args, bool packed, hipStream_t stream)
 {
     args.tiles_m = (args.M + 127) / 128;
-    args.tiles_n = args.N / 128;
+    args.tiles_n = (args.N + 127) / 128;
     const size_t tiles = static_cast<size_t>(args.tiles_m) * static_cast<size_t>(args.tiles_n);
     if (tiles > 0x7fffffffu) return hipErrorInvalidConfiguration;
     args.swizzle = (tiles % 8 == 0) ? 1 : 0;
@@ -2164,6 +2254,29 @@ hipError_t launch_gemm_bf16(size_t m, size_t n, size_t k, const uint16_t *lhs, c
         fits_buffer)
         return launch_skinny_packed(args, stream);
     size_t workspace_offset = 0;
+    // An n that is not a multiple of 128 (a vocabulary of 50257, 1000 classes) with a k the 256-row kernels take: the
+    // packed kernels run it as it is — rows of Bᵀ past n read as zero through the buffer range check, and the epilogue
+    // for a ragged n stores at any alignment.  A row-major B is packed into the stream's workspace first (one pass
+    // over B, a few per cent of such a product) — its rows start at odd addresses, which the direct-to-LDS loads do
+    // not take.  (4096×50257×768: 3455 µs on the general kernel.)
+    if (n % 128 != 0 && n > 128 && m > 64 && k >= 64 && k % 64 == 0 && aligned16(lhs) && fits_buffer &&
+        (!rhs_packed || aligned16(rhs))) {
+        const TilePlan plan = plan_tiles(m, n, k);
+        if (!rhs_packed) {
+            workspace_offset = (k * n * sizeof(uint16_t) + 255) & ~static_cast<size_t>(255);
+            const size_t behind = plan.k_splits > 1 ? plan.k_splits * m * n * sizeof(float) : 0;
+            void *workspace = nullptr;
+            hipError_t rc = stream_workspace(stream, workspace_offset + behind, &workspace);
+            if (rc != hipSuccess) return rc;
+            rc = launch_transpose_u16(k, n, rhs, static_cast<uint16_t *>(workspace), stream);
+            if (rc != hipSuccess) return rc;
+            args.B = static_cast<const uint16_t *>(workspace);
+        }
+        const size_t tiles_128 = ((m + 127) / 128) * ((n + 127) / 128);
+        if (plan.tiles < 192 && tiles_128 >= 2 * plan.tiles && plan.k_splits == 1) return launch_128(args, true, stream);
+        if (plan.narrow) return launch_256<128>(args, true, stream, workspace_offset);
+        return launch_256<256>(args, true, stream, workspace_offset);
+    }
     if (rhs_packed && (!fits_256 || skinny) && k > 0) {
         // Shapes the packed 256-row kernels do not take: unpack B into the front of the stream's workspace (sized for
         // the skinny kernel's partial sums behind it as well, so that it does not move) and go on with B as k×n.

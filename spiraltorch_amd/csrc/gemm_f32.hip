@@ -52,6 +52,12 @@ __device__ __forceinline__ float4 load_row4(const float *base, size_t row_offset
     const float *src = base + row_offset + col;
     if (VEC) {
         if (col < col_limit) v = *reinterpret_cast<const float4 *>(src);
+    } else if (col + 4 <= col_limit) {
+        // Four values inside the row at any 4-byte alignment: still one 16-byte load (global memory takes wide
+        // accesses at any alignment; the type says so, and the compiler keeps the single instruction).
+        typedef float f32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+        const f32x4_a4 w = *reinterpret_cast<const f32x4_a4 *>(src);
+        v = make_float4(w[0], w[1], w[2], w[3]);
     } else {
         if (col + 0 < col_limit) v.x = src[0];
         if (col + 1 < col_limit) v.y = src[1];

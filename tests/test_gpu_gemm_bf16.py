@@ -135,7 +135,9 @@ def test_fused_epilogue_and_bf16_output(hip, oracle, m, n, k):
                                           (8192 - 37, 2048, 128, 1), (16384 - 5, 768, 64, 1),
                                           # few tiles: the same kernels serve every shape they can address
                                           (65, 128, 64, 1), (300, 384, 192, 1), (257, 256, 64, 1), (512, 512, 512, 0),
-                                          (100, 1152, 320, 1)])
+                                          (100, 1152, 320, 1),
+                                          # n not a multiple of 128: the row-major B is packed on the way in
+                                          (2048, 1003, 128, 0), (777, 1500, 256, 1), (300, 2052, 64, 1)])
 def test_large_tile_kernels_with_epilogue(hip, oracle, m, n, k, ragged):
     """Shapes that take the 256x256 and 256x128 tile kernels, with bias + residual + GELU and
     both output types; m may be ragged."""
@@ -162,6 +164,9 @@ PACKED_SHAPES = [
     # m, n, k — the packed 256-row kernels (k % 64 == 0, n % 128 == 0), full and ragged in m, one to many k-tiles
     (256, 256, 64), (512, 512, 512), (300, 384, 192), (8192 - 37, 2048, 128), (16384, 512, 192), (257, 256, 1024),
     (100, 1152, 320), (4096, 128, 4096),
+    # n not a multiple of 128 (rows of the packed B past n read as zero, stores at any alignment): 128- and 256-wide
+    # tiles, an odd n, k split over workgroups, one long row of tiles
+    (300, 1000, 192), (1024, 257, 64), (513, 2051, 128), (4096, 129, 4096), (200, 50257, 64), (130, 3000, 1024),
     # shapes they do not take: unpacked on the device first (general kernel, skinny split-k kernel)
     (33, 40, 72), (130, 136, 264), (5, 7, 9), (16, 384, 320), (64, 128, 1024), (1, 8, 8),
 ]
