@@ -2227,6 +2227,20 @@ hipError_t launch_gemm_bf16(size_t m, size_t n, size_t k, const uint16_t *lhs, c
     if (m == 0 || n == 0) return hipSuccess;
     if (gemv_bf16_applies(m, n, k, lhs, rhs))
         return launch_gemv_bf16(m, n, k, lhs, rhs, rhs_packed, out_f32, out_bf16, epilogue, stream);
+    // An A of 2 GiB or more (the 256-row kernels address their operands through 32-bit byte offsets): row blocks of A
+    // are independent products, so the launch is cut into blocks that fit and each takes the fast path.
+    if (m * k * sizeof(uint16_t) >= (1ull << 31) && k > 0 && k * 256 * sizeof(uint16_t) < (1ull << 31)) {
+        const size_t block = ((1ull << 31) / (k * sizeof(uint16_t)) - 1) / 256 * 256;
+        for (size_t row = 0; row < m; row += block) {
+            const size_t rows = std::min(block, m - row);
+            GemmEpilogue part = epilogue;
+            if (part.residual) part.residual += row * n;
+            const hipError_t rc = launch_gemm_bf16(rows, n, k, lhs + row * k, rhs, out_f32 ? out_f32 + row * n : nullptr,
+                                                   out_bf16 ? out_bf16 + row * n : nullptr, part, stream, rhs_packed);
+            if (rc != hipSuccess) return rc;
+        }
+        return hipSuccess;
+    }
     GemmBf16Args args;
     args.A = lhs;
     args.B = rhs;

@@ -811,6 +811,19 @@ hipError_t launch_gemm_f32(size_t m, size_t n, size_t k, bool lhs_transposed, co
 {
     if (m == 0 || n == 0) return hipSuccess;
     if (!lhs_transposed && gemv_f32_applies(m, n, k, lhs, rhs)) return launch_gemv_f32(m, n, k, lhs, rhs, out, epilogue, stream);
+    // An A of 2 GiB or more (the direct-to-LDS kernels address their operands through 32-bit byte offsets): row blocks
+    // of A are independent products, so the launch is cut into blocks that fit and each takes the fast path.
+    if (!lhs_transposed && m * k * sizeof(float) >= (1ull << 31) && k > 0 && k * 256 * sizeof(float) < (1ull << 31)) {
+        const size_t block = ((1ull << 31) / (k * sizeof(float)) - 1) / 256 * 256;
+        for (size_t row = 0; row < m; row += block) {
+            const size_t rows = std::min(block, m - row);
+            GemmEpilogue part = epilogue;
+            if (part.residual) part.residual += row * n;
+            const hipError_t rc = launch_gemm_f32(rows, n, k, false, lhs + row * k, rhs, out + row * n, part, stream);
+            if (rc != hipSuccess) return rc;
+        }
+        return hipSuccess;
+    }
     GemmF32Args args;
     args.A = lhs;
     args.B = rhs;

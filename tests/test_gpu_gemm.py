@@ -175,6 +175,26 @@ def test_k_sliced_launches_against_float64(hip, m, n, k, lhs_t):
     assert (np.abs(out.reshape(m, n) - want) <= 1e-4 * np.abs(want) + 2e-5 + 2 * slack).all()
 
 
+def test_lhs_of_more_than_2_gib(hip):
+    """An A beyond 2^31 bytes is cut into row blocks the 32-bit-offset kernels can address; rows on both sides of the
+    cut and at both ends are checked against float64."""
+    m, n, k = 525000, 64, 1024
+    rng = np.random.default_rng(3)
+    a = rng.random(m * k, dtype=np.float32) - 0.5
+    b = rng.random(k * n, dtype=np.float32) - 0.5
+    bias = rng.random(n, dtype=np.float32)
+    d_a, d_b, d_bias = (hip.DeviceBuffer.from_array(v) for v in (a, b, bias))
+    d_out = hip.DeviceBuffer(m * n * 4)
+    hip.gemm_bias_act_f32_dev(m, n, k, hip.GemmActivation.Relu, d_a, d_b, d_bias, None, d_out)
+    hip.device_synchronize()
+    got = d_out.to_array(np.float32, m * n).reshape(m, n)
+    cut = ((1 << 31) // (k * 4) - 1) // 256 * 256
+    rows = np.r_[0:3, cut - 3:cut + 3, m - 3:m, rng.integers(0, m, 40)]
+    want = np.maximum(a.reshape(m, k)[rows].astype(np.float64) @ b.reshape(k, n).astype(np.float64) + bias, 0.0)
+    assert_close(got[rows], want, F32_REL, 2e-5, "rows of a 2.15 GB lhs")
+    assert np.isfinite(got).all() and (got >= 0).all()
+
+
 def test_config1_512_cubed(hip, oracle):
     """BASELINE config 1: f32 C = A.B, M=N=K=512, U[-1,1) from the fixed seeds."""
     from spiraltorch_amd import inputs

@@ -421,6 +421,29 @@ def test_config4_4096_cubed_prepacked(hip, oracle):
     assert (d_ref.to_array(np.float32, (n, n)) == 2 * out).all()
 
 
+def test_lhs_of_more_than_2_gib(hip):
+    """An A beyond 2^31 bytes is cut into row blocks the 32-bit-offset kernels can address; rows on both sides of the
+    cut and at both ends are checked against float64, for both outputs."""
+    from spiraltorch_amd import inputs
+    m, n, k = 1050000, 128, 1024
+    rng = np.random.default_rng(4)
+    a = inputs.to_bf16(rng.random(m * k, dtype=np.float32) - 0.5)
+    b = inputs.to_bf16(rng.random(k * n, dtype=np.float32) - 0.5)
+    bias = rng.random(n, dtype=np.float32)
+    d_a, d_b, d_bias = (hip.DeviceBuffer.from_array(v) for v in (a, b, bias))
+    d32, d16 = hip.DeviceBuffer(m * n * 4), hip.DeviceBuffer(m * n * 2)
+    hip.gemm_bf16_bias_act_dev(m, n, k, 0, d_a, d_b, d_bias, None, d32, d16)
+    hip.device_synchronize()
+    got = d32.to_array(np.float32, m * n).reshape(m, n)
+    cut = ((1 << 31) // (k * 2) - 1) // 256 * 256
+    rows = np.r_[0:3, cut - 3:cut + 3, m - 3:m, rng.integers(0, m, 40)]
+    want = inputs.from_bf16(a.reshape(m, k)[rows]).astype(np.float64) @ inputs.from_bf16(b).reshape(k, n).astype(np.float64) + bias
+    assert_close(got[rows], want, 1e-4, 2e-5, "rows of a 2.15 GB lhs")
+    got16 = d16.to_array(np.uint16, m * n).reshape(m, n)
+    assert (got16[rows] == inputs.to_bf16(got[rows].ravel()).reshape(len(rows), n)).all()
+    assert np.isfinite(got).all()
+
+
 def test_validation(hip):
     out = np.full(4, 13.0, np.float32)
     with pytest.raises(hip.HipErr, match="lhs buffer length 4 does not match m\\*k=6"):
