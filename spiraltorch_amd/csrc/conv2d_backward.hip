@@ -529,7 +529,7 @@ hipError_t launch_conv2d_grad_input_f32(const ConvShape &shape, const float *gra
             for (size_t i = 0; i < images; ++i) {
                 // cols_i (OH·OW × S) = G_iᵀ · W with G_i = grad_output of the image, C_out × OH·OW (k × m), W = C_out × S
                 rc = launch_gemm_f32(m, S, static_cast<size_t>(shape.c_out), true, grad_output + (first + i) * shape.c_out * m,
-                                     weight, cols + i * image_cols, plain, stream);
+                                     weight, cols + i * image_cols, plain, stream, /*scratch_free=*/false);  // cols live there
                 if (rc != hipSuccess) return rc;
             }
             const size_t total = images * image_in;

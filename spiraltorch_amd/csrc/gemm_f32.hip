@@ -554,9 +554,12 @@ __device__ __forceinline__ void gemm_f32_ring_body(const GemmF32Args &p)
         __builtin_amdgcn_sched_barrier(0);
     };
 
-    const int steps = K / BK;
-    if (steps > 0) issue(std::integral_constant<int, 0>{}, 0);
-    if (steps > 1) issue(std::integral_constant<int, 1>{}, 1);
+    // k-tiles of this workgroup: all of them, or slice blockIdx.y of a k-sliced launch (first k-tile t0).
+    const int slice_steps = p.slice_k / BK;
+    const int t0 = __builtin_amdgcn_readfirstlane(static_cast<int>(blockIdx.y) * slice_steps);
+    const int steps = p.slice_k ? min(K / BK - t0, slice_steps) : K / BK;
+    if (steps > 0) issue(std::integral_constant<int, 0>{}, t0);
+    if (steps > 1) issue(std::integral_constant<int, 1>{}, t0 + 1);
     // Drain the prologue once: loads still counted as outstanding at the loop header make the compiler's
     // wait-count insertion fall back to a full vmcnt(0) inside the loop.
     ST_F32_WAIT_VMCNT(0);
@@ -572,7 +575,7 @@ __device__ __forceinline__ void gemm_f32_ring_body(const GemmF32Args &p)
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        if (t + 2 < steps) issue(std::integral_constant<int, (SLOT + 2) % RING>{}, t + 2);
+        if (t + 2 < steps) issue(std::integral_constant<int, (SLOT + 2) % RING>{}, t0 + t + 2);
         compute(slot_tag);
     };
     int t = 0;
@@ -585,6 +588,7 @@ __device__ __forceinline__ void gemm_f32_ring_body(const GemmF32Args &p)
     if (t + 1 < steps) step(std::integral_constant<int, 1>{}, t + 1);
 
     // scale 1.0f and the bias stand-in -0.0f leave every value as it is, so neither needs a branch.
+    float *const C = p.C + static_cast<size_t>(blockIdx.y) * M * N;
     with_epilogue_ops(p.activation, p.residual != nullptr, [&](auto &&act, auto has_residual) {
 #pragma unroll
         for (int tn = 0; tn < TN; ++tn) {
@@ -601,7 +605,7 @@ __device__ __forceinline__ void gemm_f32_ring_body(const GemmF32Args &p)
                         const size_t idx = static_cast<size_t>(row) * N + col;
                         float value = tile[r] * p.scale + bias;
                         if constexpr (decltype(has_residual)::value) value += p.residual[idx];
-                        p.C[idx] = act(value);
+                        C[idx] = act(value);
                     }
                 }
             }
@@ -748,7 +752,7 @@ __global__ __launch_bounds__(256) void gemm_f32_ring_32x32_splitk_kernel(GemmF32
     }
 }
 
-hipError_t launch_splitk32(GemmF32Args args, hipStream_t stream)
+hipError_t launch_splitk32(GemmF32Args args, hipStream_t stream, bool scratch_free)
 {
     args.tiles_n = (args.N + 31) / 32;
     args.tiles_m = (args.M + 31) / 32;
@@ -760,12 +764,12 @@ hipError_t launch_splitk32(GemmF32Args args, hipStream_t stream)
     // A long k over few tiles (64×64×100000, 256×256×16384) is cut over workgroups as well: 64 k-tiles per slice keep
     // 16 for each wavefront's ring.
     const size_t k_steps = static_cast<size_t>(args.K) / 16;
-    const size_t slices = choose_k_slices(args.M, args.N, args.K, tiles, k_steps, 64);
+    const size_t slices = scratch_free ? choose_k_slices(args.M, args.N, args.K, tiles, k_steps, 64) : 1;
     if (slices > 1) return launch_k_sliced(args, slices, k_steps, 16, stream, launch);
     return launch(args, 1);
 }
 
-hipError_t launch_ring(GemmF32Args args, bool lhs_transposed, bool rhs_packed, bool big, hipStream_t stream)
+hipError_t launch_ring(GemmF32Args args, bool lhs_transposed, bool rhs_packed, bool big, hipStream_t stream, bool scratch_free)
 {
     const int bm = big ? 128 : 64, bn = big ? 128 : 64;
     args.tiles_n = (args.N + bn - 1) / bn;
@@ -780,8 +784,15 @@ hipError_t launch_ring(GemmF32Args args, bool lhs_transposed, bool rhs_packed, b
     hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                         static_cast<int>(lds_bytes));
     if (rc != hipSuccess) return rc;
-    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(tiles)), dim3(big ? 512 : 256), lds_bytes, stream, args);
-    return hipGetLastError();
+    auto launch = [&](const GemmF32Args &a, unsigned slices) {
+        hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(tiles), slices), dim3(big ? 512 : 256), lds_bytes, stream, a);
+        return hipGetLastError();
+    };
+    // Few tiles and a long k (a weight gradient Xᵀ·dY of a small layer over many rows): cut along k over workgroups.
+    const size_t k_steps = static_cast<size_t>(args.K) / 16;
+    const size_t slices = big || !scratch_free ? 1 : choose_k_slices(args.M, args.N, args.K, tiles, k_steps, 32);
+    if (slices > 1) return launch_k_sliced(args, slices, k_steps, 16, stream, launch);
+    return launch(args, 1);
 }
 
 
@@ -807,7 +818,7 @@ __global__ __launch_bounds__(256) void transpose_f32_kernel(int rows, int cols, 
 }  // namespace
 
 hipError_t launch_gemm_f32(size_t m, size_t n, size_t k, bool lhs_transposed, const float *lhs,
-                           const float *rhs, float *out, const GemmEpilogue &epilogue, hipStream_t stream)
+                           const float *rhs, float *out, const GemmEpilogue &epilogue, hipStream_t stream, bool scratch_free)
 {
     if (m == 0 || n == 0) return hipSuccess;
     if (!lhs_transposed && gemv_f32_applies(m, n, k, lhs, rhs)) return launch_gemv_f32(m, n, k, lhs, rhs, out, epilogue, stream);
@@ -819,7 +830,7 @@ hipError_t launch_gemm_f32(size_t m, size_t n, size_t k, bool lhs_transposed, co
             const size_t rows = std::min(block, m - row);
             GemmEpilogue part = epilogue;
             if (part.residual) part.residual += row * n;
-            const hipError_t rc = launch_gemm_f32(rows, n, k, false, lhs + row * k, rhs, out + row * n, part, stream);
+            const hipError_t rc = launch_gemm_f32(rows, n, k, false, lhs + row * k, rhs, out + row * n, part, stream, scratch_free);
             if (rc != hipSuccess) return rc;
         }
         return hipSuccess;
@@ -853,13 +864,13 @@ hipError_t launch_gemm_f32(size_t m, size_t n, size_t k, bool lhs_transposed, co
         const bool big = tiles128 >= 512 && (tiles128 >= 3072 || tiles128 % 768 == 0 || tiles128 % 768 >= 384);
         // Fewer 64×64 tiles than compute units: 32×32 tiles with K split over the wavefronts of a workgroup.
         const size_t tiles64 = ((m + 63) / 64) * ((n + 63) / 64);
-        if (!lhs_transposed && tiles64 <= 256 && k >= 128) return launch_splitk32(args, stream);
-        return launch_ring(args, lhs_transposed, false, big, stream);
+        if (!lhs_transposed && tiles64 <= 256 && k >= 128) return launch_splitk32(args, stream, scratch_free);
+        return launch_ring(args, lhs_transposed, false, big, stream, scratch_free);
     }
     // Shapes the ring kernels do not take.  Few tiles and a long k (a matrix-vector product, n < 4, is the common case):
     // k-sliced, so that the whole chip streams A and B.
     const size_t tiles64 = ((m + 63) / 64) * ((n + 63) / 64), k_steps = (k + kBK - 1) / kBK;
-    const size_t slices = choose_k_slices(m, n, k, tiles64, k_steps, 32);
+    const size_t slices = scratch_free ? choose_k_slices(m, n, k, tiles64, k_steps, 32) : 1;
     if (slices > 1)
         return launch_k_sliced(args, slices, k_steps, kBK, stream, [&](const GemmF32Args &a, unsigned count) {
             return launch_tile<64, 64, 2, 2>(a, lhs_transposed, vec, stream, count);
@@ -889,7 +900,8 @@ hipError_t launch_gemm_f32_packed(size_t m, size_t n, size_t k, const float *lhs
         if (rc != hipSuccess) return rc;
         rc = launch_transpose_f32(n, k, packed_rhs, static_cast<float *>(workspace), stream);
         if (rc != hipSuccess) return rc;
-        return launch_gemm_f32(m, n, k, false, lhs, static_cast<const float *>(workspace), out, epilogue, stream);
+        return launch_gemm_f32(m, n, k, false, lhs, static_cast<const float *>(workspace), out, epilogue, stream,
+                               /*scratch_free=*/false);  // the scratch buffer holds the unpacked B
     }
     GemmF32Args args;
     args.A = lhs;
@@ -904,7 +916,7 @@ hipError_t launch_gemm_f32_packed(size_t m, size_t n, size_t k, const float *lhs
     args.activation = epilogue.activation;
     const size_t tiles128 = ((m + 127) / 128) * ((n + 127) / 128);
     const bool big = tiles128 >= 512 && (tiles128 >= 3072 || tiles128 % 768 == 0 || tiles128 % 768 >= 384);
-    return launch_ring(args, false, true, big, stream);
+    return launch_ring(args, false, true, big, stream, true);
 }
 
 }  // namespace sthip

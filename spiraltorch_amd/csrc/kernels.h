@@ -15,9 +15,11 @@ struct GemmEpilogue {
 };
 
 // C(m×n) = epilogue(A·B); A is m×k (k×m when lhs_transposed), B is k×n, all f32 row-major.
+// `scratch_free`: the stream's scratch buffer is not holding anything of the caller's, so a launch of few tiles with a
+// long k may put its k-sliced partial sums there; callers that keep an operand or a result in it pass false.
 hipError_t launch_gemm_f32(size_t m, size_t n, size_t k, bool lhs_transposed, const float *lhs,
                            const float *rhs, float *out, const GemmEpilogue &epilogue,
-                           hipStream_t stream);
+                           hipStream_t stream, bool scratch_free = true);
 
 // Matrix times a few columns (n <= 3 for f32, n <= 7 for bf16; 16-byte aligned operands, k a multiple of the 16-byte
 // vector): a stream over A, one wavefront or workgroup per row.  The tiled launchers route here when `*_applies`.

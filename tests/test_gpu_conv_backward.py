@@ -155,6 +155,9 @@ GRAD_INPUT_FAMILY_CASES = [
     ("auto", "col2im", (2, 3, 30, 29, 16, (7, 7), (2, 2), (3, 3), (1, 1))),         # stem: 7×7 at stride 2
     ("auto", "col2im", (2, 8, 17, 19, 12, (3, 3), (2, 3), (1, 2), (2, 1))),         # dilation along one axis, stride 2×3
     ("auto", "col2im", (5, 16, 12, 12, 24, (2, 2), (2, 2), (0, 0), (1, 1))),        # 2×2 at stride 2 (down-sampling)
+    # many output channels: the per-image products have few tiles and a long k, and their results live in the scratch
+    # buffer a k-sliced product would write its partial sums to
+    ("auto", "col2im", (2, 3, 32, 32, 2048, (16, 16), (16, 16), (0, 0), (1, 1))),
 ]
 
 

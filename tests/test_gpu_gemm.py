@@ -141,6 +141,8 @@ def test_long_reduction_against_float64(hip):
     (300, 3, 2049, False),     # ragged k: the last slice ends inside a k-tile
     (1030, 2, 1100, True),     # A stored transposed
     (130, 70, 5000, True),
+    (256, 192, 8192, True),    # the direct-to-LDS ring kernel, A transposed (a weight gradient Xᵀ·dY), k-sliced
+    (100, 260, 4096, True),
 ])
 def test_k_sliced_launches_against_float64(hip, m, n, k, lhs_t):
     """Few output tiles and a long k: the launch is cut along k over workgroups, the partial planes are added in slice
@@ -244,7 +246,10 @@ def test_ring_kernel_128_tiles_ragged_edges(hip, oracle):
 
 
 @pytest.mark.parametrize("m,n,k", [(2, 2, 3), (33, 65, 17), (64, 64, 64), (132, 136, 48), (1000, 260, 32),
-                                   (16384, 512, 64), (3000, 2820, 16)])
+                                   (16384, 512, 64), (3000, 2820, 16),
+                                   # a k the packed kernel does not take: B is unpacked into the stream's scratch buffer,
+                                   # which the product then must not use for k-sliced partial sums
+                                   (64, 64, 1026), (40, 36, 1100)])
 def test_prepacked_rhs(hip, oracle, m, n, k):
     """B prepacked as its (n, k) transpose (PackedB): same results as the row-major GEMM, with and without
     bias / residual / GELU; ragged k takes the unpack-to-workspace path."""
