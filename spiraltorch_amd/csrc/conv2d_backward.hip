@@ -523,15 +523,14 @@ hipError_t launch_conv2d_grad_input_f32(const ConvShape &shape, const float *gra
         if (rc != hipSuccess) return rc;
         float *cols = static_cast<float *>(workspace);
         const size_t image_in = static_cast<size_t>(shape.c_in) * shape.h * shape.w;
-        GemmEpilogue plain;
         for (size_t first = 0; first < static_cast<size_t>(shape.batch); first += group) {
             const size_t images = std::min(group, static_cast<size_t>(shape.batch) - first);
-            for (size_t i = 0; i < images; ++i) {
-                // cols_i (OH·OW × S) = G_iᵀ · W with G_i = grad_output of the image, C_out × OH·OW (k × m), W = C_out × S
-                rc = launch_gemm_f32(m, S, static_cast<size_t>(shape.c_out), true, grad_output + (first + i) * shape.c_out * m,
-                                     weight, cols + i * image_cols, plain, stream, /*scratch_free=*/false);  // cols live there
-                if (rc != hipSuccess) return rc;
-            }
+            // cols_i (OH·OW × S) = G_iᵀ · W with G_i = grad_output of image i, C_out × OH·OW (k × m), W = C_out × S: one
+            // launch for the group's images (a launch per image cost 5 µs each whatever its size).
+            rc = launch_gemm_f32_batched(images, m, S, static_cast<size_t>(shape.c_out), true,
+                                         grad_output + first * shape.c_out * m, static_cast<size_t>(shape.c_out) * m, weight, cols,
+                                         image_cols, stream);
+            if (rc != hipSuccess) return rc;
             const size_t total = images * image_in;
             hipLaunchKernelGGL(conv_col2im_gather_kernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, stream,
                                shape, static_cast<int>(images), cols, grad_input + first * image_in);

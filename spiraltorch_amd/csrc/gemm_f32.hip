@@ -39,6 +39,8 @@ struct GemmF32Args {
     // its raw sums to plane y of C (the launch passes the workspace of partial planes as C, scale 1 and no bias,
     // residual or activation); gemm_f32_slice_reduce_kernel adds the planes in order and applies the epilogue.
     int slice_k = 0;  // 0: one slice, the whole of K
+    // Batched form: product blockIdx.z reads A + z·a_batch and writes C + z·c_batch (B is shared).
+    size_t a_batch = 0, c_batch = 0;
 };
 
 constexpr int kBK = 16;
@@ -103,7 +105,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_f32_kernel(GemmF32Args p)
     // This workgroup's k range [k_lo, K): K below is the END of the range, p.K stays the row stride of A.
     const int k_lo = p.slice_k ? static_cast<int>(blockIdx.y) * p.slice_k : 0;
     const int K = p.slice_k ? min(p.K, k_lo + p.slice_k) : p.K;
-    float *const C = p.C + static_cast<size_t>(blockIdx.y) * M * N;
+    float *const C = p.C + static_cast<size_t>(blockIdx.y) * M * N + static_cast<size_t>(blockIdx.z) * p.c_batch;
+    const float *const A = p.A + static_cast<size_t>(blockIdx.z) * p.a_batch;
 
     f32x16 acc[TM][TN];
 #pragma unroll
@@ -125,10 +128,10 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_f32_kernel(GemmF32Args p)
             const int f = tid + T * r;
             if (!AT) {
                 const int row = min(m0 + (f >> 2), M - 1), c4 = (f & 3) * 4;
-                a_src[r] = p.A + static_cast<size_t>(row) * p.K + c4;
+                a_src[r] = A + static_cast<size_t>(row) * p.K + c4;
             } else {
                 const int krow = f / (BM / 4), col = min(m0 + (f % (BM / 4)) * 4, M - 4);
-                a_src[r] = p.A + static_cast<size_t>(krow) * M + col;
+                a_src[r] = A + static_cast<size_t>(krow) * M + col;
             }
         }
 #pragma unroll
@@ -159,10 +162,10 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_f32_kernel(GemmF32Args p)
             if (A_VECS % T != 0 && f >= A_VECS) continue;
             if (!AT) {
                 const int row = f >> 2, c4 = (f & 3) * 4;
-                ra[r] = load_row4<VEC>(p.A, static_cast<size_t>(m0 + row) * p.K, k0 + c4, K, m0 + row < M);
+                ra[r] = load_row4<VEC>(A, static_cast<size_t>(m0 + row) * p.K, k0 + c4, K, m0 + row < M);
             } else {
                 const int krow = f / (BM / 4), c4 = (f % (BM / 4)) * 4;
-                ra[r] = load_row4<VEC>(p.A, static_cast<size_t>(k0 + krow) * M, m0 + c4, M, k0 + krow < K);
+                ra[r] = load_row4<VEC>(A, static_cast<size_t>(k0 + krow) * M, m0 + c4, M, k0 + krow < K);
             }
         }
 #pragma unroll
@@ -352,13 +355,13 @@ hipError_t launch_k_sliced(GemmF32Args args, size_t slices, size_t k_steps, int 
 }
 
 template <int BM, int BN, int WM, int WN>
-hipError_t launch_tile(GemmF32Args args, bool lhs_transposed, bool vec, hipStream_t stream, unsigned slices = 1)
+hipError_t launch_tile(GemmF32Args args, bool lhs_transposed, bool vec, hipStream_t stream, unsigned slices = 1, unsigned batch = 1)
 {
     args.tiles_n = (args.N + BN - 1) / BN;
     args.tiles_m = (args.M + BM - 1) / BM;
     const size_t tiles = static_cast<size_t>(args.tiles_n) * static_cast<size_t>(args.tiles_m);
     if (tiles > 0x7fffffffu) return hipErrorInvalidConfiguration;
-    const dim3 grid(static_cast<unsigned>(tiles), slices);
+    const dim3 grid(static_cast<unsigned>(tiles), slices, batch);
     const dim3 block(64 * WM * WN);
     if (lhs_transposed) {
         if (vec)
@@ -433,7 +436,8 @@ __device__ __forceinline__ void gemm_f32_ring_body(const GemmF32Args &p)
     const int m0 = tile_m * BM, n0 = tile_n * BN;
 
     const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<float *>(p.A), 0, static_cast<int>(static_cast<size_t>(M) * K * 4), 0x00020000);
+        const_cast<float *>(p.A + static_cast<size_t>(blockIdx.z) * p.a_batch), 0, static_cast<int>(static_cast<size_t>(M) * K * 4),
+        0x00020000);
     const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<float *>(p.B), 0, static_cast<int>(static_cast<size_t>(K) * N * 4), 0x00020000);
     constexpr unsigned kOutside = 0x80000000u;
@@ -588,7 +592,7 @@ __device__ __forceinline__ void gemm_f32_ring_body(const GemmF32Args &p)
     if (t + 1 < steps) step(std::integral_constant<int, 1>{}, t + 1);
 
     // scale 1.0f and the bias stand-in -0.0f leave every value as it is, so neither needs a branch.
-    float *const C = p.C + static_cast<size_t>(blockIdx.y) * M * N;
+    float *const C = p.C + static_cast<size_t>(blockIdx.y) * M * N + static_cast<size_t>(blockIdx.z) * p.c_batch;
     with_epilogue_ops(p.activation, p.residual != nullptr, [&](auto &&act, auto has_residual) {
 #pragma unroll
         for (int tn = 0; tn < TN; ++tn) {
@@ -769,7 +773,8 @@ hipError_t launch_splitk32(GemmF32Args args, hipStream_t stream, bool scratch_fr
     return launch(args, 1);
 }
 
-hipError_t launch_ring(GemmF32Args args, bool lhs_transposed, bool rhs_packed, bool big, hipStream_t stream, bool scratch_free)
+hipError_t launch_ring(GemmF32Args args, bool lhs_transposed, bool rhs_packed, bool big, hipStream_t stream, bool scratch_free,
+                       unsigned batch = 1)
 {
     const int bm = big ? 128 : 64, bn = big ? 128 : 64;
     args.tiles_n = (args.N + bn - 1) / bn;
@@ -785,7 +790,7 @@ hipError_t launch_ring(GemmF32Args args, bool lhs_transposed, bool rhs_packed, b
                                         static_cast<int>(lds_bytes));
     if (rc != hipSuccess) return rc;
     auto launch = [&](const GemmF32Args &a, unsigned slices) {
-        hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(tiles), slices), dim3(big ? 512 : 256), lds_bytes, stream, a);
+        hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(tiles), slices, batch), dim3(big ? 512 : 256), lds_bytes, stream, a);
         return hipGetLastError();
     };
     // Few tiles and a long k (a weight gradient Xᵀ·dY of a small layer over many rows): cut along k over workgroups.
@@ -876,6 +881,41 @@ hipError_t launch_gemm_f32(size_t m, size_t n, size_t k, bool lhs_transposed, co
             return launch_tile<64, 64, 2, 2>(a, lhs_transposed, vec, stream, count);
         });
     return launch_tile<64, 64, 2, 2>(args, lhs_transposed, vec, stream);
+}
+
+hipError_t launch_gemm_f32_batched(size_t batch, size_t m, size_t n, size_t k, bool lhs_transposed, const float *lhs,
+                                   size_t lhs_stride, const float *rhs, float *out, size_t out_stride, hipStream_t stream)
+{
+    if (batch == 0 || m == 0 || n == 0) return hipSuccess;
+    GemmF32Args args;
+    args.A = lhs;
+    args.B = rhs;
+    args.C = out;
+    args.bias = nullptr;
+    args.residual = nullptr;
+    args.M = static_cast<int>(m);
+    args.N = static_cast<int>(n);
+    args.K = static_cast<int>(k);
+    args.scale = 1.0f;
+    args.activation = ST_HIP_ACT_NONE;
+    args.a_batch = lhs_stride;
+    args.c_batch = out_stride;
+    const size_t lhs_ld = lhs_transposed ? m : k;
+    const bool vec = (lhs_ld % 4 == 0) && (n % 4 == 0) && aligned16(lhs) && aligned16(rhs) && lhs_stride % 4 == 0;
+    const bool ring_ok = vec && k >= 16 && k % 16 == 0 && m * k * 4 < (1ull << 31) && k * n * 4 < (1ull << 31) &&
+                         (!lhs_transposed || m % 4 == 0);
+    const size_t tiles128 = ((m + 127) / 128) * ((n + 127) / 128) * batch;
+    const bool big = tiles128 >= 512 && (tiles128 >= 3072 || tiles128 % 768 == 0 || tiles128 % 768 >= 384);
+    // The grid's third dimension holds at most 65535 products.
+    for (size_t first = 0; first < batch; first += 65535) {
+        const unsigned count = static_cast<unsigned>(std::min<size_t>(65535, batch - first));
+        args.A = lhs + first * lhs_stride;
+        args.C = out + first * out_stride;
+        const hipError_t rc = ring_ok ? launch_ring(args, lhs_transposed, false, big, stream, /*scratch_free=*/false, count)
+                                      : launch_tile<64, 64, 2, 2>(args, lhs_transposed, vec, stream, 1, count);
+        if (rc != hipSuccess) return rc;
+    }
+    return hipSuccess;
 }
 
 hipError_t launch_transpose_f32(size_t rows, size_t cols, const float *in, float *out, hipStream_t stream)

@@ -30,6 +30,11 @@ bool gemv_bf16_applies(size_t m, size_t n, size_t k, const uint16_t *lhs, const 
 hipError_t launch_gemv_bf16(size_t m, size_t n, size_t k, const uint16_t *lhs, const uint16_t *rhs, bool rhs_packed,
                             float *out_f32, uint16_t *out_bf16, const GemmEpilogue &epilogue, hipStream_t stream);
 
+// `batch` plain products that share B in one launch: product i reads lhs + i·lhs_stride and writes out + i·out_stride
+// (values, not bytes).  Never touches the stream's scratch buffer.
+hipError_t launch_gemm_f32_batched(size_t batch, size_t m, size_t n, size_t k, bool lhs_transposed, const float *lhs,
+                                   size_t lhs_stride, const float *rhs, float *out, size_t out_stride, hipStream_t stream);
+
 // Same with B prepacked as n×k (column-major packing, crates/st-tensor/src/pure.rs:1285-1323).
 hipError_t launch_gemm_f32_packed(size_t m, size_t n, size_t k, const float *lhs, const float *packed_rhs,
                                   float *out, const GemmEpilogue &epilogue, hipStream_t stream);
