@@ -42,6 +42,10 @@ struct ConvArgs {
     int xcd_swizzle;
     int activation;
     unsigned tap_bytes[64];  // ring kernel: byte offset of tap ky*kw + kx relative to a pixel's top-left tap
+    // General kernel, k-sliced form (few tiles, long reduction): workgroup (tile, blockIdx.y) sums reduction terms
+    // [y·k_slice, (y+1)·k_slice) and writes them, raw, to plane y of `out` (the launch passes the partial planes as
+    // `out`, no bias and no activation); conv_slice_reduce_kernel adds the planes in order and finishes.
+    int k_slice = 0;  // 0: the whole reduction; else a multiple of the 16-wide k-tile
 };
 
 
@@ -73,9 +77,11 @@ __global__ __launch_bounds__(64 * WM * WN) void conv2d_f32_kernel(ConvArgs p)
     constexpr int A_LOADS = BM * BK / 4 / T;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char conv_lds[];
-    const int K = p.K;
+    // This workgroup's part of the reduction, [k_lo, K): K below is its END; p.K stays the row stride of the weights.
+    const int k_lo = p.k_slice ? static_cast<int>(blockIdx.y) * p.k_slice : 0;
+    const int K = p.k_slice ? min(p.K, k_lo + p.k_slice) : p.K;
     // The offset table holds one segment of the reduction (kConvTableEntries entries) at a time.
-    const int k_padded = (min(K, kConvTableEntries) + 15) & ~15;
+    const int k_padded = (min(p.K, kConvTableEntries) + 15) & ~15;
     int2 *lut = reinterpret_cast<int2 *>(conv_lds);
     float *As = reinterpret_cast<float *>(conv_lds + static_cast<size_t>(k_padded) * sizeof(int2));
     float *Bs = As + 2 * A_ELEMS;
@@ -99,7 +105,7 @@ __global__ __launch_bounds__(64 * WM * WN) void conv2d_f32_kernel(ConvArgs p)
     const ConvShape &s = p.s;
     const int H = s.h, W = s.w;
     const int khw = s.kh * s.kw;
-    int seg0 = 0;  // first reduction index of the segment the table describes
+    int seg0 = k_lo;  // first reduction index of the segment the table describes
     auto fill_table = [&]() {
         const int seg_end = min(K, seg0 + kConvTableEntries);
         for (int k = seg0 + tid; k < seg_end; k += T) {
@@ -136,7 +142,7 @@ __global__ __launch_bounds__(64 * WM * WN) void conv2d_f32_kernel(ConvArgs p)
 #pragma unroll
     for (int r = 0; r < A_LOADS; ++r) {
         const int f = tid + T * r;
-        w_src[r] = p.weight + static_cast<size_t>(min(oc0 + (f >> 2), s.c_out - 1)) * K + (f & 3) * 4;
+        w_src[r] = p.weight + static_cast<size_t>(min(oc0 + (f >> 2), s.c_out - 1)) * p.K + (f & 3) * 4;
     }
     auto load_global = [&](int k0) {
 #pragma unroll
@@ -149,7 +155,7 @@ __global__ __launch_bounds__(64 * WM * WN) void conv2d_f32_kernel(ConvArgs p)
             const int row = f >> 2, c4 = (f & 3) * 4;
             float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
             if (oc0 + row < s.c_out) {
-                const float *src = p.weight + static_cast<size_t>(oc0 + row) * K + k0 + c4;
+                const float *src = p.weight + static_cast<size_t>(oc0 + row) * p.K + k0 + c4;
                 if (VEC) {
                     if (k0 + c4 < K) v = *reinterpret_cast<const float4 *>(src);
                 } else {
@@ -243,7 +249,7 @@ __global__ __launch_bounds__(64 * WM * WN) void conv2d_f32_kernel(ConvArgs p)
         }
     }
 
-    float *out_image = p.out + static_cast<size_t>(image) * s.c_out * p.spatial;
+    float *out_image = p.out + (static_cast<size_t>(blockIdx.y) * s.batch + image) * s.c_out * p.spatial;
     with_epilogue_ops(p.activation, false, [&](auto &&act, auto) {
 #pragma unroll
         for (int tn = 0; tn < TN; ++tn) {
@@ -814,8 +820,42 @@ hipError_t launch_ring(ConvArgs args, hipStream_t stream)
     return hipGetLastError();
 }
 
+// Adds the partial planes of a k-sliced launch in slice order (so the result does not depend on scheduling), then bias
+// and activation.  One thread per output value; eight planes are requested together so the loads overlap.
+__global__ __launch_bounds__(256) void conv_slice_reduce_kernel(size_t count, int slices, int c_out, int spatial, int activation,
+                                                                const float *partial, const float *bias, float *out)
+{
+    const size_t idx = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (idx >= count) return;
+    float value = 0.0f;
+    for (int s0 = 0; s0 < slices; s0 += 8) {
+        float part[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) part[j] = (s0 + j < slices) ? partial[(s0 + j) * count + idx] : 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) value += part[j];
+    }
+    if (bias) value += bias[(idx / spatial) % c_out];
+    out[idx] = apply_activation(value, activation);
+}
+
+// How many slices the reduction of `shape` is cut into: none unless the general kernel's tiles would leave three
+// quarters of the compute units idle while each walks at least 64 k-tiles; then enough for about two workgroups per
+// compute unit, at least 32 k-tiles per slice, and at most 64 MB of partial planes.
+int conv_k_slices(const ConvShape &shape)
+{
+    const size_t K = static_cast<size_t>(shape.c_in) * shape.kh * shape.kw, k_steps = (K + 15) / 16;
+    const size_t spatial = static_cast<size_t>(shape.oh) * shape.ow;
+    const size_t tiles = static_cast<size_t>(shape.batch) * ((spatial + 63) / 64) * ((shape.c_out + (shape.c_out > 64 ? 127 : 63)) / (shape.c_out > 64 ? 128 : 64));
+    if (tiles > 64 || k_steps < 64) return 1;
+    size_t slices = std::min<size_t>(512 / tiles, k_steps / 32);
+    const size_t plane_bytes = static_cast<size_t>(shape.batch) * shape.c_out * spatial * sizeof(float);
+    while (slices > 1 && slices * plane_bytes > (64u << 20)) --slices;
+    return static_cast<int>(std::max<size_t>(slices, 1));
+}
+
 template <int BM, int BN, int BK, int WM, int WN, bool TRANSPOSED = false>
-hipError_t launch_tile(ConvArgs args, bool vec, hipStream_t stream)
+hipError_t launch_tile(ConvArgs args, bool vec, hipStream_t stream, unsigned slices = 1)
 {
     args.tiles_oc = (args.s.c_out + BM - 1) / BM;
     args.tiles_px = (args.spatial + BN - 1) / BN;
@@ -825,7 +865,7 @@ hipError_t launch_tile(ConvArgs args, bool vec, hipStream_t stream)
     const size_t k_padded = (static_cast<size_t>(std::min(args.K, kConvTableEntries)) + 15) & ~static_cast<size_t>(15);
     const size_t lds_bytes = k_padded * sizeof(int2) +
                              2 * (static_cast<size_t>(BM) * (BK + 4) + static_cast<size_t>(BK) * (BN + 8)) * sizeof(float);
-    const dim3 grid(static_cast<unsigned>(tiles));
+    const dim3 grid(static_cast<unsigned>(tiles), slices);
     const dim3 block(64 * WM * WN);
     hipError_t rc;
     auto launch = [&](auto kernel) -> hipError_t {
@@ -851,7 +891,8 @@ std::atomic<int> g_forced_family{ST_HIP_CONV_FAMILY_AUTO};
 
 // The dispatcher's decision for `shape`: one of ST_HIP_CONV_KERNEL_*, or 0 when a forced family cannot serve the
 // shape.  `strip` is filled when a strip kernel is chosen.
-int choose_conv_kernel(const ConvShape &shape, bool weight_aligned, bool out_aligned, int forced, StripArgs &strip)
+int choose_conv_kernel(const ConvShape &shape, bool weight_aligned, bool out_aligned, int forced, StripArgs &strip,
+                       bool allow_slices = true)
 {
     const int K = shape.c_in * shape.kh * shape.kw;
     const int spatial = shape.oh * shape.ow;
@@ -876,6 +917,9 @@ int choose_conv_kernel(const ConvShape &shape, bool weight_aligned, bool out_ali
     case ST_HIP_CONV_FAMILY_STRIP: return image_ok && plan_strip(shape, true, strip) ? strip_kernel() : 0;
     default: break;
     }
+    // Few tiles with a long reduction (deep layers on tiny planes at small batch, one or a few output channels): every
+    // kernel here walks the reduction serially inside a workgroup, so the chip is filled by cutting the reduction.
+    if (allow_slices && conv_k_slices(shape) > 1) return ST_HIP_CONV_KERNEL_TILE_KSLICED;
     if (!ring_ok) return ST_HIP_CONV_KERNEL_TILE;
     // The ring kernel has the better steady state (several rounds of 128×64 tiles per compute unit); the strip
     // kernel, balanced to the single SIMD, wins when the ring kernel's tiles would fill the chip fewer than
@@ -896,8 +940,17 @@ int planned_conv_kernel(const ConvShape &shape, bool weight_aligned, bool out_al
     return choose_conv_kernel(shape, weight_aligned, out_aligned, g_forced_family.load(std::memory_order_relaxed), strip);
 }
 
+size_t conv2d_scratch_bytes(const ConvShape &shape, bool weight_aligned, bool out_aligned)
+{
+    StripArgs strip;
+    if (choose_conv_kernel(shape, weight_aligned, out_aligned, g_forced_family.load(std::memory_order_relaxed), strip) !=
+        ST_HIP_CONV_KERNEL_TILE_KSLICED)
+        return 0;
+    return static_cast<size_t>(conv_k_slices(shape)) * shape.batch * shape.c_out * shape.oh * shape.ow * sizeof(float);
+}
+
 hipError_t launch_conv2d_f32(const ConvShape &shape, int activation, const float *input, const float *weight,
-                             const float *bias, float *out, hipStream_t stream)
+                             const float *bias, float *out, hipStream_t stream, int scratch, size_t scratch_offset)
 {
     if (shape.batch == 0 || shape.c_out == 0 || shape.oh == 0 || shape.ow == 0) return hipSuccess;
     ConvArgs args;
@@ -919,8 +972,29 @@ hipError_t launch_conv2d_f32(const ConvShape &shape, int activation, const float
     const bool out_aligned = (reinterpret_cast<uintptr_t>(out) & 15u) == 0;
     StripArgs strip;
     const int kernel = choose_conv_kernel(shape, weight_aligned, out_aligned,
-                                          g_forced_family.load(std::memory_order_relaxed), strip);
+                                          g_forced_family.load(std::memory_order_relaxed), strip, scratch == kConvScratchStream);
     switch (kernel) {
+    case ST_HIP_CONV_KERNEL_TILE_KSLICED: {
+        const size_t slices = static_cast<size_t>(conv_k_slices(shape));
+        const size_t k_steps = (static_cast<size_t>(args.K) + 15) / 16, steps_per_slice = (k_steps + slices - 1) / slices;
+        const size_t used = (k_steps + steps_per_slice - 1) / steps_per_slice;
+        const size_t count = static_cast<size_t>(shape.batch) * shape.c_out * args.spatial;
+        void *workspace = nullptr;
+        hipError_t rc = stream_workspace(stream, scratch_offset + slices * count * sizeof(float), &workspace);
+        if (rc != hipSuccess) return rc;
+        float *partial = reinterpret_cast<float *>(static_cast<unsigned char *>(workspace) + scratch_offset);
+        args.out = partial;
+        args.bias = nullptr;
+        args.activation = ST_HIP_ACT_NONE;
+        args.k_slice = static_cast<int>(steps_per_slice * 16);
+        const bool vec = (args.K % 4 == 0) && weight_aligned;
+        rc = shape.c_out > 64 ? launch_tile<128, 64, 16, 4, 2>(args, vec, stream, static_cast<unsigned>(used))
+                              : launch_tile<64, 64, 16, 2, 2>(args, vec, stream, static_cast<unsigned>(used));
+        if (rc != hipSuccess) return rc;
+        hipLaunchKernelGGL(conv_slice_reduce_kernel, dim3(static_cast<unsigned>((count + 255) / 256)), dim3(256), 0, stream, count,
+                           static_cast<int>(used), shape.c_out, args.spatial, activation, partial, bias, out);
+        return hipGetLastError();
+    }
     case ST_HIP_CONV_KERNEL_STRIP12:
     case ST_HIP_CONV_KERNEL_STRIP12_WIDE:
     case ST_HIP_CONV_KERNEL_STRIP9:

@@ -540,9 +540,13 @@ hipError_t launch_conv2d_grad_input_f32(const ConvShape &shape, const float *gra
         return hipSuccess;
     }
     float *adjoint_weight = weight_scratch;  // room for weight_count values, owned by the caller
+    // The re-laid weights sit at the front of the stream's scratch buffer; a forward launch that cuts its reduction
+    // into slices keeps its partial sums behind them (sized here, so the buffer does not move in between).
+    const size_t weight_bytes = (weight_count * sizeof(float) + 255) & ~static_cast<size_t>(255);
     if (adjoint_weight == nullptr) {
         void *workspace = nullptr;
-        rc = stream_workspace(stream, weight_count * sizeof(float), &workspace);
+        const size_t behind = as_forward ? conv2d_scratch_bytes(t, true, (reinterpret_cast<uintptr_t>(grad_input) & 15u) == 0) : 0;
+        rc = stream_workspace(stream, weight_bytes + behind, &workspace);
         if (rc != hipSuccess) return rc;
         adjoint_weight = static_cast<float *>(workspace);
     }
@@ -551,7 +555,8 @@ hipError_t launch_conv2d_grad_input_f32(const ConvShape &shape, const float *gra
     rc = hipGetLastError();
     if (rc != hipSuccess) return rc;
     if (as_forward)
-        return launch_conv2d_f32(t, ST_HIP_ACT_NONE, grad_output, adjoint_weight, nullptr, grad_input, stream);
+        return launch_conv2d_f32(t, ST_HIP_ACT_NONE, grad_output, adjoint_weight, nullptr, grad_input, stream,
+                                 weight_scratch ? kConvScratchNone : kConvScratchStream, weight_bytes);
     return launch_conv2d_adjoint_f32(t, grad_output, adjoint_weight, grad_input, stream);
 }
 

@@ -60,8 +60,16 @@ struct ConvShape {
 // Entries of the general implicit-GEMM kernel's LDS offset table: longer reductions (c_in*kh*kw) go through it in
 // segments of this many terms.
 constexpr int kConvTableEntries = 8192;
+// `scratch`: where a launch of few tiles with a long reduction may keep its k-sliced partial sums —
+// kConvScratchStream: in the stream's scratch buffer from byte `scratch_offset` on (the caller holds what lies before
+// it and has sized the buffer with conv2d_scratch_bytes, so that it does not move); kConvScratchNone: nowhere, such
+// launches run unsliced.
+constexpr int kConvScratchStream = 0, kConvScratchNone = 1;
 hipError_t launch_conv2d_f32(const ConvShape &shape, int activation, const float *input,
-                             const float *weight, const float *bias, float *out, hipStream_t stream);
+                             const float *weight, const float *bias, float *out, hipStream_t stream,
+                             int scratch = kConvScratchStream, size_t scratch_offset = 0);
+// Bytes of the stream's scratch buffer launch_conv2d_f32 uses for `shape` (0 for most shapes).
+size_t conv2d_scratch_bytes(const ConvShape &shape, bool weight_aligned, bool out_aligned);
 
 // Which kernel launch_conv2d_f32 would run for `shape` (one of ST_HIP_CONV_KERNEL_*; 0 when the family forced with
 // set_conv_forced_family cannot serve it), and the same for launch_conv2d_grad_input_f32 on the forward `shape`.

@@ -68,17 +68,28 @@ def test_random_shapes(hip, oracle, shape):
     assert_close(got, oracle.conv2d_bias_act_f32(*shape, oracle.ACT_RELU, x, wt, None), F32_REL, F32_ABS, "no bias")
 
 
+@pytest.fixture
+def force_family(hip):
+    """Forces a conv kernel family for one test and gives the choice back to the dispatcher afterwards."""
+    yield hip.conv2d_force_family
+    hip.conv2d_force_family("auto")
+
+
+@pytest.mark.parametrize("family", ["tile", "auto"])
 @pytest.mark.parametrize("shape", [
     (1, 192, 12, 12, 40, (7, 7), (1, 1), (3, 3), (1, 1)),    # 9408 terms: two table segments (ConvNeXt-style 7×7)
     (2, 170, 9, 9, 70, (7, 7), (2, 2), (3, 3), (1, 1)),      # 8330 terms, k % 16 != 0, strided
     (1, 384, 8, 8, 33, (7, 7), (1, 1), (3, 3), (1, 1)),      # 18816 terms: three segments
     (1, 1030, 6, 6, 20, (3, 3), (1, 1), (1, 1), (1, 1)),     # 9270 terms, k % 4 != 0: scalar weight staging
 ])
-def test_reductions_longer_than_the_offset_table(hip, oracle, shape):
+def test_reductions_longer_than_the_offset_table(hip, oracle, force_family, shape, family):
     """c_in·kh·kw beyond the 8192 entries of the general kernel's LDS offset table: the table is rebuilt segment by
-    segment while the accumulators run on.  He-scaled weights; compared against the oracle with the bound a
-    reordered f32 sum of that length supports (a small multiple of unit roundoff times sum |x||w|)."""
+    segment while the accumulators run on (the general kernel forced), or — the dispatcher's own choice for these few
+    tiles — the reduction is cut into slices over workgroups.  He-scaled weights; compared against the oracle with the
+    bound a reordered f32 sum of that length supports (a small multiple of unit roundoff times sum |x||w|)."""
     batch, c_in, h, w, c_out, kernel, stride, padding, dilation = shape
+    force_family(family)
+    assert hip.conv2d_planned_kernel(*shape) == ("tile" if family == "tile" else "tile_ksliced")
     rng = np.random.default_rng(c_in * 31 + c_out)
     x = rng.normal(size=batch * c_in * h * w).astype(np.float32)
     wt = rng.normal(0, np.sqrt(2.0 / (c_in * kernel[0] * kernel[1])), c_out * c_in * kernel[0] * kernel[1]).astype(np.float32)
@@ -88,6 +99,33 @@ def test_reductions_longer_than_the_offset_table(hip, oracle, shape):
     magnitude = oracle.conv2d_bias_act_f32(*shape, oracle.ACT_NONE, np.abs(x), np.abs(wt), None)
     assert_close(got, want, F32_REL, F32_ABS + 2 * 2.0 ** -24 * float(magnitude.max()), f"conv {shape}")
     assert float(np.abs(got).max()) > 0.1  # the comparison is not about zeros
+
+
+@pytest.mark.parametrize("shape", [
+    (1, 512, 7, 7, 512, (3, 3), (1, 1), (1, 1), (1, 1)),      # deep layer on a tiny plane at batch 1: 4608 terms, 4 tiles
+    (2, 351, 7, 10, 47, (4, 4), (1, 1), (3, 1), (1, 1)),
+    (1, 130, 9, 9, 40, (3, 3), (1, 1), (1, 1), (1, 1)),       # 1170 terms: the last slice ends inside a k-tile
+    (3, 157, 19, 15, 1, (7, 7), (1, 1), (0, 0), (1, 1)),      # one output channel
+    (1, 2048, 7, 7, 512, (1, 1), (1, 1), (0, 0), (1, 1)),
+    (2, 366, 5, 44, 24, (4, 4), (2, 2), (3, 0), (2, 2)),      # strided and dilated
+])
+def test_few_tiles_with_a_long_reduction_are_cut_into_slices(hip, oracle, shape):
+    """Every kernel walks c_in·kh·kw serially inside a workgroup; when the tiles alone would leave most of the chip idle
+    the reduction is cut over workgroups, the partial planes are added in slice order and bias and activation follow."""
+    batch, c_in, h, w, c_out, kernel, stride, padding, dilation = shape
+    assert hip.conv2d_planned_kernel(*shape) == "tile_ksliced"
+    rng = np.random.default_rng(c_in * 7 + c_out)
+    x = rng.normal(size=batch * c_in * h * w).astype(np.float32)
+    wt = rng.normal(0, np.sqrt(2.0 / (c_in * kernel[0] * kernel[1])), c_out * c_in * kernel[0] * kernel[1]).astype(np.float32)
+    b = rng.uniform(-0.5, 0.5, c_out).astype(np.float32)
+    magnitude = oracle.conv2d_bias_act_f32(*shape, oracle.ACT_NONE, np.abs(x), np.abs(wt), None)
+    slack = F32_ABS + 2 * 2.0 ** -24 * float(magnitude.max())
+    for act, code in ((0, oracle.ACT_NONE), (1, oracle.ACT_RELU), (2, oracle.ACT_GELU)):
+        got = run(hip, *shape, act, x, wt, b)
+        assert_close(got, oracle.conv2d_bias_act_f32(*shape, code, x, wt, b), F32_REL, slack, f"conv {shape} act={act}")
+        assert (run(hip, *shape, act, x, wt, b) == got).all(), "slices are added in a fixed order"
+    got = run(hip, *shape, 0, x, wt, None)
+    assert_close(got, oracle.conv2d_bias_act_f32(*shape, oracle.ACT_NONE, x, wt, None), F32_REL, slack, "no bias")
 
 
 G33 = ((3, 3), (1, 1), (1, 1), (1, 1))
@@ -129,13 +167,6 @@ FAMILY_CASES = [
     ("blocks56", "tile", "tile"), ("c112", "tile", "tile"), ("stride2_c32", "tile", "tile"),
     ("dilated_c48", "tile", "tile"), ("ring_5x5", "tile", "tile"),
 ]
-
-
-@pytest.fixture
-def force_family(hip):
-    """Forces a conv kernel family for one test and gives the choice back to the dispatcher afterwards."""
-    yield hip.conv2d_force_family
-    hip.conv2d_force_family("auto")
 
 
 @pytest.mark.parametrize("name,family,kernel", FAMILY_CASES)
@@ -182,6 +213,8 @@ def test_dispatcher_choices(hip):
     assert hip.conv2d_planned_kernel(32, 64, 56, 56, 128, *G33, direction="grad_input") == "strip9"
     assert hip.conv2d_planned_kernel(64, 64, 56, 56, 256, *G33) == "ring"
     assert hip.conv2d_planned_kernel(8, 3, 32, 32, 16, *G33) == "tile"
+    assert hip.conv2d_planned_kernel(1, 512, 7, 7, 512, *G33) == "tile_ksliced"
+    assert hip.conv2d_planned_kernel(32, 512, 7, 7, 512, *G33) == "ring"
     assert hip.conv2d_planned_kernel(2, 8, 9, 9, 4, (3, 3), (2, 2), (1, 1), (1, 1), direction="grad_input") == "col2im"
     assert hip.conv2d_planned_kernel(2, 64, 9, 9, 4, (3, 3), (2, 1), (1, 1), (1, 1), direction="grad_input") == "adjoint"
     assert hip.conv2d_planned_kernel(32, 3, 224, 224, 768, (16, 16), (16, 16), (0, 0), (1, 1), direction="grad_input") == "col2im"

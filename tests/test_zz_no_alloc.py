@@ -1,8 +1,11 @@
 """The allocation-free grad_input entry point (weights re-laid into a static device array) against the entry point
-it is a variant of: bit-identical results, on two calls in a row, the second with a smaller input; oversized weights
-are refused before anything is launched."""
+it is a variant of: bit-identical results wherever both run the same kernels (within the f32 parity bar where the
+allocating entry point cuts a long reduction into slices kept in scratch memory, which this one must not touch), on
+calls in a row, each second one with a smaller input; oversized weights are refused before anything is launched."""
 import numpy as np
 import pytest
+
+from conftest import F32_ABS, F32_REL, assert_close
 
 pytestmark = pytest.mark.gpu
 
@@ -34,7 +37,10 @@ def test_matches_the_allocating_entry_point_call_after_call(hip):
             stream.synchronize()
             want, got = d_want.to_array(np.float32, n), d_got.to_array(np.float32, n)
             assert np.isfinite(want).all() and np.abs(want).max() > 0
-            assert (got == want).all(), f"{case} (pass {repeat})"
+            if hip.conv2d_planned_kernel(*case, direction="grad_input") == "tile_ksliced":
+                assert_close(got, want, F32_REL, F32_ABS, f"{case} (pass {repeat})")
+            else:
+                assert (got == want).all(), f"{case} (pass {repeat})"
     stream.destroy()
 
 
@@ -54,4 +60,6 @@ def test_weights_beyond_the_static_array_are_refused(hip):
     hip.conv2d_grad_input_f32_dev(*case, d_g, d_w, d_want)
     hip.conv2d_grad_input_f32_noalloc_dev(*case, d_g, d_w, d_got)
     hip.device_synchronize()
-    assert (d_got.to_array(np.float32, 2048 * 4) == d_want.to_array(np.float32, 2048 * 4)).all()
+    # (the allocating entry point cuts this 2048-term reduction over 16 tiles into slices; this one may not)
+    assert hip.conv2d_planned_kernel(*case, direction="grad_input") == "tile_ksliced"
+    assert_close(d_got.to_array(np.float32, 2048 * 4), d_want.to_array(np.float32, 2048 * 4), F32_REL, F32_ABS, "16 MiB of weights")
