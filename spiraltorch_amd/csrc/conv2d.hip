@@ -839,16 +839,17 @@ __global__ __launch_bounds__(256) void conv_slice_reduce_kernel(size_t count, in
     out[idx] = apply_activation(value, activation);
 }
 
-// How many slices the reduction of `shape` is cut into: none unless the general kernel's tiles would leave three
-// quarters of the compute units idle while each walks at least 64 k-tiles; then enough for about two workgroups per
-// compute unit, at least 32 k-tiles per slice, and at most 64 MB of partial planes.
+// How many slices the reduction of `shape` is cut into: none unless the general kernel's tiles would leave half of the
+// compute units idle while each walks at least 48 k-tiles (a k-tile costs a workgroup 0.5 to 1 µs of load latency
+// whatever the tile count, so 48 of them are 25 to 50 µs); then enough for about four workgroups per compute unit,
+// at least 8 k-tiles per slice, and at most 64 MB of partial planes.
 int conv_k_slices(const ConvShape &shape)
 {
     const size_t K = static_cast<size_t>(shape.c_in) * shape.kh * shape.kw, k_steps = (K + 15) / 16;
     const size_t spatial = static_cast<size_t>(shape.oh) * shape.ow;
     const size_t tiles = static_cast<size_t>(shape.batch) * ((spatial + 63) / 64) * ((shape.c_out + (shape.c_out > 64 ? 127 : 63)) / (shape.c_out > 64 ? 128 : 64));
-    if (tiles > 64 || k_steps < 64) return 1;
-    size_t slices = std::min<size_t>(512 / tiles, k_steps / 32);
+    if (tiles > 128 || k_steps < 48) return 1;
+    size_t slices = std::min<size_t>(1024 / tiles, k_steps / 8);
     const size_t plane_bytes = static_cast<size_t>(shape.batch) * shape.c_out * spatial * sizeof(float);
     while (slices > 1 && slices * plane_bytes > (64u << 20)) --slices;
     return static_cast<int>(std::max<size_t>(slices, 1));

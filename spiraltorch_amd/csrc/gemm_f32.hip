@@ -795,7 +795,7 @@ hipError_t launch_ring(GemmF32Args args, bool lhs_transposed, bool rhs_packed, b
     };
     // Few tiles and a long k (a weight gradient Xᵀ·dY of a small layer over many rows): cut along k over workgroups.
     const size_t k_steps = static_cast<size_t>(args.K) / 16;
-    const size_t slices = big || !scratch_free ? 1 : choose_k_slices(args.M, args.N, args.K, tiles, k_steps, 32);
+    const size_t slices = big || !scratch_free ? 1 : choose_k_slices(args.M, args.N, args.K, tiles, k_steps, 16);
     if (slices > 1) return launch_k_sliced(args, slices, k_steps, 16, stream, launch);
     return launch(args, 1);
 }
@@ -875,7 +875,7 @@ hipError_t launch_gemm_f32(size_t m, size_t n, size_t k, bool lhs_transposed, co
     // Shapes the ring kernels do not take.  Few tiles and a long k (a matrix-vector product, n < 4, is the common case):
     // k-sliced, so that the whole chip streams A and B.
     const size_t tiles64 = ((m + 63) / 64) * ((n + 63) / 64), k_steps = (k + kBK - 1) / kBK;
-    const size_t slices = scratch_free ? choose_k_slices(m, n, k, tiles64, k_steps, 32) : 1;
+    const size_t slices = scratch_free ? choose_k_slices(m, n, k, tiles64, k_steps, 16) : 1;
     if (slices > 1)
         return launch_k_sliced(args, slices, k_steps, kBK, stream, [&](const GemmF32Args &a, unsigned count) {
             return launch_tile<64, 64, 2, 2>(a, lhs_transposed, vec, stream, count);

@@ -214,7 +214,7 @@ def test_dispatcher_choices(hip):
     assert hip.conv2d_planned_kernel(64, 64, 56, 56, 256, *G33) == "ring"
     assert hip.conv2d_planned_kernel(8, 3, 32, 32, 16, *G33) == "tile"
     assert hip.conv2d_planned_kernel(1, 512, 7, 7, 512, *G33) == "tile_ksliced"
-    assert hip.conv2d_planned_kernel(32, 512, 7, 7, 512, *G33) == "ring"
+    assert hip.conv2d_planned_kernel(64, 512, 7, 7, 512, *G33) == "ring"
     assert hip.conv2d_planned_kernel(2, 8, 9, 9, 4, (3, 3), (2, 2), (1, 1), (1, 1), direction="grad_input") == "col2im"
     assert hip.conv2d_planned_kernel(2, 64, 9, 9, 4, (3, 3), (2, 1), (1, 1), (1, 1), direction="grad_input") == "adjoint"
     assert hip.conv2d_planned_kernel(32, 3, 224, 224, 768, (16, 16), (16, 16), (0, 0), (1, 1), direction="grad_input") == "col2im"
