@@ -167,7 +167,8 @@ PACKED_SHAPES = [
     # n not a multiple of 128 (rows of the packed B past n read as zero, stores at any alignment): 128- and 256-wide
     # tiles, an odd n, k split over workgroups, one long row of tiles
     (300, 1000, 192), (1024, 257, 64), (513, 2051, 128), (4096, 129, 4096), (200, 50257, 64), (130, 3000, 1024),
-    # shapes they do not take: unpacked on the device first (general kernel, skinny split-k kernel)
+    # shapes they do not take are unpacked on the device first (general kernel); up to 64 rows the row-major entry point
+    # runs the skinny split-k kernel, the prepacked one the 256-row kernels
     (33, 40, 72), (130, 136, 264), (5, 7, 9), (16, 384, 320), (64, 128, 1024), (1, 8, 8),
 ]
 
@@ -195,8 +196,13 @@ def test_prepacked_rhs(hip, oracle, m, n, k):
     hip.gemm_bf16_bias_act_dev(m, n, k, 2, d["a"], d["b"], d["bias"], d["res"], want32, want16)
     hip.gemm_bf16_prepacked_bias_act_dev(m, n, k, 2, d["a"], d_packed, d["bias"], d["res"], got32, got16)
     hip.device_synchronize()
-    assert (got32.to_array(np.float32, m * n) == want32.to_array(np.float32, m * n)).all()
-    assert (got16.to_array(np.uint16, m * n) == want16.to_array(np.uint16, m * n)).all()
+    if m <= 64 and n % 128 == 0 and k % 64 == 0 and k >= 256:
+        # up to 64 rows a row-major B goes to the skinny kernel while a prepacked B stays on the 256-row kernels
+        # (unpacking it would cost a pass over B per call): same sums in another order
+        assert_close(got32.to_array(np.float32, m * n), want32.to_array(np.float32, m * n), 1e-4, 1e-5, "layouts agree")
+    else:
+        assert (got32.to_array(np.float32, m * n) == want32.to_array(np.float32, m * n)).all()
+        assert (got16.to_array(np.uint16, m * n) == want16.to_array(np.uint16, m * n)).all()
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 1024, 128), (16, 4096, 4096), (17, 1024, 384), (32, 2048, 1152), (5, 1040, 2176),
