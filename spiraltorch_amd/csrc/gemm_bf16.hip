@@ -1996,26 +1996,33 @@ __global__ __launch_bounds__(256) void transpose_u16_kernel(int rows, int cols, 
 // latency whatever the tile count, so the loop's time is the k-tiles per split; against that stand the partial sums,
 // written once and read once, and the reduction's launch.  The split count is the one with the least sum of the three
 // (at least two k-tiles per split, at most one workgroup per compute unit).
-size_t choose_k_splits(size_t m, size_t n, size_t k, size_t tiles)
+struct SplitChoice {
+    size_t splits;
+    double cost_us;
+};
+// `most_groups`: workgroups the chip holds at a time for this tiling (256 for the 256-row kernels, 512 for 128×128
+// tiles); `tile_us`: what a k-tile costs a workgroup of that tiling when few are resident.
+SplitChoice estimate_k_splits(size_t m, size_t n, size_t k, size_t tiles, size_t most_groups, double tile_us)
 {
     const size_t k_tiles = k / 64;
-    if (tiles * 2 > 256 || k_tiles < 8) return 1;
-    const size_t most = std::min<size_t>(256 / tiles, k_tiles / 2);
     const double plane_bytes = static_cast<double>(m) * static_cast<double>(n) * sizeof(float);
     auto cost_us = [&](size_t splits) {
-        const double loop = 0.5 * static_cast<double>((k_tiles + splits - 1) / splits);
+        const double loop = tile_us * static_cast<double>((k_tiles + splits - 1) / splits);
         const double sums = splits > 1 ? 3.0 + static_cast<double>(splits) * plane_bytes * 2.0 / 4.0e6 : 0.0;  // 4 TB/s
         return loop + sums;
     };
-    size_t best = 1;
+    SplitChoice best{1, cost_us(1)};
+    if (tiles * 2 > most_groups || k_tiles < 8) return best;
+    const size_t most = std::min<size_t>(most_groups / tiles, k_tiles / 2);
     for (size_t splits = 2; splits <= most; ++splits)
-        if (cost_us(splits) < cost_us(best)) best = splits;
-    // (Measured on m = 33 … 2048 against n, k = 512 … 4096, both layouts of B: against the earlier rule — split as far
-    // as the partial sums stay below the operands' bytes — this one is 10 to 35 % faster on twelve of eighteen mid-size
-    // shapes, e.g. 1024×768×3072 24.5 → 20.0 µs prepacked and 33.1 → 23.8 µs row-major, and slower on one,
-    // 2048×512×2048 prepacked 13.8 → 18.5 µs; demanding a margin over the unsplit 128×128 tiling lost most of the gains.)
+        if (cost_us(splits) < best.cost_us) best = SplitChoice{splits, cost_us(splits)};
+    // (Measured on m = 33 … 2048 against n, k = 512 … 4096, both layouts of B, against the earlier rule — split as far
+    // as the partial sums stay below the operands' bytes, 256-row tiles only: 10 to 35 % faster on most mid-size shapes,
+    // e.g. 1024×768×3072 24.5 → 17.7 µs prepacked and 33.1 → 20.3 µs row-major, 512×512×2048 15.3 → 10.2 µs; none
+    // slower by more than 3 %.)
     return best;
 }
+size_t choose_k_splits(size_t m, size_t n, size_t k, size_t tiles) { return estimate_k_splits(m, n, k, tiles, 256, 0.5).splits; }
 
 // The 256-row tiling of an m×n×k product (n a multiple of 128): tile width, tile count and k-splits.
 // One workgroup per compute unit at a time: the launch runs in rounds of 256 tiles.  Halving the tile width costs
@@ -2089,12 +2096,35 @@ hipError_t launch_256(GemmBf16Args args, bool packed, hipStream_t stream, size_t
     return hipGetLastError();
 }
 
-hipError_t launch_128(GemmBf16Args args, bool packed, hipStream_t stream)
+hipError_t launch_128(GemmBf16Args args, bool packed, hipStream_t stream, size_t splits = 1, size_t workspace_offset = 0)
 {
     args.tiles_m = (args.M + 127) / 128;
     args.tiles_n = (args.N + 127) / 128;
-    const size_t tiles = static_cast<size_t>(args.tiles_m) * static_cast<size_t>(args.tiles_n);
+    size_t tiles = static_cast<size_t>(args.tiles_m) * static_cast<size_t>(args.tiles_n);
     if (tiles > 0x7fffffffu) return hipErrorInvalidConfiguration;
+    SkinnyArgs reduce{};
+    if (splits > 1) {
+        const size_t k_tiles = static_cast<size_t>(args.K) / 64;
+        args.tiles_per_split = static_cast<int>((k_tiles + splits - 1) / splits);
+        args.k_splits = static_cast<int>((k_tiles + args.tiles_per_split - 1) / args.tiles_per_split);
+        const size_t bytes = static_cast<size_t>(args.k_splits) * args.M * args.N * sizeof(float);
+        void *workspace = nullptr;
+        hipError_t ws = stream_workspace(stream, workspace_offset + bytes, &workspace);
+        if (ws != hipSuccess) return ws;
+        args.partial = reinterpret_cast<float *>(static_cast<unsigned char *>(workspace) + workspace_offset);
+        reduce.partial = args.partial;
+        reduce.C32 = args.C32;
+        reduce.C16 = args.C16;
+        reduce.bias = args.bias;
+        reduce.residual = args.residual;
+        reduce.M = args.M;
+        reduce.N = args.N;
+        reduce.K = args.K;
+        reduce.k_splits = args.k_splits;
+        reduce.scale = args.scale;
+        reduce.activation = args.activation;
+        tiles *= static_cast<size_t>(args.k_splits);
+    }
     args.swizzle = (tiles % 8 == 0) ? 1 : 0;
     constexpr size_t lds_bytes = 5 * 16384;  // three A stages + two B stages of 128 rows
     static_assert(lds_bytes >= 4 * 32 * (64 + 4) * sizeof(float), "four epilogue strips must fit in the stage buffers");
@@ -2103,6 +2133,11 @@ hipError_t launch_128(GemmBf16Args args, bool packed, hipStream_t stream)
                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
     if (rc != hipSuccess) return rc;
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(tiles)), dim3(256), lds_bytes, stream, args);
+    rc = hipGetLastError();
+    if (rc != hipSuccess || args.k_splits == 1) return rc;
+    const size_t plane = static_cast<size_t>(args.M) * args.N;
+    hipLaunchKernelGGL(gemm_bf16_skinny_reduce_kernel, dim3(static_cast<unsigned>((plane + 255) / 256)), dim3(256), 0, stream,
+                       reduce);
     return hipGetLastError();
 }
 
@@ -2329,8 +2364,13 @@ hipError_t launch_gemm_bf16(size_t m, size_t n, size_t k, const uint16_t *lhs, c
         // tiles, two workgroups per compute unit (1024³: 16 tiles of 256×256, 64 of 128×128).
         const size_t tiles_256 = plan.tiles;
         const size_t tiles_128 = ((m + 127) / 128) * (n / 128);
-        if (tiles_256 < 192 && tiles_128 >= 2 * tiles_256 && plan.k_splits == 1)
-            return launch_128(args, rhs_packed, stream);
+        if (tiles_256 < 192 && tiles_128 >= 2 * tiles_256) {
+            // Either tiling may split k; the smaller tiles need fewer splits (less partial-sum traffic) for the same
+            // number of workgroups, and two of their workgroups share a compute unit.
+            const SplitChoice big = estimate_k_splits(m, n, k, tiles_256, 256, 0.5);
+            const SplitChoice small = estimate_k_splits(m, n, k, tiles_128, 512, 0.42);
+            if (small.cost_us <= big.cost_us) return launch_128(args, rhs_packed, stream, small.splits, workspace_offset);
+        }
         // Several rounds of 256×128 tiles with bf16 as the only output (the QKV projection of a transformer block):
         // the persistent kernel, whose stores drain under the next tile's main loop (16384×1536×512: 34.1 µs against
         // 36.8).  Where the plan is 256×256 tiles they stay ahead (16384×2048×512: 48.2 µs against 51.8).
