@@ -307,6 +307,34 @@ def wl_rowops(hip, inputs, timer, warmup, steps):
     return out
 
 
+def wl_lopsided(hip, inputs, timer, warmup, steps):
+    """Shapes outside the BASELINE configs whose dispatch has kernels of its own: matrix x vector (a stream over A: the
+    f32 matrix is 1 GiB, the bf16 one 512 MiB, both beyond the 256 MiB memory-side cache), a product of few output tiles
+    with a long k (k-sliced over workgroups), and softmax over rows of 100000 values (a workgroup per row).  All
+    HBM-bound; bytes are the algorithmic reads + writes."""
+    out = []
+    m = k = 16384
+    d_a = hip.DeviceBuffer(m * k * 4)
+    d_a.zero()
+    d_x = hip.DeviceBuffer.from_array(inputs.uniform(inputs.seed_for(1, 2), k, -1.0, 1.0))
+    d_y = hip.DeviceBuffer(m * 4)
+    wall, ev = timer.run(lambda st: hip.gemm_f32_dev(m, 1, k, 1.0, False, d_a, d_x, d_y, st), warmup, steps)
+    out.append(entry(f"gemv_f32_{m}x1x{k}", "f32", 2 * m * k, 4 * (m * k + k + m), "hbm", wall, ev))
+    d_x16 = hip.DeviceBuffer.from_array(inputs.to_bf16(inputs.uniform(inputs.seed_for(1, 2), k, -1.0, 1.0)))
+    wall, ev = timer.run(lambda st: hip.gemm_bf16_f32acc_dev(m, 1, k, d_a, d_x16, d_y, st), warmup, steps)
+    out.append(entry(f"gemv_bf16_{m}x1x{k}", "bf16", 2 * m * k, 2 * (m * k + k) + 4 * m, "hbm", wall, ev))
+    m2, n2, k2 = 64, 64, 100000
+    d_c = hip.DeviceBuffer(m2 * n2 * 4)
+    wall, ev = timer.run(lambda st: hip.gemm_f32_dev(m2, n2, k2, 1.0, False, d_a, d_a, d_c, st), warmup, steps)
+    out.append(entry(f"gemm_f32_{m2}x{n2}x{k2}_k_sliced", "f32", 2 * m2 * n2 * k2, 4 * (m2 * k2 + k2 * n2 + m2 * n2), "hbm", wall, ev))
+    rows, cols = 100, 100000
+    d_in = hip.DeviceBuffer.from_array(inputs.normal(inputs.seed_for(5, 5), rows * cols))
+    d_out = hip.DeviceBuffer(rows * cols * 4)
+    wall, ev = timer.run(lambda st: hip.row_softmax_f32_dev(rows, cols, d_in, d_out, st), warmup, steps)
+    out.append(entry(f"row_softmax_f32_{rows}x{cols}", "f32", 0, 8 * rows * cols, "hbm", wall, ev))
+    return out
+
+
 def wl_calibration(hip, inputs, timer, warmup, steps):
     """Plain streaming kernel of known traffic (f32 -> bf16 rounding of 64 Mi values: 256 MiB read, 128 MiB
     written).  It anchors the FETCH_SIZE / WRITE_SIZE counters and shows the HBM rate a trivial kernel reaches."""
@@ -381,6 +409,11 @@ def cpu_baselines(inputs):
     sec = timed(lambda: oracle.gemm_bf16_f32acc(16, 4096, 4096, a16[:16 * 4096], b16, threads=cores), repeat=5)
     out["gemm_bf16_f32acc_16x4096x4096"] = _cpu(2 * 16 * 4096 * 4096, sec, cores, f"full shape, best of 5, {cores} threads")
     out["gemm_bf16_f32acc_16x4096x4096_prepacked_rhs"] = out["gemm_bf16_f32acc_16x4096x4096"]
+    # matrix x vector: 2048 of the 16384 rows, all cores over rows
+    av = inputs.uniform(inputs.seed_for(1, 3), 2048 * 16384, -1.0, 1.0)
+    xv = inputs.uniform(inputs.seed_for(1, 2), 16384, -1.0, 1.0)
+    sec = timed(lambda: oracle.gemm_f32(2048, 1, 16384, av, xv, threads=cores), repeat=3)
+    out["gemv_f32_16384x1x16384"] = _cpu(2 * 2048 * 16384, sec, cores, f"2048 of 16384 rows, best of 3, {cores} threads")
     # config 5: one layer (+ embedding, final norm, head) on one of 16 sequences, single thread, scaled
     vocab, d, heads, ff, seq = 256, 512, 8, 2048, 1024
     weights = inputs.normal(inputs.seed_for(5, 0), oracle.decoder_weight_count(vocab, d, heads, 1, ff), 0.0, 0.02)
@@ -443,6 +476,7 @@ def main():
         ("attention_bf16", lambda: wl_attention_bf16(hip, inputs, timer, warm, steps)),
         ("decoder", lambda: wl_decoder(hip, inputs, timer, long_warm, long_steps)),
         ("rowops", lambda: wl_rowops(hip, inputs, timer, warm, steps)),
+        ("lopsided", lambda: wl_lopsided(hip, inputs, timer, long_warm, long_steps)),
         ("calibration", lambda: wl_calibration(hip, inputs, timer, long_warm, long_steps)),
     ]
     for name, fn in plan:
