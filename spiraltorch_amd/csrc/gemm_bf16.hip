@@ -1751,6 +1751,34 @@ __global__ __launch_bounds__(256) void gemm_bf16_skinny_reduce_kernel(SkinnyArgs
     if (p.C16) p.C16[idx] = f32_to_bf16_rne(value);
 }
 
+// The same for many splits of a small plane (64×64×100000 on the general kernel is 195 slices of 4096 values): sixteen
+// lanes per output value, lane j adding splits j, j + 16, ... in order, then a butterfly over the sixteen — a fixed
+// tree, so still independent of scheduling.
+__global__ __launch_bounds__(256) void gemm_bf16_reduce_wide_kernel(SkinnyArgs p)
+{
+    const size_t plane = static_cast<size_t>(p.M) * p.N;
+    const int lane16 = threadIdx.x & 15;
+    const size_t idx = static_cast<size_t>(blockIdx.x) * 16 + (threadIdx.x >> 4);
+    const bool valid = idx < plane;
+    float value = 0.0f;
+    for (int s0 = lane16; s0 < p.k_splits; s0 += 128) {
+        float part[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) part[j] = (valid && s0 + 16 * j < p.k_splits) ? p.partial[(s0 + 16 * j) * plane + idx] : 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) value += part[j];
+    }
+#pragma unroll
+    for (int offset = 8; offset > 0; offset >>= 1) value += __shfl_xor(value, offset, 16);
+    if (!valid || lane16 != 0) return;
+    if (p.scale != 1.0f) value *= p.scale;
+    if (p.bias) value += p.bias[idx % p.N];
+    if (p.residual) value += p.residual[idx];
+    value = apply_activation(value, p.activation);
+    if (p.C32) p.C32[idx] = value;
+    if (p.C16) p.C16[idx] = f32_to_bf16_rne(value);
+}
+
 // The split of a skinny problem over workgroups; fills the shape fields of `sk` and returns the bytes of partial sums.
 size_t plan_skinny(const GemmBf16Args &args, SkinnyArgs &sk)
 {
@@ -2248,8 +2276,11 @@ hipError_t launch_tile(GemmBf16Args args, bool vec, hipStream_t stream, size_t w
     rc = hipGetLastError();
     if (rc != hipSuccess || args.k_splits == 1) return rc;
     const size_t plane = static_cast<size_t>(args.M) * args.N;
-    hipLaunchKernelGGL(gemm_bf16_skinny_reduce_kernel, dim3(static_cast<unsigned>((plane + 255) / 256)), dim3(256), 0, stream,
-                       reduce);
+    if (args.k_splits >= 32 && plane <= 65536)
+        hipLaunchKernelGGL(gemm_bf16_reduce_wide_kernel, dim3(static_cast<unsigned>((plane + 15) / 16)), dim3(256), 0, stream, reduce);
+    else
+        hipLaunchKernelGGL(gemm_bf16_skinny_reduce_kernel, dim3(static_cast<unsigned>((plane + 255) / 256)), dim3(256), 0, stream,
+                           reduce);
     return hipGetLastError();
 }
 

@@ -309,6 +309,30 @@ __global__ __launch_bounds__(256) void gemm_f32_slice_reduce_kernel(SliceReduceA
     p.C[idx] = apply_activation(value, p.activation);
 }
 
+// The same for many slices of a small plane (64×64×100000 is 128 slices of 4096 values: one thread per value would walk
+// 128 loads in sixteen dependent rounds on sixteen workgroups): sixteen lanes per output value, lane j adding slices
+// j, j + 16, ... in order, then a butterfly over the sixteen — a fixed tree, so still independent of scheduling.
+__global__ __launch_bounds__(256) void gemm_f32_slice_reduce_wide_kernel(SliceReduceArgs p)
+{
+    const int lane16 = threadIdx.x & 15;
+    const size_t idx = static_cast<size_t>(blockIdx.x) * 16 + (threadIdx.x >> 4);
+    const bool valid = idx < p.plane;
+    float value = 0.0f;
+    for (int s0 = lane16; s0 < p.slices; s0 += 128) {
+        float part[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) part[j] = (valid && s0 + 16 * j < p.slices) ? p.partial[(s0 + 16 * j) * p.plane + idx] : 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) value += part[j];
+    }
+#pragma unroll
+    for (int offset = 8; offset > 0; offset >>= 1) value += __shfl_xor(value, offset, 16);
+    if (!valid || lane16 != 0) return;
+    value = value * p.scale + (p.bias ? p.bias[idx % p.N] : -0.0f);
+    if (p.residual) value += p.residual[idx];
+    p.C[idx] = apply_activation(value, p.activation);
+}
+
 // How many k-slices a launch of `tiles` workgroups, each walking `k_steps` k-tiles, is cut into: none while the tiles
 // alone give every other compute unit a workgroup; otherwise enough for about two workgroups per compute unit, each
 // slice keeping at least `min_steps` k-tiles, and the partial planes (written once, read once) staying below the
@@ -349,8 +373,12 @@ hipError_t launch_k_sliced(GemmF32Args args, size_t slices, size_t k_steps, int 
     args.slice_k = static_cast<int>(steps_per_slice) * bk;
     rc = launch(args, static_cast<unsigned>(slices));
     if (rc != hipSuccess) return rc;
-    hipLaunchKernelGGL(gemm_f32_slice_reduce_kernel, dim3(static_cast<unsigned>((plane + 255) / 256)), dim3(256), 0, stream,
-                       reduce);
+    if (slices >= 32 && plane <= 65536)
+        hipLaunchKernelGGL(gemm_f32_slice_reduce_wide_kernel, dim3(static_cast<unsigned>((plane + 15) / 16)), dim3(256), 0, stream,
+                           reduce);
+    else
+        hipLaunchKernelGGL(gemm_f32_slice_reduce_kernel, dim3(static_cast<unsigned>((plane + 255) / 256)), dim3(256), 0, stream,
+                           reduce);
     return hipGetLastError();
 }
 
