@@ -337,10 +337,11 @@ __global__ __launch_bounds__(256) void gemm_f32_slice_reduce_wide_kernel(SliceRe
 // alone give every other compute unit a workgroup; otherwise enough for about two workgroups per compute unit, each
 // slice keeping at least `min_steps` k-tiles, and the partial planes (written once, read once) staying below the
 // operands' bytes.
-size_t choose_k_slices(size_t m, size_t n, size_t k, size_t tiles, size_t k_steps, size_t min_steps)
+size_t choose_k_slices(size_t m, size_t n, size_t k, size_t tiles, size_t k_steps, size_t min_steps, size_t most_tiles = 128,
+                       size_t most_groups = 512)
 {
-    if (tiles > 128 || k_steps < 2 * min_steps) return 1;
-    size_t slices = std::min<size_t>(512 / tiles, k_steps / min_steps);
+    if (tiles > most_tiles || k_steps < 2 * min_steps) return 1;
+    size_t slices = std::min<size_t>(most_groups / tiles, k_steps / min_steps);
     while (slices > 1 && slices * m * n * 2 > m * k + k * n) --slices;
     return std::max<size_t>(slices, 1);
 }
@@ -823,7 +824,9 @@ hipError_t launch_ring(GemmF32Args args, bool lhs_transposed, bool rhs_packed, b
     };
     // Few tiles and a long k (a weight gradient Xᵀ·dY of a small layer over many rows): cut along k over workgroups.
     const size_t k_steps = static_cast<size_t>(args.K) / 16;
-    const size_t slices = big || !scratch_free ? 1 : choose_k_slices(args.M, args.N, args.K, tiles, k_steps, 16);
+    // (768 of the 64×64 workgroups are resident at a time, and with fewer than half of that a 16-wide k-tile costs a
+    // workgroup half a microsecond of load latency: 1576×768×3072, 300 tiles of 192 k-tiles, took 102 µs.)
+    const size_t slices = big || !scratch_free ? 1 : choose_k_slices(args.M, args.N, args.K, tiles, k_steps, 16, 384, 768);
     if (slices > 1) return launch_k_sliced(args, slices, k_steps, 16, stream, launch);
     return launch(args, 1);
 }
@@ -889,7 +892,11 @@ hipError_t launch_gemm_f32(size_t m, size_t n, size_t k, bool lhs_transposed, co
                          (!lhs_transposed || m % 4 == 0);
     const size_t big_tiles = ((m + 255) / 256) * ((n + 255) / 256);
     const bool little_padding = (m % 256 == 0 || m >= 2048) && (n % 256 == 0 || n >= 2048);
-    if (big_tiles >= 256 && little_padding) return launch_tile<256, 256, 4, 4>(args, lhs_transposed, vec, stream);
+    // ... and in rounds of 256 that are mostly full: 300 tiles are two rounds for the work of 1.17 (6304×3072×768: 399 µs
+    // on these tiles, 74 TFLOP/s; the ring kernel's 128×128 tiles, 768 resident, quantise finer).
+    const double rounds_fill = static_cast<double>(big_tiles) / static_cast<double>((big_tiles + 255) / 256 * 256);
+    if (big_tiles >= 256 && little_padding && (rounds_fill >= 0.8 || !ring_ok))
+        return launch_tile<256, 256, 4, 4>(args, lhs_transposed, vec, stream);
     if (ring_ok) {
         // 128×128 tiles (three workgroups per compute unit, 768 at a time) when they come in full rounds or many
         // rounds; 64×64 tiles otherwise, which spread small problems and leave a shorter tail.
