@@ -147,6 +147,94 @@ __device__ __forceinline__ T block_reduce(T v, T *scratch, Op op)
     return total;
 }
 
+// Rows of up to 65536 values held in the registers of one 1024-thread workgroup (CH 16-byte pieces per thread, all
+// requested before the first reduction): the row is read once and written once, whatever its alignment — a row of
+// 50257 values starts at any 4-byte boundary, which global memory takes for 16-byte accesses; the types say so.
+typedef float f32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+typedef unsigned int u32x2_a2 __attribute__((ext_vector_type(2), aligned(2)));
+
+template <int CH>
+__global__ __launch_bounds__(1024) void layer_norm_block_kernel(int cols, const float *x, const float *residual,
+                                                                const float *gamma, const float *beta, float epsilon,
+                                                                float *out_f32, uint16_t *out_bf16)
+{
+    __shared__ float scratch[16];
+    const int tid = threadIdx.x;
+    const size_t offset = static_cast<size_t>(blockIdx.x) * cols;
+    float v[CH][4];
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+        const int c = (tid + 1024 * i) * 4;
+        if (c + 4 <= cols) {
+            const f32x4_a4 t = *reinterpret_cast<const f32x4_a4 *>(x + offset + c);
+            v[i][0] = t[0]; v[i][1] = t[1]; v[i][2] = t[2]; v[i][3] = t[3];
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[i][e] = c + e < cols ? x[offset + c + e] : 0.0f;
+        }
+    }
+    if (residual) {
+#pragma unroll
+        for (int i = 0; i < CH; ++i) {
+            const int c = (tid + 1024 * i) * 4;
+            if (c + 4 <= cols) {
+                const f32x4_a4 t = *reinterpret_cast<const f32x4_a4 *>(residual + offset + c);
+                v[i][0] += t[0]; v[i][1] += t[1]; v[i][2] += t[2]; v[i][3] += t[3];
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (c + e < cols) v[i][e] += residual[offset + c + e];
+            }
+        }
+    }
+    float sum = 0.0f, sumsq = 0.0f;
+#pragma unroll
+    for (int i = 0; i < CH; ++i)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {  // values past the end are zero
+            sum += v[i][e];
+            sumsq = fmaf(v[i][e], v[i][e], sumsq);
+        }
+    auto add = [](float a, float b) { return a + b; };
+    sum = block_reduce<1024>(sum, scratch, add);
+    sumsq = block_reduce<1024>(sumsq, scratch, add);
+    const float cols_f = static_cast<float>(cols);
+    const float mean = sum / cols_f;
+    const float var = fmaxf(sumsq / cols_f - mean * mean, 0.0f);
+    const float denom = sqrtf(var + epsilon);
+    const float inv = 1.0f / denom;
+    auto quotient = [&](float a) {  // a / denom, correctly rounded (see layer_norm_vec_kernel)
+        const float q = a * inv;
+        return fmaf(fmaf(-q, denom, a), inv, q);
+    };
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+        const int c = (tid + 1024 * i) * 4;
+        if (c >= cols) continue;
+        float o[4];
+        if (c + 4 <= cols) {
+            const f32x4_a4 g = *reinterpret_cast<const f32x4_a4 *>(gamma + c), b = *reinterpret_cast<const f32x4_a4 *>(beta + c);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] = quotient(v[i][e] - mean) * g[e] + b[e];
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] = c + e < cols ? quotient(v[i][e] - mean) * gamma[c + e] + beta[c + e] : 0.0f;
+        }
+        if (c + 4 <= cols) {
+            if (out_f32) *reinterpret_cast<f32x4_a4 *>(out_f32 + offset + c) = f32x4_a4{o[0], o[1], o[2], o[3]};
+            if (out_bf16)
+                *reinterpret_cast<u32x2_a2 *>(out_bf16 + offset + c) = u32x2_a2{pack_bf16x2_rne(o[0], o[1]), pack_bf16x2_rne(o[2], o[3])};
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                if (c + e >= cols) continue;
+                if (out_f32) out_f32[offset + c + e] = o[e];
+                if (out_bf16) out_bf16[offset + c + e] = f32_to_bf16_rne(o[e]);
+            }
+        }
+    }
+}
+
 // Long rows (more than 2048 values, or rows that are not 16-byte aligned): one workgroup per row, two sweeps over the
 // row (statistics, then the normalisation; the second sweep is served by the caches for rows of up to a few MB).
 template <int THREADS, bool VEC>
@@ -487,6 +575,79 @@ __global__ __launch_bounds__(THREADS) void row_softmax_long_kernel(int cols, con
     }
 }
 
+// The same for softmax: the row stays in the registers of a 1024-thread workgroup through all three phases.
+template <int CH>
+__global__ __launch_bounds__(1024) void row_softmax_block_kernel(int cols, const float *in, float *out)
+{
+    __shared__ float scratch_f[16];
+    __shared__ int scratch_i[16];
+    const int tid = threadIdx.x;
+    const float *x = in + static_cast<size_t>(blockIdx.x) * cols;
+    float *y = out + static_cast<size_t>(blockIdx.x) * cols;
+    float v[CH][4];
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+        const int c = (tid + 1024 * i) * 4;
+        if (c + 4 <= cols) {
+            const f32x4_a4 t = *reinterpret_cast<const f32x4_a4 *>(x + c);
+            v[i][0] = t[0]; v[i][1] = t[1]; v[i][2] = t[2]; v[i][3] = t[3];
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[i][e] = c + e < cols ? x[c + e] : __builtin_nanf("");  // skipped like NaN entries
+        }
+    }
+    float best = -INFINITY;
+    int best_index = 0x7fffffff;
+#pragma unroll
+    for (int i = 0; i < CH; ++i)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {  // ascending columns per thread: the first occurrence wins
+            const float value = v[i][e];
+            if (value != value) continue;
+            if (best_index == 0x7fffffff || value > best) {
+                best = value;
+                best_index = (tid + 1024 * i) * 4 + e;
+            }
+        }
+    const float row_max = block_reduce<1024>(best_index == 0x7fffffff ? -INFINITY : best, scratch_f,
+                                             [](float a, float b) { return fmaxf(a, b); });
+    const int candidate = block_reduce<1024>((best_index != 0x7fffffff && best == row_max) ? best_index : 0x7fffffff, scratch_i,
+                                             [](int a, int b) { return min(a, b); });
+    const bool found = candidate != 0x7fffffff;
+    const float base = (found && isfinite(row_max)) ? row_max : 0.0f;
+    float denom = 0.0f;
+#pragma unroll
+    for (int i = 0; i < CH; ++i)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float value = v[i][e];
+            const float weight = (!found || value != value) ? 0.0f : __expf(value - base);
+            v[i][e] = weight;
+            denom += weight;
+        }
+    denom = block_reduce<1024>(denom, scratch_f, [](float a, float b) { return a + b; });
+    const bool normal = isfinite(denom) && denom > 1.1920929e-7f;
+    const float inv = normal ? 1.0f / denom : 0.0f;
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+        const int c = (tid + 1024 * i) * 4;
+        if (c >= cols) continue;
+        float o[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            o[e] = v[i][e] * inv;
+            if (found && !normal) o[e] = (c + e == candidate) ? 1.0f : 0.0f;
+        }
+        if (c + 4 <= cols) {
+            *reinterpret_cast<f32x4_a4 *>(y + c) = f32x4_a4{o[0], o[1], o[2], o[3]};
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (c + e < cols) y[c + e] = o[e];
+        }
+    }
+}
+
 // Gelu::forward, crates/st-nn/src/layers/gelu.rs:78-94 (the tanh form of crates/st-tensor/src/pure.rs:12026-12031).
 __global__ __launch_bounds__(256) void gelu_forward_kernel(size_t count, const float *in, float *out)
 {
@@ -721,7 +882,20 @@ hipError_t launch_layer_norm_f32(size_t rows, size_t cols, const float *x, const
     else if (vec)
         hipLaunchKernelGGL((layer_norm_vec_kernel<8, 1>), grid, block, 0, stream, r, c, x, residual, gamma, beta, epsilon,
                            out_f32, out_bf16);
-    else if (cols > 2048) {
+    else if (cols > 4096 && cols <= 65536) {
+        // The row in the registers of a 1024-thread workgroup: 2 to 16 pieces of 16 bytes per thread.
+        const dim3 rows_grid(static_cast<unsigned>(rows));
+        const size_t pieces = (cols + 4095) / 4096;
+#define ST_LN_BLOCK(CH)                                                                                                     \
+    hipLaunchKernelGGL((layer_norm_block_kernel<CH>), rows_grid, dim3(1024), 0, stream, c, x, residual, gamma, beta, epsilon, \
+                       out_f32, out_bf16)
+        if (pieces <= 2) ST_LN_BLOCK(2);
+        else if (pieces <= 4) ST_LN_BLOCK(4);
+        else if (pieces <= 8) ST_LN_BLOCK(8);
+        else if (pieces <= 12) ST_LN_BLOCK(12);
+        else ST_LN_BLOCK(16);
+#undef ST_LN_BLOCK
+    } else if (cols > 2048) {
         // A workgroup per row: 1024 threads while the rows are few, 256 once the rows alone fill the chip.
         const bool vec_long = cols % 4 == 0 && aligned(x, 16) && aligned(residual, 16) && aligned(out_f32, 16) && aligned(out_bf16, 8);
         const dim3 rows_grid(static_cast<unsigned>(rows));
@@ -803,7 +977,16 @@ hipError_t launch_row_softmax_f32(size_t rows, size_t cols, const float *in, flo
         hipLaunchKernelGGL(row_softmax_vec_kernel<4>, grid, block, 0, stream, r, c, in, out);
     else if (vec)
         hipLaunchKernelGGL(row_softmax_vec_kernel<8>, grid, block, 0, stream, r, c, in, out);
-    else if (cols > 2048) {
+    else if (cols > 4096 && cols <= 65536) {
+        // The row in the registers of a 1024-thread workgroup: 2 to 16 pieces of 16 bytes per thread.
+        const dim3 rows_grid(static_cast<unsigned>(rows));
+        const size_t pieces = (cols + 4095) / 4096;
+        if (pieces <= 2) hipLaunchKernelGGL(row_softmax_block_kernel<2>, rows_grid, dim3(1024), 0, stream, c, in, out);
+        else if (pieces <= 4) hipLaunchKernelGGL(row_softmax_block_kernel<4>, rows_grid, dim3(1024), 0, stream, c, in, out);
+        else if (pieces <= 8) hipLaunchKernelGGL(row_softmax_block_kernel<8>, rows_grid, dim3(1024), 0, stream, c, in, out);
+        else if (pieces <= 12) hipLaunchKernelGGL(row_softmax_block_kernel<12>, rows_grid, dim3(1024), 0, stream, c, in, out);
+        else hipLaunchKernelGGL(row_softmax_block_kernel<16>, rows_grid, dim3(1024), 0, stream, c, in, out);
+    } else if (cols > 2048) {
         // A workgroup per row: 1024 threads while the rows are few, 256 once the rows alone fill the chip.
         const bool vec_long = cols % 4 == 0 && ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0;
         const dim3 rows_grid(static_cast<unsigned>(rows));

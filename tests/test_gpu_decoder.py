@@ -14,7 +14,9 @@ def test_layer_norm(hip, oracle):
     for rows, cols in ((1, 1), (5, 48), (130, 512), (7, 1000), (9, 1536), (3, 2048), (4, 2052), (6, 4100), (16384, 512),
                        (16387, 256), (16389, 1024),
                        # rows longer than 2048: a workgroup per row (1024 threads; 256 from 2048 rows on)
-                       (3, 100000), (2, 50001), (2100, 2056), (2049, 2051)):
+                       (3, 100000), (2, 50001), (2100, 2056), (2049, 2051),
+                       # 4097 to 65536 values: the row held in the registers of a 1024-thread workgroup
+                       (5, 50257), (3, 65536), (4, 20003), (2, 8192), (300, 4098)):
         x = rng.normal(1.0, 2.0, rows * cols).astype(np.float32)
         res = rng.normal(size=rows * cols).astype(np.float32)
         g, b = rng.normal(size=cols).astype(np.float32), rng.normal(size=cols).astype(np.float32)

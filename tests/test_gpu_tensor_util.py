@@ -13,8 +13,10 @@ def on_device(hip, *arrays):
 
 @pytest.mark.parametrize("rows,cols", [(1, 1), (2, 4), (5, 63), (7, 64), (3, 65), (33, 1000), (1024, 256), (4, 5000), (9, 512), (6, 516), (5, 2048), (3, 2052),
                                        (16384, 512), (16387, 128), (16389, 1024),
-                                       # rows longer than 2048: a workgroup per row (1024 threads; 256 from 2048 rows on)
-                                       (3, 100000), (2, 50001), (2100, 2052), (2049, 2051)])
+                                       # rows longer than 2048: a workgroup per row sweeping it (1024 threads; 256 from 2048 rows on)
+                                       (3, 100000), (2, 50001), (2100, 2052), (2049, 2051),
+                                       # 4097 to 65536 values: the row held in the registers of a 1024-thread workgroup
+                                       (5, 50257), (3, 65536), (4, 20003), (2, 8192), (300, 4098)])
 def test_row_softmax(hip, oracle, rows, cols):
     rng = np.random.default_rng(rows * 31 + cols)
     x = (rng.normal(size=rows * cols) * 3).astype(np.float32)
