@@ -655,6 +655,16 @@ __global__ __launch_bounds__(256) void gelu_forward_kernel(size_t count, const f
     for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < count; i += stride) out[i] = gelu_tanh(in[i]);
 }
 
+// Four values per thread and access when the buffers are 16-byte aligned.
+__global__ __launch_bounds__(256) void gelu_forward_vec_kernel(size_t count4, const float4 *in, float4 *out)
+{
+    const size_t stride = static_cast<size_t>(gridDim.x) * 256;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < count4; i += stride) {
+        const float4 v = in[i];
+        out[i] = make_float4(gelu_tanh(v.x), gelu_tanh(v.y), gelu_tanh(v.z), gelu_tanh(v.w));
+    }
+}
+
 // status[0] = number of non-finite values, status[1] = smallest index of one (status[1] must start at ~0).
 // The first workgroup resets nothing: the caller clears the two words before the launch.
 __global__ __launch_bounds__(256) void nonfinite_probe_kernel(size_t count, const float *data, unsigned long long *status)
@@ -770,6 +780,10 @@ __global__ __launch_bounds__(256) void sum_axis0_partial_kernel(int rows, int co
 
 // 16-byte aligned rows: a workgroup covers 256 columns (64 lanes × 4) and its four wavefronts take every fourth
 // row of the chunk, eight independent loads in flight each; the four partial rows are added through LDS.
+// ALIGNED: every row starts on a 16-byte boundary (cols a multiple of 4, aligned base).  Otherwise the 16-byte accesses
+// go through a vector type that says 4-byte alignment (global memory takes them), and the last group of a row, which
+// may hang over its end, is read value by value.
+template <bool ALIGNED>
 __global__ __launch_bounds__(256) void sum_axis0_partial_vec_kernel(int rows, int cols, int rows_per_chunk, const float *in,
                                                                     float *partial)
 {
@@ -778,6 +792,18 @@ __global__ __launch_bounds__(256) void sum_axis0_partial_vec_kernel(int rows, in
     const int c = (blockIdx.x * 64 + lane) * 4;
     const int r0 = blockIdx.y * rows_per_chunk;
     const int r1 = min(rows, r0 + rows_per_chunk);
+    const bool whole = c + 4 <= cols;  // all four columns exist
+    auto load = [&](const float *p) {
+        if constexpr (ALIGNED) {
+            return *reinterpret_cast<const float4 *>(p);
+        } else {
+            if (whole) {
+                const f32x4_a4 t = *reinterpret_cast<const f32x4_a4 *>(p);
+                return make_float4(t[0], t[1], t[2], t[3]);
+            }
+            return make_float4(p[0], c + 1 < cols ? p[1] : 0.0f, c + 2 < cols ? p[2] : 0.0f, 0.0f);
+        }
+    };
     float4 acc[2] = {make_float4(0.f, 0.f, 0.f, 0.f), make_float4(0.f, 0.f, 0.f, 0.f)};
     if (c < cols) {
         const float *src = in + c;
@@ -785,14 +811,14 @@ __global__ __launch_bounds__(256) void sum_axis0_partial_vec_kernel(int rows, in
         for (; r + 28 < r1; r += 32) {
             float4 t[8];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) t[u] = *reinterpret_cast<const float4 *>(src + static_cast<size_t>(r + 4 * u) * cols);
+            for (int u = 0; u < 8; ++u) t[u] = load(src + static_cast<size_t>(r + 4 * u) * cols);
 #pragma unroll
             for (int u = 0; u < 8; ++u) {
                 acc[u & 1].x += t[u].x; acc[u & 1].y += t[u].y; acc[u & 1].z += t[u].z; acc[u & 1].w += t[u].w;
             }
         }
         for (; r < r1; r += 4) {
-            const float4 t = *reinterpret_cast<const float4 *>(src + static_cast<size_t>(r) * cols);
+            const float4 t = load(src + static_cast<size_t>(r) * cols);
             acc[0].x += t.x; acc[0].y += t.y; acc[0].z += t.z; acc[0].w += t.w;
         }
     }
@@ -804,7 +830,15 @@ __global__ __launch_bounds__(256) void sum_axis0_partial_vec_kernel(int rows, in
         for (int k = 1; k < 4; ++k) {
             total.x += stage[k][lane].x; total.y += stage[k][lane].y; total.z += stage[k][lane].z; total.w += stage[k][lane].w;
         }
-        *reinterpret_cast<float4 *>(partial + static_cast<size_t>(blockIdx.y) * cols + c) = total;
+        float *dst = partial + static_cast<size_t>(blockIdx.y) * cols + c;
+        if constexpr (ALIGNED) {
+            *reinterpret_cast<float4 *>(dst) = total;
+        } else {
+            dst[0] = total.x;
+            if (c + 1 < cols) dst[1] = total.y;
+            if (c + 2 < cols) dst[2] = total.z;
+            if (c + 3 < cols) dst[3] = total.w;
+        }
     }
 }
 
@@ -1005,7 +1039,11 @@ hipError_t launch_row_softmax_f32(size_t rows, size_t cols, const float *in, flo
 hipError_t launch_gelu_f32(size_t count, const float *in, float *out, hipStream_t stream)
 {
     if (count == 0) return hipSuccess;
-    hipLaunchKernelGGL(gelu_forward_kernel, dim3(grid_for(count)), dim3(256), 0, stream, count, in, out);
+    if (count % 4 == 0 && ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0)
+        hipLaunchKernelGGL(gelu_forward_vec_kernel, dim3(grid_for(count / 4)), dim3(256), 0, stream, count / 4,
+                           reinterpret_cast<const float4 *>(in), reinterpret_cast<float4 *>(out));
+    else
+        hipLaunchKernelGGL(gelu_forward_kernel, dim3(grid_for(count)), dim3(256), 0, stream, count, in, out);
     return hipGetLastError();
 }
 
@@ -1074,7 +1112,10 @@ hipError_t launch_sum_axis0_f32(size_t rows, size_t cols, const float *in, float
     float *partial = static_cast<float *>(workspace);
     const dim3 grid(static_cast<unsigned>(col_blocks), static_cast<unsigned>(chunks));
     if (vec)
-        hipLaunchKernelGGL(sum_axis0_partial_vec_kernel, grid, dim3(256), 0, stream, static_cast<int>(rows),
+        hipLaunchKernelGGL(sum_axis0_partial_vec_kernel<true>, grid, dim3(256), 0, stream, static_cast<int>(rows),
+                           static_cast<int>(cols), static_cast<int>(rows_per_chunk), in, partial);
+    else if (cols >= 64)
+        hipLaunchKernelGGL(sum_axis0_partial_vec_kernel<false>, grid, dim3(256), 0, stream, static_cast<int>(rows),
                            static_cast<int>(cols), static_cast<int>(rows_per_chunk), in, partial);
     else
         hipLaunchKernelGGL(sum_axis0_partial_kernel, grid, dim3(256), 0, stream, static_cast<int>(rows),

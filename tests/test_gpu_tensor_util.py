@@ -129,7 +129,9 @@ def test_elementwise_kernels_on_unaligned_pointers(hip, oracle):
     assert (d_x.to_array(np.float32, n + 1)[1:] == oracle.add_row_f32(rows, cols, x[1:], bias[1:])).all()
 
 
-@pytest.mark.parametrize("rows,cols", [(1, 1), (3, 2), (64, 256), (65, 257), (1000, 19), (16384, 512), (100000, 8), (37, 260), (131, 1028), (5, 4)])
+@pytest.mark.parametrize("rows,cols", [(1, 1), (3, 2), (64, 256), (65, 257), (1000, 19), (16384, 512), (100000, 8), (37, 260), (131, 1028), (5, 4),
+                                       # rows that do not start on 16-byte boundaries: 16-byte loads all the same
+                                       (300, 1001), (4097, 67), (70, 50257), (129, 66)])
 def test_sum_axis0(hip, oracle, rows, cols):
     rng = np.random.default_rng(rows + cols)
     x = rng.normal(size=rows * cols).astype(np.float32)
@@ -253,6 +255,18 @@ def test_gelu_forward_matches_the_oracle(hip, oracle):
     x = st.Tensor(3, 50, np.linspace(-6, 6, 150).astype(np.float32))
     want = np.array([oracle.gelu(float(v)) for v in x.data()])
     assert_close(x.gelu().data(), want, F32_REL, F32_ABS, "gelu")
+    # a count that is a multiple of four takes the 128-bit kernel; the same values through both kernels agree bit for bit
+    values = np.concatenate([np.linspace(-12, 12, 4093), [0.0, -0.0, 88.0, -88.0, 1e-30, -1e-30, 3.0e38]]).astype(np.float32)
+    assert values.size % 4 == 0
+    d_in, d_out, d_odd = hip.DeviceBuffer.from_array(values), hip.DeviceBuffer(values.nbytes), hip.DeviceBuffer(values.nbytes)
+    hip.gelu_f32_dev(values.size, d_in, d_out)
+    hip.gelu_f32_dev(values.size - 1, d_in, d_odd)
+    hip.device_synchronize()
+    got = d_out.to_array(np.float32, values.size)
+    v64 = values.astype(np.float64)
+    inner = np.sqrt(2.0 / np.pi) * (v64 + 0.044715 * v64 ** 3)
+    assert_close(got, 0.5 * v64 * (1.0 + np.tanh(inner)), F32_REL, F32_ABS, "gelu, 128-bit kernel")
+    assert (got[:-1] == d_odd.to_array(np.float32, values.size - 1)).all()
 
 
 def test_raw_gemm_and_probe(hip):
