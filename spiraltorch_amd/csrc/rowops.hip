@@ -888,6 +888,11 @@ unsigned grid_for(size_t count)
 
 }  // namespace
 
+// A count that is a multiple of four takes the 128-bit kernels as a whole; a large one that is not takes them for all
+// but its last one to three values, which a second, one-workgroup launch of the scalar kernel finishes (the two
+// kernels compute the same bits).
+bool vec_with_tail(size_t count) { return count % 4 == 0 || count >= (1u << 20); }
+
 hipError_t launch_layer_norm_f32(size_t rows, size_t cols, const float *x, const float *residual, const float *gamma,
                                  const float *beta, float epsilon, float *out_f32, uint16_t *out_bf16,
                                  hipStream_t stream)
@@ -965,9 +970,11 @@ hipError_t launch_embedding_f32(size_t tokens, size_t vocab, size_t dim, const f
 hipError_t launch_f32_to_bf16(size_t count, const float *in, uint16_t *out, hipStream_t stream)
 {
     if (count == 0) return hipSuccess;
-    if (count % 4 == 0 && aligned16(in) && (reinterpret_cast<uintptr_t>(out) & 7u) == 0) {
+    if (vec_with_tail(count) && aligned16(in) && (reinterpret_cast<uintptr_t>(out) & 7u) == 0) {
+        const size_t body = count / 4 * 4;
         hipLaunchKernelGGL(f32_to_bf16_vec_kernel, dim3(grid_vec_for(count / 4)), dim3(256), 0, stream, count / 4,
                            reinterpret_cast<const float4 *>(in), reinterpret_cast<uint2 *>(out));
+        if (body < count) hipLaunchKernelGGL(f32_to_bf16_kernel, dim3(1), dim3(256), 0, stream, count - body, in + body, out + body);
         return hipGetLastError();
     }
     hipLaunchKernelGGL(f32_to_bf16_kernel, dim3(grid_for(count)), dim3(256), 0, stream, count, in, out);
@@ -1039,11 +1046,14 @@ hipError_t launch_row_softmax_f32(size_t rows, size_t cols, const float *in, flo
 hipError_t launch_gelu_f32(size_t count, const float *in, float *out, hipStream_t stream)
 {
     if (count == 0) return hipSuccess;
-    if (count % 4 == 0 && ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0)
+    if (vec_with_tail(count) && ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0) {
+        const size_t body = count / 4 * 4;
         hipLaunchKernelGGL(gelu_forward_vec_kernel, dim3(grid_for(count / 4)), dim3(256), 0, stream, count / 4,
                            reinterpret_cast<const float4 *>(in), reinterpret_cast<float4 *>(out));
-    else
+        if (body < count) hipLaunchKernelGGL(gelu_forward_kernel, dim3(1), dim3(256), 0, stream, count - body, in + body, out + body);
+    } else {
         hipLaunchKernelGGL(gelu_forward_kernel, dim3(grid_for(count)), dim3(256), 0, stream, count, in, out);
+    }
     return hipGetLastError();
 }
 
@@ -1056,10 +1066,13 @@ hipError_t launch_nonfinite_probe_f32(size_t count, const float *data, unsigned 
 hipError_t launch_gelu_backward_f32(size_t count, const float *z, const float *grad, float *out, hipStream_t stream)
 {
     if (count == 0) return hipSuccess;
-    if (count % 4 == 0 && aligned16(z) && aligned16(grad) && aligned16(out)) {
+    if (vec_with_tail(count) && aligned16(z) && aligned16(grad) && aligned16(out)) {
+        const size_t body = count / 4 * 4;
         hipLaunchKernelGGL(gelu_backward_vec_kernel, dim3(grid_vec_for(count / 4)), dim3(256), 0, stream, count / 4,
                            reinterpret_cast<const float4 *>(z), reinterpret_cast<const float4 *>(grad),
                            reinterpret_cast<float4 *>(out));
+        if (body < count)
+            hipLaunchKernelGGL(gelu_backward_kernel, dim3(1), dim3(256), 0, stream, count - body, z + body, grad + body, out + body);
         return hipGetLastError();
     }
     hipLaunchKernelGGL(gelu_backward_kernel, dim3(grid_for(count)), dim3(256), 0, stream, count, z, grad, out);
@@ -1069,9 +1082,11 @@ hipError_t launch_gelu_backward_f32(size_t count, const float *z, const float *g
 hipError_t launch_scale_f32(size_t count, const float *in, float scale, float *out, hipStream_t stream)
 {
     if (count == 0) return hipSuccess;
-    if (count % 4 == 0 && aligned16(in) && aligned16(out)) {
+    if (vec_with_tail(count) && aligned16(in) && aligned16(out)) {
+        const size_t body = count / 4 * 4;
         hipLaunchKernelGGL(scale_vec_kernel, dim3(grid_vec_for(count / 4)), dim3(256), 0, stream, count / 4,
                            reinterpret_cast<const float4 *>(in), scale, reinterpret_cast<float4 *>(out));
+        if (body < count) hipLaunchKernelGGL(scale_kernel, dim3(1), dim3(256), 0, stream, count - body, in + body, scale, out + body);
         return hipGetLastError();
     }
     hipLaunchKernelGGL(scale_kernel, dim3(grid_for(count)), dim3(256), 0, stream, count, in, scale, out);

@@ -269,6 +269,35 @@ def test_gelu_forward_matches_the_oracle(hip, oracle):
     assert (got[:-1] == d_odd.to_array(np.float32, values.size - 1)).all()
 
 
+@pytest.mark.parametrize("tail", [1, 3])
+def test_large_counts_that_are_not_multiples_of_four(hip, oracle, tail):
+    """From 2^20 values on, the 128-bit kernels take all but the last one to three values and a second launch of the
+    scalar kernel finishes them."""
+    from spiraltorch_amd import inputs
+    n = (1 << 20) + tail
+    rng = np.random.default_rng(tail)
+    x = (rng.normal(size=n) * 2).astype(np.float32)
+    g = rng.normal(size=n).astype(np.float32)
+    d_x, d_g = on_device(hip, x, g)
+    d_out = hip.DeviceBuffer(n * 4)
+    d_out.zero()
+    hip.scale_f32_dev(n, d_x, -0.37, d_out)
+    hip.device_synchronize()
+    assert (d_out.to_array(np.float32, n) == oracle.scale_f32(x, -0.37)).all()
+    hip.gelu_backward_f32_dev(n, d_x, d_g, d_out)
+    hip.device_synchronize()
+    assert_close(d_out.to_array(np.float32, n), oracle.gelu_backward_f32(x, g), F32_REL, F32_ABS, "gelu_backward")
+    hip.gelu_f32_dev(n, d_x, d_out)
+    hip.device_synchronize()
+    x64 = x.astype(np.float64)
+    want = 0.5 * x64 * (1.0 + np.tanh(np.sqrt(2.0 / np.pi) * (x64 + 0.044715 * x64 ** 3)))
+    assert_close(d_out.to_array(np.float32, n), want, F32_REL, F32_ABS, "gelu")
+    d16 = hip.DeviceBuffer(n * 2)
+    hip.f32_to_bf16_dev(n, d_x, d16)
+    hip.device_synchronize()
+    assert (d16.to_array(np.uint16, n) == inputs.to_bf16(x)).all()
+
+
 def test_raw_gemm_and_probe(hip):
     """gemm_f32_raw and probe() of crates/st-backend-hip/src/lib.rs:188-207, 760-799."""
     a = np.arange(1, 7, dtype=np.float32)
