@@ -904,10 +904,10 @@ hipError_t launch_gemm_f32(size_t m, size_t n, size_t k, bool lhs_transposed, co
         const bool big = tiles128 >= 512 && (tiles128 >= 3072 || tiles128 % 768 == 0 || tiles128 % 768 >= 384);
         // Fewer 64×64 tiles than two per compute unit: 32×32 tiles with K split over the wavefronts of a workgroup.
         const size_t tiles64 = ((m + 63) / 64) * ((n + 63) / 64);
-        // (Up to 512: with one or two 64×64 workgroups on a compute unit a SIMD holds a single wavefront and its
+        // (Up to 448: with one or two 64×64 workgroups on a compute unit a SIMD holds a single wavefront and its
         // fragment reads and MFMAs do not overlap — 1576×768×768, 300 tiles: 28.4 µs on them, 20.2 µs on 32×32 tiles;
-        // at 752 tiles, 3000×1000×1024, the larger tiles are ahead again, 51.8 against 55.4 µs.)
-        if (!lhs_transposed && tiles64 <= 512 && k >= 128) return launch_splitk32(args, stream, scratch_free);
+        // from 512 tiles on the larger tiles are ahead again: 1024×2048×512 21.7 against 24.5 µs.)
+        if (!lhs_transposed && tiles64 <= 448 && k >= 128) return launch_splitk32(args, stream, scratch_free);
         return launch_ring(args, lhs_transposed, false, big, stream, scratch_free);
     }
     // Shapes the ring kernels do not take.  Few tiles and a long k (a matrix-vector product, n < 4, is the common case):
