@@ -598,6 +598,182 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DPAD <= 64 
     }  // pass
 }
 
+// -------------------------------------------------------------------------------------------------
+// Many short contexts (windowed attention: thousands of contexts of 16 to 64 positions).  The kernels above give a
+// context a workgroup and a 128-row query tile, which is mostly padding here, and such launches are memory-bound:
+// 16384 contexts of 16 × 64 took 218 µs, 1.2 TB/s.  Here ONE WAVEFRONT owns a context of up to 64 positions: it stages
+// that context's K and V (rows past the end as zeros) in a slice of LDS of its own, so nothing in the kernel waits on
+// a workgroup barrier, and with all keys present at once the softmax is the plain one, no running maximum.  Same
+// transposed products as above: Sᵀ = K·Qᵀ leaves every lane the scores of its own query, which are the B operand of
+// Oᵀ = Vᵀ·Pᵀ as they stand.  WAVES wavefronts (contexts) per workgroup: as many as fit the LDS.
+// -------------------------------------------------------------------------------------------------
+template <int DPAD, bool CAUSAL, int ROWS, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void attention_f32_tiny_kernel(AttnArgs p)
+{
+    constexpr int KS = DPAD + 4, VS = DPAD + 8;  // row strides as in the fast kernel (conflict-free fragment reads)
+    constexpr int K_ELEMS = ROWS * KS, V_ELEMS = ROWS * VS;  // ROWS: 32 or 64 staged positions, at least S
+    constexpr int CHUNKS = DPAD / 8, DT = DPAD / 32;
+    constexpr int QUADS = DPAD / 4;              // float4 per row
+    constexpr int PER_LANE = ROWS * QUADS / 64;  // ROWS × QUADS float4 over 64 lanes
+    constexpr int BATCH = PER_LANE < 8 ? PER_LANE : 8;
+    extern __shared__ __attribute__((aligned(16))) float attn_lds[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) >> 6);
+    const int li = lane & 31, lh = lane >> 5;
+    const int S = p.S, D = p.D;
+    const int ctx = static_cast<int>(blockIdx.x) * WAVES + wave;
+    if (ctx >= p.contexts) return;  // (no workgroup barrier anywhere below)
+    float *ks = attn_lds + wave * (K_ELEMS + V_ELEMS);
+    float *vs = ks + K_ELEMS;
+    const size_t ctx_elem0 = static_cast<size_t>(ctx) * S * D;
+    const float *q = p.q + ctx_elem0, *k = p.k + ctx_elem0, *v = p.v + ctx_elem0;
+
+    // Stage K and V: float4 number f = lane + 64·r of the ROWS × DPAD tile, BATCH of them requested before the first store.
+#pragma unroll
+    for (int r0 = 0; r0 < PER_LANE; r0 += BATCH) {
+        float4 rk[BATCH], rv[BATCH];
+#pragma unroll
+        for (int r = 0; r < BATCH; ++r) {
+            const int f = lane + 64 * (r0 + r);
+            const int row = f / QUADS, c4 = (f % QUADS) * 4;
+            const bool inside = row < S && c4 < D;
+            rk[r] = inside ? *reinterpret_cast<const float4 *>(k + static_cast<size_t>(row) * D + c4) : make_float4(0.f, 0.f, 0.f, 0.f);
+            rv[r] = inside ? *reinterpret_cast<const float4 *>(v + static_cast<size_t>(row) * D + c4) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+        for (int r = 0; r < BATCH; ++r) {
+            const int f = lane + 64 * (r0 + r);
+            const int row = f / QUADS, c4 = (f % QUADS) * 4;
+            *reinterpret_cast<float4 *>(&ks[row * KS + c4]) = rk[r];
+            *reinterpret_cast<float4 *>(&vs[row * VS + c4]) = rv[r];
+        }
+    }
+    // The wavefront's own LDS writes are visible to its later reads (LDS operations of a wavefront execute in order);
+    // the fence keeps the compiler from moving the reads up.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+    const float scale_log2e = p.scale * kLog2e;  // logits in log2 units: dot · scale · log2(e), either sign
+    for (int q0 = 0; q0 < S; q0 += 32) {
+        const int my_q = q0 + li;
+        float qf[CHUNKS][4];
+#pragma unroll
+        for (int c = 0; c < CHUNKS; ++c) {
+            const int d = c * 8 + lh * 4;
+            const float4 t = (my_q < S && d < D) ? *reinterpret_cast<const float4 *>(q + static_cast<size_t>(my_q) * D + d)
+                                                 : make_float4(0.f, 0.f, 0.f, 0.f);
+            qf[c][0] = t.x; qf[c][1] = t.y; qf[c][2] = t.z; qf[c][3] = t.w;
+        }
+        const int key_limit = CAUSAL ? min(S, q0 + 32) : S;  // keys this chunk of queries can see
+        auto compute = [&](auto nt_tag) {
+            constexpr int NT = decltype(nt_tag)::value;
+            f32x16 sacc[NT];
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+                sacc[t] = f32x16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < CHUNKS; ++c) {
+                float4 kv[NT];
+#pragma unroll
+                for (int t = 0; t < NT; ++t) kv[t] = *reinterpret_cast<const float4 *>(&ks[(t * 32 + li) * KS + c * 8 + lh * 4]);
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    sacc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(kv[t].x, qf[c][0], sacc[t], 0, 0, 0);
+                    sacc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(kv[t].y, qf[c][1], sacc[t], 0, 0, 0);
+                    sacc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(kv[t].z, qf[c][2], sacc[t], 0, 0, 0);
+                    sacc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(kv[t].w, qf[c][3], sacc[t], 0, 0, 0);
+                }
+            }
+            // register r of lane half h is key 32t + (r/4)·8 + 4h + r%4 for this lane's query
+            float top = -INFINITY;
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int key = t * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
+                    float logit = sacc[t][r] * scale_log2e;
+                    if (key >= S || (CAUSAL && key > my_q)) logit = -INFINITY;
+                    sacc[t][r] = logit;
+                    top = fmaxf(top, logit);
+                }
+            top = fmaxf(top, __shfl_xor(top, 32));  // key 0 is visible to every query: finite
+            float sum = 0.0f;
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float pr = __builtin_amdgcn_exp2f(sacc[t][r] - top);
+                    sacc[t][r] = pr;
+                    sum += pr;
+                }
+            sum += __shfl_xor(sum, 32);
+            f32x16 oacc[DT];
+#pragma unroll
+            for (int t = 0; t < DT; ++t)
+                oacc[t] = f32x16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            const float *v_lane = vs + (lh * 4) * VS + li;
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    float vv[DT][4];
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) vv[dt][e] = v_lane[(t * 32 + g * 8 + e) * VS + dt * 32];
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv[dt][e], sacc[t][g * 4 + e], oacc[dt], 0, 0, 0);
+                }
+            const float inv = 1.0f / sum;
+            if (my_q < S) {
+                float *orow = p.out + ctx_elem0 + static_cast<size_t>(my_q) * D;
+#pragma unroll
+                for (int t = 0; t < DT; ++t)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const int d = t * 32 + g * 8 + lh * 4;
+                        if (d < D)
+                            *reinterpret_cast<float4 *>(orow + d) = make_float4(oacc[t][g * 4 + 0] * inv, oacc[t][g * 4 + 1] * inv,
+                                                                                oacc[t][g * 4 + 2] * inv, oacc[t][g * 4 + 3] * inv);
+                    }
+            }
+        };
+        if constexpr (ROWS > 32) {
+            if (key_limit > 32) compute(std::integral_constant<int, 2>{});
+            else compute(std::integral_constant<int, 1>{});
+        } else {
+            compute(std::integral_constant<int, 1>{});
+        }
+    }
+}
+
+template <int DPAD, bool CAUSAL, int ROWS>
+hipError_t launch_tiny_rows(const AttnArgs &args, hipStream_t stream)
+{
+    constexpr size_t wave_bytes = static_cast<size_t>(ROWS) * ((DPAD + 4) + (DPAD + 8)) * sizeof(float);
+    constexpr int WAVES = wave_bytes * 4 <= 160 * 1024 ? 4 : 2;
+    constexpr size_t lds_bytes = wave_bytes * WAVES;
+    static_assert(lds_bytes <= 160 * 1024, "the wavefronts' K and V slices fit the LDS");
+    if (args.S > ROWS) return hipErrorInvalidValue;
+    auto kernel = attention_f32_tiny_kernel<DPAD, CAUSAL, ROWS, WAVES>;
+    hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        static_cast<int>(lds_bytes));
+    if (rc != hipSuccess) return rc;
+    const unsigned blocks = static_cast<unsigned>((args.contexts + WAVES - 1) / WAVES);
+    hipLaunchKernelGGL(kernel, dim3(blocks), dim3(64 * WAVES), lds_bytes, stream, args);
+    return hipGetLastError();
+}
+
+template <int DPAD, bool CAUSAL>
+hipError_t launch_tiny(const AttnArgs &args, hipStream_t stream)
+{
+    return args.S <= 32 ? launch_tiny_rows<DPAD, CAUSAL, 32>(args, stream) : launch_tiny_rows<DPAD, CAUSAL, 64>(args, stream);
+}
+
 // Combines the key splits of the fast kernel: with m = max over splits of their reference maxima,
 // out = Σ_s 2^((m_s − m)·exp_scale)·O_s / Σ_s 2^((m_s − m)·exp_scale)·l_s, splits added in order.  One thread per four
 // output values.
@@ -784,6 +960,12 @@ hipError_t launch_attention_f32(size_t contexts, size_t sequence, size_t head_di
     const bool vec = (head_dim % 4 == 0) && aligned(q) && aligned(k) && aligned(v) && aligned(out);
     // The fast kernel addresses one context through a 32-bit buffer range.
     const bool fits_buffer = sequence * head_dim * sizeof(float) < (1ull << 31);
+    // Many contexts of at most 64 positions: a wavefront per context.
+    if (!bias && vec && fits_buffer && head_dim <= 128 && sequence <= 64 && contexts >= 256) {
+        if (head_dim <= 32) return causal ? launch_tiny<32, true>(args, stream) : launch_tiny<32, false>(args, stream);
+        if (head_dim <= 64) return causal ? launch_tiny<64, true>(args, stream) : launch_tiny<64, false>(args, stream);
+        return causal ? launch_tiny<128, true>(args, stream) : launch_tiny<128, false>(args, stream);
+    }
     if (!bias && vec && fits_buffer && head_dim <= 128) {
         if (head_dim <= 32) return causal ? launch_fast<32, true>(args, stream) : launch_fast<32, false>(args, stream);
         if (head_dim <= 64) return causal ? launch_fast<64, true>(args, stream) : launch_fast<64, false>(args, stream);

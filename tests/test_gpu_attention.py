@@ -51,6 +51,39 @@ def test_random_cases(hip, oracle, contexts, seq, dim, causal, biased):
     assert_close(ones, np.ones_like(ones), F32_REL, F32_ABS, "row sums")
 
 
+@pytest.mark.parametrize("contexts,seq,dim,causal,scale", [
+    (256, 16, 64, False, 0.125), (257, 16, 64, True, 0.125), (300, 49, 32, False, 0.1768), (301, 49, 32, True, 0.1768),
+    (1000, 1, 64, False, 0.125), (513, 31, 128, True, 0.0884), (258, 32, 128, False, 0.0884), (259, 33, 128, True, 0.0884),
+    (400, 64, 64, False, 0.125), (402, 64, 64, True, 0.125), (262, 64, 128, False, -0.2), (300, 7, 8, True, 0.35),
+    (260, 50, 40, False, 0.158), (261, 20, 100, True, 0.1), (333, 64, 32, True, 3.0), (270, 48, 64, False, 0.0),
+    (2048, 16, 32, False, 0.1768)])
+def test_many_short_contexts(hip, oracle, contexts, seq, dim, causal, scale):
+    """Windowed attention: at least 256 contexts of at most 64 positions each are handled a wavefront per context.
+    Context counts that do not fill the last workgroup, lengths either side of the 32-key tile, head sizes that are
+    padded to the next kernel (8, 40, 100), a peaked softmax (scale 3), a flat one (scale 0) and a negative scale;
+    output positions past each context's end stay untouched (the buffer's tail keeps its fill)."""
+    rng = np.random.default_rng(contexts * 131 + seq * 7 + dim)
+    n = contexts * seq * dim
+    q, k, v = (rng.normal(size=n).astype(np.float32) for _ in range(3))
+    d_q, d_k, d_v = (hip.DeviceBuffer.from_array(a) for a in (q, k, v))
+    tail = 4096
+    d_out = hip.DeviceBuffer.from_array(np.full(n + tail, 7.5, np.float32))
+    hip.attention_f32_dev(contexts, seq, dim, scale, causal, d_q, d_k, d_v, None, None, d_out)
+    hip.device_synchronize()
+    both = d_out.to_array(np.float32, n + tail)
+    got = both[:n]
+    assert (both[n:] == 7.5).all(), "wrote past the last context"
+    want = oracle.attention_f32(contexts, seq, dim, scale, q, k, v, None, None, causal, threads=8)
+    assert_close(got, want, F32_REL, F32_ABS, f"short contexts {contexts}x{seq}x{dim} causal={causal}")
+    d_ones = hip.DeviceBuffer.from_array(np.ones(n, np.float32))
+    hip.attention_f32_dev(contexts, seq, dim, scale, causal, d_q, d_k, d_ones, None, None, d_out)
+    hip.device_synchronize()
+    ones = d_out.to_array(np.float32, n)
+    assert_close(ones, np.ones_like(ones), F32_REL, F32_ABS, "row sums")
+    if causal:  # position 0 attends to itself only
+        assert_close(got.reshape(contexts, seq, dim)[:, 0], v.reshape(contexts, seq, dim)[:, 0], F32_REL, F32_ABS, "first row")
+
+
 @pytest.mark.parametrize("contexts,seq,dim,biased,scale", [
     (1, 2048, 64, True, 0.125), (1, 2048, 64, False, 0.125), (3, 1000, 32, True, 0.2), (2, 300, 128, False, -0.4),
     (1, 512, 64, False, 3.0), (5, 260, 64, True, 0.0), (1, 4096, 16, False, 0.25), (7, 384, 64, False, 0.125)])
