@@ -858,6 +858,7 @@ hipError_t launch_gemm_f32(size_t m, size_t n, size_t k, bool lhs_transposed, co
 {
     if (m == 0 || n == 0) return hipSuccess;
     if (!lhs_transposed && gemv_f32_applies(m, n, k, lhs, rhs)) return launch_gemv_f32(m, n, k, lhs, rhs, out, epilogue, stream);
+    if (lhs_transposed && scratch_free && gemv_t_f32_applies(m, n, k)) return launch_gemv_t_f32(m, n, k, lhs, rhs, out, epilogue, stream);
     // An A of 2 GiB or more (the direct-to-LDS kernels address their operands through 32-bit byte offsets): row blocks
     // of A are independent products, so the launch is cut into blocks that fit and each takes the fast path.
     if (!lhs_transposed && m * k * sizeof(float) >= (1ull << 31) && k > 0 && k * 256 * sizeof(float) < (1ull << 31)) {

@@ -1,4 +1,5 @@
-// Matrix times a few columns: C(m×n) = epilogue(A·B) with n <= 3 (f32) or n <= 7 (bf16, f32 accumulate).
+// Matrix times a few columns: C(m×n) = epilogue(A·B) with n <= 3 (f32) or n <= 7 (bf16, f32 accumulate), and
+// Aᵀ·B for an f32 A stored k×m with n <= 4 (further down).
 //
 // The same entry points as the tiled GEMMs serve these shapes (hip_sgemm, crates/st-backend-hip/src/real.rs:598-646,
 // and the bf16 GEMM beside it); a tile kernel would spend its loads on 64-byte row segments of A and its matrix
@@ -8,6 +9,7 @@
 // read through the caches by every row.  The order of the additions is fixed by the shape alone.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstdint>
 
 #include "device_math.h"
@@ -226,6 +228,120 @@ GemvArgs make_args(size_t m, size_t n, size_t k, const void *lhs, const void *rh
     return args;
 }
 
+// -------------------------------------------------------------------------------------------------
+// Aᵀ·B with A stored k×m (the gradient of a matrix-vector product with respect to the vector): the rows of the stored
+// matrix run along the OUTPUT, so a lane owns four adjacent outputs and walks down the k rows of its slice, a wavefront
+// reading 1 KB of one stored row per load.  The four wavefronts of a workgroup take eight rows each of every 32, the
+// grid's second dimension cuts k into slices, and every (slice, output) sum goes to scratch memory: the reduction
+// kernel adds the slices in order and applies the epilogue.  Rows need no alignment (16-byte loads take any address
+// here); the last lanes of a row whose four outputs straddle its end load one value at a time.
+// -------------------------------------------------------------------------------------------------
+typedef float gemv_f32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+
+struct GemvTArgs {
+    const float *A;   // k × m
+    const float *B;   // k × n
+    float *partial;   // slices × m × n
+    int M, K;
+    int rows_per_slice;  // a multiple of 32
+};
+
+template <int NC>
+__global__ __launch_bounds__(256) void gemv_t_f32_kernel(GemvTArgs p)
+{
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) >> 6);
+    const int M = p.M;
+    const int col = static_cast<int>(blockIdx.x) * 256 + lane * 4;
+    const int valid = min(4, M - col);  // <= 0: nothing of this lane's quad exists
+    const int k_begin = static_cast<int>(blockIdx.y) * p.rows_per_slice;
+    const int k_end = min(p.K, k_begin + p.rows_per_slice);
+    float acc[NC][4];
+#pragma unroll
+    for (int c = 0; c < NC; ++c)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[c][e] = 0.0f;
+    for (int k0 = k_begin + wave * 8; k0 < k_end; k0 += 32) {
+        float a[8][4];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int row = k0 + j;
+            const float *src = p.A + static_cast<size_t>(row) * M + col;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) a[j][e] = 0.0f;
+            if (row < k_end) {
+                if (valid == 4) {
+                    const gemv_f32x4_a4 t = *reinterpret_cast<const gemv_f32x4_a4 *>(src);
+                    a[j][0] = t[0]; a[j][1] = t[1]; a[j][2] = t[2]; a[j][3] = t[3];
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 3; ++e)
+                        if (e < valid) a[j][e] = src[e];
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int row = k0 + j;  // the same for the whole wavefront: B comes through the scalar cache
+            if (row < k_end) {
+#pragma unroll
+                for (int c = 0; c < NC; ++c) {
+                    const float b = p.B[static_cast<size_t>(row) * NC + c];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[c][e] = fmaf(a[j][e], b, acc[c][e]);
+                }
+            }
+        }
+    }
+    __shared__ float part[4][NC][256];
+#pragma unroll
+    for (int c = 0; c < NC; ++c)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) part[wave][c][lane * 4 + e] = acc[c][e];
+    __syncthreads();
+    const int out_col = static_cast<int>(blockIdx.x) * 256 + static_cast<int>(threadIdx.x);
+    if (out_col >= M) return;
+    float *dst = p.partial + (static_cast<size_t>(blockIdx.y) * M + out_col) * NC;
+#pragma unroll
+    for (int c = 0; c < NC; ++c)
+        dst[c] = (part[0][c][threadIdx.x] + part[1][c][threadIdx.x]) + (part[2][c][threadIdx.x] + part[3][c][threadIdx.x]);
+}
+
+struct GemvTReduceArgs {
+    const float *partial;
+    float *C;
+    const float *bias;
+    const float *residual;
+    size_t plane;  // m · n
+    int N, slices;
+    float scale;
+    int activation;
+};
+
+__global__ __launch_bounds__(256) void gemv_t_reduce_kernel(GemvTReduceArgs p)
+{
+    const size_t idx = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (idx >= p.plane) return;
+    float value = 0.0f;
+    for (int s0 = 0; s0 < p.slices; s0 += 8) {
+        float piece[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) piece[j] = (s0 + j < p.slices) ? p.partial[(s0 + j) * p.plane + idx] : 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) value += piece[j];
+    }
+    value = value * p.scale + (p.bias ? p.bias[idx % p.N] : -0.0f);
+    if (p.residual) value += p.residual[idx];
+    p.C[idx] = apply_activation(value, p.activation);
+}
+
+template <int NC>
+hipError_t launch_t_f32(const GemvTArgs &args, unsigned col_blocks, unsigned slices, hipStream_t stream)
+{
+    hipLaunchKernelGGL(gemv_t_f32_kernel<NC>, dim3(col_blocks, slices), dim3(256), 0, stream, args);
+    return hipGetLastError();
+}
+
 }  // namespace
 
 bool gemv_f32_applies(size_t m, size_t n, size_t k, const float *lhs, const float *rhs)
@@ -265,6 +381,53 @@ hipError_t launch_gemv_bf16(size_t m, size_t n, size_t k, const uint16_t *lhs, c
     case 6: return launch_bf16<6>(args, rhs_packed, stream);
     default: return launch_bf16<7>(args, rhs_packed, stream);
     }
+}
+
+bool gemv_t_f32_applies(size_t m, size_t n, size_t k)
+{
+    return n >= 1 && n <= 4 && m >= 1024 && k >= 64 && m < (1ull << 31) && k < (1ull << 31);
+}
+
+hipError_t launch_gemv_t_f32(size_t m, size_t n, size_t k, const float *lhs, const float *rhs, float *out,
+                             const GemmEpilogue &epilogue, hipStream_t stream)
+{
+    const size_t col_blocks = (m + 255) / 256;
+    // About 2048 workgroups (eight per compute unit), slices of at least 64 rows.
+    size_t slices = std::max<size_t>(1, std::min((2048 + col_blocks - 1) / col_blocks, k / 64));
+    slices = std::min<size_t>(slices, 65535);
+    const size_t rows_per_slice = ((k + slices - 1) / slices + 31) / 32 * 32;
+    slices = (k + rows_per_slice - 1) / rows_per_slice;
+    const size_t plane = m * n;
+    void *workspace = nullptr;
+    hipError_t rc = stream_workspace(stream, slices * plane * sizeof(float), &workspace);
+    if (rc != hipSuccess) return rc;
+    GemvTArgs args;
+    args.A = lhs;
+    args.B = rhs;
+    args.partial = static_cast<float *>(workspace);
+    args.M = static_cast<int>(m);
+    args.K = static_cast<int>(k);
+    args.rows_per_slice = static_cast<int>(rows_per_slice);
+    const unsigned blocks = static_cast<unsigned>(col_blocks), cuts = static_cast<unsigned>(slices);
+    switch (n) {
+    case 1: rc = launch_t_f32<1>(args, blocks, cuts, stream); break;
+    case 2: rc = launch_t_f32<2>(args, blocks, cuts, stream); break;
+    case 3: rc = launch_t_f32<3>(args, blocks, cuts, stream); break;
+    default: rc = launch_t_f32<4>(args, blocks, cuts, stream); break;
+    }
+    if (rc != hipSuccess) return rc;
+    GemvTReduceArgs reduce;
+    reduce.partial = args.partial;
+    reduce.C = out;
+    reduce.bias = epilogue.bias;
+    reduce.residual = epilogue.residual;
+    reduce.plane = plane;
+    reduce.N = static_cast<int>(n);
+    reduce.slices = static_cast<int>(slices);
+    reduce.scale = epilogue.scale;
+    reduce.activation = epilogue.activation;
+    hipLaunchKernelGGL(gemv_t_reduce_kernel, dim3(static_cast<unsigned>((plane + 255) / 256)), dim3(256), 0, stream, reduce);
+    return hipGetLastError();
 }
 
 }  // namespace sthip

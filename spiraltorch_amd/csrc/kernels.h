@@ -26,6 +26,10 @@ hipError_t launch_gemm_f32(size_t m, size_t n, size_t k, bool lhs_transposed, co
 bool gemv_f32_applies(size_t m, size_t n, size_t k, const float *lhs, const float *rhs);
 hipError_t launch_gemv_f32(size_t m, size_t n, size_t k, const float *lhs, const float *rhs, float *out,
                            const GemmEpilogue &epilogue, hipStream_t stream);
+// A stored k×m (lhs_transposed): uses the stream's scratch memory.
+bool gemv_t_f32_applies(size_t m, size_t n, size_t k);
+hipError_t launch_gemv_t_f32(size_t m, size_t n, size_t k, const float *lhs, const float *rhs, float *out,
+                             const GemmEpilogue &epilogue, hipStream_t stream);
 bool gemv_bf16_applies(size_t m, size_t n, size_t k, const uint16_t *lhs, const uint16_t *rhs);
 hipError_t launch_gemv_bf16(size_t m, size_t n, size_t k, const uint16_t *lhs, const uint16_t *rhs, bool rhs_packed,
                             float *out_f32, uint16_t *out_bf16, const GemmEpilogue &epilogue, hipStream_t stream);

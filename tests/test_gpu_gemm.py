@@ -143,6 +143,10 @@ def test_long_reduction_against_float64(hip):
     (130, 70, 5000, True),
     (256, 192, 8192, True),    # the direct-to-LDS ring kernel, A transposed (a weight gradient Xᵀ·dY), k-sliced
     (100, 260, 4096, True),
+    (10027, 1, 9472, True),    # Aᵀ·x with A stored k×m: lanes own outputs, k cut into slices; rows of odd length
+    (4096, 4, 4100, True),     # four columns; the last 32-row group of a slice is short
+    (1025, 2, 64, True),       # one slice; the last lanes' quad straddles the end of the rows
+    (2048, 3, 300, True),
 ])
 def test_k_sliced_launches_against_float64(hip, m, n, k, lhs_t):
     """Few output tiles and a long k: the launch is cut along k over workgroups, the partial planes are added in slice
@@ -161,6 +165,9 @@ def test_k_sliced_launches_against_float64(hip, m, n, k, lhs_t):
         hip.gemm_lhs_transpose_scaled_f32(m, n, k, 0.25, a, b, out)
         want = 0.25 * exact
         assert (np.abs(out.reshape(m, n) - want) <= 1e-4 * np.abs(want) + 1e-5 + slack).all()
+        twice = np.zeros(m * n, np.float32)
+        hip.gemm_lhs_transpose_scaled_f32(m, n, k, 0.25, a, b, twice)
+        assert (twice == out).all(), "the slices are added in a fixed order"
         return
     hip.gemm_scaled_f32(m, n, k, -0.5, a, b, out)
     want = -0.5 * exact
