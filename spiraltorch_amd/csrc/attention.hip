@@ -555,7 +555,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DPAD <= 64 
         if (more) load_global(key_first + (t + 1) * BKV);
         const int key0 = key_first + t * BKV;
         // Tiles entirely past the sequence end or (causal) entirely above this wavefront's rows are skipped.
-        const int limit = CAUSAL ? min(S, wq0 + 32) : S;
+        // So is everything in a wavefront whose 32 query rows lie past the sequence end (the last tile of 197 rows).
+        const int limit = wq0 >= S ? 0 : CAUSAL ? min(S, wq0 + 32) : S;
         if (key0 + 32 < limit) compute(std::integral_constant<int, 2>{}, t & 1, key0);
         else if (key0 < limit) compute(std::integral_constant<int, 1>{}, t & 1, key0);
         if (more) store_lds((t + 1) & 1);
