@@ -310,8 +310,8 @@ def wl_rowops(hip, inputs, timer, warmup, steps):
 def wl_lopsided(hip, inputs, timer, warmup, steps):
     """Shapes outside the BASELINE configs whose dispatch has kernels of its own: matrix x vector (a stream over A: the
     f32 matrix is 1 GiB, the bf16 one 512 MiB, both beyond the 256 MiB memory-side cache), a product of few output tiles
-    with a long k (k-sliced over workgroups), and softmax over rows of 100000 values (a workgroup per row).  All
-    HBM-bound; bytes are the algorithmic reads + writes."""
+    with a long k (k-sliced over workgroups), softmax over rows of 100000 values (a workgroup per row), and thousands
+    of short attention windows.  All HBM-bound; bytes are the algorithmic reads + writes."""
     out = []
     m = k = 16384
     d_a = hip.DeviceBuffer(m * k * 4)
@@ -323,6 +323,9 @@ def wl_lopsided(hip, inputs, timer, warmup, steps):
     d_x16 = hip.DeviceBuffer.from_array(inputs.to_bf16(inputs.uniform(inputs.seed_for(1, 2), k, -1.0, 1.0)))
     wall, ev = timer.run(lambda st: hip.gemm_bf16_f32acc_dev(m, 1, k, d_a, d_x16, d_y, st), warmup, steps)
     out.append(entry(f"gemv_bf16_{m}x1x{k}", "bf16", 2 * m * k, 2 * (m * k + k) + 4 * m, "hbm", wall, ev))
+    # the same stored matrix read as k x m: A^T x, the gradient of the product above with respect to x
+    wall, ev = timer.run(lambda st: hip.gemm_f32_dev(m, 1, k, 1.0, True, d_a, d_x, d_y, st), warmup, steps)
+    out.append(entry(f"gemv_f32_lhs_transposed_{m}x1x{k}", "f32", 2 * m * k, 4 * (m * k + k + m), "hbm", wall, ev))
     m2, n2, k2 = 64, 64, 100000
     d_c = hip.DeviceBuffer(m2 * n2 * 4)
     wall, ev = timer.run(lambda st: hip.gemm_f32_dev(m2, n2, k2, 1.0, False, d_a, d_a, d_c, st), warmup, steps)
@@ -332,6 +335,14 @@ def wl_lopsided(hip, inputs, timer, warmup, steps):
     d_out = hip.DeviceBuffer(rows * cols * 4)
     wall, ev = timer.run(lambda st: hip.row_softmax_f32_dev(rows, cols, d_in, d_out, st), warmup, steps)
     out.append(entry(f"row_softmax_f32_{rows}x{cols}", "f32", 0, 8 * rows * cols, "hbm", wall, ev))
+    # windowed attention: 16384 contexts of 16 positions, head size 64 (a wavefront per context)
+    ctx, seq, dim = 16384, 16, 64
+    n = ctx * seq * dim
+    d_q, d_o = hip.DeviceBuffer(n * 4), hip.DeviceBuffer(n * 4)
+    d_q.zero()
+    wall, ev = timer.run(lambda st: hip.attention_f32_dev(ctx, seq, dim, 0.125, False, d_q, d_q, d_q, None, None, d_o, st),
+                         warmup, steps)
+    out.append(entry(f"attention_f32_{ctx}_windows_of_{seq}x{dim}", "f32", 4 * ctx * seq * seq * dim, 16 * n, "hbm", wall, ev))
     return out
 
 
