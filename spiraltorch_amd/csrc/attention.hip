@@ -608,11 +608,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DPAD <= 64 
 // transposed products as above: Sᵀ = K·Qᵀ leaves every lane the scores of its own query, which are the B operand of
 // Oᵀ = Vᵀ·Pᵀ as they stand.  WAVES wavefronts (contexts) per workgroup: as many as fit the LDS.
 // -------------------------------------------------------------------------------------------------
-template <int DPAD, bool CAUSAL, int ROWS, int WAVES>
+template <int DPAD, bool CAUSAL, int ROWS, int WAVES, bool KDIRECT>
 __global__ __launch_bounds__(64 * WAVES) void attention_f32_tiny_kernel(AttnArgs p)
 {
     constexpr int KS = DPAD + 4, VS = DPAD + 8;  // row strides as in the fast kernel (conflict-free fragment reads)
-    constexpr int K_ELEMS = ROWS * KS, V_ELEMS = ROWS * VS;  // ROWS: 32 or 64 staged positions, at least S
+    // ROWS: 32 or 64 staged positions, at least S.  KDIRECT: the K fragments come straight from global memory into
+    // registers, as Q's do (a lane's fragment is 16 contiguous bytes of one row), and only V is staged: half the LDS,
+    // twice the wavefronts per SIMD to overlap one context's loads with another's products.
+    constexpr int K_ELEMS = KDIRECT ? 0 : ROWS * KS, V_ELEMS = ROWS * VS;
+    constexpr int NTMAX = ROWS / 32;
     constexpr int CHUNKS = DPAD / 8, DT = DPAD / 32;
     constexpr int QUADS = DPAD / 4;              // float4 per row
     constexpr int PER_LANE = ROWS * QUADS / 64;  // ROWS × QUADS float4 over 64 lanes
@@ -629,6 +633,17 @@ __global__ __launch_bounds__(64 * WAVES) void attention_f32_tiny_kernel(AttnArgs
     const size_t ctx_elem0 = static_cast<size_t>(ctx) * S * D;
     const float *q = p.q + ctx_elem0, *k = p.k + ctx_elem0, *v = p.v + ctx_elem0;
 
+    float4 kreg[KDIRECT ? CHUNKS : 1][NTMAX];
+    if constexpr (KDIRECT) {
+#pragma unroll
+        for (int c = 0; c < CHUNKS; ++c)
+#pragma unroll
+            for (int t = 0; t < NTMAX; ++t) {
+                const int row = t * 32 + li, d = c * 8 + lh * 4;
+                kreg[c][t] = (row < S && d < D) ? *reinterpret_cast<const float4 *>(k + static_cast<size_t>(row) * D + d)
+                                                : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+    }
     // Stage K and V: float4 number f = lane + 64·r of the ROWS × DPAD tile, BATCH of them requested before the first store.
 #pragma unroll
     for (int r0 = 0; r0 < PER_LANE; r0 += BATCH) {
@@ -638,14 +653,14 @@ __global__ __launch_bounds__(64 * WAVES) void attention_f32_tiny_kernel(AttnArgs
             const int f = lane + 64 * (r0 + r);
             const int row = f / QUADS, c4 = (f % QUADS) * 4;
             const bool inside = row < S && c4 < D;
-            rk[r] = inside ? *reinterpret_cast<const float4 *>(k + static_cast<size_t>(row) * D + c4) : make_float4(0.f, 0.f, 0.f, 0.f);
+            rk[r] = (!KDIRECT && inside) ? *reinterpret_cast<const float4 *>(k + static_cast<size_t>(row) * D + c4) : make_float4(0.f, 0.f, 0.f, 0.f);
             rv[r] = inside ? *reinterpret_cast<const float4 *>(v + static_cast<size_t>(row) * D + c4) : make_float4(0.f, 0.f, 0.f, 0.f);
         }
 #pragma unroll
         for (int r = 0; r < BATCH; ++r) {
             const int f = lane + 64 * (r0 + r);
             const int row = f / QUADS, c4 = (f % QUADS) * 4;
-            *reinterpret_cast<float4 *>(&ks[row * KS + c4]) = rk[r];
+            if constexpr (!KDIRECT) *reinterpret_cast<float4 *>(&ks[row * KS + c4]) = rk[r];
             *reinterpret_cast<float4 *>(&vs[row * VS + c4]) = rv[r];
         }
     }
@@ -677,7 +692,10 @@ __global__ __launch_bounds__(64 * WAVES) void attention_f32_tiny_kernel(AttnArgs
             for (int c = 0; c < CHUNKS; ++c) {
                 float4 kv[NT];
 #pragma unroll
-                for (int t = 0; t < NT; ++t) kv[t] = *reinterpret_cast<const float4 *>(&ks[(t * 32 + li) * KS + c * 8 + lh * 4]);
+                for (int t = 0; t < NT; ++t) {
+                    if constexpr (KDIRECT) kv[t] = kreg[c][t];
+                    else kv[t] = *reinterpret_cast<const float4 *>(&ks[(t * 32 + li) * KS + c * 8 + lh * 4]);
+                }
 #pragma unroll
                 for (int t = 0; t < NT; ++t) {
                     sacc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(kv[t].x, qf[c][0], sacc[t], 0, 0, 0);
@@ -755,12 +773,15 @@ __global__ __launch_bounds__(64 * WAVES) void attention_f32_tiny_kernel(AttnArgs
 template <int DPAD, bool CAUSAL, int ROWS>
 hipError_t launch_tiny_rows(const AttnArgs &args, hipStream_t stream)
 {
-    constexpr size_t wave_bytes = static_cast<size_t>(ROWS) * ((DPAD + 4) + (DPAD + 8)) * sizeof(float);
+    // K in registers where the staged slices would leave one or two wavefronts per SIMD (64 positions: 49 × 32 94 → 88 µs,
+    // 64 × 64 38.6 → 35.6 µs); at 32 positions it gains nothing, at 128 values a head it would take 128 registers a lane.
+    constexpr bool KDIRECT = DPAD <= 64 && ROWS == 64;
+    constexpr size_t wave_bytes = static_cast<size_t>(ROWS) * ((KDIRECT ? 0 : DPAD + 4) + (DPAD + 8)) * sizeof(float);
     constexpr int WAVES = wave_bytes * 4 <= 160 * 1024 ? 4 : 2;
     constexpr size_t lds_bytes = wave_bytes * WAVES;
     static_assert(lds_bytes <= 160 * 1024, "the wavefronts' K and V slices fit the LDS");
     if (args.S > ROWS) return hipErrorInvalidValue;
-    auto kernel = attention_f32_tiny_kernel<DPAD, CAUSAL, ROWS, WAVES>;
+    auto kernel = attention_f32_tiny_kernel<DPAD, CAUSAL, ROWS, WAVES, KDIRECT>;
     hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                         static_cast<int>(lds_bytes));
     if (rc != hipSuccess) return rc;
