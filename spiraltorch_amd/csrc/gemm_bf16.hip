@@ -2286,6 +2286,55 @@ hipError_t launch_tile(GemmBf16Args args, bool vec, hipStream_t stream, size_t w
 
 bool aligned16(const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
 
+// Copies rows × cols matrices of 16-bit values into rows_pad × cols_pad ones, zeros in the new rows and columns: two
+// matrices (the operands of a product) in one launch, the first `first_blocks` workgroups on the first.  A thread
+// moves eight adjacent values of one output row (16-byte accesses at any alignment).
+struct PadJob {
+    const uint16_t *in;
+    uint16_t *out;
+    unsigned rows, cols, rows_pad, cols_pad;
+};
+
+__global__ __launch_bounds__(256) void pad_u16_pair_kernel(PadJob first, PadJob second, unsigned first_blocks)
+{
+    typedef uint32_t pad_u32x4_a2 __attribute__((ext_vector_type(4), aligned(2)));
+    const bool is_first = blockIdx.x < first_blocks;
+    const PadJob &job = is_first ? first : second;
+    const unsigned chunks = (job.cols_pad + 7) / 8;
+    const unsigned idx = (blockIdx.x - (is_first ? 0u : first_blocks)) * 256u + threadIdx.x;  // below 2^28: the copies are below 2 GiB
+    const unsigned r = idx / chunks;
+    const unsigned c0 = (idx - r * chunks) * 8;
+    if (r >= job.rows_pad) return;
+    uint16_t *dst = job.out + static_cast<size_t>(r) * job.cols_pad + c0;
+    const uint16_t *src = job.in + static_cast<size_t>(r) * job.cols + c0;
+    if (r < job.rows && c0 + 8 <= job.cols) {
+        *reinterpret_cast<pad_u32x4_a2 *>(dst) = *reinterpret_cast<const pad_u32x4_a2 *>(src);
+        return;
+    }
+#pragma unroll
+    for (unsigned e = 0; e < 8; ++e) {
+        const unsigned c = c0 + e;
+        if (c < job.cols_pad) dst[e] = (r < job.rows && c < job.cols) ? src[e] : static_cast<uint16_t>(0);
+    }
+}
+
+PadJob pad_job(size_t rows, size_t cols, size_t rows_pad, size_t cols_pad, const uint16_t *in, uint16_t *out)
+{
+    return PadJob{in, out, static_cast<unsigned>(rows), static_cast<unsigned>(cols), static_cast<unsigned>(rows_pad),
+                  static_cast<unsigned>(cols_pad)};
+}
+
+hipError_t launch_pad_u16_pair(const PadJob &first, const PadJob &second, hipStream_t stream)
+{
+    auto blocks = [](const PadJob &job) {
+        return static_cast<unsigned>((static_cast<size_t>(job.rows_pad) * ((job.cols_pad + 7) / 8) + 255) / 256);
+    };
+    const unsigned first_blocks = blocks(first), all = first_blocks + blocks(second);
+    if (all == 0) return hipSuccess;
+    hipLaunchKernelGGL(pad_u16_pair_kernel, dim3(all), dim3(256), 0, stream, first, second, first_blocks);
+    return hipGetLastError();
+}
+
 }  // namespace
 
 hipError_t launch_transpose_u16(size_t rows, size_t cols, const uint16_t *in, uint16_t *out, hipStream_t stream)
@@ -2318,6 +2367,24 @@ hipError_t launch_gemm_bf16(size_t m, size_t n, size_t k, const uint16_t *lhs, c
             if (rc != hipSuccess) return rc;
         }
         return hipSuccess;
+    }
+    // A k that is not a multiple of 64 (784 inputs, 1000 features): the direct-to-LDS kernels take whole 64-wide k-tiles
+    // only, and the general kernel runs such a product at half their speed (8192×4096×1000: 141 µs against 65 µs at
+    // k = 1024).  Where the product is large against its operands, zero-padded copies of A and B along k (exact: the
+    // new terms are 0·0) go into the stream's second scratch buffer, one launch for both, and the product runs on them.
+    if (k % 64 != 0 && k > 64 && m >= 128 && n >= 128 && 2.0 * m * n * k >= 2e9 && m * (k + 64) * sizeof(uint16_t) < (1ull << 31) &&
+        (k + 64) * n * sizeof(uint16_t) < (1ull << 31)) {
+        const size_t k_pad = (k + 63) / 64 * 64;
+        const size_t a_bytes = (m * k_pad * sizeof(uint16_t) + 255) & ~static_cast<size_t>(255);
+        void *copies = nullptr;
+        hipError_t rc = stream_workspace_slot(stream, 1, a_bytes + k_pad * n * sizeof(uint16_t), &copies);
+        if (rc != hipSuccess) return rc;
+        uint16_t *a_pad = static_cast<uint16_t *>(copies);
+        uint16_t *b_pad = reinterpret_cast<uint16_t *>(static_cast<unsigned char *>(copies) + a_bytes);
+        rc = launch_pad_u16_pair(pad_job(m, k, m, k_pad, lhs, a_pad),
+                                 rhs_packed ? pad_job(n, k, n, k_pad, rhs, b_pad) : pad_job(k, n, k_pad, n, rhs, b_pad), stream);
+        if (rc != hipSuccess) return rc;
+        return launch_gemm_bf16(m, n, k_pad, a_pad, b_pad, out_f32, out_bf16, epilogue, stream, rhs_packed);
     }
     GemmBf16Args args;
     args.A = lhs;

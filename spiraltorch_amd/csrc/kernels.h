@@ -138,6 +138,9 @@ hipError_t launch_sum_axis0_f32(size_t rows, size_t cols, const float *in, float
 // column-sum partials).  A thread's work on a stream is ordered, so two of its launches never use the buffer at the
 // same time, and threads that share a stream (the NULL stream) do not share scratch.
 hipError_t stream_workspace(hipStream_t stream, size_t bytes, void **out);
+// A second buffer of the same kind (slot 1) for re-laid copies of a call's operands, which must stay where they are
+// while the kernels that read them take scratch from slot 0.
+hipError_t stream_workspace_slot(hipStream_t stream, int slot, size_t bytes, void **out);
 void release_stream_workspace(hipStream_t stream);
 // Host<->device copies made by the library, for tests that check where tensors live.
 void count_transfer(bool to_device, size_t bytes);

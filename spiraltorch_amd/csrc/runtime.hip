@@ -105,17 +105,20 @@ struct WorkspaceEntry {
     std::thread::id owner;
     void *ptr;
     size_t capacity;
+    int slot;
 };
 std::mutex workspace_mutex;
 std::vector<WorkspaceEntry> workspace_entries;
 }  // namespace
 
-hipError_t stream_workspace(hipStream_t stream, size_t bytes, void **out)
+hipError_t stream_workspace(hipStream_t stream, size_t bytes, void **out) { return stream_workspace_slot(stream, 0, bytes, out); }
+
+hipError_t stream_workspace_slot(hipStream_t stream, int slot, size_t bytes, void **out)
 {
     const std::thread::id me = std::this_thread::get_id();
     std::lock_guard<std::mutex> lock(workspace_mutex);
     for (WorkspaceEntry &e : workspace_entries) {
-        if (e.stream != stream || e.owner != me) continue;
+        if (e.stream != stream || e.owner != me || e.slot != slot) continue;
         if (e.capacity < bytes || e.ptr == nullptr) {
             // Grow: earlier launches of this thread on this stream may still be using the old buffer.
             hipError_t rc = hipStreamSynchronize(stream);
@@ -137,7 +140,7 @@ hipError_t stream_workspace(hipStream_t stream, size_t bytes, void **out)
         *out = e.ptr;
         return hipSuccess;
     }
-    WorkspaceEntry fresh{stream, me, nullptr, bytes ? bytes : 256};
+    WorkspaceEntry fresh{stream, me, nullptr, bytes ? bytes : 256, slot};
     hipError_t rc = hipMalloc(&fresh.ptr, fresh.capacity);
     if (rc != hipSuccess) return rc;
     workspace_entries.push_back(fresh);

@@ -332,6 +332,44 @@ def test_few_tiles_with_a_long_k_split_k(hip, oracle, m, n, k):
         assert (d16.to_array(np.uint16, m * n) == inputs.to_bf16(got32)).all()
 
 
+@pytest.mark.parametrize("m,n,k", [(1024, 1024, 1000), (2048, 512, 1001), (4096, 1000, 300), (1000, 1024, 1100), (4096, 512, 784)])
+def test_k_that_is_not_a_multiple_of_64(hip, oracle, m, n, k):
+    """Large products whose k the direct-to-LDS kernels do not take run on zero-padded copies of both operands (kept in
+    a scratch buffer of their own while the product's kernels use the other): both layouts of B, odd row lengths, a
+    ragged n, the fused epilogue with both output types, and twice in a row with another product in between (which
+    re-uses and may grow the scratch buffers)."""
+    from spiraltorch_amd import inputs
+    rng = np.random.default_rng(m + 7 * n + 3 * k)
+    a, b = bf16_pair(rng, m, n, k, std=0.5)
+    bias = rng.normal(size=n).astype(np.float32)
+    res = rng.normal(size=m * n).astype(np.float32)
+    d = {name: hip.DeviceBuffer.from_array(v) for name, v in (("a", a), ("b", b), ("bias", bias), ("res", res))}
+    d_packed = hip.DeviceBuffer.from_array(np.ascontiguousarray(b.reshape(k, n).T))
+    out, other = hip.DeviceBuffer(m * n * 4), hip.DeviceBuffer(m * n * 4)
+    base = oracle.gemm_bf16_f32acc(m, n, k, a, b, threads=8)
+    hip.gemm_bf16_f32acc_dev(m, n, k, d["a"], d["b"], out)
+    hip.device_synchronize()
+    plain = out.to_array(np.float32, m * n)
+    check(plain, base, f"row-major {m}x{n}x{k}")
+    hip.gemm_bf16_prepacked_bias_act_dev(m, n, k, 0, d["a"], d_packed, None, None, other, None)
+    hip.gemm_bf16_f32acc_dev(m, n, k, d["a"], d["b"], out)
+    hip.device_synchronize()
+    check(other.to_array(np.float32, m * n), base, f"prepacked {m}x{n}x{k}")
+    assert (out.to_array(np.float32, m * n) == plain).all(), "same bits from call to call"
+    d16 = hip.DeviceBuffer(m * n * 2)
+    pre = (base.astype(np.float64).reshape(m, n) + bias).ravel() + res
+    want = np.maximum(pre, 0.0)
+    for packed in (False, True):
+        if packed:
+            hip.gemm_bf16_prepacked_bias_act_dev(m, n, k, 1, d["a"], d_packed, d["bias"], d["res"], out, d16)
+        else:
+            hip.gemm_bf16_bias_act_dev(m, n, k, 1, d["a"], d["b"], d["bias"], d["res"], out, d16)
+        hip.device_synchronize()
+        got32 = out.to_array(np.float32, m * n)
+        assert_close(got32, want, 1e-4, 2e-5 * max(1.0, float(np.abs(base).max())), f"epilogue packed={packed}")
+        assert (d16.to_array(np.uint16, m * n) == inputs.to_bf16(got32)).all()
+
+
 @pytest.mark.parametrize("m,n,k", [(1024, 1024, 1024), (300, 1024, 512), (130, 2048, 256), (1000, 1280, 192), (2048, 2048, 64),
                                    (513, 384, 448)])
 def test_mid_size_128_row_tiles(hip, oracle, m, n, k):
