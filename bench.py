@@ -310,7 +310,7 @@ def wl_rowops(hip, inputs, timer, warmup, steps):
 def wl_lopsided(hip, inputs, timer, warmup, steps):
     """Shapes outside the BASELINE configs whose dispatch has kernels of its own: matrix x vector (a stream over A: the
     f32 matrix is 1 GiB, the bf16 one 512 MiB, both beyond the 256 MiB memory-side cache), a product of few output tiles
-    with a long k (k-sliced over workgroups), softmax over rows of 100000 values (a workgroup per row), and thousands
+    with a long k (k-sliced over workgroups), softmax over rows of 100000 values (each row cut into segments over the grid), and thousands
     of short attention windows.  All HBM-bound; bytes are the algorithmic reads + writes."""
     out = []
     m = k = 16384

@@ -575,6 +575,123 @@ __global__ __launch_bounds__(THREADS) void row_softmax_long_kernel(int cols, con
     }
 }
 
+// A few very long rows (a handful of sequences over a vocabulary): a workgroup per row would leave most of the chip
+// idle, so the grid's x cuts every row into segments.  First launch: each segment's maximum (first position, NaN
+// skipped) and the sum of its weights relative to that maximum; second launch: every workgroup combines its row's
+// segment results — in segment order, so the same bits every time — and writes its own segment.  Same edge rules
+// as the single-workgroup kernels (the base is the maximum when that is finite, else 0; a row whose sum is not a
+// normal number becomes one-hot at the first maximum).
+struct SoftmaxSegment {
+    float best;   // maximum of the segment's non-NaN values
+    int index;    // its first column, 0x7fffffff when the segment has none
+    float sum;    // sum of exp(v - base), base = best if finite else 0
+};
+
+// Four adjacent values of a row at any 4-byte alignment; past `end` they read as NaN, which every phase skips.
+__device__ __forceinline__ void load_quad_or_nan(const float *x, int c, int end, float (&v)[4])
+{
+    if (c + 4 <= end) {
+        const f32x4_a4 t = *reinterpret_cast<const f32x4_a4 *>(x + c);
+        v[0] = t[0]; v[1] = t[1]; v[2] = t[2]; v[3] = t[3];
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = (c + e < end) ? x[c + e] : __builtin_nanf("");
+    }
+}
+
+__global__ __launch_bounds__(256) void row_softmax_split_partial_kernel(int cols, int segment, const float *in, SoftmaxSegment *parts)
+{
+    __shared__ float scratch_f[4];
+    __shared__ int scratch_i[4];
+    const int tid = threadIdx.x;
+    const float *x = in + static_cast<size_t>(blockIdx.y) * cols;
+    const int c_begin = static_cast<int>(blockIdx.x) * segment, c_end = min(cols, c_begin + segment);
+    float best = -INFINITY;
+    int best_index = 0x7fffffff;
+#pragma unroll 4
+    for (int c = c_begin + tid * 4; c < c_end; c += 1024) {
+        float v[4];
+        load_quad_or_nan(x, c, c_end, v);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            if (v[e] != v[e]) continue;
+            if (best_index == 0x7fffffff || v[e] > best) {
+                best = v[e];
+                best_index = c + e;
+            }
+        }
+    }
+    const float seg_max = block_reduce<256>(best_index == 0x7fffffff ? -INFINITY : best, scratch_f,
+                                            [](float a, float b) { return fmaxf(a, b); });
+    const int candidate = block_reduce<256>((best_index != 0x7fffffff && best == seg_max) ? best_index : 0x7fffffff, scratch_i,
+                                            [](int a, int b) { return min(a, b); });
+    const bool found = candidate != 0x7fffffff;
+    const float base = (found && isfinite(seg_max)) ? seg_max : 0.0f;
+    float sum = 0.0f;
+#pragma unroll 4
+    for (int c = c_begin + tid * 4; c < c_end; c += 1024) {
+        float v[4];
+        load_quad_or_nan(x, c, c_end, v);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sum += (!found || v[e] != v[e]) ? 0.0f : __expf(v[e] - base);
+    }
+    sum = block_reduce<256>(sum, scratch_f, [](float a, float b) { return a + b; });
+    if (tid == 0) parts[static_cast<size_t>(blockIdx.y) * gridDim.x + blockIdx.x] = SoftmaxSegment{seg_max, candidate, sum};
+}
+
+__global__ __launch_bounds__(256) void row_softmax_split_write_kernel(int cols, int segment, const float *in,
+                                                                      const SoftmaxSegment *parts, float *out)
+{
+    const int tid = threadIdx.x;
+    const float *x = in + static_cast<size_t>(blockIdx.y) * cols;
+    float *y = out + static_cast<size_t>(blockIdx.y) * cols;
+    const int c_begin = static_cast<int>(blockIdx.x) * segment, c_end = min(cols, c_begin + segment);
+    const SoftmaxSegment *row_parts = parts + static_cast<size_t>(blockIdx.y) * gridDim.x;
+    // The (at most 64) segment results go through LDS, one load each; every thread then combines them itself, in order.
+    __shared__ SoftmaxSegment staged[64];
+    if (tid < static_cast<int>(gridDim.x)) staged[tid] = row_parts[tid];
+    __syncthreads();
+    float row_max = -INFINITY;
+    int candidate = 0x7fffffff;
+    for (unsigned s = 0; s < gridDim.x; ++s) {
+        const SoftmaxSegment part = staged[s];
+        if (part.index == 0x7fffffff) continue;
+        if (candidate == 0x7fffffff || part.best > row_max) {  // segments ascend: the first occurrence wins
+            row_max = part.best;
+            candidate = part.index;
+        }
+    }
+    const bool found = candidate != 0x7fffffff;
+    const float base = (found && isfinite(row_max)) ? row_max : 0.0f;
+    float denom = 0.0f;
+    for (unsigned s = 0; s < gridDim.x; ++s) {
+        const SoftmaxSegment part = staged[s];
+        if (part.index == 0x7fffffff || part.sum == 0.0f) continue;
+        const float part_base = isfinite(part.best) ? part.best : 0.0f;
+        denom += part.sum * __expf(part_base - base);
+    }
+    const bool normal = isfinite(denom) && denom > 1.1920929e-7f;
+    const float inv = normal ? 1.0f / denom : 0.0f;
+#pragma unroll 4
+    for (int c = c_begin + tid * 4; c < c_end; c += 1024) {
+        float v[4], o[4];
+        load_quad_or_nan(x, c, c_end, v);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float weight = (!found || v[e] != v[e]) ? 0.0f : __expf(v[e] - base);
+            o[e] = weight * inv;
+            if (found && !normal) o[e] = (c + e == candidate) ? 1.0f : 0.0f;
+        }
+        if (c + 4 <= c_end) {
+            *reinterpret_cast<f32x4_a4 *>(y + c) = f32x4_a4{o[0], o[1], o[2], o[3]};
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (c + e < c_end) y[c + e] = o[e];
+        }
+    }
+}
+
 // The same for softmax: the row stays in the registers of a 1024-thread workgroup through all three phases.
 template <int CH>
 __global__ __launch_bounds__(1024) void row_softmax_block_kernel(int cols, const float *in, float *out)
@@ -1018,7 +1135,22 @@ hipError_t launch_row_softmax_f32(size_t rows, size_t cols, const float *in, flo
         hipLaunchKernelGGL(row_softmax_vec_kernel<4>, grid, block, 0, stream, r, c, in, out);
     else if (vec)
         hipLaunchKernelGGL(row_softmax_vec_kernel<8>, grid, block, 0, stream, r, c, in, out);
-    else if (cols > 4096 && cols <= 65536) {
+    else if (cols > 65536 && rows <= 128) {
+        // Few rows too long for a workgroup's registers: segments of at least 8192 values, up to about 1024 workgroups,
+        // at most 64 segments a row (4 × 1000000: 34 µs; 16 × 128256: 20 µs; 100 × 100000: 35 → 30 µs.  Up to 65536
+        // values the register kernel below is as fast or faster from a handful of rows on: 128 × 50257 19 against 23 µs).
+        size_t segments = std::min<size_t>(std::min<size_t>(64, cols / 8192), std::max<size_t>(2, 1024 / rows));
+        const size_t segment = ((cols + segments - 1) / segments + 3) / 4 * 4;
+        segments = (cols + segment - 1) / segment;
+        void *workspace = nullptr;
+        const hipError_t rc = stream_workspace(stream, rows * segments * sizeof(SoftmaxSegment), &workspace);
+        if (rc != hipSuccess) return rc;
+        SoftmaxSegment *parts = static_cast<SoftmaxSegment *>(workspace);
+        const dim3 split_grid(static_cast<unsigned>(segments), static_cast<unsigned>(rows));
+        const int seg = static_cast<int>(segment);
+        hipLaunchKernelGGL(row_softmax_split_partial_kernel, split_grid, dim3(256), 0, stream, c, seg, in, parts);
+        hipLaunchKernelGGL(row_softmax_split_write_kernel, split_grid, dim3(256), 0, stream, c, seg, in, parts, out);
+    } else if (cols > 4096 && cols <= 65536) {
         // The row in the registers of a 1024-thread workgroup: 2 to 16 pieces of 16 bytes per thread.
         const dim3 rows_grid(static_cast<unsigned>(rows));
         const size_t pieces = (cols + 4095) / 4096;

@@ -16,7 +16,9 @@ def on_device(hip, *arrays):
                                        # rows longer than 2048: a workgroup per row sweeping it (1024 threads; 256 from 2048 rows on)
                                        (3, 100000), (2, 50001), (2100, 2052), (2049, 2051),
                                        # 4097 to 65536 values: the row held in the registers of a 1024-thread workgroup
-                                       (5, 50257), (3, 65536), (4, 20003), (2, 8192), (300, 4098)])
+                                       (5, 50257), (3, 65536), (4, 20003), (2, 8192), (300, 4098), (130, 50257), (129, 65536),
+                                       # at most 128 rows of more than 65536 values: every row cut into segments over the grid
+                                       (1, 65540), (8, 128256), (100, 100000), (128, 65537), (2, 1000003), (129, 100000)])
 def test_row_softmax(hip, oracle, rows, cols):
     rng = np.random.default_rng(rows * 31 + cols)
     x = (rng.normal(size=rows * cols) * 3).astype(np.float32)
@@ -30,7 +32,8 @@ def test_row_softmax(hip, oracle, rows, cols):
         # The oracle adds a row's weights one after the other in f32, as the reference does; over 100000 of them that
         # sum is itself 1.5e-4 off (measured against float64 on this input).  The kernel adds per-thread partial sums
         # in a tree and is held to the exact value; the oracle only has to agree to what its own rounding allows.
-        assert_close(got, want, 1e-3, F32_ABS, f"row_softmax {rows}x{cols} against the sequential f32 sum")
+        # (that rounding grows with the length: 1e-3 up to 100000 values, 1e-2 at a million)
+        assert_close(got, want, max(1e-3, 1e-8 * cols), F32_ABS, f"row_softmax {rows}x{cols} against the sequential f32 sum")
         x64 = x.astype(np.float64).reshape(rows, cols)
         weights = np.exp(x64 - x64.max(axis=1, keepdims=True))
         want = (weights / weights.sum(axis=1, keepdims=True)).ravel()
@@ -52,25 +55,29 @@ def test_row_softmax_reference_input_and_edge_rows(hip, oracle, golden):
     assert got[12:16].tolist() == [0.0] * 4 and got[16:20].tolist() == [0.0, 1.0, 0.0, 0.0]
 
 
-@pytest.mark.parametrize("cols", [4100, 4101])
+@pytest.mark.parametrize("cols", [4100, 4101, 40001, 100000, 100003])
 def test_row_softmax_edge_rows_of_long_rows(hip, oracle, cols):
+    """(Above 65536 values these six rows are cut into segments over the grid: the second maximum of rows 2 and 4
+    lies in the last segment, and the first segments of row 5 hold nothing but NaN.)"""
     rng = np.random.default_rng(cols)
-    x = (rng.normal(size=5 * cols) * 3).astype(np.float32).reshape(5, cols)
+    x = (rng.normal(size=6 * cols) * 3).astype(np.float32).reshape(6, cols)
     x[0, ::7] = np.nan
     x[1, :] = np.nan
-    x[2, 3000] = x[2, 1777] = np.inf      # the first of the two becomes the one-hot
+    x[2, cols - 5] = x[2, 1777] = np.inf      # the first of the two becomes the one-hot
     x[3, :] = -1000.0
     x[4, :] = -np.inf
-    x[4, 2500] = x[4, 4000] = 5.0
+    x[4, 2500] = x[4, cols - 3] = 5.0
+    x[5, :cols // 2] = np.nan
     (d_in,) = on_device(hip, x)
     d_out = hip.DeviceBuffer(x.nbytes)
-    hip.row_softmax_f32_dev(5, cols, d_in, d_out)
+    hip.row_softmax_f32_dev(6, cols, d_in, d_out)
     hip.device_synchronize()
-    got = d_out.to_array(np.float32, 5 * cols).reshape(5, cols)
-    assert_close(got.ravel(), oracle.row_softmax_f32(5, cols, x.ravel()), F32_REL, F32_ABS, "edge rows")
+    got = d_out.to_array(np.float32, 6 * cols).reshape(6, cols)
+    assert_close(got.ravel(), oracle.row_softmax_f32(6, cols, x.ravel()), 1e-3 if cols > 20000 else F32_REL, F32_ABS, "edge rows")
     assert (got[1] == 0).all()
+    assert (got[5, :cols // 2] == 0).all() and abs(float(got[5].astype(np.float64).sum()) - 1.0) < 1e-4
+    assert got[4, 2500] == 0.5 and got[4, cols - 3] == 0.5
     assert got[2, 1777] == 1.0 and got[2].sum() == 1.0
-    assert got[4, 2500] == 0.5 and got[4, 4000] == 0.5
 
 
 @pytest.mark.parametrize("multiple_of_four", [False, True])
