@@ -851,6 +851,49 @@ __global__ __launch_bounds__(256) void transpose_f32_kernel(int rows, int cols, 
     }
 }
 
+// Copies rows × cols f32 matrices into rows_pad × cols_pad ones, zeros in the new rows and columns: two matrices (the
+// operands of a product) in one launch, the first `first_blocks` workgroups on the first.  A thread moves four
+// adjacent values of one output row (16-byte accesses at any alignment).
+struct PadJobF32 {
+    const float *in;
+    float *out;
+    unsigned rows, cols, rows_pad, cols_pad;
+};
+
+__global__ __launch_bounds__(256) void pad_f32_pair_kernel(PadJobF32 first, PadJobF32 second, unsigned first_blocks)
+{
+    typedef float pad_f32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+    const bool is_first = blockIdx.x < first_blocks;
+    const PadJobF32 &job = is_first ? first : second;
+    const unsigned chunks = (job.cols_pad + 3) / 4;
+    const unsigned idx = (blockIdx.x - (is_first ? 0u : first_blocks)) * 256u + threadIdx.x;  // below 2^29: the copies are below 2 GiB
+    const unsigned r = idx / chunks;
+    const unsigned c0 = (idx - r * chunks) * 4;
+    if (r >= job.rows_pad) return;
+    float *dst = job.out + static_cast<size_t>(r) * job.cols_pad + c0;
+    const float *src = job.in + static_cast<size_t>(r) * job.cols + c0;
+    if (r < job.rows && c0 + 4 <= job.cols) {
+        *reinterpret_cast<pad_f32x4_a4 *>(dst) = *reinterpret_cast<const pad_f32x4_a4 *>(src);
+        return;
+    }
+#pragma unroll
+    for (unsigned e = 0; e < 4; ++e) {
+        const unsigned c = c0 + e;
+        if (c < job.cols_pad) dst[e] = (r < job.rows && c < job.cols) ? src[e] : 0.0f;
+    }
+}
+
+hipError_t launch_pad_f32_pair(const PadJobF32 &first, const PadJobF32 &second, hipStream_t stream)
+{
+    auto blocks = [](const PadJobF32 &job) {
+        return static_cast<unsigned>((static_cast<size_t>(job.rows_pad) * ((job.cols_pad + 3) / 4) + 255) / 256);
+    };
+    const unsigned first_blocks = blocks(first), all = first_blocks + blocks(second);
+    if (all == 0) return hipSuccess;
+    hipLaunchKernelGGL(pad_f32_pair_kernel, dim3(all), dim3(256), 0, stream, first, second, first_blocks);
+    return hipGetLastError();
+}
+
 }  // namespace
 
 hipError_t launch_gemm_f32(size_t m, size_t n, size_t k, bool lhs_transposed, const float *lhs,
@@ -859,6 +902,31 @@ hipError_t launch_gemm_f32(size_t m, size_t n, size_t k, bool lhs_transposed, co
     if (m == 0 || n == 0) return hipSuccess;
     if (!lhs_transposed && gemv_f32_applies(m, n, k, lhs, rhs)) return launch_gemv_f32(m, n, k, lhs, rhs, out, epilogue, stream);
     if (lhs_transposed && scratch_free && gemv_t_f32_applies(m, n, k)) return launch_gemv_t_f32(m, n, k, lhs, rhs, out, epilogue, stream);
+    // A k that is not a multiple of 4 (a vocabulary of 50257 as the reduction of a backward product): the rows of A start
+    // at odd addresses, which the direct-to-LDS kernels do not take, and the general kernel runs at about 0.6 of their
+    // speed (1024×1024×4099: 140 µs against 80 µs at 4096).  Where the product is large against its operands, copies
+    // of A and B zero-padded along k to a multiple of 16 (exact: the new terms are 0·0) go into the stream's second
+    // scratch buffer, one launch for both, and the product runs on them.
+    // (Only where the copies then take the fast kernels: B's rows, and A's when it is stored k×m, must be 16-byte aligned.)
+    if (k % 4 != 0 && k > 64 && m >= 128 && n >= 128 && n % 4 == 0 && (!lhs_transposed || m % 4 == 0) && scratch_free &&
+        2.0 * m * n * k >= 2e9 &&
+        m * (k + 16) * sizeof(float) < (1ull << 31) && (k + 16) * n * sizeof(float) < (1ull << 31)) {
+        const size_t k_pad = (k + 15) / 16 * 16;
+        const size_t a_bytes = (m * k_pad * sizeof(float) + 255) & ~static_cast<size_t>(255);
+        void *copies = nullptr;
+        hipError_t rc = stream_workspace_slot(stream, 1, a_bytes + k_pad * n * sizeof(float), &copies);
+        if (rc != hipSuccess) return rc;
+        float *a_pad = static_cast<float *>(copies);
+        float *b_pad = reinterpret_cast<float *>(static_cast<unsigned char *>(copies) + a_bytes);
+        auto job = [](size_t rows, size_t cols, size_t rows_pad, size_t cols_pad, const float *in, float *to) {
+            return PadJobF32{in, to, static_cast<unsigned>(rows), static_cast<unsigned>(cols), static_cast<unsigned>(rows_pad),
+                             static_cast<unsigned>(cols_pad)};
+        };
+        rc = launch_pad_f32_pair(lhs_transposed ? job(k, m, k_pad, m, lhs, a_pad) : job(m, k, m, k_pad, lhs, a_pad),
+                                 job(k, n, k_pad, n, rhs, b_pad), stream);
+        if (rc != hipSuccess) return rc;
+        return launch_gemm_f32(m, n, k_pad, lhs_transposed, a_pad, b_pad, out, epilogue, stream, true);
+    }
     // An A of 2 GiB or more (the direct-to-LDS kernels address their operands through 32-bit byte offsets): row blocks
     // of A are independent products, so the launch is cut into blocks that fit and each takes the fast path.
     if (!lhs_transposed && m * k * sizeof(float) >= (1ull << 31) && k > 0 && k * 256 * sizeof(float) < (1ull << 31)) {

@@ -143,6 +143,9 @@ def test_long_reduction_against_float64(hip):
     (130, 70, 5000, True),
     (256, 192, 8192, True),    # the direct-to-LDS ring kernel, A transposed (a weight gradient Xᵀ·dY), k-sliced
     (100, 260, 4096, True),
+    (1024, 1024, 1001, False), # large products with an odd k run on copies zero-padded along k
+    (1024, 520, 2050, True),
+    (1500, 1000, 703, False),
     (10027, 1, 9472, True),    # Aᵀ·x with A stored k×m: lanes own outputs, k cut into slices; rows of odd length
     (4096, 4, 4100, True),     # four columns; the last 32-row group of a slice is short
     (1025, 2, 64, True),       # one slice; the last lanes' quad straddles the end of the rows
