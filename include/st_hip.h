@@ -166,7 +166,8 @@ enum {
     ST_HIP_CONV_KERNEL_STRIP9 = 5,       /* strip kernel, packed weight rows (more than 104 input channels) */
     ST_HIP_CONV_KERNEL_ADJOINT = 6,      /* grad_input only: adjoint gather (stride != 1 or padding > reach) */
     ST_HIP_CONV_KERNEL_COL2IM = 7,       /* grad_input only: per-image GEMM grad_outputᵀ·W, then a col2im gather  */
-    ST_HIP_CONV_KERNEL_TILE_KSLICED = 8  /* few tiles, long reduction: general kernel cut along c_in·kh·kw + a sum */
+    ST_HIP_CONV_KERNEL_TILE_KSLICED = 8, /* few tiles, long reduction: general kernel cut along c_in·kh·kw + a sum */
+    ST_HIP_CONV_KERNEL_DIRECT = 9        /* at most four output channels over many pixels: a thread per output pixel */
 };
 int st_hip_conv2d_force_family(int family);
 int st_hip_conv2d_planned_kernel(size_t batch, size_t c_in, size_t h, size_t w, size_t c_out, size_t kh,

@@ -890,6 +890,165 @@ hipError_t launch_tile(ConvArgs args, bool vec, hipStream_t stream, unsigned sli
 // on small shapes); ST_HIP_CONV_FAMILY_AUTO in normal use.
 std::atomic<int> g_forced_family{ST_HIP_CONV_FAMILY_AUTO};
 
+// One to four output channels over many pixels (the last layer of an image generator, a regression head): an MFMA tile
+// of 64 output channels would be padding from the fourth row on, and the layer is a stream over the input.  Here a
+// thread owns one output pixel and all CO channels; the weights are the same for the whole wavefront and come through
+// the scalar cache, the input through the vector cache, neighbouring pixels sharing most of their taps.
+template <int CO>
+__global__ __launch_bounds__(256) void conv2d_f32_direct_kernel(ConvArgs p)
+{
+    const ConvShape &s = p.s;
+    const int px = static_cast<int>(blockIdx.x) * 256 + static_cast<int>(threadIdx.x);
+    const int image = static_cast<int>(blockIdx.y);
+    if (px >= p.spatial) return;
+    const int oy = px / s.ow, ox = px - oy * s.ow;
+    const int iy0 = oy * s.stride_h - s.pad_h, ix0 = ox * s.stride_w - s.pad_w;
+    const size_t plane_elems = static_cast<size_t>(s.h) * s.w;
+    const float *in = p.input + static_cast<size_t>(image) * s.c_in * plane_elems;
+    const int K = p.K;
+    float acc[CO];
+#pragma unroll
+    for (int co = 0; co < CO; ++co) acc[co] = 0.0f;
+    for (int ci = 0; ci < s.c_in; ++ci) {
+        const float *plane = in + static_cast<size_t>(ci) * plane_elems;
+        const float *w_ci = p.weight + static_cast<size_t>(ci) * s.kh * s.kw;
+        for (int ky = 0; ky < s.kh; ++ky) {
+            const int iy = iy0 + ky * s.dil_h;
+            const bool row_ok = iy >= 0 && iy < s.h;
+            const float *row = plane + static_cast<size_t>(row_ok ? iy : 0) * s.w;
+            for (int kx = 0; kx < s.kw; ++kx) {
+                const int ix = ix0 + kx * s.dil_w;
+                const float v = (row_ok && ix >= 0 && ix < s.w) ? row[ix] : 0.0f;
+                const float *w_tap = w_ci + ky * s.kw + kx;
+#pragma unroll
+                for (int co = 0; co < CO; ++co) acc[co] = fmaf(v, w_tap[static_cast<size_t>(co) * K], acc[co]);
+            }
+        }
+    }
+#pragma unroll
+    for (int co = 0; co < CO; ++co) {
+        const float value = acc[co] + (p.bias ? p.bias[co] : -0.0f);
+        p.out[(static_cast<size_t>(image) * CO + co) * p.spatial + px] = apply_activation(value, p.activation);
+    }
+}
+
+// The same for unit stride and dilation along x and a kernel width known at compile time: a thread owns four adjacent
+// pixels of an output row, so that a row segment of KW + 3 input values (one 16-byte load at any alignment plus KW - 1
+// single ones) feeds 4·KW·CO multiply-adds, and the weights (at most 64 KB) are read from LDS, every lane the same word.
+// KH: the kernel height when it equals KW and is at most 5 (the loop over its rows is then unrolled, so that the loads of all rows of
+// a channel are in flight together: a thread's chain of load → multiply-add steps is what bounds this kernel), else 0.
+template <int CO, int KW, int KH>
+__global__ __launch_bounds__(256) void conv2d_f32_direct_rows_kernel(ConvArgs p)
+{
+    typedef float direct_f32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+    extern __shared__ float direct_weights[];  // CO × K, as stored
+    const ConvShape &s = p.s;
+    const int K = p.K;
+    for (int i = static_cast<int>(threadIdx.x); i < CO * K; i += 256) direct_weights[i] = p.weight[i];
+    __syncthreads();
+    const int quads = (s.ow + 3) / 4;  // threads per output row
+    const int item = static_cast<int>(blockIdx.x) * 256 + static_cast<int>(threadIdx.x);
+    if (item >= s.oh * quads) return;
+    const int oy = item / quads, ox0 = (item - oy * quads) * 4;
+    const int image = static_cast<int>(blockIdx.y);
+    const int iy0 = oy * s.stride_h - s.pad_h, ix0 = ox0 - s.pad_w;
+    constexpr int SEG = KW + 3;
+    const bool inside_x = ix0 >= 0 && ix0 + SEG <= s.w;
+    const size_t plane_elems = static_cast<size_t>(s.h) * s.w;
+    const float *in = p.input + static_cast<size_t>(image) * s.c_in * plane_elems;
+    float acc[CO][4];
+#pragma unroll
+    for (int co = 0; co < CO; ++co)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[co][j] = 0.0f;
+    const int kh = KH > 0 ? KH : s.kh;
+#pragma unroll 2
+    for (int ci = 0; ci < s.c_in; ++ci) {
+        const float *plane = in + static_cast<size_t>(ci) * plane_elems;
+#pragma unroll
+        for (int ky = 0; ky < kh; ++ky) {
+            const int iy = iy0 + ky * s.dil_h;
+            const bool row_ok = iy >= 0 && iy < s.h;  // a row of padding reads row 0 and counts as zeros
+            const float *row = plane + static_cast<size_t>(row_ok ? iy : 0) * s.w;
+            float v[SEG];
+            if (inside_x) {
+                const direct_f32x4_a4 t = *reinterpret_cast<const direct_f32x4_a4 *>(row + ix0);
+                v[0] = t[0]; v[1] = t[1]; v[2] = t[2]; v[3] = t[3];
+#pragma unroll
+                for (int i = 4; i < SEG; ++i) v[i] = row[ix0 + i];
+            } else {
+#pragma unroll
+                for (int i = 0; i < SEG; ++i) {
+                    const int ix = ix0 + i;
+                    v[i] = (ix >= 0 && ix < s.w) ? row[ix] : 0.0f;
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < SEG; ++i) v[i] = row_ok ? v[i] : 0.0f;
+            const float *taps = direct_weights + (ci * kh + ky) * KW;
+#pragma unroll
+            for (int kx = 0; kx < KW; ++kx)
+#pragma unroll
+                for (int co = 0; co < CO; ++co) {
+                    const float weight = taps[co * K + kx];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) acc[co][j] = fmaf(v[j + kx], weight, acc[co][j]);
+                }
+        }
+    }
+#pragma unroll
+    for (int co = 0; co < CO; ++co) {
+        const float b = p.bias ? p.bias[co] : -0.0f;
+        float *dst = p.out + (static_cast<size_t>(image) * CO + co) * p.spatial + static_cast<size_t>(oy) * s.ow + ox0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (ox0 + j < s.ow) dst[j] = apply_activation(acc[co][j] + b, p.activation);
+    }
+}
+
+template <int CO, int KW>
+hipError_t launch_direct_rows(const ConvArgs &args, hipStream_t stream)
+{
+    const size_t items = static_cast<size_t>(args.s.oh) * ((args.s.ow + 3) / 4);
+    const dim3 grid(static_cast<unsigned>((items + 255) / 256), static_cast<unsigned>(args.s.batch));
+    const size_t lds_bytes = static_cast<size_t>(CO) * args.K * sizeof(float);
+    if (args.s.kh == KW && KW <= 5) hipLaunchKernelGGL((conv2d_f32_direct_rows_kernel<CO, KW, KW>), grid, dim3(256), lds_bytes, stream, args);
+    else hipLaunchKernelGGL((conv2d_f32_direct_rows_kernel<CO, KW, 0>), grid, dim3(256), lds_bytes, stream, args);
+    return hipGetLastError();
+}
+
+template <int CO>
+hipError_t launch_direct_rows_for(const ConvArgs &args, hipStream_t stream)
+{
+    switch (args.s.kw) {
+    case 1: return launch_direct_rows<CO, 1>(args, stream);
+    case 3: return launch_direct_rows<CO, 3>(args, stream);
+    case 5: return launch_direct_rows<CO, 5>(args, stream);
+    default: return launch_direct_rows<CO, 7>(args, stream);
+    }
+}
+
+template <int CO>
+hipError_t launch_direct(const ConvArgs &args, hipStream_t stream)
+{
+    const ConvShape &s = args.s;
+    if (s.stride_w == 1 && s.dil_w == 1 && (s.kw == 1 || s.kw == 3 || s.kw == 5 || s.kw == 7) &&
+        static_cast<size_t>(CO) * args.K * sizeof(float) <= 64 * 1024)
+        return launch_direct_rows_for<CO>(args, stream);
+    const dim3 grid(static_cast<unsigned>((args.spatial + 255) / 256), static_cast<unsigned>(args.s.batch));
+    hipLaunchKernelGGL(conv2d_f32_direct_kernel<CO>, grid, dim3(256), 0, stream, args);
+    return hipGetLastError();
+}
+
+// At most four output channels over at least 65536 output pixels in all, kernels of more than one tap (8 × 64 × 256 × 256
+// → 3, 3×3: 440 → 104 µs; 7×7: 2751 → 433 µs; 16 × 32 × 128 × 128 → 1: 118 → 35 µs.  With 16384 pixels there are too few
+// threads for their serial walk over c_in·kh: 4 × 128 × 64 × 64 → 4 takes 64 µs on the tile kernel, 127 µs here).
+bool conv_direct_applies(const ConvShape &shape)
+{
+    return shape.c_out <= 4 && shape.kh * shape.kw > 1 && shape.batch <= 65535 &&
+           static_cast<long long>(shape.batch) * shape.oh * shape.ow >= 65536;
+}
+
 // The dispatcher's decision for `shape`: one of ST_HIP_CONV_KERNEL_*, or 0 when a forced family cannot serve the
 // shape.  `strip` is filled when a strip kernel is chosen.
 int choose_conv_kernel(const ConvShape &shape, bool weight_aligned, bool out_aligned, int forced, StripArgs &strip,
@@ -920,6 +1079,7 @@ int choose_conv_kernel(const ConvShape &shape, bool weight_aligned, bool out_ali
     }
     // Few tiles with a long reduction (deep layers on tiny planes at small batch, one or a few output channels): every
     // kernel here walks the reduction serially inside a workgroup, so the chip is filled by cutting the reduction.
+    if (conv_direct_applies(shape)) return ST_HIP_CONV_KERNEL_DIRECT;
     if (allow_slices && conv_k_slices(shape) > 1) return ST_HIP_CONV_KERNEL_TILE_KSLICED;
     if (!ring_ok) return ST_HIP_CONV_KERNEL_TILE;
     // The ring kernel has the better steady state (several rounds of 128×64 tiles per compute unit); the strip
@@ -996,6 +1156,13 @@ hipError_t launch_conv2d_f32(const ConvShape &shape, int activation, const float
                            static_cast<int>(used), shape.c_out, args.spatial, activation, partial, bias, out);
         return hipGetLastError();
     }
+    case ST_HIP_CONV_KERNEL_DIRECT:
+        switch (shape.c_out) {
+        case 1: return launch_direct<1>(args, stream);
+        case 2: return launch_direct<2>(args, stream);
+        case 3: return launch_direct<3>(args, stream);
+        default: return launch_direct<4>(args, stream);
+        }
     case ST_HIP_CONV_KERNEL_STRIP12:
     case ST_HIP_CONV_KERNEL_STRIP12_WIDE:
     case ST_HIP_CONV_KERNEL_STRIP9:

@@ -184,7 +184,7 @@ def conv2d_output_hw(h, w, kernel, stride, padding, dilation):
 
 
 CONV_FAMILIES = {"auto": 0, "tile": 1, "ring": 2, "strip": 3}
-CONV_KERNELS = {0: None, 1: "tile", 2: "ring", 3: "strip12", 4: "strip12_wide", 5: "strip9", 6: "adjoint", 7: "col2im", 8: "tile_ksliced"}
+CONV_KERNELS = {0: None, 1: "tile", 2: "ring", 3: "strip12", 4: "strip12_wide", 5: "strip9", 6: "adjoint", 7: "col2im", 8: "tile_ksliced", 9: "direct"}
 
 
 def conv2d_force_family(family: str) -> None:

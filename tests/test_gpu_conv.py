@@ -128,6 +128,32 @@ def test_few_tiles_with_a_long_reduction_are_cut_into_slices(hip, oracle, shape)
     assert_close(got, oracle.conv2d_bias_act_f32(*shape, oracle.ACT_NONE, x, wt, None), F32_REL, slack, "no bias")
 
 
+@pytest.mark.parametrize("shape", [
+    (8, 16, 96, 96, 3, (3, 3), (1, 1), (1, 1), (1, 1)),       # an RGB head
+    (4, 5, 130, 131, 1, (5, 5), (1, 1), (2, 2), (1, 1)),      # one channel; rows that are not a multiple of 4 pixels
+    (2, 4, 190, 190, 2, (7, 7), (1, 1), (3, 3), (1, 1)),      # seven taps a row: the loop over kernel rows is not unrolled
+    (4, 3, 130, 130, 2, (3, 5), (1, 1), (1, 2), (1, 1)),      # kernel height and width differ
+    (8, 8, 200, 200, 4, (3, 3), (2, 2), (1, 1), (1, 1)),      # strided along x: a thread per pixel
+    (7, 6, 100, 101, 2, (3, 3), (1, 1), (2, 2), (2, 2)),      # dilated
+    (8, 2, 140, 120, 3, (2, 4), (1, 2), (3, 0), (1, 1)),      # padding wider than the kernel's reach on one side
+])
+def test_few_output_channels_over_many_pixels(hip, oracle, shape):
+    """At most four output channels over at least 65536 output pixels: a thread per output pixel (or per four adjacent
+    ones) instead of matrix tiles that would be mostly padding."""
+    assert hip.conv2d_planned_kernel(*shape) == "direct"
+    batch, c_in, h, w, c_out, kernel, stride, padding, dilation = shape
+    rng = np.random.default_rng(c_in * 7 + c_out + h)
+    x = rng.normal(size=batch * c_in * h * w).astype(np.float32)
+    wt = rng.normal(0, np.sqrt(2.0 / (c_in * kernel[0] * kernel[1])), c_out * c_in * kernel[0] * kernel[1]).astype(np.float32)
+    b = rng.uniform(-0.5, 0.5, c_out).astype(np.float32)
+    for act, code in ((0, oracle.ACT_NONE), (1, oracle.ACT_RELU), (2, oracle.ACT_GELU)):
+        got = run(hip, *shape, act, x, wt, b)
+        assert_close(got, oracle.conv2d_bias_act_f32(*shape, code, x, wt, b), F32_REL, F32_ABS, f"conv {shape} act={act}")
+    got = run(hip, *shape, 0, x, wt, None)
+    assert_close(got, oracle.conv2d_bias_act_f32(*shape, oracle.ACT_NONE, x, wt, None), F32_REL, F32_ABS, "no bias")
+    assert float(np.abs(got).max()) > 0.1
+
+
 G33 = ((3, 3), (1, 1), (1, 1), (1, 1))
 FAMILY_SHAPES = {
     # name: (batch, c_in, h, w, c_out, kernel, stride, padding, dilation)
