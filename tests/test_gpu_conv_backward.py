@@ -147,6 +147,8 @@ GRAD_INPUT_FAMILY_CASES = [
     ("ring", "ring", (2, 20, 13, 12, 32, (7, 7), (1, 1), (3, 3), (1, 1))),          # 49 taps
     ("tile", "tile", (2, 24, 14, 14, 112, (3, 3), (1, 1), (1, 1), (1, 1))),
     ("tile", "tile", (2, 5, 10, 11, 6, (3, 3), (1, 1), (2, 2), (1, 1))),
+    # the first layer of an image model: its grad_input has three 'output' channels over many pixels
+    ("auto", "direct", (8, 3, 96, 96, 16, (3, 3), (1, 1), (1, 1), (1, 1))),
     ("auto", "adjoint", (2, 64, 9, 9, 250, (3, 3), (2, 1), (1, 0), (1, 1))),        # whole channel tile, stride 2×1
     ("auto", "adjoint", (2, 128, 10, 11, 6, (3, 3), (1, 1), (3, 3), (1, 1))),       # padding beyond the kernel's reach
     ("auto", "col2im", (2, 22, 9, 9, 250, (3, 3), (2, 1), (1, 0), (1, 1))),         # ragged channel tile: GEMM + col2im
