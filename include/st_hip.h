@@ -199,6 +199,31 @@ int st_hip_attention_f32(size_t contexts, size_t sequence, size_t head_dim, floa
                          size_t v_len, const float *z_bias, size_t z_bias_len,
                          const float *attn_bias, size_t attn_bias_len, float *out, size_t out_len);
 
+/* ---- launch arithmetic, computed on the host (no device is touched; usable without a GPU) ---- */
+
+/* The kernels whose workgroups decode their index into (context, query tile, key chunk) are launched only after the
+ * launcher has checked, with the decode function the kernel itself uses, that the grid is the product the decode
+ * assumes and that its first and last workgroups land inside the operands (otherwise the call fails with
+ * ST_HIP_ERR_RUNTIME and nothing is launched).  st_hip_attention_f32_launch_plan reports that plan for a shape and
+ * additionally walks the whole grid: `items` distinct work items decoded, `items_expected` what the shape calls for,
+ * `out_of_range` workgroups that would read outside the operands and `duplicates` items decoded twice (both must be
+ * 0), `consistent` the launcher's own check.  No reference counterpart (the reference's CPU loop,
+ * crates/st-tensor/src/pure.rs:11845-11919, has no launch geometry). */
+enum { ST_HIP_ATTN_KERNEL_GENERAL = 1, ST_HIP_ATTN_KERNEL_FAST = 2, ST_HIP_ATTN_KERNEL_FAST_BIASED = 3, ST_HIP_ATTN_KERNEL_TINY = 4 };
+typedef struct {
+    int kernel;         /* ST_HIP_ATTN_KERNEL_* */
+    int key_splits;     /* most key chunks a query tile is cut into (1: keys not split over workgroups) */
+    int keys_per_split; /* keys per chunk */
+    int consistent;     /* the check made before every launch passed */
+    uint64_t workgroups, items, items_expected, out_of_range, duplicates;
+} st_hip_attention_plan;
+int st_hip_attention_f32_launch_plan(size_t contexts, size_t sequence, size_t head_dim, int causal, int biased,
+                                     st_hip_attention_plan *plan);
+/* Rows of A per launch when a GEMM whose A is 2 GiB or larger is cut into row blocks for the kernels that address
+ * operands through 32-bit byte offsets: a multiple of 256 with rows*k*element_bytes < 2^31, or 0 when 256 rows do not
+ * fit (such products run on the kernels with 64-bit addressing). */
+size_t st_hip_gemm_row_block(size_t k, size_t element_bytes);
+
 /* ---- device-resident forms (caller owns device buffers; asynchronous on `stream`) ---------- */
 
 int st_hip_gemm_f32_dev(size_t m, size_t n, size_t k, float scale, int lhs_transposed,

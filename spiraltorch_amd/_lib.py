@@ -36,6 +36,12 @@ class ProbeResult(ctypes.Structure):
     _fields_ = [("available", c_int), ("initialized", c_int), ("device_count", c_int), ("error", ctypes.c_char * 256)]
 
 
+class AttentionPlan(ctypes.Structure):
+    _fields_ = [("kernel", c_int), ("key_splits", c_int), ("keys_per_split", c_int), ("consistent", c_int),
+                ("workgroups", c_uint64), ("items", c_uint64), ("items_expected", c_uint64), ("out_of_range", c_uint64),
+                ("duplicates", c_uint64)]
+
+
 class DecoderConfig(ctypes.Structure):
     _fields_ = [
         ("vocab", c_size_t),
@@ -83,6 +89,8 @@ SIGNATURES = {
     "st_hip_conv2d_output_hw": (c_int, [c_size_t] * 10 + [POINTER(c_size_t), POINTER(c_size_t)]),
     "st_hip_conv2d_force_family": (c_int, [c_int]),
     "st_hip_conv2d_planned_kernel": (c_int, [c_size_t] * 13 + [c_int, POINTER(c_int)]),
+    "st_hip_attention_f32_launch_plan": (c_int, [c_size_t, c_size_t, c_size_t, c_int, c_int, POINTER(AttentionPlan)]),
+    "st_hip_gemm_row_block": (c_size_t, [c_size_t, c_size_t]),
     "st_hip_conv2d_bias_act_f32": (c_int, [c_size_t] * 13 + [c_int, c_void_p, c_size_t, c_void_p, c_size_t,
                                                              c_void_p, c_size_t, c_void_p, c_size_t]),
     "st_hip_attention_f32": (c_int, [c_size_t, c_size_t, c_size_t, c_float, c_int, c_void_p, c_size_t, c_void_p,

@@ -19,6 +19,7 @@
 // so the running max / sum / rescale factors are per-lane scalars, and the only cross-lane traffic of
 // the softmax is one exchange between lane l and lane l^32 for the row maximum.
 #include <type_traits>
+#include <vector>
 
 #include "device_math.h"
 #include "kernels.h"
@@ -51,6 +52,60 @@ struct AttnArgs {
 
 constexpr int kBQ = 128;
 constexpr float kLog2e = 1.4426950408889634f;
+
+// What workgroup `block` of the fast kernel works on.  The kernel and the host-side launch checks share this one
+// function, so the grid the launcher asks for and the items the kernel decodes cannot drift apart unnoticed.
+//   unit        query tile (non-causal) or the index of a tile pair (causal: tiles q_tiles-1-unit and unit)
+//   split       which chunk of keys_per_split keys
+//   split_tile  causal launch with split keys: the (single) query tile, -1 otherwise
+struct FastItem {
+    int ctx, unit, split, split_tile;
+};
+
+template <bool CAUSAL>
+__host__ __device__ inline FastItem decode_fast_block(const int contexts, const int q_tiles, const int swizzle, const int key_splits,
+                                                      const int keys_per_split, const int causal_items, const int block)
+{
+    // Workgroup -> (context, query tiles).  Workgroup ids are dealt round-robin to the 8 XCDs, so id & 7 picks the
+    // XCD; each XCD keeps its own slice of the contexts and walks it context by context, so the workgroups that run
+    // together read the same K/V and those stay in that XCD's L2.  Under the causal mask a query tile's cost grows
+    // with its index, so a workgroup takes a PAIR of tiles, j and q_tiles-1-j, one after the other: every workgroup
+    // then does the same amount of work (q_tiles+1 key tiles), which balances the chip without spreading each
+    // context's tiles over the whole launch (longest-first across all contexts balanced as well, but re-read K/V
+    // from memory three times over).
+    const int per_ctx = CAUSAL ? (q_tiles + 1) / 2 : q_tiles;  // workgroups per context
+    FastItem item{0, 0, 0, -1};
+    if (swizzle) {
+        const int per_xcd = contexts >> 3;
+        const int xcd = block & 7, i = block >> 3;
+        item.ctx = xcd * per_xcd + i / per_ctx;
+        item.unit = i % per_ctx;
+        return item;
+    }
+    int id = block;
+    if (CAUSAL && key_splits > 1) {
+        // (tile, chunk) items of a context, tiles from the last (most chunks) to the first
+        item.ctx = id / causal_items;
+        int rest = id - item.ctx * causal_items;
+        const int r = keys_per_split / kBQ;
+        int j = q_tiles - 1;
+        for (; j > 0; --j) {
+            const int chunks = j / r + 1;
+            if (rest < chunks) break;
+            rest -= chunks;
+        }
+        item.split_tile = j;
+        item.split = rest;
+        return item;
+    }
+    if (!CAUSAL) {  // the splits of one query tile are neighbours: they share its Q rows in the L2
+        item.split = id % key_splits;
+        id /= key_splits;
+    }
+    item.ctx = id / per_ctx;
+    item.unit = id % per_ctx;
+    return item;
+}
 
 template <bool VEC>
 __device__ __forceinline__ float4 load_d4(const float *row, int d, int D, bool row_valid)
@@ -299,47 +354,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DPAD <= 64 
     const int li = lane & 31, lh = lane >> 5;
     const int S = p.S, D = p.D;
 
-    // Workgroup -> (context, query tiles).  Workgroup ids are dealt round-robin to the 8 XCDs, so id & 7 picks the
-    // XCD; each XCD keeps its own slice of the contexts and walks it context by context, so the workgroups that run
-    // together read the same K/V and those stay in that XCD's L2.  Under the causal mask a query tile's cost grows
-    // with its index, so a workgroup takes a PAIR of tiles, j and q_tiles-1-j, one after the other: every workgroup
-    // then does the same amount of work (q_tiles+1 key tiles), which balances the chip without spreading each
-    // context's tiles over the whole launch (longest-first across all contexts balanced as well, but re-read K/V
-    // from memory three times over).
-    const int per_ctx = CAUSAL ? (p.q_tiles + 1) / 2 : p.q_tiles;  // workgroups per context
-    int ctx, unit;
-    int split = 0;
-    int split_tile = -1;  // causal with split keys: this workgroup's query tile (no pairing then)
-    if (p.swizzle) {
-        const int per_xcd = p.contexts >> 3;
-        const int xcd = blockIdx.x & 7, i = blockIdx.x >> 3;
-        ctx = xcd * per_xcd + i / per_ctx;
-        unit = i % per_ctx;
-    } else {
-        int id = blockIdx.x;
-        if (CAUSAL && p.key_splits > 1) {
-            // (tile, chunk) items of a context, tiles from the last (most chunks) to the first
-            ctx = id / p.causal_items;
-            int rest = id - ctx * p.causal_items;
-            const int r = p.keys_per_split / kBQ;
-            int j = p.q_tiles - 1;
-            for (;; --j) {
-                const int chunks = j / r + 1;
-                if (rest < chunks) break;
-                rest -= chunks;
-            }
-            split_tile = j;
-            split = rest;
-            unit = 0;
-        } else {
-            if constexpr (!CAUSAL) {  // the splits of one query tile are neighbours: they share its Q rows in the L2
-                split = id % p.key_splits;
-                id /= p.key_splits;
-            }
-            ctx = id / per_ctx;
-            unit = id % per_ctx;
-        }
-    }
+    const FastItem item = decode_fast_block<CAUSAL>(p.contexts, p.q_tiles, p.swizzle, p.key_splits, p.keys_per_split,
+                                                    p.causal_items, static_cast<int>(blockIdx.x));
+    const int ctx = item.ctx, unit = item.unit, split = item.split;
+    const int split_tile = item.split_tile;  // causal with split keys: this workgroup's query tile (no pairing then)
     const size_t ctx_elem0 = static_cast<size_t>(ctx) * S * D;
     const unsigned ctx_bytes = static_cast<unsigned>(S) * static_cast<unsigned>(D) * 4u;
     const __amdgpu_buffer_rsrc_t rsrc_q =
@@ -846,6 +864,83 @@ __global__ __launch_bounds__(256) void attention_merge_splits_kernel(AttnArgs p,
     *reinterpret_cast<float4 *>(p.out + row * D + d) = make_float4(acc.x * inv, acc.y * inv, acc.z * inv, acc.w * inv);
 }
 
+// Launch plan of the fast kernel: fills the split fields of `args` and returns the number of workgroups; `causal_r` is
+// the r of the causal key split (0 when the launch is not split that way).  Pure host arithmetic.
+size_t plan_fast(AttnArgs &args, const bool causal, int *causal_r)
+{
+    size_t blocks = static_cast<size_t>(args.contexts) * (causal ? (args.q_tiles + 1) / 2 : args.q_tiles);
+    args.key_splits = 1;
+    args.keys_per_split = args.S;
+    args.causal_items = 0;
+    *causal_r = 0;
+    constexpr size_t kTargetBlocks = 512;
+    if (blocks * 2 > kTargetBlocks || args.S < 256) return blocks;
+    if (causal) {
+        // Few contexts: pairs of query tiles leave most of the chip idle (8 contexts of 2048: 64 workgroups, slower than
+        // the non-causal call that does twice the work).  Split every tile's keys into chunks of 128·r instead, with the
+        // largest r that still gives about two workgroups per compute unit; all (tile, chunk) items then cost the same.
+        const size_t tiles = static_cast<size_t>(args.q_tiles);
+        auto items = [&](size_t r) {
+            size_t total = 0;
+            for (size_t j = 0; j < tiles; ++j) total += j / r + 1;
+            return total;
+        };
+        size_t r = tiles;
+        while (r > 1 && static_cast<size_t>(args.contexts) * items(r) < kTargetBlocks) --r;
+        const size_t per_context = items(r);
+        // (r == tiles would be one chunk per tile: nothing to merge, and the kernel tells the two forms apart by
+        // key_splits > 1 — such launches keep the pairing.)
+        if (r < tiles && static_cast<size_t>(args.contexts) * per_context > blocks) {
+            *causal_r = static_cast<int>(r);
+            args.keys_per_split = static_cast<int>(r) * kBQ;
+            args.key_splits = static_cast<int>((tiles - 1) / r + 1);
+            args.causal_items = static_cast<int>(per_context);
+            blocks = static_cast<size_t>(args.contexts) * per_context;
+        }
+    } else {
+        // Few query tiles (the reference's own caller attends within one context: crates/st-nn/src/z_rba/attention.rs:586):
+        // split the keys over workgroups until the launch offers about two workgroups per compute unit, 128 keys at least
+        // per split, and merge the partial rows in a second kernel.
+        const size_t want = (kTargetBlocks + blocks - 1) / blocks;
+        const size_t most = static_cast<size_t>(args.S) / 128;
+        const size_t splits = std::min(want, most);
+        const size_t per = ((static_cast<size_t>(args.S) + splits - 1) / splits + 63) / 64 * 64;
+        args.keys_per_split = static_cast<int>(per);
+        args.key_splits = static_cast<int>((static_cast<size_t>(args.S) + per - 1) / per);
+        blocks *= static_cast<size_t>(args.key_splits);
+    }
+    if (args.key_splits > 1) args.swizzle = 0;
+    return blocks;
+}
+
+// True when workgroup `block` of a planned launch decodes to a (context, query tile, key chunk) inside the operands.
+bool fast_block_in_range(const AttnArgs &args, const bool causal, const size_t block)
+{
+    const FastItem item = causal ? decode_fast_block<true>(args.contexts, args.q_tiles, args.swizzle, args.key_splits,
+                                                           args.keys_per_split, args.causal_items, static_cast<int>(block))
+                                 : decode_fast_block<false>(args.contexts, args.q_tiles, args.swizzle, args.key_splits,
+                                                            args.keys_per_split, args.causal_items, static_cast<int>(block));
+    if (item.ctx < 0 || item.ctx >= args.contexts || item.split < 0 || item.split >= args.key_splits) return false;
+    if (item.split_tile >= 0) {  // causal, split keys: chunk `split` of the (tile + 1)·128 keys the tile sees
+        return item.split_tile < args.q_tiles && item.split * args.keys_per_split < std::min(args.S, (item.split_tile + 1) * kBQ);
+    }
+    if (causal) return item.unit >= 0 && item.unit < (args.q_tiles + 1) / 2;
+    return item.unit >= 0 && item.unit < args.q_tiles && item.split * args.keys_per_split < args.S;
+}
+
+// The launch arithmetic, checked before every launch of the fast kernel: the grid is what the decode assumes, fits
+// the 32-bit ids the kernel computes with, and its first and last workgroups decode to items inside the operands.
+bool fast_plan_consistent(const AttnArgs &args, const bool causal, const size_t blocks)
+{
+    if (blocks == 0 || blocks > 0x7fffffffu) return false;
+    if (args.swizzle && (args.contexts % 8 != 0 || args.key_splits != 1)) return false;
+    const size_t per_ctx = causal ? (args.key_splits > 1 ? static_cast<size_t>(args.causal_items) : (args.q_tiles + 1) / 2)
+                                  : static_cast<size_t>(args.q_tiles) * args.key_splits;
+    if (blocks != static_cast<size_t>(args.contexts) * per_ctx) return false;
+    if (args.key_splits > 1 && (args.keys_per_split <= 0 || args.keys_per_split % 64 != 0)) return false;
+    return fast_block_in_range(args, causal, 0) && fast_block_in_range(args, causal, blocks - 1);
+}
+
 template <int DPAD, bool CAUSAL, bool BIAS = false>
 hipError_t launch_fast(AttnArgs args, hipStream_t stream)
 {
@@ -854,53 +949,10 @@ hipError_t launch_fast(AttnArgs args, hipStream_t stream)
     hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
     if (rc != hipSuccess) return rc;
-    size_t blocks = static_cast<size_t>(args.contexts) * (CAUSAL ? (args.q_tiles + 1) / 2 : args.q_tiles);
-    args.key_splits = 1;
-    args.keys_per_split = args.S;
-    args.causal_items = 0;
     args.part_o = args.part_ml = nullptr;
     int causal_r = 0;
-    if constexpr (CAUSAL) {
-        // Few contexts: pairs of query tiles leave most of the chip idle (8 contexts of 2048: 64 workgroups, slower than
-        // the non-causal call that does twice the work).  Split every tile's keys into chunks of 128·r instead, with the
-        // largest r that still gives about two workgroups per compute unit; all (tile, chunk) items then cost the same.
-        constexpr size_t kTargetBlocks = 512;
-        if (blocks * 2 <= kTargetBlocks && args.S >= 256) {
-            const size_t tiles = static_cast<size_t>(args.q_tiles);
-            auto items = [&](size_t r) {
-                size_t total = 0;
-                for (size_t j = 0; j < tiles; ++j) total += j / r + 1;
-                return total;
-            };
-            size_t r = tiles;
-            while (r > 1 && static_cast<size_t>(args.contexts) * items(r) < kTargetBlocks) --r;
-            const size_t per_context = items(r);
-            // (r == tiles would be one chunk per tile: nothing to merge, and the kernel tells the two forms apart by
-            // key_splits > 1 — such launches keep the pairing.)
-            if (r < tiles && static_cast<size_t>(args.contexts) * per_context > blocks) {
-                causal_r = static_cast<int>(r);
-                args.keys_per_split = static_cast<int>(r) * kBQ;
-                args.key_splits = static_cast<int>((tiles - 1) / r + 1);
-                args.causal_items = static_cast<int>(per_context);
-                blocks = static_cast<size_t>(args.contexts) * per_context;
-            }
-        }
-    }
-    if constexpr (!CAUSAL) {
-        // Few query tiles (the reference's own caller attends within one context: crates/st-nn/src/z_rba/attention.rs:586):
-        // split the keys over workgroups until the launch offers about two workgroups per compute unit, 128 keys at least
-        // per split, and merge the partial rows in a second kernel.
-        constexpr size_t kTargetBlocks = 512;
-        if (blocks * 2 <= kTargetBlocks && args.S >= 256) {
-            const size_t want = (kTargetBlocks + blocks - 1) / blocks;
-            const size_t most = static_cast<size_t>(args.S) / 128;
-            const size_t splits = std::min(want, most);
-            const size_t per = ((static_cast<size_t>(args.S) + splits - 1) / splits + 63) / 64 * 64;
-            args.keys_per_split = static_cast<int>(per);
-            args.key_splits = static_cast<int>((static_cast<size_t>(args.S) + per - 1) / per);
-        }
-        if (args.key_splits > 1) blocks *= static_cast<size_t>(args.key_splits);
-    }
+    const size_t blocks = plan_fast(args, CAUSAL, &causal_r);
+    if (!fast_plan_consistent(args, CAUSAL, blocks)) return hipErrorInvalidConfiguration;
     if (args.key_splits > 1) {
         const size_t rows = static_cast<size_t>(args.contexts) * args.S;
         const size_t o_bytes = static_cast<size_t>(args.key_splits) * rows * args.D * sizeof(float);
@@ -910,7 +962,6 @@ hipError_t launch_fast(AttnArgs args, hipStream_t stream)
         if (rc != hipSuccess) return rc;
         args.part_o = static_cast<float *>(workspace);
         args.part_ml = reinterpret_cast<float *>(static_cast<unsigned char *>(workspace) + o_bytes);
-        args.swizzle = 0;
     }
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), lds_bytes, stream, args);
     rc = hipGetLastError();
@@ -951,6 +1002,78 @@ hipError_t launch_dpad(const AttnArgs &args, bool causal, bool bias, bool vec, h
 }
 
 }  // namespace
+
+AttentionPlanReport attention_f32_plan_report(size_t contexts, size_t sequence, size_t head_dim, bool causal, bool biased)
+{
+    AttentionPlanReport report{};
+    if (contexts == 0 || sequence == 0 || head_dim == 0 || head_dim > static_cast<size_t>(kAttentionMaxHeadDim)) return report;
+    AttnArgs args{};
+    args.contexts = static_cast<int>(contexts);
+    args.S = static_cast<int>(sequence);
+    args.D = static_cast<int>(head_dim);
+    args.q_tiles = static_cast<int>((sequence + kBQ - 1) / kBQ);
+    args.swizzle = (contexts % 8 == 0) ? 1 : 0;
+    args.key_splits = 1;
+    args.keys_per_split = args.S;
+    const bool vec = head_dim % 4 == 0;
+    const bool fits_buffer = sequence * head_dim * sizeof(float) < (1ull << 31);
+    report.key_splits = 1;
+    report.keys_per_split = args.S;
+    if (!biased && vec && fits_buffer && head_dim <= 128 && sequence <= 64 && contexts >= 256) {
+        report.kernel = ST_HIP_ATTN_KERNEL_TINY;  // a wavefront per context, four (or two) contexts a workgroup
+        report.workgroups = (contexts + 3) / 4;
+        report.items = report.items_expected = contexts;
+        return report;
+    }
+    const bool fast = vec && fits_buffer && (biased ? head_dim <= 64 && sequence % 4 == 0 : head_dim <= 128);
+    if (!fast) {
+        report.kernel = ST_HIP_ATTN_KERNEL_GENERAL;  // one workgroup per (context, query tile), decoded by division
+        report.workgroups = contexts * static_cast<size_t>(args.q_tiles);
+        report.items = report.items_expected = report.workgroups;
+        return report;
+    }
+    report.kernel = biased ? ST_HIP_ATTN_KERNEL_FAST_BIASED : ST_HIP_ATTN_KERNEL_FAST;
+    int causal_r = 0;
+    const size_t blocks = plan_fast(args, causal, &causal_r);
+    report.workgroups = blocks;
+    report.key_splits = args.key_splits;
+    report.keys_per_split = args.keys_per_split;
+    report.consistent = fast_plan_consistent(args, causal, blocks) ? 1 : 0;
+    const size_t tiles = static_cast<size_t>(args.q_tiles), splits = static_cast<size_t>(args.key_splits);
+    if (causal && args.key_splits > 1) {
+        for (size_t j = 0; j < tiles; ++j) report.items_expected += contexts * (j / static_cast<size_t>(causal_r) + 1);
+    } else if (causal) {
+        report.items_expected = contexts * tiles;
+    } else {
+        report.items_expected = contexts * tiles * splits;
+    }
+    if (blocks > (1ull << 26)) return report;  // the walk below is for tests; launches are covered by `consistent`
+    std::vector<unsigned char> seen(contexts * tiles * splits, 0);
+    auto mark = [&](int ctx, int tile, int split) {
+        unsigned char &cell = seen[(static_cast<size_t>(ctx) * tiles + tile) * splits + split];
+        if (cell) ++report.duplicates; else ++report.items;
+        cell = 1;
+    };
+    for (size_t block = 0; block < blocks; ++block) {
+        if (!fast_block_in_range(args, causal, block)) {
+            ++report.out_of_range;
+            continue;
+        }
+        const FastItem item = causal ? decode_fast_block<true>(args.contexts, args.q_tiles, args.swizzle, args.key_splits,
+                                                               args.keys_per_split, args.causal_items, static_cast<int>(block))
+                                     : decode_fast_block<false>(args.contexts, args.q_tiles, args.swizzle, args.key_splits,
+                                                                args.keys_per_split, args.causal_items, static_cast<int>(block));
+        if (item.split_tile >= 0) {
+            mark(item.ctx, item.split_tile, item.split);
+        } else if (causal) {
+            mark(item.ctx, args.q_tiles - 1 - item.unit, 0);
+            if (item.unit != args.q_tiles - 1 - item.unit) mark(item.ctx, item.unit, 0);
+        } else {
+            mark(item.ctx, item.unit, item.split);
+        }
+    }
+    return report;
+}
 
 hipError_t launch_attention_f32(size_t contexts, size_t sequence, size_t head_dim, float scale, bool causal,
                                 const float *q, const float *k, const float *v, const float *z_bias,

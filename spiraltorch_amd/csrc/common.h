@@ -32,6 +32,17 @@ constexpr size_t kMaxDim = 0x7fffffffu;  // dims must fit i32 (crates/st-tensor/
 
 inline hipStream_t as_stream(void *stream) { return static_cast<hipStream_t>(stream); }
 
+// Rows of A per launch when an A of 2 GiB or more is cut into row blocks for kernels that address their operands
+// through 32-bit byte offsets: the largest multiple of 256 rows whose k·element_bytes bytes stay below 2^31, or 0 when
+// not even 256 rows fit (the caller then leaves the product to a kernel with 64-bit addressing).
+inline size_t gemm_row_block(size_t k, size_t element_bytes)
+{
+    const size_t row_bytes = k * element_bytes;
+    if (row_bytes == 0) return 0;
+    const size_t rows = ((1ull << 31) - 1) / row_bytes;  // rows·row_bytes <= 2^31 - 1
+    return rows / 256 * 256;
+}
+
 }  // namespace sthip
 
 #define ST_HIP_TRY(expr, ctx)                                        \

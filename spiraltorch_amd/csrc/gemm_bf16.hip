@@ -2356,8 +2356,8 @@ hipError_t launch_gemm_bf16(size_t m, size_t n, size_t k, const uint16_t *lhs, c
         return launch_gemv_bf16(m, n, k, lhs, rhs, rhs_packed, out_f32, out_bf16, epilogue, stream);
     // An A of 2 GiB or more (the 256-row kernels address their operands through 32-bit byte offsets): row blocks of A
     // are independent products, so the launch is cut into blocks that fit and each takes the fast path.
-    if (m * k * sizeof(uint16_t) >= (1ull << 31) && k > 0 && k * 256 * sizeof(uint16_t) < (1ull << 31)) {
-        const size_t block = ((1ull << 31) / (k * sizeof(uint16_t)) - 1) / 256 * 256;
+    if (m * k * sizeof(uint16_t) >= (1ull << 31) && gemm_row_block(k, sizeof(uint16_t)) > 0) {
+        const size_t block = gemm_row_block(k, sizeof(uint16_t));
         for (size_t row = 0; row < m; row += block) {
             const size_t rows = std::min(block, m - row);
             GemmEpilogue part = epilogue;

@@ -929,8 +929,8 @@ hipError_t launch_gemm_f32(size_t m, size_t n, size_t k, bool lhs_transposed, co
     }
     // An A of 2 GiB or more (the direct-to-LDS kernels address their operands through 32-bit byte offsets): row blocks
     // of A are independent products, so the launch is cut into blocks that fit and each takes the fast path.
-    if (!lhs_transposed && m * k * sizeof(float) >= (1ull << 31) && k > 0 && k * 256 * sizeof(float) < (1ull << 31)) {
-        const size_t block = ((1ull << 31) / (k * sizeof(float)) - 1) / 256 * 256;
+    if (!lhs_transposed && m * k * sizeof(float) >= (1ull << 31) && gemm_row_block(k, sizeof(float)) > 0) {
+        const size_t block = gemm_row_block(k, sizeof(float));
         for (size_t row = 0; row < m; row += block) {
             const size_t rows = std::min(block, m - row);
             GemmEpilogue part = epilogue;

@@ -471,6 +471,36 @@ int st_hip_conv2d_planned_kernel(size_t batch, size_t c_in, size_t h, size_t w, 
     return ST_HIP_OK;
 }
 
+int st_hip_attention_f32_launch_plan(size_t contexts, size_t sequence, size_t head_dim, int causal, int biased,
+                                     st_hip_attention_plan *plan)
+{
+    if (!plan) return fail(ST_HIP_ERR_INVALID, "attention launch_plan received a null out-pointer");
+    size_t rows = 0, volume = 0;
+    if (contexts > kMaxDim || sequence > kMaxDim || head_dim > kMaxDim || !checked_mul(contexts, sequence, &rows) ||
+        !checked_mul(rows, head_dim, &volume))
+        return fail(ST_HIP_ERR_INVALID, "attention dimensions overflow");
+    if (head_dim > static_cast<size_t>(kAttentionMaxHeadDim))
+        return fail(ST_HIP_ERR_UNSUPPORTED, "attention head_dim %zu exceeds %d", head_dim, kAttentionMaxHeadDim);
+    const AttentionPlanReport report = attention_f32_plan_report(contexts, sequence, head_dim, causal != 0, biased != 0);
+    plan->kernel = report.kernel;
+    plan->key_splits = report.key_splits;
+    plan->keys_per_split = report.keys_per_split;
+    plan->consistent = report.kernel == ST_HIP_ATTN_KERNEL_FAST || report.kernel == ST_HIP_ATTN_KERNEL_FAST_BIASED ? report.consistent : 1;
+    plan->workgroups = report.workgroups;
+    plan->items = report.items;
+    plan->items_expected = report.items_expected;
+    plan->out_of_range = report.out_of_range;
+    plan->duplicates = report.duplicates;
+    return ST_HIP_OK;
+}
+
+size_t st_hip_gemm_row_block(size_t k, size_t element_bytes)
+{
+    size_t row_bytes = 0;
+    if (!checked_mul(k, element_bytes, &row_bytes)) return 0;
+    return gemm_row_block(k, element_bytes);
+}
+
 int st_hip_conv2d_bias_act_f32(size_t batch, size_t c_in, size_t h, size_t w, size_t c_out, size_t kh, size_t kw,
                                size_t stride_h, size_t stride_w, size_t pad_h, size_t pad_w, size_t dil_h,
                                size_t dil_w, int activation, const float *input, size_t input_len,

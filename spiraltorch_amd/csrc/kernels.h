@@ -104,6 +104,14 @@ hipError_t launch_attention_f32(size_t contexts, size_t sequence, size_t head_di
                                 const float *z_bias, const float *attn_bias, float *out,
                                 hipStream_t stream);
 
+// The launch arithmetic of launch_attention_f32 for a shape (16-byte aligned operands assumed), with every workgroup
+// of the fast kernel's grid decoded on the host the way the kernel decodes it: see st_hip_attention_plan.
+struct AttentionPlanReport {
+    int kernel, key_splits, keys_per_split, consistent;
+    uint64_t workgroups, items, items_expected, out_of_range, duplicates;
+};
+AttentionPlanReport attention_f32_plan_report(size_t contexts, size_t sequence, size_t head_dim, bool causal, bool biased);
+
 // bf16 attention over heads stored as column slices of (batch·sequence, ld) matrices; head_dim 64 or 128.
 bool attention_bf16_supported(size_t sequence, size_t head_dim, size_t ld_in, size_t ld_out, const void *q,
                               const void *k, const void *v, const void *out);

@@ -224,6 +224,25 @@ def conv2d_backward_f32(batch, c_in, h, w, c_out, kernel, stride, padding, dilat
         _ptr(gb), gb.size))
 
 
+ATTENTION_KERNELS = {1: "general", 2: "fast", 3: "fast_biased", 4: "tiny"}
+
+
+def attention_f32_launch_plan(contexts, sequence, head_dim, causal=False, biased=False) -> dict:
+    """The launch arithmetic of the f32 attention for a shape, with the whole grid decoded on the host the way the
+    kernel decodes it (no device is touched)."""
+    plan = _lib.AttentionPlan()
+    _check(_lib.load().st_hip_attention_f32_launch_plan(contexts, sequence, head_dim, int(bool(causal)), int(bool(biased)),
+                                                         ctypes.byref(plan)))
+    out = {name: int(getattr(plan, name)) for name, _ in _lib.AttentionPlan._fields_}
+    out["kernel"] = ATTENTION_KERNELS.get(out["kernel"], "none")
+    return out
+
+
+def gemm_row_block(k: int, element_bytes: int) -> int:
+    """Rows of A per launch when an A of 2 GiB or more is cut into row blocks (0: not even 256 rows fit)."""
+    return int(_lib.load().st_hip_gemm_row_block(k, element_bytes))
+
+
 def attention_f32(contexts, sequence, head_dim, scale, causal, q, k, v, z_bias, attn_bias, out) -> None:
     q, k, v, out = _f32(q, "q"), _f32(k, "k"), _f32(v, "v"), _out(out, "out")
     zb = None if z_bias is None else _f32(z_bias, "z_bias")
@@ -250,6 +269,14 @@ class DeviceBuffer:
         buf = cls(a.nbytes)
         _check(_lib.load().st_hip_memcpy_h2d(buf.ptr, ctypes.c_void_p(a.ctypes.data), a.nbytes, _stream_ptr(stream)))
         return buf
+
+    def upload(self, array: np.ndarray, byte_offset: int = 0, stream=None) -> None:
+        """Copies a host array into the allocation starting `byte_offset` bytes in."""
+        a = np.ascontiguousarray(array)
+        if byte_offset < 0 or byte_offset + a.nbytes > self.nbytes:
+            raise ValueError("array does not fit the device buffer at that offset")
+        _check(_lib.load().st_hip_memcpy_h2d(ctypes.c_void_p(self.at(byte_offset)), ctypes.c_void_p(a.ctypes.data),
+                                             a.nbytes, _stream_ptr(stream)))
 
     def to_array(self, dtype, shape, stream=None) -> np.ndarray:
         out = np.empty(shape, dtype=dtype)

@@ -16,7 +16,7 @@ TARGET = os.path.join(HERE, "st-backend-hip", "src", "ffi.rs")
 
 SCALARS = {"size_t": "usize", "int": "c_int", "float": "f32", "uint64_t": "u64", "uint16_t": "u16", "char": "c_char",
            "void": "c_void", "st_hip_device_props": "StHipDeviceProps", "st_hip_probe_result": "StHipProbeResult",
-           "st_hip_decoder_config": "StHipDecoderConfig"}
+           "st_hip_decoder_config": "StHipDecoderConfig", "st_hip_attention_plan": "StHipAttentionPlan"}
 RUST_KEYWORDS = {"in": "input", "type": "kind", "ref": "reference"}
 
 STRUCTS = '''/// `st_hip_device_props`.
@@ -56,6 +56,21 @@ pub struct StHipDecoderConfig {
     pub batch: usize,
     pub seq: usize,
     pub ln_eps: f32,
+}
+
+/// `st_hip_attention_plan`.
+#[repr(C)]
+#[derive(Clone, Copy, Debug, Default, PartialEq)]
+pub struct StHipAttentionPlan {
+    pub kernel: c_int,
+    pub key_splits: c_int,
+    pub keys_per_split: c_int,
+    pub consistent: c_int,
+    pub workgroups: u64,
+    pub items: u64,
+    pub items_expected: u64,
+    pub out_of_range: u64,
+    pub duplicates: u64,
 }
 '''
 

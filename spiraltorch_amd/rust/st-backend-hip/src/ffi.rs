@@ -44,6 +44,21 @@ pub struct StHipDecoderConfig {
     pub ln_eps: f32,
 }
 
+/// `st_hip_attention_plan`.
+#[repr(C)]
+#[derive(Clone, Copy, Debug, Default, PartialEq)]
+pub struct StHipAttentionPlan {
+    pub kernel: c_int,
+    pub key_splits: c_int,
+    pub keys_per_split: c_int,
+    pub consistent: c_int,
+    pub workgroups: u64,
+    pub items: u64,
+    pub items_expected: u64,
+    pub out_of_range: u64,
+    pub duplicates: u64,
+}
+
 #[link(name = "sthip")]
 extern "C" {
     pub fn st_hip_init() -> c_int;
@@ -79,6 +94,8 @@ extern "C" {
     pub fn st_hip_conv2d_planned_kernel(batch: usize, c_in: usize, h: usize, w: usize, c_out: usize, kh: usize, kw: usize, stride_h: usize, stride_w: usize, pad_h: usize, pad_w: usize, dil_h: usize, dil_w: usize, direction: c_int, kernel: *mut c_int) -> c_int;
     pub fn st_hip_conv2d_backward_f32(batch: usize, c_in: usize, h: usize, w: usize, c_out: usize, kh: usize, kw: usize, stride_h: usize, stride_w: usize, pad_h: usize, pad_w: usize, dil_h: usize, dil_w: usize, input: *const f32, input_len: usize, weight: *const f32, weight_len: usize, grad_output: *const f32, grad_output_len: usize, grad_input: *mut f32, grad_input_len: usize, grad_weight: *mut f32, grad_weight_len: usize, grad_bias: *mut f32, grad_bias_len: usize) -> c_int;
     pub fn st_hip_attention_f32(contexts: usize, sequence: usize, head_dim: usize, scale: f32, causal: c_int, q: *const f32, q_len: usize, k: *const f32, k_len: usize, v: *const f32, v_len: usize, z_bias: *const f32, z_bias_len: usize, attn_bias: *const f32, attn_bias_len: usize, out: *mut f32, out_len: usize) -> c_int;
+    pub fn st_hip_attention_f32_launch_plan(contexts: usize, sequence: usize, head_dim: usize, causal: c_int, biased: c_int, plan: *mut StHipAttentionPlan) -> c_int;
+    pub fn st_hip_gemm_row_block(k: usize, element_bytes: usize) -> usize;
     pub fn st_hip_gemm_f32_dev(m: usize, n: usize, k: usize, scale: f32, lhs_transposed: c_int, lhs: *const f32, rhs: *const f32, out: *mut f32, stream: *mut c_void) -> c_int;
     pub fn st_hip_gemm_bias_act_f32_dev(m: usize, n: usize, k: usize, activation: c_int, lhs: *const f32, rhs: *const f32, bias: *const f32, residual: *const f32, out: *mut f32, stream: *mut c_void) -> c_int;
     pub fn st_hip_gemm_prepacked_bias_act_f32_dev(m: usize, n: usize, k: usize, activation: c_int, lhs: *const f32, packed_rhs: *const f32, bias: *const f32, residual: *const f32, out: *mut f32, stream: *mut c_void) -> c_int;
