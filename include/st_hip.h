@@ -91,6 +91,14 @@ int st_hip_stream_create(void **stream);
 int st_hip_stream_synchronize(void *stream);
 int st_hip_stream_destroy(void *stream);
 int st_hip_device_synchronize(void);
+/* Scratch memory (split-k partial sums, re-laid weights, padded operand copies) is kept per (stream, host thread) and
+ * grows on demand; a buffer whose host thread has exited is re-used by the next thread that launches on that stream,
+ * and st_hip_stream_destroy frees its stream's buffers.  st_hip_release_scratch waits for `stream` (NULL = the default
+ * stream, which is never destroyed) and frees every scratch buffer kept for it; no other thread may be launching on
+ * that stream meanwhile.  st_hip_scratch_buffer_count reports how many buffers are held in all.  No reference
+ * counterpart: the reference allocates and frees per call (crates/st-backend-hip/src/real.rs:718-756). */
+int st_hip_release_scratch(void *stream);
+size_t st_hip_scratch_buffer_count(void);
 /* Timing events recorded on the stream the kernels run on. */
 int st_hip_event_create(void **event);
 int st_hip_event_record(void *event, void *stream);

@@ -10,6 +10,6 @@ spiraltorch_amd/csrc with hipcc for gfx950.  Importing this package does not loa
 first operator call does, and raises if it is missing.
 """
 from . import hip, inputs, tensor  # noqa: F401
-from .tensor import Conv2d, PackedB, Tensor, TensorError  # noqa: F401
+from .tensor import Conv2d, LayerNorm, Linear, PackedB, Tensor, TensorError  # noqa: F401
 
-__all__ = ["hip", "inputs", "tensor", "Tensor", "TensorError", "Conv2d", "PackedB"]
+__all__ = ["hip", "inputs", "tensor", "Tensor", "TensorError", "Conv2d", "Linear", "LayerNorm", "PackedB"]

@@ -73,6 +73,8 @@ SIGNATURES = {
     "st_hip_stream_create": (c_int, [POINTER(c_void_p)]),
     "st_hip_stream_synchronize": (c_int, [c_void_p]),
     "st_hip_stream_destroy": (c_int, [c_void_p]),
+    "st_hip_release_scratch": (c_int, [c_void_p]),
+    "st_hip_scratch_buffer_count": (c_size_t, []),
     "st_hip_device_synchronize": (c_int, []),
     "st_hip_event_create": (c_int, [POINTER(c_void_p)]),
     "st_hip_event_record": (c_int, [c_void_p, c_void_p]),

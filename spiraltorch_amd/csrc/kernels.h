@@ -144,12 +144,14 @@ hipError_t launch_sum_axis0_f32(size_t rows, size_t cols, const float *in, float
 
 // One grow-only device buffer per (stream, host thread) for kernels that need scratch memory (split-k partial sums,
 // column-sum partials).  A thread's work on a stream is ordered, so two of its launches never use the buffer at the
-// same time, and threads that share a stream (the NULL stream) do not share scratch.
+// same time, and threads that share a stream (the NULL stream) do not share scratch.  A buffer whose thread has exited
+// is handed to the next thread that asks on that stream; buffers are freed when their stream is destroyed or released.
 hipError_t stream_workspace(hipStream_t stream, size_t bytes, void **out);
 // A second buffer of the same kind (slot 1) for re-laid copies of a call's operands, which must stay where they are
 // while the kernels that read them take scratch from slot 0.
 hipError_t stream_workspace_slot(hipStream_t stream, int slot, size_t bytes, void **out);
 void release_stream_workspace(hipStream_t stream);
+size_t stream_workspace_entry_count();
 // Host<->device copies made by the library, for tests that check where tensors live.
 void count_transfer(bool to_device, size_t bytes);
 

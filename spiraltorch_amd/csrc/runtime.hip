@@ -96,19 +96,55 @@ void count_transfer(bool to_device, size_t bytes)
 }
 
 namespace {
-// Scratch is keyed by (stream, host thread): launches on one stream from one thread are ordered, so they never use
-// the buffer at the same time; two host threads that share a stream (every caller that passes none shares the
+// Scratch is keyed by (stream, host thread, slot): launches on one stream from one thread are ordered, so they never
+// use the buffer at the same time; two host threads that share a stream (every caller that passes none shares the
 // NULL stream) each get a buffer of their own, so one thread growing its scratch can never free memory that a
 // kernel the other thread has just been handed is about to use.
+//
+// Lifetime: an entry lives until its stream is destroyed (st_hip_stream_destroy) or st_hip_release_scratch is called
+// for the stream.  When its host thread exits, the entry is not freed (kernels of that thread may still be queued) but
+// orphaned, and the next thread that asks for scratch on that stream and slot adopts it: work on one stream is
+// ordered and the former owner can no longer be between receiving the pointer and launching, so a pool of short-lived
+// threads keeps re-using the same few buffers instead of leaking one per thread.
 struct WorkspaceEntry {
     hipStream_t stream;
-    std::thread::id owner;
+    std::thread::id owner;  // std::thread::id() once the owning thread has exited
     void *ptr;
     size_t capacity;
     int slot;
+    bool growing;  // its owner is replacing the buffer outside the lock
 };
-std::mutex workspace_mutex;
-std::vector<WorkspaceEntry> workspace_entries;
+// Never destroyed: threads may exit (and orphan their entries) while the process is shutting down.
+std::mutex &workspace_mutex()
+{
+    static std::mutex *mutex = new std::mutex;
+    return *mutex;
+}
+std::vector<WorkspaceEntry> &workspace_entries()
+{
+    static std::vector<WorkspaceEntry> *entries = new std::vector<WorkspaceEntry>;
+    return *entries;
+}
+
+struct ThreadScratchGuard {
+    bool armed = false;
+    ~ThreadScratchGuard()
+    {
+        if (!armed) return;
+        const std::thread::id me = std::this_thread::get_id();
+        std::lock_guard<std::mutex> lock(workspace_mutex());
+        for (WorkspaceEntry &e : workspace_entries())
+            if (e.owner == me) e.owner = std::thread::id();
+    }
+};
+thread_local ThreadScratchGuard thread_scratch_guard;
+
+WorkspaceEntry *find_entry(hipStream_t stream, std::thread::id owner, int slot)
+{
+    for (WorkspaceEntry &e : workspace_entries())
+        if (e.stream == stream && e.owner == owner && e.slot == slot) return &e;
+    return nullptr;
+}
 }  // namespace
 
 hipError_t stream_workspace(hipStream_t stream, size_t bytes, void **out) { return stream_workspace_slot(stream, 0, bytes, out); }
@@ -116,47 +152,80 @@ hipError_t stream_workspace(hipStream_t stream, size_t bytes, void **out) { retu
 hipError_t stream_workspace_slot(hipStream_t stream, int slot, size_t bytes, void **out)
 {
     const std::thread::id me = std::this_thread::get_id();
-    std::lock_guard<std::mutex> lock(workspace_mutex);
-    for (WorkspaceEntry &e : workspace_entries) {
-        if (e.stream != stream || e.owner != me || e.slot != slot) continue;
-        if (e.capacity < bytes || e.ptr == nullptr) {
-            // Grow: earlier launches of this thread on this stream may still be using the old buffer.
-            hipError_t rc = hipStreamSynchronize(stream);
-            if (rc != hipSuccess) return rc;
-            if (e.ptr) {
-                rc = hipFree(e.ptr);
-                if (rc != hipSuccess) return rc;
-            }
-            e.ptr = nullptr;
-            e.capacity = 0;
-            const size_t wanted = bytes ? bytes : 256;
-            rc = hipMalloc(&e.ptr, wanted);
-            if (rc != hipSuccess) {
-                e.ptr = nullptr;
-                return rc;
-            }
-            e.capacity = wanted;
+    const size_t wanted = bytes ? bytes : 256;
+    void *old = nullptr;
+    bool adopted_or_own = false;
+    {
+        std::lock_guard<std::mutex> lock(workspace_mutex());
+        thread_scratch_guard.armed = true;
+        WorkspaceEntry *e = find_entry(stream, me, slot);
+        if (!e) {
+            e = find_entry(stream, std::thread::id(), slot);  // a buffer whose thread has exited
+            if (e) e->owner = me;
         }
-        *out = e.ptr;
-        return hipSuccess;
+        if (e) {
+            if (e->ptr != nullptr && e->capacity >= wanted) {
+                *out = e->ptr;
+                return hipSuccess;
+            }
+            // Grow: outside the lock (the wait for the stream must not stall other threads' launches).  The entry stays
+            // in the table, owned by this thread and empty, so nobody else touches it meanwhile.
+            old = e->ptr;
+            e->ptr = nullptr;
+            e->capacity = 0;
+            e->growing = true;
+            adopted_or_own = true;
+        }
     }
-    WorkspaceEntry fresh{stream, me, nullptr, bytes ? bytes : 256, slot};
-    hipError_t rc = hipMalloc(&fresh.ptr, fresh.capacity);
-    if (rc != hipSuccess) return rc;
-    workspace_entries.push_back(fresh);
-    *out = fresh.ptr;
+    if (adopted_or_own && old) {
+        // earlier launches on this stream may still be using the old buffer
+        hipError_t rc = hipStreamSynchronize(stream);
+        if (rc == hipSuccess) rc = hipFree(old);
+        if (rc != hipSuccess) {
+            std::lock_guard<std::mutex> lock(workspace_mutex());
+            if (WorkspaceEntry *e = find_entry(stream, me, slot)) e->growing = false;
+            return rc;
+        }
+    }
+    void *fresh = nullptr;
+    const hipError_t rc = hipMalloc(&fresh, wanted);
+    std::lock_guard<std::mutex> lock(workspace_mutex());
+    WorkspaceEntry *e = find_entry(stream, me, slot);
+    if (rc != hipSuccess) {
+        if (e) e->growing = false;
+        return rc;
+    }
+    if (e) {
+        e->ptr = fresh;
+        e->capacity = wanted;
+        e->growing = false;
+    } else {
+        workspace_entries().push_back(WorkspaceEntry{stream, me, fresh, wanted, slot, false});
+    }
+    *out = fresh;
     return hipSuccess;
 }
 
-// Called after the stream has been drained, before it is destroyed.
+// Called after the stream has been drained (before it is destroyed, or by st_hip_release_scratch).
 void release_stream_workspace(hipStream_t stream)
 {
-    std::lock_guard<std::mutex> lock(workspace_mutex);
-    for (size_t i = workspace_entries.size(); i-- > 0;) {
-        if (workspace_entries[i].stream != stream) continue;
-        (void)hipFree(workspace_entries[i].ptr);
-        workspace_entries.erase(workspace_entries.begin() + static_cast<long>(i));
+    std::vector<void *> doomed;
+    {
+        std::lock_guard<std::mutex> lock(workspace_mutex());
+        std::vector<WorkspaceEntry> &entries = workspace_entries();
+        for (size_t i = entries.size(); i-- > 0;) {
+            if (entries[i].stream != stream || entries[i].growing) continue;
+            if (entries[i].ptr) doomed.push_back(entries[i].ptr);
+            entries.erase(entries.begin() + static_cast<long>(i));
+        }
     }
+    for (void *ptr : doomed) (void)hipFree(ptr);
+}
+
+size_t stream_workspace_entry_count()
+{
+    std::lock_guard<std::mutex> lock(workspace_mutex());
+    return workspace_entries().size();
 }
 
 }  // namespace sthip
@@ -303,6 +372,16 @@ int st_hip_stream_destroy(void *stream)
     ST_HIP_TRY(hipStreamDestroy(as_stream(stream)), "hipStreamDestroy");
     return ST_HIP_OK;
 }
+
+int st_hip_release_scratch(void *stream)
+{
+    ST_HIP_CHECK(ensure_init());
+    ST_HIP_TRY(hipStreamSynchronize(as_stream(stream)), "hipStreamSynchronize");
+    release_stream_workspace(as_stream(stream));
+    return ST_HIP_OK;
+}
+
+size_t st_hip_scratch_buffer_count(void) { return stream_workspace_entry_count(); }
 
 int st_hip_device_synchronize(void)
 {

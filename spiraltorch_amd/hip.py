@@ -368,6 +368,15 @@ def _dev(buf):
     return buf.ptr if isinstance(buf, DeviceBuffer) else buf
 
 
+def release_scratch(stream=None) -> None:
+    """Waits for the stream (None: the default stream) and frees the scratch buffers the library keeps for it."""
+    _check(_lib.load().st_hip_release_scratch(_stream_ptr(stream)))
+
+
+def scratch_buffer_count() -> int:
+    return int(_lib.load().st_hip_scratch_buffer_count())
+
+
 def device_synchronize() -> None:
     _check(_lib.load().st_hip_device_synchronize())
 

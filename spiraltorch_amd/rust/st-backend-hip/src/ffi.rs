@@ -78,6 +78,8 @@ extern "C" {
     pub fn st_hip_stream_synchronize(stream: *mut c_void) -> c_int;
     pub fn st_hip_stream_destroy(stream: *mut c_void) -> c_int;
     pub fn st_hip_device_synchronize() -> c_int;
+    pub fn st_hip_release_scratch(stream: *mut c_void) -> c_int;
+    pub fn st_hip_scratch_buffer_count() -> usize;
     pub fn st_hip_event_create(event: *mut *mut c_void) -> c_int;
     pub fn st_hip_event_record(event: *mut c_void, stream: *mut c_void) -> c_int;
     pub fn st_hip_event_synchronize(event: *mut c_void) -> c_int;

@@ -59,6 +59,29 @@ class PackedB:
         """PackedB::from_row_major, pure.rs:1299-1316: packed[c*rows + r] = data[r*cols + c]."""
         return cls(tensor.rows, tensor.cols, np.ascontiguousarray(tensor.numpy().T).reshape(-1))
 
+    @classmethod
+    def from_tensor_on_device(cls, tensor: "Tensor") -> "PackedB":
+        """The same packing done by the GPU from the tensor's device copy (st_hip_pack_rhs_f32_dev): nothing crosses
+        the bus for a weight that already lives on the device.  The host copy is fetched only if `as_slice` asks."""
+        pack = cls(tensor.rows, tensor.cols, None)
+        try:
+            pack._dev = hip.DeviceBuffer(max(len(tensor), 1) * 4)
+            if len(tensor):
+                hip.pack_rhs_f32_dev(tensor.rows, tensor.cols, tensor._device(), pack._dev)
+        except hip.HipErr as err:
+            raise _backend_failure(err) from err
+        return pack
+
+    @classmethod
+    def from_tensor_transpose(cls, tensor: "Tensor") -> "PackedB":
+        """PackedB::from_tensor_transpose (crates/st-nn/src/module.rs:684-691): the pack of the transpose.  Packing is
+        itself a transposition, so the packed transpose of a (rows, cols) tensor is the tensor's own row-major buffer,
+        shared here, not copied."""
+        pack = cls(tensor.cols, tensor.rows, tensor._host)
+        pack._dev = tensor._dev
+        pack._source = tensor
+        return pack
+
     def inner(self) -> int:
         return self._inner
 
@@ -66,11 +89,16 @@ class PackedB:
         return self._cols
 
     def as_slice(self) -> np.ndarray:
+        if self._buf is None:
+            source = getattr(self, "_source", None)
+            self._buf = (np.array(source.data()) if source is not None
+                         else self._dev.to_array(np.float32, self._inner * self._cols))
         return self._buf
 
     def _device(self) -> hip.DeviceBuffer:
         if self._dev is None:
-            self._dev = hip.DeviceBuffer.from_array(self._buf)
+            source = getattr(self, "_source", None)
+            self._dev = source._device() if source is not None else hip.DeviceBuffer.from_array(self._buf)
         return self._dev
 
 
@@ -243,6 +271,12 @@ class Tensor:
         if residual is not None and residual.shape() != (self.rows, other.cols):
             raise TensorError("ShapeMismatch", f"left {residual.shape()} right {(self.rows, other.cols)}",
                               left=residual.shape(), right=(self.rows, other.cols))
+        # Operand checks made before the product (pure.rs:4462, 4893-4900, 5113-5120): with ReLU a NaN bias would
+        # otherwise come out as a finite 0.
+        op = label[:-len("_output")]
+        bias._require_finite(f"{op}_bias")
+        if residual is not None:
+            residual._require_finite(f"{op}_residual")
         out = Tensor._on_device_result(self.rows, other.cols)
         try:
             hip.gemm_bias_act_f32_dev(self.rows, other.cols, self.cols, activation, self._device(), other._device(),
@@ -372,6 +406,51 @@ class Tensor:
         out = self._elementwise(lambda y: hip.sum_axis0_f32_dev(self.rows, self.cols, self._device(), float(scale), y),
                                 1, self.cols)
         return np.array(out.data())
+
+    def layer_norm_affine(self, gamma: "Tensor", beta: "Tensor", epsilon: float, *,
+                          backend: Optional[str] = None) -> "Tensor":
+        """Layer normalisation over the columns with affine parameters — Tensor::layer_norm_affine_with_backend,
+        pure.rs:3702-3720; arithmetic of layer_norm_cpu, pure.rs:4008-4058."""
+        return self._layer_norm(None, gamma, beta, epsilon, backend)
+
+    def layer_norm_affine_add(self, residual: "Tensor", gamma: "Tensor", beta: "Tensor", epsilon: float, *,
+                              backend: Optional[str] = None) -> "Tensor":
+        """Layer normalisation of `self + residual` — Tensor::layer_norm_affine_add_with_backend, pure.rs:3722-3748."""
+        return self._layer_norm(residual, gamma, beta, epsilon, backend)
+
+    def _layer_norm(self, residual: Optional["Tensor"], gamma: "Tensor", beta: "Tensor", epsilon: float,
+                    backend: Optional[str]) -> "Tensor":
+        # Checks in the order of layer_norm_affine_add_impl, pure.rs:3750-3800.
+        _resolve_backend(backend)
+        if not np.isfinite(epsilon) or epsilon < 0.0:
+            raise TensorError("NonFiniteValue", f"non-finite value encountered in layernorm_epsilon: {epsilon}",
+                              label="layernorm_epsilon")
+        if self.cols == 0:
+            raise TensorError("InvalidDimensions", f"rows {self.rows} cols {self.cols}", rows=self.rows, cols=self.cols)
+        for t in (gamma, beta):
+            if t.shape() != (1, self.cols):
+                raise TensorError("ShapeMismatch", f"left {t.shape()} right {(1, self.cols)}", left=t.shape(),
+                                  right=(1, self.cols))
+        self._require_finite("layer_norm_input")
+        gamma._require_finite("layer_norm_gamma")
+        beta._require_finite("layer_norm_beta")
+        if residual is not None:
+            if residual.shape() != self.shape():
+                raise TensorError("ShapeMismatch", f"left {residual.shape()} right {self.shape()}",
+                                  left=residual.shape(), right=self.shape())
+            residual._require_finite("layer_norm_residual")
+        if self.rows == 0:
+            return Tensor.zeros(self.rows, self.cols)
+        out = self._elementwise(
+            lambda y: hip.layer_norm_f32_dev(self.rows, self.cols, self._device(),
+                                             None if residual is None else residual._device(), gamma._device(),
+                                             beta._device(), float(epsilon), y, None), self.rows, self.cols)
+        return out._validate_result("layer_norm_output")
+
+    def _sum_axis0_tensor(self, scale: float) -> "Tensor":
+        """scale · column sums as a (1, cols) tensor that stays on the device."""
+        return self._elementwise(lambda y: hip.sum_axis0_f32_dev(self.rows, self.cols, self._device(), float(scale), y),
+                                 1, self.cols)
 
     # ---- attention -------------------------------------------------------------------------------
     def scaled_dot_attention(self, keys: "Tensor", values: "Tensor", *, contexts: int, sequence: int,
@@ -508,3 +587,144 @@ class Conv2d:
     def zero_accumulators(self) -> None:
         self.weight_gradient = None
         self.bias_gradient = None
+
+
+def _accumulate(existing: Optional["Tensor"], update: "Tensor") -> "Tensor":
+    """Parameter::accumulate_euclidean (crates/st-nn/src/module.rs:329-350): the first gradient is adopted as it is
+    (on the device), later ones are added to it."""
+    if existing is None:
+        return update
+    existing.data_mut()[:] += update.data()
+    return existing
+
+
+class Linear:
+    """Fully-connected layer of crates/st-nn/src/layers/linear.rs:41-168: weight (input_dim, output_dim), bias
+    (1, output_dim), y = x·W + b.  `forward` multiplies by the weight prepacked once per parameter value
+    (Parameter::ensure_matmul_pack, crates/st-nn/src/module.rs:674) — packed on the device from the weight's device
+    copy —, `backward` returns the input gradient and accumulates the weight and bias gradients scaled by 1/batch.
+    Inputs, results and gradients stay on the device."""
+
+    def __init__(self, name: str, input_dim: int, output_dim: int):
+        if input_dim <= 0 or output_dim <= 0:
+            raise TensorError("InvalidDimensions", "input_dim and output_dim must be positive", rows=input_dim,
+                              cols=output_dim)
+        self.name = name
+        # Deterministic small parameters of Linear::new (linear.rs:56-63): 0.01, 0.02, ... accumulated in f32.
+        ramp = np.cumsum(np.full(input_dim * output_dim, 0.01, dtype=np.float32), dtype=np.float32)
+        self.weight = Tensor(input_dim, output_dim, ramp)
+        self.bias = Tensor.zeros(1, output_dim)
+        self.weight_gradient: Optional[Tensor] = None
+        self.bias_gradient: Optional[Tensor] = None
+        self._pack: Optional[PackedB] = None
+        self._pack_transpose: Optional[PackedB] = None
+        self._packed_from: Optional[Tensor] = None
+
+    def load_weight(self, weight: Tensor, bias: Optional[Tensor] = None) -> None:
+        """Parameter::load_value (module.rs:698-703): replaces the values and drops the cached packs."""
+        if weight.shape() != self.weight.shape():
+            raise TensorError("ShapeMismatch", f"left {weight.shape()} right {self.weight.shape()}",
+                              left=weight.shape(), right=self.weight.shape())
+        self.weight = weight
+        if bias is not None:
+            if bias.shape() != self.bias.shape():
+                raise TensorError("ShapeMismatch", f"left {bias.shape()} right {self.bias.shape()}",
+                                  left=bias.shape(), right=self.bias.shape())
+            self.bias = bias
+        self._pack = self._pack_transpose = self._packed_from = None
+
+    def _packs(self) -> Tuple[PackedB, PackedB]:
+        if self._packed_from is not self.weight or self._pack is None:
+            self._pack = PackedB.from_tensor_on_device(self.weight)
+            self._pack_transpose = PackedB.from_tensor_transpose(self.weight)
+            self._packed_from = self.weight
+        return self._pack, self._pack_transpose
+
+    def _validate_parameters(self) -> None:
+        self.weight._require_finite("linear_weight")
+        self.bias._require_finite("linear_bias")
+
+    @staticmethod
+    def _relabel(err: TensorError, label: str) -> TensorError:
+        if err.kind == "NonFiniteValue":  # relabel_non_finite, linear.rs:30-37
+            return TensorError("NonFiniteValue", f"non-finite value encountered in {label}", label=label)
+        return err
+
+    def forward(self, input: Tensor) -> Tensor:
+        """Linear::forward, linear.rs:87-107."""
+        if input.cols != self.weight.rows:
+            raise TensorError("ShapeMismatch", f"left {input.shape()} right {self.weight.shape()}",
+                              left=input.shape(), right=self.weight.shape())
+        input._require_finite("linear_input")
+        self._validate_parameters()
+        pack, _ = self._packs()
+        try:
+            return input.matmul_prepacked_bias(pack, self.bias)
+        except TensorError as err:
+            raise Linear._relabel(err, "linear_output") from err
+
+    def backward(self, input: Tensor, grad_output: Tensor) -> Tensor:
+        """Linear::backward, linear.rs:109-168: grad_W = inputᵀ·grad_output / batch (lhsᵀ GEMM), grad_b = column sums
+        of grad_output / batch, grad_input = grad_output·Wᵀ through the pack of the transpose."""
+        if input.rows != grad_output.rows:
+            raise TensorError("ShapeMismatch", f"left {input.shape()} right {grad_output.shape()}",
+                              left=input.shape(), right=grad_output.shape())
+        if input.cols != self.weight.rows:
+            raise TensorError("ShapeMismatch", f"left {input.shape()} right {self.weight.shape()}",
+                              left=input.shape(), right=self.weight.shape())
+        if grad_output.cols != self.weight.cols:
+            raise TensorError("ShapeMismatch", f"left {grad_output.shape()} right {(input.rows, self.weight.cols)}",
+                              left=grad_output.shape(), right=(input.rows, self.weight.cols))
+        input._require_finite("linear_backward_input")
+        grad_output._require_finite("linear_backward_grad_output")
+        self._validate_parameters()
+        if input.rows == 0:
+            return Tensor.zeros(0, input.cols)
+        scale = 1.0 / input.rows
+        steps = (("linear_weight_grad", lambda: input.matmul_lhs_transpose_scaled(grad_output, scale)),
+                 ("linear_bias_grad", lambda: grad_output._sum_axis0_tensor(scale)._validate_result("linear_bias_grad")),
+                 ("linear_input_grad", lambda: grad_output.matmul_prepacked(self._packs()[1])))
+        results = []
+        for label, run in steps:
+            try:
+                results.append(run())
+            except TensorError as err:
+                raise Linear._relabel(err, label) from err
+        grad_w, grad_b, grad_input = results
+        self.weight_gradient = _accumulate(self.weight_gradient, grad_w)
+        self.bias_gradient = _accumulate(self.bias_gradient, grad_b)
+        return grad_input
+
+    def zero_accumulators(self) -> None:
+        self.weight_gradient = None
+        self.bias_gradient = None
+
+
+class LayerNorm:
+    """LayerNorm of crates/st-nn/src/layers/normalization.rs:349-427, 1956-1969 (forward): gamma = 1 and beta = 0
+    initially, and the epsilon handed to the tensor operator is epsilon·(1 + 0.1·sqrt(−curvature))."""
+
+    def __init__(self, name: str, features: int, curvature: float, epsilon: float):
+        if features <= 0:
+            raise TensorError("InvalidDimensions", "features must be positive", rows=1, cols=features)
+        if not np.isfinite(curvature) or curvature >= 0.0:
+            raise TensorError("NonHyperbolicCurvature", f"curvature {curvature} is not negative", curvature=curvature)
+        if not np.isfinite(epsilon) or epsilon <= 0.0:
+            raise TensorError("NonFiniteValue", f"non-finite value encountered in layernorm_epsilon: {epsilon}",
+                              label="layernorm_epsilon")
+        self.name, self.features = name, int(features)
+        self.curvature, self.epsilon = float(curvature), float(epsilon)
+        self.gamma = Tensor(1, features, np.ones(features, dtype=np.float32))
+        self.beta = Tensor.zeros(1, features)
+
+    def effective_epsilon(self) -> float:
+        scale = np.sqrt(np.float32(-self.curvature))
+        return float(np.float32(self.epsilon) * (np.float32(1.0) + scale * np.float32(0.1)))
+
+    def forward(self, input: Tensor) -> Tensor:
+        if input.cols != self.features:
+            raise TensorError("ShapeMismatch", f"left {input.shape()} right {(input.rows, self.features)}",
+                              left=input.shape(), right=(input.rows, self.features))
+        if input.rows == 0:
+            return Tensor.zeros(0, input.cols)
+        return input.layer_norm_affine(self.gamma, self.beta, self.effective_epsilon())

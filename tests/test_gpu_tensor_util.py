@@ -360,3 +360,133 @@ def test_threads_sharing_the_null_stream_do_not_share_scratch(hip, oracle):
     for t in threads:
         t.join()
     assert not failures, failures
+
+
+@pytest.mark.gpu
+def test_layer_norm_through_the_tensor_mirror(hip, oracle):
+    """Tensor::layer_norm_affine[_add] (pure.rs:3702-3760) and the LayerNorm module's epsilon rule
+    (crates/st-nn/src/layers/normalization.rs:423-426) against the oracle's layer_norm_cpu restatement."""
+    import spiraltorch_amd as st
+    rng = np.random.default_rng(11)
+    for rows, cols in ((5, 3), (64, 512), (33, 777), (3, 5000)):
+        x = st.Tensor(rows, cols, rng.normal(0.3, 1.5, rows * cols).astype(np.float32))
+        res = st.Tensor(rows, cols, rng.normal(size=rows * cols).astype(np.float32))
+        gamma = st.Tensor(1, cols, rng.normal(1.0, 0.2, cols).astype(np.float32))
+        beta = st.Tensor(1, cols, rng.normal(0.0, 0.3, cols).astype(np.float32))
+        got = x.layer_norm_affine(gamma, beta, 1e-5)
+        assert got.is_device_resident()
+        assert_close(got.data(), oracle.layer_norm_f32(rows, cols, x.data(), gamma.data(), beta.data(), 1e-5),
+                     F32_REL, 2 * F32_ABS, f"layer_norm_affine {rows}x{cols}")
+        got = x.layer_norm_affine_add(res, gamma, beta, 1e-3)
+        assert_close(got.data(), oracle.layer_norm_f32(rows, cols, x.data(), gamma.data(), beta.data(), 1e-3, residual=res.data()),
+                     F32_REL, 2 * F32_ABS, f"layer_norm_affine_add {rows}x{cols}")
+    ln = st.LayerNorm("ln", 512, -1.0, 1e-5)
+    x = st.Tensor(7, 512, rng.normal(size=7 * 512).astype(np.float32))
+    want = oracle.layer_norm_f32(7, 512, x.data(), ln.gamma.data(), ln.beta.data(), ln.effective_epsilon())
+    assert_close(ln.forward(x).data(), want, F32_REL, 2 * F32_ABS, "LayerNorm::forward")
+    # an overflowing sum of squares surfaces as a non-finite result (the reference names the scalar, layer_norm_sumsq)
+    big = st.Tensor(1, 2, [np.finfo(np.float32).max, -np.finfo(np.float32).max])
+    with pytest.raises(st.TensorError, match="NonFiniteValue"):
+        big.layer_norm_affine(st.Tensor(1, 2, [1.0, 1.0]), st.Tensor.zeros(1, 2), 1e-5)
+
+
+@pytest.mark.gpu
+def test_linear_layer_forward_and_backward_stay_on_the_device(hip, oracle):
+    """Linear::forward / backward (crates/st-nn/src/layers/linear.rs:87-168) through the mirror: forward equals
+    matmul + add_row (the reference's own test, linear.rs:214-223), the gradients equal the lhs-transposed product,
+    the column sums and the product with the transposed weight, each scaled as the reference scales it; the weight is
+    packed once on the device and nothing but the inputs ever crosses the bus."""
+    import spiraltorch_amd as st
+    layer = st.Linear("fc", 3, 2)
+    x = st.Tensor(1, 3, [1.0, -2.0, 0.5])
+    expected = x.matmul(layer.weight)
+    expected.add_row_inplace(layer.bias)
+    assert (layer.forward(x).data() == expected.data()).all()
+
+    rng = np.random.default_rng(5)
+    batch, d_in, d_out = 96, 200, 72
+    layer = st.Linear("fc", d_in, d_out)
+    layer.load_weight(st.Tensor(d_in, d_out, rng.normal(0, 0.1, d_in * d_out).astype(np.float32)),
+                      st.Tensor(1, d_out, rng.normal(size=d_out).astype(np.float32)))
+    x = st.Tensor(batch, d_in, rng.normal(size=batch * d_in).astype(np.float32))
+    g = st.Tensor(batch, d_out, rng.normal(size=batch * d_out).astype(np.float32))
+    w, b = np.array(layer.weight.data()), np.array(layer.bias.data())
+
+    hip.transfer_counters(reset=True)
+    y = layer.forward(x)
+    grad_input = layer.backward(x, g)
+    moved = hip.transfer_counters()
+    assert moved["h2d_copies"] == 4                      # x, weight, bias, grad_output: once each; the pack is made on the device
+    assert moved["h2d_bytes"] == 4 * (batch * d_in + d_in * d_out + d_out + batch * d_out)
+    assert moved["d2h_copies"] == 0
+    for t in (y, grad_input, layer.weight_gradient, layer.bias_gradient):
+        assert t.is_device_resident()
+
+    want_y = oracle.gemm_f32(batch, d_out, d_in, x.data(), w).reshape(batch, d_out) + b
+    assert_close(y.data(), want_y, F32_REL, 2 * F32_ABS, "Linear::forward")
+    assert_close(layer.weight_gradient.data(), oracle.gemm_f32(d_in, d_out, batch, x.data(), g.data(), scale=1.0 / batch, lhs_transposed=True),
+                 F32_REL, 2 * F32_ABS, "linear_weight_grad")
+    assert_close(layer.bias_gradient.data(), oracle.sum_axis0_f32(batch, d_out, g.data(), 1.0 / batch), F32_REL, 2 * F32_ABS,
+                 "linear_bias_grad")
+    w_t = np.ascontiguousarray(w.reshape(d_in, d_out).T)
+    assert_close(grad_input.data(), oracle.gemm_f32(batch, d_in, d_out, g.data(), w_t), F32_REL, 2 * F32_ABS, "linear_input_grad")
+
+    # a second forward re-uses the pack: nothing is uploaded
+    hip.transfer_counters(reset=True)
+    again = layer.forward(x)
+    assert hip.transfer_counters()["h2d_copies"] == 0
+    assert (again.data() == y.data()).all()
+    # a second backward accumulates (Parameter::accumulate_euclidean)
+    first = np.array(layer.weight_gradient.data())
+    layer.backward(x, g)
+    assert_close(layer.weight_gradient.data(), 2 * first, 1e-6, 1e-7, "accumulated weight gradient")
+    # an overflowing product is reported under the layer's label (relabel_non_finite, linear.rs:30-37, test :319-333)
+    tiny = st.Linear("fc", 1, 1)
+    tiny.weight.data_mut()[0] = np.finfo(np.float32).max
+    with pytest.raises(st.TensorError) as info:
+        tiny.backward(st.Tensor(1, 1, [0.0]), st.Tensor(1, 1, [2.0]))
+    assert info.value.fields["label"] == "linear_input_grad"
+
+
+@pytest.mark.gpu
+def test_scratch_of_exited_threads_is_reused_not_leaked(hip, oracle):
+    """Scratch buffers are kept per (stream, host thread); a thread that exits leaves its buffer to the next thread
+    that launches on the stream, so a pool of short-lived threads on the default stream holds a bounded number of
+    buffers, and st_hip_release_scratch frees them."""
+    import threading
+    rows, cols = 4096, 96
+    x = np.random.default_rng(21).normal(size=rows * cols).astype(np.float32)
+    want = oracle.sum_axis0_f32(rows, cols, x)
+    d_x = hip.DeviceBuffer.from_array(x)
+    hip.release_scratch(None)
+    before = hip.scratch_buffer_count()
+    results, errors = [], []
+
+    def work():
+        try:
+            d_out = hip.DeviceBuffer(cols * 4)
+            hip.sum_axis0_f32_dev(rows, cols, d_x, 1.0, d_out)   # column sums keep their partials in scratch
+            hip.device_synchronize()
+            results.append(d_out.to_array(np.float32, cols))
+        except Exception as err:  # surfaced below: an exception in a thread would otherwise pass silently
+            errors.append(err)
+
+    for _ in range(12):                  # one after the other: each thread has exited before the next starts
+        t = threading.Thread(target=work)
+        t.start()
+        t.join()
+    assert not errors, errors
+    assert hip.scratch_buffer_count() <= before + 1, "every short-lived thread left a buffer behind"
+    for got in results:
+        assert_close(got, want, F32_REL, 1e-3, "column sums from a short-lived thread")
+    threads = [threading.Thread(target=work) for _ in range(4)]   # concurrent threads do not share a buffer
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    assert hip.scratch_buffer_count() <= before + 4
+    for got in results[-4:]:
+        assert_close(got, want, F32_REL, 1e-3, "column sums from concurrent threads")
+    hip.release_scratch(None)
+    assert hip.scratch_buffer_count() == before
