@@ -48,6 +48,16 @@ __device__ __forceinline__ float relu_or_identity(float value, bool relu)
 __device__ __forceinline__ float sum4(const float4 &v) { return (v.x + v.y) + (v.z + v.w); }
 __device__ __forceinline__ float sumsq4(const float4 &v) { return fmaf(v.x, v.x, v.y * v.y) + fmaf(v.z, v.z, v.w * v.w); }
 
+// sqrt(var + epsilon) of a layer-norm row.  The reference fails a row whose sums, variance or denominator overflow
+// (labels layer_norm_sumsq … layer_norm_denom, crates/st-tensor/src/pure.rs:4030-4045); an infinite denominator would
+// instead turn the whole row into finite zeros here, so it becomes NaN and the caller's finite check on the result
+// reports the row.  Finite denominators pass through unchanged.
+__device__ __forceinline__ float layer_norm_denominator(float var, float epsilon)
+{
+    const float denom = sqrtf(var + epsilon);
+    return denom < INFINITY ? denom : NAN;
+}
+
 // Runs `body(act, has_residual)` with the activation as a callable and the presence of a residual as a compile-time
 // constant, chosen once from the (wavefront-uniform) launch arguments: an epilogue that decides them per element
 // compiles to a chain of scalar branches around every store.

@@ -972,7 +972,7 @@ __device__ __forceinline__ void gemm_bf16_rowcomplete_body(const RowLnArgs &q)
         const float cols_f = static_cast<float>(N);
         const float mean = sum / cols_f;
         const float var = fmaxf(sumsq / cols_f - mean * mean, 0.0f);
-        const float denom = sqrtf(var + q.epsilon);
+        const float denom = layer_norm_denominator(var, q.epsilon);
         // (v - mean) / denom with one division per row: the product with the reciprocal, corrected once by its exact
         // remainder, is the correctly rounded quotient (the stand-alone layer-norm kernel does the same).
         const float inv = 1.0f / denom;

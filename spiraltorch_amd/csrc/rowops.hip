@@ -36,7 +36,7 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(int rows, int cols, con
     const float cols_f = static_cast<float>(cols);
     const float mean = sum / cols_f;
     const float var = fmaxf(sumsq / cols_f - mean * mean, 0.0f);
-    const float denom = sqrtf(var + epsilon);
+    const float denom = layer_norm_denominator(var, epsilon);
     for (int c = lane; c < cols; c += 64) {
         float v = x[offset + c];
         if (residual) v += residual[offset + c];
@@ -100,7 +100,7 @@ __global__ __launch_bounds__(256) void layer_norm_vec_kernel(int rows, int cols,
         sumsq = wave_sum(sumsq);
         const float mean = sum / cols_f;
         const float var = fmaxf(sumsq / cols_f - mean * mean, 0.0f);
-        const float denom = sqrtf(var + epsilon);
+        const float denom = layer_norm_denominator(var, epsilon);
         // (v - mean) / denom for every element, with one real division per row: the product with the correctly rounded
         // reciprocal, corrected once by its exact remainder (two fused multiply-adds), is the correctly rounded quotient
         // again, i.e. bit for bit what the division gives; only the last bit matters here, because it decides some of
@@ -201,7 +201,7 @@ __global__ __launch_bounds__(1024) void layer_norm_block_kernel(int cols, const 
     const float cols_f = static_cast<float>(cols);
     const float mean = sum / cols_f;
     const float var = fmaxf(sumsq / cols_f - mean * mean, 0.0f);
-    const float denom = sqrtf(var + epsilon);
+    const float denom = layer_norm_denominator(var, epsilon);
     const float inv = 1.0f / denom;
     auto quotient = [&](float a) {  // a / denom, correctly rounded (see layer_norm_vec_kernel)
         const float q = a * inv;
@@ -276,7 +276,7 @@ __global__ __launch_bounds__(THREADS) void layer_norm_long_kernel(int cols, cons
     const float cols_f = static_cast<float>(cols);
     const float mean = sum / cols_f;
     const float var = fmaxf(sumsq / cols_f - mean * mean, 0.0f);
-    const float denom = sqrtf(var + epsilon);
+    const float denom = layer_norm_denominator(var, epsilon);
     const float inv = 1.0f / denom;
     auto quotient = [&](float a) {  // a / denom, correctly rounded (see layer_norm_vec_kernel)
         const float q = a * inv;
