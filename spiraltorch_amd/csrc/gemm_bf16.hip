@@ -1293,6 +1293,53 @@ __device__ __forceinline__ void persistent_epilogue_bf16(const GemmBf16Args &p, 
     }
 }
 
+// The same for f32 output: the wavefront's 64×64 accumulators leave in two passes of 32 rows through the same 8 KB
+// strip (32 rows × 256 B; the 16-byte chunk q of row r sits at chunk q ^ (r & 15), which spreads the eight rows a
+// 128-bit write touches per cycle and the sixteen chunks of a row a read touches over all banks), are read back
+// row-contiguous — sixteen lanes per row, 128 bits each — and stored as whole 256-byte row segments.  Scale, bias and
+// activation are applied after the read-back, where a lane keeps the same four columns for all rows.
+template <int ACT>
+__device__ __forceinline__ void persistent_epilogue_f32(const GemmBf16Args &p, const f32x16 (&acc)[2][2], unsigned char *strip,
+                                                        int row_first, int col_base, int lane)
+{
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    const int li = lane & 31, lh = lane >> 5;
+    const float scale = p.scale;
+    const bool has_bias = p.bias != nullptr;
+    const __amdgpu_buffer_rsrc_t rsrc_bias = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float *>(p.bias), 0, has_bias ? static_cast<int>(static_cast<unsigned>(p.N) * 4u) : 0, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_c = __builtin_amdgcn_make_buffer_rsrc(
+        p.C32, 0, static_cast<int>(static_cast<unsigned>(p.M) * static_cast<unsigned>(p.N) * 4u), 0x00020000);
+    const int piece = lane & 15, sub_row = lane >> 4;
+    f32x4 bias4 = {-0.0f, -0.0f, -0.0f, -0.0f};  // x + -0.0f == x for every x
+    if (has_bias)
+        bias4 = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_bias, static_cast<unsigned>(col_base + piece * 4) * 4u, 0, 0));
+#pragma unroll
+    for (int tm = 0; tm < 2; ++tm) {
+#pragma unroll
+        for (int tn = 0; tn < 2; ++tn)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int q = tn * 8 + g * 2 + lh;
+                *reinterpret_cast<f32x4 *>(strip + li * 256 + ((q ^ (li & 15)) << 4)) =
+                    f32x4{acc[tm][tn][4 * g], acc[tm][tn][4 * g + 1], acc[tm][tn][4 * g + 2], acc[tm][tn][4 * g + 3]};
+            }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int local_row = j * 4 + sub_row;
+            f32x4 v = *reinterpret_cast<const f32x4 *>(strip + local_row * 256 + ((piece ^ (local_row & 15)) << 4));
+            v = v * scale + bias4;
+            v.x = activate<ACT>(v.x);
+            v.y = activate<ACT>(v.y);
+            v.z = activate<ACT>(v.z);
+            v.w = activate<ACT>(v.w);
+            __builtin_amdgcn_raw_buffer_store_b128(
+                __builtin_bit_cast(u32x4, v), rsrc_c,
+                (static_cast<unsigned>(row_first + tm * 32 + local_row) * static_cast<unsigned>(p.N) + col_base + piece * 4) * 4u, 0, 0);
+        }
+    }
+}
+
 // The lane index, from the hardware and opaque to the compiler: what is computed from it can neither be hoisted out of
 // a loop nor has an input that must stay in a register until then.
 __device__ __forceinline__ int fresh_lane_index()
@@ -1314,7 +1361,8 @@ __device__ __forceinline__ int fresh_lane_index()
 // and 32 KB beside the stages (wavefronts 4-7).  Layout, swizzle, fragment reads and issue order of the main loop
 // are those of the packed kernel above.
 // -------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(768) void gemm_bf16_persistent_256x128_kernel(GemmBf16Args p)
+template <bool OUT32>
+__device__ __forceinline__ void gemm_bf16_persistent_body(const GemmBf16Args &p)
 {
     constexpr int BM = 256, BN = 128, BK = 64;
     constexpr int WTM = 64, WTN = 64, TM = 2, TN = 2;
@@ -1514,10 +1562,12 @@ __global__ __launch_bounds__(768) void gemm_bf16_persistent_256x128_kernel(GemmB
             substep(1, true, a_stage, b_stage, 2);
             substep(0, true, a_stage, b_stage, 3);
             barrier();  // everyone has read k-tile f; k-tile f+1 has landed
-            if (kt + 1 < steps) {
-                substep(1, true, a_next, b_stage ^ 1, 0);
-            } else {
-                substep(1, false, 0, 0, 0);
+            // The last sub-step is the same code for every k-tile, fragment reads of the following k-tile included (after
+            // a tile's last k-tile they fetch the next tile's first fragments, which the epilogue path below fetches again:
+            // an arm of the branch that ends in MFMAs of its own made the compiler carry both arms' fragment registers
+            // through the epilogue, spill them there and reload them behind the tile's stores).
+            substep(1, true, a_next, b_stage ^ 1, 0);
+            if (kt + 1 == steps) {
                 // Strips: wavefronts 0-3 in the A stage this tile finished in, 4-7 beside the stages.
                 unsigned char *strips = wave < 4 ? lds_bytes + a_stage * A_STAGE : lds_bytes + SPARE - 4 * (TM * 32 * WTN * 2);
                 const int row_first = m0 + wm * WTM, col_base = n0 + wn * WTN;
@@ -1525,26 +1575,29 @@ __global__ __launch_bounds__(768) void gemm_bf16_persistent_256x128_kernel(GemmB
                 // would stay in registers through the main loop, which has none to spare with three wavefronts on every SIMD.)
                 const int lane_now = fresh_lane_index();
                 unsigned char *strip = strips + wave * (TM * 32 * WTN * 2);
-                if (p.activation == ST_HIP_ACT_GELU) persistent_epilogue_bf16<ST_HIP_ACT_GELU>(p, acc, strip, row_first, col_base, lane_now);
-                else if (p.activation == ST_HIP_ACT_RELU) persistent_epilogue_bf16<ST_HIP_ACT_RELU>(p, acc, strip, row_first, col_base, lane_now);
-                else persistent_epilogue_bf16<ST_HIP_ACT_NONE>(p, acc, strip, row_first, col_base, lane_now);
+                if constexpr (OUT32) {
+                    if (p.activation == ST_HIP_ACT_GELU) persistent_epilogue_f32<ST_HIP_ACT_GELU>(p, acc, strip, row_first, col_base, lane_now);
+                    else if (p.activation == ST_HIP_ACT_RELU) persistent_epilogue_f32<ST_HIP_ACT_RELU>(p, acc, strip, row_first, col_base, lane_now);
+                    else persistent_epilogue_f32<ST_HIP_ACT_NONE>(p, acc, strip, row_first, col_base, lane_now);
+                } else {
+                    if (p.activation == ST_HIP_ACT_GELU) persistent_epilogue_bf16<ST_HIP_ACT_GELU>(p, acc, strip, row_first, col_base, lane_now);
+                    else if (p.activation == ST_HIP_ACT_RELU) persistent_epilogue_bf16<ST_HIP_ACT_RELU>(p, acc, strip, row_first, col_base, lane_now);
+                    else persistent_epilogue_bf16<ST_HIP_ACT_NONE>(p, acc, strip, row_first, col_base, lane_now);
+                }
                 clear();
                 if (j + 1 < my_tiles) barrier();  // the strips are done with: the A stage may be refilled
                 // (Unconditional — after the last tile they read a stage nobody uses any more — so that nothing of the
                 // old fragments has to survive the epilogue.)
                 fragment_addresses();
                 first_fragments(a_next, b_stage ^ 1);
-#pragma unroll
-                for (int u = 0; u < 2; ++u) {  // (the other fragment buffer starts a new life too, for the same reason)
-                    asm volatile("" : "=v"(fa[1][u]));
-                    asm volatile("" : "=v"(fb[1][u]));
-                }
             }
             a_stage = a_next;
         }
     }
 }
 
+__global__ __launch_bounds__(768) void gemm_bf16_persistent_256x128_kernel(GemmBf16Args p) { gemm_bf16_persistent_body<false>(p); }
+__global__ __launch_bounds__(768) void gemm_bf16_persistent_256x128_f32out_kernel(GemmBf16Args p) { gemm_bf16_persistent_body<true>(p); }
 
 // -------------------------------------------------------------------------------------------------
 // Skinny kernel (M <= 64, decode-like): HBM-bound on B, so the job is to keep many bytes of B in flight
@@ -2179,7 +2232,7 @@ hipError_t launch_persistent_256x128(GemmBf16Args args, hipStream_t stream)
     const unsigned grid = static_cast<unsigned>(std::min<size_t>(tiles, 256));
     args.swizzle = (tiles % 8 == 0 && grid % 8 == 0) ? 1 : 0;
     constexpr size_t lds_bytes = 3 * 32768 + 2 * 16384 + 32768;  // three A stages, two B stages, strips of four wavefronts
-    auto kernel = gemm_bf16_persistent_256x128_kernel;
+    auto kernel = args.C32 ? gemm_bf16_persistent_256x128_f32out_kernel : gemm_bf16_persistent_256x128_kernel;
     hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
     if (rc != hipSuccess) return rc;
@@ -2474,6 +2527,14 @@ hipError_t launch_gemm_bf16(size_t m, size_t n, size_t k, const uint16_t *lhs, c
         // 36.8).  Where the plan is 256×256 tiles they stay ahead (16384×2048×512: 48.2 µs against 51.8).
         if (narrow && rhs_packed && out_f32 == nullptr && out_bf16 != nullptr && aligned16(out_bf16) && epilogue.residual == nullptr &&
             m % 256 == 0 && (m / 256) * (n / 128) > 256 && m * n * 2 < (1ull << 31))
+            return launch_persistent_256x128(args, stream);
+        // f32 as the only output, a short k and at least four rounds of 256×128 tiles: the same kernel with an f32
+        // epilogue — a tile's stores drain under the next tile's main loop (16384×4096×512: 89 µs against 95).  With a
+        // long k the 256×256 tiles' main loop (a third less LDS traffic per flop) is worth more than the overlap: 4096³
+        // as 512 tiles of 256×128, two per workgroup, measured 115.6 µs here against 110.0 µs, 8192×8192×4096 483 against
+        // 433 µs, and 4096×4096×1024 42.8 against 38.5 µs.
+        if (rhs_packed && out_f32 != nullptr && out_bf16 == nullptr && epilogue.residual == nullptr && m % 256 == 0 &&
+            k <= 512 && (m / 256) * (n / 128) >= 1024 && m * n * 4 < (1ull << 32))
             return launch_persistent_256x128(args, stream);
         if (narrow) return launch_256<128>(args, rhs_packed, stream, workspace_offset);
         return launch_256<256>(args, rhs_packed, stream, workspace_offset);

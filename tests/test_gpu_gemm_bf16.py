@@ -493,3 +493,31 @@ def test_validation(hip):
     with pytest.raises(hip.HipErr, match="lhs buffer length 4 does not match m\\*k=6"):
         hip.gemm_bf16_f32acc(2, 2, 3, np.zeros(4, np.uint16), np.zeros(6, np.uint16), out)
     assert (out == 13.0).all()
+
+
+@pytest.mark.parametrize("m,n,k,activation", [(16384, 4096, 512, 0), (2048, 16384, 128, 2), (4096, 8192, 320, 1)])
+def test_prepacked_f32_output_over_many_rounds_of_tiles_with_a_short_k(hip, oracle, m, n, k, activation):
+    """At least 1024 tiles of 256×128, k up to 512, f32 the only output: the persistent kernel with its f32 epilogue.
+    Bit for bit what the same call returns when it also asks for the bf16 output (which takes the one-tile-per-workgroup
+    kernel: same products added in the same order), with and without a bias; sampled rows against the oracle."""
+    rng = np.random.default_rng(2 * m + 3 * n + 5 * k)
+    a, b = bf16_pair(rng, m, n, k, std=0.5)
+    bias = rng.normal(size=n).astype(np.float32)
+    d_a, d_bias = hip.DeviceBuffer.from_array(a), hip.DeviceBuffer.from_array(bias)
+    d_packed = hip.DeviceBuffer.from_array(np.ascontiguousarray(b.reshape(k, n).T))
+    d32, d32_ref, d16 = hip.DeviceBuffer(m * n * 4), hip.DeviceBuffer(m * n * 4), hip.DeviceBuffer(m * n * 2)
+    for use_bias in (True, False):
+        d32.zero()
+        hip.gemm_bf16_prepacked_bias_act_dev(m, n, k, activation, d_a, d_packed, d_bias if use_bias else None, None, d32_ref, d16)
+        hip.gemm_bf16_prepacked_bias_act_dev(m, n, k, activation, d_a, d_packed, d_bias if use_bias else None, None, d32, None)
+        hip.device_synchronize()
+        got = d32.to_array(np.float32, m * n)
+        assert (got.view(np.uint32) == d32_ref.to_array(np.float32, m * n).view(np.uint32)).all(), f"bias={use_bias}"
+    rows = sorted(set([0, 1, 255, 256, m // 2 + 3, m - 257, m - 1]))
+    base = oracle.gemm_bf16_f32acc(len(rows), n, k, a.reshape(m, k)[rows].ravel(), b, threads=8).astype(np.float64).reshape(len(rows), n)
+    want = base  # the last call ran without a bias
+    if activation == 1:
+        want = np.maximum(want, 0.0)
+    elif activation == 2:
+        want = 0.5 * want * (1.0 + np.tanh(0.7978846 * (want + 0.044715 * want ** 3)))
+    assert_close(got.reshape(m, n)[rows].ravel(), want.ravel(), BF16_REL, 2e-5 * max(1.0, float(np.abs(base).max())), "sampled rows")
