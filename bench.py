@@ -184,6 +184,27 @@ def wl_conv2d(hip, inputs, timer):
         (x, wt, b, geom, (batch, c_in, h, w, c_out))
 
 
+def wl_conv2d_bf16(hip, inputs, timer):
+    """Config 2's layer on bf16-rounded operands (bf16 NCHW images and OIHW weights, f32 accumulation, f32 output): the
+    implicit GEMM on the bf16 matrix cores, priced against the bf16 peak.  The timed step includes the copy of the images
+    into the padded channels-last layout the kernel works on and the re-layout of the weights."""
+    batch, c_in, h, w, c_out = 32, 64, 56, 56, 128
+    x = inputs.to_bf16(inputs.normal(inputs.seed_for(2, 0), batch * c_in * h * w))
+    wt = inputs.to_bf16(inputs.normal(inputs.seed_for(2, 1), c_out * c_in * 9, 0.0, math.sqrt(2.0 / (c_in * 9))))
+    b = inputs.uniform(inputs.seed_for(2, 2), c_out, -0.1, 0.1)
+    d_x, d_w, d_b = (hip.DeviceBuffer.from_array(a) for a in (x, wt, b))
+    d_out = hip.DeviceBuffer(batch * c_out * h * w * 4)
+    geom = ((3, 3), (1, 1), (1, 1), (1, 1))
+
+    def step(stream):
+        hip.conv2d_bias_act_bf16_dev(batch, c_in, h, w, c_out, *geom, 1, d_x, d_w, d_b, d_out, None, stream)
+
+    wall, ev, sus = timer.measure(step)
+    flops = 2 * batch * c_out * h * w * c_in * 9
+    bytes_ = 2 * (x.size + wt.size) + 4 * (b.size + batch * c_out * h * w)
+    return entry("conv2d_bias_relu_bf16_f32acc_n32_c64to128_56x56_k3s1p1", "bf16", flops, bytes_, "mfma", wall, ev, sustained=sus)
+
+
 def wl_conv2d_backward(hip, inputs, timer, which):
     """Gradients of config 2's convolution: grad_input (adjoint convolution) or grad_weight (reduction over
     batch and pixels); both cost the forward's FLOPs."""
@@ -575,6 +596,7 @@ def main():
         ("attention_bf16", lambda: wl_attention_bf16(hip, inputs, timer)),
         ("gemm_f32_conv_equivalent", lambda: wl_gemm_f32(hip, inputs, timer, 100352, 128, 576,
                                                          "gemm_f32_100352x128x576_conv_equivalent")),
+        ("conv2d_bf16", lambda: wl_conv2d_bf16(hip, inputs, timer)),
         ("conv2d_grad_input", lambda: wl_conv2d_backward(hip, inputs, timer, "grad_input")),
         ("conv2d_grad_weight", lambda: wl_conv2d_backward(hip, inputs, timer, "grad_weight")),
         ("attention_bias", lambda: [wl_attention_bias(hip, inputs, timer, 1, 2048), wl_attention_bias(hip, inputs, timer, 16, 1024)]),
@@ -607,6 +629,8 @@ def main():
         for item in rows + extras:
             if item["workload"] in per_workload:
                 item["cpu_baseline"] = per_workload[item["workload"]]
+            elif item["workload"].startswith("conv2d_bias_relu_bf16"):
+                item["cpu_baseline"] = dict(cpu, sample="the f32 pass of the same layer (the port computes bf16 operands in f32)")
             elif item["workload"].startswith("conv2d_grad"):
                 item["cpu_baseline"] = dict(cpu, sample="forward pass of the same layer (the backward runs the same contraction sizes)")
     for item in rows + extras:

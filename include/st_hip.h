@@ -282,6 +282,18 @@ int st_hip_conv2d_bias_act_f32_dev(size_t batch, size_t c_in, size_t h, size_t w
                                    size_t pad_h, size_t pad_w, size_t dil_h, size_t dil_w,
                                    int activation, const float *input, const float *weight,
                                    const float *bias, float *out, void *stream);
+/* Conv2d::forward (+ bias, + optional activation) on bf16 operands — the arithmetic of
+ * crates/st-nn/src/layers/conv.rs:685-748, 2559-2599 with the image (NCHW) and the weight (OIHW) stored as bf16 bit
+ * patterns, products accumulated in f32, f32 bias (or NULL), and the NCHW result written as f32 to out_f32 and/or rounded
+ * nearest-even to bf16 into out_bf16 (either may be NULL, not both).  The reference has no bf16 path; this is the conv
+ * counterpart of st_hip_gemm_bf16_bias_act_dev.  Any geometry the f32 entry point takes; the padded channels-last copy
+ * of the input that the kernel works on (batch·(h+2·pad_h)·(w+2·pad_w)·ceil64(c_in)·2 bytes, in the stream's scratch)
+ * must stay below 2 GiB, out_f32 must be 16-byte and out_bf16 8-byte aligned: otherwise ST_HIP_ERR_UNSUPPORTED. */
+int st_hip_conv2d_bias_act_bf16_dev(size_t batch, size_t c_in, size_t h, size_t w, size_t c_out,
+                                    size_t kh, size_t kw, size_t stride_h, size_t stride_w,
+                                    size_t pad_h, size_t pad_w, size_t dil_h, size_t dil_w,
+                                    int activation, const uint16_t *input, const uint16_t *weight,
+                                    const float *bias, float *out_f32, uint16_t *out_bf16, void *stream);
 /* The three gradients of Conv2d::backward one by one (conv.rs:791-809); grad_weight and grad_bias are
  * multiplied by `scale` (the reference passes 1/batch). */
 int st_hip_conv2d_grad_input_f32_dev(size_t batch, size_t c_in, size_t h, size_t w, size_t c_out,

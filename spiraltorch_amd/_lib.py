@@ -113,6 +113,8 @@ SIGNATURES = {
     "st_hip_pack_rhs_bf16_dev": (c_int, [c_size_t, c_size_t, c_void_p, c_void_p, c_void_p]),
     "st_hip_conv2d_bias_act_f32_dev": (c_int, [c_size_t] * 13 + [c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                                                  c_void_p]),
+    "st_hip_conv2d_bias_act_bf16_dev": (c_int, [c_size_t] * 13 + [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                                                  c_void_p]),
     "st_hip_attention_f32_dev": (c_int, [c_size_t, c_size_t, c_size_t, c_float, c_int, c_void_p, c_void_p, c_void_p,
                                          c_void_p, c_void_p, c_void_p, c_void_p]),
     "st_hip_attention_bf16_dev": (c_int, [c_size_t, c_size_t, c_size_t, c_size_t, c_float, c_int, c_void_p, c_void_p,

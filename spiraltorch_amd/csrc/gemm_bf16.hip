@@ -24,6 +24,19 @@ namespace sthip {
 
 namespace {
 
+// Geometry of a convolution run as a GEMM with M = c_out, N = batch·oh·ow output pixels and K = kh·kw·c_pad, k ordered
+// (ky, kx, channel): a 64-wide k-tile is one tap and 64 consecutive channels, i.e. one contiguous 128-byte piece of the
+// channels-last image copy for every output pixel.
+struct ConvBf16Geometry {
+    int ohow, ow;          // output plane
+    int hp, wp, c_pad;     // padded image copy: hp × wp positions of c_pad channels (a multiple of 64)
+    int stride_h, stride_w, dil_h, dil_w;
+    int kw;                // taps per kernel row
+    int c_blocks;          // c_pad / 64: k-tiles per tap
+    int c_out;
+    unsigned image_bytes;  // bytes of the whole padded copy (the buffer range of operand B)
+};
+
 struct GemmBf16Args {
     const uint16_t *A;
     const uint16_t *B;
@@ -42,6 +55,9 @@ struct GemmBf16Args {
     int k_splits = 1;
     int tiles_per_split = 0;
     float *partial = nullptr;
+    // Convolution form of the packed kernels (CONV = true): A is the weight matrix re-laid as (c_out, kh·kw·c_pad), B the
+    // zero-padded channels-last copy of the images, addressed per output pixel — see conv_bf16 below.
+    ConvBf16Geometry conv = {};
 };
 
 typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
@@ -522,6 +538,75 @@ __device__ __forceinline__ void gemm_bf16_epilogue(const GemmBf16Args &p, const 
     else gemm_bf16_epilogue_rows<WTN, TM, ST_HIP_ACT_NONE>(p, acc, lds, wave, row_first, col_base, lane);
 }
 
+// Epilogue of the convolution form: rows of C are output channels, columns output pixels (image-major), and the result
+// goes to NCHW — channel o of image i is the contiguous run out[(i·c_out + o)·oh·ow ..].  Same f32 strips through LDS as
+// above; a lane's four neighbouring columns are four consecutive pixels, stored as one 16-byte (f32) / 8-byte (bf16)
+// access when the plane size is a multiple of four (then they share an image and the address is aligned), one by one
+// otherwise.  The bias is per row.
+template <int WTN, int TM>
+__device__ __forceinline__ void conv_bf16_epilogue(const GemmBf16Args &p, const f32x16 (&acc)[TM][WTN / 32], unsigned char *lds,
+                                                   int wave, int row_first, int col_base, int lane)
+{
+    constexpr int TN = WTN / 32;
+    const int li = lane & 31, lh = lane >> 5;
+    const int M = p.M, N = p.N;
+    constexpr int C_STRIDE = WTN + 4;
+    float *strip = reinterpret_cast<float *>(lds) + wave * (32 * C_STRIDE);
+    constexpr int LPR = WTN / 4;
+    constexpr int ROWS_PER_PASS = 64 / LPR;
+    constexpr int PASSES = 32 / ROWS_PER_PASS;
+    const int ohow = p.conv.ohow;
+    const int pixel0 = col_base + (lane & (LPR - 1)) * 4;  // this lane's four pixels in the read-back phase
+    const bool vector_ok = (ohow & 3) == 0;
+    // image and position of each of the four pixels (the same for every row this lane stores)
+    size_t plane_off[4];
+    bool live[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const int pixel = pixel0 + e;
+        live[e] = pixel < N;
+        const int image = pixel / ohow;
+        plane_off[e] = static_cast<size_t>(image) * p.conv.c_out * ohow + (pixel - image * ohow);
+    }
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) {
+        const int row_base = row_first + tm * 32;
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn) {
+            const f32x16 tile = acc[tm][tn];
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+                *reinterpret_cast<float4 *>(&strip[li * C_STRIDE + tn * 32 + g * 8 + lh * 4]) =
+                    make_float4(tile[4 * g], tile[4 * g + 1], tile[4 * g + 2], tile[4 * g + 3]);
+        }
+#pragma unroll
+        for (int j = 0; j < PASSES; ++j) {
+            const int local_row = j * ROWS_PER_PASS + lane / LPR;
+            const int row = row_base + local_row;  // output channel
+            const float4 s4 = *reinterpret_cast<const float4 *>(&strip[local_row * C_STRIDE + (lane & (LPR - 1)) * 4]);
+            if (row >= M || !live[0]) continue;
+            const float bias = p.bias ? p.bias[row] : -0.0f;
+            float v[4] = {s4.x, s4.y, s4.z, s4.w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = apply_activation(v[e] + bias, p.activation);
+            const size_t channel_off = static_cast<size_t>(row) * ohow;
+            if (vector_ok) {
+                const size_t idx = plane_off[0] + channel_off;
+                if (p.C32) *reinterpret_cast<float4 *>(p.C32 + idx) = make_float4(v[0], v[1], v[2], v[3]);
+                if (p.C16) *reinterpret_cast<uint2 *>(p.C16 + idx) = make_uint2(pack_bf16x2_rne(v[0], v[1]), pack_bf16x2_rne(v[2], v[3]));
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    if (!live[e]) continue;
+                    const size_t idx = plane_off[e] + channel_off;
+                    if (p.C32) p.C32[idx] = v[e];
+                    if (p.C16) p.C16[idx] = f32_to_bf16_rne(v[e]);
+                }
+            }
+        }
+    }
+}
+
 // Epilogue of a 256-row kernel's workgroup: the launch's own, or — when k is split over workgroups — the raw sums of
 // this split into its plane of the partial buffer (the reduction kernel applies scale, bias, residual and activation).
 template <int WTN, int TM>
@@ -559,7 +644,7 @@ __device__ __forceinline__ void gemm_bf16_finish(const GemmBf16Args &p, int spli
 // -------------------------------------------------------------------------------------------------
 #define ST_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
 
-template <int BN, int WAVES, int BM = 256>
+template <int BN, int WAVES, int BM = 256, bool CONV = false>
 __device__ __forceinline__ void gemm_bf16_packed_body(const GemmBf16Args &p)
 {
     static_assert(BN == 256 || BN == 128, "tile width");
@@ -602,7 +687,8 @@ __device__ __forceinline__ void gemm_bf16_packed_body(const GemmBf16Args &p)
     const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint16_t *>(p.A), 0, static_cast<int>(static_cast<unsigned>(M) * static_cast<unsigned>(K) * 2u), 0x00020000);
     const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint16_t *>(p.B), 0, static_cast<int>(static_cast<unsigned>(K) * static_cast<unsigned>(N) * 2u), 0x00020000);
+        const_cast<uint16_t *>(p.B), 0,
+        static_cast<int>(CONV ? p.conv.image_bytes : static_cast<unsigned>(K) * static_cast<unsigned>(N) * 2u), 0x00020000);
 
     // Direct loads: instruction r of wavefront w fills rows (r*WAVES + w)*8 .. +7 of a stage (1 KB of LDS, lane l at
     // chunk position l&7 of row l>>3), so lane l fetches logical chunk (l&7) ^ swz(row), swz(r) = ((r>>1) ^ (r>>4)) & 7.
@@ -616,9 +702,35 @@ __device__ __forceinline__ void gemm_bf16_packed_body(const GemmBf16Args &p)
         for (int r = 0; r < NMAX; ++r) {
             const int chunk = ((lane & 7) ^ sw_base ^ ((r * WAVES / 2) & 7)) & 7;
             if (r < NA) a_off[r] = (static_cast<unsigned>(m0 + r * WAVES * 8 + row_in) * K + k_first + chunk * 8) * 2u;
-            if (r < NB) b_off[r] = (static_cast<unsigned>(n0 + r * WAVES * 8 + row_in) * K + k_first + chunk * 8) * 2u;
+            if (r < NB) {
+                if constexpr (CONV) {
+                    // Row n of operand B is output pixel n: its 128-byte pieces start at the pixel's first tap in the
+                    // padded channels-last copy.  (Pixels past the end repeat the last one; they are never stored.)
+                    const int pixel = min(n0 + r * WAVES * 8 + row_in, N - 1);
+                    const int image = pixel / p.conv.ohow, rest = pixel - image * p.conv.ohow;
+                    const int oy = rest / p.conv.ow, ox = rest - oy * p.conv.ow;
+                    const unsigned position = (static_cast<unsigned>(image) * p.conv.hp + oy * p.conv.stride_h) * p.conv.wp + ox * p.conv.stride_w;
+                    b_off[r] = (position * p.conv.c_pad + chunk * 8) * 2u;
+                } else {
+                    b_off[r] = (static_cast<unsigned>(n0 + r * WAVES * 8 + row_in) * K + k_first + chunk * 8) * 2u;
+                }
+            }
         }
     }
+    // CONV: byte offset of the k-tile whose B loads are issued next (tiles are requested strictly in order): tap
+    // (ky, kx), channel block cb, kept on the scalar unit and advanced without a division.
+    int conv_cb = 0, conv_kx = 0, conv_row_off = 0;  // conv_row_off = ky·dil_h·wp
+    unsigned conv_off = 0;
+    auto conv_advance = [&]() {
+        if (++conv_cb == p.conv.c_blocks) {
+            conv_cb = 0;
+            if (++conv_kx == p.conv.kw) {
+                conv_kx = 0;
+                conv_row_off += p.conv.dil_h * p.conv.wp;
+            }
+        }
+        conv_off = (static_cast<unsigned>(conv_row_off + conv_kx * p.conv.dil_w) * p.conv.c_pad + conv_cb * 64) * 2u;
+    };
     const int lds_row_block = wave * 1024;  // wavefront-uniform part of every load's LDS destination
     auto load_a1 = [&](int stage, int r, unsigned k_off) {
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_ptr)(lds_bytes + stage * A_STAGE + r * (WAVES * 1024) + lds_row_block),
@@ -626,7 +738,11 @@ __device__ __forceinline__ void gemm_bf16_packed_body(const GemmBf16Args &p)
     };
     auto load_b1 = [&](int stage, int r, unsigned k_off) {
         __builtin_amdgcn_raw_ptr_buffer_load_lds(
-            rsrc_b, (lds_void_ptr)(lds_bytes + B_REGION + stage * B_STAGE + r * (WAVES * 1024) + lds_row_block), 16, b_off[r], k_off, 0, 0);
+            rsrc_b, (lds_void_ptr)(lds_bytes + B_REGION + stage * B_STAGE + r * (WAVES * 1024) + lds_row_block), 16, b_off[r],
+            CONV ? conv_off : k_off, 0, 0);
+        if constexpr (CONV) {
+            if (r == NB - 1) conv_advance();  // the last load of this k-tile: the next ones belong to the next tile
+        }
     };
 
     f32x16 acc[TM][TN];
@@ -738,7 +854,8 @@ __device__ __forceinline__ void gemm_bf16_packed_body(const GemmBf16Args &p)
     iteration(std::false_type{}, std::false_type{}, t);
 
     __syncthreads();
-    gemm_bf16_finish<WTN, TM>(p, split, acc, lds_bytes, wave, m0 + wm * WTM, n0 + wn * WTN, lane);
+    if constexpr (CONV) conv_bf16_epilogue<WTN, TM>(p, acc, lds_bytes, wave, m0 + wm * WTM, n0 + wn * WTN, lane);
+    else gemm_bf16_finish<WTN, TM>(p, split, acc, lds_bytes, wave, m0 + wm * WTM, n0 + wn * WTN, lane);
 }
 
 // -------------------------------------------------------------------------------------------------
@@ -1234,6 +1351,92 @@ __global__ __launch_bounds__(512) void gemm_bf16_256x128w8_packed_kernel(GemmBf1
 // fragment read of its own (the 256-row forms need three for four), so its main loop is LDS-bound; it serves launches
 // that would otherwise leave most compute units without a tile (1024³ is 16 tiles of 256×256).
 __global__ __launch_bounds__(256, 2) void gemm_bf16_128x128w4_packed_kernel(GemmBf16Args p) { gemm_bf16_packed_body<128, 4, 128>(p); }
+// Convolution forms (conv_bf16 below): 128 output channels × 128 pixels with four wavefronts, two workgroups per compute
+// unit, and 256 output channels × 128 / 256 pixels with eight.
+__global__ __launch_bounds__(256, 2) void conv2d_bf16_128x128w4_kernel(GemmBf16Args p) { gemm_bf16_packed_body<128, 4, 128, true>(p); }
+__global__ __launch_bounds__(512) void conv2d_bf16_256x128w8_kernel(GemmBf16Args p) { gemm_bf16_packed_body<128, 8, 256, true>(p); }
+__global__ __launch_bounds__(512) void conv2d_bf16_256x256w8_kernel(GemmBf16Args p) { gemm_bf16_packed_body<256, 8, 256, true>(p); }
+
+// Zero-padded channels-last copy of NCHW bf16 images: out[image][yp][xp][c_pad], yp = y + pad_h, xp = x + pad_w, channels
+// past c_in and the border positions zero.  One workgroup per (64-channel block, padded row, image): the row's
+// [64 channels][w] block is read along x, four pixels (8 bytes, at whatever alignment the row has) per lane, and written
+// along the channels, 16 bytes per lane, through a transposing LDS tile.  The workgroups behind those of the images
+// re-lay the weights in the same launch: OIHW -> (c_out, kh·kw·c_pad) with k ordered (ky, kx, channel), channels past c_in zero.
+struct ConvBf16Relayout {
+    const uint16_t *in;
+    uint16_t *out;
+    const uint16_t *weight_in;
+    uint16_t *weight_out;
+    int batch, c_in, h, w, c_pad, hp, wp, pad_h, pad_w, c_out, taps;
+    unsigned image_blocks;  // workgroups that copy image rows; the ones behind them re-lay the weights
+};
+
+__global__ __launch_bounds__(256) void conv_bf16_relayout_kernel(ConvBf16Relayout p)
+{
+    constexpr int TILE_W = 256;
+    __shared__ __attribute__((aligned(8))) uint16_t tile[64][TILE_W + 4];
+    typedef uint32_t u32x2_a2 __attribute__((ext_vector_type(2), aligned(2)));
+    const int tid = threadIdx.x;
+    if (blockIdx.x >= p.image_blocks) {  // the weights: 1024 values per workgroup
+        const size_t row = static_cast<size_t>(p.taps) * p.c_pad, total = static_cast<size_t>(p.c_out) * row;
+        const size_t first = static_cast<size_t>(blockIdx.x - p.image_blocks) * 1024 + tid;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const size_t idx = first + i * 256;
+            if (idx >= total) break;
+            const int o = static_cast<int>(idx / row);
+            const int rest = static_cast<int>(idx - static_cast<size_t>(o) * row);
+            const int tap = rest / p.c_pad, c = rest - tap * p.c_pad;
+            p.weight_out[idx] = c < p.c_in ? p.weight_in[(static_cast<size_t>(o) * p.c_in + c) * p.taps + tap] : static_cast<uint16_t>(0);
+        }
+        return;
+    }
+    const int c_blocks = p.c_pad / 64;
+    const int cb = blockIdx.x % c_blocks, yp = (blockIdx.x / c_blocks) % p.hp, image = blockIdx.x / (c_blocks * p.hp);
+    const int y = yp - p.pad_h, w = p.w;
+    uint16_t *row_out = p.out + ((static_cast<size_t>(image) * p.hp + yp) * p.wp) * p.c_pad + cb * 64;
+    const bool row_inside = y >= 0 && y < p.h;
+    const int channels = min(64, p.c_in - cb * 64);  // channels of this block that exist
+    for (int x0 = 0; x0 < w || x0 == 0; x0 += TILE_W) {  // x0: first image column of this piece
+        const int piece_w = min(TILE_W, w - x0), quads = (piece_w + 3) / 4;
+        __syncthreads();
+        if (row_inside) {
+            for (int idx = tid; idx < channels * quads; idx += 256) {
+                const int c = idx / quads, x = (idx - c * quads) * 4;
+                const uint16_t *src = p.in + ((static_cast<size_t>(image) * p.c_in + cb * 64 + c) * p.h + y) * w + x0 + x;
+                uint16_t v[4] = {0, 0, 0, 0};
+                if (x + 4 <= piece_w) {
+                    const u32x2_a2 two = *reinterpret_cast<const u32x2_a2 *>(src);
+                    v[0] = static_cast<uint16_t>(two[0]); v[1] = static_cast<uint16_t>(two[0] >> 16);
+                    v[2] = static_cast<uint16_t>(two[1]); v[3] = static_cast<uint16_t>(two[1] >> 16);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (x + e < piece_w) v[e] = src[e];
+                }
+                *reinterpret_cast<uint2 *>(&tile[c][x]) = make_uint2(v[0] | (static_cast<uint32_t>(v[1]) << 16), v[2] | (static_cast<uint32_t>(v[3]) << 16));
+            }
+        }
+        __syncthreads();
+        // Padded columns this piece covers: the left border with the first piece, the right border with the last.
+        const int first_xp = x0 == 0 ? 0 : x0 + p.pad_w;
+        const int last_xp = x0 + piece_w >= w ? p.wp : x0 + piece_w + p.pad_w;
+        for (int idx = tid; idx < (last_xp - first_xp) * 8; idx += 256) {
+            const int xp = first_xp + (idx >> 3), part = idx & 7;
+            const int col = xp - p.pad_w - x0;  // column within the tile (outside [0, piece_w): border)
+            uint32_t words[4] = {0u, 0u, 0u, 0u};
+            if (row_inside && col >= 0 && col < piece_w) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int c = part * 8 + 2 * e;
+                    const uint32_t lo = c < channels ? tile[c][col] : 0u, hi = c + 1 < channels ? tile[c + 1][col] : 0u;
+                    words[e] = lo | (hi << 16);
+                }
+            }
+            *reinterpret_cast<uint4 *>(row_out + static_cast<size_t>(xp) * p.c_pad + part * 8) = make_uint4(words[0], words[1], words[2], words[3]);
+        }
+    }
+}
 
 // Epilogue of the persistent kernel: the arithmetic and the strip layout of gemm_bf16_epilogue_bf16<64, 2, ACT, true>
 // (same bits), written to need few registers — the kernel runs three wavefronts per SIMD, 168 registers each, and
@@ -2540,6 +2743,114 @@ hipError_t launch_gemm_bf16(size_t m, size_t n, size_t k, const uint16_t *lhs, c
         return launch_256<256>(args, rhs_packed, stream, workspace_offset);
     }
     return launch_tile<128, 128, 32>(args, vec, stream, workspace_offset);
+}
+
+// bf16 convolution as an implicit GEMM on the packed kernels' machinery (crates/st-nn/src/layers/conv.rs:685-748,
+// 2559-2599 on bf16 operands): the images are copied once into a zero-padded channels-last layout, in which the 64
+// channels of one tap of one output pixel are 128 contiguous bytes — one row of a 64-wide k-tile, fetched straight into
+// LDS like a row of a prepacked B — and the weights are re-laid to match (k ordered tap-major).  No patch matrix.
+size_t conv2d_bf16_workspace_bytes(const ConvShape &c)
+{
+    const size_t c_pad = (static_cast<size_t>(c.c_in) + 63) / 64 * 64;
+    const size_t hp = static_cast<size_t>(c.h) + 2 * c.pad_h, wp = static_cast<size_t>(c.w) + 2 * c.pad_w;
+    const size_t image_bytes = (static_cast<size_t>(c.batch) * hp * wp * c_pad * 2 + 255) & ~static_cast<size_t>(255);
+    return image_bytes + static_cast<size_t>(c.c_out) * c.kh * c.kw * c_pad * 2;
+}
+
+bool conv2d_bf16_supported(const ConvShape &c)
+{
+    if (c.batch <= 0 || c.c_out <= 0 || c.oh <= 0 || c.ow <= 0) return true;  // nothing to compute
+    const size_t c_pad = (static_cast<size_t>(c.c_in) + 63) / 64 * 64;
+    const size_t hp = static_cast<size_t>(c.h) + 2 * c.pad_h, wp = static_cast<size_t>(c.w) + 2 * c.pad_w;
+    const size_t image_bytes = static_cast<size_t>(c.batch) * hp * wp * c_pad * 2;
+    const size_t k = static_cast<size_t>(c.kh) * c.kw * c_pad;
+    const size_t pixels = static_cast<size_t>(c.batch) * c.oh * c.ow;
+    // 32-bit byte offsets into both operands, 32-bit pixel and tile counts
+    return image_bytes < (1ull << 31) && static_cast<size_t>(c.c_out) * k * 2 < (1ull << 31) && pixels < (1ull << 31) &&
+           k < (1ull << 31);
+}
+
+hipError_t launch_conv2d_bf16(const ConvShape &c, int activation, const uint16_t *input, const uint16_t *weight, const float *bias,
+                              float *out_f32, uint16_t *out_bf16, hipStream_t stream)
+{
+    if (c.batch <= 0 || c.c_out <= 0 || c.oh <= 0 || c.ow <= 0) return hipSuccess;
+    if (!conv2d_bf16_supported(c)) return hipErrorInvalidValue;
+    const int c_pad = (c.c_in + 63) / 64 * 64;
+    const int hp = c.h + 2 * c.pad_h, wp = c.w + 2 * c.pad_w;
+    const int taps = c.kh * c.kw;
+    const size_t image_bytes = (static_cast<size_t>(c.batch) * hp * wp * c_pad * 2 + 255) & ~static_cast<size_t>(255);
+    void *workspace = nullptr;
+    hipError_t rc = stream_workspace(stream, conv2d_bf16_workspace_bytes(c), &workspace);
+    if (rc != hipSuccess) return rc;
+    uint16_t *images = static_cast<uint16_t *>(workspace);
+    uint16_t *weights = reinterpret_cast<uint16_t *>(static_cast<unsigned char *>(workspace) + image_bytes);
+    ConvBf16Relayout relayout;
+    relayout.in = input;
+    relayout.out = images;
+    relayout.weight_in = weight;
+    relayout.weight_out = weights;
+    relayout.batch = c.batch;
+    relayout.c_in = c.c_in;
+    relayout.h = c.h;
+    relayout.w = c.w;
+    relayout.c_pad = c_pad;
+    relayout.hp = hp;
+    relayout.wp = wp;
+    relayout.pad_h = c.pad_h;
+    relayout.pad_w = c.pad_w;
+    relayout.c_out = c.c_out;
+    relayout.taps = taps;
+    // one launch: a workgroup per (channel block, padded row, image), then one per 1024 weight values
+    const size_t image_blocks = static_cast<size_t>(c_pad / 64) * hp * c.batch;
+    const size_t weight_blocks = (static_cast<size_t>(c.c_out) * taps * c_pad + 1023) / 1024;
+    if (image_blocks + weight_blocks > 0x7fffffffu) return hipErrorInvalidConfiguration;
+    relayout.image_blocks = static_cast<unsigned>(image_blocks);
+    hipLaunchKernelGGL(conv_bf16_relayout_kernel, dim3(static_cast<unsigned>(image_blocks + weight_blocks)), dim3(256), 0, stream, relayout);
+    rc = hipGetLastError();
+    if (rc != hipSuccess) return rc;
+
+    GemmBf16Args args;
+    args.A = weights;
+    args.B = images;
+    args.C32 = out_f32;
+    args.C16 = out_bf16;
+    args.bias = bias;
+    args.residual = nullptr;
+    args.M = c.c_out;
+    args.N = static_cast<int>(static_cast<size_t>(c.batch) * c.oh * c.ow);
+    args.K = taps * c_pad;
+    args.scale = 1.0f;
+    args.activation = activation;
+    args.conv.ohow = c.oh * c.ow;
+    args.conv.ow = c.ow;
+    args.conv.hp = hp;
+    args.conv.wp = wp;
+    args.conv.c_pad = c_pad;
+    args.conv.stride_h = c.stride_h;
+    args.conv.stride_w = c.stride_w;
+    args.conv.dil_h = c.dil_h;
+    args.conv.dil_w = c.dil_w;
+    args.conv.kw = c.kw;
+    args.conv.c_blocks = c_pad / 64;
+    args.conv.c_out = c.c_out;
+    args.conv.image_bytes = static_cast<unsigned>(static_cast<size_t>(c.batch) * hp * wp * c_pad * 2);
+    // Tiles: 256 channels where the layer has them, 128 otherwise; 256 pixels wide only when that still gives every
+    // compute unit a tile.
+    const bool tall = c.c_out > 128;
+    const size_t tiles_m = (static_cast<size_t>(c.c_out) + (tall ? 255 : 127)) / (tall ? 256 : 128);
+    const bool wide = tall && tiles_m * ((static_cast<size_t>(args.N) + 255) / 256) >= 256;
+    const size_t bn = wide ? 256 : 128;
+    args.tiles_m = static_cast<int>(tiles_m);
+    args.tiles_n = static_cast<int>((static_cast<size_t>(args.N) + bn - 1) / bn);
+    const size_t tiles = static_cast<size_t>(args.tiles_m) * args.tiles_n;
+    if (tiles > 0x7fffffffu) return hipErrorInvalidConfiguration;
+    args.swizzle = (tiles % 8 == 0) ? 1 : 0;
+    auto kernel = !tall ? conv2d_bf16_128x128w4_kernel : wide ? conv2d_bf16_256x256w8_kernel : conv2d_bf16_256x128w8_kernel;
+    const size_t lds_bytes = tall ? 5 * 32768 : 5 * 16384;
+    rc = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
+    if (rc != hipSuccess) return rc;
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(tiles)), dim3(tall ? 512 : 256), lds_bytes, stream, args);
+    return hipGetLastError();
 }
 
 // out_f32 = (lhs·rhs + bias) + residual, out_ln = layer_norm(out_f32; gamma, beta, epsilon) rounded to bf16; rhs packed n×k.

@@ -817,6 +817,27 @@ int st_hip_conv2d_bias_act_f32_dev(size_t batch, size_t c_in, size_t h, size_t w
                          "conv2d launch");
 }
 
+int st_hip_conv2d_bias_act_bf16_dev(size_t batch, size_t c_in, size_t h, size_t w, size_t c_out, size_t kh, size_t kw,
+                                    size_t stride_h, size_t stride_w, size_t pad_h, size_t pad_w, size_t dil_h,
+                                    size_t dil_w, int activation, const uint16_t *input, const uint16_t *weight,
+                                    const float *bias, float *out_f32, uint16_t *out_bf16, void *stream)
+{
+    ST_HIP_CHECK(ensure_init());
+    ConvPlan plan;
+    ST_HIP_CHECK(plan_conv(batch, c_in, h, w, c_out, kh, kw, stride_h, stride_w, pad_h, pad_w, dil_h, dil_w, &plan));
+    ST_HIP_CHECK(validate_activation(activation, true));
+    if (plan.out_len == 0) return ST_HIP_OK;
+    if (!input || !weight || (!out_f32 && !out_bf16))
+        return fail(ST_HIP_ERR_INVALID, "conv2d received a null pointer; provide contiguous buffers");
+    const auto misaligned = [](const void *ptr, uintptr_t a) { return (reinterpret_cast<uintptr_t>(ptr) & (a - 1)) != 0; };
+    if (misaligned(out_f32, 16) || misaligned(out_bf16, 8))
+        return fail(ST_HIP_ERR_UNSUPPORTED, "bf16 conv2d needs a 16-byte aligned f32 output and an 8-byte aligned bf16 output");
+    if (!conv2d_bf16_supported(plan.shape))
+        return fail(ST_HIP_ERR_UNSUPPORTED, "bf16 conv2d: the padded channels-last copy of the input or the re-laid weights exceed 2 GiB");
+    return launch_status(launch_conv2d_bf16(plan.shape, activation, input, weight, bias, out_f32, out_bf16, as_stream(stream)),
+                         "conv2d bf16 launch");
+}
+
 int st_hip_conv2d_grad_input_f32_dev(size_t batch, size_t c_in, size_t h, size_t w, size_t c_out, size_t kh, size_t kw,
                                      size_t stride_h, size_t stride_w, size_t pad_h, size_t pad_w, size_t dil_h,
                                      size_t dil_w, const float *grad_output, const float *weight, float *grad_input,

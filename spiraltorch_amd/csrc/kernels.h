@@ -81,6 +81,12 @@ int planned_conv_kernel(const ConvShape &shape, bool weight_aligned, bool out_al
 int planned_conv_grad_input_kernel(const ConvShape &shape);
 void set_conv_forced_family(int family);
 
+// The same convolution on bf16 images and weights (NCHW / OIHW bit patterns), f32 accumulation, f32 bias, f32 and/or bf16
+// output (either may be null).  Uses the stream's scratch buffer for the re-laid operands.
+bool conv2d_bf16_supported(const ConvShape &shape);
+hipError_t launch_conv2d_bf16(const ConvShape &shape, int activation, const uint16_t *input, const uint16_t *weight,
+                              const float *bias, float *out_f32, uint16_t *out_bf16, hipStream_t stream);
+
 // Adjoint gather of the implicit GEMM (`shape` is the virtual forward problem: grad_output as the image, input
 // positions as output pixels, original stride/padding/dilation; weight laid out [c_in][c_out·kh·kw]).
 hipError_t launch_conv2d_adjoint_f32(const ConvShape &shape, const float *grad_output,

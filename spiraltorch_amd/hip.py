@@ -441,6 +441,15 @@ def conv2d_bias_act_f32_dev(batch, c_in, h, w, c_out, kernel, stride, padding, d
         dilation[1], int(activation), _dev(input), _dev(weight), _dev(bias), _dev(out), _stream_ptr(stream)))
 
 
+def conv2d_bias_act_bf16_dev(batch, c_in, h, w, c_out, kernel, stride, padding, dilation, activation, input, weight,
+                             bias, out_f32, out_bf16, stream=None) -> None:
+    """Fused conv2d on bf16 NCHW images and OIHW weights (bit patterns), f32 accumulation; f32 and/or bf16 output."""
+    _check(_lib.load().st_hip_conv2d_bias_act_bf16_dev(
+        batch, c_in, h, w, c_out, kernel[0], kernel[1], stride[0], stride[1], padding[0], padding[1], dilation[0],
+        dilation[1], int(activation), _dev(input), _dev(weight), _dev(bias), _dev(out_f32), _dev(out_bf16),
+        _stream_ptr(stream)))
+
+
 def conv2d_grad_input_f32_dev(batch, c_in, h, w, c_out, kernel, stride, padding, dilation, grad_output, weight,
                               grad_input, stream=None) -> None:
     _check(_lib.load().st_hip_conv2d_grad_input_f32_dev(

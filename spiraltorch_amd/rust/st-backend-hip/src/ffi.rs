@@ -108,6 +108,7 @@ extern "C" {
     pub fn st_hip_gemm_bf16_prepacked_residual_layer_norm_dev(m: usize, n: usize, k: usize, lhs: *const u16, packed_rhs: *const u16, bias: *const f32, residual: *const f32, gamma: *const f32, beta: *const f32, epsilon: f32, out_f32: *mut f32, out_ln_bf16: *mut u16, stream: *mut c_void) -> c_int;
     pub fn st_hip_pack_rhs_bf16_dev(k: usize, n: usize, rhs: *const u16, packed: *mut u16, stream: *mut c_void) -> c_int;
     pub fn st_hip_conv2d_bias_act_f32_dev(batch: usize, c_in: usize, h: usize, w: usize, c_out: usize, kh: usize, kw: usize, stride_h: usize, stride_w: usize, pad_h: usize, pad_w: usize, dil_h: usize, dil_w: usize, activation: c_int, input: *const f32, weight: *const f32, bias: *const f32, out: *mut f32, stream: *mut c_void) -> c_int;
+    pub fn st_hip_conv2d_bias_act_bf16_dev(batch: usize, c_in: usize, h: usize, w: usize, c_out: usize, kh: usize, kw: usize, stride_h: usize, stride_w: usize, pad_h: usize, pad_w: usize, dil_h: usize, dil_w: usize, activation: c_int, input: *const u16, weight: *const u16, bias: *const f32, out_f32: *mut f32, out_bf16: *mut u16, stream: *mut c_void) -> c_int;
     pub fn st_hip_conv2d_grad_input_f32_dev(batch: usize, c_in: usize, h: usize, w: usize, c_out: usize, kh: usize, kw: usize, stride_h: usize, stride_w: usize, pad_h: usize, pad_w: usize, dil_h: usize, dil_w: usize, grad_output: *const f32, weight: *const f32, grad_input: *mut f32, stream: *mut c_void) -> c_int;
     pub fn st_hip_conv2d_grad_input_f32_noalloc_dev(batch: usize, c_in: usize, h: usize, w: usize, c_out: usize, kh: usize, kw: usize, stride_h: usize, stride_w: usize, pad_h: usize, pad_w: usize, dil_h: usize, dil_w: usize, grad_output: *const f32, weight: *const f32, grad_input: *mut f32, stream: *mut c_void) -> c_int;
     pub fn st_hip_conv2d_grad_weight_f32_dev(batch: usize, c_in: usize, h: usize, w: usize, c_out: usize, kh: usize, kw: usize, stride_h: usize, stride_w: usize, pad_h: usize, pad_w: usize, dil_h: usize, dil_w: usize, input: *const f32, grad_output: *const f32, scale: f32, grad_weight: *mut f32, stream: *mut c_void) -> c_int;
