@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the HIP hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-sustained] [--only NAME] [--all]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-sustained] [--only NAME] [--all] [--probes]
 
 A "step" is one pass of the headline workload over one batch of synthetic input that is already
 resident in HBM: BASELINE config 2, the fused conv2d + bias + ReLU (f32, N32 C64->128 56x56 3x3 s1 p1).
@@ -451,6 +451,86 @@ def wl_calibration(hip, inputs, timer):
     return entry("calibration_f32_to_bf16_64mi", "f32", 0, count * 6, "hbm", wall, ev, sustained=sus)
 
 
+def probe_ceilings(hip, inputs, timer):
+    """What frames the bf16 GEMM figures on this box, measured in this process (stderr lines only, with --probes):
+    (1) a loop of bf16 matrix instructions alone, on all-zero and on N(0, 0.02^2) register operands: the rate the matrix
+        pipes sustain on those bits with no memory instruction in the way (power, hence clock, depends on the bits);
+    (2) the vendor library (torch.mm -> hipBLASLt) on config 4's operands, B row-major (NN) and transposed (NT), under
+        the same two protocols as the workloads.  torch is imported for this probe only; nothing else here uses it."""
+    out = []
+    sink = hip.DeviceBuffer(256 * 256 * 4)
+    for label, values in (("zeros", np.zeros(32768, np.float32)),
+                          ("normal_0.02", inputs.normal(inputs.seed_for(4, 3), 32768, 0.0, 0.02))):
+        d_ops = hip.DeviceBuffer.from_array(inputs.to_bf16(values))
+        iterations = 4000  # 256 workgroups x 4 wavefronts x 32 x 4000 matrix instructions: about 10 ms
+        _, ev = timer.run(lambda st: hip.probe_mfma_bf16_dev(256, iterations, d_ops, sink, st), 2, 10)
+        flops = 256 * 4 * iterations * 32 * 2 * 32 * 32 * 16
+        out.append({"probe": f"mfma_bf16_32x32x16_only_{label}", "kernel_ms": round(ev, 4),
+                    "tflops": round(flops / (ev * 1e-3) / 1e12, 1), "frac_of_bf16_peak": round(flops / (ev * 1e-3) / 1e12 / PEAK_TFLOPS["bf16"], 4)})
+    # this library's prepacked kernel with bf16 as the only output: what the vendor library's bf16-out figures compare with
+    m = n = k = 4096
+    d_a = hip.DeviceBuffer.from_array(inputs.to_bf16(inputs.normal(inputs.seed_for(4, 0), m * k, 0.0, 0.02)))
+    d_b = hip.DeviceBuffer.from_array(inputs.to_bf16(inputs.normal(inputs.seed_for(4, 1), k * n, 0.0, 0.02)))
+    d_packed, d_c16 = hip.DeviceBuffer(k * n * 2), hip.DeviceBuffer(m * n * 2)
+    hip.pack_rhs_bf16_dev(k, n, d_b, d_packed)
+    step = lambda st: hip.gemm_bf16_prepacked_bias_act_dev(m, n, k, 0, d_a, d_packed, None, None, None, d_c16, st)
+    _, first = timer.run(step, timer.warmup, timer.steps)
+    _, second = timer.run(step, SUSTAINED_WARMUP, SUSTAINED_STEPS)
+    frac = lambda ms: round(2 * m * n * k / (ms * 1e-3) / 1e12 / PEAK_TFLOPS["bf16"], 4)
+    out.append({"probe": "this_library_prepacked_bf16_4096_cubed_bf16_out", "kernel_ms_per_step": round(first, 5), "frac": frac(first),
+                "sustained_kernel_ms_per_step": round(second, 5), "sustained_frac": frac(second)})
+    # torch brings a HIP runtime of its own, which finds no device once this process has initialised the system's: the
+    # library probe runs as a child process (the parent is idle meanwhile) and hands its lines back on stdout.
+    import subprocess
+    child = subprocess.run([sys.executable, "-c", VENDOR_PROBE, ROOT, str(timer.warmup), str(timer.steps),
+                            str(SUSTAINED_WARMUP), str(SUSTAINED_STEPS), str(PEAK_TFLOPS["bf16"])],
+                           stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300)
+    lines = [line for line in child.stdout.splitlines() if line.startswith("{")]
+    if child.returncode != 0 or not lines:
+        out.append({"probe": "vendor_library", "skipped": (child.stderr.strip().splitlines() or ["no output"])[-1][:200]})
+    out.extend(json.loads(line) for line in lines)
+    return out
+
+
+# The vendor library on config 4's operands (torch.mm -> hipBLASLt), B row-major (NN) and transposed (NT), bf16 output,
+# under the protocol asked for and the sustained one.  A probe for comparison only; run as `python -c`.
+VENDOR_PROBE = r"""
+import json, sys
+root, warmup, steps, sus_warmup, sus_steps, peak = sys.argv[1], int(sys.argv[2]), int(sys.argv[3]), int(sys.argv[4]), int(sys.argv[5]), float(sys.argv[6])
+sys.path.insert(0, root)
+import torch
+from spiraltorch_amd import inputs
+n = 4096
+a = torch.from_numpy(inputs.normal(inputs.seed_for(4, 0), n * n, 0.0, 0.02).reshape(n, n)).cuda().to(torch.bfloat16)
+b = torch.from_numpy(inputs.normal(inputs.seed_for(4, 1), n * n, 0.0, 0.02).reshape(n, n)).cuda().to(torch.bfloat16)
+bt = b.t().contiguous()
+c = torch.empty(n, n, dtype=torch.bfloat16, device="cuda")
+start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+def timed(fn, w, k):
+    for _ in range(w):
+        fn()
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(k):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / k
+cases = [("NN_bf16_out", lambda: torch.mm(a, b, out=c)), ("NT_bf16_out", lambda: torch.mm(a, bt.t(), out=c))]
+try:  # f32 output, what config 4 asks for, where this torch offers it
+    torch.mm(a, b, out_dtype=torch.float32)
+    cases += [("NN_f32_out", lambda: torch.mm(a, b, out_dtype=torch.float32)), ("NT_f32_out", lambda: torch.mm(a, bt.t(), out_dtype=torch.float32))]
+except Exception:
+    pass
+for label, fn in cases:
+    first = timed(fn, warmup, steps)
+    second = timed(fn, sus_warmup, sus_steps)
+    frac = lambda ms: round(2 * n ** 3 / (ms * 1e-3) / 1e12 / peak, 4)
+    print(json.dumps({"probe": "vendor_library_torch_mm_bf16_4096_cubed_" + label, "kernel_ms_per_step": round(first, 5),
+                      "frac": frac(first), "sustained_kernel_ms_per_step": round(second, 5), "sustained_frac": frac(second)}), flush=True)
+"""
+
+
 # ---- CPU baselines: the C restatement of the reference's CPU path, timed on the host cores of this box ------------
 
 def _cpu(flops, seconds, cores, sample):
@@ -564,6 +644,9 @@ def main():
     parser.add_argument("--no-cpu-baseline", action="store_true")
     parser.add_argument("--no-sustained", action="store_true", help="skip the second (50 + 200 steps) measurement")
     parser.add_argument("--only", default=None, help="run only the headline plus workloads whose name contains this")
+    parser.add_argument("--probes", action="store_true",
+                        help="also measure the bf16 ceilings of this box: a matrix-instruction-only loop and the vendor library "
+                             "(stderr lines only)")
     parser.add_argument("--all", action="store_true",
                         help="also run the workloads that are no BASELINE configuration (stderr lines only)")
     args = parser.parse_args()
@@ -620,6 +703,9 @@ def main():
 
     rows = run(plan)
     extras = run(extra_plan) if args.all else []
+    if args.probes:
+        for item in probe_ceilings(hip, inputs, timer):
+            log(json.dumps(item))
 
     cpu = None
     if not args.no_cpu_baseline:

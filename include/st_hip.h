@@ -227,6 +227,18 @@ typedef struct {
 } st_hip_attention_plan;
 int st_hip_attention_f32_launch_plan(size_t contexts, size_t sequence, size_t head_dim, int causal, int biased,
                                      st_hip_attention_plan *plan);
+/* The same for the 256-row bf16 GEMM kernels, whose workgroups decode their index into (k-split, tile): the tiling and
+ * k-split launch_gemm would use for an m×n×k product (k a multiple of 64), the launcher's own check (`consistent`) and a
+ * walk over the whole grid (`items` must equal `workgroups`, `out_of_range` and `duplicates` must be 0). */
+typedef struct {
+    int tile_cols;          /* 256 or 128 columns per tile (256 rows) */
+    int tiles_m, tiles_n;
+    int k_splits;           /* workgroups along k per tile (1: not split) */
+    int k_tiles_per_split;  /* 64-wide k-tiles each of them walks */
+    int consistent;
+    uint64_t workgroups, items, out_of_range, duplicates;
+} st_hip_gemm_tile_plan;
+int st_hip_gemm_bf16_tile_plan(size_t m, size_t n, size_t k, st_hip_gemm_tile_plan *plan);
 /* Rows of A per launch when a GEMM whose A is 2 GiB or larger is cut into row blocks for the kernels that address
  * operands through 32-bit byte offsets: a multiple of 256 with rows*k*element_bytes < 2^31, or 0 when 256 rows do not
  * fit (such products run on the kernels with 64-bit addressing). */
@@ -302,12 +314,19 @@ int st_hip_conv2d_grad_input_f32_dev(size_t batch, size_t c_in, size_t h, size_t
                                      const float *grad_output, const float *weight,
                                      float *grad_input, void *stream);
 /* No counterpart in the reference.  st_hip_conv2d_grad_input_f32_dev for callers that cannot allocate device
- * memory (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): same arguments, same
- * kernels and bit-identical results, but the flipped weights the kernels read go to a static device array of
- * ST_HIP_NOALLOC_SCRATCH_BYTES instead of the stream's grow-on-demand workspace, and the call performs no hipMalloc /
- * hipFree on any path.  c_out*c_in*kh*kw*4 bytes must fit the array, otherwise ST_HIP_ERR_UNSUPPORTED (nothing is
- * launched).  Every call on a GPU shares that GPU's array: calls that overlap on one GPU (different streams or
- * threads) race; calls on one stream are ordered and safe.  st_hip_init must have succeeded first. */
+ * memory (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): same arguments, but the
+ * flipped weights the kernels read go to a static device array of ST_HIP_NOALLOC_SCRATCH_BYTES instead of the stream's
+ * grow-on-demand workspace, and the call performs no hipMalloc / hipFree on any path.  The two routes of the allocating
+ * entry point that need further scratch memory are not taken here: a long reduction over few tiles is not cut into
+ * k-slices (st_hip_conv2d_planned_kernel reports ST_HIP_CONV_KERNEL_TILE_KSLICED for such shapes: same products, added
+ * in another order, so results agree within the f32 parity bar, not bit for bit, and the call is slower), and strided
+ * layers whose adjoint gather is wasteful do not go through the per-image GEMM + col2im route (reported as
+ * ST_HIP_CONV_KERNEL_COL2IM: the gather kernel runs instead, correct but up to three orders of magnitude slower on
+ * patch-embedding-like shapes — such callers should give the allocating entry point one warm-up call outside the
+ * capture instead).  For every other shape the kernels, and the result bits, are those of the allocating entry point.
+ * c_out*c_in*kh*kw*4 bytes must fit the array, otherwise ST_HIP_ERR_UNSUPPORTED (nothing is launched).  Every call on a
+ * GPU shares that GPU's array: calls that overlap on one GPU (different streams or threads) race; calls on one stream
+ * are ordered and safe.  st_hip_init must have succeeded first. */
 #define ST_HIP_NOALLOC_SCRATCH_BYTES (16u << 20)
 int st_hip_conv2d_grad_input_f32_noalloc_dev(size_t batch, size_t c_in, size_t h, size_t w, size_t c_out,
                                              size_t kh, size_t kw, size_t stride_h, size_t stride_w,
@@ -382,6 +401,14 @@ int st_hip_split_heads_f32_dev(size_t batch, size_t seq, size_t heads, size_t he
 int st_hip_merge_heads_f32_dev(size_t batch, size_t seq, size_t heads, size_t head_dim,
                                const float *contexts_in, float *out_f32, uint16_t *out_bf16,
                                void *stream);
+
+/* ---- measurement aid ---------------------------------------------------------------------------- */
+/* A loop of nothing but bf16 matrix instructions (v_mfma_f32_32x32x16_bf16) on register operands: `workgroups` × 4
+ * wavefronts each issue 32·iterations of them (2·32·32·16 flop each) on fragments read once from `operands` (device,
+ * 32768 bf16 values, 16-byte aligned); `sink` (device, workgroups·256 floats) receives the sums so that nothing is
+ * optimised away.  What the matrix pipes deliver on given operand bits with no memory instruction in the way — the
+ * ceiling bench.py --probes reports beside the bf16 GEMM.  No reference counterpart. */
+int st_hip_probe_mfma_bf16_dev(size_t workgroups, size_t iterations, const uint16_t *operands, float *sink, void *stream);
 
 /* ---- byte-level decoder stack (built from the ops above) ------------------------------------ */
 typedef struct {

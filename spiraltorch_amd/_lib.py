@@ -42,6 +42,12 @@ class AttentionPlan(ctypes.Structure):
                 ("duplicates", c_uint64)]
 
 
+class GemmTilePlan(ctypes.Structure):
+    _fields_ = [("tile_cols", c_int), ("tiles_m", c_int), ("tiles_n", c_int), ("k_splits", c_int), ("k_tiles_per_split", c_int),
+                ("consistent", c_int), ("workgroups", c_uint64), ("items", c_uint64), ("out_of_range", c_uint64),
+                ("duplicates", c_uint64)]
+
+
 class DecoderConfig(ctypes.Structure):
     _fields_ = [
         ("vocab", c_size_t),
@@ -93,6 +99,8 @@ SIGNATURES = {
     "st_hip_conv2d_planned_kernel": (c_int, [c_size_t] * 13 + [c_int, POINTER(c_int)]),
     "st_hip_attention_f32_launch_plan": (c_int, [c_size_t, c_size_t, c_size_t, c_int, c_int, POINTER(AttentionPlan)]),
     "st_hip_gemm_row_block": (c_size_t, [c_size_t, c_size_t]),
+    "st_hip_probe_mfma_bf16_dev": (c_int, [c_size_t, c_size_t, c_void_p, c_void_p, c_void_p]),
+    "st_hip_gemm_bf16_tile_plan": (c_int, [c_size_t, c_size_t, c_size_t, POINTER(GemmTilePlan)]),
     "st_hip_conv2d_bias_act_f32": (c_int, [c_size_t] * 13 + [c_int, c_void_p, c_size_t, c_void_p, c_size_t,
                                                              c_void_p, c_size_t, c_void_p, c_size_t]),
     "st_hip_attention_f32": (c_int, [c_size_t, c_size_t, c_size_t, c_float, c_int, c_void_p, c_size_t, c_void_p,

@@ -1140,6 +1140,10 @@ hipError_t launch_conv2d_f32(const ConvShape &shape, int activation, const float
         const size_t k_steps = (static_cast<size_t>(args.K) + 15) / 16, steps_per_slice = (k_steps + slices - 1) / slices;
         const size_t used = (k_steps + steps_per_slice - 1) / steps_per_slice;
         const size_t count = static_cast<size_t>(shape.batch) * shape.c_out * args.spatial;
+        // The kernel's workgroup (tile, y) walks k-tiles [y·steps_per_slice, (y+1)·steps_per_slice) and writes plane y:
+        // every launched slice has k-tiles, together they cover the reduction, and their planes fit the scratch asked for.
+        if (used == 0 || used > slices || used > 65535 || (used - 1) * steps_per_slice >= k_steps || used * steps_per_slice < k_steps)
+            return hipErrorInvalidConfiguration;
         void *workspace = nullptr;
         hipError_t rc = stream_workspace(stream, scratch_offset + slices * count * sizeof(float), &workspace);
         if (rc != hipSuccess) return rc;

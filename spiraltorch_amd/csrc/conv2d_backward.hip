@@ -60,15 +60,15 @@ namespace {
 __global__ __launch_bounds__(256) void conv_weight_to_adjoint_kernel(int c_out, int c_in, int kh, int kw, int flip,
                                                                      const float *src, float *dst)
 {
-    const int total = c_out * c_in * kh * kw;
-    const int i = blockIdx.x * 256 + threadIdx.x;
+    const size_t total = static_cast<size_t>(c_out) * c_in * kh * kw;  // (may exceed 2^31 values)
+    const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
     if (i >= total) return;
-    const int kx = i % kw;
-    int rest = i / kw;
-    const int ky = rest % kh;
+    const int kx = static_cast<int>(i % kw);
+    size_t rest = i / kw;
+    const int ky = static_cast<int>(rest % kh);
     rest /= kh;
-    const int oc = rest % c_out;
-    const int ic = rest / c_out;
+    const int oc = static_cast<int>(rest % c_out);
+    const int ic = static_cast<int>(rest / c_out);
     const int sy = flip ? kh - 1 - ky : ky, sx = flip ? kw - 1 - kx : kx;
     dst[i] = src[((static_cast<size_t>(oc) * c_in + ic) * kh + sy) * kw + sx];
 }

@@ -2332,19 +2332,50 @@ TilePlan plan_tiles(size_t m, size_t n, size_t k)
     return plan;
 }
 
-template <int BN>
-hipError_t launch_256(GemmBf16Args args, bool packed, hipStream_t stream, size_t workspace_offset)
+// The launch arithmetic of the tiled kernels whose workgroups decode their index into (k-split, tile), checked on the
+// host before every launch: the grid is tiles × k-splits and fits the 32-bit ids the kernels compute with, the tiles
+// cover the matrix without an empty row or column of tiles, every split has k-tiles to walk and together they cover K,
+// and the XCD remap only runs on a grid it divides.  A plan that fails is an error code, not a launch.
+bool tile_launch_consistent(const GemmBf16Args &a, size_t grid, int bm, int bn)
+{
+    if (a.M <= 0 || a.N <= 0 || a.K < 64 || a.K % 64 != 0 || a.tiles_m <= 0 || a.tiles_n <= 0) return false;
+    const size_t tiles = static_cast<size_t>(a.tiles_m) * static_cast<size_t>(a.tiles_n), k_tiles = static_cast<size_t>(a.K) / 64;
+    if (grid == 0 || grid > 0x7fffffffu || a.k_splits < 1 || grid != tiles * static_cast<size_t>(a.k_splits)) return false;
+    if (static_cast<size_t>(a.tiles_m) * bm < static_cast<size_t>(a.M) || static_cast<size_t>(a.tiles_m - 1) * bm >= static_cast<size_t>(a.M)) return false;
+    if (static_cast<size_t>(a.tiles_n) * bn < static_cast<size_t>(a.N) || static_cast<size_t>(a.tiles_n - 1) * bn >= static_cast<size_t>(a.N)) return false;
+    if (a.k_splits > 1) {
+        const size_t per = static_cast<size_t>(a.tiles_per_split);
+        if (a.tiles_per_split < 1 || a.partial == nullptr) return false;
+        if (static_cast<size_t>(a.k_splits - 1) * per >= k_tiles || static_cast<size_t>(a.k_splits) * per < k_tiles) return false;
+    }
+    return !a.swizzle || grid % 8 == 0;
+}
+
+// Tiles and k-splits of a 256-row launch (BN columns per tile) filled into `args`; returns the grid.
+size_t plan_256(GemmBf16Args &args, int bn)
 {
     args.tiles_m = (args.M + 255) / 256;
-    args.tiles_n = (args.N + BN - 1) / BN;  // the packed kernels take a ragged N: rows of Bᵀ past it read as zero
+    args.tiles_n = (args.N + bn - 1) / bn;  // the packed kernels take a ragged N: rows of Bᵀ past it read as zero
     size_t tiles = static_cast<size_t>(args.tiles_m) * static_cast<size_t>(args.tiles_n);
-    if (tiles > 0x7fffffffu) return hipErrorInvalidConfiguration;
     const size_t k_tiles = static_cast<size_t>(args.K) / 64;
     const size_t splits = choose_k_splits(args.M, args.N, args.K, tiles);
-    SkinnyArgs reduce{};
+    args.k_splits = 1;
     if (splits > 1) {
         args.tiles_per_split = static_cast<int>((k_tiles + splits - 1) / splits);
         args.k_splits = static_cast<int>((k_tiles + args.tiles_per_split - 1) / args.tiles_per_split);
+        tiles *= static_cast<size_t>(args.k_splits);
+    }
+    args.swizzle = (tiles % 8 == 0) ? 1 : 0;
+    return tiles;
+}
+
+template <int BN>
+hipError_t launch_256(GemmBf16Args args, bool packed, hipStream_t stream, size_t workspace_offset)
+{
+    const size_t tiles = plan_256(args, BN);
+    if (tiles > 0x7fffffffu) return hipErrorInvalidConfiguration;
+    SkinnyArgs reduce{};
+    if (args.k_splits > 1) {
         const size_t bytes = static_cast<size_t>(args.k_splits) * args.M * args.N * sizeof(float);
         void *workspace = nullptr;
         hipError_t rc = stream_workspace(stream, workspace_offset + bytes, &workspace);
@@ -2361,9 +2392,8 @@ hipError_t launch_256(GemmBf16Args args, bool packed, hipStream_t stream, size_t
         reduce.k_splits = args.k_splits;
         reduce.scale = args.scale;
         reduce.activation = args.activation;
-        tiles *= static_cast<size_t>(args.k_splits);
     }
-    args.swizzle = (tiles % 8 == 0) ? 1 : 0;
+    if (!tile_launch_consistent(args, tiles, 256, BN)) return hipErrorInvalidConfiguration;
     constexpr size_t lds_bytes = 5 * 32768;  // three A stages + two B stages
     static_assert(lds_bytes >= 8 * 32 * (128 + 4) * sizeof(float), "eight epilogue strips must fit in the stage buffers");
     auto kernel = BN == 256 ? (packed ? gemm_bf16_256w8_packed_kernel : gemm_bf16_256rm_kernel)
@@ -2410,6 +2440,7 @@ hipError_t launch_128(GemmBf16Args args, bool packed, hipStream_t stream, size_t
         tiles *= static_cast<size_t>(args.k_splits);
     }
     args.swizzle = (tiles % 8 == 0) ? 1 : 0;
+    if (!tile_launch_consistent(args, tiles, 128, 128)) return hipErrorInvalidConfiguration;
     constexpr size_t lds_bytes = 5 * 16384;  // three A stages + two B stages of 128 rows
     static_assert(lds_bytes >= 4 * 32 * (64 + 4) * sizeof(float), "four epilogue strips must fit in the stage buffers");
     auto kernel = packed ? gemm_bf16_128x128w4_packed_kernel : gemm_bf16_128x128w4_rm_kernel;
@@ -2434,6 +2465,9 @@ hipError_t launch_persistent_256x128(GemmBf16Args args, hipStream_t stream)
     if (tiles > 0x7fffffffu) return hipErrorInvalidConfiguration;
     const unsigned grid = static_cast<unsigned>(std::min<size_t>(tiles, 256));
     args.swizzle = (tiles % 8 == 0 && grid % 8 == 0) ? 1 : 0;
+    // whole tiles only (the epilogues store without row or column checks), no k-splits, and a walk every workgroup ends
+    if (args.M % 256 != 0 || args.N % 128 != 0 || args.K < 64 || args.K % 64 != 0 || args.k_splits != 1 || grid == 0)
+        return hipErrorInvalidConfiguration;
     constexpr size_t lds_bytes = 3 * 32768 + 2 * 16384 + 32768;  // three A stages, two B stages, strips of four wavefronts
     auto kernel = args.C32 ? gemm_bf16_persistent_256x128_f32out_kernel : gemm_bf16_persistent_256x128_kernel;
     hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -2745,6 +2779,54 @@ hipError_t launch_gemm_bf16(size_t m, size_t n, size_t k, const uint16_t *lhs, c
     return launch_tile<128, 128, 32>(args, vec, stream, workspace_offset);
 }
 
+// The 256-row tiling launch_gemm_bf16 would use for an m×n×k product (k a multiple of 64, n of 128, 16-byte aligned
+// operands), with the launcher's own consistency check evaluated on it: what st_hip_gemm_bf16_tile_plan reports.
+GemmTilePlanReport gemm_bf16_tile_plan_report(size_t m, size_t n, size_t k)
+{
+    GemmTilePlanReport report{};
+    if (m == 0 || n == 0 || k < 64 || k % 64 != 0 || m > 0x7fffffffu || n > 0x7fffffffu || k > 0x7fffffffu) return report;
+    const TilePlan plan = plan_tiles(m, n, k);
+    GemmBf16Args args{};
+    args.M = static_cast<int>(m);
+    args.N = static_cast<int>(n);
+    args.K = static_cast<int>(k);
+    const int bn = plan.narrow ? 128 : 256;
+    const size_t grid = plan_256(args, bn);
+    static float placeholder;
+    if (args.k_splits > 1) args.partial = &placeholder;  // the launcher points this at scratch memory
+    report.tile_cols = bn;
+    report.tiles_m = args.tiles_m;
+    report.tiles_n = args.tiles_n;
+    report.k_splits = args.k_splits;
+    report.k_tiles_per_split = args.k_splits > 1 ? args.tiles_per_split : static_cast<int>(k / 64);
+    report.workgroups = grid;
+    report.consistent = tile_launch_consistent(args, grid, 256, bn) ? 1 : 0;
+    // every (split, tile) a workgroup decodes to, walked the way the kernels decode it
+    const size_t tiles = static_cast<size_t>(args.tiles_m) * args.tiles_n;
+    if (grid <= (1u << 24)) {
+        std::vector<unsigned char> seen(grid, 0);
+        for (size_t block = 0; block < grid; ++block) {
+            size_t logical = block;
+            if (args.swizzle) logical = (block & 7) * (grid >> 3) + (block >> 3);
+            const size_t split = logical / tiles, rest = logical - split * tiles;
+            const size_t width = 4 * static_cast<size_t>(args.tiles_n), group = rest / width, first_m = group * 4;
+            const size_t group_size = std::min<size_t>(args.tiles_m - first_m, 4);
+            const size_t tile_m = first_m + (rest % width) % group_size, tile_n = (rest % width) / group_size;
+            const size_t first_k = split * static_cast<size_t>(args.tiles_per_split);
+            const bool inside = split < static_cast<size_t>(args.k_splits) && tile_m < static_cast<size_t>(args.tiles_m) &&
+                                tile_n < static_cast<size_t>(args.tiles_n) && tile_m * 256 < m && tile_n * bn < n && first_k < k / 64;
+            if (!inside) {
+                ++report.out_of_range;
+                continue;
+            }
+            unsigned char &cell = seen[(split * args.tiles_m + tile_m) * args.tiles_n + tile_n];
+            if (cell) ++report.duplicates; else ++report.items;
+            cell = 1;
+        }
+    }
+    return report;
+}
+
 // bf16 convolution as an implicit GEMM on the packed kernels' machinery (crates/st-nn/src/layers/conv.rs:685-748,
 // 2559-2599 on bf16 operands): the images are copied once into a zero-padded channels-last layout, in which the 64
 // channels of one tap of one output pixel are 128 contiguous bytes — one row of a 64-wide k-tile, fetched straight into
@@ -2845,6 +2927,7 @@ hipError_t launch_conv2d_bf16(const ConvShape &c, int activation, const uint16_t
     const size_t tiles = static_cast<size_t>(args.tiles_m) * args.tiles_n;
     if (tiles > 0x7fffffffu) return hipErrorInvalidConfiguration;
     args.swizzle = (tiles % 8 == 0) ? 1 : 0;
+    if (!tile_launch_consistent(args, tiles, tall ? 256 : 128, static_cast<int>(bn))) return hipErrorInvalidConfiguration;
     auto kernel = !tall ? conv2d_bf16_128x128w4_kernel : wide ? conv2d_bf16_256x256w8_kernel : conv2d_bf16_256x128w8_kernel;
     const size_t lds_bytes = tall ? 5 * 32768 : 5 * 16384;
     rc = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));

@@ -494,6 +494,34 @@ int st_hip_attention_f32_launch_plan(size_t contexts, size_t sequence, size_t he
     return ST_HIP_OK;
 }
 
+int st_hip_probe_mfma_bf16_dev(size_t workgroups, size_t iterations, const uint16_t *operands, float *sink, void *stream)
+{
+    ST_HIP_CHECK(ensure_init());
+    if (!operands || !sink) return fail(ST_HIP_ERR_INVALID, "mfma probe received a null pointer");
+    if ((reinterpret_cast<uintptr_t>(operands) & 15u) != 0) return fail(ST_HIP_ERR_UNSUPPORTED, "mfma probe operands must be 16-byte aligned");
+    return launch_status(launch_probe_mfma_bf16(workgroups, iterations, operands, sink, as_stream(stream)), "mfma probe launch");
+}
+
+int st_hip_gemm_bf16_tile_plan(size_t m, size_t n, size_t k, st_hip_gemm_tile_plan *plan)
+{
+    if (!plan) return fail(ST_HIP_ERR_INVALID, "gemm tile_plan received a null out-pointer");
+    if (m > kMaxDim || n > kMaxDim || k > kMaxDim) return fail(ST_HIP_ERR_INVALID, "gemm dimensions exceed i32");
+    if (m == 0 || n == 0 || k < 64 || k % 64 != 0)
+        return fail(ST_HIP_ERR_UNSUPPORTED, "the 256-row kernels take k a positive multiple of 64 (received %zu)", k);
+    const GemmTilePlanReport report = gemm_bf16_tile_plan_report(m, n, k);
+    plan->tile_cols = report.tile_cols;
+    plan->tiles_m = report.tiles_m;
+    plan->tiles_n = report.tiles_n;
+    plan->k_splits = report.k_splits;
+    plan->k_tiles_per_split = report.k_tiles_per_split;
+    plan->consistent = report.consistent;
+    plan->workgroups = report.workgroups;
+    plan->items = report.items;
+    plan->out_of_range = report.out_of_range;
+    plan->duplicates = report.duplicates;
+    return ST_HIP_OK;
+}
+
 size_t st_hip_gemm_row_block(size_t k, size_t element_bytes)
 {
     size_t row_bytes = 0;

@@ -50,6 +50,14 @@ hipError_t launch_transpose_f32(size_t rows, size_t cols, const float *in, float
 hipError_t launch_gemm_bf16(size_t m, size_t n, size_t k, const uint16_t *lhs, const uint16_t *rhs,
                             float *out_f32, uint16_t *out_bf16, const GemmEpilogue &epilogue,
                             hipStream_t stream, bool rhs_packed = false);
+// The launch arithmetic of the 256-row bf16 kernels for a shape, every workgroup decoded on the host: see
+// st_hip_gemm_tile_plan.
+struct GemmTilePlanReport {
+    int tile_cols, tiles_m, tiles_n, k_splits, k_tiles_per_split, consistent;
+    uint64_t workgroups, items, out_of_range, duplicates;
+};
+GemmTilePlanReport gemm_bf16_tile_plan_report(size_t m, size_t n, size_t k);
+
 // out_f32 = (lhs·rhs + bias) + residual and out_ln = layer_norm(out_f32) rounded to bf16, rhs packed n×k: Linear + residual +
 // LayerNorm of a transformer block (crates/st-vision/src/models/vit.rs:256-265) in one launch where the shape allows.
 hipError_t launch_gemm_bf16_residual_layer_norm(size_t m, size_t n, size_t k, const uint16_t *lhs, const uint16_t *packed_rhs,
@@ -147,6 +155,10 @@ hipError_t launch_gelu_backward_f32(size_t count, const float *z, const float *g
 hipError_t launch_scale_f32(size_t count, const float *in, float scale, float *out, hipStream_t stream);
 hipError_t launch_add_row_f32(size_t rows, size_t cols, float *data, const float *bias, hipStream_t stream);
 hipError_t launch_sum_axis0_f32(size_t rows, size_t cols, const float *in, float scale, float *out, hipStream_t stream);
+
+// Measurement aid: `workgroups` × 4 wavefronts each issue 32·iterations bf16 32x32x16 matrix instructions on register
+// operands read once from `operands` (32768 bf16 values); sink receives workgroups·256 floats.
+hipError_t launch_probe_mfma_bf16(size_t workgroups, size_t iterations, const uint16_t *operands, float *sink, hipStream_t stream);
 
 // One grow-only device buffer per (stream, host thread) for kernels that need scratch memory (split-k partial sums,
 // column-sum partials).  A thread's work on a stream is ordered, so two of its launches never use the buffer at the

@@ -238,6 +238,13 @@ def attention_f32_launch_plan(contexts, sequence, head_dim, causal=False, biased
     return out
 
 
+def gemm_bf16_tile_plan(m: int, n: int, k: int) -> dict:
+    """Tiling and k-split of the 256-row bf16 GEMM kernels for a shape, with the whole grid decoded on the host."""
+    plan = _lib.GemmTilePlan()
+    _check(_lib.load().st_hip_gemm_bf16_tile_plan(m, n, k, ctypes.byref(plan)))
+    return {name: int(getattr(plan, name)) for name, _ in _lib.GemmTilePlan._fields_}
+
+
 def gemm_row_block(k: int, element_bytes: int) -> int:
     """Rows of A per launch when an A of 2 GiB or more is cut into row blocks (0: not even 256 rows fit)."""
     return int(_lib.load().st_hip_gemm_row_block(k, element_bytes))
@@ -496,6 +503,11 @@ def attention_bf16_dev(batch, heads, sequence, head_dim, scale, causal, q, k, v,
     DeviceBuffers or raw device addresses (DeviceBuffer.at) of bf16 bit patterns."""
     _check(_lib.load().st_hip_attention_bf16_dev(batch, heads, sequence, head_dim, scale, int(bool(causal)), _dev(q),
                                                  _dev(k), _dev(v), ld_in, _dev(out), ld_out, _stream_ptr(stream)))
+
+
+def probe_mfma_bf16_dev(workgroups, iterations, operands, sink, stream=None) -> None:
+    """A loop of bf16 matrix instructions on register operands (measurement aid; see st_hip_probe_mfma_bf16_dev)."""
+    _check(_lib.load().st_hip_probe_mfma_bf16_dev(workgroups, iterations, _dev(operands), _dev(sink), _stream_ptr(stream)))
 
 
 def row_softmax_f32_dev(rows, cols, src, dst, stream=None) -> None:

@@ -16,7 +16,8 @@ TARGET = os.path.join(HERE, "st-backend-hip", "src", "ffi.rs")
 
 SCALARS = {"size_t": "usize", "int": "c_int", "float": "f32", "uint64_t": "u64", "uint16_t": "u16", "char": "c_char",
            "void": "c_void", "st_hip_device_props": "StHipDeviceProps", "st_hip_probe_result": "StHipProbeResult",
-           "st_hip_decoder_config": "StHipDecoderConfig", "st_hip_attention_plan": "StHipAttentionPlan"}
+           "st_hip_decoder_config": "StHipDecoderConfig", "st_hip_attention_plan": "StHipAttentionPlan",
+           "st_hip_gemm_tile_plan": "StHipGemmTilePlan"}
 RUST_KEYWORDS = {"in": "input", "type": "kind", "ref": "reference"}
 
 STRUCTS = '''/// `st_hip_device_props`.
@@ -69,6 +70,22 @@ pub struct StHipAttentionPlan {
     pub workgroups: u64,
     pub items: u64,
     pub items_expected: u64,
+    pub out_of_range: u64,
+    pub duplicates: u64,
+}
+
+/// `st_hip_gemm_tile_plan`.
+#[repr(C)]
+#[derive(Clone, Copy, Debug, Default, PartialEq)]
+pub struct StHipGemmTilePlan {
+    pub tile_cols: c_int,
+    pub tiles_m: c_int,
+    pub tiles_n: c_int,
+    pub k_splits: c_int,
+    pub k_tiles_per_split: c_int,
+    pub consistent: c_int,
+    pub workgroups: u64,
+    pub items: u64,
     pub out_of_range: u64,
     pub duplicates: u64,
 }

@@ -59,6 +59,22 @@ pub struct StHipAttentionPlan {
     pub duplicates: u64,
 }
 
+/// `st_hip_gemm_tile_plan`.
+#[repr(C)]
+#[derive(Clone, Copy, Debug, Default, PartialEq)]
+pub struct StHipGemmTilePlan {
+    pub tile_cols: c_int,
+    pub tiles_m: c_int,
+    pub tiles_n: c_int,
+    pub k_splits: c_int,
+    pub k_tiles_per_split: c_int,
+    pub consistent: c_int,
+    pub workgroups: u64,
+    pub items: u64,
+    pub out_of_range: u64,
+    pub duplicates: u64,
+}
+
 #[link(name = "sthip")]
 extern "C" {
     pub fn st_hip_init() -> c_int;
@@ -97,6 +113,7 @@ extern "C" {
     pub fn st_hip_conv2d_backward_f32(batch: usize, c_in: usize, h: usize, w: usize, c_out: usize, kh: usize, kw: usize, stride_h: usize, stride_w: usize, pad_h: usize, pad_w: usize, dil_h: usize, dil_w: usize, input: *const f32, input_len: usize, weight: *const f32, weight_len: usize, grad_output: *const f32, grad_output_len: usize, grad_input: *mut f32, grad_input_len: usize, grad_weight: *mut f32, grad_weight_len: usize, grad_bias: *mut f32, grad_bias_len: usize) -> c_int;
     pub fn st_hip_attention_f32(contexts: usize, sequence: usize, head_dim: usize, scale: f32, causal: c_int, q: *const f32, q_len: usize, k: *const f32, k_len: usize, v: *const f32, v_len: usize, z_bias: *const f32, z_bias_len: usize, attn_bias: *const f32, attn_bias_len: usize, out: *mut f32, out_len: usize) -> c_int;
     pub fn st_hip_attention_f32_launch_plan(contexts: usize, sequence: usize, head_dim: usize, causal: c_int, biased: c_int, plan: *mut StHipAttentionPlan) -> c_int;
+    pub fn st_hip_gemm_bf16_tile_plan(m: usize, n: usize, k: usize, plan: *mut StHipGemmTilePlan) -> c_int;
     pub fn st_hip_gemm_row_block(k: usize, element_bytes: usize) -> usize;
     pub fn st_hip_gemm_f32_dev(m: usize, n: usize, k: usize, scale: f32, lhs_transposed: c_int, lhs: *const f32, rhs: *const f32, out: *mut f32, stream: *mut c_void) -> c_int;
     pub fn st_hip_gemm_bias_act_f32_dev(m: usize, n: usize, k: usize, activation: c_int, lhs: *const f32, rhs: *const f32, bias: *const f32, residual: *const f32, out: *mut f32, stream: *mut c_void) -> c_int;
@@ -127,6 +144,7 @@ extern "C" {
     pub fn st_hip_f32_to_bf16_dev(count: usize, input: *const f32, out: *mut u16, stream: *mut c_void) -> c_int;
     pub fn st_hip_split_heads_f32_dev(batch: usize, seq: usize, heads: usize, head_dim: usize, qkv: *const f32, q: *mut f32, k: *mut f32, v: *mut f32, stream: *mut c_void) -> c_int;
     pub fn st_hip_merge_heads_f32_dev(batch: usize, seq: usize, heads: usize, head_dim: usize, contexts_in: *const f32, out_f32: *mut f32, out_bf16: *mut u16, stream: *mut c_void) -> c_int;
+    pub fn st_hip_probe_mfma_bf16_dev(workgroups: usize, iterations: usize, operands: *const u16, sink: *mut f32, stream: *mut c_void) -> c_int;
     pub fn st_hip_decoder_weight_count(config: *const StHipDecoderConfig) -> usize;
     pub fn st_hip_decoder_create(config: *const StHipDecoderConfig, host_weights: *const f32, weight_len: usize, decoder: *mut *mut c_void) -> c_int;
     pub fn st_hip_decoder_forward_dev(decoder: *mut c_void, tokens: *const f32, logits: *mut f32, stream: *mut c_void) -> c_int;

@@ -56,3 +56,22 @@ def test_the_shape_that_once_read_past_its_operands_keeps_the_pairing():
     # the reference's caller: one context with a bias matrix, keys split over workgroups
     plan = hip.attention_f32_launch_plan(1, 2048, 64, False, True)
     assert plan["kernel"] == "fast_biased" and plan["key_splits"] > 1 and plan["workgroups"] == 16 * plan["key_splits"]
+
+
+def test_bf16_tile_grids_decode_to_every_split_and_tile_once():
+    # few tiles under a long k are split over workgroups: every (k-split, tile) the grid decodes to must exist, have
+    # k-tiles to walk, and be decoded exactly once — also where the XCD remap reorders the workgroups
+    ms = (1, 33, 64, 65, 100, 255, 256, 257, 300, 512, 1000, 1024, 2048, 4096, 16384)
+    ns = (128, 256, 384, 512, 1000, 1536, 2048, 4096, 50257)
+    ks = (64, 128, 512, 576, 1024, 2048, 4096, 8192, 65536)
+    for m, n, k in itertools.product(ms, ns, ks):
+        plan = hip.gemm_bf16_tile_plan(m, n, k)
+        where = (m, n, k, plan)
+        assert plan["consistent"] == 1, where
+        assert plan["out_of_range"] == 0 and plan["duplicates"] == 0, where
+        assert plan["items"] == plan["workgroups"] == plan["tiles_m"] * plan["tiles_n"] * plan["k_splits"], where
+        assert plan["k_splits"] * plan["k_tiles_per_split"] >= k // 64 > (plan["k_splits"] - 1) * plan["k_tiles_per_split"], where
+    assert hip.gemm_bf16_tile_plan(100, 4096, 4096)["k_splits"] > 1       # a batch of 100 rows against a large weight
+    assert hip.gemm_bf16_tile_plan(4096, 4096, 4096)["k_splits"] == 1     # BASELINE config 4: 256 tiles of 256×256
+    with pytest.raises(hip.HipErr):
+        hip.gemm_bf16_tile_plan(128, 128, 100)                            # k not a multiple of 64: another kernel family
