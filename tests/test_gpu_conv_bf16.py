@@ -54,6 +54,10 @@ SHAPES = [
     (3, 192, 14, 14, 300, (3, 3), (1, 1), (1, 1), (1, 1)),  # three channel blocks, two row tiles of 256 channels
     (40, 64, 28, 28, 256, (3, 3), (1, 1), (1, 1), (1, 1)),  # 31360 pixels × 256 channels: the 256×256 tiles
     (2, 16, 7, 7, 8, (7, 7), (1, 1), (3, 3), (1, 1)),       # 49 taps
+    (17, 8, 55, 53, 70, (3, 3), (1, 1), (1, 1), (1, 1)),    # 49555 pixels (odd planes) × 70 channels: pixels on the 256-row side
+    (16, 128, 64, 64, 128, (1, 1), (1, 1), (0, 0), (1, 1)), # the same tiling, two channel blocks, one tap
+    (2, 3, 3, 1000, 4, (1, 3), (1, 1), (0, 1), (1, 1)),     # rows wider than the re-layout tile: copied in pieces
+    (1, 5, 40, 225, 6, (3, 3), (1, 2), (2, 2), (1, 1)),     # one row per re-layout group, several rows of padding
 ]
 
 
