@@ -1401,8 +1401,9 @@ __global__ __launch_bounds__(256) void conv_bf16_relayout_kernel(ConvBf16Relayou
         const int piece_w = min(TILE_W, w - x0), quads = (piece_w + 3) / 4;
         __syncthreads();
         if (row_inside) {
-            for (int idx = tid; idx < channels * quads; idx += 256) {
-                const int c = idx / quads, x = (idx - c * quads) * 4;
+            // sixteen lanes per channel row, four pixels each; sixteen channels per pass
+            for (int c = tid >> 4; c < channels; c += 16)
+            for (int x = (tid & 15) * 4; x < quads * 4; x += 64) {
                 const uint16_t *src = p.in + ((static_cast<size_t>(image) * p.c_in + cb * 64 + c) * p.h + y) * w + x0 + x;
                 uint16_t v[4] = {0, 0, 0, 0};
                 if (x + 4 <= piece_w) {
