@@ -47,6 +47,7 @@ MEASURED_TRAFFIC_BYTES = {
     "conv2d_bias_relu_f32_n32_c64to128_56x56_k3s1p1": (14291 * 2 + 50176) * 1024,
     "conv2d_grad_input_f32_n32_c64to128_56x56_k3s1p1": ((32964 + 660) * 2 + 25088 + 288) * 1024,
     "conv2d_grad_weight_f32_n32_c64to128_56x56_k3s1p1": ((44170 + 36161) * 2 + 72288 + 288) * 1024,
+    "conv2d_bias_relu_bf16_f32acc_n32_c64to128_56x56_k3s1p1": ((12703 + 8123) * 2 + 13600 + 50176) * 1024,
     "gemm_bf16_f32acc_4096x4096x4096": (98511 * 2 + 65536) * 1024,
     "gemm_bf16_f32acc_4096x4096x4096_prepacked_rhs": (98406 * 2 + 65536) * 1024,
     "gemm_bf16_f32acc_16x4096x4096": ((16927 + 1045) * 2 + 2048 + 256) * 1024,
@@ -436,6 +437,29 @@ def wl_lopsided(hip, inputs, timer):
     return out
 
 
+def wl_decoder_gemms(hip, inputs, timer):
+    """The four projections of one decoder layer on their own (config 5's shapes: 16384 tokens, d_model 512, 2048-wide
+    MLP; bf16 operands prepacked as the decoder holds them), so that profiles can attribute counters to each: QKV
+    (bf16 out: the persistent kernel), out-proj and fc2 (f32 out + residual), fc1 (GELU, bf16 out)."""
+    T, d, ff = 16384, 512, 2048
+    out = []
+    d_res = hip.DeviceBuffer.from_array(inputs.normal(inputs.seed_for(5, 7), T * d))
+    for name, n, k, act, residual, out16 in (("qkv", 3 * d, d, 0, False, True), ("out_proj", d, d, 0, True, False),
+                                             ("fc1_gelu", ff, d, 2, False, True), ("fc2", d, ff, 0, True, False)):
+        d_a = hip.DeviceBuffer.from_array(inputs.to_bf16(inputs.normal(inputs.seed_for(5, 8), T * k)))
+        d_b = hip.DeviceBuffer.from_array(inputs.to_bf16(inputs.normal(inputs.seed_for(5, 9), k * n, 0.0, 0.02)))
+        d_packed = hip.DeviceBuffer(k * n * 2)
+        hip.pack_rhs_bf16_dev(k, n, d_b, d_packed)
+        d_bias = hip.DeviceBuffer.from_array(inputs.normal(inputs.seed_for(5, 10), n, 0.0, 0.02))
+        d32 = None if out16 else hip.DeviceBuffer(T * n * 4)
+        d16 = hip.DeviceBuffer(T * n * 2) if out16 else None
+        step = lambda st: hip.gemm_bf16_prepacked_bias_act_dev(T, n, k, act, d_a, d_packed, d_bias, d_res if residual else None, d32, d16, st)
+        wall, ev, sus = timer.measure(step)
+        bytes_ = 2 * (T * k + k * n) + (2 if out16 else 4) * T * n + (4 * T * n if residual else 0)
+        out.append(entry(f"decoder_gemm_{name}_bf16_{T}x{n}x{k}", "bf16", 2 * T * n * k, bytes_, "mfma", wall, ev, sustained=sus))
+    return out
+
+
 def wl_calibration(hip, inputs, timer):
     """Plain streaming kernel of known traffic (f32 -> bf16 rounding of 64 Mi values: 256 MiB read, 128 MiB
     written).  It anchors the FETCH_SIZE / WRITE_SIZE counters and shows the HBM rate a trivial kernel reaches."""
@@ -687,6 +711,7 @@ def main():
     # Not BASELINE configurations: stderr lines only, and only when asked for.
     extra_plan = [
         ("gemm_f32_4096", lambda: wl_gemm_f32(hip, inputs, timer, 4096, 4096, 4096, "gemm_f32_4096x4096x4096", long=True)),
+        ("decoder_gemms", lambda: wl_decoder_gemms(hip, inputs, timer)),
         ("rowops", lambda: wl_rowops(hip, inputs, timer)),
         ("lopsided", lambda: wl_lopsided(hip, inputs, timer)),
         ("calibration", lambda: wl_calibration(hip, inputs, timer)),
