@@ -294,9 +294,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 64 ? (
 // -------------------------------------------------------------------------------------------------
 // head_dim 64: the same arithmetic in the same order as the kernel above (bit for bit the same output), with K and V
 // going straight from global memory into LDS (buffer_load ... lds: no staging registers, no LDS write instructions).
-// A stage is 64 rows of 128 bytes with the 16-byte chunks XOR-swizzled: chunk q of K row r sits at q ^ (r & 7) (the
-// 128-bit fragment reads of eight consecutive rows then cover all banks), chunk q of V row r at q ^ 4·((r >> 1) & 1)
-// (the four rows × 64 bytes one pass of a transposing read touches then cover all banks).
+// A stage is 64 rows of 128 bytes with the 16-byte chunks XOR-swizzled: chunk q of K row r sits at q ^ ((r >> 1) & 7):
+// a 128-bit fragment read serves sixteen lanes — sixteen consecutive rows — per cycle from 64 banks, a row is 32 banks
+// long, so rows 2i and 2i+1 lie on different bank halves and need the same shift, and the eight pairs eight different
+// ones (with q ^ (r & 7), rows r and r + 8 met on the same banks: 32 % of the LDS cycles were bank conflicts).  Chunk q
+// of V row r sits at q ^ 4·((r >> 1) & 1) (the four rows × 64 bytes one pass of a transposing read touches then cover
+// all banks).
 // -------------------------------------------------------------------------------------------------
 typedef __attribute__((address_space(3))) void *lds_void_ptr16;
 
@@ -360,7 +363,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     for (int i = 0; i < 2; ++i) {
         const int r = (i * 4 + wave) * 8 + (lane >> 3);
         const int c = lane & 7;
-        k_voff[i] = static_cast<unsigned>(r) * row_bytes + static_cast<unsigned>((c ^ (r & 7)) * 16);
+        k_voff[i] = static_cast<unsigned>(r) * row_bytes + static_cast<unsigned>((c ^ ((r >> 1) & 7)) * 16);
         v_voff[i] = static_cast<unsigned>(r) * row_bytes + static_cast<unsigned>((c ^ (((r >> 1) & 1) * 4)) * 16);
     }
     auto load_stage = [&](int stage) {
@@ -379,7 +382,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     // within each 16-lane group lane i16 supplies row i16/4 and 8-byte piece i16%4 of a 4-row × 16-column block.
     unsigned k_read[KC];
 #pragma unroll
-    for (int c = 0; c < KC; ++c) k_read[c] = static_cast<unsigned>(li * 128 + (((2 * c + lh) ^ (li & 7)) * 16));
+    for (int c = 0; c < KC; ++c) k_read[c] = static_cast<unsigned>(li * 128 + (((2 * c + lh) ^ ((li >> 1) & 7)) * 16));
     const int i16 = lane & 15, c16 = (lane >> 4) & 1;
     unsigned v_read[DT];
 #pragma unroll
