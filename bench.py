@@ -479,6 +479,7 @@ def probe_ceilings(hip, inputs, timer):
     """What frames the bf16 GEMM figures on this box, measured in this process (stderr lines only, with --probes):
     (1) a loop of bf16 matrix instructions alone, on all-zero and on N(0, 0.02^2) register operands: the rate the matrix
         pipes sustain on those bits with no memory instruction in the way (power, hence clock, depends on the bits);
+    (1b) a loop of direct-to-LDS loads alone: what a compute unit streams out of L2, the memory-side cache and HBM;
     (2) the vendor library (torch.mm -> hipBLASLt) on config 4's operands, B row-major (NN) and transposed (NT), under
         the same two protocols as the workloads.  torch is imported for this probe only; nothing else here uses it."""
     out = []
@@ -491,6 +492,18 @@ def probe_ceilings(hip, inputs, timer):
         flops = 256 * 4 * iterations * 32 * 2 * 32 * 32 * 16
         out.append({"probe": f"mfma_bf16_32x32x16_only_{label}", "kernel_ms": round(ev, 4),
                     "tflops": round(flops / (ev * 1e-3) / 1e12, 1), "frac_of_bf16_peak": round(flops / (ev * 1e-3) / 1e12 / PEAK_TFLOPS["bf16"], 4)})
+    # (1b) a loop of direct-to-LDS loads in the GEMM kernels' access shape, one workgroup per compute unit, over a region
+    #      that fits every XCD's L2 (2 MiB), only the memory-side cache (64 MiB), or neither (1 GiB)
+    for label, mib in (("l2_2mib", 2), ("memory_side_cache_64mib", 64), ("hbm_1gib", 1024)):
+        region_bytes = mib << 20
+        d_region = hip.DeviceBuffer(region_bytes)
+        d_region.zero()  # every page touched; the values do not matter to a load
+        iterations = 400  # 256 workgroups x 8 wavefronts x 400 x 8 KB = 6.7 GB per launch
+        _, ev = timer.run(lambda st: hip.probe_stream_lds_dev(256, iterations, d_region, region_bytes, st), 2, 5)
+        total = 256 * 8 * iterations * 8192
+        out.append({"probe": f"direct_to_lds_stream_{label}", "kernel_ms": round(ev, 4), "tb_per_s": round(total / (ev * 1e-3) / 1e12, 2),
+                    "gb_per_s_per_compute_unit": round(total / 256 / (ev * 1e-3) / 1e9, 1)})
+        del d_region
     # this library's prepacked kernel with bf16 as the only output: what the vendor library's bf16-out figures compare with
     m = n = k = 4096
     d_a = hip.DeviceBuffer.from_array(inputs.to_bf16(inputs.normal(inputs.seed_for(4, 0), m * k, 0.0, 0.02)))

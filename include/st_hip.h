@@ -409,6 +409,11 @@ int st_hip_merge_heads_f32_dev(size_t batch, size_t seq, size_t heads, size_t he
  * optimised away.  What the matrix pipes deliver on given operand bits with no memory instruction in the way — the
  * ceiling bench.py --probes reports beside the bf16 GEMM.  No reference counterpart. */
 int st_hip_probe_mfma_bf16_dev(size_t workgroups, size_t iterations, const uint16_t *operands, float *sink, void *stream);
+/* A loop of nothing but direct-to-LDS loads: `workgroups` × 8 wavefronts each fetch 8·iterations KB of `region` (device,
+ * region_bytes from 64 KiB to below 2 GiB) in the access shape of a bf16 operand k-tile (eight 128-byte rows, 1 KB apart, per
+ * instruction; 8 to 16 KB in flight per wavefront), walking all of the region: the rate one compute unit streams at out of
+ * L2, the memory-side cache or HBM, depending on region_bytes.  Nothing is written.  No reference counterpart. */
+int st_hip_probe_stream_lds_dev(size_t workgroups, size_t iterations, const void *region, size_t region_bytes, void *stream);
 
 /* ---- byte-level decoder stack (built from the ops above) ------------------------------------ */
 typedef struct {

@@ -502,6 +502,15 @@ int st_hip_probe_mfma_bf16_dev(size_t workgroups, size_t iterations, const uint1
     return launch_status(launch_probe_mfma_bf16(workgroups, iterations, operands, sink, as_stream(stream)), "mfma probe launch");
 }
 
+int st_hip_probe_stream_lds_dev(size_t workgroups, size_t iterations, const void *region, size_t region_bytes, void *stream)
+{
+    ST_HIP_CHECK(ensure_init());
+    if (!region) return fail(ST_HIP_ERR_INVALID, "stream probe received a null pointer");
+    if (region_bytes < 65536 || region_bytes >= (1ull << 31))
+        return fail(ST_HIP_ERR_UNSUPPORTED, "stream probe takes a region of 64 KiB to below 2 GiB (received %zu bytes)", region_bytes);
+    return launch_status(launch_probe_stream_lds(workgroups, iterations, region, region_bytes, as_stream(stream)), "stream probe launch");
+}
+
 int st_hip_gemm_bf16_tile_plan(size_t m, size_t n, size_t k, st_hip_gemm_tile_plan *plan)
 {
     if (!plan) return fail(ST_HIP_ERR_INVALID, "gemm tile_plan received a null out-pointer");

@@ -1,7 +1,9 @@
 // Measurement aids that are part of the library so that benchmarks and profiles run committed code only: a loop of
 // nothing but bf16 matrix instructions on register operands.  It shows what the matrix pipes of this chip deliver on
 // given operand bits with no memory instruction in the way (the clock a chip settles at under matrix load depends on
-// how many operand bits toggle), i.e. the ceiling the bf16 GEMM kernels are to be read against.
+// how many operand bits toggle), i.e. the ceiling the bf16 GEMM kernels are to be read against; and a loop of nothing
+// but direct-to-LDS loads, which shows what one compute unit can stream out of L2, the memory-side cache or HBM
+// (depending on the size of the region it walks) with the GEMM kernels' own access shape.
 #include "kernels.h"
 
 namespace sthip {
@@ -47,7 +49,48 @@ __global__ __launch_bounds__(256) void probe_mfma_bf16_kernel(const u32x4 *opera
     sink[static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x] = total;
 }
 
+typedef __attribute__((address_space(3))) void *probe_lds_ptr;
+
+// Eight wavefronts per workgroup; per iteration a wavefront issues eight buffer_load_dwordx4 ... lds of 1 KB — eight
+// rows of 128 B at a row pitch of 1 KB, the shape of a bf16 operand k-tile at K = 512 — and waits for the eight of the
+// iteration before, so 8 to 16 KB per wavefront are in flight.  Workgroups start at different places of the region and
+// walk all of it.
+__global__ __launch_bounds__(512) void probe_stream_lds_kernel(const unsigned char *region, unsigned region_bytes, int iterations)
+{
+    extern __shared__ __attribute__((aligned(16))) unsigned char probe_lds[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const __amdgpu_buffer_rsrc_t rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char *>(region), 0, static_cast<int>(region_bytes), 0x00020000);
+    const unsigned voff = (lane >> 3) * 1024u + (lane & 7) * 16u;
+    const unsigned span = region_bytes - 8192u;  // a batch covers 8 KB from its first byte
+    unsigned pos = (blockIdx.x * 7919u * 8192u + wave * 8192u) % span;
+    for (int it = 0; it < iterations; ++it) {
+#pragma unroll
+        for (int d = 0; d < 8; ++d)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (probe_lds_ptr)(probe_lds + wave * 8192 + d * 1024), 16, voff,
+                                                     __builtin_amdgcn_readfirstlane(pos + d * 128u), 0, 0);
+        pos = (pos + 8u * 8192u) % span;
+        __builtin_amdgcn_s_waitcnt(8 | (7 << 4) | (15 << 8));  // vmcnt(8): the batch before this one has landed
+    }
+    __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8));
+}
+
 }  // namespace
+
+hipError_t launch_probe_stream_lds(size_t workgroups, size_t iterations, const void *region, size_t region_bytes, hipStream_t stream)
+{
+    if (workgroups == 0 || iterations == 0) return hipSuccess;
+    if (workgroups > 0x7fffffffu || iterations > 0x7fffffffu || region_bytes < 65536 || region_bytes >= (1ull << 31))
+        return hipErrorInvalidValue;
+    constexpr size_t lds_bytes = 8 * 8192;
+    hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void *>(probe_stream_lds_kernel),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
+    if (rc != hipSuccess) return rc;
+    hipLaunchKernelGGL(probe_stream_lds_kernel, dim3(static_cast<unsigned>(workgroups)), dim3(512), lds_bytes, stream,
+                       static_cast<const unsigned char *>(region), static_cast<unsigned>(region_bytes), static_cast<int>(iterations));
+    return hipGetLastError();
+}
 
 hipError_t launch_probe_mfma_bf16(size_t workgroups, size_t iterations, const uint16_t *operands, float *sink, hipStream_t stream)
 {
