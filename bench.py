@@ -492,6 +492,13 @@ def probe_ceilings(hip, inputs, timer):
         flops = 256 * 4 * iterations * 32 * 2 * 32 * 32 * 16
         out.append({"probe": f"mfma_bf16_32x32x16_only_{label}", "kernel_ms": round(ev, 4),
                     "tflops": round(flops / (ev * 1e-3) / 1e12, 1), "frac_of_bf16_peak": round(flops / (ev * 1e-3) / 1e12 / PEAK_TFLOPS["bf16"], 4)})
+    for label, values in (("zeros", np.zeros(4096, np.float32)), ("normal_1", inputs.normal(inputs.seed_for(2, 3), 4096, 0.0, 1.0))):
+        d_ops = hip.DeviceBuffer.from_array(values.astype(np.float32))
+        iterations = 4000
+        _, ev = timer.run(lambda st: hip.probe_mfma_f32_dev(256, iterations, d_ops, sink, st), 2, 10)
+        flops = 256 * 4 * iterations * 32 * 2 * 32 * 32 * 2
+        out.append({"probe": f"mfma_f32_32x32x2_only_{label}", "kernel_ms": round(ev, 4),
+                    "tflops": round(flops / (ev * 1e-3) / 1e12, 1), "frac_of_f32_peak": round(flops / (ev * 1e-3) / 1e12 / PEAK_TFLOPS["f32"], 4)})
     # (1b) a loop of direct-to-LDS loads in the GEMM kernels' access shape, one workgroup per compute unit, over a region
     #      that fits every XCD's L2 (2 MiB), only the memory-side cache (64 MiB), or neither (1 GiB)
     for label, mib in (("l2_2mib", 2), ("memory_side_cache_64mib", 64), ("hbm_1gib", 1024)):

@@ -409,6 +409,9 @@ int st_hip_merge_heads_f32_dev(size_t batch, size_t seq, size_t heads, size_t he
  * optimised away.  What the matrix pipes deliver on given operand bits with no memory instruction in the way — the
  * ceiling bench.py --probes reports beside the bf16 GEMM.  No reference counterpart. */
 int st_hip_probe_mfma_bf16_dev(size_t workgroups, size_t iterations, const uint16_t *operands, float *sink, void *stream);
+/* The same with the f32 matrix instruction (v_mfma_f32_32x32x2_f32, 2·32·32·2 flop each) of the f32 GEMM, convolution and
+ * attention kernels; `operands` holds 4096 f32 values.  No reference counterpart. */
+int st_hip_probe_mfma_f32_dev(size_t workgroups, size_t iterations, const float *operands, float *sink, void *stream);
 /* A loop of nothing but direct-to-LDS loads: `workgroups` × 8 wavefronts each fetch 8·iterations KB of `region` (device,
  * region_bytes from 64 KiB to below 2 GiB) in the access shape of a bf16 operand k-tile (eight 128-byte rows, 1 KB apart, per
  * instruction; 8 to 16 KB in flight per wavefront), walking all of the region: the rate one compute unit streams at out of

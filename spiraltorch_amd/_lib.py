@@ -100,6 +100,7 @@ SIGNATURES = {
     "st_hip_attention_f32_launch_plan": (c_int, [c_size_t, c_size_t, c_size_t, c_int, c_int, POINTER(AttentionPlan)]),
     "st_hip_gemm_row_block": (c_size_t, [c_size_t, c_size_t]),
     "st_hip_probe_mfma_bf16_dev": (c_int, [c_size_t, c_size_t, c_void_p, c_void_p, c_void_p]),
+    "st_hip_probe_mfma_f32_dev": (c_int, [c_size_t, c_size_t, c_void_p, c_void_p, c_void_p]),
     "st_hip_probe_stream_lds_dev": (c_int, [c_size_t, c_size_t, c_void_p, c_size_t, c_void_p]),
     "st_hip_gemm_bf16_tile_plan": (c_int, [c_size_t, c_size_t, c_size_t, POINTER(GemmTilePlan)]),
     "st_hip_conv2d_bias_act_f32": (c_int, [c_size_t] * 13 + [c_int, c_void_p, c_size_t, c_void_p, c_size_t,

@@ -502,6 +502,13 @@ int st_hip_probe_mfma_bf16_dev(size_t workgroups, size_t iterations, const uint1
     return launch_status(launch_probe_mfma_bf16(workgroups, iterations, operands, sink, as_stream(stream)), "mfma probe launch");
 }
 
+int st_hip_probe_mfma_f32_dev(size_t workgroups, size_t iterations, const float *operands, float *sink, void *stream)
+{
+    ST_HIP_CHECK(ensure_init());
+    if (!operands || !sink) return fail(ST_HIP_ERR_INVALID, "mfma probe received a null pointer");
+    return launch_status(launch_probe_mfma_f32(workgroups, iterations, operands, sink, as_stream(stream)), "mfma probe launch");
+}
+
 int st_hip_probe_stream_lds_dev(size_t workgroups, size_t iterations, const void *region, size_t region_bytes, void *stream)
 {
     ST_HIP_CHECK(ensure_init());

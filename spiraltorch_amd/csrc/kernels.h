@@ -159,6 +159,7 @@ hipError_t launch_sum_axis0_f32(size_t rows, size_t cols, const float *in, float
 // Measurement aid: `workgroups` × 4 wavefronts each issue 32·iterations bf16 32x32x16 matrix instructions on register
 // operands read once from `operands` (32768 bf16 values); sink receives workgroups·256 floats.
 hipError_t launch_probe_mfma_bf16(size_t workgroups, size_t iterations, const uint16_t *operands, float *sink, hipStream_t stream);
+hipError_t launch_probe_mfma_f32(size_t workgroups, size_t iterations, const float *operands, float *sink, hipStream_t stream);
 hipError_t launch_probe_stream_lds(size_t workgroups, size_t iterations, const void *region, size_t region_bytes, hipStream_t stream);
 
 // One grow-only device buffer per (stream, host thread) for kernels that need scratch memory (split-k partial sums,

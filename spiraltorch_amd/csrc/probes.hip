@@ -49,6 +49,41 @@ __global__ __launch_bounds__(256) void probe_mfma_bf16_kernel(const u32x4 *opera
     sink[static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x] = total;
 }
 
+// The same for the f32 matrix instruction of the f32 GEMM, convolution and attention kernels: four wavefronts per
+// workgroup, 2 × 4 A and B values per lane (v_mfma_f32_32x32x2_f32 takes one f32 per lane and operand), 32 instructions
+// per iteration into sixteen independent accumulators.
+__global__ __launch_bounds__(256) void probe_mfma_f32_kernel(const float *operands, float *sink, int iterations)
+{
+    f32x16 acc[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][r] = 0.0f;
+    float a[2][4], b[2][4];
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            a[s][i] = operands[threadIdx.x + 256 * (s * 8 + i)];
+            b[s][i] = operands[threadIdx.x + 256 * (s * 8 + 4 + i)];
+        }
+    for (int it = 0; it < iterations; ++it) {
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    acc[i * 4 + j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s][i], b[s][j], acc[i * 4 + j], 0, 0, 0);
+    }
+    float total = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) total += acc[i][r];
+    sink[static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x] = total;
+}
+
 typedef __attribute__((address_space(3))) void *probe_lds_ptr;
 
 // Eight wavefronts per workgroup; per iteration a wavefront issues eight buffer_load_dwordx4 ... lds of 1 KB — eight
@@ -89,6 +124,15 @@ hipError_t launch_probe_stream_lds(size_t workgroups, size_t iterations, const v
     if (rc != hipSuccess) return rc;
     hipLaunchKernelGGL(probe_stream_lds_kernel, dim3(static_cast<unsigned>(workgroups)), dim3(512), lds_bytes, stream,
                        static_cast<const unsigned char *>(region), static_cast<unsigned>(region_bytes), static_cast<int>(iterations));
+    return hipGetLastError();
+}
+
+hipError_t launch_probe_mfma_f32(size_t workgroups, size_t iterations, const float *operands, float *sink, hipStream_t stream)
+{
+    if (workgroups == 0 || iterations == 0) return hipSuccess;
+    if (workgroups > 0x7fffffffu || iterations > 0x7fffffffu) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(probe_mfma_f32_kernel, dim3(static_cast<unsigned>(workgroups)), dim3(256), 0, stream, operands, sink,
+                       static_cast<int>(iterations));
     return hipGetLastError();
 }
 

@@ -510,6 +510,11 @@ def probe_mfma_bf16_dev(workgroups, iterations, operands, sink, stream=None) -> 
     _check(_lib.load().st_hip_probe_mfma_bf16_dev(workgroups, iterations, _dev(operands), _dev(sink), _stream_ptr(stream)))
 
 
+def probe_mfma_f32_dev(workgroups, iterations, operands, sink, stream=None) -> None:
+    """A loop of f32 matrix instructions on register operands (measurement aid; see st_hip_probe_mfma_f32_dev)."""
+    _check(_lib.load().st_hip_probe_mfma_f32_dev(workgroups, iterations, _dev(operands), _dev(sink), _stream_ptr(stream)))
+
+
 def probe_stream_lds_dev(workgroups, iterations, region, region_bytes, stream=None) -> None:
     """A loop of direct-to-LDS loads over a device region (measurement aid; see st_hip_probe_stream_lds_dev)."""
     _check(_lib.load().st_hip_probe_stream_lds_dev(workgroups, iterations, _dev(region), region_bytes, _stream_ptr(stream)))

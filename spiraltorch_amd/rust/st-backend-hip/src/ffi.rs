@@ -145,6 +145,7 @@ extern "C" {
     pub fn st_hip_split_heads_f32_dev(batch: usize, seq: usize, heads: usize, head_dim: usize, qkv: *const f32, q: *mut f32, k: *mut f32, v: *mut f32, stream: *mut c_void) -> c_int;
     pub fn st_hip_merge_heads_f32_dev(batch: usize, seq: usize, heads: usize, head_dim: usize, contexts_in: *const f32, out_f32: *mut f32, out_bf16: *mut u16, stream: *mut c_void) -> c_int;
     pub fn st_hip_probe_mfma_bf16_dev(workgroups: usize, iterations: usize, operands: *const u16, sink: *mut f32, stream: *mut c_void) -> c_int;
+    pub fn st_hip_probe_mfma_f32_dev(workgroups: usize, iterations: usize, operands: *const f32, sink: *mut f32, stream: *mut c_void) -> c_int;
     pub fn st_hip_probe_stream_lds_dev(workgroups: usize, iterations: usize, region: *const c_void, region_bytes: usize, stream: *mut c_void) -> c_int;
     pub fn st_hip_decoder_weight_count(config: *const StHipDecoderConfig) -> usize;
     pub fn st_hip_decoder_create(config: *const StHipDecoderConfig, host_weights: *const f32, weight_len: usize, decoder: *mut *mut c_void) -> c_int;
