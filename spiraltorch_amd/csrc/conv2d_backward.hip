@@ -222,7 +222,12 @@ struct GradWeightArgs {
 // are fixed for the whole kernel) are fetched into registers while the MFMAs of the previous step run, then written to
 // the other LDS stage.  The big tile (TM = 2, TN = 3: 128 × 192, three of which span a 3×3 layer's 576 columns exactly
 // for 64 input channels) reads 5 fragments per 24 MFMAs instead of 2 per 4.
-template <bool VEC, int TM, int TN>
+//
+// SETS > 1: the workgroup is SETS such groups of four wavefronts working on the same tile.  Each takes its own run of
+// steps (chunk·SETS + set) through LDS stages of its own; at the end the sets' accumulators are added through LDS in
+// the order ((0 + 1) + 2) and set 0 stores the one partial tile — a third of the partial tiles, of the bytes the
+// chunk reduction reads back, and of the store burst at the end of the launch, for the same wavefronts per SIMD.
+template <bool VEC, int TM, int TN, int SETS = 1>
 __device__ __forceinline__ void conv_grad_weight_body(const GradWeightArgs &p, float *As, float *Bs)
 {
     constexpr int BM = 64 * TM, BN = 64 * TN, BK = 16;
@@ -231,7 +236,13 @@ __device__ __forceinline__ void conv_grad_weight_body(const GradWeightArgs &p, f
     constexpr int A_STRIDE = BK + 4, B_STRIDE = BK + 4;
     constexpr int A_STAGE = BM * A_STRIDE, B_STAGE = BN * B_STRIDE;
 
-    const int tid = threadIdx.x;
+    const int set = SETS > 1 ? __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 8)) : 0;
+    float *const lds_all = As;  // (SETS > 1: As is the start of the workgroup's LDS, [set][A stages | B stages])
+    if constexpr (SETS > 1) {
+        As = lds_all + set * (2 * A_STAGE + 2 * B_STAGE);
+        Bs = As + 2 * A_STAGE;
+    }
+    const int tid = threadIdx.x & 255;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: the pixel bookkeeping below stays off the VALU
     const int wm = wave >> 1, wn = wave & 1;
@@ -248,7 +259,7 @@ __device__ __forceinline__ void conv_grad_weight_body(const GradWeightArgs &p, f
     bid /= p.tiles_s;
     const int tiles_oc = (s.c_out + BM - 1) / BM;
     const int tile_oc = bid % tiles_oc;
-    const int chunk = bid / tiles_oc;
+    const int chunk = (bid / tiles_oc) * SETS + set;
     const int oc0 = tile_oc * BM, s0 = tile_s * BN;
 
     // This thread's patch columns (lane + 64·j) and their fixed taps.
@@ -412,15 +423,53 @@ __device__ __forceinline__ void conv_grad_weight_body(const GradWeightArgs &p, f
         store_lds(0);
     }
     __syncthreads();
-    for (int t = 0; t < total_steps; ++t) {
+    // (SETS > 1: every set goes through the barriers of the longest run; a set whose run is shorter idles.)
+    const int barrier_steps = SETS > 1 ? p.steps_per_chunk : total_steps;
+    for (int t = 0; t < barrier_steps; ++t) {
         const bool more = t + 1 < total_steps;
         if (more) load_global();
-        compute(t & 1);
+        if (t < total_steps) compute(t & 1);
         if (more) store_lds((t + 1) & 1);
         __syncthreads();
     }
 
-    float *dst = p.partial + static_cast<size_t>(chunk) * s.c_out * p.S;
+    if constexpr (SETS > 1) {
+        // Thread t's 16·TM·TN accumulator values as 128-bit pieces e at (e·256 + t)·16 bytes: conflict-free both ways.
+        static_assert(TM * TN * 16 * 256 * 4 <= SETS * (2 * A_STAGE + 2 * B_STAGE) * 4, "the tile fits the workgroup's LDS");
+        f32x4 *exchange = reinterpret_cast<f32x4 *>(lds_all);
+#pragma unroll
+        for (int other = 1; other < SETS; ++other) {
+            if (set == other) {
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q)
+                            exchange[((i * TN + j) * 4 + q) * 256 + tid] =
+                                f32x4{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+            }
+            __syncthreads();
+            if (set == 0) {
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            const f32x4 v = exchange[((i * TN + j) * 4 + q) * 256 + tid];
+                            acc[i][j][4 * q] += v[0];
+                            acc[i][j][4 * q + 1] += v[1];
+                            acc[i][j][4 * q + 2] += v[2];
+                            acc[i][j][4 * q + 3] += v[3];
+                        }
+            }
+            __syncthreads();
+        }
+        if (set != 0) return;
+    }
+
+    float *dst = p.partial + static_cast<size_t>(SETS > 1 ? chunk / SETS : chunk) * s.c_out * p.S;
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
         const int out_col = s0 + wn * 32 * TN + j * 32 + li;
@@ -452,6 +501,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     __shared__ __attribute__((aligned(16))) float As[2 * 128 * 20];
     __shared__ __attribute__((aligned(16))) float Bs[2 * 192 * 20];
     conv_grad_weight_body<VEC, 2, 3>(p, As, Bs);
+}
+
+// The same tile with three sets of four wavefronts in one workgroup (one workgroup per compute unit, 153,600 B of LDS).
+template <bool VEC>
+__global__ __launch_bounds__(768) __attribute__((amdgpu_waves_per_eu(3, 3))) void conv_grad_weight_big3_kernel(GradWeightArgs p)
+{
+    extern __shared__ __attribute__((aligned(16))) float grad_weight_lds[];
+    conv_grad_weight_body<VEC, 2, 3, 3>(p, grad_weight_lds, nullptr);
 }
 
 }  // namespace
@@ -614,6 +671,9 @@ hipError_t launch_conv2d_grad_weight_f32(const ConvShape &shape, const float *in
     if (chunks < 1) chunks = 1;
     args.steps_per_chunk = static_cast<int>(total_steps > 0 ? (total_steps + chunks - 1) / chunks : 1);
     chunks = total_steps > 0 ? (total_steps + args.steps_per_chunk - 1) / args.steps_per_chunk : 1;
+    // Big tiles with at least three runs of steps per tile: three runs share a workgroup (and a partial tile).
+    const bool three_sets = big && chunks >= 3;
+    if (three_sets) chunks = (chunks + 2) / 3;
     void *workspace = nullptr;
     hipError_t rc = stream_workspace(stream, static_cast<size_t>(chunks) * count * sizeof(float), &workspace);
     if (rc != hipSuccess) return rc;
@@ -623,7 +683,14 @@ hipError_t launch_conv2d_grad_weight_f32(const ConvShape &shape, const float *in
     if (workgroups > 0x7ffffff0u) return hipErrorInvalidConfiguration;
     args.workgroups = static_cast<int>(workgroups);
     const dim3 grid(static_cast<unsigned>((workgroups + 7) / 8 * 8));
-    if (big && vec)
+    if (three_sets) {
+        constexpr size_t lds_bytes = 3 * (2 * 128 * 20 + 2 * 192 * 20) * sizeof(float);
+        auto kernel = vec ? conv_grad_weight_big3_kernel<true> : conv_grad_weight_big3_kernel<false>;
+        rc = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                 static_cast<int>(lds_bytes));
+        if (rc != hipSuccess) return rc;
+        hipLaunchKernelGGL(kernel, grid, dim3(768), lds_bytes, stream, args);
+    } else if (big && vec)
         hipLaunchKernelGGL(conv_grad_weight_big_kernel<true>, grid, dim3(256), 0, stream, args);
     else if (big)
         hipLaunchKernelGGL(conv_grad_weight_big_kernel<false>, grid, dim3(256), 0, stream, args);

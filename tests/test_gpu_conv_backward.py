@@ -26,6 +26,10 @@ CASES = [
     (1, 24, 10, 10, 192, (7, 7), (1, 1), (3, 3), (1, 1)),  # c_out*kh*kw = 9408: more than one offset-table segment
     (1, 20, 11, 11, 180, (7, 7), (2, 2), (3, 3), (1, 1)),  # stride 2, 8820 terms: GEMM + col2im
     (1, 128, 11, 11, 180, (7, 7), (1, 2), (3, 3), (1, 1)), # the same through the adjoint gather (whole channel tile, stride 1×2)
+    # grad_weight with three runs of steps per workgroup (128 × 192 tiles, at least three runs per tile):
+    (1, 64, 25, 25, 128, (3, 3), (1, 1), (1, 1), (1, 1)),  # 40 runs of one step: the last workgroup has one busy set of three
+    (7, 64, 33, 31, 128, (3, 3), (1, 1), (1, 1), (1, 1)),  # 224 runs of two steps: the last workgroup has two busy sets
+    (2, 128, 12, 12, 256, (3, 3), (1, 1), (1, 1), (1, 1)), # twelve tiles (two channel tiles × six column tiles), 18 runs
 ]
 
 
