@@ -46,7 +46,7 @@ PEAK_HBM_GBS = 8000.0
 MEASURED_TRAFFIC_BYTES = {
     "conv2d_bias_relu_f32_n32_c64to128_56x56_k3s1p1": (14291 * 2 + 50176) * 1024,
     "conv2d_grad_input_f32_n32_c64to128_56x56_k3s1p1": ((32964 + 660) * 2 + 25088 + 288) * 1024,
-    "conv2d_grad_weight_f32_n32_c64to128_56x56_k3s1p1": ((44170 + 36161) * 2 + 72288 + 288) * 1024,
+    "conv2d_grad_weight_f32_n32_c64to128_56x56_k3s1p1": ((44801 + 12109) * 2 + 24192 + 288) * 1024,
     "conv2d_bias_relu_bf16_f32acc_n32_c64to128_56x56_k3s1p1": ((12703 + 8123) * 2 + 13600 + 50176) * 1024,
     "gemm_bf16_f32acc_4096x4096x4096": (98511 * 2 + 65536) * 1024,
     "gemm_bf16_f32acc_4096x4096x4096_prepacked_rhs": (98406 * 2 + 65536) * 1024,
