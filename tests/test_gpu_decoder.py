@@ -54,6 +54,15 @@ def test_embedding_split_merge_and_rounding(hip, oracle):
     hip.embedding_f32_dev(many.size, 4, 72, hip.DeviceBuffer.from_array(many), hip.DeviceBuffer.from_array(wide), d_wide)
     hip.device_synchronize()
     assert (d_wide.to_array(np.float32, many.size * 72) == oracle.embedding_f32(many.size, 4, 72, many, wide)).all()
+    # two token rows per wavefront (rows of up to 2048 values; an odd number of tokens), and the per-piece gather beyond
+    rng = np.random.default_rng(4)
+    for tokens, vocab, dim in ((509, 256, 512), (33, 7, 2048), (5, 3, 2052), (1, 2, 4)):
+        table_n = rng.normal(size=vocab * dim).astype(np.float32)
+        ids_n = rng.uniform(-2, vocab + 2, tokens).astype(np.float32)
+        d_n = hip.DeviceBuffer(tokens * dim * 4)
+        hip.embedding_f32_dev(tokens, vocab, dim, hip.DeviceBuffer.from_array(ids_n), hip.DeviceBuffer.from_array(table_n), d_n)
+        hip.device_synchronize()
+        assert (d_n.to_array(np.float32, tokens * dim) == oracle.embedding_f32(tokens, vocab, dim, ids_n, table_n)).all(), (tokens, vocab, dim)
 
     vals = np.random.default_rng(0).normal(size=1000).astype(np.float32)
     # ties (round to even in both directions), the largest finite value, infinities, denormals and signed zero
