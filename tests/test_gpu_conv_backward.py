@@ -261,6 +261,33 @@ def test_config2_shape_adjoint_identity(hip):
     assert_close(gb, want_gb, 1e-4, 1e-4, "grad_bias")
 
 
+def test_config2_grad_weight_sampled_entries_against_float64(hip):
+    """BASELINE config 2 at full size through the kernel its shape takes (three runs of steps per workgroup, 251 runs: the
+    last workgroup has two busy sets): 96 entries of grad_weight — every tap, the first and last channels of both kinds,
+    and random ones — against their definition in float64,
+    grad_weight[o, c, ky, kx] = scale · Σ_{n, y, x} grad_output[n, o, y, x] · input[n, c, y + ky − 1, x + kx − 1]."""
+    from spiraltorch_amd import inputs
+    batch, c_in, h, w, c_out = 32, 64, 56, 56, 128
+    geom = ((3, 3), (1, 1), (1, 1), (1, 1))
+    x = inputs.normal(201, batch * c_in * h * w)
+    g = inputs.normal(202, batch * c_out * h * w)
+    d_gw = hip.DeviceBuffer(c_out * c_in * 9 * 4)
+    hip.conv2d_grad_weight_f32_dev(batch, c_in, h, w, c_out, *geom, hip.DeviceBuffer.from_array(x), hip.DeviceBuffer.from_array(g),
+                                   1.0 / batch, d_gw)
+    hip.device_synchronize()
+    gw = d_gw.to_array(np.float32, c_out * c_in * 9).reshape(c_out, c_in, 3, 3)
+    X = np.zeros((batch, c_in, h + 2, w + 2), np.float64)
+    X[:, :, 1:-1, 1:-1] = x.reshape(batch, c_in, h, w)
+    G = g.reshape(batch, c_out, h, w).astype(np.float64)
+    rng = np.random.default_rng(5)
+    entries = [(o, c, ky, kx) for (o, c) in ((0, 0), (127, 63)) for ky in range(3) for kx in range(3)]
+    entries += [(int(rng.integers(c_out)), int(rng.integers(c_in)), int(rng.integers(3)), int(rng.integers(3))) for _ in range(78)]
+    got = np.array([gw[e] for e in entries], np.float64)
+    want = np.array([float((G[:, o] * X[:, c, ky:ky + h, kx:kx + w]).sum()) / batch for (o, c, ky, kx) in entries])
+    assert_close(got, want, 1e-4, 1e-4, "config 2 grad_weight, sampled entries")
+    assert np.isfinite(gw).all()
+
+
 def test_validation(hip):
     gi, gw, gb = np.zeros(4, np.float32), np.zeros(1, np.float32), np.zeros(1, np.float32)
     with pytest.raises(hip.HipErr, match="grad_output buffer length 3"):
