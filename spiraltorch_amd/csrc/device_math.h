@@ -58,6 +58,20 @@ __device__ __forceinline__ float layer_norm_denominator(float var, float epsilon
     return denom < INFINITY ? denom : NAN;
 }
 
+// The two places of a layer-norm row where the compiler may or may not fuse a multiply with the addition behind it,
+// in separately rounded steps as the reference computes them (crates/st-tensor/src/pure.rs:4030-4056; Rust does not
+// contract): var = E[x²] − mean² clamped at 0, and normalised·γ + β.  Left to the compiler, two kernels that normalise
+// the same row (the stand-alone kernels, the GEMM kernel that normalises its own rows) could round one value in a million
+// differently.
+__device__ __forceinline__ float layer_norm_variance(float sumsq, float mean, float cols_f)
+{
+    return fmaxf(__fsub_rn(sumsq / cols_f, __fmul_rn(mean, mean)), 0.0f);
+}
+__device__ __forceinline__ float layer_norm_scale_shift(float normalised, float gamma, float beta)
+{
+    return __fadd_rn(__fmul_rn(normalised, gamma), beta);
+}
+
 // Runs `body(act, has_residual)` with the activation as a callable and the presence of a residual as a compile-time
 // constant, chosen once from the (wavefront-uniform) launch arguments: an epilogue that decides them per element
 // compiles to a chain of scalar branches around every store.

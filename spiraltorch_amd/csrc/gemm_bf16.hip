@@ -1088,7 +1088,7 @@ __device__ __forceinline__ void gemm_bf16_rowcomplete_body(const RowLnArgs &q)
         }
         const float cols_f = static_cast<float>(N);
         const float mean = sum / cols_f;
-        const float var = fmaxf(sumsq / cols_f - mean * mean, 0.0f);
+        const float var = layer_norm_variance(sumsq, mean, cols_f);
         const float denom = layer_norm_denominator(var, q.epsilon);
         // (v - mean) / denom with one division per row: the product with the reciprocal, corrected once by its exact
         // remainder, is the correctly rounded quotient (the stand-alone layer-norm kernel does the same).
@@ -1099,8 +1099,8 @@ __device__ __forceinline__ void gemm_bf16_rowcomplete_body(const RowLnArgs &q)
         };
         const float4 v = xs[j];
         uint2 packed;
-        packed.x = pack_bf16x2_rne(quotient(v.x - mean) * gamma4.x + beta4.x, quotient(v.y - mean) * gamma4.y + beta4.y);
-        packed.y = pack_bf16x2_rne(quotient(v.z - mean) * gamma4.z + beta4.z, quotient(v.w - mean) * gamma4.w + beta4.w);
+        packed.x = pack_bf16x2_rne(layer_norm_scale_shift(quotient(v.x - mean), gamma4.x, beta4.x), layer_norm_scale_shift(quotient(v.y - mean), gamma4.y, beta4.y));
+        packed.y = pack_bf16x2_rne(layer_norm_scale_shift(quotient(v.z - mean), gamma4.z, beta4.z), layer_norm_scale_shift(quotient(v.w - mean), gamma4.w, beta4.w));
         if (row < M) *reinterpret_cast<uint2 *>(q.ln_bf16 + static_cast<size_t>(row) * N + col0) = packed;
     }
 }

@@ -35,12 +35,12 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(int rows, int cols, con
     sumsq = wave_sum(sumsq);
     const float cols_f = static_cast<float>(cols);
     const float mean = sum / cols_f;
-    const float var = fmaxf(sumsq / cols_f - mean * mean, 0.0f);
+    const float var = layer_norm_variance(sumsq, mean, cols_f);
     const float denom = layer_norm_denominator(var, epsilon);
     for (int c = lane; c < cols; c += 64) {
         float v = x[offset + c];
         if (residual) v += residual[offset + c];
-        const float value = ((v - mean) / denom) * gamma[c] + beta[c];
+        const float value = layer_norm_scale_shift((v - mean) / denom, gamma[c], beta[c]);
         if (out_f32) out_f32[offset + c] = value;
         if (out_bf16) out_bf16[offset + c] = f32_to_bf16_rne(value);
     }
@@ -99,7 +99,7 @@ __global__ __launch_bounds__(256) void layer_norm_vec_kernel(int rows, int cols,
         sum = wave_sum(sum);
         sumsq = wave_sum(sumsq);
         const float mean = sum / cols_f;
-        const float var = fmaxf(sumsq / cols_f - mean * mean, 0.0f);
+        const float var = layer_norm_variance(sumsq, mean, cols_f);
         const float denom = layer_norm_denominator(var, epsilon);
         // (v - mean) / denom for every element, with one real division per row: the product with the correctly rounded
         // reciprocal, corrected once by its exact remainder (two fused multiply-adds), is the correctly rounded quotient
@@ -115,10 +115,10 @@ __global__ __launch_bounds__(256) void layer_norm_vec_kernel(int rows, int cols,
             const int c = (lane + 64 * i) * 4;
             if (c >= cols) continue;
             float4 o;
-            o.x = quotient(v[r][i].x - mean) * g[i].x + b[i].x;
-            o.y = quotient(v[r][i].y - mean) * g[i].y + b[i].y;
-            o.z = quotient(v[r][i].z - mean) * g[i].z + b[i].z;
-            o.w = quotient(v[r][i].w - mean) * g[i].w + b[i].w;
+            o.x = layer_norm_scale_shift(quotient(v[r][i].x - mean), g[i].x, b[i].x);
+            o.y = layer_norm_scale_shift(quotient(v[r][i].y - mean), g[i].y, b[i].y);
+            o.z = layer_norm_scale_shift(quotient(v[r][i].z - mean), g[i].z, b[i].z);
+            o.w = layer_norm_scale_shift(quotient(v[r][i].w - mean), g[i].w, b[i].w);
             if (out_f32) *reinterpret_cast<float4 *>(out_f32 + offset + c) = o;
             if (out_bf16) {
                 uint2 packed;
@@ -200,7 +200,7 @@ __global__ __launch_bounds__(1024) void layer_norm_block_kernel(int cols, const 
     sumsq = block_reduce<1024>(sumsq, scratch, add);
     const float cols_f = static_cast<float>(cols);
     const float mean = sum / cols_f;
-    const float var = fmaxf(sumsq / cols_f - mean * mean, 0.0f);
+    const float var = layer_norm_variance(sumsq, mean, cols_f);
     const float denom = layer_norm_denominator(var, epsilon);
     const float inv = 1.0f / denom;
     auto quotient = [&](float a) {  // a / denom, correctly rounded (see layer_norm_vec_kernel)
@@ -215,10 +215,10 @@ __global__ __launch_bounds__(1024) void layer_norm_block_kernel(int cols, const 
         if (c + 4 <= cols) {
             const f32x4_a4 g = *reinterpret_cast<const f32x4_a4 *>(gamma + c), b = *reinterpret_cast<const f32x4_a4 *>(beta + c);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) o[e] = quotient(v[i][e] - mean) * g[e] + b[e];
+            for (int e = 0; e < 4; ++e) o[e] = layer_norm_scale_shift(quotient(v[i][e] - mean), g[e], b[e]);
         } else {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) o[e] = c + e < cols ? quotient(v[i][e] - mean) * gamma[c + e] + beta[c + e] : 0.0f;
+            for (int e = 0; e < 4; ++e) o[e] = c + e < cols ? layer_norm_scale_shift(quotient(v[i][e] - mean), gamma[c + e], beta[c + e]) : 0.0f;
         }
         if (c + 4 <= cols) {
             if (out_f32) *reinterpret_cast<f32x4_a4 *>(out_f32 + offset + c) = f32x4_a4{o[0], o[1], o[2], o[3]};
@@ -275,7 +275,7 @@ __global__ __launch_bounds__(THREADS) void layer_norm_long_kernel(int cols, cons
     sumsq = block_reduce<THREADS>(sumsq, scratch, add);
     const float cols_f = static_cast<float>(cols);
     const float mean = sum / cols_f;
-    const float var = fmaxf(sumsq / cols_f - mean * mean, 0.0f);
+    const float var = layer_norm_variance(sumsq, mean, cols_f);
     const float denom = layer_norm_denominator(var, epsilon);
     const float inv = 1.0f / denom;
     auto quotient = [&](float a) {  // a / denom, correctly rounded (see layer_norm_vec_kernel)
@@ -287,7 +287,7 @@ __global__ __launch_bounds__(THREADS) void layer_norm_long_kernel(int cols, cons
         float v[W], o[W];
         load(c, v);
 #pragma unroll
-        for (int e = 0; e < W; ++e) o[e] = quotient(v[e] - mean) * gamma[c + e] + beta[c + e];
+        for (int e = 0; e < W; ++e) o[e] = layer_norm_scale_shift(quotient(v[e] - mean), gamma[c + e], beta[c + e]);
         if constexpr (VEC) {
             if (out_f32) *reinterpret_cast<float4 *>(out_f32 + offset + c) = make_float4(o[0], o[1], o[2], o[3]);
             if (out_bf16) {

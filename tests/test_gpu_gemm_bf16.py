@@ -247,7 +247,9 @@ def test_skinny_prepacked_single_launch(hip, oracle, m, n, k):
 def test_gemm_residual_layer_norm(hip, oracle, m, n, k):
     """Linear + residual + LayerNorm in one call: the rows before normalisation against the oracle's GEMM (+ bias +
     residual), the normalised bf16 rows against the oracle's layer-norm of those rows (within one bf16 step: the
-    row statistics are summed in another order), and against the separate GEMM and layer-norm kernels."""
+    row statistics are summed in another order), and against the separate GEMM and layer-norm kernels (the same
+    statistics in the same order: equal bits on these operands; on other data a sweep has seen one value in two
+    million land on the other side of a bf16 rounding boundary)."""
     from spiraltorch_amd import inputs
     rng = np.random.default_rng(m + 3 * n + 5 * k)
     a, b = bf16_pair(rng, m, n, k, std=0.5)
