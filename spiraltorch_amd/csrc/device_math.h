@@ -60,16 +60,22 @@ __device__ __forceinline__ float layer_norm_denominator(float var, float epsilon
 
 // The two places of a layer-norm row where the compiler may or may not fuse a multiply with the addition behind it,
 // in separately rounded steps as the reference computes them (crates/st-tensor/src/pure.rs:4030-4056; Rust does not
-// contract): var = E[x²] − mean² clamped at 0, and normalised·γ + β.  Left to the compiler, two kernels that normalise
-// the same row (the stand-alone kernels, the GEMM kernel that normalises its own rows) could round one value in a million
-// differently.
+// contract): var = E[x²] − mean² clamped at 0, and normalised·γ + β.  Contraction is switched off for these statements
+// (__fmul_rn and friends are plain operators here and fuse like any other): left to the compiler, the stand-alone
+// kernels fused both while the GEMM kernel that normalises its own rows fused only the second, the variances of a few
+// rows in a thousand differed in their last bit, and one value in two million came out one bf16 step apart.
 __device__ __forceinline__ float layer_norm_variance(float sumsq, float mean, float cols_f)
 {
-    return fmaxf(__fsub_rn(sumsq / cols_f, __fmul_rn(mean, mean)), 0.0f);
+#pragma clang fp contract(off)
+    const float mean_of_squares = sumsq / cols_f;
+    const float square_of_mean = mean * mean;
+    return fmaxf(mean_of_squares - square_of_mean, 0.0f);
 }
 __device__ __forceinline__ float layer_norm_scale_shift(float normalised, float gamma, float beta)
 {
-    return __fadd_rn(__fmul_rn(normalised, gamma), beta);
+#pragma clang fp contract(off)
+    const float scaled = normalised * gamma;
+    return scaled + beta;
 }
 
 // Runs `body(act, has_residual)` with the activation as a callable and the presence of a residual as a compile-time

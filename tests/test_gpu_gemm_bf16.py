@@ -248,8 +248,7 @@ def test_gemm_residual_layer_norm(hip, oracle, m, n, k):
     """Linear + residual + LayerNorm in one call: the rows before normalisation against the oracle's GEMM (+ bias +
     residual), the normalised bf16 rows against the oracle's layer-norm of those rows (within one bf16 step: the
     row statistics are summed in another order), and against the separate GEMM and layer-norm kernels (the same
-    statistics in the same order: equal bits on these operands; on other data a sweep has seen one value in two
-    million land on the other side of a bf16 rounding boundary)."""
+    arithmetic in the same order: equal bits)."""
     from spiraltorch_amd import inputs
     rng = np.random.default_rng(m + 3 * n + 5 * k)
     a, b = bf16_pair(rng, m, n, k, std=0.5)
@@ -523,3 +522,63 @@ def test_prepacked_f32_output_over_many_rounds_of_tiles_with_a_short_k(hip, orac
     elif activation == 2:
         want = 0.5 * want * (1.0 + np.tanh(0.7978846 * (want + 0.044715 * want ** 3)))
     assert_close(got.reshape(m, n)[rows].ravel(), want.ravel(), BF16_REL, 2e-5 * max(1.0, float(np.abs(base).max())), "sampled rows")
+
+
+def test_layer_norm_routes_round_alike_next_to_a_bf16_boundary(hip):
+    """A row a randomised sweep found (tests/golden/layer_norm_row_near_bf16_boundary.npz: 512 values, gamma, beta): with
+    E[x²] − mean² and normalised·γ + β in separately rounded steps — the reference's arithmetic — element 481 lands exactly on
+    a bf16 rounding boundary (0xbd6e8000 → 0xbd6e); a fused multiply-add in either place moves it by 2 or 7 ulps, and when
+    the stand-alone kernel fused both and the GEMM kernel that normalises its own rows only the second, the two routes
+    came out one bf16 step apart.  Both routes against an f32 emulation of the arithmetic, operation by operation."""
+    import os
+    from spiraltorch_amd import inputs
+    row = np.load(os.path.join(os.path.dirname(__file__), "golden", "layer_norm_row_near_bf16_boundary.npz"))
+    x, gamma, beta = row["x"], row["gamma"], row["beta"]
+    n, eps = 512, np.float32(1e-5)
+    f32 = np.float32
+
+    def fma(a, b, c):  # the product of two f32 is exact in f64
+        return f32(np.float64(a) * np.float64(b) + np.float64(c))
+
+    lane_sum, lane_sq = [], []
+    for lane in range(64):  # lane L of the row's wavefront holds columns 4L.. and 256 + 4L..
+        s, q = f32(0), f32(0)
+        for i in range(2):
+            v = x[(lane + 64 * i) * 4:(lane + 64 * i) * 4 + 4]
+            s = f32(s + f32(f32(v[0] + v[1]) + f32(v[2] + v[3])))
+            q = f32(q + f32(fma(v[0], v[0], f32(v[1] * v[1])) + fma(v[2], v[2], f32(v[3] * v[3]))))
+        lane_sum.append(s)
+        lane_sq.append(q)
+    for offset in (32, 16, 8, 4, 2, 1):  # the exchanges over 32, 16, ... 1 lanes
+        lane_sum = [f32(lane_sum[i] + lane_sum[i ^ offset]) for i in range(64)]
+        lane_sq = [f32(lane_sq[i] + lane_sq[i ^ offset]) for i in range(64)]
+    mean = f32(lane_sum[0] / f32(n))
+    var = max(f32(f32(lane_sq[0] / f32(n)) - f32(mean * mean)), f32(0))
+    denom = f32(np.sqrt(np.float64(f32(var + eps))))
+    inv = f32(f32(1) / denom)
+    want = np.zeros(n, np.float32)
+    for c in range(n):
+        a = f32(x[c] - mean)
+        t = f32(a * inv)
+        quotient = fma(fma(-t, denom, a), inv, t)  # the correctly rounded a / denom
+        want[c] = f32(f32(quotient * gamma[c]) + beta[c])
+    assert want[481:482].view(np.uint32)[0] == 0xbd6e8000
+
+    rows = 130  # more than 64: the fused call takes the kernel that normalises its own rows
+    d_x = hip.DeviceBuffer.from_array(np.tile(x, rows))
+    d_g, d_b = hip.DeviceBuffer.from_array(gamma), hip.DeviceBuffer.from_array(beta)
+    d_f32, d_16 = hip.DeviceBuffer(rows * n * 4), hip.DeviceBuffer(rows * n * 2)
+    hip.layer_norm_f32_dev(rows, n, d_x, None, d_g, d_b, float(eps), d_f32, d_16)
+    hip.device_synchronize()
+    got = d_f32.to_array(np.float32, rows * n).reshape(rows, n)
+    assert (got == want[None, :]).all(), "stand-alone layer norm, f32"
+    assert (d_16.to_array(np.uint16, rows * n).reshape(rows, n) == inputs.to_bf16(want)[None, :]).all(), "stand-alone layer norm, bf16"
+    # the GEMM route: a zero product, so that the rows before normalisation are the residual rows exactly
+    k = 64
+    d_a = hip.DeviceBuffer.from_array(np.zeros(rows * k, np.uint16))
+    d_w = hip.DeviceBuffer.from_array(inputs.to_bf16(np.random.default_rng(0).normal(size=n * k).astype(np.float32)))
+    x32, ln16 = hip.DeviceBuffer(rows * n * 4), hip.DeviceBuffer(rows * n * 2)
+    hip.gemm_bf16_prepacked_residual_layer_norm_dev(rows, n, k, d_a, d_w, None, d_x, d_g, d_b, float(eps), x32, ln16)
+    hip.device_synchronize()
+    assert (x32.to_array(np.float32, rows * n).reshape(rows, n) == x[None, :]).all()
+    assert (ln16.to_array(np.uint16, rows * n).reshape(rows, n) == inputs.to_bf16(want)[None, :]).all(), "GEMM + residual + layer norm"
