@@ -108,7 +108,11 @@ def set_gains(weights, vocab, d, layers, ff):
     return w
 
 
-@pytest.mark.parametrize("cfg", [(32, 16, 2, 2, 24, 2, 9), (256, 128, 2, 2, 256, 2, 160)])
+@pytest.mark.parametrize("cfg", [(32, 16, 2, 2, 24, 2, 9), (256, 128, 2, 2, 256, 2, 160),
+                                 # heads of 24 (f32 attention over split heads), of 128 at d_model 1024, and of 4 with one token
+                                 (100, 96, 4, 2, 100, 3, 65), (300, 1024, 8, 2, 24, 1, 257), (7, 4, 1, 3, 8, 4, 1),
+                                 # a vocabulary that is no multiple of the GEMM tile, an MLP wider than the model by 16
+                                 (1000, 128, 2, 2, 2048, 1, 200)])
 def test_decoder_matches_the_oracle(hip, oracle, cfg):
     vocab, d, heads, layers, ff, batch, seq = cfg
     weights, tokens = decoder_case(*cfg, seed=500)
