@@ -196,11 +196,18 @@ int st_hip_decoder_forward_dev(void *decoder, const float *tokens, float *logits
         if (st_launch_rc_ != hipSuccess) return hip_fail(st_launch_rc_, ctx); \
     } while (0)
 
-    ST_LAUNCH(launch_embedding_f32(T, c.vocab, d, tokens, dec.embed, dec.x, stream), "embedding launch");
+    // The lookup and the layer norm that reads it (the first layer's, or the final one of a stack without layers) are
+    // one launch: the embedded rows go to the residual stream and, normalised, to the first GEMM's operand.
+    const float *first_gamma = dec.layers.empty() ? dec.lnf_g : dec.layers.front().ln1_g;
+    const float *first_beta = dec.layers.empty() ? dec.lnf_b : dec.layers.front().ln1_b;
+    ST_LAUNCH(launch_embedding_layer_norm_f32(T, c.vocab, d, tokens, dec.embed, dec.x, first_gamma, first_beta, c.ln_eps,
+                                              dec.h16, stream),
+              "embedding + layer_norm launch");
     for (const LayerWeights &w : dec.layers) {
         GemmEpilogue ep;
-        ST_LAUNCH(launch_layer_norm_f32(T, d, dec.x, nullptr, w.ln1_g, w.ln1_b, c.ln_eps, nullptr, dec.h16, stream),
-                  "layer_norm launch");
+        if (&w != &dec.layers.front())
+            ST_LAUNCH(launch_layer_norm_f32(T, d, dec.x, nullptr, w.ln1_g, w.ln1_b, c.ln_eps, nullptr, dec.h16, stream),
+                      "layer_norm launch");
         ep = GemmEpilogue();
         ep.bias = w.b_qkv;
         if (dec.fused_attention) {
@@ -236,8 +243,9 @@ int st_hip_decoder_forward_dev(void *decoder, const float *tokens, float *logits
         ep.residual = dec.x2;
         ST_LAUNCH(launch_gemm_bf16(T, d, ff, dec.u16, w.w_fc2, dec.x, nullptr, ep, stream, true), "fc2 gemm launch");
     }
-    ST_LAUNCH(launch_layer_norm_f32(T, d, dec.x, nullptr, dec.lnf_g, dec.lnf_b, c.ln_eps, nullptr, dec.h16, stream),
-              "layer_norm launch");
+    if (!dec.layers.empty())
+        ST_LAUNCH(launch_layer_norm_f32(T, d, dec.x, nullptr, dec.lnf_g, dec.lnf_b, c.ln_eps, nullptr, dec.h16, stream),
+                  "layer_norm launch");
     GemmEpilogue head;
     head.bias = dec.b_head;
     ST_LAUNCH(launch_gemm_bf16(T, c.vocab, d, dec.h16, dec.w_head, logits, nullptr, head, stream, true), "head gemm launch");

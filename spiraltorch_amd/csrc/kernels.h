@@ -136,6 +136,9 @@ hipError_t launch_attention_bf16(size_t batch, size_t heads, size_t sequence, si
 hipError_t launch_layer_norm_f32(size_t rows, size_t cols, const float *x, const float *residual,
                                  const float *gamma, const float *beta, float epsilon, float *out_f32,
                                  uint16_t *out_bf16, hipStream_t stream);
+hipError_t launch_embedding_layer_norm_f32(size_t tokens, size_t vocab, size_t dim, const float *token_ids, const float *table,
+                                           float *embedded, const float *gamma, const float *beta, float epsilon,
+                                           uint16_t *out_bf16, hipStream_t stream);
 hipError_t launch_embedding_f32(size_t tokens, size_t vocab, size_t dim, const float *token_ids,
                                 const float *table, float *out, hipStream_t stream);
 hipError_t launch_f32_to_bf16(size_t count, const float *in, uint16_t *out, hipStream_t stream);

@@ -7,6 +7,19 @@ namespace sthip {
 
 namespace {
 
+// A token id stored as f32 -> a row of the table: rounded to the nearest integer, clamped to [0, vocab - 1], anything
+// that is not finite to row 0 (token_to_index, crates/st-nn/src/layers/embedding.rs:325-330).
+__device__ __forceinline__ int token_to_index(float value, int vocab)
+{
+    int index = 0;
+    if (isfinite(value)) {
+        const float rounded = roundf(value);
+        if (rounded > 0.0f) index = rounded >= static_cast<float>(vocab) ? vocab - 1 : static_cast<int>(rounded);
+        if (index > vocab - 1) index = vocab - 1;
+    }
+    return index;
+}
+
 __device__ __forceinline__ float wave_sum(float v)
 {
 #pragma unroll
@@ -48,10 +61,19 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(int rows, int cols, con
 
 // Same, for rows of at most 2048 values with 16-byte aligned rows: the row is read once, 128 bits per lane, and
 // stays in registers between the statistics and the normalisation.
-template <int CHUNKS, int ROWS>
+// GATHER: row r of the input is row token_to_index(token_ids[r]) of the table `x` (an embedding lookup,
+// crates/st-nn/src/layers/embedding.rs:42-100), which is also written to `gathered` as it passes: the lookup and the
+// layer norm that follows it in a pre-norm stack as one launch, the same arithmetic on the same values in the same order.
+struct RowGather {
+    const float *token_ids;
+    float *gathered;
+    int vocab;
+};
+
+template <int CHUNKS, int ROWS, bool GATHER = false>
 __global__ __launch_bounds__(256) void layer_norm_vec_kernel(int rows, int cols, const float *x, const float *residual,
                                                              const float *gamma, const float *beta, float epsilon,
-                                                             float *out_f32, uint16_t *out_bf16)
+                                                             float *out_f32, uint16_t *out_bf16, RowGather gather)
 {
     // A wavefront takes ROWS consecutive rows and has all their loads in flight before the first reduction: with one
     // short row per wavefront the launch is bound by the latency of that one load, not by bandwidth.
@@ -62,12 +84,17 @@ __global__ __launch_bounds__(256) void layer_norm_vec_kernel(int rows, int cols,
 #pragma unroll
     for (int r = 0; r < ROWS; ++r) {
         const size_t offset = static_cast<size_t>(row0 + r) * cols;
+        size_t source = offset;
+        if constexpr (GATHER) {
+            if (row0 + r < rows) source = static_cast<size_t>(token_to_index(gather.token_ids[row0 + r], gather.vocab)) * cols;
+        }
 #pragma unroll
         for (int i = 0; i < CHUNKS; ++i) {
             const int c = (lane + 64 * i) * 4;
             v[r][i] = make_float4(0.f, 0.f, 0.f, 0.f);
             if (c < cols && row0 + r < rows) {
-                v[r][i] = *reinterpret_cast<const float4 *>(x + offset + c);
+                v[r][i] = *reinterpret_cast<const float4 *>(x + source + c);
+                if constexpr (GATHER) *reinterpret_cast<float4 *>(gather.gathered + offset + c) = v[r][i];
                 if (residual) {
                     const float4 q = *reinterpret_cast<const float4 *>(residual + offset + c);
                     v[r][i].x += q.x; v[r][i].y += q.y; v[r][i].z += q.z; v[r][i].w += q.w;
@@ -311,12 +338,7 @@ __global__ __launch_bounds__(256) void embedding_kernel(int tokens, int vocab, i
     const int token = blockIdx.x;
     if (token >= tokens) return;
     const float value = token_ids[token];
-    int index = 0;
-    if (isfinite(value)) {
-        const float rounded = roundf(value);
-        if (rounded > 0.0f) index = rounded >= static_cast<float>(vocab) ? vocab - 1 : static_cast<int>(rounded);
-        if (index > vocab - 1) index = vocab - 1;
-    }
+    const int index = token_to_index(value, vocab);
     const float *src = table + static_cast<size_t>(index) * dim;
     float *dst = out + static_cast<size_t>(token) * dim;
     for (int c = threadIdx.x; c < dim; c += 256) dst[c] = src[c];
@@ -332,12 +354,7 @@ __global__ __launch_bounds__(256) void embedding_vec_kernel(size_t chunks, int v
     const size_t token = i / static_cast<size_t>(dim4);
     const int c = static_cast<int>(i - token * dim4);
     const float value = token_ids[token];
-    int index = 0;
-    if (isfinite(value)) {
-        const float rounded = roundf(value);
-        if (rounded > 0.0f) index = rounded >= static_cast<float>(vocab) ? vocab - 1 : static_cast<int>(rounded);
-        if (index > vocab - 1) index = vocab - 1;
-    }
+    const int index = token_to_index(value, vocab);
     out[i] = table[static_cast<size_t>(index) * dim4 + c];
 }
 
@@ -1025,19 +1042,19 @@ hipError_t launch_layer_norm_f32(size_t rows, size_t cols, const float *x, const
     const dim3 grid2(static_cast<unsigned>((rows + 7) / 8));
     if (vec && cols <= 512 && two_rows)
         hipLaunchKernelGGL((layer_norm_vec_kernel<2, 2>), grid2, block, 0, stream, r, c, x, residual, gamma, beta, epsilon,
-                           out_f32, out_bf16);
+                           out_f32, out_bf16, RowGather{});
     else if (vec && cols <= 512)
         hipLaunchKernelGGL((layer_norm_vec_kernel<2, 1>), grid, block, 0, stream, r, c, x, residual, gamma, beta, epsilon,
-                           out_f32, out_bf16);
+                           out_f32, out_bf16, RowGather{});
     else if (vec && cols <= 1024 && two_rows)
         hipLaunchKernelGGL((layer_norm_vec_kernel<4, 2>), grid2, block, 0, stream, r, c, x, residual, gamma, beta, epsilon,
-                           out_f32, out_bf16);
+                           out_f32, out_bf16, RowGather{});
     else if (vec && cols <= 1024)
         hipLaunchKernelGGL((layer_norm_vec_kernel<4, 1>), grid, block, 0, stream, r, c, x, residual, gamma, beta, epsilon,
-                           out_f32, out_bf16);
+                           out_f32, out_bf16, RowGather{});
     else if (vec)
         hipLaunchKernelGGL((layer_norm_vec_kernel<8, 1>), grid, block, 0, stream, r, c, x, residual, gamma, beta, epsilon,
-                           out_f32, out_bf16);
+                           out_f32, out_bf16, RowGather{});
     else if (cols > 4096 && cols <= 65536) {
         // The row in the registers of a 1024-thread workgroup: 2 to 16 pieces of 16 bytes per thread.
         const dim3 rows_grid(static_cast<unsigned>(rows));
@@ -1065,6 +1082,37 @@ hipError_t launch_layer_norm_f32(size_t rows, size_t cols, const float *x, const
     } else
         hipLaunchKernelGGL(layer_norm_kernel, grid, block, 0, stream, r, c, x, residual, gamma, beta, epsilon, out_f32,
                            out_bf16);
+    return hipGetLastError();
+}
+
+// Embedding lookup followed by the layer norm of the looked-up rows: `embedded` receives the rows (the residual stream
+// of a pre-norm stack), `out_bf16` their layer norm.  One launch where the 128-bit row kernel applies, two otherwise;
+// same values either way.
+hipError_t launch_embedding_layer_norm_f32(size_t tokens, size_t vocab, size_t dim, const float *token_ids, const float *table,
+                                           float *embedded, const float *gamma, const float *beta, float epsilon,
+                                           uint16_t *out_bf16, hipStream_t stream)
+{
+    if (tokens == 0 || dim == 0) return hipSuccess;
+    const bool vec = dim % 4 == 0 && dim <= 2048 && aligned16(table) && aligned16(embedded) && aligned16(gamma) && aligned16(beta) &&
+                     (reinterpret_cast<uintptr_t>(out_bf16) & 7u) == 0 && tokens < 0x7fffffffull && vocab < 0x7fffffffull;
+    if (!vec) {
+        const hipError_t rc = launch_embedding_f32(tokens, vocab, dim, token_ids, table, embedded, stream);
+        if (rc != hipSuccess) return rc;
+        return launch_layer_norm_f32(tokens, dim, embedded, nullptr, gamma, beta, epsilon, nullptr, out_bf16, stream);
+    }
+    const RowGather gather{token_ids, embedded, static_cast<int>(vocab)};
+    const int r = static_cast<int>(tokens), c = static_cast<int>(dim);
+    const dim3 grid(static_cast<unsigned>((tokens + 3) / 4)), grid2(static_cast<unsigned>((tokens + 7) / 8)), block(256);
+    const bool two_rows = tokens >= 8192;  // the same choice of kernel as launch_layer_norm_f32: the same sums in the same order
+#define ST_LN_GATHER(CHUNKS, ROWS, GRID)                                                                                  \
+    hipLaunchKernelGGL((layer_norm_vec_kernel<CHUNKS, ROWS, true>), GRID, block, 0, stream, r, c, table, nullptr, gamma, beta, \
+                       epsilon, nullptr, out_bf16, gather)
+    if (dim <= 512 && two_rows) ST_LN_GATHER(2, 2, grid2);
+    else if (dim <= 512) ST_LN_GATHER(2, 1, grid);
+    else if (dim <= 1024 && two_rows) ST_LN_GATHER(4, 2, grid2);
+    else if (dim <= 1024) ST_LN_GATHER(4, 1, grid);
+    else ST_LN_GATHER(8, 1, grid);
+#undef ST_LN_GATHER
     return hipGetLastError();
 }
 

@@ -160,6 +160,39 @@ def test_config5_full_shape_sampled_sequences(hip, oracle):
         assert_close(got[index], want[slot], BF16_REL, BF16_REL * rms, f"config 5, sequence {index}")
 
 
+@pytest.mark.parametrize("vocab,d,batch,seq", [(256, 512, 9, 1000), (100, 1024, 2, 50), (50, 2048, 1, 7), (50, 2052, 3, 7), (30, 96, 4, 33),
+                                               (1000, 256, 8200, 1)])
+def test_a_stack_without_layers_is_lookup_layer_norm_and_head(hip, vocab, d, batch, seq):
+    """The decoder looks its tokens up and normalises them in one launch.  With no layers in between, its logits must
+    be, bit for bit, what the separate entry points give: embedding, layer norm to bf16, the head projection on the
+    packed bf16 weight.  Token ids outside the vocabulary, negative and NaN included."""
+    from spiraltorch_amd import inputs
+    heads, ff = next(h for h in range(1, d + 1) if d % h == 0 and d // h <= 128), 8
+    count = hip.Decoder.weight_count(vocab, d, heads, 0, ff)
+    assert count == vocab * d + 2 * d + d * vocab + vocab
+    weights = inputs.normal(77, count, 0.0, 0.5)
+    tokens = inputs.tokens(78, batch * seq, vocab).copy()
+    tokens[:4] = [vocab + 5.0, -3.0, np.nan, 1.5]
+    rows = batch * seq
+    dec = hip.Decoder(vocab, d, heads, 0, ff, batch, seq, 1e-5, weights)
+    d_tok = hip.DeviceBuffer.from_array(tokens)
+    d_logits = hip.DeviceBuffer(rows * vocab * 4)
+    dec.forward_dev(d_tok, d_logits)
+    hip.device_synchronize()
+    got = d_logits.to_array(np.float32, rows * vocab)
+
+    table, rest = weights[:vocab * d], weights[vocab * d:]
+    gamma, beta, w_head, b_head = rest[:d], rest[d:2 * d], rest[2 * d:2 * d + d * vocab], rest[2 * d + d * vocab:]
+    d_x, d_h16, d_out = hip.DeviceBuffer(rows * d * 4), hip.DeviceBuffer(rows * d * 2), hip.DeviceBuffer(rows * vocab * 4)
+    hip.embedding_f32_dev(rows, vocab, d, d_tok, hip.DeviceBuffer.from_array(table), d_x)
+    hip.layer_norm_f32_dev(rows, d, d_x, None, hip.DeviceBuffer.from_array(gamma), hip.DeviceBuffer.from_array(beta), 1e-5, None, d_h16)
+    packed = np.ascontiguousarray(inputs.to_bf16(w_head).reshape(d, vocab).T)
+    hip.gemm_bf16_prepacked_bias_act_dev(rows, vocab, d, 0, d_h16, hip.DeviceBuffer.from_array(packed),
+                                         hip.DeviceBuffer.from_array(b_head), None, d_out, None)
+    hip.device_synchronize()
+    assert (got == d_out.to_array(np.float32, rows * vocab)).all()
+
+
 def test_decoder_validation(hip):
     with pytest.raises(hip.HipErr, match="not divisible"):
         hip.Decoder(32, 10, 3, 1, 8, 1, 4, 1e-5, np.zeros(hip.Decoder.weight_count(32, 10, 3, 1, 8), np.float32))
