@@ -167,8 +167,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 64 ? (
     const float scale_log2e = fmaxf(fabsf(p.scale) * kLog2e16, 1e-30f);
     const float lag = 8.0f / scale_log2e;  // 2^8 in units of the raw dot product
     // NT = number of 32-key tiles of this stage this wavefront works on (1 or 2).
-    auto compute = [&](auto nt_tag, int stage, int key0) {
+    // MAY_MASK = false: the caller knows that every key of the stage exists and (causal) lies at or below every query
+    // row of this wavefront.
+    auto compute = [&](auto nt_tag, auto may_mask_tag, int stage, int key0) {
         constexpr int NT = decltype(nt_tag)::value;
+        constexpr bool MAY_MASK = decltype(may_mask_tag)::value;
         const uint16_t *ks = Ks + stage * K_ELEMS;
         const uint16_t *vs = Vs + stage * V_ELEMS;
         f32x16 sacc[NT];
@@ -187,7 +190,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 64 ? (
         // The running maximum is kept in units of the raw dot product (scale >= 0 here), so the scale costs no pass
         // of its own: p = exp2(dot·scale·log2e − max·scale·log2e) is one fused multiply-add and one exp2.  Masking
         // only where a tile crosses the sequence end or the diagonal.
-        const bool need_mask = (key0 + NT * 32 > S) || (CAUSAL && key0 + NT * 32 - 1 > wq0);
+        const bool need_mask = MAY_MASK && ((key0 + NT * 32 > S) || (CAUSAL && key0 + NT * 32 - 1 > wq0));
         float tile_max = -INFINITY;
         if (need_mask) {
 #pragma unroll
@@ -262,14 +265,28 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 64 ? (
         store_lds(0);
     }
     __syncthreads();
-    for (int t = 0; t < stages; ++t) {
+    // The stages whose 64 keys all exist and need no causal mask for any row of this wavefront come first, in a loop
+    // with one path through it: a loop body that branches between the one-tile, the two-tile and the skipped form has
+    // the output accumulators merged after the branch, and the compiler then copies all of their registers twice per
+    // stage — behind the stage's last matrix instructions, whose latency the copies wait out.  The stages on and beyond
+    // the diagonal (two per workgroup at most) and a ragged last stage take the branching loop after it.
+    const int limit = CAUSAL ? min(S, wq0 + 32) : S;
+    const int plain_stages = min(stages, (CAUSAL ? min(S, wq0 + 1) : S) / BKV);
+    int t = 0;
+    for (; t < plain_stages; ++t) {
+        const bool more = t + 1 < stages;
+        if (more) load_global((t + 1) * BKV);
+        compute(std::integral_constant<int, 2>{}, std::false_type{}, t & 1, t * BKV);
+        if (more) store_lds((t + 1) & 1);
+        __syncthreads();
+    }
+    for (; t < stages; ++t) {
         const bool more = t + 1 < stages;
         if (more) load_global((t + 1) * BKV);
         const int key0 = t * BKV;
         // Tiles entirely past the sequence end or (causal) entirely above this wavefront's rows are skipped.
-        const int limit = CAUSAL ? min(S, wq0 + 32) : S;
-        if (key0 + 32 < limit) compute(std::integral_constant<int, 2>{}, t & 1, key0);
-        else if (key0 < limit) compute(std::integral_constant<int, 1>{}, t & 1, key0);
+        if (key0 + 32 < limit) compute(std::integral_constant<int, 2>{}, std::true_type{}, t & 1, key0);
+        else if (key0 < limit) compute(std::integral_constant<int, 1>{}, std::true_type{}, t & 1, key0);
         if (more) store_lds((t + 1) & 1);
         __syncthreads();
     }
@@ -437,8 +454,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     const float lag = 8.0f / scale_log2e;
 
     // NT = number of 32-key tiles of this stage this wavefront works on (1 or 2).
-    auto compute = [&](auto nt_tag, int stage, int key0) {
+    // MAY_MASK = false: the caller knows that every key of the stage exists and (causal) lies at or below every query
+    // row of this wavefront.
+    auto compute = [&](auto nt_tag, auto may_mask_tag, int stage, int key0) {
         constexpr int NT = decltype(nt_tag)::value;
+        constexpr bool MAY_MASK = decltype(may_mask_tag)::value;
         const unsigned char *ks = k_lds + stage * STAGE;
         f32x16 sacc[NT];
 #pragma unroll
@@ -452,7 +472,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 #pragma unroll
             for (int t = 0; t < NT; ++t) sacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[t], qf[c], sacc[t], 0, 0, 0);
         }
-        const bool need_mask = (key0 + NT * 32 > S) || (CAUSAL && key0 + NT * 32 - 1 > wq0);
+        const bool need_mask = MAY_MASK && ((key0 + NT * 32 > S) || (CAUSAL && key0 + NT * 32 - 1 > wq0));
         float tile_max = -INFINITY;
         if (need_mask) {
 #pragma unroll
@@ -517,14 +537,27 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     load_stage(0);
     __builtin_amdgcn_s_waitcnt(0x0070 | (15 << 8));  // vmcnt(0): Q and stage 0 have landed
     __syncthreads();
-    for (int t = 0; t < stages; ++t) {
+    // The stages whose 64 keys all exist and need no causal mask for any row of this wavefront come first, in a loop
+    // with one path through it: a loop body that branches between the one-tile, the two-tile and the skipped form has
+    // the output accumulators merged after the branch, and the compiler then copies all 32 of their registers twice
+    // per stage — behind the stage's last matrix instructions, whose latency the copies wait out.  The stages on and
+    // beyond the diagonal (two per workgroup at most) and a ragged last stage take the branching loop after it.
+    const int limit = CAUSAL ? min(S, wq0 + 32) : S;
+    const int plain_stages = min(stages, (CAUSAL ? min(S, wq0 + 1) : S) / BKV);
+    int t = 0;
+    for (; t < plain_stages; ++t) {
+        if (t + 1 < stages) load_stage(t + 1);
+        compute(std::integral_constant<int, 2>{}, std::false_type{}, t & 1, t * BKV);
+        __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0), lgkmcnt(0): the next stage has landed, this one has been read
+        __syncthreads();
+    }
+    for (; t < stages; ++t) {
         const bool more = t + 1 < stages;
         if (more) load_stage(t + 1);
         const int key0 = t * BKV;
-        const int limit = CAUSAL ? min(S, wq0 + 32) : S;
-        if (key0 + 32 < limit) compute(std::integral_constant<int, 2>{}, t & 1, key0);
-        else if (key0 < limit) compute(std::integral_constant<int, 1>{}, t & 1, key0);
-        __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0), lgkmcnt(0): the next stage has landed, this one has been read
+        if (key0 + 32 < limit) compute(std::integral_constant<int, 2>{}, std::true_type{}, t & 1, key0);
+        else if (key0 < limit) compute(std::integral_constant<int, 1>{}, std::true_type{}, t & 1, key0);
+        __builtin_amdgcn_s_waitcnt(0x0070);
         __syncthreads();
     }
 
