@@ -350,7 +350,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DPAD <= 64 
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // the same in every lane, and known to be
     const int li = lane & 31, lh = lane >> 5;
     const int S = p.S, D = p.D;
 
@@ -440,8 +440,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DPAD <= 64 
     const float *ab_row = BIAS && p.attn_bias && my_q < S
                               ? p.attn_bias + (static_cast<size_t>(ctx) * S + my_q) * static_cast<size_t>(S) : nullptr;
     // NT = number of 32-key tiles of this stage this wavefront works on (1 or 2).
-    auto compute = [&](auto nt_tag, int stage, int key0) {
+    // MAY_MASK = false: the caller knows that every key of the stage exists and (causal) lies at or below every query
+    // row of this wavefront.
+    auto compute = [&](auto nt_tag, auto may_mask_tag, int stage, int key0) {
         constexpr int NT = decltype(nt_tag)::value;
+        constexpr bool MAY_MASK = decltype(may_mask_tag)::value;
         const float *ks = Ks + stage * K_ELEMS;
         const float *vs = Vs + stage * V_ELEMS;
         f32x16 sacc[NT];
@@ -494,7 +497,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DPAD <= 64 
                 }
         }
         // logits in log2 units; the masking code only runs where a tile crosses the sequence end or the diagonal
-        const bool need_mask = (key0 + NT * 32 > S) || (CAUSAL && key0 + NT * 32 - 1 > wq0);
+        const bool need_mask = MAY_MASK && ((key0 + NT * 32 > S) || (CAUSAL && key0 + NT * 32 - 1 > wq0));
         float tile_max = -INFINITY;
         if (need_mask) {
 #pragma unroll
@@ -568,15 +571,31 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DPAD <= 64 
         store_lds(0);
     }
     __syncthreads();
-    for (int t = 0; t < stages; ++t) {
+    // The stages whose keys all exist and need no causal mask for any row of this wavefront come first, in a loop with
+    // one path through it: a loop body that branches between the one-tile, the two-tile and the skipped form has the
+    // output accumulators merged after the branch, and the compiler then copies all of their registers once per stage
+    // behind the stage's last matrix instructions, whose latency the copies wait out.  The stages on and beyond the
+    // diagonal, a ragged last stage and wavefronts whose rows lie past the sequence end take the branching loop after it.
+    static_assert(BKV == 64, "a stage is two 32-key tiles");
+    const int limit = wq0 >= S ? 0 : CAUSAL ? min(S, wq0 + 32) : S;
+    const int plain_end = wq0 >= S ? key_first : CAUSAL ? min(S, wq0 + 1) : S;
+    const int plain_stages = max(0, min(stages, (plain_end - key_first) / BKV));
+    int t = 0;
+    for (; t < plain_stages; ++t) {
+        const bool more = t + 1 < stages;
+        if (more) load_global(key_first + (t + 1) * BKV);
+        compute(std::integral_constant<int, 2>{}, std::false_type{}, t & 1, key_first + t * BKV);
+        if (more) store_lds((t + 1) & 1);
+        __syncthreads();
+    }
+    for (; t < stages; ++t) {
         const bool more = t + 1 < stages;
         if (more) load_global(key_first + (t + 1) * BKV);
         const int key0 = key_first + t * BKV;
         // Tiles entirely past the sequence end or (causal) entirely above this wavefront's rows are skipped.
         // So is everything in a wavefront whose 32 query rows lie past the sequence end (the last tile of 197 rows).
-        const int limit = wq0 >= S ? 0 : CAUSAL ? min(S, wq0 + 32) : S;
-        if (key0 + 32 < limit) compute(std::integral_constant<int, 2>{}, t & 1, key0);
-        else if (key0 < limit) compute(std::integral_constant<int, 1>{}, t & 1, key0);
+        if (key0 + 32 < limit) compute(std::integral_constant<int, 2>{}, std::true_type{}, t & 1, key0);
+        else if (key0 < limit) compute(std::integral_constant<int, 1>{}, std::true_type{}, t & 1, key0);
         if (more) store_lds((t + 1) & 1);
         __syncthreads();
     }
