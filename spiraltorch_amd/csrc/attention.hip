@@ -499,6 +499,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DPAD <= 64 
         // logits in log2 units; the masking code only runs where a tile crosses the sequence end or the diagonal
         const bool need_mask = MAY_MASK && ((key0 + NT * 32 > S) || (CAUSAL && key0 + NT * 32 - 1 > wq0));
         float tile_max = -INFINITY;
+        // the last key this lane's query sees: one comparison per score (a causal row never looks past the sequence end)
+        const int last_key = CAUSAL ? min(my_q, S - 1) : S - 1;
         if (need_mask) {
 #pragma unroll
             for (int t = 0; t < NT; ++t)
@@ -506,7 +508,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DPAD <= 64 
                 for (int r = 0; r < 16; ++r) {
                     const int key = key0 + t * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
                     float v = sacc[t][r];
-                    if (key >= S || (CAUSAL && key > my_q)) v = -INFINITY;
+                    if (key > last_key) v = -INFINITY;
                     sacc[t][r] = v;
                     tile_max = fmaxf(tile_max, v);
                 }

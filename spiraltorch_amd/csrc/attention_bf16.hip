@@ -192,6 +192,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 64 ? (
         // only where a tile crosses the sequence end or the diagonal.
         const bool need_mask = MAY_MASK && ((key0 + NT * 32 > S) || (CAUSAL && key0 + NT * 32 - 1 > wq0));
         float tile_max = -INFINITY;
+        // the last key this lane's query sees: one comparison per score (a causal row never looks past the sequence end)
+        const int last_key = CAUSAL ? min(my_q, S - 1) : S - 1;
         if (need_mask) {
 #pragma unroll
             for (int t = 0; t < NT; ++t)
@@ -199,7 +201,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 64 ? (
                 for (int r = 0; r < 16; ++r) {
                     const int key = key0 + t * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
                     float v = sacc[t][r];
-                    if (key >= S || (CAUSAL && key > my_q)) v = -INFINITY;
+                    if (key > last_key) v = -INFINITY;
                     sacc[t][r] = v;
                     tile_max = fmaxf(tile_max, v);
                 }
@@ -474,6 +476,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         }
         const bool need_mask = MAY_MASK && ((key0 + NT * 32 > S) || (CAUSAL && key0 + NT * 32 - 1 > wq0));
         float tile_max = -INFINITY;
+        // the last key this lane's query sees: one comparison per score (a causal row never looks past the sequence end)
+        const int last_key = CAUSAL ? min(my_q, S - 1) : S - 1;
         if (need_mask) {
 #pragma unroll
             for (int t = 0; t < NT; ++t)
@@ -481,7 +485,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
                 for (int r = 0; r < 16; ++r) {
                     const int key = key0 + t * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
                     float v = sacc[t][r];
-                    if (key >= S || (CAUSAL && key > my_q)) v = -INFINITY;
+                    if (key > last_key) v = -INFINITY;
                     sacc[t][r] = v;
                     tile_max = fmaxf(tile_max, v);
                 }
