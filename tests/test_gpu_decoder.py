@@ -158,6 +158,12 @@ def test_config5_full_shape_sampled_sequences(hip, oracle):
     rms = float(np.sqrt(np.mean(np.square(want))))
     for slot, index in enumerate(picked):
         assert_close(got[index], want[slot], BF16_REL, BF16_REL * rms, f"config 5, sequence {index}")
+        # The elementwise bar is met with little to spare: the difference to the f32 oracle is noise from the bf16
+        # rounding of every GEMM operand, 0.45–0.47 % of the logits' rms on every sequence and seed measured, and the
+        # largest of a sequence's 262144 values lies between 0.91 and 1.00 of the bar (a 4.5 sigma tail).  The rms
+        # itself is the sharper check: a wrong rounding point or a dropped term moves it at once.
+        error_rms = float(np.sqrt(np.mean(np.square(got[index] - want[slot]))))
+        assert error_rms <= 0.006 * rms, f"config 5, sequence {index}: rms error {error_rms / rms:.4f} of the logits' rms"
 
 
 @pytest.mark.parametrize("vocab,d,batch,seq", [(256, 512, 9, 1000), (100, 1024, 2, 50), (50, 2048, 1, 7), (50, 2052, 3, 7), (30, 96, 4, 33),
