@@ -46,6 +46,9 @@ def assert_close(actual, expected, rel, abs_tol, what=""):
     err = np.abs(a - e)
     bound = abs_tol + rel * np.abs(e)
     worst = int(np.argmax(err - bound))
+    if os.environ.get("ST_PRINT_MARGINS") and a.size:  # how much of each bar a run uses: `pytest -s` with this set
+        used = float(np.max(err / np.maximum(bound, 1e-300))) if np.all(bound > 0) else float("nan")
+        print(f"\n[margin] {used:8.3f} of the bar  {what}  ({a.size} values)", flush=True)
     assert (err <= bound).all(), (
         f"{what}: {int((err > bound).sum())} of {a.size} elements out of tolerance; worst at {worst}: "
         f"actual {a[worst]!r} expected {e[worst]!r} |diff| {err[worst]:.3e} bound {bound[worst]:.3e}")
