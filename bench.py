@@ -53,7 +53,7 @@ MEASURED_TRAFFIC_BYTES = {
     "gemm_bf16_f32acc_16x4096x4096": ((16927 + 1045) * 2 + 2048 + 256) * 1024,
     "gemm_bf16_f32acc_16x4096x4096_prepacked_rhs": (16924 * 2 + 256) * 1024,
     "attention_f32_b8_h16_s2048_d64_noncausal": (98379 * 2 + 65536) * 1024,
-    "attention_f32_b8_h16_s2048_d64_causal": (138815 * 2 + 65537) * 1024,
+    "attention_f32_b8_h16_s2048_d64_causal": (134572 * 2 + 65547) * 1024,
     "attention_f32_attn_bias_c1_s2048_d64": ((10840 + 4260) * 2 + 8448 + 512) * 1024,
     "attention_f32_attn_bias_c16_s1024_d64": ((49240 + 8484) * 2 + 16896 + 4096) * 1024,
     "gemm_f32_100352x128x576_conv_equivalent": (136982 * 2 + 50176) * 1024,
